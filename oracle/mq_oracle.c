@@ -1,0 +1,544 @@
+/*
+ * mq_oracle.c -- CPU restatement of the Miles weight-quantization hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the parity checker for the HIP
+ * kernels in miles_amd/csrc and the "port" CPU baseline timed by bench.py.
+ * Nothing in the product package may import, link or call it.
+ *
+ * Every function cites the reference file:line (relative to the reference
+ * repository root) whose arithmetic it follows.  All arithmetic is IEEE
+ * binary32 round-to-nearest-even; build with -ffp-contract=off so that the
+ * compiler never fuses a multiply and an add (see oracle/Makefile).
+ *
+ * Pin status of each function (what independent evidence fixes its output)
+ * is listed in oracle/README.md; functions that restate third-party
+ * arithmetic whose source is not in the reference repository (Transformer
+ * Engine's MXFP8 / NVFP4 quantizers) are marked "parity unpinned" there.
+ *
+ * Input dtype codes: 0 = bfloat16, 1 = float16, 2 = float32.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define MQ_BF16 0
+#define MQ_F16 1
+#define MQ_F32 2
+
+/* ------------------------------------------------------------------ */
+/* bit-level helpers                                                    */
+/* ------------------------------------------------------------------ */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+static inline float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* float32 -> bfloat16, round to nearest even; NaN -> 0x7FC0 (PyTorch's
+ * c10::BFloat16 rounding). */
+static inline uint16_t f32_to_bf16(float f) {
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+static inline float f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1Fu;
+    uint32_t m = h & 0x3FFu;
+    if (e == 0) {
+        if (m == 0) return u2f(sign);
+        /* subnormal: value = m * 2^-24 */
+        float v = (float)m * 5.9604644775390625e-8f;
+        return u2f(f2u(v) | sign);
+    }
+    if (e == 31) return u2f(sign | 0x7F800000u | (m << 13));
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* float32 -> float16 round to nearest even (IEEE), used only for the
+ * dtype-generic INT4 python-half chain. */
+static inline uint16_t f32_to_f16(float f) {
+    uint32_t u = f2u(f);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7E00;
+    if (a >= 0x477FF000u) return sign | 0x7C00; /* >= 65520 -> inf */
+    if (a < 0x38800000u) {                      /* < 2^-14: subnormal half */
+        float v = u2f(a) * 16777216.0f;         /* * 2^24, exact */
+        float r = nearbyintf(v);
+        return sign | (uint16_t)r;
+    }
+    uint32_t lsb = (a >> 13) & 1u;
+    a += 0xFFFu + lsb;
+    return sign | (uint16_t)((a - 0x38000000u) >> 13);
+}
+
+static inline float load_as_f32(const void* p, int64_t i, int dtype) {
+    switch (dtype) {
+        case MQ_BF16: return bf16_to_f32(((const uint16_t*)p)[i]);
+        case MQ_F16: return f16_to_f32(((const uint16_t*)p)[i]);
+        default: return ((const float*)p)[i];
+    }
+}
+
+/* round a float to the storage dtype and widen back (torch elementwise ops
+ * on a low-precision tensor compute in fp32 and round the result once). */
+static inline float round_to_dtype(float f, int dtype) {
+    switch (dtype) {
+        case MQ_BF16: return bf16_to_f32(f32_to_bf16(f));
+        case MQ_F16: return f16_to_f32(f32_to_f16(f));
+        default: return f;
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* float32 -> float8_e4m3fn                                            */
+/* ------------------------------------------------------------------ */
+/* Shared core: |x| finite, below 480.  Returns the 7-bit magnitude code
+ * (may be 0x7F when the value rounds past 448). */
+static inline uint8_t e4m3_mag_rne(uint32_t a) {
+    if (a < 0x3C800000u) { /* |x| < 2^-6: e4m3 subnormal, step 2^-9 */
+        float k = nearbyintf(u2f(a) * 512.0f); /* exact scaling, RNE */
+        return (uint8_t)k;                     /* 0..8 ; 8 == 0x08 == 2^-6 */
+    }
+    int e = (int)(a >> 23) - 127; /* -6 .. 8 */
+    uint32_t m = a & 0x7FFFFFu;
+    uint32_t m3 = m >> 20;
+    uint32_t rem = m & 0xFFFFFu;
+    if (rem > 0x80000u || (rem == 0x80000u && (m3 & 1u))) m3++;
+    if (m3 == 8) { m3 = 0; e++; }
+    uint32_t code = ((uint32_t)(e + 7) << 3) | m3;
+    return code > 0x7Fu ? 0x7F : (uint8_t)code;
+}
+
+/* PyTorch `tensor.to(torch.float8_e4m3fn)` (c10::Float8_e4m3fn): RNE, NO
+ * saturation: |x| > 464 (incl. inf) and NaN -> 0x7F | sign; 464 ties to 448.
+ * Follows tools/convert_hf_to_fp8.py:65 (the .to(float8_e4m3fn) cast). */
+uint8_t mqo_f32_to_e4m3fn(float x) {
+    uint32_t u = f2u(x);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a >= 0x43F00000u) return sign | 0x7F; /* >= 480, inf, NaN */
+    return sign | e4m3_mag_rne(a);
+}
+
+/* Saturating variant (PTX cvt.rn.satfinite.e4m3x2.f32 as used at
+ * miles/kernels/quant/nvfp4_qdq.py:489-511 and by Transformer Engine's
+ * casts): |x| >= 448 and inf -> 448 with sign; NaN -> 0x7F. */
+uint8_t mqo_f32_to_e4m3fn_sat(float x) {
+    uint32_t u = f2u(x);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return 0x7F;
+    if (a >= 0x43E00000u) return sign | 0x7E; /* >= 448 */
+    return sign | e4m3_mag_rne(a);
+}
+
+float mqo_e4m3fn_to_f32(uint8_t c) {
+    uint32_t sign = (uint32_t)(c & 0x80u) << 24;
+    uint32_t e = (c >> 3) & 0xFu, m = c & 7u;
+    if (e == 15 && m == 7) return u2f(sign | 0x7FC00000u);
+    if (e == 0) return u2f(f2u((float)m * 0.001953125f) | sign); /* m * 2^-9 */
+    return u2f(sign | ((e + 120u) << 23) | (m << 20));
+}
+
+/* ------------------------------------------------------------------ */
+/* float32 -> e2m1 (4-bit)                                             */
+/* ------------------------------------------------------------------ */
+/* PTX cvt.rn.satfinite.e2m1x2.f32 (miles/kernels/quant/nvfp4_qdq.py:541-585):
+ * grid {0,.5,1,1.5,2,3,4,6}, round to nearest, ties to the even code,
+ * |x| > 6 and inf saturate to 6, NaN -> 0x7, bit 3 is the sign (-0 -> 0x8). */
+uint8_t mqo_f32_to_e2m1(float x) {
+    uint32_t u = f2u(x);
+    uint8_t sign = (uint8_t)((u >> 28) & 0x8u);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return 0x7;
+    float v = u2f(a);
+    uint8_t c;
+    if (v <= 0.25f) c = 0;
+    else if (v < 0.75f) c = 1;
+    else if (v <= 1.25f) c = 2;
+    else if (v < 1.75f) c = 3;
+    else if (v <= 2.5f) c = 4;
+    else if (v < 3.5f) c = 5;
+    else if (v <= 5.0f) c = 6;
+    else c = 7;
+    return sign | c;
+}
+
+/* ------------------------------------------------------------------ */
+/* A-1a  block_fp8   (tools/convert_hf_to_fp8.py:39-70)                */
+/* ------------------------------------------------------------------ */
+/* w: [M,K] with row stride ldw (elements).  q: [M,K] contiguous e4m3fn.
+ * scale: [ceil(M/bm), ceil(K/bk)] fp32.
+ *   amax  = max |w| over the zero-padded tile           (:49-58)
+ *   scale = f32(amax) / 448                             (:60)  true division
+ *   q     = e4m3fn( clamp(f32(w)/scale, -448, 448) )    (:61-66) true division
+ * A tile whose amax is 0 gives scale 0 and 0/0 = NaN for every element; the
+ * x86 default NaN has its sign bit set, so the byte is 0xFF (clamp keeps NaN). */
+void mqo_block_fp8(const void* w, int dtype, int64_t M, int64_t K, int64_t ldw,
+                   int bm, int bk, uint8_t* q, float* scale) {
+    int64_t nt = (M + bm - 1) / bm, kt = (K + bk - 1) / bk;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t ti = 0; ti < nt; ti++) {
+        for (int64_t tj = 0; tj < kt; tj++) {
+            int64_t r0 = ti * bm, r1 = r0 + bm < M ? r0 + bm : M;
+            int64_t c0 = tj * bk, c1 = c0 + bk < K ? c0 + bk : K;
+            float amax = 0.0f;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) {
+                    float a = fabsf(load_as_f32(w, r * ldw + c, dtype));
+                    /* torch.max propagates NaN */
+                    if (a > amax || a != a) amax = a;
+                }
+            float s = amax / 448.0f;
+            scale[ti * kt + tj] = s;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) {
+                    float x = load_as_f32(w, r * ldw + c, dtype);
+                    float v = x / s;
+                    uint8_t code;
+                    if (v != v) {
+                        /* x86 SSE: 0/0 produces the default NaN (sign set);
+                         * a NaN operand propagates with its own sign. */
+                        uint32_t sign = (x != x) ? (f2u(x) >> 31)
+                                       : (s != s) ? (f2u(s) >> 31) : 1u;
+                        code = (uint8_t)(0x7F | (sign << 7));
+                    } else {
+                        if (v < -448.0f) v = -448.0f;
+                        if (v > 448.0f) v = 448.0f;
+                        code = mqo_f32_to_e4m3fn(v);
+                    }
+                    q[r * K + c] = code;
+                }
+        }
+    }
+}
+
+/* a2: tensor_fp8 / channel_fp8 (tools/convert_hf_to_fp8.py:73-86) and the
+ * per-tensor branch of the sync path (quantizer_fp8.py:153-158):
+ *   scale = f32( max(amax_in_dtype, dtype(1e-12)) ) / 448 ; q = e4m3fn(clamp(w/scale))
+ * per_channel != 0: one scale per row ([M,1]), quotient in fp32; else one 0-dim scale,
+ * quotient rounded to the weight dtype before the clamp (torch type promotion).
+ * floor_in_dtype is 1e-12 already rounded to the tensor dtype by the caller. */
+void mqo_fp8_per_tensor_or_channel(const void* w, int dtype, int64_t M, int64_t K,
+                                   int64_t ldw, int per_channel, float floor_in_dtype,
+                                   uint8_t* q, float* scale) {
+    float tmax = 0.0f;
+    if (!per_channel) {
+        for (int64_t r = 0; r < M; r++)
+            for (int64_t c = 0; c < K; c++) {
+                float a = fabsf(load_as_f32(w, r * ldw + c, dtype));
+                if (a > tmax || a != a) tmax = a;
+            }
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++) {
+        float amax = tmax;
+        if (per_channel) {
+            amax = 0.0f;
+            for (int64_t c = 0; c < K; c++) {
+                float a = fabsf(load_as_f32(w, r * ldw + c, dtype));
+                if (a > amax || a != a) amax = a;
+            }
+        }
+        if (amax < floor_in_dtype) amax = floor_in_dtype;
+        float s = amax / 448.0f;
+        if (per_channel) scale[r] = s; else if (r == 0) scale[0] = s;
+        for (int64_t c = 0; c < K; c++) {
+            float v = load_as_f32(w, r * ldw + c, dtype) / s;
+            /* a 0-dim scale does not promote the result: `weight / scale` stays in the
+             * weight's dtype (one extra rounding) for the per-tensor strategy only */
+            if (!per_channel) v = round_to_dtype(v, dtype);
+            if (v < -448.0f) v = -448.0f;
+            if (v > 448.0f) v = 448.0f;
+            q[r * K + c] = mqo_f32_to_e4m3fn(v);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* A-1b  fp8_blockwise_cast (miles/kernels/quant/fp8_blockwise.py:43-58)*/
+/* ------------------------------------------------------------------ */
+/*   absmax = max( max|f32(x)| over tile , 1e-10f )      (:51)
+ *   x_s    = absmax / 448   ; s_inv = 1 / x_s           (:52-53) IEEE division
+ *   y      = e4m3( clamp(f32(x) * s_inv, -448, 448) )   (:54)
+ * strides in elements for x; y contiguous; S contiguous. */
+void mqo_fp8_blockwise_cast(const void* x, int dtype, int64_t M, int64_t N,
+                            int64_t sxm, int64_t sxn, int bm, int bn,
+                            uint8_t* y, float* S) {
+    int64_t nt = (M + bm - 1) / bm, kt = (N + bn - 1) / bn;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t ti = 0; ti < nt; ti++) {
+        for (int64_t tj = 0; tj < kt; tj++) {
+            int64_t r0 = ti * bm, r1 = r0 + bm < M ? r0 + bm : M;
+            int64_t c0 = tj * bn, c1 = c0 + bn < N ? c0 + bn : N;
+            float amax = 0.0f;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) {
+                    float a = fabsf(load_as_f32(x, r * sxm + c * sxn, dtype));
+                    if (a > amax) amax = a;
+                }
+            float absmax = amax > 1e-10f ? amax : 1e-10f;
+            float x_s = absmax / 448.0f;
+            float s_inv = 1.0f / x_s;
+            S[ti * kt + tj] = x_s;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) {
+                    float v = load_as_f32(x, r * sxm + c * sxn, dtype) * s_inv;
+                    if (v < -448.0f) v = -448.0f;
+                    if (v > 448.0f) v = 448.0f;
+                    y[r * N + c] = mqo_f32_to_e4m3fn(v);
+                }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* A-5  FP8 block dequant (tools/fp8_cast_bf16.py:15-40;               */
+/*      tools/convert_mimo_v2_to_bf16.py:44-47)                        */
+/* ------------------------------------------------------------------ */
+/* y[i,j] = bf16_rne( f32(e4m3(x[i,j])) * s[i/B, j/B] ) */
+void mqo_fp8_block_dequant(const uint8_t* x, const float* s, int64_t M, int64_t N,
+                           int block, uint16_t* y) {
+    int64_t kt = (N + block - 1) / block;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t c = 0; c < N; c++) {
+            float v = mqo_e4m3fn_to_f32(x[r * N + c]) * s[(r / block) * kt + c / block];
+            y[r * N + c] = f32_to_bf16(v);
+        }
+}
+
+/* ------------------------------------------------------------------ */
+/* A-2  MXFP8 1x32 E8M0 (miles/utils/mxfp8.py:51-78; arithmetic is     */
+/*      Transformer Engine 2.17 MXFP8Quantizer -- third party)          */
+/* ------------------------------------------------------------------ */
+/* E8M0 = ceil-to-power-of-two of amax * f32(1/448), saturating at 0xFE;
+ * corroborated in-repo by miles/kernels/quant/fake_quant.py:15-21. */
+uint8_t mqo_f32_to_e8m0_ceil(float v) {
+    uint32_t u = f2u(v);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0xFF;
+    if ((u & 0x7FFFFFFFu) == 0x7F800000u) return 0xFE;
+    if (v == 0.0f) return 0;
+    uint32_t e = (u >> 23) & 0xFFu, m = u & 0x7FFFFFu;
+    if ((m > 0 && e != 0xFE) && !(e == 0 && m <= 0x400000u)) e++;
+    return (uint8_t)e;
+}
+
+void mqo_mxfp8(const void* w, int dtype, int64_t rows, int64_t K, uint8_t* q, uint8_t* scale) {
+    const float inv448 = u2f(0x3B124925u); /* f32(1/448) */
+    int64_t g = K / 32;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t j = 0; j < g; j++) {
+            int64_t base = r * K + j * 32;
+            float amax = 0.0f;
+            for (int i = 0; i < 32; i++) {
+                float a = fabsf(load_as_f32(w, base + i, dtype));
+                if (a > amax) amax = a;
+            }
+            uint8_t e = mqo_f32_to_e8m0_ceil(amax * inv448);
+            float inv;                                   /* 2^(127-e), exact */
+            if (e == 0) inv = 1.0f;
+            else if (e == 254) inv = u2f(0x00400000u);   /* 2^-127, subnormal */
+            else if (e == 255) inv = u2f(0x00200000u);   /* NaN amax: 2^-128 */
+            else inv = u2f((uint32_t)(254 - e) << 23);
+            scale[r * g + j] = e;
+            for (int i = 0; i < 32; i++)
+                q[base + i] = mqo_f32_to_e4m3fn_sat(load_as_f32(w, base + i, dtype) * inv);
+        }
+}
+
+/* ------------------------------------------------------------------ */
+/* A-3  INT4 fake quant (miles/kernels/quant/int4_fake/                 */
+/*      fake_int4_quant_cuda.cu:159-259 for (1,G); :29-91 for (1,32))   */
+/* ------------------------------------------------------------------ */
+/* symmetric:  scale = fmaxf(amax * (1.0f/7.0f), 1e-5f); out = rintf(x/scale)
+ * asymmetric: scale = fmaxf((max-min) * (1.0f/15.0f), 1e-5f);
+ *             zero  = clamp(-rintf(min/scale), 0, 15); out = rintf(x/scale)+zero
+ * out/scale/zero are stored in the input dtype (.cu:251-254).  Columns past N
+ * in a ragged last group read as 0 (.cu:209-213). */
+void mqo_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int G, int sym,
+                         void* out, void* scale_out, void* zero_out) {
+    const float SYM = 1.0f / 7.0f, ASYM = 1.0f / 15.0f;
+    int64_t ng = (N + G - 1) / G;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t j = 0; j < ng; j++) {
+            int64_t c0 = j * G, c1 = c0 + G < N ? c0 + G : N;
+            float mx = -INFINITY, mn = INFINITY;
+            for (int64_t c = c0; c < c0 + G; c++) {
+                float v = c < N ? load_as_f32(x, r * N + c, dtype) : 0.0f;
+                if (sym) mx = fmaxf(mx, fabsf(v));
+                else { mx = fmaxf(mx, v); mn = fminf(mn, v); }
+            }
+            float scale, zero = 0.0f;
+            if (sym) scale = fmaxf(mx * SYM, 1e-5f);
+            else {
+                scale = fmaxf((mx - mn) * ASYM, 1e-5f);
+                zero = fminf(fmaxf(-rintf(mn / scale), 0.0f), 15.0f);
+            }
+            for (int64_t c = c0; c < c1; c++) {
+                float v = rintf(load_as_f32(x, r * N + c, dtype) / scale); /* keeps -0 */
+                if (!sym) v = v + zero;
+                if (dtype == MQ_F32) ((float*)out)[r * N + c] = v;
+                else ((uint16_t*)out)[r * N + c] = dtype == MQ_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+            }
+            if (dtype == MQ_F32) {
+                ((float*)scale_out)[r * ng + j] = scale;
+                if (!sym) ((float*)zero_out)[r * ng + j] = zero;
+            } else {
+                ((uint16_t*)scale_out)[r * ng + j] = dtype == MQ_BF16 ? f32_to_bf16(scale) : f32_to_f16(scale);
+                if (!sym)
+                    ((uint16_t*)zero_out)[r * ng + j] = dtype == MQ_BF16 ? f32_to_bf16(zero) : f32_to_f16(zero);
+            }
+        }
+}
+
+/* pack_layer(weight, G, sym=True)
+ * (miles/backends/megatron_utils/megatron_to_hf/processors/
+ *  quantizer_compressed_tensors.py:235-265; quantize :196-225;
+ *  round_to_quantized_type_dtype :183-193; pack_to_int32 :137-180):
+ *   (out, scale_b) = fake_int4_quant(x)         -- in the input dtype
+ *   w = dtype(out * scale_b)                    (:241)
+ *   r = dtype(w / scale_b)                      (:213)
+ *   q = int8(round_half_even(clamp(r,-128,127)))(:190)
+ *   code = uint8(q + 8)                         (:153-155)
+ *   packed[m,j] = sum_i code[m,8j+i] << 4i      (:173-175) int32 wraparound
+ * K must be a multiple of G and of 8. */
+void mqo_int4_pack_layer(const void* w, int dtype, int64_t M, int64_t K, int G,
+                         int32_t* packed, void* scale_out) {
+    size_t esz = dtype == MQ_F32 ? 4 : 2;
+    void* out = malloc((size_t)M * K * esz);
+    mqo_int4_fake_quant(w, dtype, M, K, G, 1, out, scale_out, NULL);
+    int64_t ng = K / G, np = K / 8;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t j = 0; j < np; j++) {
+            uint32_t word = 0;
+            for (int i = 0; i < 8; i++) {
+                int64_t c = j * 8 + i;
+                float q0 = load_as_f32(out, r * K + c, dtype);
+                float sb = load_as_f32(scale_out, r * ng + c / G, dtype);
+                float wv = round_to_dtype(q0 * sb, dtype);
+                float rv = round_to_dtype(wv / sb, dtype);
+                if (rv < -128.0f) rv = -128.0f;
+                if (rv > 127.0f) rv = 127.0f;
+                int8_t qi = (int8_t)nearbyintf(rv);
+                uint8_t code = (uint8_t)(qi + 8);
+                word += (uint32_t)code << (4 * i);
+            }
+            packed[r * np + j] = (int32_t)word;
+        }
+    free(out);
+}
+
+/* ------------------------------------------------------------------ */
+/* A-4  NVFP4 (miles/utils/nvfp4.py:19-134; block arithmetic restated   */
+/*      from miles/kernels/quant/nvfp4_qdq.py:716-743,859-889,1079-1081)*/
+/* ------------------------------------------------------------------ */
+#define MQO_FLT_MAX 3.402823466e+38f
+
+/* global amax = max |f32(x)| over the tensor (nvfp4_qdq.py:1213-1217). */
+float mqo_nvfp4_amax(const void* w, int dtype, int64_t numel) {
+    float amax = 0.0f;
+#pragma omp parallel for reduction(max : amax) schedule(static)
+    for (int64_t i = 0; i < numel; i++) {
+        float a = fabsf(load_as_f32(w, i, dtype));
+        if (a > amax) amax = a;
+    }
+    return amax;
+}
+
+/* Published global scale (miles/utils/nvfp4.py:19-39):
+ *   enc = min(e4m3_max*6 / amax, FLT_MAX); enc == 0 -> 1; weight_scale_2 = 1/enc
+ * torch.clamp_max / torch.min propagate NaN. */
+float mqo_nvfp4_global_encode_scale(float amax, int e4m3_max) {
+    float enc = ((float)e4m3_max * 6.0f) / amax;
+    if (enc == enc && enc > MQO_FLT_MAX) enc = MQO_FLT_MAX;
+    if (enc == 0.0f) enc = 1.0f;
+    return enc;
+}
+float mqo_nvfp4_global_decode_scale(float amax, int e4m3_max) {
+    return 1.0f / mqo_nvfp4_global_encode_scale(amax, e4m3_max);
+}
+
+/* In-kernel encode scale (nvfp4_qdq.py:859-867): additionally amax == 0 -> 1;
+ * PTX min.f32 returns the non-NaN operand. */
+static inline float nvfp4_kernel_encode_scale(float amax, int e4m3_max) {
+    float enc = ((float)e4m3_max * 6.0f) / amax;
+    enc = fminf(enc, MQO_FLT_MAX);
+    if (amax == 0.0f) enc = 1.0f;
+    if (enc == 0.0f) enc = 1.0f;
+    return enc;
+}
+
+/* w: [M,K] contiguous, K % 16 == 0.  q: [M,K/2] (element 2i in the low
+ * nibble).  s8: [M,K/16] e4m3fn bytes.  amax: global amax (for a gate/up
+ * pair: over both tensors). */
+void mqo_nvfp4_quant(const void* w, int dtype, int64_t M, int64_t K, float amax,
+                     int e4m3_max, uint8_t* q, uint8_t* s8) {
+    const float sixth = u2f(0x3E2AAAABu);
+    float S_enc = nvfp4_kernel_encode_scale(amax, e4m3_max);
+    float S_dec = 1.0f / S_enc;                      /* nvfp4_qdq.py:1081 */
+    float enc_sixth = S_enc * sixth;                 /* :728 association */
+    int64_t nb = K / 16;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t b = 0; b < nb; b++) {
+            int64_t base = r * K + b * 16;
+            float bmax = 0.0f;
+            for (int i = 0; i < 16; i++) {
+                float a = fabsf(load_as_f32(w, base + i, dtype));
+                if (a > bmax) bmax = a;
+            }
+            float s_hp = (bmax == 0.0f) ? 0.0f : bmax * enc_sixth; /* :716-743 */
+            uint8_t sc = mqo_f32_to_e4m3fn_sat(s_hp);             /* :489-511 */
+            s8[r * nb + b] = sc;
+            float s_f = mqo_e4m3fn_to_f32(sc);
+            float inv = fminf(1.0f / (s_f * S_dec), MQO_FLT_MAX); /* :870-873 */
+            for (int i = 0; i < 16; i += 2) {
+                uint8_t lo = mqo_f32_to_e2m1(load_as_f32(w, base + i, dtype) * inv);
+                uint8_t hi = mqo_f32_to_e2m1(load_as_f32(w, base + i + 1, dtype) * inv);
+                q[(base + i) / 2] = (uint8_t)(lo | (hi << 4));    /* :571-575 */
+            }
+        }
+}
+
+/* ------------------------------------------------------------------ */
+/* decode helpers used by round-trip property tests                     */
+/* ------------------------------------------------------------------ */
+float mqo_e2m1_to_f32(uint8_t c) {
+    static const float tab[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+    float v = tab[c & 7];
+    return (c & 8) ? -v : v;
+}
+
+/* vector forms so that tests can sweep many values quickly */
+void mqo_f32_to_e4m3fn_vec(const float* x, int64_t n, uint8_t* out, int sat) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) out[i] = sat ? mqo_f32_to_e4m3fn_sat(x[i]) : mqo_f32_to_e4m3fn(x[i]);
+}
+void mqo_f32_to_e2m1_vec(const float* x, int64_t n, uint8_t* out) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) out[i] = mqo_f32_to_e2m1(x[i]);
+}
+void mqo_f32_to_bf16_vec(const float* x, int64_t n, uint16_t* out) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) out[i] = f32_to_bf16(x[i]);
+}
+void mqo_f32_to_e8m0_vec(const float* x, int64_t n, uint8_t* out) {
+    for (int64_t i = 0; i < n; i++) out[i] = mqo_f32_to_e8m0_ceil(x[i]);
+}
+
+/* 64-bit FNV-1a over a byte range: cheap whole-tensor fingerprint for the
+ * full-size parity checks (the same routine hashes oracle and GPU output). */
+uint64_t mqo_fnv1a64(const uint8_t* p, int64_t n) {
+    uint64_t h = 1469598103934665603ull;
+    for (int64_t i = 0; i < n; i++) { h ^= p[i]; h *= 1099511628211ull; }
+    return h;
+}

@@ -1,0 +1,283 @@
+"""ctypes front end of the CPU oracle (oracle/mq_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg as the checker / reported baseline.  The product
+package (miles_amd) never imports this module.
+
+All functions take and return CPU torch tensors; bf16 / fp16 / fp32 inputs.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_build", "libmq_oracle.so")
+
+_DTYPE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+
+def build(force: bool = False) -> str:
+    """Compile oracle/mq_oracle.c with gcc (see oracle/Makefile)."""
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(
+        os.path.join(_HERE, "mq_oracle.c")
+    ):
+        subprocess.check_call(["make", "-C", _HERE, "-B"], stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = ctypes.CDLL(_SO)
+        c = ctypes
+        vp, i64, i32, f32 = c.c_void_p, c.c_int64, c.c_int, c.c_float
+        L.mqo_f32_to_e4m3fn.restype = c.c_uint8
+        L.mqo_f32_to_e4m3fn.argtypes = [f32]
+        L.mqo_f32_to_e4m3fn_sat.restype = c.c_uint8
+        L.mqo_f32_to_e4m3fn_sat.argtypes = [f32]
+        L.mqo_e4m3fn_to_f32.restype = f32
+        L.mqo_e4m3fn_to_f32.argtypes = [c.c_uint8]
+        L.mqo_f32_to_e2m1.restype = c.c_uint8
+        L.mqo_f32_to_e2m1.argtypes = [f32]
+        L.mqo_e2m1_to_f32.restype = f32
+        L.mqo_e2m1_to_f32.argtypes = [c.c_uint8]
+        L.mqo_f32_to_e8m0_ceil.restype = c.c_uint8
+        L.mqo_f32_to_e8m0_ceil.argtypes = [f32]
+        L.mqo_block_fp8.restype = None
+        L.mqo_block_fp8.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, vp]
+        L.mqo_fp8_per_tensor_or_channel.restype = None
+        L.mqo_fp8_per_tensor_or_channel.argtypes = [vp, i32, i64, i64, i64, i32, f32, vp, vp]
+        L.mqo_fp8_blockwise_cast.restype = None
+        L.mqo_fp8_blockwise_cast.argtypes = [vp, i32, i64, i64, i64, i64, i32, i32, vp, vp]
+        L.mqo_fp8_block_dequant.restype = None
+        L.mqo_fp8_block_dequant.argtypes = [vp, vp, i64, i64, i32, vp]
+        L.mqo_mxfp8.restype = None
+        L.mqo_mxfp8.argtypes = [vp, i32, i64, i64, vp, vp]
+        L.mqo_int4_fake_quant.restype = None
+        L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
+        L.mqo_int4_pack_layer.restype = None
+        L.mqo_int4_pack_layer.argtypes = [vp, i32, i64, i64, i32, vp, vp]
+        L.mqo_nvfp4_amax.restype = f32
+        L.mqo_nvfp4_amax.argtypes = [vp, i32, i64]
+        L.mqo_nvfp4_global_encode_scale.restype = f32
+        L.mqo_nvfp4_global_encode_scale.argtypes = [f32, i32]
+        L.mqo_nvfp4_global_decode_scale.restype = f32
+        L.mqo_nvfp4_global_decode_scale.argtypes = [f32, i32]
+        L.mqo_nvfp4_quant.restype = None
+        L.mqo_nvfp4_quant.argtypes = [vp, i32, i64, i64, f32, i32, vp, vp]
+        L.mqo_f32_to_e4m3fn_vec.restype = None
+        L.mqo_f32_to_e4m3fn_vec.argtypes = [vp, i64, vp, i32]
+        L.mqo_f32_to_e2m1_vec.restype = None
+        L.mqo_f32_to_e2m1_vec.argtypes = [vp, i64, vp]
+        L.mqo_f32_to_bf16_vec.restype = None
+        L.mqo_f32_to_bf16_vec.argtypes = [vp, i64, vp]
+        L.mqo_f32_to_e8m0_vec.restype = None
+        L.mqo_f32_to_e8m0_vec.argtypes = [vp, i64, vp]
+        L.mqo_fnv1a64.restype = c.c_uint64
+        L.mqo_fnv1a64.argtypes = [vp, i64]
+        _lib = L
+    return _lib
+
+
+def _check_cpu(t: torch.Tensor) -> None:
+    assert t.device.type == "cpu", "the oracle runs on CPU tensors"
+    assert t.dtype in _DTYPE, f"unsupported dtype {t.dtype}"
+
+
+def ceil_div(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+# --------------------------------------------------------------------------
+# FP8 128x128
+# --------------------------------------------------------------------------
+def block_fp8(weight: torch.Tensor, block_size=(128, 128)):
+    """tools/convert_hf_to_fp8.py:39-70 -> (float8_e4m3fn [M,K], float32 [nt,kt])."""
+    _check_cpu(weight)
+    assert weight.dim() == 2 and weight.stride(1) == 1
+    M, K = weight.shape
+    bm, bk = int(block_size[0]), int(block_size[1])
+    q = torch.empty((M, K), dtype=torch.uint8)
+    s = torch.empty((ceil_div(M, bm), ceil_div(K, bk)), dtype=torch.float32)
+    lib().mqo_block_fp8(weight.data_ptr(), _DTYPE[weight.dtype], M, K, weight.stride(0), bm, bk,
+                        q.data_ptr(), s.data_ptr())
+    return q.view(torch.float8_e4m3fn), s
+
+
+def tensor_fp8(weight: torch.Tensor):
+    """tools/convert_hf_to_fp8.py:81-86 -> (e4m3fn [M,K], float32 [1])."""
+    return _per_tensor_or_channel(weight, False)
+
+
+def channel_fp8(weight: torch.Tensor):
+    """tools/convert_hf_to_fp8.py:73-78 -> (e4m3fn [M,K], float32 [M,1])."""
+    return _per_tensor_or_channel(weight, True)
+
+
+def _per_tensor_or_channel(weight, per_channel):
+    _check_cpu(weight)
+    assert weight.dim() == 2 and weight.stride(1) == 1
+    M, K = weight.shape
+    floor = float(torch.tensor(1e-12, dtype=weight.dtype).float())
+    q = torch.empty((M, K), dtype=torch.uint8)
+    s = torch.empty((M, 1) if per_channel else (1,), dtype=torch.float32)
+    lib().mqo_fp8_per_tensor_or_channel(weight.data_ptr(), _DTYPE[weight.dtype], M, K, weight.stride(0),
+                                        int(per_channel), floor, q.data_ptr(), s.data_ptr())
+    return q.view(torch.float8_e4m3fn), s
+
+
+def fp8_blockwise_cast(x: torch.Tensor, block_size=None):
+    """miles/kernels/quant/fp8_blockwise.py:61-79 (any strides)."""
+    _check_cpu(x)
+    assert x.dim() == 2
+    bm, bn = (128, 128) if not block_size else (int(block_size[0]), int(block_size[1]))
+    M, N = x.shape
+    y = torch.empty((M, N), dtype=torch.uint8)
+    s = torch.empty((ceil_div(M, bm), ceil_div(N, bn)), dtype=torch.float32)
+    lib().mqo_fp8_blockwise_cast(x.data_ptr(), _DTYPE[x.dtype], M, N, x.stride(0), x.stride(1), bm, bn,
+                                 y.data_ptr(), s.data_ptr())
+    return y.view(torch.float8_e4m3fn), s
+
+
+def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
+    """tools/fp8_cast_bf16.py:30-40 -> bf16 [M,N]."""
+    assert x.is_contiguous() and s.is_contiguous() and x.dim() == 2 and s.dim() == 2
+    assert x.element_size() == 1 and s.dtype == torch.float32
+    M, N = x.shape
+    y = torch.empty((M, N), dtype=torch.bfloat16)
+    lib().mqo_fp8_block_dequant(x.data_ptr(), s.data_ptr(), M, N, int(block_size), y.data_ptr())
+    return y
+
+
+# --------------------------------------------------------------------------
+# MXFP8
+# --------------------------------------------------------------------------
+def mxfp8_quantize(weight: torch.Tensor):
+    """miles/utils/mxfp8.py:51-78 -> (e4m3fn like weight, uint8 [..., K/32])."""
+    _check_cpu(weight)
+    weight = weight.contiguous()
+    k = weight.shape[-1]
+    if k % 32 != 0:
+        raise ValueError(f"Last dim {k} must be divisible by 32 for MXFP8.")
+    rows = weight.numel() // k
+    q = torch.empty(weight.shape, dtype=torch.uint8)
+    s = torch.empty((*weight.shape[:-1], k // 32), dtype=torch.uint8)
+    lib().mqo_mxfp8(weight.data_ptr(), _DTYPE[weight.dtype], rows, k, q.data_ptr(), s.data_ptr())
+    return q.view(torch.float8_e4m3fn), s
+
+
+# --------------------------------------------------------------------------
+# INT4
+# --------------------------------------------------------------------------
+def fake_int4_quant(x: torch.Tensor, block_size, sym: bool):
+    """fake_int4_quant_cuda.cu:319-364 for block (1, G) -> (out, scale, zero) in x.dtype."""
+    _check_cpu(x)
+    assert x.dim() == 2 and int(block_size[0]) == 1
+    x = x.contiguous()
+    G = int(block_size[1])
+    M, N = x.shape
+    out = torch.empty_like(x)
+    scale = torch.empty((M, ceil_div(N, G)), dtype=x.dtype)
+    zero = torch.zeros_like(scale)
+    lib().mqo_int4_fake_quant(x.data_ptr(), _DTYPE[x.dtype], M, N, G, int(sym), out.data_ptr(),
+                              scale.data_ptr(), zero.data_ptr())
+    return out, scale, zero
+
+
+def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
+    """quantizer_compressed_tensors.py:235-265 (sym) -> (int32 [M,K/8], dtype [M,K/G], None)."""
+    _check_cpu(weight)
+    assert sym, "the oracle restates the symmetric branch"
+    weight = weight.contiguous()
+    M, K = weight.shape
+    assert K % group_size == 0 and K % 8 == 0
+    packed = torch.empty((M, K // 8), dtype=torch.int32)
+    scale = torch.empty((M, K // group_size), dtype=weight.dtype)
+    lib().mqo_int4_pack_layer(weight.data_ptr(), _DTYPE[weight.dtype], M, K, int(group_size),
+                              packed.data_ptr(), scale.data_ptr())
+    return packed, scale, None
+
+
+# --------------------------------------------------------------------------
+# NVFP4
+# --------------------------------------------------------------------------
+def nvfp4_amax(weight: torch.Tensor) -> float:
+    _check_cpu(weight)
+    w = weight.contiguous()
+    return float(lib().mqo_nvfp4_amax(w.data_ptr(), _DTYPE[w.dtype], w.numel()))
+
+
+def nvfp4_global_encode_scale(amax: float, e4m3_max: int = 448) -> float:
+    return float(lib().mqo_nvfp4_global_encode_scale(amax, e4m3_max))
+
+
+def nvfp4_global_decode_scale(amax: float, e4m3_max: int = 448) -> float:
+    return float(lib().mqo_nvfp4_global_decode_scale(amax, e4m3_max))
+
+
+def nvfp4_quantize_1d(weight: torch.Tensor, amax: float | None = None, e4m3_max: int = 448):
+    """miles/utils/nvfp4.py:54-82 -> (uint8 [M,K/2], e4m3fn [M,K/16], float32 [])."""
+    _check_cpu(weight)
+    assert weight.dim() == 2
+    w = weight.contiguous()
+    M, K = w.shape
+    assert K % 16 == 0
+    if amax is None:
+        amax = nvfp4_amax(w)
+    q = torch.empty((M, K // 2), dtype=torch.uint8)
+    s = torch.empty((M, K // 16), dtype=torch.uint8)
+    lib().mqo_nvfp4_quant(w.data_ptr(), _DTYPE[w.dtype], M, K, amax, e4m3_max, q.data_ptr(), s.data_ptr())
+    g = torch.tensor(nvfp4_global_decode_scale(amax, e4m3_max), dtype=torch.float32)
+    return q, s.view(torch.float8_e4m3fn), g
+
+
+def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor, e4m3_max: int = 448):
+    """miles/utils/nvfp4.py:85-114: one amax over both tensors."""
+    amax = max(nvfp4_amax(first), nvfp4_amax(second))
+    return nvfp4_quantize_1d(first, amax, e4m3_max), nvfp4_quantize_1d(second, amax, e4m3_max)
+
+
+# --------------------------------------------------------------------------
+# scalar / vector conversion helpers
+# --------------------------------------------------------------------------
+def f32_to_e4m3fn(x: torch.Tensor, sat: bool = False) -> torch.Tensor:
+    x = x.contiguous().float()
+    out = torch.empty(x.shape, dtype=torch.uint8)
+    lib().mqo_f32_to_e4m3fn_vec(x.data_ptr(), x.numel(), out.data_ptr(), int(sat))
+    return out
+
+
+def f32_to_e2m1(x: torch.Tensor) -> torch.Tensor:
+    x = x.contiguous().float()
+    out = torch.empty(x.shape, dtype=torch.uint8)
+    lib().mqo_f32_to_e2m1_vec(x.data_ptr(), x.numel(), out.data_ptr())
+    return out
+
+
+def f32_to_bf16_bits(x: torch.Tensor) -> torch.Tensor:
+    x = x.contiguous().float()
+    out = torch.empty(x.shape, dtype=torch.int16)
+    lib().mqo_f32_to_bf16_vec(x.data_ptr(), x.numel(), out.data_ptr())
+    return out
+
+
+def f32_to_e8m0(x: torch.Tensor) -> torch.Tensor:
+    x = x.contiguous().float()
+    out = torch.empty(x.shape, dtype=torch.uint8)
+    lib().mqo_f32_to_e8m0_vec(x.data_ptr(), x.numel(), out.data_ptr())
+    return out
+
+
+def fnv1a64(t: torch.Tensor) -> int:
+    t = t.contiguous()
+    return int(lib().mqo_fnv1a64(t.data_ptr(), t.numel() * t.element_size()))

@@ -1,0 +1,472 @@
+"""Pins the CPU oracle (oracle/mq_oracle.c) BEFORE it is trusted as the parity checker.
+
+Each oracle function is compared with evidence that does not come from the oracle:
+  * PyTorch's own CPU routines (float8_e4m3fn / bfloat16 casts, true fp32 division, clamp,
+    round-half-even, bf16 elementwise ops) chained exactly as the reference chains them;
+  * the golden vectors and known-answer tests the reference's own tests hold for this path;
+  * closed forms / invariants (decode tables, per-tile max == 448, ceil-to-power-of-two,
+    constant rows, all 256 fp8 codes).
+MXFP8 and the NVFP4 block arithmetic restate Transformer Engine (third party, source not in the
+reference repository): the checks here fix them against the published closed form and an
+independent torch restatement only -- "parity unpinned" against TE itself.
+"""
+
+import math
+
+import pytest
+import torch
+
+from miles_amd import workloads as W
+
+F8 = torch.float8_e4m3fn
+FP8_MAX = 448.0
+
+
+# ----------------------------------------------------------------------------------------------
+# conversions
+# ----------------------------------------------------------------------------------------------
+def _interesting_floats() -> torch.Tensor:
+    """Every (sign, exponent, top-3-mantissa) prefix with the low 20 bits at each rounding-decisive
+    pattern, plus 2^22 random bit patterns."""
+    hi = torch.arange(0, 1 << 12, dtype=torch.int64) << 20
+    lows = torch.tensor([0x0, 0x1, 0x7FFFF, 0x80000, 0x80001, 0xFFFFF, 0x40000, 0xC0000], dtype=torch.int64)
+    grid = (hi[:, None] | lows[None, :]).reshape(-1)
+    g = torch.Generator().manual_seed(7)
+    rnd = torch.randint(0, 1 << 32, (1 << 22,), generator=g, dtype=torch.int64)
+    bits = torch.cat([grid, rnd])
+    bits = torch.where(bits >= (1 << 31), bits - (1 << 32), bits).to(torch.int32)
+    return bits.view(torch.float32)
+
+
+def test_e4m3fn_cast_matches_torch(oracle):
+    x = _interesting_floats()
+    want = x.to(F8).view(torch.uint8)
+    got = oracle.f32_to_e4m3fn(x)
+    nan = torch.isnan(x)
+    assert torch.equal(got[~nan], want[~nan])
+    # NaN: magnitude 0x7F; torch keeps the sign bit
+    assert torch.equal(got[nan] & 0x7F, torch.full_like(got[nan], 0x7F))
+    assert torch.equal(got[nan], want[nan])
+
+
+def test_e4m3fn_cast_known_answers(oracle):
+    # PyTorch float8_e4m3fn semantics: RNE, subnormal step 2^-9, 464 ties to 448, >464 -> NaN code
+    x = torch.tensor([2.0**-10, 1.5 * 2.0**-10, 17, 18, 19, 21, 448, 464, 465, float("nan"), -0.0])
+    assert oracle.f32_to_e4m3fn(x).tolist() == [0, 1, 88, 89, 90, 90, 126, 126, 127, 127, 128]
+    # saturating form: >=448 and inf clamp to 0x7E, NaN -> 0x7F
+    y = torch.tensor([448.0, 464.0, 465.0, 1e30, float("inf"), -float("inf"), -500.0, float("nan")])
+    assert oracle.f32_to_e4m3fn(y, sat=True).tolist() == [126, 126, 126, 126, 126, 254, 254, 127]
+
+
+def test_e4m3fn_sat_equals_clamp_then_torch_cast(oracle):
+    x = _interesting_floats()
+    x = x[~torch.isnan(x)]
+    want = x.clamp(-FP8_MAX, FP8_MAX).to(F8).view(torch.uint8)
+    assert torch.equal(oracle.f32_to_e4m3fn(x, sat=True), want)
+
+
+def test_e4m3fn_decode_table(oracle):
+    codes = torch.arange(256, dtype=torch.uint8)
+    want = codes.view(F8).float()
+    got = torch.tensor([oracle.lib().mqo_e4m3fn_to_f32(int(c)) for c in codes])
+    nan = torch.isnan(want)
+    assert nan.sum() == 2 and torch.equal(torch.isnan(got), nan)
+    assert torch.equal(got[~nan].view(torch.int32), want[~nan].view(torch.int32))
+
+
+def test_bf16_rounding_matches_torch(oracle):
+    x = _interesting_floats()
+    hi = torch.arange(0, 1 << 16, dtype=torch.int64) << 16
+    lows = torch.tensor([0x0, 0x1, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=torch.int64)
+    grid = (hi[:, None] | lows[None, :]).reshape(-1)
+    grid = torch.where(grid >= (1 << 31), grid - (1 << 32), grid).to(torch.int32).view(torch.float32)
+    x = torch.cat([x, grid])
+    x = x[~torch.isnan(x)]
+    assert torch.equal(oracle.f32_to_bf16_bits(x), x.to(torch.bfloat16).view(torch.int16))
+
+
+def test_e2m1_grid_ties_and_saturation(oracle):
+    # closed form: grid {0,.5,1,1.5,2,3,4,6}; ties go to the even code; satfinite; NaN -> +6 code
+    x = torch.tensor([0.0, 0.25, 0.2500001, 0.5, 0.75, 1.0, 1.25, 1.2500001, 1.5, 1.75, 2.0, 2.5, 2.5000002, 3.0,
+                      3.5, 4.0, 5.0, 5.0000005, 6.0, 7.0, 1e30, float("inf"), float("nan"), -0.0, -0.25, -0.75,
+                      -6.5, -float("inf")])
+    want = [0, 0, 1, 1, 2, 2, 2, 3, 3, 4, 4, 4, 5, 5, 6, 6, 6, 7, 7, 7, 7, 7, 7, 8, 8, 10, 15, 15]
+    assert oracle.f32_to_e2m1(x).tolist() == want
+
+
+def test_e2m1_matches_round_to_fp4_grid(oracle):
+    # independent statement of RNE on the e2m1 grid: tests/fast-gpu/kernels/quant/test_fake_quant.py:29-32
+    g = torch.Generator().manual_seed(3)
+    x = torch.cat([8 * torch.rand(1 << 18, generator=g) - 4, torch.linspace(-7, 7, 2241)])
+    mag = x.abs().clamp(max=6.0)
+    step = torch.where(mag < 2.0, 0.5, torch.where(mag < 4.0, 1.0, 2.0))
+    want = torch.round(mag / step) * step
+    codes = oracle.f32_to_e2m1(x)
+    table = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    assert torch.equal(table[(codes & 7).long()], want)
+    assert torch.equal((codes >> 3).bool(), torch.signbit(x))
+
+
+def test_e8m0_is_ceil_pow2(oracle):
+    # ceil-to-power-of-two, corroborated by miles/kernels/quant/fake_quant.py:15-21 and the frexp form
+    # of tests/fast-gpu/kernels/quant/test_fake_quant.py:24-26
+    g = torch.Generator().manual_seed(5)
+    v = torch.cat([torch.rand(1 << 16, generator=g) * 10 ** (torch.rand(1 << 16, generator=g) * 60 - 30),
+                   2.0 ** torch.arange(-120, 120, dtype=torch.float32)])
+    mant, expo = torch.frexp(v)
+    p2 = torch.ldexp(torch.ones_like(v), torch.where(mant == 0.5, expo - 1, expo))
+    want = (torch.log2(p2).round() + 127).to(torch.uint8)
+    assert torch.equal(oracle.f32_to_e8m0(v), want)
+    special = torch.tensor([0.0, float("inf"), float("nan"), 2.0**-127, 1.5 * 2.0**-127, 2.0**-126, 3e38])
+    assert oracle.f32_to_e8m0(special).tolist() == [0, 254, 255, 0, 1, 1, 254]
+
+
+# ----------------------------------------------------------------------------------------------
+# A-1a block_fp8 : tools/convert_hf_to_fp8.py:39-70 chained through torch's CPU kernels
+# ----------------------------------------------------------------------------------------------
+def torch_block_fp8(weight, block_size):
+    bn, bk = block_size
+    n, k = weight.shape
+    nt, kt = -(-n // bn), -(-k // bk)
+    padded = torch.nn.functional.pad(weight, (0, kt * bk - k, 0, nt * bn - n), mode="constant", value=0.0)
+    tiles = padded.reshape(nt, bn, kt, bk)
+    amax = tiles.abs().max(dim=1, keepdim=True)[0].max(dim=3, keepdim=True)[0]
+    scale = amax.to(torch.float32) / FP8_MAX
+    q = (tiles / scale).clamp(min=-FP8_MAX, max=FP8_MAX).reshape(nt * bn, kt * bk).to(F8)
+    return q[:n, :k].clone(), scale.reshape(nt, kt)
+
+
+def _same_fp8(a, b):
+    return torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(130, 257), (1, 1), (127, 129)])
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_block_fp8_matches_torch_chain(oracle, shape, kind):
+    w = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    q, s = oracle.block_fp8(w, (128, 128))
+    q_t, s_t = torch_block_fp8(w, (128, 128))
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32))
+    assert _same_fp8(q, q_t)
+
+
+def test_block_fp8_c1_slice_with_zero_tile(oracle):
+    w = W.gaussian_outliers((384, 512), std=0.02, p_outlier=0.001, gain=20.0, seed=1001)
+    w[128:256, 128:256] = 0
+    w[300, 7] = -0.0
+    q, s = oracle.block_fp8(w, (128, 128))
+    q_t, s_t = torch_block_fp8(w, (128, 128))
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(q, q_t)
+    # scale 0 and 0/0: every byte of the zero tile is the negative NaN code
+    assert s[1, 1].item() == 0.0
+    assert torch.all(q.view(torch.uint8)[128:256, 128:256] == 0xFF)
+    # invariant: a tile with amax > 0 reaches +-448 somewhere
+    dec = q.float()
+    for ti in range(3):
+        for tj in range(4):
+            if (ti, tj) != (1, 1):
+                assert dec[ti * 128:(ti + 1) * 128, tj * 128:(tj + 1) * 128].abs().max().item() == FP8_MAX
+
+
+def test_block_fp8_other_block_sizes_and_dtypes(oracle):
+    g = torch.Generator().manual_seed(11)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        w = (0.05 * torch.randn((96, 160), generator=g)).to(dtype)
+        for bs in ((32, 32), (64, 128), (128, 64)):
+            q, s = oracle.block_fp8(w, bs)
+            q_t, s_t = torch_block_fp8(w, bs)
+            assert torch.equal(s, s_t) and _same_fp8(q, q_t), (dtype, bs)
+
+
+def test_tensor_and_channel_fp8_match_torch_chain(oracle):
+    # tools/convert_hf_to_fp8.py:73-86
+    g = torch.Generator().manual_seed(12)
+    for dtype in (torch.bfloat16, torch.float32):
+        w = (0.02 * torch.randn((64, 96), generator=g)).to(dtype)
+        w[3] = 0
+        s_t = w.abs().max().clamp(min=1e-12).to(torch.float32) / FP8_MAX
+        q_t = (w / s_t).clamp(min=-FP8_MAX, max=FP8_MAX).to(F8)
+        q, s = oracle.tensor_fp8(w)
+        assert torch.equal(s, s_t.view(1)) and _same_fp8(q, q_t)
+        s_c = w.abs().max(dim=-1, keepdim=True)[0].clamp(min=1e-12).to(torch.float32) / FP8_MAX
+        q_c = (w / s_c).clamp(min=-FP8_MAX, max=FP8_MAX).to(F8)
+        q, s = oracle.channel_fp8(w)
+        assert torch.equal(s, s_c) and _same_fp8(q, q_c)
+
+
+# ----------------------------------------------------------------------------------------------
+# A-1b fp8_blockwise_cast : miles/kernels/quant/fp8_blockwise.py:51-58 with IEEE division
+# ----------------------------------------------------------------------------------------------
+def torch_fp8_blockwise_cast(x, bm=128, bn=128):
+    m, n = x.shape
+    mt, nt = -(-m // bm), -(-n // bn)
+    xf = torch.zeros((mt * bm, nt * bn), dtype=torch.float32)
+    xf[:m, :n] = x.float()
+    tiles = xf.reshape(mt, bm, nt, bn)
+    absmax = torch.maximum(tiles.abs().amax(dim=(1, 3), keepdim=True), torch.tensor(1e-10, dtype=torch.float32))
+    x_s = absmax / torch.tensor(FP8_MAX, dtype=torch.float32)
+    s_inv = torch.tensor(1.0, dtype=torch.float32) / x_s
+    y = (tiles * s_inv).clamp(-FP8_MAX, FP8_MAX).reshape(mt * bm, nt * bn)[:m, :n].to(F8)
+    return y, x_s.reshape(mt, nt)
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(130, 257)])
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_fp8_blockwise_cast_matches_torch_chain(oracle, shape, kind):
+    x = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    y, s = oracle.fp8_blockwise_cast(x)
+    y_t, s_t = torch_fp8_blockwise_cast(x)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(y, y_t)
+    if kind == "zeros":  # epsilon floor: scale 1e-10/448, codes 0
+        assert torch.all(y.view(torch.uint8) == 0) and s[0, 0].item() == pytest.approx(1e-10 / 448, rel=1e-6)
+
+
+def test_fp8_blockwise_cast_strided_input(oracle):
+    base = W.gaussian_outliers((256, 300), std=0.02, p_outlier=0.001, gain=20.0, seed=5)
+    for view in (base[:, :256], base.t(), base[::2, 1::2]):
+        y, s = oracle.fp8_blockwise_cast(view)
+        y_t, s_t = torch_fp8_blockwise_cast(view.contiguous())
+        assert torch.equal(s, s_t) and _same_fp8(y, y_t)
+
+
+# ----------------------------------------------------------------------------------------------
+# A-5 dequant : tools/fp8_cast_bf16.py:15-40 == tools/convert_mimo_v2_to_bf16.py:44-47
+# ----------------------------------------------------------------------------------------------
+def torch_dequant_fp8_block(weight, scale_inv):
+    rows, cols = weight.shape
+    scale = scale_inv.float().repeat_interleave(128, dim=0)[:rows].repeat_interleave(128, dim=1)
+    return (weight.float() * scale[:, :cols]).to(torch.bfloat16)
+
+
+def test_dequant_all_codes_random_scales(oracle):
+    g = torch.Generator().manual_seed(21)
+    codes = torch.arange(256, dtype=torch.uint8).repeat(300, 2)[:, :400].contiguous()  # [300,400]
+    s = torch.exp(torch.randn((3, 4), generator=g) * 4).float()
+    y = oracle.weight_dequant(codes.view(F8), s)
+    y_t = torch_dequant_fp8_block(codes.view(F8), s)
+    nan = torch.isnan(y_t)
+    assert torch.equal(torch.isnan(y), nan)
+    assert torch.equal(y.view(torch.int16)[~nan], y_t.view(torch.int16)[~nan])
+
+
+def test_quant_dequant_round_trip_as_reference_test(oracle):
+    # tests/fast/tools/test_convert_mimo_v2_to_bf16.py:17-54: quantise with clamp(1e-12), dequantise, compare
+    # exactly with float(q) * scale -> bf16 and loosely with the source.
+    g = torch.Generator().manual_seed(22)
+    weight = torch.randn((448, 256), generator=g)
+    padded = torch.zeros(512, 256)
+    padded[:448] = weight
+    blocks = padded.view(4, 128, 2, 128)
+    scale = blocks.abs().amax(dim=(1, 3)).clamp(min=1e-12) / FP8_MAX
+    quant = (blocks / scale[:, None, :, None]).view_as(padded)[:448].to(F8)
+    out = oracle.weight_dequant(quant.contiguous(), scale.contiguous())
+    expected = (quant.float() * scale.repeat_interleave(128, 0)[:448].repeat_interleave(128, 1)).to(torch.bfloat16)
+    assert torch.equal(out, expected)
+    assert (out.float() - weight).abs().max() < 0.07 * weight.abs().max()
+    # and the oracle's own block quantiser agrees with that formula when no tile is all-zero
+    q2, s2 = oracle.block_fp8(weight, (128, 128))
+    assert torch.equal(s2, scale) and _same_fp8(q2, quant)
+
+
+# ----------------------------------------------------------------------------------------------
+# A-2 MXFP8 (closed form; Transformer Engine itself is not available -> parity unpinned vs TE)
+# ----------------------------------------------------------------------------------------------
+def torch_mxfp8(w):
+    k = w.shape[-1]
+    x = w.float().reshape(-1, k // 32, 32)
+    amax = x.abs().amax(dim=-1, keepdim=True)
+    v = amax * torch.tensor(0x3B124925, dtype=torch.int32).view(torch.float32)  # f32(1/448)
+    mant, expo = torch.frexp(v)
+    e_unb = torch.where(mant == 0.5, expo - 1, expo)            # ceil(log2 v)
+    e = torch.where(v == 0, torch.zeros_like(e_unb), (e_unb + 127).clamp(0, 254))
+    # v below 2^-127 has no representable ceil power in E8M0: code 0 up to 2^-127, code 1 above
+    e = torch.where((v > 0) & (v <= 2.0**-127), torch.zeros_like(e), e)
+    e = torch.where((v > 2.0**-127) & (v <= 2.0**-126), torch.ones_like(e), e)
+    inv = torch.where(e == 0, torch.ones_like(v), torch.ldexp(torch.ones_like(v), 127 - e))
+    q = (x * inv).clamp(-FP8_MAX, FP8_MAX).to(F8)
+    return q.reshape(w.shape), e.to(torch.uint8).reshape(*w.shape[:-1], k // 32)
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES)
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_mxfp8_matches_closed_form(oracle, shape, kind):
+    w = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    q, s = oracle.mxfp8_quantize(w)
+    q_t, s_t = torch_mxfp8(w)
+    assert q.shape == w.shape and q.dtype == F8 and s.dtype == torch.uint8
+    assert s.shape == (*w.shape[:-1], w.shape[-1] // 32)  # tests/fast-gpu/test_mxfp8_quantizer.py:165-168
+    assert torch.equal(s, s_t) and _same_fp8(q, q_t)
+
+
+def test_mxfp8_student_t_rows_and_invariants(oracle):
+    w = W.student_t_rows((96, 2048), std=0.02, seed=3001)
+    q, s = oracle.mxfp8_quantize(w)
+    q_t, s_t = torch_mxfp8(w)
+    assert torch.equal(s, s_t) and _same_fp8(q, q_t)
+    # scale is the smallest power of two with amax/scale <= 448: decoded magnitudes lie in (224, 448]
+    dec = q.float().reshape(96, 64, 32).abs().amax(dim=-1)
+    nz = w.float().reshape(96, 64, 32).abs().amax(dim=-1) > 0
+    assert torch.all(dec[nz] <= 448) and torch.all(dec[nz] >= 224)
+    with pytest.raises(ValueError, match="must be divisible by 32"):
+        oracle.mxfp8_quantize(torch.zeros(4, 48, dtype=torch.bfloat16))
+
+
+# ----------------------------------------------------------------------------------------------
+# A-3 INT4
+# ----------------------------------------------------------------------------------------------
+def torch_fake_int4_sym(x, G):
+    """fake_int4_quant_cuda.cu:216-252 as fp32 tensor ops on the CPU (true division)."""
+    m, n = x.shape
+    xf = x.float().reshape(m, n // G, G)
+    amax = xf.abs().amax(dim=-1, keepdim=True)
+    scale = torch.maximum(amax * torch.tensor(1.0 / 7.0, dtype=torch.float32), torch.tensor(1e-5, dtype=torch.float32))
+    out = torch.round(xf / scale)
+    return out.reshape(m, n).to(x.dtype), scale.reshape(m, n // G).to(x.dtype)
+
+
+def torch_pack_layer_python_half(w, scale, G):
+    """quantizer_compressed_tensors.py:237-264 given the kernel's (w, scale) in the input dtype."""
+    m, k = w.shape
+    w4 = w.view(m, 1, k // G, G)
+    s4 = scale.view(m, 1, k // G, 1)
+    deq = (w4 * s4).view(m, k)
+    scale2 = s4.view(m, -1).contiguous()
+    x = deq.unflatten(-1, (k // G, G))
+    scaled = x / scale2.unsqueeze(-1)
+    q = torch.round(torch.clamp(scaled, -128, 127)).to(torch.int8).flatten(start_dim=-2)
+    value = (q + 8).to(torch.uint8)
+    reshaped = value.view(m, k // 8, 8).to(torch.int32)
+    shifts = torch.arange(8, dtype=torch.int32) * 4
+    return (reshaped << shifts).sum(dim=2, dtype=torch.int32), scale2
+
+
+@pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((8, 7168), 128),
+                                     ((16, 256), 32), ((5, 96), 32)])
+def test_int4_matches_torch_chain(oracle, shape, G):
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.0005, gain=30.0, seed=4001)
+    w[0] = 0            # amax < 7e-5 -> scale floor 1e-5
+    w[1, :G] = 3e-6
+    out, scale, _ = oracle.fake_int4_quant(w, (1, G), True)
+    out_t, scale_t = torch_fake_int4_sym(w, G)
+    assert torch.equal(out.view(torch.int16), out_t.view(torch.int16))
+    assert torch.equal(scale.view(torch.int16), scale_t.view(torch.int16))
+    packed, pscale, zp = oracle.pack_layer(w, G)
+    packed_t, pscale_t = torch_pack_layer_python_half(out_t, scale_t, G)
+    assert zp is None and torch.equal(packed, packed_t) and torch.equal(pscale.view(torch.int16), pscale_t.view(torch.int16))
+    # codes are rint(x/scale_f32)+8 in [1,15]: the bf16 round trip of pack_layer never moves a code
+    nib = torch.stack([(packed >> (4 * i)) & 0xF for i in range(8)], dim=-1).reshape(shape)
+    assert nib.min() >= 1 and nib.max() <= 15
+    assert torch.equal(nib.to(torch.float32) - 8, out.float())
+
+
+def test_int4_constant_rows_known_answer(oracle):
+    for c in (0.5, 0.013, 3.0):
+        w = torch.full((2, 128), c, dtype=torch.bfloat16)
+        w[1] = -w[1]
+        packed, scale, _ = oracle.pack_layer(w, 128)
+        assert torch.all(packed[0] == torch.tensor(0xFFFFFFFF - (1 << 32), dtype=torch.int64).to(torch.int32))  # code 15
+        assert torch.all(packed[1] == 0x11111111)  # code 1
+        want = (w[0, :1].float() * torch.tensor(1.0 / 7.0, dtype=torch.float32)).to(torch.bfloat16)
+        assert torch.all(scale == want)
+
+
+def test_pack_to_int32_nibble_order(oracle):
+    # nibble i of each int32 is element 8j+i (sequential order): quantizer_compressed_tensors.py:171-175
+    row = torch.tensor([[-7, -5, -3, -1, 1, 3, 5, 7] * 16], dtype=torch.float32)
+    w = (row * (7.0 / 7.0)).to(torch.bfloat16)
+    packed, scale, _ = oracle.pack_layer(w, 128)
+    want = sum((int(v) + 8) << (4 * i) for i, v in enumerate([-7, -5, -3, -1, 1, 3, 5, 7]))
+    assert scale[0, 0].item() == 1.0
+    assert (packed[0, 0].item() & 0xFFFFFFFF) == want
+
+
+# ----------------------------------------------------------------------------------------------
+# A-4 NVFP4
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("e4m3_max", [256, 448])
+def test_nvfp4_global_scale_vectors(oracle, e4m3_max):
+    # tests/fast-gpu/test_nvfp4_quantizer.py:108-143: overflow clamp, underflow repair, NaN propagation
+    values = torch.tensor([0.0, 1.0, 3.5, torch.finfo(torch.float32).tiny, torch.finfo(torch.float32).max,
+                           float("inf"), -float("inf"), float("nan")], dtype=torch.float32)
+    numerator = torch.tensor(float(e4m3_max), dtype=torch.float32) * torch.tensor(6.0, dtype=torch.float32)
+    expected = torch.div(numerator, values)
+    expected = torch.min(expected, torch.tensor(torch.finfo(torch.float32).max))
+    expected = torch.where(expected == 0.0, torch.ones_like(expected), expected)
+    for v, enc in zip(values.tolist(), expected.tolist()):
+        got = oracle.nvfp4_global_encode_scale(v, e4m3_max)
+        dec = oracle.nvfp4_global_decode_scale(v, e4m3_max)
+        if math.isnan(enc):
+            assert math.isnan(got) and math.isnan(dec)
+        else:
+            assert got == enc
+            assert dec == torch.div(1.0, torch.tensor(enc, dtype=torch.float32)).item()
+    # zero tensor: decode scale is 1/FLT_MAX, not 1
+    assert oracle.nvfp4_global_decode_scale(0.0) == torch.div(1.0, torch.tensor(torch.finfo(torch.float32).max)).item()
+
+
+def torch_nvfp4(w, amax=None):
+    """Block arithmetic of miles/kernels/quant/nvfp4_qdq.py:716-743,859-889 in fp32 tensor ops."""
+    f32 = torch.float32
+    m, k = w.shape
+    x = w.float().reshape(m, k // 16, 16)
+    if amax is None:
+        amax = x.abs().max()
+    amax = torch.as_tensor(amax, dtype=f32)
+    flt_max = torch.tensor(torch.finfo(f32).max)
+    s_enc = torch.min(torch.tensor(2688.0, dtype=f32) / amax, flt_max)
+    if amax == 0 or s_enc == 0:
+        s_enc = torch.tensor(1.0, dtype=f32)
+    s_dec = torch.tensor(1.0, dtype=f32) / s_enc
+    sixth = torch.tensor(0x3E2AAAAB, dtype=torch.int32).view(f32)
+    bmax = x.abs().amax(dim=-1, keepdim=True)
+    s_hp = torch.where(bmax == 0, torch.zeros_like(bmax), bmax * (s_enc * sixth))
+    s8 = s_hp.clamp(max=FP8_MAX).to(F8)
+    inv = torch.min(torch.tensor(1.0, dtype=f32) / (s8.float() * s_dec), flt_max)
+    y = x * inv
+    mag = y.abs().clamp(max=6.0)
+    step = torch.where(mag < 2.0, 0.5, torch.where(mag < 4.0, 1.0, 2.0))
+    val = torch.round(mag / step) * step
+    code = torch.bucketize(val, torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])).to(torch.uint8)
+    code = code | (torch.signbit(y).to(torch.uint8) << 3)
+    code = code.reshape(m, k)
+    return code[:, 0::2] | (code[:, 1::2] << 4), s8.reshape(m, k // 16)
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(1, 16), (3, 48), (31, 128)])
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+def test_nvfp4_matches_torch_chain(oracle, shape, kind):
+    w = W.reference_pattern(kind, shape, spread=12.0)
+    if kind == "random" and shape[0] > 1:
+        w[0].zero_()
+    q, s, g = oracle.nvfp4_quantize_1d(w)
+    q_t, s_t = torch_nvfp4(w)
+    assert q.shape == (shape[0], shape[1] // 2) and s.shape == (shape[0], shape[1] // 16) and g.shape == ()
+    assert _same_fp8(s, s_t) and torch.equal(q, q_t)
+    amax = w.float().abs().max()
+    enc = torch.div(2688.0, amax).clamp_max(torch.finfo(torch.float32).max)
+    enc = torch.where(enc == 0.0, 1.0, enc)
+    assert g.item() == torch.div(1.0, enc).item()   # miles/utils/nvfp4.py:19-39
+    if kind == "signed_zeros":   # zero-amax blocks keep the sign bit: nibbles 0x8 / 0x0
+        assert torch.all(q == 0x08) and torch.all(s.view(torch.uint8) == 0)
+
+
+def test_nvfp4_nibble_order_golden(oracle):
+    # tests/fast/backends/megatron_utils/test_quantizer_mxfp4.py:6-16 pins the e2m1 code table and that
+    # element 2i sits in the low nibble: bytes 0x10 0x32 0x54 0x76 decode to codes 0..7 in order.
+    row = torch.tensor([[0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]])
+    q, s, g = oracle.nvfp4_quantize_1d(row.to(torch.bfloat16))
+    assert q[0].tolist() == [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]
+    assert s.view(torch.uint8).item() == 0x7E      # block scale 448 = amax * (2688/amax) / 6
+    assert g.item() == pytest.approx(6.0 / 2688.0, rel=1e-6)
+    table = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for c in range(16):
+        assert oracle.lib().mqo_e2m1_to_f32(c) == (-table[c & 7] if c & 8 else table[c & 7])
+
+
+def test_nvfp4_pair_shares_one_amax(oracle):
+    gate = W.reference_pattern("random", (16, 64), spread=12.0, seed=1)
+    up = 3 * W.reference_pattern("random", (24, 64), spread=12.0, seed=2)
+    (gq, gs, gg), (uq, us, ug) = oracle.nvfp4_quantize_1d_pair(gate, up)
+    cq, cs, cg = oracle.nvfp4_quantize_1d(torch.cat((gate, up), dim=0))
+    assert torch.equal(torch.cat((gq, uq)), cq) and _same_fp8(torch.cat((gs, us)), cs)
+    assert gg.item() == ug.item() == cg.item()
