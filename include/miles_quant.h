@@ -1,0 +1,103 @@
+/*
+ * miles_quant.h -- C ABI of the MI355X (gfx950) weight-quantization library.
+ *
+ * Drop-in boundary for the per-tensor quantize / dequantize kernels of Miles' weight path.  The
+ * reference has no FFI for this path: its quantizers are Python callables backed by Triton, a
+ * pybind11 CUDA extension and Transformer Engine.  Each entry point below names the reference
+ * callable it stands in for (paths relative to the reference repository root); the Python
+ * wrappers in miles_amd/ keep those callables' signatures and bind these symbols with ctypes.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless stated otherwise; plain pointers and sizes only;
+ *   - outputs are allocated by the caller; inputs are never written;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls only enqueue
+ *     work, they never synchronise and never allocate, so they are safe from several host threads;
+ *   - return value: MQ_OK (0) or a negative MQ_ERR_* code; mq_last_error() returns a
+ *     thread-local message for the last failure on the calling thread;
+ *   - dtype codes: MQ_BF16, MQ_F16, MQ_F32.
+ */
+#ifndef MILES_QUANT_H_
+#define MILES_QUANT_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MQ_VERSION 1
+
+enum { MQ_BF16 = 0, MQ_F16 = 1, MQ_F32 = 2 };
+enum { MQ_OK = 0, MQ_ERR_ARG = -1, MQ_ERR_HIP = -2, MQ_ERR_UNSUPPORTED = -3 };
+
+int mq_version(void);
+const char* mq_last_error(void);
+
+/* block_fp8(weight, block_size)                      tools/convert_hf_to_fp8.py:39-70
+ *   w      [M,K] dtype, row stride ldw elements, unit column stride
+ *   q      [M,K] e4m3fn bytes, contiguous
+ *   scale  [ceil(M/block_m), ceil(K/block_k)] fp32 = amax/448; an all-zero tile: scale 0, bytes 0xFF */
+int mq_fp8_block_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
+                       int block_m, int block_k, void* stream);
+
+/* fp8_blockwise_cast(x, block_size)                  miles/kernels/quant/fp8_blockwise.py:61-79
+ *   x any strides (elements); y [M,N] e4m3fn contiguous; s [ceil(M/bm), ceil(N/bn)] fp32
+ *   absmax floored at 1e-10, multiply by the rounded reciprocal of the scale */
+int mq_fp8_blockwise_cast(const void* x, int dtype, int64_t stride_m, int64_t stride_n, void* y, float* s,
+                          int64_t M, int64_t N, int block_m, int block_n, void* stream);
+
+/* tensor_fp8 / channel_fp8                           tools/convert_hf_to_fp8.py:73-86
+ * and the per-tensor branch of the sync path         .../processors/quantizer_fp8.py:153-158
+ *   per_channel != 0: scale [M] (one per row); else scale [1]
+ *   floor_in_dtype: 1e-12 rounded to the weight dtype; amax_ws: >= max(M,1) uint32 of scratch */
+int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws, int64_t M,
+                        int64_t K, int per_channel, float floor_in_dtype, void* stream);
+
+/* weight_dequant(x, s, block_size)                   tools/fp8_cast_bf16.py:30-40
+ *   x [M,N] e4m3fn contiguous; s [ceil(M/block), ceil(N/block)] fp32; y [M,N] bf16 */
+int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block, void* stream);
+
+/* mxfp8_quantize(weight)                             miles/utils/mxfp8.py:51-78
+ *   w [rows,K] contiguous, K % 32 == 0; q [rows,K] e4m3fn; scale [rows,K/32] E8M0 bytes */
+int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K, void* stream);
+
+/* fake_int4_quant_cuda(x, (1, group), sym)           miles/kernels/quant/int4_fake/fake_int4_quant_cuda.cu:319-364
+ *   x [M,N] contiguous; out [M,N], scale [M,ceil(N/group)], zero (asym only) in the dtype of x */
+int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
+                       int group, int sym, void* stream);
+
+/* pack_layer(weight, group_size, sym=True)           .../processors/quantizer_compressed_tensors.py:235-265
+ *                                                    (== tools/convert_hf_to_int4_direct.py:121-151)
+ *   w [M,K] contiguous, K % group == 0, K % 8 == 0
+ *   packed [M,K/8] int32 (nibble i of word j = code of element 8j+i, code = q+8)
+ *   scale  [M,K/group] in the dtype of w */
+int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* scale, int64_t M, int64_t K,
+                             int group, void* stream);
+
+/* NVFP4                                              miles/utils/nvfp4.py:54-114
+ * mq_nvfp4_amax: amax_bits[0] = max(amax_bits[0], bits(max|w|)) -- clear it with mq_fill_u32 first; call it
+ * once per tensor of a gate/up pair to share one amax (nvfp4.py:100-103).
+ * mq_nvfp4_quant: w [M,K] contiguous, K % 16 == 0; q [M,K/2] (element 2i in the low nibble);
+ *   block_scale [M,K/16] e4m3fn bytes; global_scale (may be NULL) receives weight_scale_2 =
+ *   1 / min(e4m3_max*6/amax, FLT_MAX) as one fp32 (nvfp4.py:19-39). */
+int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream);
+int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* amax_bits, void* stream);
+int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, void* q, void* block_scale, float* global_scale,
+                   int64_t M, int64_t K, int e4m3_max, void* stream);
+
+/* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the
+ * software round-to-nearest-even forms over every fp32 bit pattern.  counts: 8 uint64 on the device
+ * (cleared by the call): [0] e4m3 mismatches for |x| <= 448, [1] NaN inputs whose e4m3 code is not
+ * 0x7F/0xFF, [2] e2m1 mismatches over all non-NaN inputs, [3] bf16 mismatches over all non-NaN
+ * inputs, [4] e4m3 decode mismatches (256 codes), [5] NaN inputs whose e2m1 code is not +-6,
+ * [6] inputs in (448, 464] whose e4m3 code is not +-448, [7] 1 if the packed e2m1 convert does not put
+ * its first operand in the low nibble.  The kernels rely on [0], [2], [3], [4], [7] being zero. */
+int mq_selftest_convert(uint64_t* counts, void* stream);
+
+/* Plain 16-byte-per-lane copy used to calibrate achievable HBM bandwidth and rocprof counters. */
+int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MILES_QUANT_H_ */

@@ -1,0 +1,54 @@
+"""Builds libmiles_quant.so (the C-ABI HIP library) for gfx950 with hipcc, in-tree.
+
+    python -m miles_amd.build
+
+-ffp-contract=off keeps every fp32 operation separately rounded (a fused multiply-add appears only
+where the source writes one); packed-fp32 instruction selection is switched off.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libmiles_quant.so")
+
+SOURCES = ["mq_core.hip", "mq_fp8_block.hip", "mq_mxfp8.hip", "mq_int4.hip", "mq_nvfp4.hip", "mq_selftest.hip",
+           "mq_sync.hip"]
+
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    "-ffp-contract=off",
+    "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+]
+
+
+def build(verbose: bool = False) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    cmd = ["hipcc", *FLAGS, "-o", LIB_PATH, *srcs]
+    if verbose:
+        print(" ".join(cmd))
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(line for line in proc.stdout.splitlines() if "is not a recognized feature" not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed:\n{out}")
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))
+    sys.exit(0)

@@ -1,0 +1,330 @@
+// FP8 e4m3 block-scale quantizers and the block dequantizer for gfx950.
+//
+//   mode 0  "block_fp8"          scale = amax/448 (true division), q = e4m3(clamp(w/scale)); an all-zero
+//                                tile has scale 0 and every byte 0xFF   (reference: tools/convert_hf_to_fp8.py:39-70)
+//   mode 1  "fp8_blockwise_cast" absmax = max(amax,1e-10), x_s = absmax/448, q = e4m3(clamp(x * (1/x_s)))
+//                                                                       (reference: miles/kernels/quant/fp8_blockwise.py:43-58)
+//   dequant y = bf16(float(q) * s[i/B][j/B])                            (reference: tools/fp8_cast_bf16.py:15-40)
+//
+// Fast path (bf16, 128x128 tiles, 16-byte aligned rows): one 256-lane workgroup owns one tile.  Lane t
+// loads eight 16-byte row segments (rows t/16 + 16 i, columns 8 (t%16) ..+8) so that sixteen lanes read one
+// contiguous 256-byte tile row; the 64 values stay in registers, the tile amax is reduced with DPP inside each
+// wavefront and through four LDS words across the wavefronts, and the tile is quantized from registers:
+// HBM traffic is one read of the input and one write of the codes and scale.
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+
+namespace mq {
+
+constexpr int kTile = 128;
+constexpr int kTileThreads = 256;
+constexpr int kRowsPerThread = 8;
+
+template <int MODE>
+__global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const uint16_t* __restrict__ w, int64_t ldw,
+                                                                    uint8_t* __restrict__ q, int64_t ldq,
+                                                                    float* __restrict__ scale, int64_t M, int64_t K,
+                                                                    int tiles_k) {
+    __shared__ uint32_t wave_amax[kTileThreads / kWave];
+    const int t = threadIdx.x;
+    const int64_t tile = blockIdx.x;
+    const int64_t ti = tile / tiles_k, tj = tile - ti * tiles_k;
+    const int64_t col = tj * kTile + (t & 15) * 8;
+    const int64_t row0 = ti * kTile + (t >> 4);
+    const bool col_ok = col < K;  // K % 8 == 0: an 8-wide segment is entirely inside or outside
+
+    u32x4 v[kRowsPerThread];
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; i++) {
+        const int64_t r = row0 + 16 * i;
+        v[i] = (col_ok && r < M) ? ld16(w + r * ldw + col) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; i++) {
+        m2 = max2_u16(m2, abs2(v[i].x));
+        m2 = max2_u16(m2, abs2(v[i].y));
+        m2 = max2_u16(m2, abs2(v[i].z));
+        m2 = max2_u16(m2, abs2(v[i].w));
+    }
+    uint32_t m = wave_max(hmax_u16(m2));
+    if ((t & (kWave - 1)) == 0) wave_amax[t >> 6] = m;
+    __syncthreads();
+    m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
+    const float amax = u2f(m << 16);
+
+    float s, y;
+    if (MODE == 0) {
+        s = amax / kFp8Max;
+        y = 1.0f / s;
+    } else {
+        const float absmax = amax > 1e-10f ? amax : 1e-10f;
+        s = absmax / kFp8Max;
+        y = 1.0f / s;
+    }
+    if (t == 0) scale[tile] = s;
+
+    if (MODE == 0 && !(amax > 0.0f) && amax == amax) {
+        // all-zero tile: 0/0 on every element; the reference's CPU result is the negative NaN code
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; i++) {
+            const int64_t r = row0 + 16 * i;
+            if (col_ok && r < M) st8(q + r * ldq + col, u32x2{0xFFFFFFFFu, 0xFFFFFFFFu});
+        }
+        return;
+    }
+    const bool fast_div = (MODE == 1) || shared_div_ok(s);
+
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; i++) {
+        const int64_t r = row0 + 16 * i;
+        float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                      bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            float x;
+            if (MODE == 1) x = f[j] * y;
+            else x = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
+            f[j] = __builtin_amdgcn_fmed3f(x, -kFp8Max, kFp8Max);
+        }
+        u32x2 o;
+        o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
+        o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
+        if (col_ok && r < M) st8(q + r * ldq + col, o);
+    }
+}
+
+// Any dtype, any strides, any block size: one workgroup per tile, two passes over the tile (the second
+// one is served by the caches).  Correctness path for shapes the fast kernel does not take.
+template <int MODE>
+__global__ __launch_bounds__(kTileThreads) void fp8_block_generic_kernel(const void* __restrict__ w, int dtype,
+                                                                         int64_t sxm, int64_t sxn,
+                                                                         uint8_t* __restrict__ q, int64_t ldq,
+                                                                         float* __restrict__ scale, int64_t M,
+                                                                         int64_t K, int bm, int bk, int tiles_k) {
+    __shared__ uint32_t wave_amax[kTileThreads / kWave];
+    const int t = threadIdx.x;
+    const int64_t tile = blockIdx.x;
+    const int64_t ti = tile / tiles_k, tj = tile - ti * tiles_k;
+    const int64_t r0 = ti * bm, c0 = tj * bk;
+    const int n = bm * bk;
+    uint32_t m = 0;
+    for (int idx = t; idx < n; idx += kTileThreads) {
+        const int64_t r = r0 + idx / bk, c = c0 + idx % bk;
+        if (r < M && c < K) m = umax(m, f2u(load_f32(w, r * sxm + c * sxn, dtype)) & 0x7FFFFFFFu);
+    }
+    m = wave_max(m);
+    if ((t & (kWave - 1)) == 0) wave_amax[t >> 6] = m;
+    __syncthreads();
+    m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
+    const float amax = u2f(m);
+    float s, y;
+    if (MODE == 0) {
+        s = amax / kFp8Max;
+        y = 0.0f;
+    } else {
+        const float absmax = amax > 1e-10f ? amax : 1e-10f;
+        s = absmax / kFp8Max;
+        y = 1.0f / s;
+    }
+    if (t == 0) scale[tile] = s;
+    const bool zero_tile = MODE == 0 && !(amax > 0.0f) && amax == amax;
+    for (int idx = t; idx < n; idx += kTileThreads) {
+        const int64_t r = r0 + idx / bk, c = c0 + idx % bk;
+        if (r < M && c < K) {
+            uint32_t code;
+            if (zero_tile) code = 0xFFu;
+            else {
+                const float x = load_f32(w, r * sxm + c * sxn, dtype);
+                float v = MODE == 1 ? x * y : x / s;
+                v = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+                code = sw_e4m3fn(v);
+            }
+            q[r * ldq + c] = (uint8_t)code;
+        }
+    }
+}
+
+// ---- per-tensor / per-channel (reference: tools/convert_hf_to_fp8.py:73-86,
+//      quantizer_fp8.py:153-158) ---------------------------------------------------------------
+// pass 1: amax per row (per_channel) or per tensor (atomic max on the float bit pattern)
+__global__ __launch_bounds__(256) void fp8_row_amax_kernel(const void* __restrict__ w, int dtype, int64_t ldw,
+                                                           int64_t K, uint32_t* __restrict__ amax_bits,
+                                                           int per_channel) {
+    __shared__ uint32_t wave_amax[4];
+    const int t = threadIdx.x;
+    const int64_t r = blockIdx.x;
+    uint32_t m = 0;
+    for (int64_t c = t; c < K; c += 256) m = umax(m, f2u(load_f32(w, r * ldw + c, dtype)) & 0x7FFFFFFFu);
+    m = wave_max(m);
+    if ((t & 63) == 0) wave_amax[t >> 6] = m;
+    __syncthreads();
+    if (t == 0) {
+        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
+        if (per_channel) amax_bits[r] = m;
+        else atomicMax(amax_bits, m);
+    }
+}
+// pass 2: scale = max(amax, floor)/448 ; q = e4m3(clamp(w/scale)).  With one scale for the whole
+// tensor the quotient is first rounded to the weight's dtype (torch keeps `weight / zero_dim_scale`
+// in the weight's dtype).
+__global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restrict__ w, int dtype, int64_t ldw,
+                                                            int64_t K, const uint32_t* __restrict__ amax_bits,
+                                                            float floor_v, int per_channel,
+                                                            uint8_t* __restrict__ q, float* __restrict__ scale) {
+    const int t = threadIdx.x;
+    const int64_t r = blockIdx.x;
+    float amax = u2f(per_channel ? amax_bits[r] : amax_bits[0]);
+    if (amax < floor_v) amax = floor_v;
+    const float s = amax / kFp8Max;
+    if (t == 0 && (per_channel || r == 0)) scale[per_channel ? r : 0] = s;
+    for (int64_t c = t; c < K; c += 256) {
+        float v = load_f32(w, r * ldw + c, dtype) / s;
+        if (!per_channel) v = round_to_dtype(v, dtype);
+        v = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+        q[r * K + c] = (uint8_t)sw_e4m3fn(v);
+    }
+}
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// ---- dequant ----------------------------------------------------------------------------------
+// Fast path: N % 16 == 0, block % 16 == 0, 16-byte aligned.  Each lane turns 16 codes (one 16-byte load)
+// into 16 bf16 (two 16-byte stores); a wavefront covers 1 KiB of codes.
+__global__ __launch_bounds__(256) void fp8_dequant_kernel(const uint8_t* __restrict__ x, const float* __restrict__ s,
+                                                          uint16_t* __restrict__ y, int64_t M, int64_t N, int block,
+                                                          int tiles_n, int64_t chunks_per_row, int64_t total_chunks) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < total_chunks; ch += stride) {
+        const int64_t r = ch / chunks_per_row;
+        const int64_t c = (ch - r * chunks_per_row) * 16;
+        const u32x4 in = ld16(x + r * N + c);
+        const float sc = s[(r / block) * tiles_n + c / block];
+        const uint32_t wd[4] = {in.x, in.y, in.z, in.w};
+        uint32_t o[8];
+        // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0
+        bool special = (f2u(sc) & 0x7F800000u) == 0x7F800000u;
+#pragma unroll
+        for (int k = 0; k < 4; k++) special |= (((wd[k] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u) != 0u;
+        if (!special) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const f32x2 a = hw_e4m3x2_decode<false>(wd[k]);
+                const f32x2 b = hw_e4m3x2_decode<true>(wd[k]);
+                o[2 * k] = hw_bf16x2(a.x * sc, a.y * sc);
+                o[2 * k + 1] = hw_bf16x2(b.x * sc, b.y * sc);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                uint32_t h[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) h[b] = sw_bf16(sw_e4m3fn_decode((wd[k] >> (8 * b)) & 0xFFu) * sc);
+                o[2 * k] = h[0] | (h[1] << 16);
+                o[2 * k + 1] = h[2] | (h[3] << 16);
+            }
+        }
+        uint16_t* dst = y + r * N + c;
+        st16(dst, u32x4{o[0], o[1], o[2], o[3]});
+        st16(dst + 8, u32x4{o[4], o[5], o[6], o[7]});
+    }
+}
+
+__global__ __launch_bounds__(256) void fp8_dequant_generic_kernel(const uint8_t* __restrict__ x,
+                                                                  const float* __restrict__ s,
+                                                                  uint16_t* __restrict__ y, int64_t M, int64_t N,
+                                                                  int block, int tiles_n) {
+    const int64_t total = M * N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / N, c = i - r * N;
+        y[i] = (uint16_t)sw_bf16(sw_e4m3fn_decode(x[i]) * s[(r / block) * tiles_n + c / block]);
+    }
+}
+
+}  // namespace mq
+
+using namespace mq;
+
+static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int64_t sxn, void* q, float* scale,
+                            int64_t M, int64_t K, int bm, int bk, hipStream_t stream) {
+    if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (M < 0 || K < 0 || bm <= 0 || bk <= 0) return mq_fail(MQ_ERR_ARG, "bad shape or block size");
+    if (dtype < MQ_BF16 || dtype > MQ_F32) return mq_fail(MQ_ERR_ARG, "unsupported dtype");
+    if (M == 0 || K == 0) return MQ_OK;
+    const int64_t tiles_m = (M + bm - 1) / bm, tiles_k = (K + bk - 1) / bk;
+    const int64_t tiles = tiles_m * tiles_k;
+    if (tiles > 0x7FFFFFFF || tiles_k > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
+    const bool fast = dtype == MQ_BF16 && bm == kTile && bk == kTile && sxn == 1 && (K % 8) == 0 && (sxm % 8) == 0 &&
+                      ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
+    dim3 grid((unsigned)tiles), blk(kTileThreads);
+    if (fast) {
+        if (mode == 0)
+            hipLaunchKernelGGL(fp8_block128_kernel<0>, grid, blk, 0, stream, (const uint16_t*)w, sxm, (uint8_t*)q, K,
+                               scale, M, K, (int)tiles_k);
+        else
+            hipLaunchKernelGGL(fp8_block128_kernel<1>, grid, blk, 0, stream, (const uint16_t*)w, sxm, (uint8_t*)q, K,
+                               scale, M, K, (int)tiles_k);
+    } else {
+        if ((int64_t)bm * bk > (1 << 24)) return mq_fail(MQ_ERR_ARG, "block too large");
+        if (mode == 0)
+            hipLaunchKernelGGL(fp8_block_generic_kernel<0>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K,
+                               scale, M, K, bm, bk, (int)tiles_k);
+        else
+            hipLaunchKernelGGL(fp8_block_generic_kernel<1>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K,
+                               scale, M, K, bm, bk, (int)tiles_k);
+    }
+    return mq_check_launch("fp8 block quant");
+}
+
+extern "C" int mq_fp8_block_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
+                                  int block_m, int block_k, void* stream) {
+    return fp8_block_launch(0, w, dtype, ldw, 1, q, scale, M, K, block_m, block_k, (hipStream_t)stream);
+}
+
+extern "C" int mq_fp8_blockwise_cast(const void* x, int dtype, int64_t stride_m, int64_t stride_n, void* y, float* s,
+                                     int64_t M, int64_t N, int block_m, int block_n, void* stream) {
+    return fp8_block_launch(1, x, dtype, stride_m, stride_n, y, s, M, N, block_m, block_n, (hipStream_t)stream);
+}
+
+extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws,
+                                   int64_t M, int64_t K, int per_channel, float floor_in_dtype, void* stream) {
+    if (!w || !q || !scale || !amax_ws) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (M == 0 || K == 0) return MQ_OK;
+    if (M > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    if (!per_channel) hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)amax_ws, 0u, 1);
+    hipLaunchKernelGGL(fp8_row_amax_kernel, dim3((unsigned)M), dim3(256), 0, st, w, dtype, ldw, K,
+                       (uint32_t*)amax_ws, per_channel);
+    hipLaunchKernelGGL(fp8_row_quant_kernel, dim3((unsigned)M), dim3(256), 0, st, w, dtype, ldw, K,
+                       (const uint32_t*)amax_ws, floor_in_dtype, per_channel, (uint8_t*)q, scale);
+    return mq_check_launch("fp8 scaled quant");
+}
+
+extern "C" int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block,
+                                    void* stream) {
+    if (!x || !s || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (M < 0 || N < 0 || block <= 0) return mq_fail(MQ_ERR_ARG, "bad shape or block size");
+    if (M == 0 || N == 0) return MQ_OK;
+    const int64_t tiles_n = (N + block - 1) / block;
+    if (tiles_n > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
+    hipStream_t st = (hipStream_t)stream;
+    const bool fast = (N % 16) == 0 && (block % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0;
+    if (fast) {
+        const int64_t cpr = N / 16, total = M * cpr;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+        hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint8_t*)x, s,
+                           (uint16_t*)y, M, N, block, (int)tiles_n, cpr, total);
+    } else {
+        int64_t blocks = (M * N + 255) / 256;
+        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+        hipLaunchKernelGGL(fp8_dequant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint8_t*)x, s,
+                           (uint16_t*)y, M, N, block, (int)tiles_n);
+    }
+    return mq_check_launch("fp8 block dequant");
+}

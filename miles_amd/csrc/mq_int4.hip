@@ -1,0 +1,200 @@
+// INT4 group quantization for gfx950.
+//
+//  mq_int4_fake_quant       restates fake_int4_quant_cuda for block (1, G)
+//                           (reference: miles/kernels/quant/int4_fake/fake_int4_quant_cuda.cu:29-91,159-259):
+//                             sym : scale = fmaxf(amax*(1/7), 1e-5);  out = rintf(x/scale)
+//                             asym: scale = fmaxf((max-min)*(1/15), 1e-5); zero = clamp(-rintf(min/scale),0,15);
+//                                   out = rintf(x/scale) + zero
+//                           out / scale / zero are stored in the dtype of x.
+//  mq_int4_group_quant_pack fuses the symmetric kernel with pack_layer's Python half
+//                           (reference: .../processors/quantizer_compressed_tensors.py:137-265):
+//                           code = rintf(x/scale_f32) + 8 in [1,15]; eight codes per int32, element 8j+i in bits
+//                           4i..4i+3; scale stored as bf16.  The bf16 round trip that pack_layer performs
+//                           (w = q*scale_b, q' = round(w/scale_b)) returns q for every |q| <= 7 and every scale
+//                           below 4.8e37, so the codes come straight from the fp32 quotient.
+//
+// Packed fast path (bf16, G = 8 * LANES): LANES lanes own one group, 16 bytes each; the group amax is a DPP
+// max over the LANES-lane segment; x/scale uses the shared-divisor sequence (3 FMA-class ops per element,
+// exactly rounded) and rint + the +8 offset are one fp32 add of 1.5*2^23 + 8.
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+
+namespace mq {
+
+constexpr float kSymCons = 1.0f / 7.0f;
+constexpr float kAsymCons = 1.0f / 15.0f;
+constexpr int kI4Threads = 256;
+constexpr int kI4Unroll = 4;
+
+template <int LANES>
+__device__ __forceinline__ uint32_t seg_max(uint32_t v) {
+    if (LANES == 16) return group_max16(v);
+    if (LANES == 8) return group_max8(v);
+    if (LANES == 4) return group_max4(v);
+    if (LANES == 2) return group_max2(v);
+    return v;
+}
+
+// nibble = (rint(q) + 8) & 15 taken from the low bits of q + (1.5*2^23 + 8)
+__device__ __forceinline__ uint32_t code_bits(float q) { return f2u(q + 12582920.0f); }
+
+template <int LANES>
+__global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const uint16_t* __restrict__ w,
+                                                                    uint32_t* __restrict__ packed,
+                                                                    uint16_t* __restrict__ scale, int64_t total_units) {
+    const int t = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll);
+    u32x4 v[kI4Unroll];
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads + t;
+        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads + t;
+        const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
+        const uint32_t mb = seg_max<LANES>(hmax_u16(m2));
+        const float amax = u2f(mb << 16);
+        const float s = __builtin_fmaxf(amax * kSymCons, 1e-5f);
+        const float y = 1.0f / s;
+        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const bool fast = shared_div_ok(s);
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float qv = fast ? div_by_shared(f[j], s, y) : f[j] / s;
+            word |= (code_bits(qv) & 0xFu) << (4 * j);
+        }
+        if (unit < total_units) {
+            packed[unit] = word;
+            if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
+        }
+    }
+}
+
+// One wavefront per group, lanes stride the columns: any dtype, any G, ragged last group, sym and asym.
+// PACK: additionally emit the packed int32 words (sym only, G % 8 == 0 handled by the caller).
+__global__ __launch_bounds__(256) void int4_fake_generic_kernel(const void* __restrict__ x, int dtype,
+                                                                void* __restrict__ out, void* __restrict__ scale_out,
+                                                                void* __restrict__ zero_out, int64_t M, int64_t N,
+                                                                int G, int64_t groups_per_row, int sym) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int64_t total = M * groups_per_row;
+    for (int64_t g = wave; g < total; g += nwaves) {
+        const int64_t r = g / groups_per_row, j = g - r * groups_per_row;
+        const int64_t c0 = j * G;
+        float mx = -__builtin_inff(), mn = __builtin_inff();
+        for (int k = lane; k < G; k += 64) {
+            const int64_t c = c0 + k;
+            const float val = c < N ? load_f32(x, r * N + c, dtype) : 0.0f;
+            if (sym) mx = __builtin_fmaxf(mx, __builtin_fabsf(val));
+            else { mx = __builtin_fmaxf(mx, val); mn = __builtin_fminf(mn, val); }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+        }
+        float s, zero = 0.0f;
+        if (sym) s = __builtin_fmaxf(mx * kSymCons, 1e-5f);
+        else {
+            s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
+            zero = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f);
+        }
+        for (int k = lane; k < G; k += 64) {
+            const int64_t c = c0 + k;
+            if (c < N) {
+                float qv = __builtin_rintf(load_f32(x, r * N + c, dtype) / s);
+                if (!sym) qv = qv + zero;
+                store_dtype(out, r * N + c, qv, dtype);
+            }
+        }
+        if (lane == 0) {
+            store_dtype(scale_out, g, s, dtype);
+            if (!sym) store_dtype(zero_out, g, zero, dtype);
+        }
+    }
+}
+
+// pack_layer for dtypes / group sizes the fast kernel does not take: follows the reference chain literally,
+// one lane per packed word.
+__global__ __launch_bounds__(256) void int4_pack_generic_kernel(const void* __restrict__ w, int dtype,
+                                                                uint32_t* __restrict__ packed,
+                                                                void* __restrict__ scale_out, int64_t M, int64_t K,
+                                                                int G) {
+    const int64_t words_per_row = K / 8, total = M * words_per_row, gpr = K / G;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / words_per_row, j = i - r * words_per_row;
+        uint32_t word = 0;
+        for (int k = 0; k < 8; k++) {
+            const int64_t c = j * 8 + k;
+            const int64_t g0 = (c / G) * G;
+            float amax = -__builtin_inff();
+            for (int e = 0; e < G; e++) amax = __builtin_fmaxf(amax, __builtin_fabsf(load_f32(w, r * K + g0 + e, dtype)));
+            const float s = __builtin_fmaxf(amax * kSymCons, 1e-5f);
+            const float q0 = round_to_dtype(__builtin_rintf(load_f32(w, r * K + c, dtype) / s), dtype);
+            const float sb = round_to_dtype(s, dtype);
+            const float wv = round_to_dtype(q0 * sb, dtype);
+            float rv = round_to_dtype(wv / sb, dtype);
+            rv = __builtin_fminf(__builtin_fmaxf(rv, -128.0f), 127.0f);
+            const int qi = (int)__builtin_rintf(rv);
+            word += (uint32_t)((qi + 8) & 0xFF) << (4 * k);
+            if (c == g0) store_dtype(scale_out, r * gpr + c / G, s, dtype);
+        }
+        packed[i] = word;
+    }
+}
+
+}  // namespace mq
+
+using namespace mq;
+
+extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
+                                  int group, int sym, void* stream) {
+    if (!x || !out || !scale || (!sym && !zero)) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || N < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (group % 32 != 0) return mq_fail(MQ_ERR_ARG, "block_m * block_n must be divisible by 32");
+    if (M == 0 || N == 0) return MQ_OK;
+    const int64_t gpr = (N + group - 1) / group;
+    const int64_t waves = M * gpr;
+    int64_t blocks = (waves + 3) / 4;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(int4_fake_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, dtype,
+                       out, scale, zero, M, N, group, gpr, sym);
+    return mq_check_launch("int4 fake quant");
+}
+
+extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* scale, int64_t M, int64_t K,
+                                        int group, void* stream) {
+    if (!w || !packed || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (K % group != 0 || K % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and of 8");
+    if (M == 0 || K == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const bool aligned = dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0;
+    const int64_t units = M * (K / 8);
+    const int64_t per_block = kI4Threads * kI4Unroll;
+    const int64_t fblocks = (units + per_block - 1) / per_block;
+    if (fblocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    dim3 grid((unsigned)fblocks), blk(kI4Threads);
+    if (aligned && group == 128)
+        hipLaunchKernelGGL(int4_pack_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
+                           (uint16_t*)scale, units);
+    else if (aligned && group == 64)
+        hipLaunchKernelGGL(int4_pack_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
+                           (uint16_t*)scale, units);
+    else if (aligned && group == 32)
+        hipLaunchKernelGGL(int4_pack_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
+                           (uint16_t*)scale, units);
+    else {
+        int64_t blocks = (units + 255) / 256;
+        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+        hipLaunchKernelGGL(int4_pack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype,
+                           (uint32_t*)packed, scale, M, K, group);
+    }
+    return mq_check_launch("int4 pack");
+}

@@ -1,0 +1,113 @@
+// MXFP8 (e4m3 codes, one E8M0 scale per 1x32 group along K) for gfx950.
+// Reference: miles/utils/mxfp8.py:51-78 (layout: compact row-major scales [rows, K/32]); the arithmetic is
+// Transformer Engine's rowwise MXFP8 quantizer:
+//   amax = max|x| over the group; e = ceil_pow2_exponent(amax * f32(1/448)) (saturating at 0xFE, 0 for amax 0);
+//   q = sat_e4m3(x * 2^(127-e)).
+//
+// The tensor is a flat run of groups.  Four lanes own one group (8 bf16 = 16 bytes each), so a wavefront
+// reads 1 KiB of consecutive input per load instruction; the group amax is a two-step DPP max inside the
+// quad.  Scaling by a power of two is exact, so the only rounding is the e4m3 conversion.
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+
+namespace mq {
+
+constexpr int kMxThreads = 256;
+constexpr int kMxUnroll = 4;  // 16-byte units per lane per workgroup pass
+
+__device__ __forceinline__ uint32_t e8m0_ceil(float v) {
+    const uint32_t u = f2u(v);
+    uint32_t e = u >> 23, m = u & 0x7FFFFFu;
+    if (u >= 0x7F800000u) return u == 0x7F800000u ? 0xFEu : 0xFFu;
+    if ((m > 0 && e != 0xFEu) && !(e == 0 && m <= 0x400000u)) e++;
+    return e;
+}
+__device__ __forceinline__ float e8m0_inverse(uint32_t e) {
+    if (e == 0) return 1.0f;
+    if (e >= 254) return u2f(e == 254 ? 0x00400000u : 0x00200000u);
+    return u2f((254u - e) << 23);
+}
+
+__global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ q,
+                                                                uint8_t* __restrict__ scale, int64_t total_units) {
+    const float inv448 = u2f(0x3B124925u);
+    const int t = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kMxThreads * kMxUnroll);
+    u32x4 v[kMxUnroll];
+#pragma unroll
+    for (int i = 0; i < kMxUnroll; i++) {
+        const int64_t unit = base + i * kMxThreads + t;
+        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < kMxUnroll; i++) {
+        const int64_t unit = base + i * kMxThreads + t;
+        uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
+        const uint32_t mb = group_max4(hmax_u16(m2));   // bf16 pattern of the group amax, quad-uniform
+        const float amax = u2f(mb << 16);
+        const uint32_t e = e8m0_ceil(amax * inv448);
+        const float inv = e8m0_inverse(e);
+        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        u32x2 o;
+        if (mb < 0x7F80u) {
+            // finite group: |x * inv| <= 448 by construction, no clamp needed
+            o.x = hw_e4m3x4(f[0] * inv, f[1] * inv, f[2] * inv, f[3] * inv);
+            o.y = hw_e4m3x4(f[4] * inv, f[5] * inv, f[6] * inv, f[7] * inv);
+        } else {
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn_sat(f[j] * inv);
+            o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+        }
+        if (unit < total_units) {
+            st8(q + unit * 8, o);
+            if ((t & 3) == 0) scale[unit >> 2] = (uint8_t)e;
+        }
+    }
+}
+
+// any dtype: one lane per group
+__global__ __launch_bounds__(256) void mxfp8_generic_kernel(const void* __restrict__ w, int dtype,
+                                                            uint8_t* __restrict__ q, uint8_t* __restrict__ scale,
+                                                            int64_t groups) {
+    const float inv448 = u2f(0x3B124925u);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups; g += stride) {
+        uint32_t m = 0;
+        for (int j = 0; j < 32; j++) m = umax(m, f2u(load_f32(w, g * 32 + j, dtype)) & 0x7FFFFFFFu);
+        const uint32_t e = e8m0_ceil(u2f(m) * inv448);
+        const float inv = e8m0_inverse(e);
+        scale[g] = (uint8_t)e;
+        for (int j = 0; j < 32; j++) q[g * 32 + j] = (uint8_t)sw_e4m3fn_sat(load_f32(w, g * 32 + j, dtype) * inv);
+    }
+}
+
+}  // namespace mq
+
+using namespace mq;
+
+extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K,
+                              void* stream) {
+    if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || rows < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (K % 32 != 0) return mq_fail(MQ_ERR_ARG, "Last dim must be divisible by 32 for MXFP8.");
+    if (rows == 0 || K == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t groups = rows * (K / 32);
+    if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0) {
+        const int64_t units = groups * 4;
+        const int64_t per_block = kMxThreads * kMxUnroll;
+        const int64_t blocks = (units + per_block - 1) / per_block;
+        if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+        hipLaunchKernelGGL(mxfp8_bf16_kernel, dim3((unsigned)blocks), dim3(kMxThreads), 0, st, (const uint16_t*)w,
+                           (uint8_t*)q, scale, units);
+    } else {
+        int64_t blocks = (groups + 255) / 256;
+        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+        hipLaunchKernelGGL(mxfp8_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (uint8_t*)q, scale,
+                           groups);
+    }
+    return mq_check_launch("mxfp8 quant");
+}

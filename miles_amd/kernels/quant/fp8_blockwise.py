@@ -1,0 +1,37 @@
+"""FP8 e4m3 block-scale cast used on the weight-sync path.
+
+Same call as the reference's `miles.kernels.quant.fp8_blockwise.fp8_blockwise_cast`
+(miles/kernels/quant/fp8_blockwise.py:61-79); the Triton kernel there (:24-58) is replaced by the
+gfx950 kernel behind `mq_fp8_blockwise_cast`.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from miles_amd import _lib
+
+fp8_dtype = torch.float8_e4m3fn
+fp8_max = torch.finfo(fp8_dtype).max
+fp8_min = -fp8_max
+
+
+def ceil_div(x: int, y: int) -> int:
+    return -(-x // y)
+
+
+def fp8_blockwise_cast(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, torch.Tensor]:
+    """x [M, N] (any strides) -> (float8_e4m3fn [M, N] contiguous, float32 [ceil(M/bm), ceil(N/bn)]).
+
+    Per tile: absmax = max(max|x|, 1e-10); scale = absmax / 448; y = e4m3(clamp(x * (1 / scale), +-448)).
+    """
+    bm, bn = (128, 128) if not block_size else (int(block_size[0]), int(block_size[1]))
+    _lib.require_gpu(x, "fp8_blockwise_cast")
+    M, N = x.shape
+    y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
+    s = torch.empty(ceil_div(M, bm), ceil_div(N, bn), dtype=torch.float32, device=x.device)
+    rc = _lib.load().mq_fp8_blockwise_cast(x.data_ptr(), _lib.dtype_code(x, "fp8_blockwise_cast"), x.stride(0),
+                                           x.stride(1), y.data_ptr(), s.data_ptr(), M, N, bm, bn,
+                                           _lib.stream_ptr(x.device))
+    _lib.check(rc)
+    return y, s

@@ -1,0 +1,54 @@
+"""MXFP8 (e4m3 + 1x32 E8M0) weight quantization.
+
+Mirror of the reference's `miles/utils/mxfp8.py` (constants :4-25, `should_use_mxfp8` :27-48,
+`mxfp8_quantize` :51-78).  The reference pads rows to a multiple of 32 for Transformer Engine and crops
+the swizzle-padded scale buffer afterwards; groups are row-local, so the gfx950 kernel writes the compact
+[..., K/32] scale tensor directly and needs neither.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from miles_amd import _lib
+
+MXFP8_GROUP_SIZE = 32
+
+MXFP8_SKIP_WEIGHT_SUBSTRINGS = (
+    "layernorm", "embed", "router", "mlp.gate.", "norm", "lm_head", "eh_proj", "weights_proj", "head.", "wo_a",
+    "ffn.gate.", "compressor.",
+)
+
+MXFP8_SOURCE_FP8_DTYPES = (torch.float8_e4m3fn,) + (
+    (torch.float8_e4m3fnuz,) if hasattr(torch, "float8_e4m3fnuz") else ()
+)
+
+
+def should_use_mxfp8(name: str, shape: tuple[int, ...], dtype: torch.dtype, *,
+                     skip_substrings: tuple[str, ...] = MXFP8_SKIP_WEIGHT_SUBSTRINGS,
+                     allow_source_fp8: bool = False, packed_mxfp4_experts: bool = False) -> bool:
+    """Whether a checkpoint tensor is stored as MXFP8 in the rollout layout."""
+    if not name.endswith(".weight"):
+        return False
+    if any(s in name for s in skip_substrings) or len(shape) < 2:
+        return False
+    if packed_mxfp4_experts:
+        return (2 * shape[-1]) % MXFP8_GROUP_SIZE == 0  # two e2m1 weights per stored byte
+    ok_dtypes = (torch.float16, torch.bfloat16, torch.float32) + (MXFP8_SOURCE_FP8_DTYPES if allow_source_fp8 else ())
+    return dtype in ok_dtypes and shape[-1] % MXFP8_GROUP_SIZE == 0
+
+
+def mxfp8_quantize(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """weight [..., K] -> (float8_e4m3fn, same shape; uint8 E8M0 scales [..., K/32], compact, unswizzled)."""
+    k = weight.shape[-1]
+    if k % MXFP8_GROUP_SIZE != 0:
+        raise ValueError(f"Last dim {k} must be divisible by {MXFP8_GROUP_SIZE} for MXFP8.")
+    _lib.require_gpu(weight, "mxfp8_quantize")
+    w = weight.contiguous()
+    rows = w.numel() // k if k else 0
+    q = torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=w.device)
+    scale = torch.empty((*w.shape[:-1], k // MXFP8_GROUP_SIZE), dtype=torch.uint8, device=w.device)
+    rc = _lib.load().mq_mxfp8_quant(w.data_ptr(), _lib.dtype_code(w, "mxfp8_quantize"), q.data_ptr(),
+                                    scale.data_ptr(), rows, k, _lib.stream_ptr(w.device))
+    _lib.check(rc)
+    return q, scale

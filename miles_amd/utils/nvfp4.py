@@ -1,0 +1,103 @@
+"""NVFP4 (e2m1 + 1x16 e4m3 block scales + fp32 global scale) weight quantization.
+
+Mirror of the reference's `miles/utils/nvfp4.py`: `nvfp4_weight_e4m3_max` (:11-16), the global scale closed
+forms (:19-39), `nvfp4_quantize_1d` (:54-82) and `nvfp4_quantize_1d_pair` (:85-114).  Transformer Engine's
+quantizer is replaced by the two gfx950 passes `mq_nvfp4_amax` / `mq_nvfp4_quant`; the global amax never
+leaves the device, and a gate/up pair shares it by reducing both tensors into the same word instead of
+concatenating them.
+"""
+
+from __future__ import annotations
+
+import os
+
+import torch
+
+from miles_amd import _lib
+
+FP4_E2M1_MAX = 6.0
+FP8_E4M3_MAX = 448.0
+NVFP4_GROUP_SIZE = 16
+
+
+def nvfp4_weight_e4m3_max() -> int:
+    four_over_six = os.getenv("NVTE_NVFP4_4OVER6", "").strip().lower() in ("weights", "all")
+    use_256 = os.getenv("NVTE_NVFP4_4OVER6_E4M3_USE_256", "all").strip().lower() in ("weights", "all")
+    return 256 if four_over_six and use_256 else int(FP8_E4M3_MAX)
+
+
+def _nvfp4_4over6_enabled() -> bool:
+    return os.getenv("NVTE_NVFP4_4OVER6", "").strip().lower() in ("weights", "all")
+
+
+def nvfp4_global_encode_scale_te(global_amax: torch.Tensor, nvfp4_e4m3_max: int = int(FP8_E4M3_MAX)) -> torch.Tensor:
+    """min(e4m3_max * 6 / amax, FLT_MAX), with an exact zero repaired to 1; no host read of the amax."""
+    enc = torch.div(float(nvfp4_e4m3_max) * FP4_E2M1_MAX, global_amax.to(torch.float32))
+    enc = enc.clamp_max(torch.finfo(torch.float32).max)
+    return torch.where(enc == 0.0, 1.0, enc)
+
+
+def nvfp4_global_decode_scale_te(global_amax: torch.Tensor, nvfp4_e4m3_max: int = int(FP8_E4M3_MAX)) -> torch.Tensor:
+    return torch.div(1.0, nvfp4_global_encode_scale_te(global_amax, nvfp4_e4m3_max))
+
+
+def _check_supported() -> int:
+    if _nvfp4_4over6_enabled():
+        raise NotImplementedError("NVTE_NVFP4_4OVER6 (four-over-six block scaling) is not implemented on gfx950")
+    return nvfp4_weight_e4m3_max()
+
+
+def _amax_word(device) -> torch.Tensor:
+    word = torch.empty(1, dtype=torch.int32, device=device)
+    _lib.check(_lib.load().mq_fill_u32(word.data_ptr(), 0, 1, _lib.stream_ptr(device)))
+    return word
+
+
+def _reduce_amax(word: torch.Tensor, w: torch.Tensor) -> None:
+    rc = _lib.load().mq_nvfp4_amax(w.data_ptr(), _lib.dtype_code(w, "nvfp4"), w.numel(), word.data_ptr(),
+                                   _lib.stream_ptr(w.device))
+    _lib.check(rc)
+
+
+def _quantize_with_amax(w: torch.Tensor, word: torch.Tensor, e4m3_max: int):
+    rows, cols = w.shape
+    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+    block_scale = torch.empty((rows, cols // NVFP4_GROUP_SIZE), dtype=torch.float8_e4m3fn, device=w.device)
+    global_scale = torch.empty((), dtype=torch.float32, device=w.device)
+    rc = _lib.load().mq_nvfp4_quant(w.data_ptr(), _lib.dtype_code(w, "nvfp4"), word.data_ptr(), q.data_ptr(),
+                                    block_scale.data_ptr(), global_scale.data_ptr(), rows, cols, e4m3_max,
+                                    _lib.stream_ptr(w.device))
+    _lib.check(rc)
+    return q, block_scale, global_scale
+
+
+def nvfp4_quantize_1d(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """weight [M, K] -> (uint8 [M, K/2], float8_e4m3fn [M, K/16], float32 [] = weight_scale_2)."""
+    _lib.require_gpu(weight, "nvfp4_quantize_1d")
+    e4m3_max = _check_supported()
+    w = weight.contiguous()
+    if w.shape[1] % NVFP4_GROUP_SIZE != 0:
+        raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {w.shape[1]}.")
+    word = _amax_word(w.device)
+    _reduce_amax(word, w)
+    return _quantize_with_amax(w, word, e4m3_max)
+
+
+def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
+    """Quantize a gate/up pair with ONE global amax taken over both tensors."""
+    if first.dim() != 2 or second.dim() != 2:
+        raise ValueError("nvfp4_quantize_1d_pair expects two 2D tensors.")
+    if first.shape[1] != second.shape[1]:
+        raise ValueError(
+            f"NVFP4 paired quantization requires matching K dimensions, got {first.shape[1]} and {second.shape[1]}."
+        )
+    _lib.require_gpu(first, "nvfp4_quantize_1d_pair")
+    _lib.require_gpu(second, "nvfp4_quantize_1d_pair")
+    e4m3_max = _check_supported()
+    a, b = first.contiguous(), second.contiguous()
+    if a.shape[1] % NVFP4_GROUP_SIZE != 0:
+        raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {a.shape[1]}.")
+    word = _amax_word(a.device)
+    _reduce_amax(word, a)
+    _reduce_amax(word, b)
+    return _quantize_with_amax(a, word, e4m3_max), _quantize_with_amax(b, word, e4m3_max)

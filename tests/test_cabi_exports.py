@@ -1,0 +1,52 @@
+"""The C-ABI library loads and exports every symbol include/miles_quant.h declares (no GPU needed)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "miles_quant.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = _declared_symbols()
+    for required in ["mq_fp8_block_quant", "mq_fp8_blockwise_cast", "mq_fp8_block_dequant", "mq_mxfp8_quant",
+                     "mq_int4_group_quant_pack", "mq_int4_fake_quant", "mq_nvfp4_amax", "mq_nvfp4_quant"]:
+        assert required in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from miles_amd import _lib
+
+    if not os.path.exists(_lib.lib_path()):
+        pytest.fail(f"{_lib.lib_path()} not built: run `python -m miles_amd.build`")
+    lib = ctypes.CDLL(_lib.lib_path())
+    missing = [s for s in _declared_symbols() if not hasattr(lib, s)]
+    assert not missing, f"declared in miles_quant.h but not exported: {missing}"
+    assert _lib.load().mq_version() == 1
+    # the ctypes signature table covers every declared compute entry point
+    declared = set(_declared_symbols()) - {"mq_version", "mq_last_error"}
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+
+
+def test_wrappers_refuse_cpu_tensors():
+    import torch
+
+    from miles_amd import _lib
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    w = torch.zeros(32, 64, dtype=torch.bfloat16)
+    for fn, args in [(block_fp8, (w, [128, 128])), (fp8_blockwise_cast, (w,)), (mxfp8_quantize, (w,)),
+                     (nvfp4_quantize_1d, (w,))]:
+        with pytest.raises(_lib.MilesQuantError, match="GPU"):
+            fn(*args)

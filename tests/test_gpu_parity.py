@@ -1,0 +1,407 @@
+"""GPU parity: every entry point of libmiles_quant.so, called through the reference-shaped Python wrappers
+(ctypes -> C ABI), against the CPU oracle on the same seeded inputs.  Bit-exact everywhere: codes, scales,
+packed words; dequant 0 ULP in bf16.
+"""
+
+import pytest
+import torch
+
+from miles_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+F8 = torch.float8_e4m3fn
+DEV = "cuda:0"
+
+
+def _u8(t):
+    return t.detach().cpu().contiguous().view(torch.uint8)
+
+
+def _bits(t):
+    t = t.detach().cpu().contiguous()
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32}[t.element_size()])
+
+
+def _assert_same(got, want, what):
+    g, w = _bits(got), _bits(want)
+    assert g.shape == w.shape, f"{what}: shape {tuple(g.shape)} vs {tuple(w.shape)}"
+    if not torch.equal(g, w):
+        bad = (g != w).nonzero()
+        i = tuple(bad[0].tolist())
+        raise AssertionError(f"{what}: {bad.shape[0]} of {g.numel()} differ; first at {i}: got {g[i].item()} want {w[i].item()}")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from miles_amd import _lib
+
+    return _lib.load()
+
+
+# ---------------------------------------------------------------------------------------------------
+def test_hardware_converts_agree_with_software_rne(lib):
+    counts = torch.zeros(16, dtype=torch.int64, device=DEV)
+    assert lib.mq_selftest_convert(counts.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    c = counts.cpu().tolist()
+    print("selftest counts", c[:8])
+    assert c[0] == 0, "v_cvt_pk_fp8_f32 differs from RNE e4m3fn inside +-448"
+    assert c[2] == 0, "v_cvt_scalef32_pk_fp4_f32 differs from RNE satfinite e2m1"
+    assert c[3] == 0, "f32->bf16 convert differs from RNE"
+    assert c[4] == 0, "v_cvt_pk_f32_fp8 decode table differs"
+    assert c[7] == 0, "packed e2m1 convert nibble order"
+
+
+# ---------------------------------------------------------------------------------------------------
+FP8_SHAPES = W.SMALL_REFERENCE_SHAPES + [(130, 264), (1, 8), (127, 136), (200, 1000), (5, 3)]
+
+
+@pytest.mark.parametrize("shape", FP8_SHAPES)
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_block_fp8(oracle, shape, kind):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    w = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    q, s = block_fp8(w.to(DEV), [128, 128])
+    q_o, s_o = oracle.block_fp8(w, (128, 128))
+    assert q.dtype == F8 and s.dtype == torch.float32 and q.is_contiguous()
+    _assert_same(s, s_o, "scale")
+    _assert_same(q, q_o, "codes")
+
+
+def test_block_fp8_zero_tile_negative_zero_and_row_stride(oracle):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    w = W.gaussian_outliers((384, 640), std=0.02, p_outlier=0.001, gain=20.0, seed=1001)
+    w[128:256, 128:256] = 0
+    w[300, 7] = -0.0
+    w[5, 5] = 1e-30   # |w/scale| far below the e4m3 subnormal step
+    w[6, 6] = -1e-38
+    q, s = block_fp8(w.to(DEV), [128, 128])
+    q_o, s_o = oracle.block_fp8(w, (128, 128))
+    _assert_same(s, s_o, "scale")
+    _assert_same(q, q_o, "codes")
+    assert torch.all(_u8(q)[128:256, 128:256] == 0xFF) and s[1, 1].item() == 0.0
+    view = w.to(DEV)[:, :512]          # row stride 640, unit column stride
+    q, s = block_fp8(view, [128, 128])
+    q_o, s_o = oracle.block_fp8(w[:, :512].contiguous(), (128, 128))
+    _assert_same(s, s_o, "scale (strided)")
+    _assert_same(q, q_o, "codes (strided)")
+
+
+def test_block_fp8_extreme_scales(oracle):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    g = torch.Generator().manual_seed(9)
+    base = torch.randn((128, 512), generator=g)
+    w = torch.cat([base[:, :128] * 1e-36, base[:, 128:256] * 1e30, base[:, 256:384] * 3e-39, base[:, 384:] * 1e37],
+                  dim=1).to(torch.bfloat16)
+    q, s = block_fp8(w.to(DEV), [128, 128])
+    q_o, s_o = oracle.block_fp8(w, (128, 128))
+    _assert_same(s, s_o, "scale")
+    _assert_same(q, q_o, "codes")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bs", [(32, 32), (64, 128), (128, 64), (128, 128)])
+def test_block_fp8_generic_blocks_and_dtypes(oracle, dtype, bs):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+
+    g = torch.Generator().manual_seed(11)
+    w = (0.05 * torch.randn((200, 330), generator=g)).to(dtype)
+    w[0:32, 0:32] = 0
+    q, s = quant_fp8(w.to(DEV), "block", list(bs))
+    q_o, s_o = oracle.block_fp8(w, bs)
+    _assert_same(s, s_o, "scale")
+    _assert_same(q, q_o, "codes")
+    assert block_fp8 is not None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_tensor_and_channel_fp8(oracle, dtype):
+    from miles_amd.tools.convert_hf_to_fp8 import quant_fp8
+
+    g = torch.Generator().manual_seed(12)
+    w = (0.02 * torch.randn((96, 200), generator=g)).to(dtype)
+    w[3] = 0
+    q, s = quant_fp8(w.to(DEV), "tensor")
+    q_o, s_o = oracle.tensor_fp8(w)
+    assert s.shape == (1,)
+    _assert_same(s, s_o, "tensor scale")
+    _assert_same(q, q_o, "tensor codes")
+    q, s = quant_fp8(w.to(DEV), "channel")
+    q_o, s_o = oracle.channel_fp8(w)
+    assert s.shape == (96, 1)
+    _assert_same(s, s_o, "channel scale")
+    _assert_same(q, q_o, "channel codes")
+
+
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", FP8_SHAPES)
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_fp8_blockwise_cast(oracle, shape, kind):
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    x = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    y, s = fp8_blockwise_cast(x.to(DEV))
+    y_o, s_o = oracle.fp8_blockwise_cast(x)
+    assert y.dtype == F8 and y.is_contiguous() and s.dtype == torch.float32
+    _assert_same(s, s_o, "scale")
+    _assert_same(y, y_o, "codes")
+
+
+def test_fp8_blockwise_cast_strided_and_block_size(oracle):
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    base = W.gaussian_outliers((256, 304), std=0.02, p_outlier=0.001, gain=20.0, seed=5)
+    dev = base.to(DEV)
+    for view_fn in (lambda t: t[:, :256], lambda t: t.t(), lambda t: t[::2, 1::2], lambda t: t.chunk(2, dim=0)[1]):
+        y, s = fp8_blockwise_cast(view_fn(dev))
+        y_o, s_o = oracle.fp8_blockwise_cast(view_fn(base))
+        _assert_same(s, s_o, "scale")
+        _assert_same(y, y_o, "codes")
+    y, s = fp8_blockwise_cast(dev, [64, 32])
+    y_o, s_o = oracle.fp8_blockwise_cast(base, [64, 32])
+    _assert_same(s, s_o, "scale 64x32")
+    _assert_same(y, y_o, "codes 64x32")
+
+
+# ---------------------------------------------------------------------------------------------------
+def test_weight_dequant_all_codes(oracle):
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+
+    g = torch.Generator().manual_seed(21)
+    for shape in [(300, 400), (128, 1024), (257, 144), (5, 7)]:
+        codes = torch.randint(0, 256, shape, generator=g, dtype=torch.int32).to(torch.uint8)
+        codes[0, : min(256, shape[1])] = torch.arange(min(256, shape[1]), dtype=torch.uint8)
+        s = torch.exp(torch.randn((-(-shape[0] // 128), -(-shape[1] // 128)), generator=g) * 4).float()
+        y = weight_dequant(codes.view(F8).to(DEV), s.to(DEV))
+        y_o = oracle.weight_dequant(codes.view(F8), s)
+        assert y.dtype == torch.bfloat16
+        _assert_same(y, y_o, f"dequant {shape}")   # NaN codes give 0x7FC0 on both sides
+
+
+def test_quant_dequant_round_trip(oracle):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+
+    w = W.gaussian_outliers((512, 896), std=0.02, p_outlier=0.0, gain=1.0, seed=5001)
+    q, s = block_fp8(w.to(DEV), [128, 128])
+    y = weight_dequant(q, s)
+    y_o = oracle.weight_dequant(*oracle.block_fp8(w, (128, 128)))
+    _assert_same(y, y_o, "round trip")
+    err = (y.float().cpu() - w.float()).abs()
+    bound = s.cpu().repeat_interleave(128, 0).repeat_interleave(128, 1) * 16.0 + 1e-9   # half an e4m3 step at 448
+    assert torch.all(err <= bound * 1.01)
+    with pytest.raises(AssertionError):
+        weight_dequant(q.t(), s)
+
+
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(7, 96), (1024, 2048)])
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_mxfp8(oracle, shape, kind):
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+
+    w = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    q, s = mxfp8_quantize(w.to(DEV))
+    q_o, s_o = oracle.mxfp8_quantize(w)
+    assert q.shape == w.shape and q.dtype == F8 and s.dtype == torch.uint8
+    assert s.shape == (*w.shape[:-1], w.shape[-1] // 32)
+    _assert_same(s, s_o, "scales")
+    _assert_same(q, q_o, "codes")
+
+
+def test_mxfp8_heavy_tails_3d_dtypes_and_errors(oracle):
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+
+    w = W.student_t_rows((768, 2048), std=0.02, seed=3001)
+    w[3, :64] = 0
+    w[4, :32] = 1e-38
+    w[5, 32:64] = float("inf")
+    q, s = mxfp8_quantize(w.to(DEV))
+    q_o, s_o = oracle.mxfp8_quantize(w)
+    _assert_same(s, s_o, "scales")
+    _assert_same(q, q_o, "codes")
+    w3 = W.student_t_rows((6 * 16, 64), std=1.0, seed=1).reshape(6, 16, 64)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        q, s = mxfp8_quantize(w3.to(dtype).to(DEV))
+        q_o, s_o = oracle.mxfp8_quantize(w3.to(dtype))
+        assert s.shape == (6, 16, 2)
+        _assert_same(s, s_o, f"scales {dtype}")
+        _assert_same(q, q_o, f"codes {dtype}")
+    q, s = mxfp8_quantize(w.to(DEV).t()[:2048:2].t())    # non-contiguous input is made contiguous
+    q_o, s_o = oracle.mxfp8_quantize(w.t()[:2048:2].t())
+    _assert_same(q, q_o, "codes (strided)")
+    with pytest.raises(ValueError, match="Last dim 48 must be divisible by 32 for MXFP8."):
+        mxfp8_quantize(torch.zeros(4, 48, dtype=torch.bfloat16, device=DEV))
+
+
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((24, 7168), 128),
+                                     ((16, 256), 32), ((5, 96), 32), ((9, 192), 64), ((3, 160), 160)])
+def test_int4_pack_layer(oracle, shape, G):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.0005, gain=30.0, seed=4001)
+    w[0] = 0
+    w[1, :G] = 3e-6
+    w[2, :G] = torch.linspace(-1, 1, G)     # exact ties of x/scale are likely here
+    packed, scale, zp = pack_layer(w.to(DEV), G)
+    packed_o, scale_o, _ = oracle.pack_layer(w, G)
+    assert zp is None and packed.dtype == torch.int32 and scale.dtype == torch.bfloat16
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(packed, packed_o, "packed")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_int4_pack_layer_other_dtypes(oracle, dtype):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    w = W.gaussian_outliers((8, 256), std=0.015, p_outlier=0.0, gain=1.0, seed=7, dtype=dtype)
+    packed, scale, _ = pack_layer(w.to(DEV), 128)
+    packed_o, scale_o, _ = oracle.pack_layer(w, 128)
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(packed, packed_o, "packed")
+
+
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("shape,G", [((16, 256), 128), ((8, 200), 32), ((4, 128), 32), ((3, 7168), 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fake_int4_quant(oracle, sym, shape, G, dtype):
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
+
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.001, gain=30.0, seed=4002, dtype=dtype)
+    w[0] = 0
+    out, scale, zero = fake_int4_quant_cuda(w.to(DEV), (1, G), sym)
+    out_o, scale_o, zero_o = oracle.fake_int4_quant(w, (1, G), sym)
+    assert out.dtype == dtype and scale.shape == (shape[0], -(-shape[1] // G))
+    _assert_same(out, out_o, "values")          # includes the -0.0 produced by rint of small negatives
+    _assert_same(scale, scale_o, "scales")
+    if not sym:
+        _assert_same(zero, zero_o, "zero points")
+
+
+def test_fake_int4_quant_argument_checks():
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
+
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="must be divisible by 32"):
+        fake_int4_quant_cuda(x, (1, 48), True)
+    with pytest.raises(RuntimeError, match="Input must be 2D"):
+        fake_int4_quant_cuda(x.reshape(2, 2, 64), (1, 32), True)
+    with pytest.raises(RuntimeError, match="Input must be on CUDA"):
+        fake_int4_quant_cuda(x.cpu(), (1, 32), True)
+
+
+# ---------------------------------------------------------------------------------------------------
+NV_SHAPES = W.SMALL_REFERENCE_SHAPES + [(1, 16), (1, 32), (3, 48), (31, 128), (256, 256), (1024, 2048)]
+
+
+@pytest.mark.parametrize("shape", NV_SHAPES)
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_nvfp4_quantize_1d(oracle, shape, kind, dtype):
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    if dtype == torch.float32 and shape[0] * shape[1] > 300000:
+        pytest.skip("generic-dtype path is covered by the smaller shapes")
+    w = W.reference_pattern(kind, shape, dtype=dtype, spread=12.0)
+    if kind == "random" and shape[0] > 1:
+        w[0].zero_()
+    q, s, g = nvfp4_quantize_1d(w.to(DEV))
+    q_o, s_o, g_o = oracle.nvfp4_quantize_1d(w)
+    assert q.dtype == torch.uint8 and s.dtype == F8 and g.dtype == torch.float32 and g.shape == ()
+    _assert_same(g, g_o, "global scale")
+    _assert_same(s, s_o, "block scales")
+    _assert_same(q, q_o, "codes")
+
+
+def test_nvfp4_pair_and_global_scale_helpers(oracle):
+    from miles_amd.utils import nvfp4 as N
+
+    base = W.reference_pattern("random", (64, 256), spread=12.0, seed=3)
+    base[40:] *= 5
+    dev = base.to(DEV)
+    gate, up = dev.chunk(2, dim=0)
+    (gq, gs, gg), (uq, us, ug) = N.nvfp4_quantize_1d_pair(gate, up)
+    (gq_o, gs_o, gg_o), (uq_o, us_o, ug_o) = oracle.nvfp4_quantize_1d_pair(base[:32], base[32:])
+    for got, want, what in [(gq, gq_o, "gate codes"), (gs, gs_o, "gate scales"), (gg, gg_o, "gate global"),
+                            (uq, uq_o, "up codes"), (us, us_o, "up scales"), (ug, ug_o, "up global")]:
+        _assert_same(got, want, what)
+    assert gg.data_ptr() != ug.data_ptr() and gg.item() == ug.item()
+    with pytest.raises(ValueError, match="expects two 2D tensors"):
+        N.nvfp4_quantize_1d_pair(gate[0], up)
+    with pytest.raises(ValueError, match="matching K dimensions"):
+        N.nvfp4_quantize_1d_pair(gate, up[:, :128])
+    # closed forms on the device without a host read (tests/fast-gpu/test_nvfp4_quantizer.py:108-143)
+    values = torch.tensor([0.0, 1.0, 3.5, torch.finfo(torch.float32).tiny, torch.finfo(torch.float32).max,
+                           float("inf"), -float("inf"), float("nan")], dtype=torch.float32)
+    for e4m3_max in (256, 448):
+        expected = torch.div(torch.tensor(float(e4m3_max)) * torch.tensor(6.0), values)
+        expected = torch.min(expected, torch.tensor(torch.finfo(torch.float32).max))
+        expected = torch.where(expected == 0.0, torch.ones_like(expected), expected)
+        enc = N.nvfp4_global_encode_scale_te(values.to(DEV), e4m3_max).cpu()
+        dec = N.nvfp4_global_decode_scale_te(values.to(DEV), e4m3_max).cpu()
+        torch.testing.assert_close(enc, expected, rtol=0, atol=0, equal_nan=True)
+        torch.testing.assert_close(dec, torch.div(1.0, expected), rtol=0, atol=0, equal_nan=True)
+
+
+# ---------------------------------------------------------------------------------------------------
+# benchmark-sized tensors: full byte comparison against the oracle
+# ---------------------------------------------------------------------------------------------------
+def test_c1_full_size_block_fp8(oracle):
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    for name, w in W.c1_mlp().items():
+        q, s = block_fp8(w.to(DEV), [128, 128])
+        q_o, s_o = oracle.block_fp8(w, (128, 128))
+        _assert_same(s, s_o, f"C1 {name} scale")
+        _assert_same(q, q_o, f"C1 {name} codes")
+
+
+def test_c2_layer_full_size_blockwise_cast(oracle):
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    for idx, (name, shape) in enumerate(W.c2_layer_shapes()):
+        w = W.c2_tensor(17, idx, shape)
+        y, s = fp8_blockwise_cast(w.to(DEV))
+        y_o, s_o = oracle.fp8_blockwise_cast(w)
+        _assert_same(s, s_o, f"C2 {name} scale")
+        _assert_same(y, y_o, f"C2 {name} codes")
+
+
+def test_c3_c4_c5_full_size_experts(oracle):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    for which in (0, 2):
+        w = W.c3_expert(5, 77, which)
+        q, s = mxfp8_quantize(w.to(DEV))
+        q_o, s_o = oracle.mxfp8_quantize(w)
+        _assert_same(s, s_o, "C3 scales")
+        _assert_same(q, q_o, "C3 codes")
+    for which in (1, 2):
+        w = W.c4_expert(3, which)
+        p, s, _ = pack_layer(w.to(DEV), 128)
+        p_o, s_o, _ = oracle.pack_layer(w, 128)
+        _assert_same(s, s_o, "C4 scales")
+        _assert_same(p, p_o, "C4 packed")
+    gate, up, down = (W.c5_expert(9, i) for i in range(3))
+    both = torch.cat((gate, up), dim=0).to(DEV)
+    (gq, gs, gg), (uq, us, ug) = nvfp4_quantize_1d_pair(*both.chunk(2, dim=0))
+    (gq_o, gs_o, gg_o), (uq_o, us_o, ug_o) = oracle.nvfp4_quantize_1d_pair(gate, up)
+    for got, want, what in [(gq, gq_o, "C5 gate codes"), (gs, gs_o, "C5 gate scales"), (gg, gg_o, "C5 gate global"),
+                            (uq, uq_o, "C5 up codes"), (us, us_o, "C5 up scales"), (ug, ug_o, "C5 up global")]:
+        _assert_same(got, want, what)
+    dq, ds, dg = nvfp4_quantize_1d(down.to(DEV))
+    dq_o, ds_o, dg_o = oracle.nvfp4_quantize_1d(down)
+    _assert_same(dq, dq_o, "C5 down codes")
+    _assert_same(ds, ds_o, "C5 down scales")
+    _assert_same(dg, dg_o, "C5 down global")
+    q, s = block_fp8(down.to(DEV), [128, 128])
+    y = weight_dequant(q, s)
+    _assert_same(y, oracle.weight_dequant(*oracle.block_fp8(down, (128, 128))), "C5b round trip")
