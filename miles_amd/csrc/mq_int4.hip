@@ -18,13 +18,17 @@
 // exactly rounded) and rint + the +8 offset are one fp32 add of 1.5*2^23 + 8.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
+#include "mq_group.hpp"
 
 namespace mq {
 
 constexpr float kSymCons = 1.0f / 7.0f;
 constexpr float kAsymCons = 1.0f / 15.0f;
 constexpr int kI4Threads = 256;
-constexpr int kI4Unroll = 4;
+#ifndef MQ_I4_UNROLL
+#define MQ_I4_UNROLL 1
+#endif
+constexpr int kI4Unroll = MQ_I4_UNROLL;
 
 template <int LANES>
 __device__ __forceinline__ uint32_t seg_max(uint32_t v) {
@@ -39,11 +43,16 @@ __device__ __forceinline__ uint32_t seg_max(uint32_t v) {
 __device__ __forceinline__ uint32_t code_bits(float q) { return f2u(q + 12582920.0f); }
 
 template <int LANES>
-__global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const uint16_t* __restrict__ w,
-                                                                    uint32_t* __restrict__ packed,
-                                                                    uint16_t* __restrict__ scale, int64_t total_units) {
+__global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTable tab) {
+    const int64_t item = blockIdx.x;
+    const int ji = find_job(tab, item);
+    const FlatJob& job = tab.job[ji];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ packed = (uint32_t*)job.q;
+    uint16_t* __restrict__ scale = (uint16_t*)job.s;
+    const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll);
+    const int64_t base = (item - (ji ? tab.end[ji - 1] : 0)) * (kI4Threads * kI4Unroll);
     u32x4 v[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
@@ -68,7 +77,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const uint16
             word |= (code_bits(qv) & 0xFu) << (4 * j);
         }
         if (unit < total_units) {
-            packed[unit] = word;
+            st4(packed + unit, word);
             if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
         }
     }
@@ -168,6 +177,26 @@ extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* sca
     return mq_check_launch("int4 fake quant");
 }
 
+bool mq_int4_pack_fast_ok(const void* w, int dtype, int group) {
+    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32);
+}
+
+int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st) {
+    int64_t blocks = 0;
+    const int64_t per_block = kI4Threads * kI4Unroll;
+    for (int i = 0; i < tab.n; i++) {
+        blocks += (tab.job[i].units + per_block - 1) / per_block;
+        tab.end[i] = blocks;
+    }
+    if (blocks == 0) return MQ_OK;
+    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    dim3 grid((unsigned)blocks), blk(kI4Threads);
+    if (group == 128) hipLaunchKernelGGL(int4_pack_bf16_kernel<16>, grid, blk, 0, st, tab);
+    else if (group == 64) hipLaunchKernelGGL(int4_pack_bf16_kernel<8>, grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL(int4_pack_bf16_kernel<4>, grid, blk, 0, st, tab);
+    return mq_check_launch("int4 pack");
+}
+
 extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* scale, int64_t M, int64_t K,
                                         int group, void* stream) {
     if (!w || !packed || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -175,26 +204,16 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
     if (K % group != 0 || K % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and of 8");
     if (M == 0 || K == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
-    const bool aligned = dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0;
     const int64_t units = M * (K / 8);
-    const int64_t per_block = kI4Threads * kI4Unroll;
-    const int64_t fblocks = (units + per_block - 1) / per_block;
-    if (fblocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    dim3 grid((unsigned)fblocks), blk(kI4Threads);
-    if (aligned && group == 128)
-        hipLaunchKernelGGL(int4_pack_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
-                           (uint16_t*)scale, units);
-    else if (aligned && group == 64)
-        hipLaunchKernelGGL(int4_pack_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
-                           (uint16_t*)scale, units);
-    else if (aligned && group == 32)
-        hipLaunchKernelGGL(int4_pack_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed,
-                           (uint16_t*)scale, units);
-    else {
-        int64_t blocks = (units + 255) / 256;
-        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
-        hipLaunchKernelGGL(int4_pack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype,
-                           (uint32_t*)packed, scale, M, K, group);
+    if (mq_int4_pack_fast_ok(w, dtype, group)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, packed, scale, nullptr, units};
+        return mq_int4_pack_launch_group(tab, group, st);
     }
+    int64_t blocks = (units + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(int4_pack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (uint32_t*)packed,
+                       scale, M, K, group);
     return mq_check_launch("int4 pack");
 }

@@ -9,11 +9,15 @@
 // quad.  Scaling by a power of two is exact, so the only rounding is the e4m3 conversion.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
+#include "mq_group.hpp"
 
 namespace mq {
 
 constexpr int kMxThreads = 256;
-constexpr int kMxUnroll = 4;  // 16-byte units per lane per workgroup pass
+#ifndef MQ_MX_UNROLL
+#define MQ_MX_UNROLL 1
+#endif
+constexpr int kMxUnroll = MQ_MX_UNROLL;  // 16-byte units per lane; 1 streams fastest on MI355X (many short wavefronts)
 
 __device__ __forceinline__ uint32_t e8m0_ceil(float v) {
     const uint32_t u = f2u(v);
@@ -28,11 +32,17 @@ __device__ __forceinline__ float e8m0_inverse(uint32_t e) {
     return u2f((254u - e) << 23);
 }
 
-__global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ q,
-                                                                uint8_t* __restrict__ scale, int64_t total_units) {
+__global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const FlatTable tab) {
     const float inv448 = u2f(0x3B124925u);
+    const int64_t item = blockIdx.x;
+    const int ji = find_job(tab, item);
+    const FlatJob& job = tab.job[ji];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint8_t* __restrict__ q = (uint8_t*)job.q;
+    uint8_t* __restrict__ scale = (uint8_t*)job.s;
+    const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kMxThreads * kMxUnroll);
+    const int64_t base = (item - (ji ? tab.end[ji - 1] : 0)) * (kMxThreads * kMxUnroll);
     u32x4 v[kMxUnroll];
 #pragma unroll
     for (int i = 0; i < kMxUnroll; i++) {
@@ -88,6 +98,24 @@ __global__ __launch_bounds__(256) void mxfp8_generic_kernel(const void* __restri
 
 using namespace mq;
 
+bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q) {
+    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
+}
+
+// tab.job[i].units set by the caller; fills tab.end and launches
+int mq_mxfp8_launch_group(FlatTable& tab, hipStream_t st) {
+    int64_t blocks = 0;
+    const int64_t per_block = kMxThreads * kMxUnroll;
+    for (int i = 0; i < tab.n; i++) {
+        blocks += (tab.job[i].units + per_block - 1) / per_block;
+        tab.end[i] = blocks;
+    }
+    if (blocks == 0) return MQ_OK;
+    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    hipLaunchKernelGGL(mxfp8_bf16_kernel, dim3((unsigned)blocks), dim3(kMxThreads), 0, st, tab);
+    return mq_check_launch("mxfp8 quant");
+}
+
 extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K,
                               void* stream) {
     if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -96,18 +124,15 @@ extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale,
     if (rows == 0 || K == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
     const int64_t groups = rows * (K / 32);
-    if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0) {
-        const int64_t units = groups * 4;
-        const int64_t per_block = kMxThreads * kMxUnroll;
-        const int64_t blocks = (units + per_block - 1) / per_block;
-        if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-        hipLaunchKernelGGL(mxfp8_bf16_kernel, dim3((unsigned)blocks), dim3(kMxThreads), 0, st, (const uint16_t*)w,
-                           (uint8_t*)q, scale, units);
-    } else {
-        int64_t blocks = (groups + 255) / 256;
-        if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
-        hipLaunchKernelGGL(mxfp8_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (uint8_t*)q, scale,
-                           groups);
+    if (mq_mxfp8_fast_ok(w, dtype, q)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, q, scale, nullptr, groups * 4};
+        return mq_mxfp8_launch_group(tab, st);
     }
+    int64_t blocks = (groups + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(mxfp8_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (uint8_t*)q, scale,
+                       groups);
     return mq_check_launch("mxfp8 quant");
 }

@@ -11,32 +11,44 @@
 // amax is one DPP step, and each lane emits four bytes of codes.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
+#include "mq_group.hpp"
 
 namespace mq {
 
 constexpr int kNvThreads = 256;
-constexpr int kNvUnroll = 4;
+#ifndef MQ_NV_UNROLL
+#define MQ_NV_UNROLL 1
+#endif
+constexpr int kNvUnroll = MQ_NV_UNROLL;
 constexpr float kSixth = 0.16666667163372040f;  // 0x3E2AAAAB
 
-__global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const uint16_t* __restrict__ w, int64_t n16,
-                                                              int64_t numel, uint32_t* __restrict__ amax_bits) {
+// one 16-byte unit per lane; job.units counts whole units, job.s holds the element count so that the
+// last workgroup of a tensor can fold in a tail shorter than one unit
+__global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable tab) {
     __shared__ uint32_t wave_amax[4];
+    const int64_t item = blockIdx.x;
+    const int ji = find_job(tab, item);
+    const FlatJob& job = tab.job[ji];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ amax_bits = (uint32_t*)job.aux;
+    const int64_t n16 = job.units, numel = (int64_t)(uintptr_t)job.s;
     const int t = threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    uint32_t m2 = 0;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + t; i < n16; i += stride) {
-        const u32x4 v = ld16(w + i * 8);
-        m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+    const int64_t local = item - (ji ? tab.end[ji - 1] : 0);
+    const int64_t unit = local * 256 + t;
+    uint32_t m = 0;
+    if (unit < n16) {
+        const u32x4 v = ld16_keep(w + unit * 8);
+        m = hmax_u16(max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
     }
-    uint32_t m = hmax_u16(m2);
-    if (blockIdx.x == 0 && t == 0)
+    if (local == 0 && t == 0)
         for (int64_t i = n16 * 8; i < numel; i++) m = umax(m, (uint32_t)(w[i] & 0x7FFFu));
     m = wave_max(m);
     if ((t & 63) == 0) wave_amax[t >> 6] = m;
     __syncthreads();
     if (t == 0) {
-        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
-        if (m) atomicMax(amax_bits, m << 16);
+        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3])) << 16;
+        // most workgroups lose against the running maximum: read it first, touch the atomic only to raise it
+        if (m > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax_bits, m);
     }
 }
 
@@ -76,13 +88,18 @@ __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
     return 1.0f / enc;
 }
 
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const uint16_t* __restrict__ w,
-                                                                      const uint32_t* __restrict__ amax_bits,
-                                                                      uint32_t* __restrict__ q, uint8_t* __restrict__ s8,
-                                                                      float* __restrict__ global_scale, float numer,
-                                                                      int64_t total_units) {
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float numer) {
+    const int64_t item = blockIdx.x;
+    const int ji = find_job(tab, item);
+    const FlatJob& job = tab.job[ji];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ q = (uint32_t*)job.q;
+    uint8_t* __restrict__ s8 = (uint8_t*)job.s;
+    const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
+    const int64_t total_units = job.units;
+    const int64_t local = item - (ji ? tab.end[ji - 1] : 0);
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kNvThreads * kNvUnroll);
+    const int64_t base = local * (kNvThreads * kNvUnroll);
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
@@ -91,7 +108,6 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const uint
     }
     const float amax = u2f(amax_bits[0]);
     const NvScales gs = nv_scales(amax, numer);
-    if (global_scale && blockIdx.x == 0 && t == 0) *global_scale = nv_published_scale(amax, numer);
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
@@ -119,10 +135,22 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const uint
             for (int j = 0; j < 8; j++) word |= sw_e2m1(f[j] * inv) << (4 * j);
         }
         if (unit < total_units) {
-            q[unit] = word;
+            st4(q + unit, word);
             if ((t & 1) == 0) s8[unit >> 1] = (uint8_t)sc;
         }
     }
+}
+
+// weight_scale_2 of every tensor of a group: out[i] = 1 / min(numer / amax_i, FLT_MAX) (zero repaired to 1)
+struct NvGlobalTable {
+    int32_t n;
+    int32_t pad;
+    const uint32_t* amax[kMaxGroup];
+    float* out[kMaxGroup];
+};
+__global__ void nvfp4_global_scale_kernel(const NvGlobalTable tab, float numer) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < tab.n && tab.out[i]) *tab.out[i] = nv_published_scale(u2f(*tab.amax[i]), numer);
 }
 
 __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __restrict__ w, int dtype,
@@ -154,24 +182,61 @@ __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __
 
 using namespace mq;
 
+bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q) {
+    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 4) == 0;
+}
+
+// tab.job[i]: w, aux = amax word, units = numel / 8, s = (void*)numel
+int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
+    int64_t blocks = 0;
+    for (int i = 0; i < tab.n; i++) {
+        int64_t b = (tab.job[i].units + 255) / 256;
+        if (b < 1 && (int64_t)(uintptr_t)tab.job[i].s > 0) b = 1;
+        blocks += b;
+        tab.end[i] = blocks;
+    }
+    if (blocks == 0) return MQ_OK;
+    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, tab);
+    return mq_check_launch("nvfp4 amax");
+}
+
+// tab.job[i]: w, q, s = block scales, aux = amax word, units = numel / 8; global_out[i] may be null
+int mq_nvfp4_quant_launch_group(FlatTable& tab, float* const* global_out, int e4m3_max, hipStream_t st) {
+    const float numer = (float)e4m3_max * 6.0f;
+    int64_t blocks = 0;
+    const int64_t per_block = kNvThreads * kNvUnroll;
+    NvGlobalTable gt{};
+    gt.n = tab.n;
+    bool any_global = false;
+    for (int i = 0; i < tab.n; i++) {
+        blocks += (tab.job[i].units + per_block - 1) / per_block;
+        tab.end[i] = blocks;
+        gt.amax[i] = (const uint32_t*)tab.job[i].aux;
+        gt.out[i] = global_out ? global_out[i] : nullptr;
+        any_global |= gt.out[i] != nullptr;
+    }
+    if (any_global) hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(64), 0, st, gt, numer);
+    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (blocks > 0) hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)blocks), dim3(kNvThreads), 0, st, tab, numer);
+    return mq_check_launch("nvfp4 quant");
+}
+
 extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* amax_bits, void* stream) {
     if (!w || !amax_bits) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (numel == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0) {
-        const int64_t n16 = numel / 8;
-        int64_t blocks = (n16 + 255) / 256;
-        if (blocks > 2048) blocks = 2048;
-        if (blocks < 1) blocks = 1;
-        hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t*)w, n16,
-                           numel, (uint32_t*)amax_bits);
-    } else {
-        int64_t blocks = (numel + 255) / 256;
-        if (blocks > 2048) blocks = 2048;
-        hipLaunchKernelGGL(nvfp4_amax_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, numel,
-                           (uint32_t*)amax_bits);
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, nullptr, (void*)(uintptr_t)numel, amax_bits, numel / 8};
+        return mq_nvfp4_amax_launch_group(tab, st);
     }
+    int64_t blocks = (numel + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(nvfp4_amax_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, numel,
+                       (uint32_t*)amax_bits);
     return mq_check_launch("nvfp4 amax");
 }
 
@@ -184,25 +249,15 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, v
     hipStream_t st = (hipStream_t)stream;
     const float numer = (float)e4m3_max * 6.0f;
     const int64_t blocks16 = M * (K / 16);
-    if (blocks16 == 0) {
-        // empty tensor: only the global scale is defined
-        if (global_scale)
-            hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3(1), dim3(64), 0, st, w, dtype, (const uint32_t*)amax_bits,
-                               (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer, (int64_t)0);
-        return mq_check_launch("nvfp4 quant");
+    if (blocks16 == 0 || mq_nvfp4_fast_ok(w, dtype, q)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(amax_bits), blocks16 * 2};
+        return mq_nvfp4_quant_launch_group(tab, &global_scale, e4m3_max, st);
     }
-    if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 4) == 0) {
-        const int64_t units = blocks16 * 2;
-        const int64_t per_block = kNvThreads * kNvUnroll;
-        const int64_t nb = (units + per_block - 1) / per_block;
-        if (nb > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-        hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)nb), dim3(kNvThreads), 0, st, (const uint16_t*)w,
-                           (const uint32_t*)amax_bits, (uint32_t*)q, (uint8_t*)block_scale, global_scale, numer, units);
-    } else {
-        int64_t nb = (blocks16 + 255) / 256;
-        if (nb > mq_grid_cap()) nb = mq_grid_cap();
-        hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
-                           (const uint32_t*)amax_bits, (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer, blocks16);
-    }
+    int64_t nb = (blocks16 + 255) / 256;
+    if (nb > mq_grid_cap()) nb = mq_grid_cap();
+    hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
+                       (const uint32_t*)amax_bits, (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer, blocks16);
     return mq_check_launch("nvfp4 quant");
 }

@@ -1,0 +1,222 @@
+// Batched driver: turns a list of per-tensor quantization jobs into grouped kernel launches.
+//
+// One launch carries up to kMaxGroup tensors (descriptors in the kernel argument segment), so a weight sync
+// issues a few launches per layer instead of several per tensor.  Jobs that do not qualify for a grouped
+// fast path (other dtypes, block sizes, strides, alignment) run through the single-tensor entry points, in
+// list order.
+#include <vector>
+
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+#include "mq_group.hpp"
+
+using namespace mq;
+
+// grouped launchers implemented next to their kernels
+bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, const void* q, int64_t M, int64_t K,
+                         int bm, int bk);
+int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st);
+bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block);
+int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st);
+bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q);
+int mq_mxfp8_launch_group(FlatTable& tab, hipStream_t st);
+bool mq_int4_pack_fast_ok(const void* w, int dtype, int group);
+int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st);
+bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
+int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
+int mq_nvfp4_quant_launch_group(FlatTable& tab, float* const* global_out, int e4m3_max, hipStream_t st);
+
+namespace mq {
+struct WordTable {
+    int32_t n;
+    int32_t pad;
+    uint32_t* p[kMaxGroup];
+};
+__global__ void clear_words_kernel(const WordTable tab) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < tab.n) *tab.p[i] = 0u;
+}
+}  // namespace mq
+
+// The amax pass and the quantize pass of an NVFP4 group read the same input; keeping a group's input
+// below this many bytes lets the second read be served by the 256 MB memory-side cache.
+static const int64_t kNvfp4GroupBytes = 96ll << 20;
+
+static bool job_fast(const mq_job& j) {
+    switch (j.kind) {
+        case MQ_JOB_FP8_BLOCK:
+        case MQ_JOB_FP8_BLOCKWISE_CAST:
+            return mq_fp8_tile_fast_ok(j.in, j.dtype, j.ld, 1, j.out, j.rows, j.cols, j.p0, j.p1);
+        case MQ_JOB_FP8_DEQUANT:
+            return mq_fp8_dequant_fast_ok(j.in, j.out, j.rows, j.cols, j.p0);
+        case MQ_JOB_MXFP8:
+            return mq_mxfp8_fast_ok(j.in, j.dtype, j.out) && j.cols % 32 == 0;
+        case MQ_JOB_INT4_PACK:
+            return mq_int4_pack_fast_ok(j.in, j.dtype, j.p0) && j.cols % j.p0 == 0 && j.cols % 8 == 0;
+        case MQ_JOB_NVFP4:
+            return mq_nvfp4_fast_ok(j.in, j.dtype, j.out) && j.cols % 16 == 0 && (j.p0 == 448 || j.p0 == 256);
+        default:
+            return false;
+    }
+}
+
+static int check_job(const mq_job& j) {
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_NVFP4) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
+    if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
+    if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
+    if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax word");
+    return MQ_OK;
+}
+
+static int run_single(const mq_job& j, void* stream) {
+    switch (j.kind) {
+        case MQ_JOB_FP8_BLOCK:
+            return mq_fp8_block_quant(j.in, j.dtype, j.ld, j.out, (float*)j.scale, j.rows, j.cols, j.p0, j.p1, stream);
+        case MQ_JOB_FP8_BLOCKWISE_CAST:
+            return mq_fp8_blockwise_cast(j.in, j.dtype, j.ld, 1, j.out, (float*)j.scale, j.rows, j.cols, j.p0, j.p1,
+                                         stream);
+        case MQ_JOB_FP8_DEQUANT:
+            return mq_fp8_block_dequant(j.in, (const float*)j.aux, j.out, j.rows, j.cols, j.p0, stream);
+        case MQ_JOB_MXFP8:
+            return mq_mxfp8_quant(j.in, j.dtype, j.out, (uint8_t*)j.scale, j.rows, j.cols, stream);
+        case MQ_JOB_INT4_PACK:
+            return mq_int4_group_quant_pack(j.in, j.dtype, (int32_t*)j.out, j.scale, j.rows, j.cols, j.p0, stream);
+        default:
+            return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    }
+}
+
+static bool same_group(const mq_job& a, const mq_job& b) {
+    return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
+}
+
+// NVFP4 run [i, j): all jobs fast or not, processed as amax-phase then quantize-phase per chunk
+static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    while (i < j) {
+        // a chunk ends at the group / byte limit, but never between two jobs that share an amax word
+        int64_t k = i, bytes = 0;
+        while (k < j) {
+            const bool tied = k > i && jobs[k].aux == jobs[k - 1].aux;
+            const int64_t b = jobs[k].rows * jobs[k].cols * (jobs[k].dtype == MQ_F32 ? 4 : 2);
+            if (!tied && k > i && (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0)) break;
+            if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax word");
+            bytes += b;
+            k++;
+        }
+        const int n = (int)(k - i);
+        WordTable words{};
+        words.n = n;
+        for (int t = 0; t < n; t++) words.p[t] = (uint32_t*)jobs[i + t].aux;
+        hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(64), 0, st, words);
+        bool all_fast = true;
+        for (int t = 0; t < n; t++) all_fast &= job_fast(jobs[i + t]);
+        if (all_fast) {
+            FlatTable tab{};
+            tab.n = n;
+            for (int t = 0; t < n; t++) {
+                const mq_job& jb = jobs[i + t];
+                const int64_t numel = jb.rows * jb.cols;
+                tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8};
+            }
+            int rc = mq_nvfp4_amax_launch_group(tab, st);
+            if (rc) return rc;
+            float* gout[kMaxGroup];
+            for (int t = 0; t < n; t++) {
+                const mq_job& jb = jobs[i + t];
+                tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8};
+                gout[t] = (float*)jb.aux2;
+            }
+            rc = mq_nvfp4_quant_launch_group(tab, gout, jobs[i].p0, st);
+            if (rc) return rc;
+        } else {
+            for (int t = 0; t < n; t++) {
+                const mq_job& jb = jobs[i + t];
+                int rc = mq_nvfp4_amax(jb.in, jb.dtype, jb.rows * jb.cols, jb.aux, stream);
+                if (rc) return rc;
+            }
+            for (int t = 0; t < n; t++) {
+                const mq_job& jb = jobs[i + t];
+                int rc = mq_nvfp4_quant(jb.in, jb.dtype, jb.aux, jb.out, jb.scale, (float*)jb.aux2, jb.rows, jb.cols,
+                                        jb.p0, stream);
+                if (rc) return rc;
+            }
+        }
+        i = k;
+    }
+    return mq_check_launch("nvfp4 group");
+}
+
+extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
+    if (n < 0 || (n > 0 && !jobs)) return mq_fail(MQ_ERR_ARG, "bad job list");
+    hipStream_t st = (hipStream_t)stream;
+    for (int64_t i = 0; i < n; i++) {
+        int rc = check_job(jobs[i]);
+        if (rc) return rc;
+    }
+    int64_t i = 0;
+    while (i < n) {
+        const mq_job& head = jobs[i];
+        if (head.kind == MQ_JOB_NVFP4) {
+            int64_t j = i + 1;
+            while (j < n && jobs[j].kind == MQ_JOB_NVFP4) j++;
+            int rc = run_nvfp4(jobs, i, j, stream);
+            if (rc) return rc;
+            i = j;
+            continue;
+        }
+        if (head.rows == 0 || head.cols == 0) { i++; continue; }
+        if (!job_fast(head)) {
+            int rc = run_single(head, stream);
+            if (rc) return rc;
+            i++;
+            continue;
+        }
+        int64_t j = i + 1;
+        while (j < n && j - i < kMaxGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
+               jobs[j].cols > 0)
+            j++;
+        const int cnt = (int)(j - i);
+        int rc = MQ_OK;
+        switch (head.kind) {
+            case MQ_JOB_FP8_BLOCK:
+            case MQ_JOB_FP8_BLOCKWISE_CAST: {
+                TileTable tab{};
+                tab.n = cnt;
+                for (int t = 0; t < cnt; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, jb.ld, (int32_t)jb.rows, (int32_t)jb.cols, 0, 0};
+                }
+                rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : 1, tab, st);
+                break;
+            }
+            case MQ_JOB_FP8_DEQUANT: {
+                MqDequantArgs a[kMaxGroup];
+                for (int t = 0; t < cnt; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    a[t] = MqDequantArgs{jb.in, (const float*)jb.aux, jb.out, jb.rows, jb.cols, jb.p0};
+                }
+                rc = mq_fp8_dequant_launch_group(a, cnt, st);
+                break;
+            }
+            case MQ_JOB_MXFP8:
+            case MQ_JOB_INT4_PACK: {
+                FlatTable tab{};
+                tab.n = cnt;
+                for (int t = 0; t < cnt; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8};
+                }
+                rc = head.kind == MQ_JOB_MXFP8 ? mq_mxfp8_launch_group(tab, st)
+                                               : mq_int4_pack_launch_group(tab, head.p0, st);
+                break;
+            }
+            default:
+                rc = mq_fail(MQ_ERR_ARG, "unknown job kind");
+        }
+        if (rc) return rc;
+        i = j;
+    }
+    return MQ_OK;
+}

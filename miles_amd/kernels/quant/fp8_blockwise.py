@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 fp8_dtype = torch.float8_e4m3fn
 fp8_max = torch.finfo(fp8_dtype).max
@@ -27,11 +27,15 @@ def fp8_blockwise_cast(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, 
     """
     bm, bn = (128, 128) if not block_size else (int(block_size[0]), int(block_size[1]))
     _lib.require_gpu(x, "fp8_blockwise_cast")
+    _lib.dtype_code(x, "fp8_blockwise_cast")
     M, N = x.shape
     y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
     s = torch.empty(ceil_div(M, bm), ceil_div(N, bn), dtype=torch.float32, device=x.device)
-    rc = _lib.load().mq_fp8_blockwise_cast(x.data_ptr(), _lib.dtype_code(x, "fp8_blockwise_cast"), x.stride(0),
-                                           x.stride(1), y.data_ptr(), s.data_ptr(), M, N, bm, bn,
-                                           _lib.stream_ptr(x.device))
-    _lib.check(rc)
+    if x.stride(1) == 1 or N <= 1:
+        launch.submit(_lib.JOB_FP8_BLOCKWISE_CAST, x, y, s, None, None, M, N, x.stride(0), bm, bn)
+    else:  # general column stride: direct entry point, not batchable
+        rc = _lib.load().mq_fp8_blockwise_cast(x.data_ptr(), _lib.dtype_code(x, "fp8_blockwise_cast"), x.stride(0),
+                                               x.stride(1), y.data_ptr(), s.data_ptr(), M, N, bm, bn,
+                                               _lib.stream_ptr(x.device))
+        _lib.check(rc)
     return y, s

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 
 def fake_int4_quant_cuda(x: torch.Tensor, block_size, sym: bool):
@@ -58,7 +58,6 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
     w = weight.contiguous()
     packed = torch.empty((M, K // 8), dtype=torch.int32, device=w.device)
     scale = torch.empty((M, K // group_size), dtype=w.dtype, device=w.device)
-    rc = _lib.load().mq_int4_group_quant_pack(w.data_ptr(), _lib.dtype_code(w, "pack_layer"), packed.data_ptr(),
-                                              scale.data_ptr(), M, K, int(group_size), _lib.stream_ptr(w.device))
-    _lib.check(rc, RuntimeError)
+    _lib.dtype_code(w, "pack_layer")
+    launch.submit(_lib.JOB_INT4_PACK, w, packed, scale, None, None, M, K, K, int(group_size), 0)
     return packed, scale, None

@@ -1,0 +1,89 @@
+"""Submission of quantization jobs to libmiles_quant.so: immediately, or deferred into one batched call.
+
+Outside a `deferred()` block every quantizer wrapper runs its job at once (one `mq_run_jobs` call with a
+single job).  Inside the block the wrappers still allocate and return their output tensors, but the jobs
+are only recorded; leaving the block submits the whole list with ONE call, which the library turns into
+grouped kernel launches (up to 64 tensors per launch).  The returned tensors must not be read before the
+block ends.  This is how the weight-sync driver keeps thousands of per-parameter quantizer calls from being
+launch-bound without changing the per-tensor call signatures.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import threading
+
+import torch
+
+from miles_amd import _lib
+
+_state = threading.local()
+
+
+class JobBatch:
+    """An ordered list of mq_job records plus the tensors they reference."""
+
+    def __init__(self) -> None:
+        self._records: list[tuple] = []
+        self._keep: list[torch.Tensor] = []
+        self._array = None
+        self.device = None
+
+    def __len__(self) -> int:
+        return len(self._records)
+
+    def add(self, kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1, keep=()) -> None:
+        self._records.append((kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1))
+        self._keep.extend(keep)
+        self._array = None
+
+    def freeze(self):
+        """Materialise the ctypes job array (done once; `run` can then be repeated)."""
+        if self._array is None:
+            arr = (_lib.Job * len(self._records))()
+            for i, rec in enumerate(self._records):
+                arr[i] = _lib.Job(*rec)
+            self._array = arr
+        return self._array
+
+    def run(self, stream: int | None = None) -> None:
+        if not self._records:
+            return
+        arr = self.freeze()
+        if stream is None:
+            stream = _lib.stream_ptr(self.device)
+        _lib.check(_lib.load().mq_run_jobs(arr, len(self._records), stream))
+
+
+def active_batch() -> JobBatch | None:
+    return getattr(_state, "batch", None)
+
+
+@contextlib.contextmanager
+def deferred():
+    """Record the quantizer calls made inside the block and submit them together on exit."""
+    if active_batch() is not None:
+        raise _lib.MilesQuantError("deferred() blocks do not nest")
+    batch = JobBatch()
+    _state.batch = batch
+    try:
+        yield batch
+    finally:
+        _state.batch = None
+    batch.run()
+
+
+def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0) -> None:
+    """Run (or record) one job.  Tensor arguments may be None where the job kind has no such operand."""
+    rec = (kind, _lib.DTYPE_CODE.get(inp.dtype, 0), inp.data_ptr(), out.data_ptr(),
+           scale.data_ptr() if scale is not None else None, aux.data_ptr() if aux is not None else None,
+           aux2.data_ptr() if aux2 is not None else None, rows, cols, ld, p0, p1)
+    keep = [t for t in (inp, out, scale, aux, aux2) if t is not None]
+    batch = active_batch()
+    if batch is not None:
+        if batch.device is None:
+            batch.device = inp.device
+        batch.add(*rec, keep=keep)
+        return
+    one = (_lib.Job * 1)(_lib.Job(*rec))
+    _lib.check(_lib.load().mq_run_jobs(one, 1, _lib.stream_ptr(inp.device)))

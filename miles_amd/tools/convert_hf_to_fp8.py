@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 FP8_INFO = torch.finfo(torch.float8_e4m3fn)
 FP8_MAX, FP8_MIN = FP8_INFO.max, FP8_INFO.min
@@ -31,9 +31,8 @@ def block_fp8(weight: torch.Tensor, block_size):
     w = weight if weight.stride(1) == 1 else weight.contiguous()
     q = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((ceildiv(n, bn), ceildiv(k, bk)), dtype=torch.float32, device=w.device)
-    rc = _lib.load().mq_fp8_block_quant(w.data_ptr(), _lib.dtype_code(w, "block_fp8"), w.stride(0), q.data_ptr(),
-                                        scale.data_ptr(), n, k, bn, bk, _lib.stream_ptr(w.device))
-    _lib.check(rc)
+    _lib.dtype_code(w, "block_fp8")
+    launch.submit(_lib.JOB_FP8_BLOCK, w, q, scale, None, None, n, k, w.stride(0), bn, bk)
     return q, scale
 
 

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 
 def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
@@ -23,7 +23,5 @@ def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> t
         raise _lib.MilesQuantError(f"weight_dequant expects float32 scales, got {s.dtype}")
     M, N = x.size()
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    rc = _lib.load().mq_fp8_block_dequant(x.data_ptr(), s.data_ptr(), y.data_ptr(), M, N, int(block_size),
-                                          _lib.stream_ptr(x.device))
-    _lib.check(rc)
+    launch.submit(_lib.JOB_FP8_DEQUANT, x, y, None, s, None, M, N, N, int(block_size), 0)
     return y

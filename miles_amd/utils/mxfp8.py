@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 MXFP8_GROUP_SIZE = 32
 
@@ -48,7 +48,6 @@ def mxfp8_quantize(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     rows = w.numel() // k if k else 0
     q = torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((*w.shape[:-1], k // MXFP8_GROUP_SIZE), dtype=torch.uint8, device=w.device)
-    rc = _lib.load().mq_mxfp8_quant(w.data_ptr(), _lib.dtype_code(w, "mxfp8_quantize"), q.data_ptr(),
-                                    scale.data_ptr(), rows, k, _lib.stream_ptr(w.device))
-    _lib.check(rc)
+    _lib.dtype_code(w, "mxfp8_quantize")
+    launch.submit(_lib.JOB_MXFP8, w, q, scale, None, None, rows, k, k)
     return q, scale

@@ -13,7 +13,7 @@ import os
 
 import torch
 
-from miles_amd import _lib
+from miles_amd import _lib, launch
 
 FP4_E2M1_MAX = 6.0
 FP8_E4M3_MAX = 448.0
@@ -47,27 +47,13 @@ def _check_supported() -> int:
     return nvfp4_weight_e4m3_max()
 
 
-def _amax_word(device) -> torch.Tensor:
-    word = torch.empty(1, dtype=torch.int32, device=device)
-    _lib.check(_lib.load().mq_fill_u32(word.data_ptr(), 0, 1, _lib.stream_ptr(device)))
-    return word
-
-
-def _reduce_amax(word: torch.Tensor, w: torch.Tensor) -> None:
-    rc = _lib.load().mq_nvfp4_amax(w.data_ptr(), _lib.dtype_code(w, "nvfp4"), w.numel(), word.data_ptr(),
-                                   _lib.stream_ptr(w.device))
-    _lib.check(rc)
-
-
-def _quantize_with_amax(w: torch.Tensor, word: torch.Tensor, e4m3_max: int):
+def _alloc_outputs(w: torch.Tensor):
+    """The three outputs of one tensor: packed codes, block scales, global scale."""
     rows, cols = w.shape
+    _lib.dtype_code(w, "nvfp4")
     q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
     block_scale = torch.empty((rows, cols // NVFP4_GROUP_SIZE), dtype=torch.float8_e4m3fn, device=w.device)
     global_scale = torch.empty((), dtype=torch.float32, device=w.device)
-    rc = _lib.load().mq_nvfp4_quant(w.data_ptr(), _lib.dtype_code(w, "nvfp4"), word.data_ptr(), q.data_ptr(),
-                                    block_scale.data_ptr(), global_scale.data_ptr(), rows, cols, e4m3_max,
-                                    _lib.stream_ptr(w.device))
-    _lib.check(rc)
     return q, block_scale, global_scale
 
 
@@ -78,9 +64,10 @@ def nvfp4_quantize_1d(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor,
     w = weight.contiguous()
     if w.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {w.shape[1]}.")
-    word = _amax_word(w.device)
-    _reduce_amax(word, w)
-    return _quantize_with_amax(w, word, e4m3_max)
+    word = torch.empty(1, dtype=torch.int32, device=w.device)   # cleared and reduced into by the job driver
+    out = _alloc_outputs(w)
+    launch.submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max)
+    return out
 
 
 def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
@@ -97,7 +84,26 @@ def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
     a, b = first.contiguous(), second.contiguous()
     if a.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {a.shape[1]}.")
-    word = _amax_word(a.device)
-    _reduce_amax(word, a)
-    _reduce_amax(word, b)
-    return _quantize_with_amax(a, word, e4m3_max), _quantize_with_amax(b, word, e4m3_max)
+    word = torch.empty(1, dtype=torch.int32, device=a.device)
+    outs = (_alloc_outputs(a), _alloc_outputs(b))
+    # two adjacent jobs on one amax word: the driver reduces both tensors before it quantizes either
+    with _pair_scope() as submit:
+        for w, out in zip((a, b), outs):
+            submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max)
+    return outs
+
+
+class _pair_scope:
+    """Submits the two jobs of a pair together even when no deferred() block is active."""
+
+    def __enter__(self):
+        self._own = launch.active_batch() is None
+        if self._own:
+            self._ctx = launch.deferred()
+            self._ctx.__enter__()
+        return launch.submit
+
+    def __exit__(self, *exc):
+        if self._own:
+            return self._ctx.__exit__(*exc)
+        return False
