@@ -26,11 +26,11 @@ constexpr int kTileWaves = kTileThreads / kWave;
 template <int MODE>
 __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTable tab) {
     __shared__ uint32_t wave_amax[kTileWaves];
-    const int64_t item = xcd_contiguous_item(tab.end[tab.n - 1]);
+    const int32_t item = xcd_contiguous_item(tab.total);
     if (item < 0) return;
-    const int ji = find_job(tab, item);
-    const TileJob& job = tab.job[ji];
-    const int64_t tile = item - (ji ? tab.end[ji - 1] : 0);
+    const JobRef ref = find_job(tab, item);
+    const TileJob& job = tab.job[ref.ji];
+    const int64_t tile = item - ref.start;
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint8_t* __restrict__ q = (uint8_t*)job.q;
     const int64_t M = job.M, K = job.K, ldw = job.ldw;
@@ -203,60 +203,73 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 }
 
 // ---- dequant ----------------------------------------------------------------------------------
-// Fast path: N % 16 == 0, block % 16 == 0, 16-byte aligned.  Each lane turns 16 codes (one 16-byte load)
-// into 16 bf16 (two 16-byte stores); a wavefront covers 1 KiB of codes.
+// Fast path: N % 8 == 0, block a power of two >= 8, aligned pointers.  The tensor is a flat run of 8-code
+// units; each lane turns kDqUnroll units (8-byte loads) into bf16 (16-byte stores), so a wavefront writes
+// 1 KiB of consecutive output per store instruction.  Row and column of a unit come from a multiply-high
+// division by the row length (exact for every 32-bit unit index), not from an integer divide.
+constexpr int kDqThreads = 256;
+constexpr int kDqUnroll = 2;
 struct DequantJob {
     const uint8_t* x;
     const float* s;
     uint16_t* y;
-    int64_t units;          // M * N / 16
-    uint32_t units_per_row; // N / 16
-    int32_t block, tiles_n, pad;
+    uint32_t units;          // M * N / 8
+    uint32_t units_per_row;  // N / 8
+    uint32_t magic, shift;   // floor(n / units_per_row) == (t + ((n - t) >> 1)) >> shift, t = mulhi(magic, n)
+    int32_t block_shift;     // log2(block)
+    int32_t tiles_n;
 };
 struct DequantTable {
     int32_t n;
-    int32_t pad;
-    int64_t end[kMaxGroup];
+    int32_t max_blocks;
     DequantJob job[kMaxGroup];
 };
 
-__global__ __launch_bounds__(256) void fp8_dequant_kernel(const DequantTable tab) {
-    const int64_t item = blockIdx.x;
-    const int ji = find_job(tab, item);
-    const DequantJob& job = tab.job[ji];
-    const int64_t unit = (item - (ji ? tab.end[ji - 1] : 0)) * 256 + threadIdx.x;
-    if (unit >= job.units) return;
-    const uint32_t r = (uint32_t)(unit / job.units_per_row);
-    const uint32_t c = ((uint32_t)(unit - (int64_t)r * job.units_per_row)) * 16u;
-    const u32x4 in = ld16(job.x + unit * 16);
-    const float sc = job.s[(int64_t)(r / (uint32_t)job.block) * job.tiles_n + c / (uint32_t)job.block];
-    const uint32_t wd[4] = {in.x, in.y, in.z, in.w};
-    uint32_t o[8];
-    // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0
-    bool special = (f2u(sc) & 0x7F800000u) == 0x7F800000u;
+__global__ __launch_bounds__(kDqThreads) void fp8_dequant_kernel(const DequantTable tab) {
+    const DequantJob& job = tab.job[blockIdx.y];
+    const uint32_t base = blockIdx.x * (kDqThreads * kDqUnroll);
+    if (base >= job.units) return;
+    u32x2 in[kDqUnroll];
 #pragma unroll
-    for (int k = 0; k < 4; k++) special |= (((wd[k] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u) != 0u;
-    if (!special) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const f32x2 a = hw_e4m3x2_decode<false>(wd[k]);
-            const f32x2 b = hw_e4m3x2_decode<true>(wd[k]);
-            o[2 * k] = hw_bf16x2(a.x * sc, a.y * sc);
-            o[2 * k + 1] = hw_bf16x2(b.x * sc, b.y * sc);
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            uint32_t h[4];
-#pragma unroll
-            for (int b = 0; b < 4; b++) h[b] = sw_bf16(sw_e4m3fn_decode((wd[k] >> (8 * b)) & 0xFFu) * sc);
-            o[2 * k] = h[0] | (h[1] << 16);
-            o[2 * k + 1] = h[2] | (h[3] << 16);
-        }
+    for (int i = 0; i < kDqUnroll; i++) {
+        const uint32_t unit = base + i * kDqThreads + threadIdx.x;
+        in[i] = unit < job.units ? __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(job.x + (int64_t)unit * 8))
+                                 : u32x2{0u, 0u};
     }
-    uint16_t* dst = job.y + unit * 16;
-    st16(dst, u32x4{o[0], o[1], o[2], o[3]});
-    st16(dst + 8, u32x4{o[4], o[5], o[6], o[7]});
+#pragma unroll
+    for (int i = 0; i < kDqUnroll; i++) {
+        const uint32_t unit = base + i * kDqThreads + threadIdx.x;
+        if (unit >= job.units) continue;
+        const uint32_t th = __umulhi(job.magic, unit);
+        const uint32_t r = (th + ((unit - th) >> 1)) >> job.shift;
+        const uint32_t c = (unit - r * job.units_per_row) * 8u;
+        const float sc = job.s[(int64_t)(r >> job.block_shift) * job.tiles_n + (c >> job.block_shift)];
+        const uint32_t wd[2] = {in[i].x, in[i].y};
+        uint32_t o[4];
+        // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0
+        bool special = (f2u(sc) & 0x7F800000u) == 0x7F800000u;
+#pragma unroll
+        for (int k = 0; k < 2; k++) special |= (((wd[k] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u) != 0u;
+        if (!special) {
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const f32x2 a = hw_e4m3x2_decode<false>(wd[k]);
+                const f32x2 b = hw_e4m3x2_decode<true>(wd[k]);
+                o[2 * k] = hw_bf16x2(a.x * sc, a.y * sc);
+                o[2 * k + 1] = hw_bf16x2(b.x * sc, b.y * sc);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                uint32_t h[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) h[b] = sw_bf16(sw_e4m3fn_decode((wd[k] >> (8 * b)) & 0xFFu) * sc);
+                o[2 * k] = h[0] | (h[1] << 16);
+                o[2 * k + 1] = h[2] | (h[3] << 16);
+            }
+        }
+        st16(job.y + (int64_t)unit * 8, u32x4{o[0], o[1], o[2], o[3]});
+    }
 }
 
 __global__ __launch_bounds__(256) void fp8_dequant_generic_kernel(const uint8_t* __restrict__ x,
@@ -288,11 +301,12 @@ int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
         TileJob& j = tab.job[i];
         j.tiles_k = (j.K + kTile - 1) / kTile;
         tiles += (int64_t)((j.M + kTile - 1) / kTile) * j.tiles_k;
-        tab.end[i] = tiles;
+        if (tiles >= 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "too many tiles");
+        tab.end[i] = (int32_t)tiles;
     }
     if (tiles == 0) return MQ_OK;
+    seal_table(tab);
     const int64_t grid = xcd_grid(tiles);
-    if (grid > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many tiles");
     if (mode == 0) hipLaunchKernelGGL(fp8_block128_kernel<0>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
     else hipLaunchKernelGGL(fp8_block128_kernel<1>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
     return mq_check_launch("fp8 block quant");
@@ -350,29 +364,37 @@ extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* 
 }
 
 bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block) {
-    return (N % 16) == 0 && (block % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
-           N / 16 <= 0x7FFFFFFF && M <= 0x7FFFFFFF;
+    const bool pow2 = block >= 8 && (block & (block - 1)) == 0;
+    return (N % 8) == 0 && N >= 16 && pow2 && ((uintptr_t)x % 8) == 0 && ((uintptr_t)y % 16) == 0 &&
+           M * (N / 8) < 0xFFFFFFF0ll;
 }
 
 int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st) {
     DequantTable tab{};
     tab.n = n;
-    int64_t blocks = 0;
+    int64_t mx = 0;
     for (int i = 0; i < n; i++) {
         DequantJob& j = tab.job[i];
         j.x = (const uint8_t*)a[i].x;
         j.s = a[i].s;
         j.y = (uint16_t*)a[i].y;
-        j.units = a[i].M * (a[i].N / 16);
-        j.units_per_row = (uint32_t)(a[i].N / 16);
-        j.block = a[i].block;
+        j.units = (uint32_t)(a[i].M * (a[i].N / 8));
+        const uint32_t d = (uint32_t)(a[i].N / 8);   // >= 2
+        j.units_per_row = d;
+        uint32_t l = 0;
+        while ((1ull << l) < d) l++;                 // ceil(log2 d) >= 1
+        j.magic = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+        j.shift = l - 1;
+        int bs = 0;
+        while ((1 << bs) < a[i].block) bs++;
+        j.block_shift = bs;
         j.tiles_n = (int32_t)((a[i].N + a[i].block - 1) / a[i].block);
-        blocks += (j.units + 255) / 256;
-        tab.end[i] = blocks;
+        const int64_t b = ((int64_t)j.units + kDqThreads * kDqUnroll - 1) / (kDqThreads * kDqUnroll);
+        if (b > mx) mx = b;
     }
-    if (blocks == 0) return MQ_OK;
-    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, tab);
+    if (mx == 0) return MQ_OK;
+    tab.max_blocks = (int32_t)mx;
+    hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)mx, (unsigned)n), dim3(kDqThreads), 0, st, tab);
     return mq_check_launch("fp8 block dequant");
 }
 

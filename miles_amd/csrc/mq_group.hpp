@@ -15,11 +15,11 @@ constexpr int kMaxGroup = 64;
 constexpr int kXcds = 8;
 
 // work item (after remap) of this workgroup, or -1 if it falls past the end
-__device__ __forceinline__ int64_t xcd_contiguous_item(int64_t total) {
-    const int64_t per = (total + kXcds - 1) / kXcds;
-    const int64_t bid = blockIdx.x;
-    const int64_t x = bid % kXcds, k = bid / kXcds;
-    const int64_t item = x * per + k;
+__device__ __forceinline__ int32_t xcd_contiguous_item(int32_t total) {
+    const int32_t per = (total + kXcds - 1) / kXcds;
+    const int32_t bid = blockIdx.x;
+    const int32_t x = bid % kXcds, k = bid / kXcds;
+    const int32_t item = x * per + k;
     return (k < per && item < total) ? item : -1;
 }
 inline int64_t xcd_grid(int64_t total) { return ((total + kXcds - 1) / kXcds) * kXcds; }
@@ -35,8 +35,8 @@ struct TileJob {      // one 2-D tensor cut into 128x128 tiles
 };
 struct TileTable {
     int32_t n;
-    int32_t pad;
-    int64_t end[kMaxGroup];   // running count of tiles: tensor i owns [end[i-1], end[i])
+    int32_t total;            // all work items of the launch
+    int32_t end[kMaxGroup];   // running count of tiles: tensor i owns [end[i-1], end[i]); INT32_MAX past n
     TileJob job[kMaxGroup];
 };
 
@@ -47,18 +47,49 @@ struct FlatJob {      // one tensor seen as a flat run of 16-byte input units
     void* aux;        // NVFP4: amax word; unused otherwise
     int64_t units;
 };
+// Flat kernels are launched on a 2-D grid: blockIdx.y selects the tensor, blockIdx.x the workgroup inside
+// it, so a workgroup reads its descriptor with one scalar load and no search.  grid.x is the largest
+// per-tensor workgroup count of the group; the batched driver only groups tensors of similar size.
 struct FlatTable {
     int32_t n;
-    int32_t pad;
-    int64_t end[kMaxGroup];   // running count of workgroups
+    int32_t max_blocks;
     FlatJob job[kMaxGroup];
 };
+// workgroups a tensor of `units` 16-byte units needs when each covers `per_block` units; fills max_blocks
+inline bool flat_grid(FlatTable& tab, int64_t per_block) {
+    int64_t mx = 0;
+    for (int i = 0; i < tab.n; i++) {
+        const int64_t b = (tab.job[i].units + per_block - 1) / per_block;
+        if (b > mx) mx = b;
+    }
+    tab.max_blocks = (int32_t)mx;
+    return mx < 0x7FFFFFF0;
+}
 
+// Index of the tensor that owns work item `item`: the number of running counts not above it.  The loop has
+// a fixed trip count and no early exit, so the compiler fetches the whole `end` array with a few wide scalar
+// loads and the comparison chain runs on the scalar unit: a short, latency-free prologue even for
+// workgroups that only move a few KiB.
+struct JobRef {
+    int ji;         // index into tab.job
+    int32_t start;  // first work item of that tensor
+};
 template <class Table>
-__device__ __forceinline__ int find_job(const Table& tab, int64_t item) {
-    int i = 0;
-    while (i < tab.n - 1 && item >= tab.end[i]) i++;
-    return i;
+__device__ __forceinline__ JobRef find_job(const Table& tab, int32_t item) {
+    JobRef r{0, 0};
+#pragma unroll
+    for (int i = 0; i < kMaxGroup - 1; i++) {
+        const bool past = item >= tab.end[i];
+        r.ji += past ? 1 : 0;
+        r.start = past ? tab.end[i] : r.start;
+    }
+    return r;
+}
+// host side: after end[0..n) holds the running counts, record the total and pad the rest of `end`
+template <class Table>
+inline void seal_table(Table& tab) {
+    tab.total = tab.n > 0 ? tab.end[tab.n - 1] : 0;
+    for (int i = tab.n > 0 ? tab.n - 1 : 0; i < kMaxGroup; i++) tab.end[i] = 0x7FFFFFFF;
 }
 
 }  // namespace mq

@@ -26,7 +26,7 @@ constexpr float kSymCons = 1.0f / 7.0f;
 constexpr float kAsymCons = 1.0f / 15.0f;
 constexpr int kI4Threads = 256;
 #ifndef MQ_I4_UNROLL
-#define MQ_I4_UNROLL 1
+#define MQ_I4_UNROLL 2
 #endif
 constexpr int kI4Unroll = MQ_I4_UNROLL;
 
@@ -44,15 +44,14 @@ __device__ __forceinline__ uint32_t code_bits(float q) { return f2u(q + 12582920
 
 template <int LANES>
 __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTable tab) {
-    const int64_t item = blockIdx.x;
-    const int ji = find_job(tab, item);
-    const FlatJob& job = tab.job[ji];
+    const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
     uint16_t* __restrict__ scale = (uint16_t*)job.s;
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (item - (ji ? tab.end[ji - 1] : 0)) * (kI4Threads * kI4Unroll);
+    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll);
+    if (base >= total_units) return;
     u32x4 v[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
@@ -182,15 +181,9 @@ bool mq_int4_pack_fast_ok(const void* w, int dtype, int group) {
 }
 
 int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st) {
-    int64_t blocks = 0;
-    const int64_t per_block = kI4Threads * kI4Unroll;
-    for (int i = 0; i < tab.n; i++) {
-        blocks += (tab.job[i].units + per_block - 1) / per_block;
-        tab.end[i] = blocks;
-    }
-    if (blocks == 0) return MQ_OK;
-    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    dim3 grid((unsigned)blocks), blk(kI4Threads);
+    if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) return MQ_OK;
+    dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kI4Threads);
     if (group == 128) hipLaunchKernelGGL(int4_pack_bf16_kernel<16>, grid, blk, 0, st, tab);
     else if (group == 64) hipLaunchKernelGGL(int4_pack_bf16_kernel<8>, grid, blk, 0, st, tab);
     else hipLaunchKernelGGL(int4_pack_bf16_kernel<4>, grid, blk, 0, st, tab);

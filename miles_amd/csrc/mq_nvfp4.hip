@@ -17,30 +17,34 @@ namespace mq {
 
 constexpr int kNvThreads = 256;
 #ifndef MQ_NV_UNROLL
-#define MQ_NV_UNROLL 1
+#define MQ_NV_UNROLL 2
 #endif
 constexpr int kNvUnroll = MQ_NV_UNROLL;
 constexpr float kSixth = 0.16666667163372040f;  // 0x3E2AAAAB
 
-// one 16-byte unit per lane; job.units counts whole units, job.s holds the element count so that the
-// last workgroup of a tensor can fold in a tail shorter than one unit
+// kAmaxUnroll 16-byte units per lane; job.units counts whole units, job.s holds the element count so that
+// the first workgroup of a tensor can fold in a tail shorter than one unit
+constexpr int kAmaxUnroll = 8;
 __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable tab) {
     __shared__ uint32_t wave_amax[4];
-    const int64_t item = blockIdx.x;
-    const int ji = find_job(tab, item);
-    const FlatJob& job = tab.job[ji];
+    const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ amax_bits = (uint32_t*)job.aux;
     const int64_t n16 = job.units, numel = (int64_t)(uintptr_t)job.s;
     const int t = threadIdx.x;
-    const int64_t local = item - (ji ? tab.end[ji - 1] : 0);
-    const int64_t unit = local * 256 + t;
-    uint32_t m = 0;
-    if (unit < n16) {
-        const u32x4 v = ld16_keep(w + unit * 8);
-        m = hmax_u16(max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+    const int64_t base = (int64_t)blockIdx.x * (256 * kAmaxUnroll);
+    if (base >= n16 && !(blockIdx.x == 0 && numel > 0)) return;
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int i = 0; i < kAmaxUnroll; i++) {
+        const int64_t unit = base + i * 256 + t;
+        if (unit < n16) {
+            const u32x4 v = ld16_keep(w + unit * 8);
+            m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+        }
     }
-    if (local == 0 && t == 0)
+    uint32_t m = hmax_u16(m2);
+    if (blockIdx.x == 0 && t == 0)
         for (int64_t i = n16 * 8; i < numel; i++) m = umax(m, (uint32_t)(w[i] & 0x7FFFu));
     m = wave_max(m);
     if ((t & 63) == 0) wave_amax[t >> 6] = m;
@@ -89,17 +93,15 @@ __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
 }
 
 __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float numer) {
-    const int64_t item = blockIdx.x;
-    const int ji = find_job(tab, item);
-    const FlatJob& job = tab.job[ji];
+    const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
     const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
     const int64_t total_units = job.units;
-    const int64_t local = item - (ji ? tab.end[ji - 1] : 0);
     const int t = threadIdx.x;
-    const int64_t base = local * (kNvThreads * kNvUnroll);
+    const int64_t base = (int64_t)blockIdx.x * (kNvThreads * kNvUnroll);
+    if (base >= total_units) return;
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
@@ -188,37 +190,28 @@ bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q) {
 
 // tab.job[i]: w, aux = amax word, units = numel / 8, s = (void*)numel
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
-    int64_t blocks = 0;
-    for (int i = 0; i < tab.n; i++) {
-        int64_t b = (tab.job[i].units + 255) / 256;
-        if (b < 1 && (int64_t)(uintptr_t)tab.job[i].s > 0) b = 1;
-        blocks += b;
-        tab.end[i] = blocks;
-    }
-    if (blocks == 0) return MQ_OK;
-    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, tab);
+    if (!flat_grid(tab, 256 * kAmaxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) tab.max_blocks = 1;   // tensors shorter than one unit still have a tail
+    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(256), 0, st, tab);
     return mq_check_launch("nvfp4 amax");
 }
 
 // tab.job[i]: w, q, s = block scales, aux = amax word, units = numel / 8; global_out[i] may be null
 int mq_nvfp4_quant_launch_group(FlatTable& tab, float* const* global_out, int e4m3_max, hipStream_t st) {
     const float numer = (float)e4m3_max * 6.0f;
-    int64_t blocks = 0;
-    const int64_t per_block = kNvThreads * kNvUnroll;
     NvGlobalTable gt{};
     gt.n = tab.n;
     bool any_global = false;
     for (int i = 0; i < tab.n; i++) {
-        blocks += (tab.job[i].units + per_block - 1) / per_block;
-        tab.end[i] = blocks;
         gt.amax[i] = (const uint32_t*)tab.job[i].aux;
         gt.out[i] = global_out ? global_out[i] : nullptr;
         any_global |= gt.out[i] != nullptr;
     }
     if (any_global) hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(64), 0, st, gt, numer);
-    if (blocks > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    if (blocks > 0) hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)blocks), dim3(kNvThreads), 0, st, tab, numer);
+    if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks > 0)
+        hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0,
+                           st, tab, numer);
     return mq_check_launch("nvfp4 quant");
 }
 

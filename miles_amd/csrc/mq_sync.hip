@@ -96,11 +96,16 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
     hipStream_t st = (hipStream_t)stream;
     while (i < j) {
         // a chunk ends at the group / byte limit, but never between two jobs that share an amax word
-        int64_t k = i, bytes = 0;
+        int64_t k = i, bytes = 0, mx = 0;
         while (k < j) {
             const bool tied = k > i && jobs[k].aux == jobs[k - 1].aux;
             const int64_t b = jobs[k].rows * jobs[k].cols * (jobs[k].dtype == MQ_F32 ? 4 : 2);
-            if (!tied && k > i && (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0)) break;
+            const int64_t nmx = b > mx ? b : mx;
+            const bool ragged = nmx * (k - i + 1) * 4 > (bytes + b) * 5;
+            if (!tied && k > i &&
+                (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 || ragged))
+                break;
+            mx = nmx;
             if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax word");
             bytes += b;
             k++;
@@ -173,10 +178,18 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
             i++;
             continue;
         }
-        int64_t j = i + 1;
+        // flat kinds run on a (largest tensor) x (tensors) grid: keep the padding of a group under 25 %
+        const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST;
+        int64_t j = i + 1, sum = head.rows * head.cols, mx = sum;
         while (j < n && j - i < kMaxGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
-               jobs[j].cols > 0)
+               jobs[j].cols > 0) {
+            const int64_t e = jobs[j].rows * jobs[j].cols;
+            const int64_t nmx = e > mx ? e : mx;
+            if (flat && nmx * (j - i + 1) * 4 > (sum + e) * 5) break;
+            sum += e;
+            mx = nmx;
             j++;
+        }
         const int cnt = (int)(j - i);
         int rc = MQ_OK;
         switch (head.kind) {
