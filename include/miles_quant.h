@@ -26,6 +26,9 @@ extern "C" {
 #endif
 
 #define MQ_VERSION 1
+#define MQ_NVFP4_SECTION_WORDS 256
+#define MQ_NVFP4_SECTIONS 4
+#define MQ_NVFP4_RECORD_WORDS (MQ_NVFP4_SECTION_WORDS * MQ_NVFP4_SECTIONS)
 
 enum { MQ_BF16 = 0, MQ_F16 = 1, MQ_F32 = 2 };
 enum { MQ_OK = 0, MQ_ERR_ARG = -1, MQ_ERR_HIP = -2, MQ_ERR_UNSUPPORTED = -3 };
@@ -75,15 +78,19 @@ int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* sc
                              int group, void* stream);
 
 /* NVFP4                                              miles/utils/nvfp4.py:54-114
- * mq_nvfp4_amax: amax_bits[0] = max(amax_bits[0], bits(max|w|)) -- clear it with mq_fill_u32 first; call it
- * once per tensor of a gate/up pair to share one amax (nvfp4.py:100-103).
+ * The global amax travels on the device in an "amax record": MQ_NVFP4_RECORD_WORDS uint32 words made of
+ * MQ_NVFP4_SECTIONS sections of MQ_NVFP4_SECTION_WORDS partial maxima (float bit patterns).  Each tensor that
+ * shares the amax writes ONE whole section (no atomics, nothing to clear beforehand); the amax is the maximum
+ * over the first n_sections sections.  A single tensor uses section 0 with n_sections = 1; a gate/up pair
+ * uses sections 0 and 1 with n_sections = 2 (nvfp4.py:100-103).
+ * mq_nvfp4_amax: record section <- partial maxima of |w| (every word of the section is written).
  * mq_nvfp4_quant: w [M,K] contiguous, K % 16 == 0; q [M,K/2] (element 2i in the low nibble);
  *   block_scale [M,K/16] e4m3fn bytes; global_scale (may be NULL) receives weight_scale_2 =
  *   1 / min(e4m3_max*6/amax, FLT_MAX) as one fp32 (nvfp4.py:19-39). */
 int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream);
-int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* amax_bits, void* stream);
-int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, void* q, void* block_scale, float* global_scale,
-                   int64_t M, int64_t K, int e4m3_max, void* stream);
+int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream);
+int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
+                   float* global_scale, int64_t M, int64_t K, int e4m3_max, void* stream);
 
 /* Batched driver: runs a list of quantization jobs on one stream, in order, with the same results as calling
  * the single-tensor entry points one by one.  Consecutive jobs of the same kind are fused into grouped
@@ -99,11 +106,11 @@ int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, void* q, voi
  *   MQ_JOB_FP8_DEQUANT          e4m3          bf16          -              aux = fp32 tile scales (in) block, -
  *   MQ_JOB_MXFP8                w             e4m3          E8M0 bytes     -                           -
  *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
- *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = uint32 amax word,     e4m3_max, -
+ *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, -
  *                                                                          aux2 = fp32 weight_scale_2
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere.
- * NVFP4: the driver clears each amax word, reduces every job's tensor into its word and then quantizes; jobs
- * that share one amax word (a gate/up pair) must be adjacent in the list. */
+ * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
+ * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list. */
 enum {
     MQ_JOB_FP8_BLOCK = 0,
     MQ_JOB_FP8_BLOCKWISE_CAST = 1,

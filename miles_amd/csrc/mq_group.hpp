@@ -44,8 +44,11 @@ struct FlatJob {      // one tensor seen as a flat run of 16-byte input units
     const void* w;
     void* q;
     void* s;
-    void* aux;        // NVFP4: amax word; unused otherwise
+    void* aux;        // NVFP4: amax record; unused otherwise
     int64_t units;
+    void* aux2;       // NVFP4: fp32 global scale output; unused otherwise
+    int32_t section;  // NVFP4 amax: section of the record to write; quantize: number of sections to read
+    int32_t pad;
 };
 // Flat kernels are launched on a 2-D grid: blockIdx.y selects the tensor, blockIdx.x the workgroup inside
 // it, so a workgroup reads its descriptor with one scalar load and no search.  grid.x is the largest

@@ -201,7 +201,7 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
     if (mq_int4_pack_fast_ok(w, dtype, group)) {
         FlatTable tab{};
         tab.n = 1;
-        tab.job[0] = FlatJob{w, packed, scale, nullptr, units};
+        tab.job[0] = FlatJob{w, packed, scale, nullptr, units, nullptr, 0, 0};
         return mq_int4_pack_launch_group(tab, group, st);
     }
     int64_t blocks = (units + 255) / 256;

@@ -120,7 +120,7 @@ extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale,
     if (mq_mxfp8_fast_ok(w, dtype, q)) {
         FlatTable tab{};
         tab.n = 1;
-        tab.job[0] = FlatJob{w, q, scale, nullptr, groups * 4};
+        tab.job[0] = FlatJob{w, q, scale, nullptr, groups * 4, nullptr, 0, 0};
         return mq_mxfp8_launch_group(tab, st);
     }
     int64_t blocks = (groups + 255) / 256;

@@ -6,9 +6,12 @@
 //              inv = min(1 / (f32(s8) * S_dec), FLT_MAX);  code = sat_e2m1(x * inv)
 //   published global scale: 1 / min(e4m3_max*6/amax, FLT_MAX) with only the ==0 repair (nvfp4.py:19-39)
 //
-// Pass 1 (mq_nvfp4_amax) reduces max|x| to one uint32 with one atomic per workgroup; a gate/up pair calls
-// it twice on the same word.  Pass 2 (mq_nvfp4_quant): two lanes own one block (16 bytes each), the block
-// amax is one DPP step, and each lane emits four bytes of codes.
+// Pass 1 (mq_nvfp4_amax): 256 workgroups per tensor stream its elements and each writes one partial maximum
+// into the tensor's section of the amax record: plain stores, no atomics (thousands of agent-scope atomics
+// on one address serialise at ~8 ns each on this multi-XCD part) and nothing to clear.  Pass 2
+// (mq_nvfp4_quant): every workgroup first folds the record's sections into the amax (one cached load per
+// lane), then two lanes own one 16-element block (16 bytes each), the block amax is one DPP step, and each
+// lane emits four bytes of codes.  A gate/up pair writes two sections of one record.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -22,26 +25,39 @@ constexpr int kNvThreads = 256;
 constexpr int kNvUnroll = MQ_NV_UNROLL;
 constexpr float kSixth = 0.16666667163372040f;  // 0x3E2AAAAB
 
-// kAmaxUnroll 16-byte units per lane; job.units counts whole units, job.s holds the element count so that
-// the first workgroup of a tensor can fold in a tail shorter than one unit
-constexpr int kAmaxUnroll = 8;
+constexpr int kSectionWords = MQ_NVFP4_SECTION_WORDS;   // = workgroups of the amax pass per tensor
+constexpr int kAmaxUnroll = 4;                          // 16-byte units per lane per loop trip
+
+// amax of a record: lanes read the partial maxima of the first n_sections sections, then a workgroup max
+__device__ __forceinline__ float record_amax(const uint32_t* rec, int n_sections, uint32_t* lds4) {
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < n_sections * kSectionWords; i += blockDim.x) m = umax(m, rec[i]);
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = m;
+    __syncthreads();
+    return u2f(umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3])));
+}
+
+// grid (kSectionWords, tensors): workgroup b of a tensor strides over its 16 KiB chunks and writes word b of
+// the section.  job.units counts whole 16-byte units; job.s carries the element count for the sub-unit tail.
 __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable tab) {
     __shared__ uint32_t wave_amax[4];
     const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
-    uint32_t* __restrict__ amax_bits = (uint32_t*)job.aux;
+    uint32_t* __restrict__ section = (uint32_t*)job.aux + job.section * kSectionWords;
     const int64_t n16 = job.units, numel = (int64_t)(uintptr_t)job.s;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (256 * kAmaxUnroll);
-    if (base >= n16 && !(blockIdx.x == 0 && numel > 0)) return;
     uint32_t m2 = 0;
+    for (int64_t base = (int64_t)blockIdx.x * (256 * kAmaxUnroll); base < n16; base += (int64_t)kSectionWords * 256 * kAmaxUnroll) {
+        u32x4 v[kAmaxUnroll];
 #pragma unroll
-    for (int i = 0; i < kAmaxUnroll; i++) {
-        const int64_t unit = base + i * 256 + t;
-        if (unit < n16) {
-            const u32x4 v = ld16_keep(w + unit * 8);
-            m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+        for (int i = 0; i < kAmaxUnroll; i++) {
+            const int64_t unit = base + i * 256 + t;
+            v[i] = unit < n16 ? ld16_keep(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
         }
+#pragma unroll
+        for (int i = 0; i < kAmaxUnroll; i++)
+            m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w))));
     }
     uint32_t m = hmax_u16(m2);
     if (blockIdx.x == 0 && t == 0)
@@ -49,15 +65,11 @@ __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable ta
     m = wave_max(m);
     if ((t & 63) == 0) wave_amax[t >> 6] = m;
     __syncthreads();
-    if (t == 0) {
-        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3])) << 16;
-        // most workgroups lose against the running maximum: read it first, touch the atomic only to raise it
-        if (m > __hip_atomic_load(amax_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(amax_bits, m);
-    }
+    if (t == 0) section[blockIdx.x] = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3])) << 16;
 }
 
 __global__ __launch_bounds__(256) void nvfp4_amax_generic_kernel(const void* __restrict__ w, int dtype, int64_t numel,
-                                                                 uint32_t* __restrict__ amax_bits) {
+                                                                 uint32_t* __restrict__ section) {
     __shared__ uint32_t wave_amax[4];
     const int t = threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -67,10 +79,7 @@ __global__ __launch_bounds__(256) void nvfp4_amax_generic_kernel(const void* __r
     m = wave_max(m);
     if ((t & 63) == 0) wave_amax[t >> 6] = m;
     __syncthreads();
-    if (t == 0) {
-        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
-        if (m) atomicMax(amax_bits, m);
-    }
+    if (t == 0) section[blockIdx.x] = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
 }
 
 struct NvScales {
@@ -101,15 +110,17 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
     const int64_t base = (int64_t)blockIdx.x * (kNvThreads * kNvUnroll);
-    if (base >= total_units) return;
+    if (base >= total_units && blockIdx.x != 0) return;
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
         v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
     }
-    const float amax = u2f(amax_bits[0]);
+    __shared__ uint32_t lds4[4];
+    const float amax = record_amax(amax_bits, job.section, lds4);
     const NvScales gs = nv_scales(amax, numer);
+    if (job.aux2 && blockIdx.x == 0 && t == 0) *(float*)job.aux2 = nv_published_scale(amax, numer);
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
@@ -143,24 +154,13 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     }
 }
 
-// weight_scale_2 of every tensor of a group: out[i] = 1 / min(numer / amax_i, FLT_MAX) (zero repaired to 1)
-struct NvGlobalTable {
-    int32_t n;
-    int32_t pad;
-    const uint32_t* amax[kMaxGroup];
-    float* out[kMaxGroup];
-};
-__global__ void nvfp4_global_scale_kernel(const NvGlobalTable tab, float numer) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < tab.n && tab.out[i]) *tab.out[i] = nv_published_scale(u2f(*tab.amax[i]), numer);
-}
-
 __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __restrict__ w, int dtype,
-                                                                  const uint32_t* __restrict__ amax_bits,
+                                                                  const uint32_t* __restrict__ amax_bits, int n_sections,
                                                                   uint8_t* __restrict__ q, uint8_t* __restrict__ s8,
                                                                   float* __restrict__ global_scale, float numer,
                                                                   int64_t blocks16) {
-    const float amax = u2f(amax_bits[0]);
+    __shared__ uint32_t lds4[4];
+    const float amax = record_amax(amax_bits, n_sections, lds4);
     const NvScales gs = nv_scales(amax, numer);
     if (global_scale && blockIdx.x == 0 && threadIdx.x == 0) *global_scale = nv_published_scale(amax, numer);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -188,55 +188,44 @@ bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q) {
     return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 4) == 0;
 }
 
-// tab.job[i]: w, aux = amax word, units = numel / 8, s = (void*)numel
+// tab.job[i]: w, aux = amax record, section, units = numel / 8, s = (void*)numel
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
-    if (!flat_grid(tab, 256 * kAmaxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    if (tab.max_blocks == 0) tab.max_blocks = 1;   // tensors shorter than one unit still have a tail
-    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(256), 0, st, tab);
+    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3(kSectionWords, (unsigned)tab.n), dim3(256), 0, st, tab);
     return mq_check_launch("nvfp4 amax");
 }
 
-// tab.job[i]: w, q, s = block scales, aux = amax word, units = numel / 8; global_out[i] may be null
-int mq_nvfp4_quant_launch_group(FlatTable& tab, float* const* global_out, int e4m3_max, hipStream_t st) {
+// tab.job[i]: w, q, s = block scales, aux = amax record, section = sections to read, aux2 = fp32 global scale
+// out (may be null), units = numel / 8
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st) {
     const float numer = (float)e4m3_max * 6.0f;
-    NvGlobalTable gt{};
-    gt.n = tab.n;
-    bool any_global = false;
-    for (int i = 0; i < tab.n; i++) {
-        gt.amax[i] = (const uint32_t*)tab.job[i].aux;
-        gt.out[i] = global_out ? global_out[i] : nullptr;
-        any_global |= gt.out[i] != nullptr;
-    }
-    if (any_global) hipLaunchKernelGGL(nvfp4_global_scale_kernel, dim3(1), dim3(64), 0, st, gt, numer);
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    if (tab.max_blocks > 0)
-        hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0,
-                           st, tab, numer);
+    if (tab.max_blocks == 0) tab.max_blocks = 1;   // an empty tensor still publishes its global scale
+    hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0, st,
+                       tab, numer);
     return mq_check_launch("nvfp4 quant");
 }
 
-extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* amax_bits, void* stream) {
-    if (!w || !amax_bits) return mq_fail(MQ_ERR_ARG, "null pointer");
+extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream) {
+    if (!w || !record) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
-    if (numel == 0) return MQ_OK;
+    if (section < 0 || section >= MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section");
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0) {
         FlatTable tab{};
         tab.n = 1;
-        tab.job[0] = FlatJob{w, nullptr, (void*)(uintptr_t)numel, amax_bits, numel / 8};
+        tab.job[0] = FlatJob{w, nullptr, (void*)(uintptr_t)numel, record, numel / 8, nullptr, section, 0};
         return mq_nvfp4_amax_launch_group(tab, st);
     }
-    int64_t blocks = (numel + 255) / 256;
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(nvfp4_amax_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, numel,
-                       (uint32_t*)amax_bits);
+    hipLaunchKernelGGL(nvfp4_amax_generic_kernel, dim3(kSectionWords), dim3(256), 0, st, w, dtype, numel,
+                       (uint32_t*)record + section * kSectionWords);
     return mq_check_launch("nvfp4 amax");
 }
 
-extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, void* q, void* block_scale,
+extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
                               float* global_scale, int64_t M, int64_t K, int e4m3_max, void* stream) {
-    if (!w || !amax_bits || !q || !block_scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (!w || !record || !q || !block_scale) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (n_sections < 1 || n_sections > MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section count");
     if (K % 16 != 0) return mq_fail(MQ_ERR_ARG, "Last dim must be divisible by 16 for NVFP4");
     if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");
     hipStream_t st = (hipStream_t)stream;
@@ -245,12 +234,13 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* amax_bits, v
     if (blocks16 == 0 || mq_nvfp4_fast_ok(w, dtype, q)) {
         FlatTable tab{};
         tab.n = 1;
-        tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(amax_bits), blocks16 * 2};
-        return mq_nvfp4_quant_launch_group(tab, &global_scale, e4m3_max, st);
+        tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), blocks16 * 2, global_scale, n_sections, 0};
+        return mq_nvfp4_quant_launch_group(tab, e4m3_max, st);
     }
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
-                       (const uint32_t*)amax_bits, (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer, blocks16);
+                       (const uint32_t*)record, n_sections, (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer,
+                       blocks16);
     return mq_check_launch("nvfp4 quant");
 }

@@ -24,19 +24,7 @@ bool mq_int4_pack_fast_ok(const void* w, int dtype, int group);
 int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st);
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
-int mq_nvfp4_quant_launch_group(FlatTable& tab, float* const* global_out, int e4m3_max, hipStream_t st);
-
-namespace mq {
-struct WordTable {
-    int32_t n;
-    int32_t pad;
-    uint32_t* p[kMaxGroup];
-};
-__global__ void clear_words_kernel(const WordTable tab) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < tab.n) *tab.p[i] = 0u;
-}
-}  // namespace mq
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st);
 
 // The amax pass and the quantize pass of an NVFP4 group read the same input; keeping a group's input
 // below this many bytes lets the second read be served by the 256 MB memory-side cache.
@@ -106,15 +94,18 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
                 (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 || ragged))
                 break;
             mx = nmx;
-            if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax word");
+            if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
             bytes += b;
             k++;
         }
         const int n = (int)(k - i);
-        WordTable words{};
-        words.n = n;
-        for (int t = 0; t < n; t++) words.p[t] = (uint32_t*)jobs[i + t].aux;
-        hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(64), 0, st, words);
+        // section of each job inside its record, and how many sections the record ends up with
+        int section[kMaxGroup], sections[kMaxGroup];
+        for (int t = 0; t < n; t++) section[t] = (t > 0 && jobs[i + t].aux == jobs[i + t - 1].aux) ? section[t - 1] + 1 : 0;
+        for (int t = n - 1; t >= 0; t--)
+            sections[t] = (t + 1 < n && jobs[i + t + 1].aux == jobs[i + t].aux) ? sections[t + 1] : section[t] + 1;
+        for (int t = 0; t < n; t++)
+            if (section[t] >= MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
         bool all_fast = true;
         for (int t = 0; t < n; t++) all_fast &= job_fast(jobs[i + t]);
         if (all_fast) {
@@ -123,28 +114,26 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
                 const int64_t numel = jb.rows * jb.cols;
-                tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8};
+                tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8, nullptr, section[t], 0};
             }
             int rc = mq_nvfp4_amax_launch_group(tab, st);
             if (rc) return rc;
-            float* gout[kMaxGroup];
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
-                tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8};
-                gout[t] = (float*)jb.aux2;
+                tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, sections[t], 0};
             }
-            rc = mq_nvfp4_quant_launch_group(tab, gout, jobs[i].p0, st);
+            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, st);
             if (rc) return rc;
         } else {
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
-                int rc = mq_nvfp4_amax(jb.in, jb.dtype, jb.rows * jb.cols, jb.aux, stream);
+                int rc = mq_nvfp4_amax(jb.in, jb.dtype, jb.rows * jb.cols, jb.aux, section[t], stream);
                 if (rc) return rc;
             }
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
-                int rc = mq_nvfp4_quant(jb.in, jb.dtype, jb.aux, jb.out, jb.scale, (float*)jb.aux2, jb.rows, jb.cols,
-                                        jb.p0, stream);
+                int rc = mq_nvfp4_quant(jb.in, jb.dtype, jb.aux, sections[t], jb.out, jb.scale, (float*)jb.aux2, jb.rows,
+                                        jb.cols, jb.p0, stream);
                 if (rc) return rc;
             }
         }

@@ -18,6 +18,7 @@ from miles_amd import _lib, launch
 FP4_E2M1_MAX = 6.0
 FP8_E4M3_MAX = 448.0
 NVFP4_GROUP_SIZE = 16
+AMAX_RECORD_WORDS = 1024   # MQ_NVFP4_RECORD_WORDS: per-workgroup partial maxima of a tensor (or pair) on the device
 
 
 def nvfp4_weight_e4m3_max() -> int:
@@ -64,7 +65,7 @@ def nvfp4_quantize_1d(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor,
     w = weight.contiguous()
     if w.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {w.shape[1]}.")
-    word = torch.empty(1, dtype=torch.int32, device=w.device)   # cleared and reduced into by the job driver
+    word = torch.empty(AMAX_RECORD_WORDS, dtype=torch.int32, device=w.device)   # written by the amax pass of the job driver
     out = _alloc_outputs(w)
     launch.submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max)
     return out
@@ -84,7 +85,7 @@ def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
     a, b = first.contiguous(), second.contiguous()
     if a.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {a.shape[1]}.")
-    word = torch.empty(1, dtype=torch.int32, device=a.device)
+    word = torch.empty(AMAX_RECORD_WORDS, dtype=torch.int32, device=a.device)
     outs = (_alloc_outputs(a), _alloc_outputs(b))
     # two adjacent jobs on one amax word: the driver reduces both tensors before it quantizes either
     with _pair_scope() as submit:
