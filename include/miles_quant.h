@@ -108,7 +108,8 @@ int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections,
  *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
  *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, -
  *                                                                          aux2 = fp32 weight_scale_2
- * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere.
+ * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
+ * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
  * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list. */
 enum {
@@ -129,6 +130,10 @@ typedef struct mq_job {
     void* aux2;
     int64_t rows, cols, ld;
     int32_t p0, p1;
+    /* FP8 quantizers only: the input rows come in blocks of rows_per_block consecutive rows (stride ld) whose
+     * first rows are block_stride elements apart -- e.g. the q / k / v rows of a fused per-group QKV weight,
+     * read in place.  0 / 0 = one block (plain matrix).  rows_per_block must be a multiple of the tile height. */
+    int64_t rows_per_block, block_stride;
 } mq_job;
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 

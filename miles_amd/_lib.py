@@ -44,7 +44,7 @@ class Job(_c.Structure):
 
     _fields_ = [("kind", _c.c_int32), ("dtype", _c.c_int32), ("inp", _vp), ("out", _vp), ("scale", _vp),
                 ("aux", _vp), ("aux2", _vp), ("rows", _i64), ("cols", _i64), ("ld", _i64), ("p0", _c.c_int32),
-                ("p1", _c.c_int32)]
+                ("p1", _c.c_int32), ("rows_per_block", _i64), ("block_stride", _i64)]
 
 
 _lib = None

@@ -40,6 +40,11 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
     const int64_t col = tj * kTile + (t & 15) * 8;
     const int64_t row0 = ti * kTile + (t >> 4);
     const bool col_ok = col < K;  // K % 8 == 0: an 8-wide segment is entirely inside or outside
+    // row-blocked input: the tile's rows sit in block ti / tiles_per_block, at the same offset inside it
+    if (job.tiles_per_block > 0) {
+        const int64_t blk = ti / job.tiles_per_block;
+        w += blk * job.block_stride - blk * job.tiles_per_block * (int64_t)kTile * ldw;
+    }
 
     u32x4 v[kRowsPerThread];
 #pragma unroll
@@ -321,7 +326,7 @@ static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int
     if (mq_fp8_tile_fast_ok(w, dtype, sxm, sxn, q, M, K, bm, bk)) {
         TileTable tab{};
         tab.n = 1;
-        tab.job[0] = TileJob{w, q, scale, sxm, (int32_t)M, (int32_t)K, 0, 0};
+        tab.job[0] = TileJob{w, q, scale, sxm, (int32_t)M, (int32_t)K, 0, 0, 0};
         return mq_fp8_tile_launch_group(mode, tab, stream);
     }
     const int64_t tiles_m = (M + bm - 1) / bm, tiles_k = (K + bk - 1) / bk;

@@ -31,7 +31,8 @@ struct TileJob {      // one 2-D tensor cut into 128x128 tiles
     int64_t ldw;      // input row stride, elements
     int32_t M, K;
     int32_t tiles_k;
-    int32_t pad;
+    int32_t tiles_per_block;  // tile rows per input row block (row-blocked inputs), 0 = plain matrix
+    int64_t block_stride;     // elements between the first rows of consecutive row blocks
 };
 struct TileTable {
     int32_t n;

@@ -34,7 +34,8 @@ static bool job_fast(const mq_job& j) {
     switch (j.kind) {
         case MQ_JOB_FP8_BLOCK:
         case MQ_JOB_FP8_BLOCKWISE_CAST:
-            return mq_fp8_tile_fast_ok(j.in, j.dtype, j.ld, 1, j.out, j.rows, j.cols, j.p0, j.p1);
+            return mq_fp8_tile_fast_ok(j.in, j.dtype, j.ld, 1, j.out, j.rows, j.cols, j.p0, j.p1) &&
+                   (j.block_stride % 8) == 0;
         case MQ_JOB_FP8_DEQUANT:
             return mq_fp8_dequant_fast_ok(j.in, j.out, j.rows, j.cols, j.p0);
         case MQ_JOB_MXFP8:
@@ -53,7 +54,12 @@ static int check_job(const mq_job& j) {
     if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
-    if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax word");
+    if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
+    if (j.rows_per_block != 0) {
+        const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST;
+        if (!fp8q || j.rows_per_block < 0 || j.rows_per_block % 128 != 0 || j.p0 != 128 || j.p1 != 128 || j.dtype != MQ_BF16)
+            return mq_fail(MQ_ERR_ARG, "row-blocked input needs a bf16 FP8 128x128 job with rows_per_block % 128 == 0");
+    }
     return MQ_OK;
 }
 
@@ -162,6 +168,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
         }
         if (head.rows == 0 || head.cols == 0) { i++; continue; }
         if (!job_fast(head)) {
+            if (head.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "row-blocked input is not 16-byte aligned");
             int rc = run_single(head, stream);
             if (rc) return rc;
             i++;
@@ -188,7 +195,8 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) {
                     const mq_job& jb = jobs[i + t];
-                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, jb.ld, (int32_t)jb.rows, (int32_t)jb.cols, 0, 0};
+                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, jb.ld, (int32_t)jb.rows, (int32_t)jb.cols, 0,
+                                         (int32_t)(jb.rows_per_block / 128), jb.block_stride};
                 }
                 rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : 1, tab, st);
                 break;

@@ -24,16 +24,31 @@ def fp8_blockwise_cast(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, 
     """x [M, N] (any strides) -> (float8_e4m3fn [M, N] contiguous, float32 [ceil(M/bm), ceil(N/bn)]).
 
     Per tile: absmax = max(max|x|, 1e-10); scale = absmax / 448; y = e4m3(clamp(x * (1 / scale), +-448)).
+
+    Extension used by the sync driver: x may also be a 3-D view [B, R, N] whose rows are contiguous
+    (strides (s, N, 1)) with R a multiple of 128 -- B blocks of R rows, e.g. the q rows of a fused per-group
+    QKV weight.  It is quantized in place as the [B*R, N] matrix it stands for, without a regrouping copy.
     """
     bm, bn = (128, 128) if not block_size else (int(block_size[0]), int(block_size[1]))
     _lib.require_gpu(x, "fp8_blockwise_cast")
     _lib.dtype_code(x, "fp8_blockwise_cast")
+    if x.dim() == 3:
+        B, R, N = x.shape
+        if not (x.stride(2) == 1 and x.stride(1) == N and R % 128 == 0 and (bm, bn) == (128, 128)
+                and x.dtype == torch.bfloat16):
+            return fp8_blockwise_cast(x.reshape(B * R, N), block_size)
+        M = B * R
+        y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
+        s = torch.empty(ceil_div(M, bm), ceil_div(N, bn), dtype=torch.float32, device=x.device)
+        launch.submit(_lib.JOB_FP8_BLOCKWISE_CAST, x, y, s, None, None, M, N, N, bm, bn, R, x.stride(0))
+        return y, s
     M, N = x.shape
     y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
     s = torch.empty(ceil_div(M, bm), ceil_div(N, bn), dtype=torch.float32, device=x.device)
     if x.stride(1) == 1 or N <= 1:
         launch.submit(_lib.JOB_FP8_BLOCKWISE_CAST, x, y, s, None, None, M, N, x.stride(0), bm, bn)
     else:  # general column stride: direct entry point, not batchable
+        launch.note_direct_call()
         rc = _lib.load().mq_fp8_blockwise_cast(x.data_ptr(), _lib.dtype_code(x, "fp8_blockwise_cast"), x.stride(0),
                                                x.stride(1), y.data_ptr(), s.data_ptr(), M, N, bm, bn,
                                                _lib.stream_ptr(x.device))

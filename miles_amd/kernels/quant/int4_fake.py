@@ -31,6 +31,7 @@ def fake_int4_quant_cuda(x: torch.Tensor, block_size, sym: bool):
     out = torch.empty_like(xc)
     scale = torch.empty((M, -(-N // block_n)), dtype=x.dtype, device=x.device)
     zero = torch.empty_like(scale)  # left unwritten in symmetric mode, as in the reference
+    launch.note_direct_call()
     rc = _lib.load().mq_int4_fake_quant(xc.data_ptr(), _lib.dtype_code(x, "fake_int4_quant_cuda"), out.data_ptr(),
                                         scale.data_ptr(), zero.data_ptr(), M, N, block_n, int(bool(sym)),
                                         _lib.stream_ptr(x.device))

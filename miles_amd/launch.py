@@ -11,6 +11,7 @@ launch-bound without changing the per-tensor call signatures.
 from __future__ import annotations
 
 import contextlib
+import ctypes
 import threading
 
 import torch
@@ -28,12 +29,15 @@ class JobBatch:
         self._keep: list[torch.Tensor] = []
         self._array = None
         self.device = None
+        self.direct_calls = 0   # kernels launched inside the block without going through the job list
 
     def __len__(self) -> int:
         return len(self._records)
 
-    def add(self, kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1, keep=()) -> None:
-        self._records.append((kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1))
+    def add(self, kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1, rows_per_block=0,
+            block_stride=0, keep=()) -> None:
+        self._records.append((kind, dtype, inp, out, scale, aux, aux2, rows, cols, ld, p0, p1, rows_per_block,
+                              block_stride))
         self._keep.extend(keep)
         self._array = None
 
@@ -47,12 +51,21 @@ class JobBatch:
         return self._array
 
     def run(self, stream: int | None = None) -> None:
-        if not self._records:
+        self.run_range(0, len(self._records), stream)
+
+    def run_range(self, start: int, stop: int, stream: int | None = None) -> None:
+        """Submit jobs [start, stop) of the list (a cut never separates two NVFP4 jobs sharing a record,
+        because callers cut at parameter boundaries)."""
+        if stop <= start:
             return
         arr = self.freeze()
         if stream is None:
             stream = _lib.stream_ptr(self.device)
-        _lib.check(_lib.load().mq_run_jobs(arr, len(self._records), stream))
+        ptr = ctypes.byref(arr, start * ctypes.sizeof(_lib.Job))
+        _lib.check(_lib.load().mq_run_jobs(ptr, stop - start, stream))
+
+    def input_pointers(self) -> list[int]:
+        return [rec[2] for rec in self._records]
 
 
 def active_batch() -> JobBatch | None:
@@ -61,9 +74,15 @@ def active_batch() -> JobBatch | None:
 
 @contextlib.contextmanager
 def deferred():
-    """Record the quantizer calls made inside the block and submit them together on exit."""
-    if active_batch() is not None:
-        raise _lib.MilesQuantError("deferred() blocks do not nest")
+    """Record the quantizer calls made inside the block and submit them together on exit.
+
+    Inside an enclosing `deferred()` / `recording()` block this is a pass-through: the jobs join the outer
+    batch and run when that one does.
+    """
+    outer = active_batch()
+    if outer is not None:
+        yield outer
+        return
     batch = JobBatch()
     _state.batch = batch
     try:
@@ -73,11 +92,34 @@ def deferred():
     batch.run()
 
 
-def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0) -> None:
+@contextlib.contextmanager
+def recording():
+    """Like `deferred()`, but nothing is submitted on exit: the caller keeps the batch and runs (and re-runs)
+    it with `JobBatch.run` / `JobBatch.run_range`."""
+    if active_batch() is not None:
+        raise _lib.MilesQuantError("recording() cannot start inside another batch")
+    batch = JobBatch()
+    _state.batch = batch
+    try:
+        yield batch
+    finally:
+        _state.batch = None
+
+
+def note_direct_call() -> None:
+    """Called by wrappers whose kernel cannot be expressed as a job and is launched at once; a recorded batch
+    that saw one cannot reproduce the whole computation on replay."""
+    batch = active_batch()
+    if batch is not None:
+        batch.direct_calls += 1
+
+
+def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0,
+           rows_per_block=0, block_stride=0) -> None:
     """Run (or record) one job.  Tensor arguments may be None where the job kind has no such operand."""
     rec = (kind, _lib.DTYPE_CODE.get(inp.dtype, 0), inp.data_ptr(), out.data_ptr(),
            scale.data_ptr() if scale is not None else None, aux.data_ptr() if aux is not None else None,
-           aux2.data_ptr() if aux2 is not None else None, rows, cols, ld, p0, p1)
+           aux2.data_ptr() if aux2 is not None else None, rows, cols, ld, p0, p1, rows_per_block, block_stride)
     keep = [t for t in (inp, out, scale, aux, aux2) if t is not None]
     batch = active_batch()
     if batch is not None:

@@ -43,6 +43,7 @@ def _scaled_fp8(weight: torch.Tensor, per_channel: bool):
     q = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((n, 1) if per_channel else (1,), dtype=torch.float32, device=w.device)
     ws = torch.empty(max(n, 1), dtype=torch.int32, device=w.device)
+    launch.note_direct_call()
     floor = float(torch.tensor(1e-12, dtype=w.dtype).float())  # clamp(min=1e-12) acts in the weight dtype
     rc = _lib.load().mq_fp8_scaled_quant(w.data_ptr(), _lib.dtype_code(w, "fp8"), w.stride(0), q.data_ptr(),
                                          scale.data_ptr(), ws.data_ptr(), n, k, int(per_channel), floor,

@@ -1,0 +1,94 @@
+"""Weight-sync driver: streams quantized HF buckets of a model to a consumer.
+
+Single-process form of the reference's `WeightUpdater.update_weights`
+(miles/backends/training_utils/weight_update/updater.py:123-171): the engine session calls, Gloo barriers and
+transfer protocols of the reference are outside this path; what remains is the loop
+`for bucket in iterator.iter_hf_weights(weights): protocol.send_bucket(bucket)` wrapped in the same two
+wall-clock spans ("update_weights_implementation", "finalize_and_resume_engines").  `send_bucket` is any
+callable taking a list of (hf_name, tensor).  After the first sync the recorded `SyncPlan` is replayed as long
+as the parameter set is unchanged.
+"""
+
+from __future__ import annotations
+
+import time
+from argparse import Namespace
+from collections.abc import Callable, Mapping
+
+import torch
+
+from miles_amd.weight_update.bucketing import Unit
+from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorDirect
+from miles_amd.weight_update.sync_plan import SyncPlan
+
+
+def _fp8_row_block_views_ok(args: Namespace, quantization_config: dict | None) -> bool:
+    """q / k / v can be quantized in place when every group's row block is a whole number of 128-row tiles."""
+    if not quantization_config or quantization_config.get("quant_method") != "fp8":
+        return False
+    if list(quantization_config.get("weight_block_size") or []) != [128, 128]:
+        return False
+    try:
+        kv = getattr(args, "kv_channels", None)
+        head_dim = kv if kv is not None else args.hidden_size // args.num_attention_heads
+        q_per_group = args.num_attention_heads // args.num_query_groups
+    except AttributeError:
+        return False
+    return head_dim % 128 == 0 and (head_dim * q_per_group) % 128 == 0 and args.hidden_size % 8 == 0
+
+
+class WeightUpdater:
+    def __init__(self, args: Namespace, *, weights_getter: Callable[[], Mapping[str, torch.Tensor]], model_name: str,
+                 quantization_config: dict | None, send_bucket: Callable[[Unit], None],
+                 packed_weight_basenames: set[str] | None = None, use_plan: bool = True) -> None:
+        self.args = Namespace(**vars(args))
+        if _fp8_row_block_views_ok(self.args, quantization_config):
+            self.args.qkv_row_block_views = True
+        self.weights_getter = weights_getter
+        self.send_bucket = send_bucket
+        self.use_plan = use_plan
+        self.weight_version = 0
+        self._iterator = _RowBlockAwareIterator(self.args, model_name=model_name,
+                                                quantization_config=quantization_config,
+                                                packed_weight_basenames=packed_weight_basenames)
+        self._plan: SyncPlan | None = None
+        self._metrics: dict[str, float] = {}
+
+    def pop_metrics(self) -> dict[str, float]:
+        """Wall-clock spans of the last sync, in seconds; cleared by the call."""
+        out, self._metrics = self._metrics, {}
+        return out
+
+    @torch.no_grad()
+    def update_weights(self) -> None:
+        self.weight_version += 1
+        weights = self.weights_getter()
+        t0 = time.perf_counter()
+        for bucket in self._iter_buckets(weights):
+            self.send_bucket(bucket)
+        t1 = time.perf_counter()
+        self._metrics["update_weights_implementation"] = t1 - t0
+        self._metrics["finalize_and_resume_engines"] = time.perf_counter() - t1
+
+    def _iter_buckets(self, weights):
+        if not self.use_plan:
+            yield from self._iterator.iter_hf_weights(weights)
+            return
+        if self._plan is not None and self._plan.matches(weights):
+            yield from self._plan.replay()
+            return
+        self._plan = SyncPlan.record(self._iterator, weights)
+        yield from self._plan.buckets
+
+
+class _RowBlockAwareIterator(HfWeightIteratorDirect):
+    """Flattens row-blocked [groups, rows, hidden] views that ended up unquantized back to 2-D."""
+
+    def _convert_batch(self, named_params):
+        units = super()._convert_batch(named_params)
+        if getattr(self.args, "qkv_row_block_views", False):
+            for unit in units:
+                for i, (name, t) in enumerate(unit):
+                    if t.dim() == 3 and name.endswith(("q_proj.weight", "k_proj.weight", "v_proj.weight")):
+                        unit[i] = (name, t.reshape(-1, t.shape[-1]))
+        return units

@@ -1,0 +1,332 @@
+"""Host-side logic of the sync path on the CPU: bucketing, gather batches, name maps and the quantizer
+dispatch (with the kernels replaced by shape-only stand-ins).  The bucketing cases restate the reference's
+tests/fast/backends/training_utils/weight_update/test_bucketing.py and
+tests/fast/backends/megatron_utils/test_hf_weight_iterator_direct.py:109-120; the dispatch cases restate
+tests/fast-gpu/test_mxfp8_quantizer.py:85-147 and tests/fast-gpu/test_nvfp4_quantizer.py:146-231."""
+
+from argparse import Namespace
+
+import pytest
+import torch
+
+from miles_amd.megatron_to_hf import convert_to_hf, name_maps
+from miles_amd.megatron_to_hf import processors as P
+from miles_amd.megatron_to_hf.processors import quantizer_fp8, quantizer_mxfp8, quantizer_nvfp4
+from miles_amd.utils.mxfp8 import should_use_mxfp8
+from miles_amd.weight_update.bucketing import (AtomicUpdateGroup, assemble_atomic_update_groups,
+                                               get_hf_atomic_update_groups, pack_units_by_size)
+from miles_amd.weight_update.hf_weight_iterator import ParamInfo, _pack_param_infos_by_size
+
+
+def _unit(*names, numel=4):
+    return [(name, torch.zeros(numel, dtype=torch.uint8)) for name in names]
+
+
+def _names(units):
+    return [[n for n, _ in u] for u in units]
+
+
+PAIR = AtomicUpdateGroup("pair", (".b.weight", ".c.weight"))
+
+
+class TestAtomicGroups:
+    def test_ungrouped_units_stream_through(self):
+        opt = AtomicUpdateGroup("pair", (".b.weight", ".c.weight"), optional=True)
+        out = list(assemble_atomic_update_groups([_unit("layers.0.a.weight"), _unit("layers.1.a.weight")], [opt]))
+        assert _names(out) == [["layers.0.a.weight"], ["layers.1.a.weight"]]
+
+    def test_members_merge_in_suffix_order(self):
+        units = [_unit("layers.0.a.weight"), _unit("layers.0.c.weight"), _unit("layers.0.b.weight")]
+        out = list(assemble_atomic_update_groups(units, [PAIR]))
+        assert _names(out) == [["layers.0.a.weight"], ["layers.0.b.weight", "layers.0.c.weight"]]
+
+    def test_merge_is_per_prefix(self):
+        units = [_unit("layers.0.b.weight"), _unit("layers.1.b.weight"), _unit("layers.1.c.weight"),
+                 _unit("layers.0.c.weight")]
+        out = list(assemble_atomic_update_groups(units, [PAIR]))
+        assert _names(out) == [["layers.1.b.weight", "layers.1.c.weight"], ["layers.0.b.weight", "layers.0.c.weight"]]
+
+    def test_scales_ride_with_their_weight(self):
+        units = [_unit("layers.0.b.weight", "layers.0.b.weight_scale_inv"),
+                 _unit("layers.0.c.weight", "layers.0.c.weight_scale_inv")]
+        out = list(assemble_atomic_update_groups(units, [PAIR]))
+        assert _names(out) == [["layers.0.b.weight", "layers.0.b.weight_scale_inv", "layers.0.c.weight",
+                                "layers.0.c.weight_scale_inv"]]
+
+    def test_empty_units_are_skipped(self):
+        assert _names(assemble_atomic_update_groups([[], _unit("layers.0.a.weight")], [])) == [["layers.0.a.weight"]]
+
+    @pytest.mark.parametrize("units,groups,message", [
+        ([_unit("layers.0.b.weight")], [PAIR], "Incomplete atomic update groups"),
+        ([_unit("layers.0.a.weight")], [PAIR], "matched no params"),
+        ([_unit("layers.0.b.weight", "layers.0.c.weight")], [PAIR], "matches multiple"),
+        ([], [AtomicUpdateGroup("empty", ())], "has no suffixes"),
+        ([], [AtomicUpdateGroup("dup", (".a", ".a"))], "duplicate suffixes"),
+        ([], [AtomicUpdateGroup("k", (".a",)), AtomicUpdateGroup("k", (".b",))], "Duplicate atomic update group keys"),
+    ])
+    def test_errors(self, units, groups, message):
+        with pytest.raises(AssertionError, match=message):
+            list(assemble_atomic_update_groups(units, groups))
+
+    def test_optional_group_may_match_nothing(self):
+        opt = AtomicUpdateGroup("pair", (".b.weight", ".c.weight"), optional=True)
+        assert len(list(assemble_atomic_update_groups([_unit("layers.0.a.weight")], [opt]))) == 1
+
+    def test_model_groups(self):
+        assert get_hf_atomic_update_groups("qwen3") == []
+        assert [g.key for g in get_hf_atomic_update_groups("DeepSeek-V3", q_lora_rank=1536)] == ["q_lora_a_proj"]
+        assert [g.key for g in get_hf_atomic_update_groups("deepseek_v4")][0] == "wqkv_a"
+        assert get_hf_atomic_update_groups("deepseekv41")[0].suffixes == (".attn.wq_a.weight", ".attn.wkv.weight")
+
+
+class TestPacking:
+    def test_bucket_closes_when_next_unit_would_reach_the_limit(self):
+        units = [_unit("a"), _unit("b"), _unit("c")]
+        assert _names(pack_units_by_size(units, max_bytes=9)) == [["a", "b"], ["c"]]
+        assert _names(pack_units_by_size(units, max_bytes=8)) == [["a"], ["b"], ["c"]]   # 4 + 4 >= 8 closes
+
+    def test_units_are_never_split(self):
+        assert _names(pack_units_by_size([_unit("a"), _unit("b1", "b2")], max_bytes=6)) == [["a"], ["b1", "b2"]]
+
+    def test_empty_stream(self):
+        assert list(pack_units_by_size([], max_bytes=8)) == []
+
+    def test_gather_batches_by_size_only(self):
+        infos = [ParamInfo(n, torch.float32, torch.Size([s]), s) for n, s in [("layer.a", 4), ("layer.b", 2), ("layer.c", 4)]]
+        args = Namespace(update_weight_buffer_size=6)
+        assert [[i.name for i in b] for b in _pack_param_infos_by_size(args, infos)] == [["layer.a", "layer.b"], ["layer.c"]]
+        assert [[i.name for i in b] for b in _pack_param_infos_by_size(args, infos, size_multiplier=2)] == \
+            [["layer.a"], ["layer.b"], ["layer.c"]]
+
+
+# ---------------------------------------------------------------------------------------------------------
+QWEN_ARGS = Namespace(hidden_size=64, num_attention_heads=4, num_query_groups=2, kv_channels=16, vocab_size=100,
+                      num_layers=4)
+
+
+class TestNameMaps:
+    def test_qwen2_layer(self):
+        L = "module.module.decoder.layers.3."
+        qkv = torch.arange((4 + 2 * 2) * 16 * 64, dtype=torch.float32).reshape(-1, 64)
+        out = name_maps.convert_qwen2_to_hf(QWEN_ARGS, L + "self_attention.linear_qkv.weight", qkv)
+        assert [n for n, _ in out] == [f"model.layers.3.self_attn.{p}_proj.weight" for p in "qkv"]
+        q, k, v = (t for _, t in out)
+        assert q.shape == (64, 64) and k.shape == (32, 64) and v.shape == (32, 64)
+        grouped = qkv.view(2, 4, 16, 64)     # per group: 2 q heads, 1 k, 1 v
+        assert torch.equal(q, grouped[:, :2].reshape(-1, 64)) and torch.equal(k, grouped[:, 2].reshape(-1, 64))
+        assert torch.equal(v, grouped[:, 3].reshape(-1, 64))
+        fc1 = torch.randn(40, 64)
+        gate_up = name_maps.convert_qwen2_to_hf(QWEN_ARGS, L + "mlp.linear_fc1.weight", fc1)
+        assert [n for n, _ in gate_up] == ["model.layers.3.mlp.gate_proj.weight", "model.layers.3.mlp.up_proj.weight"]
+        gate, up = gate_up[0][1], gate_up[1][1]
+        assert gate.data_ptr() == fc1.data_ptr() and up.data_ptr() == fc1[20:].data_ptr()   # views, not copies
+        for rest, hf in [("self_attention.linear_proj.weight", "self_attn.o_proj.weight"),
+                         ("mlp.linear_fc2.weight", "mlp.down_proj.weight"),
+                         ("self_attention.linear_qkv.layer_norm_weight", "input_layernorm.weight"),
+                         ("mlp.linear_fc1.layer_norm_weight", "post_attention_layernorm.weight"),
+                         ("self_attention.q_layernorm.weight", "self_attn.q_norm.weight")]:
+            assert name_maps.convert_qwen2_to_hf(QWEN_ARGS, L + rest, fc1)[0][0] == "model.layers.3." + hf
+        assert name_maps.convert_qwen2_to_hf(QWEN_ARGS, "module.module.embedding.word_embeddings.weight", fc1)[0][0] \
+            == "model.embed_tokens.weight"
+        with pytest.raises(ValueError, match="Unknown parameter name"):
+            name_maps.convert_qwen2_to_hf(QWEN_ARGS, L + "mlp.router.weight", fc1)
+
+    def test_row_block_views_opt_in(self):
+        args = Namespace(**vars(QWEN_ARGS), qkv_row_block_views=True)
+        qkv = torch.randn((4 + 2 * 2) * 16, 64)
+        out = name_maps.convert_qwen2_to_hf(args, "module.module.decoder.layers.0.self_attention.linear_qkv.weight", qkv)
+        ref = name_maps.convert_qwen2_to_hf(QWEN_ARGS, "module.module.decoder.layers.0.self_attention.linear_qkv.weight", qkv)
+        for (n, view), (n2, copy) in zip(out, ref):
+            assert n == n2 and view.dim() == 3 and view.untyped_storage().data_ptr() == qkv.untyped_storage().data_ptr()
+            assert torch.equal(view.reshape(-1, 64), copy)
+
+    def test_moe_experts(self):
+        fc1 = torch.randn(32, 64)
+        L = "module.module.decoder.layers.7."
+        for fn, shared in [(name_maps.convert_qwen3moe_to_hf, "shared_expert"), (name_maps.convert_deepseekv3_to_hf, "shared_experts")]:
+            out = fn(QWEN_ARGS, L + "mlp.experts.linear_fc1.weight12", fc1)
+            assert [n for n, _ in out] == ["model.layers.7.mlp.experts.12.gate_proj.weight",
+                                           "model.layers.7.mlp.experts.12.up_proj.weight"]
+            assert fn(QWEN_ARGS, L + "mlp.experts.linear_fc2.weight3", fc1)[0][0] == "model.layers.7.mlp.experts.3.down_proj.weight"
+            assert fn(QWEN_ARGS, L + "mlp.shared_experts.linear_fc2.weight", fc1)[0][0] == f"model.layers.7.mlp.{shared}.down_proj.weight"
+            assert fn(QWEN_ARGS, L + "mlp.router.weight", fc1)[0][0] == "model.layers.7.mlp.gate.weight"
+        out = name_maps.convert_deepseekv3_to_hf(QWEN_ARGS, L + "self_attention.linear_kv_down_proj.weight", fc1)
+        assert out[0][0] == "model.layers.7.self_attn.kv_a_proj_with_mqa.weight"
+        out = name_maps.convert_deepseekv3_to_hf(QWEN_ARGS, "module.module.mtp.layers.0.eh_proj.weight", fc1)
+        assert out[0][0] == "model.layers.4.eh_proj.weight"
+        out = name_maps.convert_deepseekv3_to_hf(QWEN_ARGS, "module.module.mtp.layers.1.transformer_layer.mlp.linear_fc2.weight", fc1)
+        assert out[0][0] == "model.layers.5.mlp.down_proj.weight"
+
+    def test_convert_to_hf_strips_vocab_padding_and_picks_family(self):
+        emb = torch.randn(128, 64)
+        out = convert_to_hf(QWEN_ARGS, "qwen3", "module.module.embedding.word_embeddings.weight", emb)
+        assert out[0][1].shape == (100, 64)
+        with pytest.raises(ValueError, match="Unsupported model"):
+            convert_to_hf(QWEN_ARGS, "mystery", "module.module.embedding.word_embeddings.weight", emb)
+
+
+# ---------------------------------------------------------------------------------------------------------
+@pytest.fixture
+def fake_kernels(monkeypatch):
+    """Shape-only stand-ins for the GPU quantizers so that the dispatch logic runs on the CPU."""
+    calls = []
+
+    def fake_cast(w, block_size=None):
+        calls.append(("fp8", tuple(w.shape)))
+        return torch.zeros(w.shape, dtype=torch.uint8), torch.zeros(1)
+
+    def fake_tensor(w):
+        calls.append(("fp8_tensor", tuple(w.shape)))
+        return torch.zeros(w.shape, dtype=torch.uint8), torch.zeros(1)
+
+    def fake_mx(w):
+        calls.append(("mxfp8", tuple(w.shape)))
+        return torch.zeros(w.shape, dtype=torch.uint8), torch.zeros((*w.shape[:-1], w.shape[-1] // 32), dtype=torch.uint8)
+
+    def nv_outputs(w):
+        return torch.zeros(w.shape[0], w.shape[1] // 2, dtype=torch.uint8), torch.zeros(w.shape[0], w.shape[1] // 16), torch.ones(())
+
+    def fake_nv(w):
+        calls.append(("nvfp4", tuple(w.shape)))
+        return nv_outputs(w)
+
+    def fake_pair(a, b):
+        calls.append(("nvfp4_pair", tuple(a.shape), tuple(b.shape)))
+        return nv_outputs(a), nv_outputs(b)
+
+    monkeypatch.setattr(quantizer_fp8, "fp8_blockwise_cast", fake_cast)
+    monkeypatch.setattr(quantizer_fp8, "tensor_fp8", fake_tensor)
+    monkeypatch.setattr(quantizer_mxfp8, "mxfp8_quantize", fake_mx)
+    monkeypatch.setattr(quantizer_nvfp4, "nvfp4_quantize_1d", fake_nv)
+    monkeypatch.setattr(quantizer_nvfp4, "nvfp4_quantize_1d_pair", fake_pair)
+    return calls
+
+
+FP8_CFG = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
+W = torch.zeros(4, 32, dtype=torch.bfloat16)
+
+
+class TestDispatch:
+    def test_none_config_and_unmatched_names_return_the_same_list(self, fake_kernels):
+        params = [("model.norm.weight", W)]
+        assert P.quantize_params(None, "module.module.decoder.final_layernorm.weight", params, None) is params
+        for cfg in (FP8_CFG, {"quant_method": "mxfp8"}, {"quant_method": "nvfp4"}):
+            assert P.quantize_params(None, "module.module.decoder.final_layernorm.weight", params, cfg) is params
+            assert P.quantize_params(None, "module.module.decoder.layers.0.self_attention.q_layernorm.weight", params, cfg) is params
+        assert fake_kernels == []
+
+    def test_fp8_names_and_scale_suffix(self, fake_kernels):
+        params = [("model.layers.0.self_attn.o_proj.weight", W)]
+        out = P.quantize_params(None, "module.module.decoder.layers.0.self_attention.linear_proj.weight", params, FP8_CFG)
+        assert [n for n, _ in out] == ["model.layers.0.self_attn.o_proj.weight", "model.layers.0.self_attn.o_proj.weight_scale_inv"]
+        cfg = {k: v for k, v in FP8_CFG.items() if k != "weight_block_size"}
+        out = P.quantize_params(None, "module.module.decoder.layers.0.self_attention.linear_proj.weight", params, cfg)
+        assert [n for n, _ in out][1] == "model.layers.0.self_attn.o_proj.weight_scale" and fake_kernels[-1][0] == "fp8_tensor"
+
+    def test_fp8_experts_drop_bf16_scale_entries_and_mtp_layers_match(self, fake_kernels):
+        params = [("model.layers.1.mlp.experts.5.down_proj.weight", W), ("model.layers.1.mlp.experts.5.down_proj.weight_scale", W)]
+        out = P.quantize_params(None, "module.module.decoder.layers.1.mlp.experts.linear_fc2.weight5", params, FP8_CFG)
+        assert [n for n, _ in out] == ["model.layers.1.mlp.experts.5.down_proj.weight", "model.layers.1.mlp.experts.5.down_proj.weight_scale_inv"]
+        out = P.quantize_params(None, "module.module.mtp.layers.0.transformer_layer.mlp.linear_fc2.weight",
+                                [("model.layers.4.mlp.down_proj.weight", W)], FP8_CFG)
+        assert len(out) == 2
+        shared = P.quantize_params(None, "module.module.decoder.layers.1.mlp.shared_experts.linear_fc1.weight",
+                                   [("a.gate_proj.weight", W), ("a.up_proj.weight", W)], FP8_CFG)
+        assert len(shared) == 4
+
+    def test_fp8_honours_modules_to_not_convert_and_indexer_flag(self, fake_kernels):
+        cfg = dict(FP8_CFG, modules_to_not_convert=["model.layers.0.self_attn.o_proj"])
+        params = [("model.layers.0.self_attn.o_proj.weight", W)]
+        out = P.quantize_params(None, "module.module.decoder.layers.0.self_attention.linear_proj.weight", params, cfg)
+        assert out == params and fake_kernels == []
+        wk = [("model.layers.0.self_attn.indexer.wk.weight", W)]
+        name = "module.module.decoder.layers.0.self_attention.wk.weight"
+        assert len(P.quantize_params(Namespace(indexer_rope_interleave=False), name, wk, FP8_CFG)) == 2
+        assert P.quantize_params(Namespace(indexer_rope_interleave=True), name, wk, FP8_CFG) is wk
+
+    def test_fused_module_must_be_skipped_whole(self):
+        mapping = {"qkv_proj": ["q_proj", "k_proj", "v_proj"]}
+        assert quantizer_fp8.is_layer_skipped("m.qkv_proj", ["m.q_proj", "m.k_proj", "m.v_proj"], mapping)
+        assert not quantizer_fp8.is_layer_skipped("m.qkv_proj", [], mapping)
+        with pytest.raises(ValueError, match="some but not all shards"):
+            quantizer_fp8.is_layer_skipped("m.qkv_proj", ["m.q_proj"], mapping)
+
+    def test_mxfp8_respects_extra_high_precision_and_bf16_head_tail(self, fake_kernels):
+        params = [("model.layers.0.mlp.experts.0.down_proj.weight", W)]
+        cfg = {"quant_method": "mxfp8"}
+        args = Namespace(extra_high_precision_layers_megatron=("linear_fc2",))
+        assert P.quantize_params(args, "decoder.layers.0.mlp.experts.linear_fc2.weight0", params, cfg) is params
+        args = Namespace(first_last_layers_bf16=True, num_layers=4, num_layers_at_start_in_bf16=1, num_layers_at_end_in_bf16=1)
+        for layer in (0, 3):
+            assert P.quantize_params(args, f"decoder.layers.{layer}.mlp.experts.linear_fc2.weight0", params, cfg) is params
+        out = P.quantize_params(args, "decoder.layers.1.mlp.experts.linear_fc2.weight0", params, cfg)
+        assert [n for n, _ in out] == ["model.layers.0.mlp.experts.0.down_proj.weight", "model.layers.0.mlp.experts.0.down_proj.weight_scale_inv"]
+        assert out[1][1].dtype == torch.uint8
+
+    def test_should_use_mxfp8(self):
+        name = "model.layers.0.mlp.experts.0.down_proj.weight"
+        assert should_use_mxfp8(name, (4, 32), torch.bfloat16)
+        assert not should_use_mxfp8(name, (4, 32), torch.bfloat16, skip_substrings=("mlp.experts.0",))
+        assert should_use_mxfp8(name, (4, 32), torch.bfloat16, skip_substrings=("mlp.experts.1",))
+        assert not should_use_mxfp8(name, (4, 48), torch.bfloat16) and not should_use_mxfp8(name, (32,), torch.bfloat16)
+        assert not should_use_mxfp8("model.norm.weight", (4, 32), torch.bfloat16)
+        assert not should_use_mxfp8(name, (4, 32), torch.float8_e4m3fn) and should_use_mxfp8(name, (4, 32), torch.float8_e4m3fn, allow_source_fp8=True)
+        assert should_use_mxfp8(name, (4, 16), torch.uint8, packed_mxfp4_experts=True)
+
+    def test_nvfp4_pairs_gate_and_up_and_names_outputs(self, fake_kernels):
+        cfg = {"quant_method": "nvfp4"}
+        fc1 = [("model.layers.0.mlp.experts.0.gate_proj.weight", W), ("model.layers.0.mlp.experts.0.up_proj.weight", W)]
+        out = P.quantize_params(None, "decoder.layers.0.mlp.experts.linear_fc1.weight0", fc1, cfg)
+        assert [n for n, _ in out] == [f"model.layers.0.mlp.experts.0.{p}_proj.{s}" for p in ("gate", "up")
+                                       for s in ("weight", "weight_scale", "weight_scale_2")]
+        assert fake_kernels == [("nvfp4_pair", (4, 32), (4, 32))]
+        assert not any(n.endswith("input_scale") for n, _ in out)
+        down = [("model.layers.0.mlp.experts.0.down_proj.weight", W)]
+        assert len(P.quantize_params(None, "module.module.decoder.layers.0.mlp.experts.linear_fc2.weight0", down, cfg)) == 3
+        # dense layers, MTP layers and non-decoder towers stay in high precision
+        dense = [("model.layers.0.mlp.down_proj.weight", W)]
+        assert P.quantize_params(None, "module.module.decoder.layers.0.mlp.linear_fc2.weight", dense, cfg) is dense
+        assert P.quantize_params(None, "module.module.mtp.layers.0.mlp.experts.linear_fc2.weight0", down, cfg) is down
+
+    def test_nvfp4_errors_and_ignore_rules(self, fake_kernels):
+        cfg = {"quant_method": "nvfp4"}
+        gate_only = [("model.layers.0.mlp.experts.0.gate_proj.weight", W)]
+        with pytest.raises(ValueError, match="requires gate/up tensors to be quantized together"):
+            P.quantize_params(None, "decoder.layers.0.mlp.experts.linear_fc1.weight0", gate_only, cfg)
+        with pytest.raises(ValueError, match="must be divisible by 16"):
+            P.quantize_params(None, "decoder.layers.0.mlp.experts.linear_fc2.weight0",
+                              [("model.layers.0.mlp.experts.0.down_proj.weight", torch.zeros(4, 24, dtype=torch.bfloat16))], cfg)
+        with pytest.raises(NotImplementedError, match="fp4-param-gather"):
+            P.quantize_params(Namespace(fp4_param=True), "decoder.layers.0.mlp.experts.linear_fc2.weight0", gate_only, cfg)
+        args = Namespace(extra_high_precision_layers_megatron=("linear_fc1",))
+        assert P.quantize_params(args, "decoder.layers.0.mlp.experts.linear_fc1.weight0", gate_only, cfg) is gate_only
+        down = [("model.layers.0.mlp.experts.0.down_proj.weight", W)]
+        for rules in (["model.layers.0.mlp.experts"], ["re:model\\.layers\\.0\\..*"], "model.layers.0"):
+            out = P.quantize_params(None, "decoder.layers.0.mlp.experts.linear_fc2.weight0", down, dict(cfg, ignore=rules))
+            assert out == down
+        out = P.quantize_params(None, "decoder.layers.0.mlp.experts.linear_fc2.weight0", down,
+                                dict(cfg, exclude_modules=["model.layers.1"]))
+        assert len(out) == 3
+
+    def test_nvfp4_three_dimensional_weights_are_stacked(self, fake_kernels):
+        q, s, g = quantizer_nvfp4.quantize_nvfp4(torch.zeros(3, 4, 32, dtype=torch.bfloat16))
+        assert q.shape == (3, 4, 16) and s.shape == (3, 4, 2) and g.shape == (3,)
+        with pytest.raises(ValueError, match="Unsupported weight rank"):
+            quantizer_nvfp4.quantize_nvfp4(torch.zeros(32))
+
+    def test_compressed_tensors_output_names(self, monkeypatch):
+        from miles_amd.megatron_to_hf.processors import quantizer_compressed_tensors as C
+
+        monkeypatch.setattr(C, "pack_layer", lambda w, g, sym: (torch.zeros(w.shape[0], w.shape[1] // 8, dtype=torch.int32),
+                                                                 torch.zeros(w.shape[0], w.shape[1] // g, dtype=w.dtype), None))
+        cfg = {"quant_method": "compressed-tensors", "format": "pack-quantized",
+               "config_groups": {"group_0": {"weights": {"group_size": 32, "symmetric": True, "num_bits": 4}}}}
+        params = [("model.layers.0.mlp.experts.0.down_proj.weight", W), ("model.layers.0.mlp.gate.weight", W)]
+        out = P.quantize_params(None, "x", params, cfg, {"model.layers.0.mlp.experts.0.down_proj"})
+        assert [n for n, _ in out] == ["model.layers.0.mlp.experts.0.down_proj.weight_packed",
+                                       "model.layers.0.mlp.experts.0.down_proj.weight_scale",
+                                       "model.layers.0.mlp.experts.0.down_proj.weight_shape",
+                                       "model.layers.0.mlp.gate.weight"]
+        assert out[2][1].tolist() == [4, 32] and out[2][1].dtype == torch.int32
+        with pytest.raises(AssertionError, match="packed weight names"):
+            P.quantize_params(None, "x", params, cfg)
