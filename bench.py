@@ -1,0 +1,304 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-quantization hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu-baseline]
+
+One step = one full Qwen3-4B weight sync to FP8 128x128 block scales (BASELINE.json configs[1]): the 36
+layers' Megatron-named bf16 parameters, resident in HBM, stream through the sync driver
+(name map -> fp8_blockwise_cast -> buckets) exactly as a trainer->engine update would, with the consumer
+replaced by a no-op.  `value` is algorithmic GB/s of that sync (input read once + codes and scales written
+once, 3.000244 B/element) and `ms_per_step` the wall-clock milliseconds per full-model sync.
+
+The JSON line also carries
+  roofline      the dominant kernel (fp8_block128_kernel, one grouped launch per bucket) timed live with
+                events on the launch stream; peak = 8 TB/s HBM
+  cpu_baseline  the CPU oracle (bit-exact port) timed on the host cores on a bounded sample of the workload
+  per_quantizer GB/s of every quantizer on its BASELINE.json configuration shape (not part of `value`)
+  parity        a sample of the step's outputs compared byte for byte with the oracle
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from argparse import Namespace
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 + 2, "mxfp8": 2 + 1 + 1 / 32,
+                  "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16}
+# HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
+# scaled by the same counter on a plain copy of known size (profiles/fp8_block128_c2_pmc.md); None until measured
+MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = None
+
+METRIC = "HBM GB/s (% of peak) per quantizer; ms per full-model BF16->FP8 weight sync"
+DEV = "cuda:0"
+
+
+def _synth(shape, gen, *, std=0.02, p=0.001, gain=20.0):
+    """bf16 N(0, std) with a fraction p of entries multiplied by gain, generated on the GPU."""
+    x = torch.randn(shape, generator=gen, device=DEV, dtype=torch.float32) * std
+    if p > 0:
+        x = torch.where(torch.rand(shape, generator=gen, device=DEV) < p, x * gain, x)
+    return x.to(torch.bfloat16)
+
+
+def qwen3_4b_megatron_weights(gen):
+    """Megatron-named parameters of Qwen3-4B: hidden 2560, 32 q heads / 8 kv groups of 128, ffn 9728, 36 layers."""
+    h, heads, groups, hd, ffn, layers, vocab = 2560, 32, 8, 128, 9728, 36, 151936
+    w = {"module.module.embedding.word_embeddings.weight": _synth((vocab, h), gen, p=0)}
+    for i in range(layers):
+        L = f"module.module.decoder.layers.{i}."
+        w[L + "self_attention.linear_qkv.layer_norm_weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
+        w[L + "self_attention.linear_qkv.weight"] = _synth(((heads + 2 * groups) * hd, h), gen)
+        w[L + "self_attention.q_layernorm.weight"] = torch.ones(hd, device=DEV, dtype=torch.bfloat16)
+        w[L + "self_attention.k_layernorm.weight"] = torch.ones(hd, device=DEV, dtype=torch.bfloat16)
+        w[L + "self_attention.linear_proj.weight"] = _synth((h, heads * hd), gen)
+        w[L + "mlp.linear_fc1.layer_norm_weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
+        w[L + "mlp.linear_fc1.weight"] = _synth((2 * ffn, h), gen)
+        w[L + "mlp.linear_fc2.weight"] = _synth((h, ffn), gen)
+    w["module.module.decoder.final_layernorm.weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
+    args = Namespace(hidden_size=h, num_attention_heads=heads, num_query_groups=groups, kv_channels=hd,
+                     vocab_size=vocab, num_layers=layers, update_weight_buffer_size=512 * 1024**2, q_lora_rank=None)
+    quantized_elems = layers * (heads * hd * h + 2 * groups * hd * h + h * heads * hd + 3 * ffn * h)
+    return args, w, quantized_elems
+
+
+def _event_ms(fn, iters):
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def _record(build):
+    """Record the quantizer calls of `build()` into a replayable batch."""
+    from miles_amd import launch
+
+    with launch.recording() as batch:
+        outs = build()
+    batch.device = torch.device(DEV)
+    batch.freeze()
+    batch.run()
+    torch.cuda.synchronize()
+    return batch, outs
+
+
+def per_quantizer(gen):
+    """GB/s of each quantizer on its configuration shape (a bounded number of tensors, replayed batches)."""
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    res = {}
+
+    def run(name, key, elems, build, note):
+        batch, outs = _record(build)
+        ms = _event_ms(batch.run, 5)
+        gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
+        res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+                     "elements": elems, "workload": note}
+        del batch, outs
+        torch.cuda.empty_cache()
+
+    # C1: one Qwen3-4B MLP, block_fp8; 8 distinct copies so that the 256 MB memory-side cache cannot hold the input
+    mlp = [[_synth((9728, 2560), gen), _synth((9728, 2560), gen), _synth((2560, 9728), gen)] for _ in range(8)]
+    mlp[0][0][128:256, 128:256] = 0
+    run("C1_block_fp8", "fp8_block", 8 * 3 * 9728 * 2560,
+        lambda: [block_fp8(t, [128, 128]) for m in mlp for t in m], "8 x Qwen3-4B MLP (gate, up, down), block_fp8")
+    del mlp
+    # C3: Qwen3-30B-A3B experts, MXFP8; 2 layers of 128 experts
+    experts = [(_synth((1536, 2048), gen, p=0), _synth((2048, 768), gen, p=0)) for _ in range(256)]
+    run("C3_mxfp8", "mxfp8", 256 * 3 * 768 * 2048,
+        lambda: [mxfp8_quantize(t) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
+        "2 layers x 128 experts (gate, up [768,2048], down [2048,768])")
+    del experts
+    # C4 / C5: Kimi-K2- / DeepSeek-V3-shaped experts, 32 experts
+    experts = [(_synth((4096, 7168), gen, std=0.015, p=0.0005, gain=30.0), _synth((7168, 2048), gen, std=0.015, p=0.0005, gain=30.0))
+               for _ in range(32)]
+    n = 32 * 3 * 2048 * 7168
+    run("C4_int4_g128_pack", "int4_g128", n,
+        lambda: [pack_layer(t, 128) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
+        "32 experts (gate, up [2048,7168], down [7168,2048]), pack_layer group 128")
+
+    def nvfp4_all():
+        out = []
+        for fc1, fc2 in experts:
+            out.append(nvfp4_quantize_1d_pair(*fc1.chunk(2, dim=0)))
+            out.append(nvfp4_quantize_1d(fc2))
+        return out
+
+    run("C5a_nvfp4", "nvfp4", n, nvfp4_all, "32 experts, gate/up paired + down, amax pass + quantize pass")
+    run("C5b_block_fp8", "fp8_block", n,
+        lambda: [block_fp8(t, [128, 128]) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
+        "32 experts, block_fp8")
+    quantized = [block_fp8(t, [128, 128]) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)]
+    torch.cuda.synchronize()
+    del experts
+    run("C5b_fp8_dequant", "fp8_dequant", n, lambda: [weight_dequant(q, s) for q, s in quantized],
+        "32 experts, FP8 block -> bf16")
+    return res
+
+
+def roofline(plan, jobs_meta):
+    """Time every kernel launch of one sync (same launch partition as a step) with events on the launch stream."""
+    spans = []
+    done = 0
+    for mark in plan.jobs_done_at_bucket:
+        a = done
+        while a < mark:      # mq_run_jobs fuses up to 64 consecutive same-kind jobs into one launch
+            b = min(a + 64, mark)
+            spans.append((a, b))
+            a = b
+        done = max(done, mark)
+    total_ms, total_bytes = 0.0, 0.0
+    reps = 3
+    for _ in range(reps):
+        for a, b in spans:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            plan.batch.run_range(a, b)
+            e1.record()
+            e1.synchronize()
+            total_ms += e0.elapsed_time(e1)
+            total_bytes += sum(jobs_meta[a:b]) * BYTES_PER_ELEM["fp8_block"]
+    launches = reps * len(spans)
+    achieved = total_bytes / total_ms / 1e6
+    elems_per_launch = total_bytes / BYTES_PER_ELEM["fp8_block"] / launches
+    traffic = None if MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM is None else MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems_per_launch
+    return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "launches_per_sync": len(spans), "avg_launch_us": round(total_ms / launches * 1e3, 2),
+            "algorithmic_bytes_per_launch": round(total_bytes / launches)}
+
+
+def cpu_baseline(weights, args, budget_s=12.0):
+    """The oracle's fp8_blockwise_cast on layer 0's HF tensors, repeated until `budget_s` of CPU time is spent."""
+    from miles_amd.megatron_to_hf import name_maps
+    from oracle import mq_oracle
+
+    mq_oracle.build()
+    tensors = []
+    for rest in ("self_attention.linear_qkv.weight", "self_attention.linear_proj.weight", "mlp.linear_fc1.weight",
+                 "mlp.linear_fc2.weight"):
+        name = "module.module.decoder.layers.0." + rest
+        for _hf, t in name_maps.convert_qwen2_to_hf(args, name, weights[name].cpu()):
+            tensors.append(t.contiguous())
+    elems = sum(t.numel() for t in tensors)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        for t in tensors:
+            mq_oracle.fp8_blockwise_cast(t)
+        reps += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(reps * elems * BYTES_PER_ELEM["fp8_block"] / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "kind": "port", "sample": f"{reps} x one Qwen3-4B layer (q,k,v,o,gate,up,down = {elems} elements) through "
+                                       f"the OpenMP C oracle's fp8_blockwise_cast, {dt:.1f} s"}
+
+
+def parity_sample(weights, args, plan):
+    """Byte-compare layer 0's quantized tensors of the timed sync with the oracle."""
+    from miles_amd.megatron_to_hf import name_maps
+    from oracle import mq_oracle
+
+    got = {n: t for bucket in plan.buckets for n, t in bucket}
+    checked = 0
+    for rest in ("self_attention.linear_qkv.weight", "mlp.linear_fc1.weight", "mlp.linear_fc2.weight"):
+        name = "module.module.decoder.layers.0." + rest
+        for hf, t in name_maps.convert_qwen2_to_hf(args, name, weights[name].cpu()):
+            q, s = mq_oracle.fp8_blockwise_cast(t.contiguous())
+            ok = torch.equal(got[hf].cpu().view(torch.uint8), q.view(torch.uint8)) and \
+                torch.equal(got[hf.replace(".weight", ".weight_scale_inv")].cpu(), s)
+            if not ok:
+                raise SystemExit(f"PARITY FAILURE: {hf} differs from the oracle")
+            checked += 1
+    return f"ok ({checked} tensors of layer 0 byte-identical to the oracle)"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-extras", action="store_true", help="skip the per-quantizer section")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs the MI355X: no GPU visible")
+    from miles_amd import _lib
+    from miles_amd.weight_update.updater import WeightUpdater
+
+    _lib.load()   # fails loudly if the HIP library is not built
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(2001)
+    args, weights, elems = qwen3_4b_megatron_weights(gen)
+    fp8_cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
+    sent = {"buckets": 0, "bytes": 0}
+
+    def consume(bucket):
+        sent["buckets"] += 1
+        sent["bytes"] += sum(t.nbytes for _n, t in bucket)
+
+    updater = WeightUpdater(args, weights_getter=lambda: weights, model_name="qwen3", quantization_config=fp8_cfg,
+                            send_bucket=consume)
+    updater.update_weights()          # builds the plan (first sync pays the per-parameter Python work)
+    for _ in range(a.warmup):
+        updater.update_weights()
+    torch.cuda.synchronize()
+    sent.update(buckets=0, bytes=0)
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        updater.update_weights()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / a.steps * 1e3
+    algorithmic_bytes = elems * BYTES_PER_ELEM["fp8_block"]
+    value = algorithmic_bytes / (dt / a.steps) / 1e9
+
+    plan = updater._plan
+    assert plan is not None and plan.replayable, "the benchmark expects the replayable plan path"
+    jobs_meta = [rec[7] * rec[8] for rec in plan.batch._records]     # rows * cols of every job
+    line = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: full Qwen3-4B weight sync to FP8 e4m3 128x128 block scales, 36 layers "
+                               "(q[4096,2560] k/v[1024,2560] o[2560,4096] gate/up[9728,2560] down[2560,9728]), bf16 "
+                               "N(0,0.02) + 0.1% x20 outliers, embeddings and norms passed through as bf16",
+                   "quantizer": "fp8_blockwise_cast (sync path)", "quantized_elements": elems,
+                   "algorithmic_bytes": round(algorithmic_bytes), "buckets_per_sync": sent["buckets"] // max(a.steps, 1),
+                   "bucket_bytes": args.update_weight_buffer_size},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "roofline": roofline(plan, jobs_meta),
+        "parity": parity_sample(weights, args, plan),
+    }
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(weights, args)
+    if not a.no_extras:
+        del updater, plan
+        weights.clear()
+        torch.cuda.empty_cache()
+        line["per_quantizer"] = per_quantizer(gen)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
