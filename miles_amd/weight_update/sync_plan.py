@@ -53,7 +53,8 @@ class SyncPlan:
         batch.freeze()
         replayable = batch.direct_calls == 0 and cls._inputs_alias(weights, batch)
         plan = cls(batch, buckets, marks, weights_signature(weights), replayable)
-        batch.run()
+        for _ in plan.replay():     # the first execution uses the same launch partition as every replay
+            pass
         return plan
 
     @staticmethod
