@@ -28,7 +28,7 @@ extern "C" {
 #define MQ_VERSION 1
 #define MQ_NVFP4_SECTION_WORDS 256
 #define MQ_NVFP4_SECTIONS 4
-#define MQ_NVFP4_RECORD_WORDS (MQ_NVFP4_SECTION_WORDS * MQ_NVFP4_SECTIONS)
+#define MQ_NVFP4_RECORD_WORDS (MQ_NVFP4_SECTION_WORDS * (MQ_NVFP4_SECTIONS + 1))
 
 enum { MQ_BF16 = 0, MQ_F16 = 1, MQ_F32 = 2 };
 enum { MQ_OK = 0, MQ_ERR_ARG = -1, MQ_ERR_HIP = -2, MQ_ERR_UNSUPPORTED = -3 };
@@ -82,9 +82,11 @@ int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* sc
  * MQ_NVFP4_SECTIONS sections of MQ_NVFP4_SECTION_WORDS partial maxima (float bit patterns).  Each tensor that
  * shares the amax writes ONE whole section (no atomics, nothing to clear beforehand); the amax is the maximum
  * over the first n_sections sections.  A single tensor uses section 0 with n_sections = 1; a gate/up pair
- * uses sections 0 and 1 with n_sections = 2 (nvfp4.py:100-103).
+ * uses sections 0 and 1 with n_sections = 2 (nvfp4.py:100-103).  The words after the last section hold the
+ * folded amax and the two scale factors derived from it (written by mq_nvfp4_quant).
  * mq_nvfp4_amax: record section <- partial maxima of |w| (every word of the section is written).
- * mq_nvfp4_quant: w [M,K] contiguous, K % 16 == 0; q [M,K/2] (element 2i in the low nibble);
+ * mq_nvfp4_quant: folds the record, then quantizes: w [M,K] contiguous, K % 16 == 0; q [M,K/2] (element 2i in
+ *   the low nibble);
  *   block_scale [M,K/16] e4m3fn bytes; global_scale (may be NULL) receives weight_scale_2 =
  *   1 / min(e4m3_max*6/amax, FLT_MAX) as one fp32 (nvfp4.py:19-39). */
 int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream);

@@ -8,10 +8,11 @@
 //
 // Pass 1 (mq_nvfp4_amax): 256 workgroups per tensor stream its elements and each writes one partial maximum
 // into the tensor's section of the amax record: plain stores, no atomics (thousands of agent-scope atomics
-// on one address serialise at ~8 ns each on this multi-XCD part) and nothing to clear.  Pass 2
-// (mq_nvfp4_quant): every workgroup first folds the record's sections into the amax (one cached load per
-// lane), then two lanes own one 16-element block (16 bytes each), the block amax is one DPP step, and each
-// lane emits four bytes of codes.  A gate/up pair writes two sections of one record.
+// on one address serialise at ~8 ns each on this multi-XCD part) and nothing to clear.  A one-workgroup-per-
+// record fold kernel turns the partial maxima into the amax, S_enc/6, 1/S_enc and the published global scale.
+// Pass 2 (mq_nvfp4_quant) reads those two factors with a scalar load; two lanes own one 16-element block
+// (16 bytes each), the block amax is one DPP step, and each lane emits four bytes of codes.  A gate/up pair
+// writes two sections of one record.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -26,17 +27,13 @@ constexpr int kNvUnroll = MQ_NV_UNROLL;
 constexpr float kSixth = 0.16666667163372040f;  // 0x3E2AAAAB
 
 constexpr int kSectionWords = MQ_NVFP4_SECTION_WORDS;   // = workgroups of the amax pass per tensor
-constexpr int kAmaxUnroll = 4;                          // 16-byte units per lane per loop trip
-
-// amax of a record: lanes read the partial maxima of the first n_sections sections, then a workgroup max
-__device__ __forceinline__ float record_amax(const uint32_t* rec, int n_sections, uint32_t* lds4) {
-    uint32_t m = 0;
-    for (int i = threadIdx.x; i < n_sections * kSectionWords; i += blockDim.x) m = umax(m, rec[i]);
-    m = wave_max(m);
-    if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = m;
-    __syncthreads();
-    return u2f(umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3])));
-}
+#ifndef MQ_AMAX_UNROLL
+#define MQ_AMAX_UNROLL 4
+#endif
+#ifndef MQ_AMAX_NT
+#define MQ_AMAX_NT 1
+#endif
+constexpr int kAmaxUnroll = MQ_AMAX_UNROLL;             // 16-byte units per lane per loop trip
 
 // grid (kSectionWords, tensors): workgroup b of a tensor strides over its 16 KiB chunks and writes word b of
 // the section.  job.units counts whole 16-byte units; job.s carries the element count for the sub-unit tail.
@@ -53,7 +50,7 @@ __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable ta
 #pragma unroll
         for (int i = 0; i < kAmaxUnroll; i++) {
             const int64_t unit = base + i * 256 + t;
-            v[i] = unit < n16 ? ld16_keep(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+            v[i] = unit < n16 ? (MQ_AMAX_NT ? ld16(w + unit * 8) : ld16_keep(w + unit * 8)) : u32x4{0u, 0u, 0u, 0u};
         }
 #pragma unroll
         for (int i = 0; i < kAmaxUnroll; i++)
@@ -101,7 +98,33 @@ __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
     return 1.0f / enc;
 }
 
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float numer) {
+// words of a record behind its sections
+constexpr int kRecAmax = MQ_NVFP4_SECTIONS * kSectionWords;   // folded amax (float bits)
+constexpr int kRecEncSixth = kRecAmax + 1;                     // S_enc * (1/6)
+constexpr int kRecSDec = kRecAmax + 2;                         // 1 / S_enc
+
+// one workgroup per tensor: fold the first job.section sections of its record and publish the scales.
+// Tensors that share a record compute the same values and write them twice.
+__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, float numer) {
+    __shared__ uint32_t lds4[4];
+    const FlatJob& job = tab.job[blockIdx.x];
+    uint32_t* rec = (uint32_t*)job.aux;
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < job.section * kSectionWords; i += 256) m = umax(m, rec[i]);
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float amax = u2f(umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3])));
+        const NvScales gs = nv_scales(amax, numer);
+        rec[kRecAmax] = f2u(amax);
+        rec[kRecEncSixth] = f2u(gs.enc_sixth);
+        rec[kRecSDec] = f2u(gs.s_dec);
+        if (job.aux2) *(float*)job.aux2 = nv_published_scale(amax, numer);
+    }
+}
+
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab) {
     const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
@@ -110,17 +133,16 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
     const int64_t base = (int64_t)blockIdx.x * (kNvThreads * kNvUnroll);
-    if (base >= total_units && blockIdx.x != 0) return;
+    if (base >= total_units) return;
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
         v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
     }
-    __shared__ uint32_t lds4[4];
-    const float amax = record_amax(amax_bits, job.section, lds4);
-    const NvScales gs = nv_scales(amax, numer);
-    if (job.aux2 && blockIdx.x == 0 && t == 0) *(float*)job.aux2 = nv_published_scale(amax, numer);
+    NvScales gs;
+    gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
+    gs.s_dec = u2f(amax_bits[kRecSDec]);
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
@@ -155,14 +177,12 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
 }
 
 __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __restrict__ w, int dtype,
-                                                                  const uint32_t* __restrict__ amax_bits, int n_sections,
+                                                                  const uint32_t* __restrict__ amax_bits,
                                                                   uint8_t* __restrict__ q, uint8_t* __restrict__ s8,
-                                                                  float* __restrict__ global_scale, float numer,
                                                                   int64_t blocks16) {
-    __shared__ uint32_t lds4[4];
-    const float amax = record_amax(amax_bits, n_sections, lds4);
-    const NvScales gs = nv_scales(amax, numer);
-    if (global_scale && blockIdx.x == 0 && threadIdx.x == 0) *global_scale = nv_published_scale(amax, numer);
+    NvScales gs;
+    gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
+    gs.s_dec = u2f(amax_bits[kRecSDec]);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks16; b += stride) {
         uint32_t m = 0;
@@ -194,14 +214,15 @@ int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
     return mq_check_launch("nvfp4 amax");
 }
 
-// tab.job[i]: w, q, s = block scales, aux = amax record, section = sections to read, aux2 = fp32 global scale
-// out (may be null), units = numel / 8
+// tab.job[i]: w, q, s = block scales, aux = amax record, section = sections to fold, aux2 = fp32 global scale
+// out (may be null), units = numel / 8.  Launches the fold kernel, then the quantize pass.
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st) {
     const float numer = (float)e4m3_max * 6.0f;
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    if (tab.max_blocks == 0) tab.max_blocks = 1;   // an empty tensor still publishes its global scale
-    hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0, st,
-                       tab, numer);
+    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3((unsigned)tab.n), dim3(256), 0, st, tab, numer);
+    if (tab.max_blocks > 0)
+        hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0,
+                           st, tab);
     return mq_check_launch("nvfp4 quant");
 }
 
@@ -237,10 +258,13 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
         tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), blocks16 * 2, global_scale, n_sections, 0};
         return mq_nvfp4_quant_launch_group(tab, e4m3_max, st);
     }
+    FlatTable fold{};
+    fold.n = 1;
+    fold.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), 0, global_scale, n_sections, 0};
+    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3(1), dim3(256), 0, st, fold, numer);
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
-                       (const uint32_t*)record, n_sections, (uint8_t*)q, (uint8_t*)block_scale, global_scale, numer,
-                       blocks16);
+                       (const uint32_t*)record, (uint8_t*)q, (uint8_t*)block_scale, blocks16);
     return mq_check_launch("nvfp4 quant");
 }

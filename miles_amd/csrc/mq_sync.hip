@@ -26,9 +26,13 @@ bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st);
 
-// The amax pass and the quantize pass of an NVFP4 group read the same input; keeping a group's input
-// below this many bytes lets the second read be served by the 256 MB memory-side cache.
-static const int64_t kNvfp4GroupBytes = 96ll << 20;
+// Upper bound on the input bytes of one NVFP4 group (amax launch + fold + quantize launch).  Measured on
+// MI355X the second read of a tensor gains nothing from the memory-side cache at any group size, so groups
+// are as large as the 64-tensor table allows: fewer launch boundaries.
+#ifndef MQ_NV_GROUP_MB
+#define MQ_NV_GROUP_MB (1 << 20)
+#endif
+static const int64_t kNvfp4GroupBytes = (int64_t)MQ_NV_GROUP_MB << 20;
 
 static bool job_fast(const mq_job& j) {
     switch (j.kind) {

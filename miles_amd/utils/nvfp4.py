@@ -18,7 +18,7 @@ from miles_amd import _lib, launch
 FP4_E2M1_MAX = 6.0
 FP8_E4M3_MAX = 448.0
 NVFP4_GROUP_SIZE = 16
-AMAX_RECORD_WORDS = 1024   # MQ_NVFP4_RECORD_WORDS: per-workgroup partial maxima of a tensor (or pair) on the device
+AMAX_RECORD_WORDS = 1280   # MQ_NVFP4_RECORD_WORDS: per-workgroup partial maxima of a tensor (or pair) on the device
 
 
 def nvfp4_weight_e4m3_max() -> int:

@@ -493,11 +493,11 @@ def test_c_abi_single_tensor_entry_points(oracle, lib):
     p_o, s_o, _ = oracle.pack_layer(w, 128)
     _assert_same(packed, p_o, "mq_int4_group_quant_pack words")
     _assert_same(s16, s_o, "mq_int4_group_quant_pack scales")
-    word = torch.empty(1024, dtype=torch.int32, device=DEV)
+    word = torch.empty(1280, dtype=torch.int32, device=DEV)
     q4 = torch.empty((M, K // 2), dtype=torch.uint8, device=DEV)
     s8 = torch.empty((M, K // 16), dtype=torch.uint8, device=DEV)
     g = torch.empty((), dtype=torch.float32, device=DEV)
-    assert lib.mq_fill_u32(word.data_ptr(), 0x7F800000, 1024, None) == 0   # stale contents must not matter
+    assert lib.mq_fill_u32(word.data_ptr(), 0x7F800000, 1280, None) == 0   # stale contents must not matter
     assert lib.mq_nvfp4_amax(d.data_ptr(), 0, M * K, word.data_ptr(), 0, None) == 0
     assert lib.mq_nvfp4_quant(d.data_ptr(), 0, word.data_ptr(), 1, q4.data_ptr(), s8.data_ptr(), g.data_ptr(), M, K, 448,
                               None) == 0
