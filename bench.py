@@ -110,8 +110,7 @@ def per_quantizer(gen):
         gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
         res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                      "elements": elems, "workload": note}
-        del batch, outs
-        torch.cuda.empty_cache()
+        del batch, outs     # no empty_cache(): freshly mapped device memory streams measurably slower than reused blocks
 
     # C1: one Qwen3-4B MLP, block_fp8; 8 distinct copies so that the 256 MB memory-side cache cannot hold the input
     mlp = [[_synth((9728, 2560), gen), _synth((9728, 2560), gen), _synth((2560, 9728), gen)] for _ in range(8)]
@@ -295,7 +294,6 @@ def main():
     if not a.no_extras:
         del updater, plan
         weights.clear()
-        torch.cuda.empty_cache()
         line["per_quantizer"] = per_quantizer(gen)
     print(json.dumps(line))
 
