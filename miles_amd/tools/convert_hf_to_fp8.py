@@ -1,15 +1,24 @@
-"""FP8 e4m3 weight quantizers of the offline converter.
+"""FP8 e4m3 offline converter: quantizers and the checkpoint shell around them.
 
-Mirror of the reference's tools/convert_hf_to_fp8.py quantizer functions: `block_fp8` (:39-70),
-`channel_fp8` (:73-78), `tensor_fp8` (:81-86), `quant_fp8` (:89-95).  The chain of ~8 full-tensor
-PyTorch kernels there is one gfx950 kernel here (`mq_fp8_block_quant` / `mq_fp8_scaled_quant`).
+    python -m miles_amd.tools.convert_hf_to_fp8 --model-dir SRC --save-dir DST [--strategy block|channel|tensor]
+                                                [--block-size 128 128] [--max-workers N]
+
+Mirror of the reference's tools/convert_hf_to_fp8.py: `block_fp8` (:39-70), `channel_fp8` (:73-78),
+`tensor_fp8` (:81-86), `quant_fp8` (:89-95), `process_file` (:116-160), `convert_fp8` (:163-247).  The chain of
+~8 full-tensor PyTorch kernels per weight there is one gfx950 kernel here, and all weights of a shard are
+submitted as one batched call.
 """
 
 from __future__ import annotations
 
+import argparse
+import os
+from concurrent.futures import ThreadPoolExecutor
+
 import torch
 
 from miles_amd import _lib, launch
+from miles_amd.tools import _checkpoint as ckpt
 
 FP8_INFO = torch.finfo(torch.float8_e4m3fn)
 FP8_MAX, FP8_MIN = FP8_INFO.max, FP8_INFO.min
@@ -68,3 +77,91 @@ def quant_fp8(weight, strategy, block_size=None):
     if strategy == "channel":
         return channel_fp8(weight)
     return block_fp8(weight, block_size)
+
+
+# substrings of tensor names that stay in high precision (reference: tools/convert_hf_to_fp8.py:129-146)
+FP8_SKIP_SUBSTRINGS = ("layernorm", "embed", "router", "mlp.gate.", "norm", "lm_head", "eh_proj", "weights_proj",
+                       "head.", "wo_a", "ffn.gate.", "compressor.", "vision_tower", "mm_projector")
+
+
+def should_quantize_fp8(key: str) -> bool:
+    return "weight" in key and not any(s in key for s in FP8_SKIP_SUBSTRINGS)
+
+
+def process_file(input_path, output_path, filename, strategy, block_size, result_collector, device="cuda"):
+    """Quantize one shard: `<name>.weight` -> e4m3 plus `<name>.weight_scale_inv` (block) or `.weight_scale`."""
+    if not filename.endswith(".safetensors"):
+        return
+    weights = ckpt.load_shard(input_path, filename, device)
+    out: dict[str, torch.Tensor] = {}
+    skipped: list[str] = []
+    with launch.deferred():
+        for key, tensor in weights.items():
+            if should_quantize_fp8(key):
+                q, scale = quant_fp8(tensor, strategy, block_size)
+                out[key] = q
+                out[key.replace(".weight", ".weight_scale_inv" if block_size else ".weight_scale")] = scale
+            else:
+                skipped.append(key.replace(".weight", ""))
+                out[key] = tensor
+    ckpt.save_shard(out, output_path, filename)
+    result_collector.add(filename, out, skipped)
+
+
+def fp8_quantization_config(strategy, block_size, results) -> dict:
+    """`quantization_config` entry of config.json (reference: tools/convert_hf_to_fp8.py:186-236)."""
+    skipped = list(set(results.modules_to_not_convert))
+    if strategy in ("block", "tensor"):
+        cfg = {"activation_scheme": "dynamic", "fmt": "e4m3", "quant_method": "fp8"}
+        if block_size:
+            cfg["weight_block_size"] = block_size
+            if results.has_dsa_layers:
+                cfg["scale_fmt"] = "ue8m0"
+        if skipped:
+            cfg["modules_to_not_convert"] = skipped
+        return cfg
+    common = {"actorder": None, "block_structure": None, "group_size": None, "num_bits": 8, "observer_kwargs": {},
+              "symmetric": True, "type": "float"}
+    group = {
+        "input_activations": {**common, "dynamic": True, "observer": None, "strategy": "token"},
+        "output_activations": None,
+        "targets": ["Linear"],
+        "weights": {**common, "dynamic": False, "observer": "minmax", "strategy": strategy},
+    }
+    return {"config_groups": {"group_0": group}, "format": "float-quantized", "ignore": skipped,
+            "quant_method": "compressed-tensors", "quantization_status": "compressed"}
+
+
+def convert_fp8(input_path, output_path, strategy, block_size=None, max_workers=4, device="cuda"):
+    input_path = os.path.abspath(input_path)
+    os.makedirs(output_path, exist_ok=True)
+    ckpt.copy_side_files(input_path, output_path)
+    results = ckpt.ShardResults(size_in_bytes=False)
+    with ThreadPoolExecutor(max_workers=max_workers) as pool:
+        futures = [pool.submit(process_file, input_path, output_path, f, strategy, block_size, results, device)
+                   for f in ckpt.list_shards(input_path)]
+        for fut in futures:
+            fut.result()
+    cfg = ckpt.read_config(input_path)
+    if cfg is not None:
+        cfg["quantization_config"] = fp8_quantization_config(strategy, block_size, results)
+        ckpt.write_config(output_path, cfg)
+    ckpt.write_index(output_path, results.weight_map, results.total_size)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--model-dir", type=str, help="Path to the directory of the HF safetensors model.")
+    ap.add_argument("--save-dir", type=str, help="Path to the directory to save the converted model.")
+    ap.add_argument("--strategy", type=str, default="block", choices=["block", "channel", "tensor"])
+    ap.add_argument("--block-size", type=int, nargs="*", default=None, help="eg. --block-size 32 32")
+    ap.add_argument("--max-workers", type=int, default=1, help="Number of worker threads for parallel processing")
+    args = ap.parse_args(argv)
+    if os.path.exists(args.save_dir) and not os.path.isdir(args.save_dir):
+        raise ValueError("The save_dir should be a directory.")
+    os.makedirs(args.save_dir, exist_ok=True)
+    convert_fp8(args.model_dir, args.save_dir, args.strategy, args.block_size, args.max_workers)
+
+
+if __name__ == "__main__":
+    main()

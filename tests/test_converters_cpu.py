@@ -1,0 +1,130 @@
+"""Converter shells on the CPU: name scopes, config / index emitters, scale relabelling.  Cases with reference
+counterparts restate tests/fast-gpu/test_nvfp4_quantizer.py:233-283 (HF name scope, compact MoE prefixes)."""
+
+import json
+
+import pytest
+import safetensors.torch
+import torch
+
+from miles_amd.tools import _checkpoint as ckpt
+from miles_amd.tools import convert_hf_to_fp8 as FP8
+from miles_amd.tools import convert_hf_to_int4_direct as INT4
+from miles_amd.tools import convert_hf_to_mxfp8 as MX
+from miles_amd.tools import convert_hf_to_nvfp4 as NV
+
+
+def test_fp8_name_filter_matches_the_reference_list():
+    keep = ["model.layers.0.self_attn.q_proj.weight", "model.layers.3.mlp.experts.7.down_proj.weight",
+            "model.layers.0.mlp.shared_experts.up_proj.weight"]
+    skip = ["model.embed_tokens.weight", "model.norm.weight", "lm_head.weight", "model.layers.0.input_layernorm.weight",
+            "model.layers.0.mlp.gate.weight", "model.layers.0.mlp.router.weight", "model.layers.0.self_attn.q_proj.bias",
+            "model.layers.61.eh_proj.weight", "vision_tower.blocks.0.attn.weight", "model.layers.0.self_attn.indexer.weights_proj.weight",
+            "model.layers.0.self_attn.wo_a.weight", "model.layers.0.ffn.gate.weight", "model.layers.0.attn.compressor.wkv.weight"]
+    assert all(FP8.should_quantize_fp8(k) for k in keep)
+    assert not any(FP8.should_quantize_fp8(k) for k in skip)
+
+
+def test_fp8_quantization_config_variants():
+    r = ckpt.ShardResults(size_in_bytes=False)
+    r.add("a.safetensors", {"model.layers.0.self_attn.indexer.wq_b.weight": torch.zeros(4, 2)}, ["model.norm", "model.norm"])
+    cfg = FP8.fp8_quantization_config("block", [128, 128], r)
+    assert cfg == {"activation_scheme": "dynamic", "fmt": "e4m3", "quant_method": "fp8", "weight_block_size": [128, 128],
+                   "scale_fmt": "ue8m0", "modules_to_not_convert": ["model.norm"]}
+    assert r.total_size == 4      # the FP8 tool counts len(tensor), not bytes
+    r2 = ckpt.ShardResults(size_in_bytes=False)
+    assert FP8.fp8_quantization_config("tensor", None, r2) == {"activation_scheme": "dynamic", "fmt": "e4m3", "quant_method": "fp8"}
+    ch = FP8.fp8_quantization_config("channel", None, r2)
+    assert ch["quant_method"] == "compressed-tensors" and ch["format"] == "float-quantized"
+    assert ch["config_groups"]["group_0"]["weights"]["strategy"] == "channel"
+    assert ch["config_groups"]["group_0"]["input_activations"]["strategy"] == "token"
+
+
+def test_int4_ignore_rules_and_config():
+    rules = INT4.DEFAULT_IGNORE_RULES
+    assert INT4.is_ignored("model.layers.0.self_attn.q_proj.weight", rules)
+    assert INT4.is_ignored("model.layers.0.mlp.gate_proj.weight", rules) and INT4.is_ignored("lm_head.weight", rules)
+    assert INT4.is_ignored("model.layers.1.mlp.shared_experts.down_proj.weight", rules)
+    assert not INT4.is_ignored("model.layers.1.mlp.experts.3.down_proj.weight", rules)
+    assert INT4.is_ignored("abc.def", ["abc"]) and INT4.is_ignored("abc", ["abc"]) and not INT4.is_ignored("xabc", ["abc"])
+    cfg = INT4.int4_quantization_config(128, True, ["re:.*norm.*"])
+    w = cfg["config_groups"]["group_0"]["weights"]
+    assert (cfg["format"], cfg["quant_method"], w["num_bits"], w["group_size"], w["strategy"], w["symmetric"], w["type"]) == \
+        ("pack-quantized", "compressed-tensors", 4, 128, "group", True, "int")
+    assert cfg["ignore"] == ["re:.*norm.*"] and cfg["kv_cache_scheme"] is None
+
+
+def test_nvfp4_name_scope():
+    w = torch.zeros(4, 16, dtype=torch.bfloat16)
+    name = "model.layers.0.mlp.experts.0.gate_proj.weight"
+    assert NV.should_quantize(name, w)
+    assert not NV.should_quantize(name, w, skip_weight_substrings=("mlp.experts.0",))
+    assert NV.should_quantize(name, w, skip_weight_substrings=("mlp.experts.1",))
+    assert not NV.should_quantize(name, w, num_hidden_layers=0)                      # MTP layers appended after the decoder
+    assert NV.should_quantize("language_model.model.layers.2.mlp.experts.1.w2.weight", w, num_hidden_layers=3)
+    assert not NV.should_quantize("model.layers.0.mlp.shared_experts.gate_proj.weight", w)
+    assert not NV.should_quantize("model.layers.0.mlp.gate_proj.weight", w)
+    assert not NV.should_quantize("vision_tower.layers.0.mlp.experts.0.gate_proj.weight", w)
+    assert not NV.should_quantize(name, w.to(torch.int8))
+    with pytest.raises(ValueError, match="must be divisible by 16"):
+        NV.should_quantize(name, torch.zeros(4, 24, dtype=torch.bfloat16))
+
+
+def test_nvfp4_ignore_list_and_configs(tmp_path):
+    got = NV._augment_ignore_list(["model.layers.0.self_attn.q_proj", "model.layers.0.mlp.experts.3.down_proj",
+                                   "model.layers.1.mlp.experts.gate_up_proj", "model.norm"])
+    assert got == sorted({"model.layers.0.self_attn.q_proj", "model.layers.0.self_attn.qkv_proj",
+                          "model.layers.0.mlp.experts.3.down_proj", "model.layers.0.mlp.experts",
+                          "model.layers.1.mlp.experts.gate_up_proj", "model.layers.1.mlp.experts", "model.norm"})
+    cfg = {"text_config": {"quantization_config": {}}, "quantization_config": {"config_groups": {"g": {"weights": {}}}}}
+    NV._update_quantization_config(cfg, ["a"])
+    q = cfg["quantization_config"]
+    assert (q["quant_algo"], q["quant_method"], q["group_size"], q["ignore"]) == ("NVFP4", "modelopt", 16, ["a"])
+    assert q["kv_cache_scheme"] == {"dynamic": False, "num_bits": 8, "type": "float"}
+    assert q["config_groups"]["g"]["weights"] == {"dynamic": False, "num_bits": 4, "type": "float", "group_size": 16}
+    assert cfg["text_config"]["quantization_config"]["quant_algo"] == "NVFP4"
+    NV._write_hf_quant_config(str(tmp_path), ["a"], str(tmp_path))
+    doc = json.loads((tmp_path / "hf_quant_config.json").read_text())
+    assert doc == {"producer": {"name": "modelopt"}, "quantization": {"quant_algo": "NVFP4", "kv_cache_quant_algo": "FP8",
+                                                                        "group_size": 16, "exclude_modules": ["a"]}}
+
+
+def test_nvfp4_converter_uses_compact_bf16_moe_prefixes(tmp_path):
+    # every layer kept in bf16: nothing is quantized, so the conversion runs without a GPU
+    model_dir, save_dir = tmp_path / "model", tmp_path / "converted"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text('{"num_hidden_layers": 1}')
+    weights = {f"model.layers.0.mlp.experts.{e}.{p}.weight": torch.ones((1, 16), dtype=torch.bfloat16)
+               for e in range(128) for p in ("gate_proj", "up_proj", "down_proj")}
+    weights["model.layers.0.input_layernorm.weight"] = torch.ones(16, dtype=torch.bfloat16)
+    safetensors.torch.save_file(weights, model_dir / "model.safetensors", metadata={"format": "pt"})
+    NV.convert_nvfp4(str(model_dir), str(save_dir), device="cpu", num_layers_at_end_in_bf16=1)
+    expected = ["model.layers.0.", "model.layers.0.input_layernorm", "model.layers.0.mlp.experts"]
+    assert json.loads((save_dir / "config.json").read_text())["quantization_config"]["ignore"] == expected
+    assert json.loads((save_dir / "hf_quant_config.json").read_text())["quantization"]["exclude_modules"] == expected
+    with safetensors.safe_open(save_dir / "model.safetensors", framework="pt", device="cpu") as f:
+        assert all("weight_scale" not in k for k in f.keys())
+        assert f.get_tensor("model.layers.0.mlp.experts.127.down_proj.weight").dtype == torch.bfloat16
+    index = json.loads((save_dir / "model.safetensors.index.json").read_text())
+    assert index["metadata"]["total_size"] == sum(t.numel() * 2 for t in weights.values())   # bytes for this tool
+
+
+def test_mxfp8_source_detection_and_scale_relabelling():
+    assert MX._source_kind({}) == "bf16" and MX._source_kind({"quantization_config": {"quant_method": "bf16"}}) == "bf16"
+    fp8 = {"quantization_config": {"quant_method": "fp8", "weight_block_size": [128, 128], "scale_fmt": "ue8m0"}}
+    assert MX._source_kind(fp8) == "fp8_ue8m0"
+    with pytest.raises(ValueError, match="Unsupported source quantization_config"):
+        MX._source_kind({"quantization_config": {"quant_method": "fp8", "weight_block_size": [128, 128]}})
+    w = torch.zeros(200, 288, dtype=torch.uint8)
+    u8 = torch.tensor([[120, 121, 122], [130, 131, 132]], dtype=torch.uint8)
+    out = MX._source_fp8_to_mxfp8_scale_u8(w, u8)
+    assert out.shape == (200, 9)
+    assert out[0].tolist() == [120] * 4 + [121] * 4 + [122] and out[199].tolist() == [130] * 4 + [131] * 4 + [132]
+    # fp32 power-of-two scales are recognised and turned into exponents; others are not
+    weights = {"a.weight": w, "a.weight_scale_inv": torch.tensor([[0.5, 2.0, 1.0], [4.0, 0.25, 8.0]])}
+    f32, e, key = MX._load_source_scale_u8(weights, "a.weight", w, {"a.weight_scale_inv": "s"}, ".", "cpu", "s")
+    assert key == "a.weight_scale_inv" and e.tolist() == [[126, 128, 127], [129, 125, 130]]
+    weights["a.weight_scale_inv"] = torch.tensor([[0.5, 3.0, 1.0], [4.0, 0.25, 8.0]])
+    assert MX._load_source_scale_u8(weights, "a.weight", w, {"a.weight_scale_inv": "s"}, ".", "cpu", "s")[1] is None
+    with pytest.raises(ValueError, match="Expected key ending"):
+        MX._strip_weight_suffix("a.bias")

@@ -1,0 +1,218 @@
+"""Offline converters end to end on the GPU: tiny sharded checkpoints in, converted checkpoints out, every
+tensor compared with the oracle.  The cross-shard / same-shard gated-pair cases restate
+tests/fast-gpu/test_nvfp4_quantizer.py:286-366."""
+
+import json
+
+import pytest
+import safetensors
+import safetensors.torch
+import torch
+
+from miles_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+F8 = torch.float8_e4m3fn
+
+
+def _load_all(path):
+    out = {}
+    for f in sorted(path.glob("*.safetensors")):
+        with safetensors.safe_open(f, framework="pt", device="cpu") as h:
+            for k in h.keys():
+                out[k] = h.get_tensor(k)
+    return out
+
+
+def _bits(t):
+    t = t.contiguous()
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32}[t.element_size()])
+
+
+def _same(a, b, what):
+    assert a.shape == b.shape and torch.equal(_bits(a), _bits(b)), f"{what} differs"
+
+
+def _checkpoint(tmp_path, shards, config=None):
+    model = tmp_path / "model"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(config or {"num_hidden_layers": 2}))
+    (model / "tokenizer.json").write_text("{}")
+    weight_map = {}
+    for i, tensors in enumerate(shards):
+        name = f"model-{i:05d}-of-{len(shards):05d}.safetensors"
+        safetensors.torch.save_file(tensors, model / name, metadata={"format": "pt"})
+        weight_map.update({k: name for k in tensors})
+    (model / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map, "metadata": {}}))
+    return model
+
+
+def _rand(shape, seed, dtype=torch.bfloat16):
+    return W.gaussian_outliers(shape, std=0.02, p_outlier=0.001, gain=20.0, seed=seed, dtype=dtype)
+
+
+def _dense_shards():
+    a = {"model.embed_tokens.weight": _rand((64, 256), 1), "model.layers.0.input_layernorm.weight": _rand((256,), 2),
+         "model.layers.0.self_attn.q_proj.weight": _rand((384, 256), 3), "model.layers.0.mlp.gate.weight": _rand((8, 256), 4),
+         "model.layers.0.self_attn.q_proj.bias": _rand((384,), 5)}
+    b = {"model.layers.1.mlp.down_proj.weight": _rand((256, 640), 6), "model.layers.1.mlp.experts.0.up_proj.weight": _rand((130, 256), 7),
+         "lm_head.weight": _rand((64, 256), 8)}
+    return [a, b]
+
+
+def test_convert_fp8_block_and_back(oracle, tmp_path):
+    from miles_amd.tools.convert_hf_to_fp8 import convert_fp8
+    from miles_amd.tools.fp8_cast_bf16 import main as fp8_cast_bf16
+
+    shards = _dense_shards()
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "fp8"
+    convert_fp8(str(model), str(out), "block", [128, 128], max_workers=2)
+    got = _load_all(out)
+    src = {k: v for s in shards for k, v in s.items()}
+    quantized = ["model.layers.0.self_attn.q_proj.weight", "model.layers.1.mlp.down_proj.weight",
+                 "model.layers.1.mlp.experts.0.up_proj.weight"]
+    for k in quantized:
+        q, s = oracle.block_fp8(src[k], (128, 128))
+        _same(got[k], q, k)
+        _same(got[k.replace(".weight", ".weight_scale_inv")], s, k + " scale")
+    for k in set(src) - set(quantized):
+        _same(got[k], src[k], k)
+    cfg = json.loads((out / "config.json").read_text())["quantization_config"]
+    assert cfg["quant_method"] == "fp8" and cfg["weight_block_size"] == [128, 128] and cfg["fmt"] == "e4m3"
+    assert set(cfg["modules_to_not_convert"]) == {"model.embed_tokens", "model.layers.0.input_layernorm", "lm_head",
+                                                  "model.layers.0.mlp.gate", "model.layers.0.self_attn.q_proj.bias"}
+    index = json.loads((out / "model.safetensors.index.json").read_text())
+    assert set(index["weight_map"]) == set(got) and (out / "tokenizer.json").exists()
+    # and back to bf16: weights whose scales sit in the same or another shard
+    back = tmp_path / "bf16"
+    fp8_cast_bf16(str(out), str(back))
+    rt = _load_all(back)
+    assert not any(k.endswith("_scale_inv") for k in rt)
+    for k in quantized:
+        _same(rt[k], oracle.weight_dequant(*oracle.block_fp8(src[k], (128, 128))), k + " round trip")
+    assert not any(k.endswith("_scale_inv") for k in json.loads((back / "model.safetensors.index.json").read_text())["weight_map"])
+
+
+@pytest.mark.parametrize("strategy", ["tensor", "channel"])
+def test_convert_fp8_tensor_and_channel(oracle, tmp_path, strategy):
+    from miles_amd.tools.convert_hf_to_fp8 import convert_fp8
+
+    shards = _dense_shards()
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "fp8"
+    convert_fp8(str(model), str(out), strategy, None, max_workers=1)
+    got = _load_all(out)
+    k = "model.layers.1.mlp.down_proj.weight"
+    q, s = (oracle.tensor_fp8 if strategy == "tensor" else oracle.channel_fp8)(shards[1][k])
+    _same(got[k], q, k)
+    _same(got[k.replace(".weight", ".weight_scale")], s, k + " scale")
+
+
+def _moe_shards():
+    a, b = {}, {}
+    for e in range(3):
+        a[f"model.layers.0.mlp.experts.{e}.gate_proj.weight"] = _rand((96, 256), 10 + e)
+        (a if e < 2 else b)[f"model.layers.0.mlp.experts.{e}.up_proj.weight"] = _rand((96, 256), 20 + e)   # expert 2: pair split over shards
+        b[f"model.layers.0.mlp.experts.{e}.down_proj.weight"] = _rand((256, 96), 30 + e)
+    a["model.layers.0.mlp.gate.weight"] = _rand((3, 256), 40)
+    a["model.layers.0.self_attn.o_proj.weight"] = _rand((256, 256), 41)
+    b["model.layers.1.mlp.experts.0.down_proj.weight"] = _rand((256, 96), 42)      # layer 1: kept in bf16 below
+    b["model.layers.0.mlp.shared_experts.down_proj.weight"] = _rand((256, 96), 43)
+    return [a, b]
+
+
+def test_convert_nvfp4_pairs_across_shards(oracle, tmp_path):
+    from miles_amd.tools.convert_hf_to_nvfp4 import convert_nvfp4
+
+    shards = _moe_shards()
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "nvfp4"
+    convert_nvfp4(str(model), str(out), device="cuda:0", num_layers_at_end_in_bf16=1)
+    got = _load_all(out)
+    src = {k: v for s in shards for k, v in s.items()}
+    for e in range(3):
+        base = f"model.layers.0.mlp.experts.{e}"
+        (gq, gs, gg), (uq, us, ug) = oracle.nvfp4_quantize_1d_pair(src[base + ".gate_proj.weight"], src[base + ".up_proj.weight"])
+        dq, ds, dg = oracle.nvfp4_quantize_1d(src[base + ".down_proj.weight"])
+        for proj, (q, s, g) in (("gate_proj", (gq, gs, gg)), ("up_proj", (uq, us, ug)), ("down_proj", (dq, ds, dg))):
+            _same(got[f"{base}.{proj}.weight"], q, f"{base}.{proj} codes")
+            _same(got[f"{base}.{proj}.weight_scale"], s, f"{base}.{proj} block scales")
+            _same(got[f"{base}.{proj}.weight_scale_2"], g, f"{base}.{proj} global scale")
+            assert got[f"{base}.{proj}.input_scale"].item() == 1.0
+        assert got[base + ".gate_proj.weight_scale_2"].item() == got[base + ".up_proj.weight_scale_2"].item()
+    for k in ("model.layers.1.mlp.experts.0.down_proj.weight", "model.layers.0.mlp.shared_experts.down_proj.weight",
+              "model.layers.0.self_attn.o_proj.weight", "model.layers.0.mlp.gate.weight"):
+        _same(got[k], src[k], k)
+    ignore = json.loads((out / "config.json").read_text())["quantization_config"]["ignore"]
+    assert "model.layers.1." in ignore and "model.layers.1.mlp.experts" in ignore and "model.layers.0.self_attn.o_proj" in ignore
+    hf = json.loads((out / "hf_quant_config.json").read_text())["quantization"]
+    assert hf["quant_algo"] == "NVFP4" and hf["exclude_modules"] == ignore
+    # the up tensor of expert 2 was written into the shard that holds it in the source
+    index = json.loads((out / "model.safetensors.index.json").read_text())["weight_map"]
+    assert index["model.layers.0.mlp.experts.2.up_proj.weight"] == "model-00001-of-00002.safetensors"
+    assert index["model.layers.0.mlp.experts.2.gate_proj.weight"] == "model-00000-of-00002.safetensors"
+
+
+def test_convert_mxfp8_from_bf16_and_from_pow2_fp8(oracle, tmp_path):
+    from miles_amd.tools.convert_hf_to_mxfp8 import convert_mxfp8
+
+    shards = _moe_shards()
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "mx"
+    convert_mxfp8(str(model), str(out), "cuda:0", num_layers_at_end_in_bf16=1, extra_high_precision_layers_hf=(".shared_experts.",))
+    got = _load_all(out)
+    src = {k: v for s in shards for k, v in s.items()}
+    for k in (f"model.layers.0.mlp.experts.{e}.{p}.weight" for e in range(3) for p in ("gate_proj", "up_proj", "down_proj")):
+        q, s = oracle.mxfp8_quantize(src[k])
+        _same(got[k], q, k)
+        _same(got[k.replace(".weight", ".weight_scale_inv")], s, k + " scale")
+    q, s = oracle.mxfp8_quantize(src["model.layers.0.self_attn.o_proj.weight"])
+    _same(got["model.layers.0.self_attn.o_proj.weight"], q, "o_proj")
+    for k in ("model.layers.1.mlp.experts.0.down_proj.weight", "model.layers.0.mlp.shared_experts.down_proj.weight",
+              "model.layers.0.mlp.gate.weight"):
+        _same(got[k], src[k], k)
+    cfg = json.loads((out / "config.json").read_text())["quantization_config"]
+    assert cfg["quant_method"] == "mxfp8" and cfg["weight_block_size"] == [1, 32] and cfg["scale_fmt"] == "ue8m0"
+    assert cfg["modules_to_not_convert"] == ["model.layers.0.mlp.gate", "model.layers.0.mlp.shared_experts.down_proj", "model.layers.1."]
+    # FP8 source with power-of-two tile scales: codes are kept, exponents are repeated per 1x32 group
+    codes = torch.randint(0, 120, (256, 384), dtype=torch.int32).to(torch.uint8).view(F8)
+    tile_scale = torch.tensor([[0.5, 2.0, 1.0], [4.0, 0.25, 8.0]])
+    (tmp_path / "x").mkdir()
+    fp8_model = _checkpoint(tmp_path / "x", [{"model.layers.0.mlp.down_proj.weight": codes,
+                                               "model.layers.0.mlp.down_proj.weight_scale_inv": tile_scale,
+                                               "model.layers.0.mlp.gate.weight": codes.clone(),
+                                               "model.layers.0.mlp.gate.weight_scale_inv": tile_scale.clone()}],
+                            config={"num_hidden_layers": 1, "quantization_config": {
+                                "quant_method": "fp8", "weight_block_size": [128, 128], "scale_fmt": "ue8m0"}})
+    out2 = tmp_path / "mx2"
+    convert_mxfp8(str(fp8_model), str(out2), "cuda:0")
+    got2 = _load_all(out2)
+    _same(got2["model.layers.0.mlp.down_proj.weight"], codes, "relabelled codes")
+    want = tile_scale.view(torch.int32).bitwise_right_shift(23).to(torch.uint8).repeat_interleave(128, 0).repeat_interleave(4, 1)
+    _same(got2["model.layers.0.mlp.down_proj.weight_scale_inv"], want, "relabelled exponents")
+    # the router stays out of MXFP8 and is dequantized to bf16 with its tile scales
+    _same(got2["model.layers.0.mlp.gate.weight"], oracle.weight_dequant(codes, tile_scale), "router dequant")
+    assert "model.layers.0.mlp.gate.weight_scale_inv" not in got2
+
+
+def test_convert_int4_direct(oracle, tmp_path):
+    from miles_amd.tools.convert_hf_to_int4_direct import DEFAULT_IGNORE_RULES, convert_int4
+
+    shards = _moe_shards()
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "int4"
+    convert_int4(str(model), str(out), 32, True, DEFAULT_IGNORE_RULES, max_workers=2)
+    got = _load_all(out)
+    src = {k: v for s in shards for k, v in s.items()}
+    for k, w in src.items():
+        if ".experts." in k and "shared" not in k:
+            p, s, _ = oracle.pack_layer(w, 32)
+            _same(got[k.replace(".weight", ".weight_packed")], p, k + " packed")
+            _same(got[k.replace(".weight", ".weight_scale")], s, k + " scale")
+            assert got[k.replace(".weight", ".weight_shape")].tolist() == list(w.shape)
+            assert k not in got
+        else:
+            _same(got[k], w, k)
+    cfg = json.loads((out / "config.json").read_text())["quantization_config"]
+    assert cfg["format"] == "pack-quantized" and cfg["config_groups"]["group_0"]["weights"]["group_size"] == 32
