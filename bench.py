@@ -35,8 +35,8 @@ HBM_PEAK_GBPS = 8000.0
 BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 + 2, "mxfp8": 2 + 1 + 1 / 32,
                   "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
-# scaled by the same counter on a plain copy of known size (profiles/fp8_block128_c2_pmc.md); None until measured
-MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = None
+# scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0003 B per element)
+MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0005
 
 METRIC = "HBM GB/s (% of peak) per quantizer; ms per full-model BF16->FP8 weight sync"
 DEV = "cuda:0"
@@ -176,7 +176,7 @@ def roofline(plan, jobs_meta):
     launches = reps * len(spans)
     achieved = total_bytes / total_ms / 1e6
     elems_per_launch = total_bytes / BYTES_PER_ELEM["fp8_block"] / launches
-    traffic = None if MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM is None else MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems_per_launch
+    traffic = round(MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems_per_launch)
     return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
             "launches_per_sync": len(spans), "avg_launch_us": round(total_ms / launches * 1e3, 2),
@@ -237,6 +237,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-extras", action="store_true", help="skip the per-quantizer section")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-workload", action="store_true",
+                    help="counter-collection run: three 1 GiB plain copies (calibration), three syncs, no timing")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
@@ -259,6 +261,17 @@ def main():
     updater = WeightUpdater(args, weights_getter=lambda: weights, model_name="qwen3", quantization_config=fp8_cfg,
                             send_bucket=consume)
     updater.update_weights()          # builds the plan (first sync pays the per-parameter Python work)
+    if a.pmc_workload:
+        n = 1 << 30
+        src, dst = torch.empty(n, dtype=torch.uint8, device=DEV), torch.empty(n, dtype=torch.uint8, device=DEV)
+        src.fill_(1)
+        for _ in range(3):
+            _lib.check(_lib.load().mq_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
+        for _ in range(2):
+            updater.update_weights()
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_workload": "3 x mq_copy_bytes(1 GiB), 3 x Qwen3-4B FP8 sync", "quantized_elements": elems}))
+        return
     for _ in range(a.warmup):
         updater.update_weights()
     torch.cuda.synchronize()
