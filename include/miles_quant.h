@@ -64,6 +64,16 @@ int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int6
  *   w [rows,K] contiguous, K % 32 == 0; q [rows,K] e4m3fn; scale [rows,K/32] E8M0 bytes */
 int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K, void* stream);
 
+/* quantize_mxfp4(weight, group_size)                  miles/utils/mxfp4.py:11-31
+ *   w: numel elements, contiguous, groups of `group` consecutive elements (numel % group == 0, numel % 2 == 0)
+ *   packed [numel/2] bytes (element 2j in the low nibble: magnitude code | sign << 3); scale [numel/group] E8M0 */
+int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t* scale, int64_t numel, int group,
+                   void* stream);
+
+/* dequantize_mxfp4(weight_packed, weight_scale, group_size)   miles/utils/mxfp4.py:34-59
+ *   packed [bytes]; scale [2*bytes/group]; y [2*bytes] bf16 */
+int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, void* y, int64_t bytes, int group, void* stream);
+
 /* fake_int4_quant_cuda(x, (1, group), sym)           miles/kernels/quant/int4_fake/fake_int4_quant_cuda.cu:319-364
  *   x [M,N] contiguous; out [M,N], scale [M,ceil(N/group)], zero (asym only) in the dtype of x */
 int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
@@ -76,6 +86,16 @@ int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* z
  *   scale  [M,K/group] in the dtype of w */
 int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* scale, int64_t M, int64_t K,
                              int group, void* stream);
+
+/* pack_layer(weight, group_size, sym=False)          .../processors/quantizer_compressed_tensors.py:235-265
+ *   w [M,K] contiguous and 16-byte aligned, K % group == 0, group % 8 == 0, M % 8 == 0
+ *   packed    [M,K/8] int32: sum_i code(8j+i) << 4i with int32 wraparound; codes are uint8 in [0,255] after the
+ *             reference's dequantize/requantize round trip in the dtype of w (nothing clamps them to 15)
+ *   scale     [M,K/group] in the dtype of w
+ *   zero      [M,K/group] uint8 zero points in [0,15] (also the staging area for packed_zp)
+ *   packed_zp [K/group, M/8] int32: zero point of row 8j+i in nibble {0,4,1,5,2,6,3,7}[i] */
+int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
+                                  int32_t* packed_zp, int64_t M, int64_t K, int group, void* stream);
 
 /* NVFP4                                              miles/utils/nvfp4.py:54-114
  * The global amax travels on the device in an "amax record": MQ_NVFP4_RECORD_WORDS uint32 words made of
@@ -109,6 +129,7 @@ int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections,
  *   MQ_JOB_MXFP8                w             e4m3          E8M0 bytes     -                           -
  *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
  *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, -
+ *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *                                                                          aux2 = fp32 weight_scale_2
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
@@ -120,7 +141,8 @@ enum {
     MQ_JOB_FP8_DEQUANT = 2,
     MQ_JOB_MXFP8 = 3,
     MQ_JOB_INT4_PACK = 4,
-    MQ_JOB_NVFP4 = 5
+    MQ_JOB_NVFP4 = 5,
+    MQ_JOB_MXFP4 = 6
 };
 typedef struct mq_job {
     int32_t kind;

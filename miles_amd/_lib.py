@@ -27,7 +27,10 @@ SIGNATURES = {
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp8_quant": [_vp, _i32, _vp, _vp, _i64, _i64, _vp],
     "mq_int4_fake_quant": [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
+    "mq_mxfp4_quant": [_vp, _i32, _vp, _vp, _i64, _i32, _vp],
+    "mq_mxfp4_dequant": [_vp, _vp, _vp, _i64, _i32, _vp],
     "mq_int4_group_quant_pack": [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp],
+    "mq_int4_group_quant_pack_asym": [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_fill_u32": [_vp, _u32, _i64, _vp],
     "mq_nvfp4_amax": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mq_nvfp4_quant": [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
@@ -36,7 +39,7 @@ SIGNATURES = {
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 
-(JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4) = range(6)
+(JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4) = range(7)
 
 
 class Job(_c.Structure):

@@ -110,7 +110,8 @@ __global__ __launch_bounds__(256) void int4_fake_generic_kernel(const void* __re
         if (sym) s = __builtin_fmaxf(mx * kSymCons, 1e-5f);
         else {
             s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
-            zero = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f);
+            // max(-0, +0) is +0 in the reference's device code: adding +0 makes that explicit
+            zero = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
         }
         for (int k = lane; k < G; k += 64) {
             const int64_t c = c0 + k;
@@ -154,6 +155,112 @@ __global__ __launch_bounds__(256) void int4_pack_generic_kernel(const void* __re
             if (c == g0) store_dtype(scale_out, r * gpr + c / G, s, dtype);
         }
         packed[i] = word;
+    }
+}
+
+// ---- asymmetric pack_layer ---------------------------------------------------------------------
+// The reference runs the asymmetric fake-quant kernel and then dequantizes / requantizes in the weight's
+// dtype D before packing (quantizer_compressed_tensors.py:235-264).  With rd() = round to D:
+//   s = fmaxf((max-min)*(1/15), 1e-5);  z = clamp(-rintf(min/s), 0, 15)          (.cu:226-229)
+//   w1 = rd(rintf(x/s) + z);  sb = rd(s)                                          (.cu:244-254)
+//   w2 = rd(rd(w1 - z) * sb)                                                      (py:243)
+//   r  = rd(rd(w2 / sb) + z);  code = uint8(round_half_even(clamp(r, 0, 255)))    (py:213-220,190)
+//   word = sum_i code_i << 4i  (int32 wraparound: codes above 15 carry)           (py:173-175)
+// Nothing clamps w1, so codes above 15 do occur (a group whose minimum is far above zero); the carry
+// is part of the reference's result and is kept.
+template <int DT>
+__device__ __forceinline__ void load8(const void* p, int64_t word, float f[8]) {
+    if (DT == MQ_F32) {
+        const u32x4 a = ld16((const float*)p + word * 8), b = ld16((const float*)p + word * 8 + 4);
+        f[0] = u2f(a.x); f[1] = u2f(a.y); f[2] = u2f(a.z); f[3] = u2f(a.w);
+        f[4] = u2f(b.x); f[5] = u2f(b.y); f[6] = u2f(b.z); f[7] = u2f(b.w);
+    } else {
+        const u32x4 a = ld16((const uint16_t*)p + word * 8);
+        const uint32_t u[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (DT == MQ_BF16) { f[2 * i] = bf16_lo(u[i]); f[2 * i + 1] = bf16_hi(u[i]); }
+            else {
+                f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] & 0xFFFFu));
+                f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] >> 16));
+            }
+        }
+    }
+}
+
+// 16 lanes own one group; a lane handles the 8-element words lane, lane+16, ... of it.
+template <int DT>
+__global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restrict__ w,
+                                                             uint32_t* __restrict__ packed,
+                                                             void* __restrict__ scale_out,
+                                                             uint8_t* __restrict__ zero_out, int64_t total_groups,
+                                                             int words_per_group) {
+    const int lane = threadIdx.x & 15;
+    const int64_t team = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int64_t nteams = ((int64_t)gridDim.x * blockDim.x) >> 4;
+    // every lane of a wavefront runs the same number of trips so the shuffles below always see all 64 lanes
+    const int64_t trips = (total_groups + nteams - 1) / nteams;
+    for (int64_t it = 0; it < trips; it++) {
+        const int64_t g = team + it * nteams;
+        const bool live = g < total_groups;
+        const int64_t word0 = live ? g * words_per_group : 0;
+        float mx = -__builtin_inff(), mn = __builtin_inff();
+        float f[8];
+        if (live)
+            for (int k = lane; k < words_per_group; k += 16) {
+                load8<DT>(w, word0 + k, f);
+#pragma unroll
+                for (int i = 0; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
+            }
+        for (int off = 8; off > 0; off >>= 1) {
+            mx = __builtin_fmaxf(mx, __shfl_xor(mx, off, 64));
+            mn = __builtin_fminf(mn, __shfl_xor(mn, off, 64));
+        }
+        if (!live) continue;
+        const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
+        const float z = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
+        const float sb = round_to_dtype(s, DT);
+        const float ys = 1.0f / s, yb = 1.0f / sb;
+        // the shared-divisor sequence needs finite intermediates: quotients stay far below 2^100
+        const float big = __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
+        const bool fast = DT != MQ_F32 && shared_div_ok(s) && shared_div_ok(sb) && big * ys < 1e30f;
+        for (int k = lane; k < words_per_group; k += 16) {
+            load8<DT>(w, word0 + k, f);
+            uint32_t word = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float q = fast ? div_by_shared(f[i], s, ys) : f[i] / s;
+                const float w1 = round_to_dtype(__builtin_rintf(q) + z, DT);
+                const float w2 = round_to_dtype(round_to_dtype(w1 - z, DT) * sb, DT);
+                const float d = fast ? div_by_shared(w2, sb, yb) : w2 / sb;
+                float r = round_to_dtype(round_to_dtype(d, DT) + z, DT);
+                r = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
+                word += (uint32_t)__builtin_rintf(r) << (4 * i);
+            }
+            packed[word0 + k] = word;
+        }
+        if (lane == 0) {
+            store_dtype(scale_out, g, s, DT);
+            zero_out[g] = (uint8_t)z;
+        }
+    }
+}
+
+// packed_zp[g, j] = sum_i zero[8j+i, g] << 4*order[i], order = {0,4,1,5,2,6,3,7}   (py:249-254)
+__global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
+                                                             uint32_t* __restrict__ packed_zp, int64_t M,
+                                                             int64_t groups_per_row) {
+    const int64_t rows8 = M / 8, total = groups_per_row * rows8;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t g = i / rows8, j = i - g * rows8;
+        uint32_t word = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int nib = (k >> 1) + 4 * (k & 1);
+            word += (uint32_t)zero[(j * 8 + k) * groups_per_row + g] << (4 * nib);
+        }
+        packed_zp[i] = word;
     }
 }
 
@@ -209,4 +316,32 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
     hipLaunchKernelGGL(int4_pack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (uint32_t*)packed,
                        scale, M, K, group);
     return mq_check_launch("int4 pack");
+}
+
+extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
+                                             int32_t* packed_zp, int64_t M, int64_t K, int group, void* stream) {
+    if (!w || !packed || !scale || !zero || !packed_zp) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (K % group != 0 || group % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and the group size of 8");
+    if (M % 8 != 0) return mq_fail(MQ_ERR_ARG, "asymmetric packing needs a multiple of 8 rows");
+    if (((uintptr_t)w % 16) != 0) return mq_fail(MQ_ERR_ARG, "weight must be 16-byte aligned");
+    if (M == 0 || K == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t gpr = K / group, groups = M * gpr;
+    int64_t blocks = (groups + 15) / 16;
+    if (blocks > mq_grid_cap() * 4) blocks = mq_grid_cap() * 4;
+    const int wpg = group / 8;
+    if (dtype == MQ_BF16)
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+    else if (dtype == MQ_F16)
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+    else
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F32>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+    int rc = mq_check_launch("int4 asymmetric pack");
+    if (rc != MQ_OK) return rc;
+    const int64_t zp_words = gpr * (M / 8);
+    int64_t zblocks = (zp_words + 255) / 256;
+    if (zblocks > mq_grid_cap()) zblocks = mq_grid_cap();
+    hipLaunchKernelGGL(int4_zero_pack_kernel, dim3((unsigned)zblocks), dim3(256), 0, st, zero, (uint32_t*)packed_zp, M, gpr);
+    return mq_check_launch("int4 zero-point pack");
 }

@@ -1,0 +1,204 @@
+// MXFP4 (e2m1 codes, two per byte, one E8M0 scale per group) for gfx950.
+// Reference: miles/utils/mxfp4.py:11-31 (quantize_mxfp4) and :34-59 (dequantize_mxfp4), plain tensor ops:
+//   amax = max|x| over the group;  e = clamp(ceil(log2(amax / 6)), -127, 127);  scale byte = e + 127
+//   n = f32(x) * 2^-e;  magnitude = #{b in (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5) : |n| > b}   (ties round DOWN)
+//   code = magnitude | signbit(n) << 3;  byte j = code(2j) | code(2j+1) << 4
+//   dequantize: bf16(sign * {0, .5, 1, 1.5, 2, 3, 4, 6}[magnitude] * 2^(scale - 127))
+//
+// ceil(log2(q)) is taken from the bits of q = amax / 6.0f (exponent, plus one when the mantissa is not zero).
+// For bf16 and fp16 inputs this is what a float log2 followed by ceil returns: q is either an exact power of
+// two or at least 2^-11 away from one in relative terms, far more than the rounding of any log2.  For fp32
+// inputs within a few ulp above a power of two a float log2 rounds to the integer below and the two differ;
+// there the reference's own result depends on the device's log2.
+//
+// Packed fast path (bf16, group 32): four lanes own one group, 16 bytes in and 4 bytes out per lane.
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+#include "mq_group.hpp"
+
+namespace mq {
+
+constexpr int kM4Threads = 256;
+constexpr int kM4Unroll = 2;
+
+// clamp(ceil(log2(q)), -127, 127) + 127 for q >= 0 (q == 0 -> -inf -> 0; inf -> 254)
+__device__ __forceinline__ uint32_t mxfp4_scale_byte(float q) {
+    const uint32_t u = f2u(q) & 0x7FFFFFFFu;
+    const uint32_t e = u >> 23, m = u & 0x7FFFFFu;
+    if (e == 0) return m > 0x400000u ? 1u : 0u;   // below 2^-126: -126 only above 2^-127
+    uint32_t s = e + (m != 0);
+    return s > 254u ? 254u : s;
+}
+// 2^(127 - byte): the multiplier that normalizes a group
+__device__ __forceinline__ float mxfp4_normalizer(uint32_t byte) {
+    return u2f(byte == 254u ? 0x00400000u : (254u - byte) << 23);
+}
+__device__ __forceinline__ uint32_t mxfp4_code(float x, float mult) {
+    const float a = __builtin_fabsf(x * mult);
+    const uint32_t mag = (a > 0.25f) + (a > 0.75f) + (a > 1.25f) + (a > 1.75f) + (a > 2.5f) + (a > 3.5f) + (a > 5.0f);
+    return mag | ((f2u(x) >> 31) << 3);
+}
+
+__global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const FlatTable tab) {
+    const FlatJob& job = tab.job[blockIdx.y];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ packed = (uint32_t*)job.q;
+    uint8_t* __restrict__ scale = (uint8_t*)job.s;
+    const int64_t total_units = job.units;
+    const int t = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kM4Threads * kM4Unroll);
+    if (base >= total_units) return;
+    u32x4 v[kM4Unroll];
+#pragma unroll
+    for (int i = 0; i < kM4Unroll; i++) {
+        const int64_t unit = base + i * kM4Threads + t;
+        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int i = 0; i < kM4Unroll; i++) {
+        const int64_t unit = base + i * kM4Threads + t;
+        const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
+        const uint32_t mb = group_max4(hmax_u16(m2));
+        const uint32_t byte = mxfp4_scale_byte(u2f(mb << 16) / 6.0f);
+        const float mult = mxfp4_normalizer(byte);
+        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) word |= mxfp4_code(f[j], mult) << (4 * j);
+        if (unit < total_units) {
+            st4(packed + unit, word);
+            if ((t & 3) == 0) scale[unit >> 2] = (uint8_t)byte;
+        }
+    }
+}
+
+// any dtype, any group size: scales first (one lane per group), then one lane per output byte
+__global__ __launch_bounds__(256) void mxfp4_scale_generic_kernel(const void* __restrict__ w, int dtype,
+                                                                  uint8_t* __restrict__ scale, int64_t groups,
+                                                                  int G) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups; g += stride) {
+        uint32_t m = 0;
+        for (int j = 0; j < G; j++) m = umax(m, f2u(load_f32(w, g * G + j, dtype)) & 0x7FFFFFFFu);
+        scale[g] = (uint8_t)mxfp4_scale_byte(u2f(m) / 6.0f);
+    }
+}
+__global__ __launch_bounds__(256) void mxfp4_pack_generic_kernel(const void* __restrict__ w, int dtype,
+                                                                 const uint8_t* __restrict__ scale,
+                                                                 uint8_t* __restrict__ packed, int64_t bytes, int G) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < bytes; b += stride) {
+        const int64_t i0 = 2 * b, i1 = 2 * b + 1;
+        const uint32_t lo = mxfp4_code(load_f32(w, i0, dtype), mxfp4_normalizer(scale[i0 / G]));
+        const uint32_t hi = mxfp4_code(load_f32(w, i1, dtype), mxfp4_normalizer(scale[i1 / G]));
+        packed[b] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+// ---- dequantize ---------------------------------------------------------------------------------
+// bf16 bit patterns of +{0, .5, 1, 1.5, 2, 3, 4, 6}
+__device__ __forceinline__ uint32_t e2m1_bf16_bits(uint32_t mag) {
+    const uint64_t lo = 0x3FC03F803F000000ull, hi = 0x40C0408040404000ull;
+    return (uint32_t)(((mag & 4u) ? hi : lo) >> ((mag & 3u) * 16)) & 0xFFFFu;
+}
+// bf16(sign * value * 2^(s-127)): the product has at most two significant bits and bf16 shares fp32's exponent
+// range, so it is exact whenever it is finite; s == 255 means 2^128 = inf (0 * inf = NaN, emitted as 0x7FC0).
+__device__ __forceinline__ uint32_t mxfp4_decode(uint32_t code, uint32_t s) {
+    const uint32_t mag = code & 7u, sign = (code & 8u) << 12;
+    if (s == 255u) return mag == 0 ? 0x7FC0u : (sign | 0x7F80u);
+    const float factor = u2f(s == 0 ? 0x00400000u : s << 23);
+    const float v = u2f(e2m1_bf16_bits(mag) << 16) * factor;
+    return sign | (f2u(v) >> 16);
+}
+
+// flat: one lane per 4 packed bytes (8 codes -> 16 bytes of bf16); G = 8 << group_shift
+__global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint32_t* __restrict__ packed,
+                                                            const uint8_t* __restrict__ scale,
+                                                            uint16_t* __restrict__ y, int64_t units,
+                                                            int group_shift) {
+    const int64_t unit = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (unit >= units) return;
+    const uint32_t word = __builtin_nontemporal_load(packed + unit);
+    const uint32_t s = scale[unit >> group_shift];
+    uint32_t c[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) c[j] = mxfp4_decode((word >> (4 * j)) & 0xFu, s);
+    st16(y + unit * 8, u32x4{c[0] | (c[1] << 16), c[2] | (c[3] << 16), c[4] | (c[5] << 16), c[6] | (c[7] << 16)});
+}
+__global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_t* __restrict__ packed,
+                                                                    const uint8_t* __restrict__ scale,
+                                                                    uint16_t* __restrict__ y, int64_t bytes, int G) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < bytes; b += stride) {
+        const uint32_t p = packed[b];
+        y[2 * b] = (uint16_t)mxfp4_decode(p & 0xFu, scale[(2 * b) / G]);
+        y[2 * b + 1] = (uint16_t)mxfp4_decode(p >> 4, scale[(2 * b + 1) / G]);
+    }
+}
+
+}  // namespace mq
+
+using namespace mq;
+
+bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group) {
+    return dtype == MQ_BF16 && group == 32 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)packed % 4) == 0;
+}
+
+int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st) {
+    if (!flat_grid(tab, kM4Threads * kM4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) return MQ_OK;
+    hipLaunchKernelGGL(mxfp4_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kM4Threads), 0, st, tab);
+    return mq_check_launch("mxfp4 quant");
+}
+
+extern "C" int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t* scale, int64_t numel, int group,
+                              void* stream) {
+    if (!w || !packed || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (numel % group != 0 || numel % 2 != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the group size and of 2");
+    if (numel == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (mq_mxfp4_fast_ok(w, dtype, packed, group)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, packed, scale, nullptr, numel / 8, nullptr, 0, 0};
+        return mq_mxfp4_launch_group(tab, st);
+    }
+    const int64_t groups = numel / group, bytes = numel / 2;
+    int64_t blocks = (groups + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(mxfp4_scale_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, scale, groups, group);
+    int rc = mq_check_launch("mxfp4 scales");
+    if (rc != MQ_OK) return rc;
+    blocks = (bytes + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(mxfp4_pack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, dtype, (const uint8_t*)scale, packed, bytes, group);
+    return mq_check_launch("mxfp4 pack");
+}
+
+extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, void* y, int64_t bytes, int group,
+                                void* stream) {
+    if (!packed || !scale || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (bytes < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if ((2 * bytes) % group != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the group size");
+    if (bytes == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int upg = group / 8;
+    if (group % 8 == 0 && (upg & (upg - 1)) == 0 && bytes % 4 == 0 && ((uintptr_t)packed % 4) == 0 &&
+        ((uintptr_t)y % 16) == 0) {
+        int shift = 0;
+        while ((1 << shift) < upg) shift++;
+        const int64_t units = bytes / 4;
+        const int64_t blocks = (units + 255) / 256;
+        if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+        hipLaunchKernelGGL(mxfp4_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)packed, scale,
+                           (uint16_t*)y, units, shift);
+        return mq_check_launch("mxfp4 dequant");
+    }
+    int64_t blocks = (bytes + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(mxfp4_dequant_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, packed, scale, (uint16_t*)y,
+                       bytes, group);
+    return mq_check_launch("mxfp4 dequant");
+}

@@ -25,6 +25,8 @@ int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st);
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st);
+bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
+int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 
 // Upper bound on the input bytes of one NVFP4 group (amax launch + fold + quantize launch).  Measured on
 // MI355X the second read of a tensor gains nothing from the memory-side cache at any group size, so groups
@@ -48,13 +50,15 @@ static bool job_fast(const mq_job& j) {
             return mq_int4_pack_fast_ok(j.in, j.dtype, j.p0) && j.cols % j.p0 == 0 && j.cols % 8 == 0;
         case MQ_JOB_NVFP4:
             return mq_nvfp4_fast_ok(j.in, j.dtype, j.out) && j.cols % 16 == 0 && (j.p0 == 448 || j.p0 == 256);
+        case MQ_JOB_MXFP4:
+            return mq_mxfp4_fast_ok(j.in, j.dtype, j.out, j.p0);
         default:
             return false;
     }
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_NVFP4) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_MXFP4) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
@@ -80,6 +84,8 @@ static int run_single(const mq_job& j, void* stream) {
             return mq_mxfp8_quant(j.in, j.dtype, j.out, (uint8_t*)j.scale, j.rows, j.cols, stream);
         case MQ_JOB_INT4_PACK:
             return mq_int4_group_quant_pack(j.in, j.dtype, (int32_t*)j.out, j.scale, j.rows, j.cols, j.p0, stream);
+        case MQ_JOB_MXFP4:
+            return mq_mxfp4_quant(j.in, j.dtype, (uint8_t*)j.out, (uint8_t*)j.scale, j.rows * j.cols, j.p0, stream);
         default:
             return mq_fail(MQ_ERR_ARG, "unknown job kind");
     }
@@ -215,6 +221,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                 break;
             }
             case MQ_JOB_MXFP8:
+            case MQ_JOB_MXFP4:
             case MQ_JOB_INT4_PACK: {
                 FlatTable tab{};
                 tab.n = cnt;
@@ -222,8 +229,9 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                     const mq_job& jb = jobs[i + t];
                     tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8};
                 }
-                rc = head.kind == MQ_JOB_MXFP8 ? mq_mxfp8_launch_group(tab, st)
-                                               : mq_int4_pack_launch_group(tab, head.p0, st);
+                rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_group(tab, st)
+                     : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_group(tab, st)
+                                                 : mq_int4_pack_launch_group(tab, head.p0, st);
                 break;
             }
             default:

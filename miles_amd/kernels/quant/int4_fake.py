@@ -40,20 +40,21 @@ def fake_int4_quant_cuda(x: torch.Tensor, block_size, sym: bool):
 
 
 def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
-    """weight [M, K] -> (int32 [M, K/8], weight.dtype [M, K/group_size], None).
+    """weight [M, K] -> (int32 [M, K/8], weight.dtype [M, K/group_size], packed zero points or None).
 
     Fused form of the reference's `pack_layer`
     (miles/backends/megatron_utils/megatron_to_hf/processors/quantizer_compressed_tensors.py:235-265,
-    identical to tools/convert_hf_to_int4_direct.py:121-151) for the symmetric case: the fake-quant
-    kernel, the bf16 dequantize/requantize round trip and pack_to_int32 collapse into one pass that writes
-    the packed words and the scales directly.
+    identical to tools/convert_hf_to_int4_direct.py:121-151): the fake-quant kernel, the dequantize/requantize
+    round trip in the weight's dtype and pack_to_int32 collapse into one pass that writes the packed words
+    and the scales directly.  With sym=False the third result is the AWQ-ordered int32 [K/group_size, M/8]
+    zero-point tensor; with sym=True it is None.
     """
     _lib.require_gpu(weight, "pack_layer")
-    if not sym:
-        raise NotImplementedError("asymmetric pack_layer is not implemented on gfx950")
     if weight.dim() != 2:
         raise RuntimeError("Input must be 2D")
     M, K = weight.shape
+    if not sym:
+        return _pack_layer_asym(weight, int(group_size))
     if K % group_size != 0 or K % 8 != 0:
         raise RuntimeError(f"shape {tuple(weight.shape)} is not divisible into groups of {group_size} and words of 8")
     w = weight.contiguous()
@@ -62,3 +63,22 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
     _lib.dtype_code(w, "pack_layer")
     launch.submit(_lib.JOB_INT4_PACK, w, packed, scale, None, None, M, K, K, int(group_size), 0)
     return packed, scale, None
+
+
+def _pack_layer_asym(weight: torch.Tensor, group_size: int):
+    M, K = weight.shape
+    if K % group_size != 0 or group_size % 8 != 0 or M % 8 != 0:
+        raise RuntimeError(f"shape {tuple(weight.shape)} is not divisible into groups of {group_size}, "
+                           f"words of 8 and zero-point words of 8 rows")
+    w = weight.contiguous()
+    groups = K // group_size
+    packed = torch.empty((M, K // 8), dtype=torch.int32, device=w.device)
+    scale = torch.empty((M, groups), dtype=w.dtype, device=w.device)
+    zero = torch.empty((M, groups), dtype=torch.uint8, device=w.device)
+    packed_zp = torch.empty((groups, M // 8), dtype=torch.int32, device=w.device)
+    launch.note_direct_call()
+    rc = _lib.load().mq_int4_group_quant_pack_asym(w.data_ptr(), _lib.dtype_code(w, "pack_layer"), packed.data_ptr(),
+                                                   scale.data_ptr(), zero.data_ptr(), packed_zp.data_ptr(), M, K,
+                                                   group_size, _lib.stream_ptr(w.device))
+    _lib.check(rc, RuntimeError)
+    return packed, scale, packed_zp

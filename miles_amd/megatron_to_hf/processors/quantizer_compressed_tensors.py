@@ -10,6 +10,7 @@ from __future__ import annotations
 import torch
 
 from miles_amd.kernels.quant.int4_fake import pack_layer
+from miles_amd.utils.mxfp4 import quantize_mxfp4
 
 __all__ = ["quantize_params_compressed_tensors", "pack_layer"]
 
@@ -18,13 +19,22 @@ def quantize_params_compressed_tensors(converted_named_params, quantization_conf
     weights_cfg = quantization_config["config_groups"]["group_0"]["weights"]
     group_size = weights_cfg["group_size"]
     symmetric = weights_cfg["symmetric"]
-    if quantization_config["format"] == "mxfp4-pack-quantized":
-        raise NotImplementedError("mxfp4-pack-quantized checkpoints are not implemented on gfx950")
+    is_mxfp4 = quantization_config["format"] == "mxfp4-pack-quantized"
+    if is_mxfp4:
+        assert weights_cfg["type"] == "float"
+        assert weights_cfg["num_bits"] == 4
+        assert weights_cfg["scale_dtype"] == "torch.uint8"
+        assert symmetric
 
     out = []
     for name, param in converted_named_params:
         if not (name.endswith(".weight") and name.removesuffix(".weight") in packed_weight_basenames):
             out.append((name, param))
+            continue
+        if is_mxfp4:   # only the packed codes and the E8M0 scales are published for this format
+            packed, scale = quantize_mxfp4(param, group_size)
+            out.append((name.replace(".weight", ".weight_packed"), packed))
+            out.append((name.replace(".weight", ".weight_scale"), scale))
             continue
         packed, scale, zero_point = pack_layer(param, group_size, symmetric)
         shape = torch.tensor(param.shape, dtype=torch.int32, device=param.device)

@@ -354,6 +354,54 @@ void mqo_mxfp8(const void* w, int dtype, int64_t rows, int64_t K, uint8_t* q, ui
 }
 
 /* ------------------------------------------------------------------ */
+/* MXFP4 (miles/utils/mxfp4.py:11-59): torch ops restated one by one    */
+/* ------------------------------------------------------------------ */
+/* quantize_mxfp4 (:11-31).  Groups of G consecutive elements of the flattened tensor.
+ *   amax = max|x| (.float())                      (:16)
+ *   e = clamp(ceil(log2(amax / 6.0)), -127, 127)  (:17)  log2f(0) = -inf clamps to -127
+ *   n = f32(x) * exp2(-e)                         (:18)  exp2 of an integer is an exact power of two
+ *   magnitude = number of bounds below |n|        (:20-22) strict '>': a tie takes the smaller magnitude
+ *   code = magnitude | signbit(n) << 3            (:23)
+ *   byte j = code[2j] | code[2j+1] << 4           (:25)
+ *   scale = uint8(e + 127)                        (:27) */
+void mqo_mxfp4_quant(const void* w, int dtype, int64_t numel, int G, uint8_t* packed, uint8_t* scale) {
+    static const float bound[7] = {0.25f, 0.75f, 1.25f, 1.75f, 2.5f, 3.5f, 5.0f};
+    int64_t groups = numel / G;
+    uint8_t* code = (uint8_t*)malloc((size_t)numel + 1);
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < groups; g++) {
+        float amax = 0.0f;
+        for (int j = 0; j < G; j++) amax = fmaxf(amax, fabsf(load_as_f32(w, g * G + j, dtype)));
+        float e = ceilf(log2f(amax / 6.0f));
+        if (e < -127.0f) e = -127.0f;
+        if (e > 127.0f) e = 127.0f;
+        float mult = ldexpf(1.0f, -(int)e);
+        for (int j = 0; j < G; j++) {
+            float n = load_as_f32(w, g * G + j, dtype) * mult;
+            uint8_t mag = 0;
+            for (int b = 0; b < 7; b++) mag += fabsf(n) > bound[b];
+            code[g * G + j] = (uint8_t)(mag | ((signbit(n) ? 1 : 0) << 3));
+        }
+        scale[g] = (uint8_t)(e + 127.0f);
+    }
+    for (int64_t j = 0; j < numel / 2; j++) packed[j] = (uint8_t)(code[2 * j] | (code[2 * j + 1] << 4));
+    free(code);
+}
+
+/* dequantize_mxfp4 (:34-59): value = sign * {0,.5,1,1.5,2,3,4,6}[code & 7], sign = 1 - 2*bit3 (so a set sign
+ * bit on magnitude 0 gives -0); y = bf16(value * exp2(scale - 127)); exp2(128) overflows to inf. */
+void mqo_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, int64_t bytes, int G, uint16_t* y) {
+    static const float value[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < 2 * bytes; i++) {
+        uint8_t c = (i & 1) ? (packed[i / 2] >> 4) : (packed[i / 2] & 0xF);
+        float sign = 1.0f - 2.0f * (float)((c >> 3) & 1);
+        float s = ldexpf(1.0f, (int)scale[i / G] - 127);
+        y[i] = f32_to_bf16(sign * value[c & 7] * s);
+    }
+}
+
+/* ------------------------------------------------------------------ */
 /* A-3  INT4 fake quant (miles/kernels/quant/int4_fake/                 */
 /*      fake_int4_quant_cuda.cu:159-259 for (1,G); :29-91 for (1,32))   */
 /* ------------------------------------------------------------------ */
@@ -381,6 +429,9 @@ void mqo_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int G, 
             else {
                 scale = fmaxf((mx - mn) * ASYM, 1e-5f);
                 zero = fminf(fmaxf(-rintf(mn / scale), 0.0f), 15.0f);
+                /* the device max orders -0 below +0, so a group whose minimum is 0 gets +0 (C's fmaxf
+                 * may return either zero) */
+                if (zero == 0.0f) zero = 0.0f;
             }
             for (int64_t c = c0; c < c1; c++) {
                 float v = rintf(load_as_f32(x, r * N + c, dtype) / scale); /* keeps -0 */
@@ -435,6 +486,51 @@ void mqo_int4_pack_layer(const void* w, int dtype, int64_t M, int64_t K, int G,
             packed[r * np + j] = (int32_t)word;
         }
     free(out);
+}
+
+/* pack_layer(weight, G, sym=False)  (same file, :235-264):
+ *   (out, scale_b, zero_b) = fake_int4_quant(x, sym=False)   -- in the input dtype
+ *   w  = dtype(dtype(out - zero_b) * scale_b)                (:243)
+ *   r  = dtype(dtype(w / scale_b) + zero_b)                  (:213-217)
+ *   q  = uint8(round_half_even(clamp(r, 0, 255)))            (:190)
+ *   packed[m,j] = sum_i q[m,8j+i] << 4i                      (:173-175; no offset when sym=False, :153)
+ *   packed_zp[g,j] = sum_i int32(zero[8j+i,g]) << 4*{0,4,1,5,2,6,3,7}[i]   (:247-254)
+ * K % G == 0, G % 8 == 0, M % 8 == 0. */
+void mqo_int4_pack_layer_asym(const void* w, int dtype, int64_t M, int64_t K, int G,
+                              int32_t* packed, void* scale_out, int32_t* packed_zp) {
+    static const int order[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+    size_t esz = dtype == MQ_F32 ? 4 : 2;
+    int64_t ng = K / G, np = K / 8;
+    void* out = malloc((size_t)M * K * esz);
+    void* zero = malloc((size_t)M * ng * esz);
+    mqo_int4_fake_quant(w, dtype, M, K, G, 0, out, scale_out, zero);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t j = 0; j < np; j++) {
+            uint32_t word = 0;
+            for (int i = 0; i < 8; i++) {
+                int64_t c = j * 8 + i;
+                float q0 = load_as_f32(out, r * K + c, dtype);
+                float sb = load_as_f32(scale_out, r * ng + c / G, dtype);
+                float zb = load_as_f32(zero, r * ng + c / G, dtype);
+                float wv = round_to_dtype(round_to_dtype(q0 - zb, dtype) * sb, dtype);
+                float rv = round_to_dtype(round_to_dtype(wv / sb, dtype) + zb, dtype);
+                if (rv < 0.0f) rv = 0.0f;
+                if (rv > 255.0f) rv = 255.0f;
+                uint8_t code = (uint8_t)nearbyintf(rv);
+                word += (uint32_t)code << (4 * i);
+            }
+            packed[r * np + j] = (int32_t)word;
+        }
+    for (int64_t g = 0; g < ng; g++)
+        for (int64_t j = 0; j < M / 8; j++) {
+            uint32_t word = 0;
+            for (int i = 0; i < 8; i++)
+                word += (uint32_t)(int32_t)load_as_f32(zero, (j * 8 + i) * ng + g, dtype) << (4 * order[i]);
+            packed_zp[g * (M / 8) + j] = (int32_t)word;
+        }
+    free(out);
+    free(zero);
 }
 
 /* ------------------------------------------------------------------ */

@@ -65,8 +65,14 @@ def lib() -> ctypes.CDLL:
         L.mqo_mxfp8.argtypes = [vp, i32, i64, i64, vp, vp]
         L.mqo_int4_fake_quant.restype = None
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
+        L.mqo_mxfp4_quant.restype = None
+        L.mqo_mxfp4_quant.argtypes = [vp, i32, i64, i32, vp, vp]
+        L.mqo_mxfp4_dequant.restype = None
+        L.mqo_mxfp4_dequant.argtypes = [vp, vp, i64, i32, vp]
         L.mqo_int4_pack_layer.restype = None
         L.mqo_int4_pack_layer.argtypes = [vp, i32, i64, i64, i32, vp, vp]
+        L.mqo_int4_pack_layer_asym.restype = None
+        L.mqo_int4_pack_layer_asym.argtypes = [vp, i32, i64, i64, i32, vp, vp, vp]
         L.mqo_nvfp4_amax.restype = f32
         L.mqo_nvfp4_amax.argtypes = [vp, i32, i64]
         L.mqo_nvfp4_global_encode_scale.restype = f32
@@ -195,17 +201,50 @@ def fake_int4_quant(x: torch.Tensor, block_size, sym: bool):
 
 
 def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
-    """quantizer_compressed_tensors.py:235-265 (sym) -> (int32 [M,K/8], dtype [M,K/G], None)."""
+    """quantizer_compressed_tensors.py:235-265 -> (int32 [M,K/8], dtype [M,K/G], None | int32 [K/G,M/8])."""
     _check_cpu(weight)
-    assert sym, "the oracle restates the symmetric branch"
     weight = weight.contiguous()
     M, K = weight.shape
     assert K % group_size == 0 and K % 8 == 0
     packed = torch.empty((M, K // 8), dtype=torch.int32)
     scale = torch.empty((M, K // group_size), dtype=weight.dtype)
+    if not sym:
+        assert group_size % 8 == 0 and M % 8 == 0
+        packed_zp = torch.empty((K // group_size, M // 8), dtype=torch.int32)
+        lib().mqo_int4_pack_layer_asym(weight.data_ptr(), _DTYPE[weight.dtype], M, K, int(group_size),
+                                       packed.data_ptr(), scale.data_ptr(), packed_zp.data_ptr())
+        return packed, scale, packed_zp
     lib().mqo_int4_pack_layer(weight.data_ptr(), _DTYPE[weight.dtype], M, K, int(group_size),
                               packed.data_ptr(), scale.data_ptr())
     return packed, scale, None
+
+
+# --------------------------------------------------------------------------
+# MXFP4
+# --------------------------------------------------------------------------
+def quantize_mxfp4(weight: torch.Tensor, group_size: int):
+    """miles/utils/mxfp4.py:11-31 -> (uint8 [..., K/2], uint8 [..., K/group_size])."""
+    _check_cpu(weight)
+    assert weight.shape[-1] % group_size == 0
+    assert weight.shape[-1] % 2 == 0
+    w = weight.contiguous()
+    k = w.shape[-1]
+    packed = torch.empty((*w.shape[:-1], k // 2), dtype=torch.uint8)
+    scale = torch.empty((*w.shape[:-1], k // group_size), dtype=torch.uint8)
+    lib().mqo_mxfp4_quant(w.data_ptr(), _DTYPE[w.dtype], w.numel(), int(group_size), packed.data_ptr(),
+                          scale.data_ptr())
+    return packed, scale
+
+
+def dequantize_mxfp4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, group_size: int) -> torch.Tensor:
+    """miles/utils/mxfp4.py:34-59 -> bfloat16 [..., K]."""
+    assert weight_packed.device.type == "cpu" and weight_scale.device.type == "cpu", "the oracle runs on CPU tensors"
+    assert weight_packed.dtype == torch.uint8 and weight_scale.dtype == torch.uint8 and group_size > 0
+    p, s = weight_packed.contiguous(), weight_scale.contiguous()
+    assert (2 * p.numel()) % group_size == 0 and s.numel() == 2 * p.numel() // group_size
+    out = torch.empty((*p.shape[:-1], p.shape[-1] * 2), dtype=torch.bfloat16)
+    lib().mqo_mxfp4_dequant(p.data_ptr(), s.data_ptr(), p.numel(), int(group_size), out.data_ptr())
+    return out
 
 
 # --------------------------------------------------------------------------

@@ -266,6 +266,38 @@ def test_int4_pack_layer_other_dtypes(oracle, dtype):
     _assert_same(packed, packed_o, "packed")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((8, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((24, 7168), 128),
+                                     ((16, 256), 32), ((24, 192), 64), ((8, 2048), 1024), ((2048, 7168), 128)])
+def test_int4_pack_layer_asymmetric(oracle, shape, G, dtype):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    if shape[0] > 1000 and dtype != torch.bfloat16:
+        pytest.skip("the full-size tensor is checked in bf16 only")
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.0005, gain=30.0, seed=4101, dtype=dtype)
+    w[0] = 0                      # zero range: scale floor, zero point +0
+    w[1] = w[1].abs() + 0.25      # minimum far above zero: codes run past 15 and carry into the next nibble
+    w[2] = -w[2].abs() - 0.25     # maximum far below zero: zero point clamps to 15, codes clamp at 0
+    w[3, :G] = 3e-6
+    w[4, :G] = torch.linspace(-1, 1, G).to(dtype)
+    packed, scale, zp = pack_layer(w.to(DEV), G, sym=False)
+    packed_o, scale_o, zp_o = oracle.pack_layer(w, G, sym=False)
+    assert packed.dtype == torch.int32 and scale.dtype == dtype and zp.dtype == torch.int32
+    assert zp.shape == (shape[1] // G, shape[0] // 8)
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(zp, zp_o, "packed zero points")
+    _assert_same(packed, packed_o, "packed")
+
+
+def test_int4_pack_layer_asymmetric_argument_checks():
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    with pytest.raises(RuntimeError, match="not divisible"):
+        pack_layer(torch.zeros(4, 128, dtype=torch.bfloat16, device=DEV), 128, sym=False)   # rows % 8
+    with pytest.raises(RuntimeError, match="not divisible"):
+        pack_layer(torch.zeros(8, 96, dtype=torch.bfloat16, device=DEV), 128, sym=False)
+
+
 @pytest.mark.parametrize("sym", [True, False])
 @pytest.mark.parametrize("shape,G", [((16, 256), 128), ((8, 200), 32), ((4, 128), 32), ((3, 7168), 128)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -293,6 +325,99 @@ def test_fake_int4_quant_argument_checks():
         fake_int4_quant_cuda(x.reshape(2, 2, 64), (1, 32), True)
     with pytest.raises(RuntimeError, match="Input must be on CUDA"):
         fake_int4_quant_cuda(x.cpu(), (1, 32), True)
+
+
+# ---------------------------------------------------------------------------------------------------
+# MXFP4 (miles/utils/mxfp4.py)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((16, 64), 32), ((3, 128), 32), ((64, 64), 32), ((8, 2048), 32), ((4, 64), 16),
+                                     ((5, 24), 4), ((2, 3, 64), 32), ((513, 7168), 32)])
+def test_mxfp4_quantize(oracle, shape, G, dtype):
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+
+    rows = 1
+    for d in shape[:-1]:
+        rows *= d
+    w = W.student_t_rows((rows, shape[-1]), std=0.02, seed=6001).reshape(shape).to(dtype)
+    flat = w.reshape(-1, shape[-1])
+    flat[0, :G] = 0
+    flat[1, :G] = torch.tensor([6.0, -6.0, 3.0, 0.25] * (G // 4)).to(dtype)
+    flat[2, :4] = torch.tensor([0.75, 1.75, 3.5, -0.0]).to(dtype)
+    flat[2, 4] = 6.0
+    packed, scale = quantize_mxfp4(w.to(DEV), G)
+    packed_o, scale_o = oracle.quantize_mxfp4(w, G)
+    assert packed.dtype == torch.uint8 and scale.dtype == torch.uint8
+    assert packed.shape == packed_o.shape and scale.shape == scale_o.shape
+    _assert_same(scale, scale_o, "E8M0 scales")
+    _assert_same(packed, packed_o, "packed codes")
+
+
+def test_mxfp4_quantize_extreme_magnitudes(oracle):
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+
+    # groups of denormals (scale exponent clamps at -127), of the largest finite bf16 values, and ties at every bound
+    tiny = torch.tensor([1, 2, 3, 0x40, 0x7F, 0x80, 0x81, 0x100] * 4, dtype=torch.int16).view(torch.bfloat16)
+    huge = torch.tensor([0x7F7F, 0x7F00, 0x7E80, -0x7F7F + 0x10000 - 0x10000] * 8, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4, dtype=torch.bfloat16)
+    w = torch.stack([tiny, -tiny, huge, ties, ties * 2 ** -20, -ties * 2 ** 40])
+    packed, scale = quantize_mxfp4(w.to(DEV), 32)
+    packed_o, scale_o = oracle.quantize_mxfp4(w, 32)
+    _assert_same(scale, scale_o, "E8M0 scales")
+    _assert_same(packed, packed_o, "packed codes")
+
+
+def test_mxfp4_dequantize_reference_golden_and_all_codes(oracle):
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4
+
+    packed = torch.tensor([[0x10, 0x32, 0x54, 0x76]], dtype=torch.uint8)
+    scales = torch.tensor([127, 128], dtype=torch.uint8)
+    expected = torch.tensor([[0.0, 0.5, 1.0, 1.5, 4.0, 6.0, 8.0, 12.0]], dtype=torch.bfloat16)
+    got = dequantize_mxfp4(packed.to(DEV), scales.to(DEV), 4)      # tests/fast/.../test_quantizer_mxfp4.py:6-16
+    assert got.dtype == torch.bfloat16 and torch.equal(got.cpu(), expected)
+    # every byte under every scale byte (0 = 2^-127 ... 254 = 2^127, 255 = 2^128 = inf), packed and generic paths
+    packed = torch.arange(256, dtype=torch.uint8).repeat(256, 1)
+    scales = torch.arange(256, dtype=torch.int32).to(torch.uint8).repeat_interleave(16)
+    for G, sc in ((32, scales), (512, torch.arange(256, dtype=torch.int32).to(torch.uint8)), (2, None)):
+        if sc is None:
+            sc = torch.arange(256, dtype=torch.int32).to(torch.uint8).repeat_interleave(256)
+        got = dequantize_mxfp4(packed.to(DEV), sc.to(DEV), G)
+        want = oracle.dequantize_mxfp4(packed, sc, G)
+        _assert_same(got, want, f"dequantized values, group {G}")
+
+
+def test_mxfp4_requantizing_a_checkpoint_is_the_identity():
+    from miles_amd.megatron_to_hf.processors.quantizer_compressed_tensors import quantize_params_compressed_tensors
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+
+    # tests/fast-gpu/test_quantizer_ci.py:41-91
+    g = torch.Generator().manual_seed(11)
+    packed = torch.randint(0, 256, (16, 64), dtype=torch.uint8, generator=g).to(DEV)
+    scale = torch.randint(96, 144, (16, 4), dtype=torch.uint8, generator=g).to(DEV)
+    weight = dequantize_mxfp4(packed, scale, 32)
+    p2, s2 = quantize_mxfp4(weight, 32)
+    assert torch.equal(dequantize_mxfp4(p2, s2, 32).view(torch.int16), weight.view(torch.int16))
+    config = {"format": "mxfp4-pack-quantized",
+              "config_groups": {"group_0": {"weights": {"group_size": 32, "symmetric": True, "type": "float",
+                                                        "num_bits": 4, "scale_dtype": "torch.uint8"}}}}
+    results = quantize_params_compressed_tensors(
+        [("model.layers.0.experts.0.w1.weight", torch.randn(64, 64, device=DEV))], config,
+        {"model.layers.0.experts.0.w1"})
+    assert [(n, t.dtype, tuple(t.shape)) for n, t in results] == [
+        ("model.layers.0.experts.0.w1.weight_packed", torch.uint8, (64, 32)),
+        ("model.layers.0.experts.0.w1.weight_scale", torch.uint8, (64, 2))]
+
+
+def test_mxfp4_grouped_jobs(oracle):
+    from miles_amd import launch
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+
+    ws = [W.student_t_rows((96 + 32 * i, 256), std=0.02, seed=6100 + i) for i in range(5)]
+    with launch.deferred():
+        outs = [quantize_mxfp4(w.to(DEV), 32) for w in ws]
+    for w, (p, s) in zip(ws, outs):
+        p_o, s_o = oracle.quantize_mxfp4(w, 32)
+        _assert_same(s, s_o, "E8M0 scales (grouped)")
+        _assert_same(p, p_o, "packed codes (grouped)")
 
 
 # ---------------------------------------------------------------------------------------------------

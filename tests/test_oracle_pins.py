@@ -13,6 +13,7 @@ independent torch restatement only -- "parity unpinned" against TE itself.
 
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -312,6 +313,102 @@ def test_mxfp8_student_t_rows_and_invariants(oracle):
 
 
 # ----------------------------------------------------------------------------------------------
+# MXFP4 (miles/utils/mxfp4.py) -- the reference is plain torch ops, restated here op for op
+# ----------------------------------------------------------------------------------------------
+def torch_quantize_mxfp4(weight, group_size):
+    """miles/utils/mxfp4.py:11-31."""
+    blocks = weight.reshape(-1, group_size)
+    amax = blocks.abs().amax(dim=-1, keepdim=True).float()
+    scale_exp = torch.ceil(torch.log2(amax / 6.0)).clamp_(-127, 127)
+    normalized = blocks.float() * torch.exp2(-scale_exp)
+    magnitude = torch.zeros_like(normalized, dtype=torch.uint8)
+    for bound in (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0):
+        magnitude.add_(normalized.abs() > bound)
+    encoded = magnitude | (torch.signbit(normalized).to(torch.uint8) << 3)
+    packed = encoded[:, 0::2] | (encoded[:, 1::2] << 4)
+    packed = packed.reshape(*weight.shape[:-1], weight.shape[-1] // 2).contiguous()
+    scale = (scale_exp + 127).to(torch.uint8)
+    return packed, scale.reshape(*weight.shape[:-1], weight.shape[-1] // group_size).contiguous()
+
+
+def torch_dequantize_mxfp4(weight_packed, weight_scale, group_size):
+    """miles/utils/mxfp4.py:34-59."""
+    unpacked = torch.empty(*weight_packed.shape[:-1], weight_packed.shape[-1] * 2, dtype=torch.uint8)
+    unpacked[..., 0::2] = weight_packed & 0x0F
+    unpacked[..., 1::2] = (weight_packed >> 4) & 0x0F
+    signs = 1.0 - 2.0 * ((unpacked & 0b1000) >> 3).float()
+    values = torch.tensor((0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0), dtype=torch.float32)
+    dequantized = (signs * values[(unpacked & 0b0111).long()]).reshape(-1, group_size)
+    scales = torch.exp2(weight_scale.float().reshape(-1, 1) - 127.0)
+    return (dequantized * scales).reshape(unpacked.shape).to(torch.bfloat16).contiguous()
+
+
+def test_mxfp4_dequantize_reference_golden(oracle):
+    # tests/fast/backends/megatron_utils/test_quantizer_mxfp4.py:6-16: nibble order, sign bit, E8M0 bias
+    packed = torch.tensor([[0x10, 0x32, 0x54, 0x76]], dtype=torch.uint8)
+    scales = torch.tensor([127, 128], dtype=torch.uint8)
+    expected = torch.tensor([[0.0, 0.5, 1.0, 1.5, 4.0, 6.0, 8.0, 12.0]], dtype=torch.bfloat16)
+    assert torch.equal(oracle.dequantize_mxfp4(packed, scales, 4), expected)
+
+
+def test_mxfp4_dequantize_all_codes_all_scales(oracle):
+    packed = torch.arange(256, dtype=torch.uint8).repeat(255, 1)            # [255, 256] -> 512 values per row
+    scales = torch.arange(255, dtype=torch.uint8).repeat_interleave(16)     # group 32: 16 groups per row
+    got = oracle.dequantize_mxfp4(packed, scales, 32)
+    want = torch_dequantize_mxfp4(packed, scales, 32)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((16, 64), 32), ((3, 128), 32), ((64, 64), 32), ((8, 2048), 32), ((4, 64), 16),
+                                     ((5, 24), 4), ((2, 3, 64), 32)])
+def test_mxfp4_quantize_matches_torch_chain(oracle, shape, G, dtype):
+    w = W.student_t_rows((int(np.prod(shape[:-1])), shape[-1]), std=0.02, seed=6001).reshape(shape).to(dtype)
+    flat = w.reshape(-1, shape[-1])
+    flat[0, :G] = 0
+    flat[1, :G] = torch.tensor([6.0, -6.0, 3.0, 0.25] * (G // 4)).to(dtype)          # amax/6 an exact power of two
+    flat[2, :4] = torch.tensor([0.75, 1.75, 3.5, -0.0]).to(dtype); flat[2, 4] = 6.0    # ties round down; -0 keeps its sign
+    packed, scale = oracle.quantize_mxfp4(w, G)
+    packed_t, scale_t = torch_quantize_mxfp4(w, G)
+    assert packed.shape == packed_t.shape and scale.shape == scale_t.shape
+    assert torch.equal(scale, scale_t) and torch.equal(packed, packed_t)
+
+
+def test_mxfp4_ties_and_signed_zero_known_answer(oracle):
+    w = torch.tensor([[0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, -0.0, -0.25, -0.75, 0.76, 0.26, 5.25, -6.0, 0.0]],
+                     dtype=torch.bfloat16)
+    packed, scale = oracle.quantize_mxfp4(w, 16)
+    codes = torch.stack([packed & 0xF, packed >> 4], dim=-1).reshape(-1).tolist()
+    assert scale.item() == 127
+    assert codes == [0, 1, 2, 3, 4, 5, 6, 7, 8, 8, 9, 2, 1, 7, 15, 0]
+
+
+def test_mxfp4_requantizing_a_checkpoint_is_the_identity(oracle):
+    # tests/fast-gpu/test_quantizer_ci.py:41-60: any value an MXFP4 checkpoint can hold re-encodes to the same bits
+    g = torch.Generator().manual_seed(11)
+    packed = torch.randint(0, 256, (16, 64), dtype=torch.uint8, generator=g)
+    scale = torch.randint(96, 144, (16, 4), dtype=torch.uint8, generator=g)
+    weight = oracle.dequantize_mxfp4(packed, scale, 32)
+    p2, s2 = oracle.quantize_mxfp4(weight, 32)
+    assert torch.equal(oracle.dequantize_mxfp4(p2, s2, 32).view(torch.int16), weight.view(torch.int16))
+
+
+def test_mxfp4_scale_exponent_from_bits_equals_float_log2_for_16_bit_inputs():
+    # the gfx950 kernel reads ceil(log2(amax/6)) off the bits of the quotient; for every bf16 and fp16 amax this
+    # equals ceil(log2f(.)) as the reference computes it
+    for dt in (torch.bfloat16, torch.float16):
+        bits = torch.arange(0, 0x7C00 if dt == torch.float16 else 0x7F80, dtype=torch.int32).to(torch.int16)
+        amax = bits.view(dt).float()
+        q = amax / 6.0
+        want = torch.ceil(torch.log2(q)).clamp_(-127, 127) + 127
+        u = q.view(torch.int32)
+        e, m = u >> 23, u & 0x7FFFFF
+        got = torch.where(e == 0, (m > 0x400000).to(torch.int32), torch.clamp(e + (m != 0).to(torch.int32), max=254))
+        assert torch.equal(got, want.to(torch.int32))
+
+
+
+# ----------------------------------------------------------------------------------------------
 # A-3 INT4
 # ----------------------------------------------------------------------------------------------
 def torch_fake_int4_sym(x, G):
@@ -358,6 +455,78 @@ def test_int4_matches_torch_chain(oracle, shape, G):
     assert nib.min() >= 1 and nib.max() <= 15
     assert torch.equal(nib.to(torch.float32) - 8, out.float())
 
+
+
+def torch_fake_int4_asym(x, G):
+    """fake_int4_quant_cuda.cu:216-254, asymmetric branch, as fp32 tensor ops on the CPU."""
+    m, n = x.shape
+    xf = x.float().reshape(m, n // G, G)
+    mx, mn = xf.amax(dim=-1, keepdim=True), xf.amin(dim=-1, keepdim=True)
+    scale = torch.maximum((mx - mn) * torch.tensor(1.0 / 15.0, dtype=torch.float32),
+                          torch.tensor(1e-5, dtype=torch.float32))
+    zero = torch.clamp(-torch.round(mn / scale), 0.0, 15.0) + 0.0   # device max(-0, +0) = +0
+    out = torch.round(xf / scale) + zero
+    return out.reshape(m, n).to(x.dtype), scale.reshape(m, n // G).to(x.dtype), zero.reshape(m, n // G).to(x.dtype)
+
+
+def torch_pack_layer_asym_python_half(w, scale, zp, G):
+    """quantizer_compressed_tensors.py:237-264 with sym=False, the reference's tensor ops in their order."""
+    m, k = w.shape
+    w4 = w.view(m, 1, k // G, G)
+    s4 = scale.view(m, 1, k // G, 1)
+    z4 = zp.view(m, 1, k // G, 1)
+    deq = ((w4 - z4) * s4).view(m, k)
+    scale2 = s4.view(m, -1).contiguous()
+    zp2 = z4.view(m, -1)
+    zeros = zp2.t().contiguous().to(torch.float32).to(torch.int32)
+    zeros = zeros.reshape(-1, zeros.shape[1] // 8, 8)
+    zeros = zeros << (torch.tensor([0, 4, 1, 5, 2, 6, 3, 7]) * 4)
+    packed_zp = torch.sum(zeros, dim=-1).to(torch.int32)
+    x = deq.unflatten(-1, (k // G, G))
+    scaled = x / scale2.unsqueeze(-1)
+    scaled += zp2.unsqueeze(-1).to(x.dtype)
+    q = torch.round(torch.clamp(scaled, 0, 255)).to(torch.uint8).flatten(start_dim=-2)
+    reshaped = q.view(m, k // 8, 8).to(torch.int32)
+    shifts = torch.arange(8, dtype=torch.int32) * 4
+    return (reshaped << shifts).sum(dim=2, dtype=torch.int32), scale2, packed_zp
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((8, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((8, 7168), 128),
+                                     ((16, 256), 32), ((24, 192), 64)])
+def test_int4_asym_matches_torch_chain(oracle, shape, G, dtype):
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.0005, gain=30.0, seed=4101).to(dtype)
+    w[0] = 0                      # range 0 -> scale floor
+    w[1] = w[1].abs() + 0.25      # minimum far above zero: zero point clamps to 0 and codes run past 15
+    w[2] = -w[2].abs() - 0.25     # maximum far below zero: zero point clamps to 15, codes clamp at 0
+    w[3, :G] = 3e-6
+    out, scale, zero = oracle.fake_int4_quant(w, (1, G), False)
+    out_t, scale_t, zero_t = torch_fake_int4_asym(w, G)
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    assert torch.equal(out.view(bits), out_t.view(bits))
+    assert torch.equal(scale.view(bits), scale_t.view(bits))
+    assert torch.equal(zero.view(bits), zero_t.view(bits))
+    packed, pscale, pzp = oracle.pack_layer(w, G, sym=False)
+    packed_t, pscale_t, pzp_t = torch_pack_layer_asym_python_half(out_t, scale_t, zero_t, G)
+    assert torch.equal(packed, packed_t)
+    assert torch.equal(pscale.view(bits), pscale_t.view(bits))
+    assert pzp.shape == (shape[1] // G, shape[0] // 8) and torch.equal(pzp, pzp_t)
+
+
+def test_int4_asym_known_answers(oracle):
+    # a group spanning [0, 15] exactly: scale 1, zero 0, codes are the values themselves
+    row = torch.arange(16, dtype=torch.float32).repeat(8)
+    w = row.to(torch.bfloat16).repeat(8, 1)
+    w[1] = w[1] - 15          # [-15, 0]: zero point 15, same codes
+    w[2] = w[2] - 7           # [-7, 8]: zero point 7
+    packed, scale, pzp = oracle.pack_layer(w, 128, sym=False)
+    want = sum(i << (4 * i) for i in range(8))
+    want2 = sum((8 + i) << (4 * i) for i in range(8))
+    for r in range(3):
+        assert scale[r, 0].item() == 1.0
+        assert (packed[r, 0].item() & 0xFFFFFFFF) == want and (packed[r, 1].item() & 0xFFFFFFFF) == want2
+    # rows 0..7 carry zero points 0,15,7,0,0,0,0,0 in nibbles 0,4,1,5,2,6,3,7
+    assert (pzp[0, 0].item() & 0xFFFFFFFF) == (0 << 0) | (15 << 16) | (7 << 4)
 
 def test_int4_constant_rows_known_answer(oracle):
     for c in (0.5, 0.013, 3.0):
