@@ -97,6 +97,12 @@ int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* sc
 int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
                                   int32_t* packed_zp, int64_t M, int64_t K, int group, void* stream);
 
+/* _dequantize_tensor(weight_packed, weight_scale, weight_shape, group_size)   tools/convert_kimi_int4_to_bf16.py:57-86
+ *   packed [M, ceil(K/8)] int32 (nibble i of word j = element 8j+i, code = value + 8)
+ *   scale  [M, K/group] bf16 / fp16 / fp32;  y [M,K] bf16 = bf16(f32(code - 8) * f32(scale)) */
+int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M, int64_t K,
+                           int group, void* stream);
+
 /* NVFP4                                              miles/utils/nvfp4.py:54-114
  * The global amax travels on the device in an "amax record": MQ_NVFP4_RECORD_WORDS uint32 words made of
  * MQ_NVFP4_SECTIONS sections of MQ_NVFP4_SECTION_WORDS partial maxima (float bit patterns).  Each tensor that

@@ -264,6 +264,39 @@ __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __re
     }
 }
 
+// ---- unpack + dequantize (symmetric codes) ------------------------------------------------------
+// Inverse of the symmetric pack: tools/convert_kimi_int4_to_bf16.py:57-86 unpacks nibble i of word j into
+// element 8j+i, subtracts the offset 8 (compressed-tensors' unpack_from_int32), multiplies by the group's scale
+// in fp32 and rounds to bf16.  The product of a 4-bit integer and a bf16/fp16 scale is exact in fp32, so the only
+// rounding is the final one.
+template <int SDT>
+__global__ __launch_bounds__(256) void int4_unpack_kernel(const uint32_t* __restrict__ packed,
+                                                          const void* __restrict__ scale, uint16_t* __restrict__ y,
+                                                          int64_t words, int group_shift) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= words) return;
+    const uint32_t word = __builtin_nontemporal_load(packed + i);
+    const float s = load_f32(scale, i >> group_shift, SDT);
+    float f[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) f[k] = (float)((int)((word >> (4 * k)) & 0xFu) - 8) * s;
+    st16(y + i * 8, u32x4{hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])});
+}
+// any K (rows padded to whole words), any group size, any scale dtype: one lane per element
+__global__ __launch_bounds__(256) void int4_unpack_generic_kernel(const uint32_t* __restrict__ packed,
+                                                                  const void* __restrict__ scale, int sdt,
+                                                                  uint16_t* __restrict__ y, int64_t M, int64_t K,
+                                                                  int G) {
+    const int64_t wpr = (K + 7) / 8, gpr = K / G, total = M * K;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / K, c = i - r * K;
+        const uint32_t word = packed[r * wpr + c / 8];
+        const float v = (float)((int)((word >> (4 * (c & 7))) & 0xFu) - 8) * load_f32(scale, r * gpr + c / G, sdt);
+        y[i] = (uint16_t)f32_to_bf16_bits(v);
+    }
+}
+
 }  // namespace mq
 
 using namespace mq;
@@ -344,4 +377,33 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     if (zblocks > mq_grid_cap()) zblocks = mq_grid_cap();
     hipLaunchKernelGGL(int4_zero_pack_kernel, dim3((unsigned)zblocks), dim3(256), 0, st, zero, (uint32_t*)packed_zp, M, gpr);
     return mq_check_launch("int4 zero-point pack");
+}
+
+extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M,
+                                      int64_t K, int group, void* stream) {
+    if (!packed || !scale || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (scale_dtype < MQ_BF16 || scale_dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (K % group != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size");
+    if (M == 0 || K == 0) return MQ_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int upg = group / 8;
+    if (K % 8 == 0 && group % 8 == 0 && (upg & (upg - 1)) == 0 && ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0) {
+        int shift = 0;
+        while ((1 << shift) < upg) shift++;
+        const int64_t words = M * (K / 8), blocks = (words + 255) / 256;
+        if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+        const dim3 grid((unsigned)blocks), blk(256);
+        if (scale_dtype == MQ_BF16)
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_BF16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+        else if (scale_dtype == MQ_F16)
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+        else
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F32>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+        return mq_check_launch("int4 unpack");
+    }
+    int64_t blocks = (M * K + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    hipLaunchKernelGGL(int4_unpack_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)packed, scale,
+                       scale_dtype, (uint16_t*)y, M, K, group);
+    return mq_check_launch("int4 unpack");
 }

@@ -533,6 +533,21 @@ void mqo_int4_pack_layer_asym(const void* w, int dtype, int64_t M, int64_t K, in
     free(zero);
 }
 
+/* _dequantize_tensor (tools/convert_kimi_int4_to_bf16.py:57-86): compressed-tensors' unpack_from_int32 (third
+ * party, not in the reference tree; its published algorithm: element 8j+i = ((word_j >> 4i) & 15) - 8, rows
+ * cropped to K) followed by bf16(f32(value) * f32(scale)) with one scale per G columns. */
+void mqo_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, int64_t M, int64_t K, int G,
+                             uint16_t* y) {
+    int64_t wpr = (K + 7) / 8, gpr = K / G;
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t c = 0; c < K; c++) {
+            uint32_t word = (uint32_t)packed[r * wpr + c / 8];
+            float v = (float)((int)((word >> (4 * (c & 7))) & 0xFu) - 8);
+            y[r * K + c] = f32_to_bf16(v * load_as_f32(scale, r * gpr + c / G, scale_dtype));
+        }
+}
+
 /* ------------------------------------------------------------------ */
 /* A-4  NVFP4 (miles/utils/nvfp4.py:19-134; block arithmetic restated   */
 /*      from miles/kernels/quant/nvfp4_qdq.py:716-743,859-889,1079-1081)*/

@@ -65,6 +65,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_mxfp8.argtypes = [vp, i32, i64, i64, vp, vp]
         L.mqo_int4_fake_quant.restype = None
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
+        L.mqo_int4_unpack_dequant.restype = None
+        L.mqo_int4_unpack_dequant.argtypes = [vp, vp, i32, i64, i64, i32, vp]
         L.mqo_mxfp4_quant.restype = None
         L.mqo_mxfp4_quant.argtypes = [vp, i32, i64, i32, vp, vp]
         L.mqo_mxfp4_dequant.restype = None
@@ -217,6 +219,18 @@ def pack_layer(weight: torch.Tensor, group_size: int, sym: bool = True):
     lib().mqo_int4_pack_layer(weight.data_ptr(), _DTYPE[weight.dtype], M, K, int(group_size),
                               packed.data_ptr(), scale.data_ptr())
     return packed, scale, None
+
+
+def int4_unpack_dequant(weight_packed: torch.Tensor, weight_scale: torch.Tensor, weight_shape, group_size: int):
+    """tools/convert_kimi_int4_to_bf16.py:57-86 -> bfloat16 [M, K]."""
+    assert weight_packed.device.type == "cpu" and weight_packed.dtype == torch.int32
+    _check_cpu(weight_scale)
+    M, K = (int(v) for v in (weight_shape.view(-1).tolist() if isinstance(weight_shape, torch.Tensor) else weight_shape))
+    p, s = weight_packed.contiguous(), weight_scale.contiguous()
+    assert p.shape == (M, -(-K // 8)) and K % group_size == 0 and s.numel() == M * (K // group_size)
+    out = torch.empty((M, K), dtype=torch.bfloat16)
+    lib().mqo_int4_unpack_dequant(p.data_ptr(), s.data_ptr(), _DTYPE[s.dtype], M, K, int(group_size), out.data_ptr())
+    return out
 
 
 # --------------------------------------------------------------------------

@@ -216,3 +216,67 @@ def test_convert_int4_direct(oracle, tmp_path):
             _same(got[k], w, k)
     cfg = json.loads((out / "config.json").read_text())["quantization_config"]
     assert cfg["format"] == "pack-quantized" and cfg["config_groups"]["group_0"]["weights"]["group_size"] == 32
+
+
+def test_convert_kimi_int4_to_bf16(tmp_path, oracle):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools import convert_kimi_int4_to_bf16 as tool
+
+    cfg = {"text_config": {"hidden_size": 256, "moe_intermediate_size": 128,
+                           "quantization_config": {"config_groups": {"group_0": {"weights": {"group_size": 32}}}}}}
+    shard = {"model.embed_tokens.weight": _rand((64, 256), 1)}
+    originals = {}
+    for e in range(2):
+        for proj, shape in (("gate_proj", (128, 256)), ("up_proj", (128, 256)), ("down_proj", (256, 128))):
+            w = _rand(shape, 40 + 3 * e + len(proj))
+            packed, scale, _ = pack_layer(w.cuda(), 32)
+            base = f"model.layers.0.mlp.experts.{e}.{proj}"
+            shard[f"{base}.weight_packed"] = packed.cpu()
+            shard[f"{base}.weight_scale"] = scale.cpu()
+            shard[f"{base}.weight_shape"] = torch.tensor(shape, dtype=torch.int32)
+            originals[base] = (packed.cpu(), scale.cpu(), shape)
+    # an incomplete triple and a shared expert stay as they are
+    shard["model.layers.0.mlp.experts.9.up_proj.weight_packed"] = torch.zeros((4, 4), dtype=torch.int32)
+    shard["model.layers.0.mlp.shared_experts.up_proj.weight_packed"] = torch.ones((4, 4), dtype=torch.int32)
+    model = _checkpoint(tmp_path, [shard], cfg)
+    out = tmp_path / "bf16"
+    tool.main(["--model-dir", str(model), "--output-dir", str(out)])
+    got = _load_all(out)
+    for base, (packed, scale, shape) in originals.items():
+        want = oracle.int4_unpack_dequant(packed, scale.float(), shape, 32)
+        _same(got[f"{base}.weight"], want, base)
+        assert f"{base}.weight_packed" not in got and f"{base}.weight_scale" not in got
+    assert "model.layers.0.mlp.experts.9.up_proj.weight_packed" in got
+    assert "model.layers.0.mlp.shared_experts.up_proj.weight_packed" in got
+    _same(got["model.embed_tokens.weight"], shard["model.embed_tokens.weight"], "embed")
+    index = json.loads((out / "model.safetensors.index.json").read_text())
+    assert set(index["weight_map"]) == set(got) and (out / "tokenizer.json").exists()
+
+
+def test_convert_mxfp4_to_bf16(tmp_path, oracle):
+    from miles_amd.tools import convert_mxfp4_to_bf16 as tool
+
+    cfg = {"num_hidden_layers": 1,
+           "quantization_config": {"format": "mxfp4-pack-quantized",
+                                   "config_groups": {"group_0": {"weights": {"group_size": 32, "type": "float", "num_bits": 4,
+                                                                             "scale_dtype": "torch.uint8"}}}}}
+    g = torch.Generator().manual_seed(5)
+    shards = []
+    for i in range(2):
+        shards.append({f"model.layers.0.mlp.experts.{i}.w1.weight_packed": torch.randint(0, 256, (64, 128), dtype=torch.uint8, generator=g),
+                       f"model.layers.0.mlp.experts.{i}.w1.weight_scale": torch.randint(100, 140, (64, 8), dtype=torch.uint8, generator=g),
+                       f"model.layers.0.norm{i}.weight": _rand((256,), 60 + i)})
+    model = _checkpoint(tmp_path, shards, cfg)
+    out = tmp_path / "bf16"
+    tool.main(["--model-dir", str(model), "--save-dir", str(out)])
+    got = _load_all(out)
+    for i, shard in enumerate(shards):
+        base = f"model.layers.0.mlp.experts.{i}.w1"
+        want = oracle.dequantize_mxfp4(shard[f"{base}.weight_packed"], shard[f"{base}.weight_scale"], 32)
+        _same(got[f"{base}.weight"], want, base)
+        assert f"{base}.weight_packed" not in got and f"{base}.weight_scale" not in got
+        _same(got[f"model.layers.0.norm{i}.weight"], shard[f"model.layers.0.norm{i}.weight"], "norm")
+    assert "quantization_config" not in json.loads((out / "config.json").read_text())
+    index = json.loads((out / "model.safetensors.index.json").read_text())
+    assert set(index["weight_map"]) == set(got)
+    assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for t in got.values())

@@ -298,6 +298,37 @@ def test_int4_pack_layer_asymmetric_argument_checks():
         pack_layer(torch.zeros(8, 96, dtype=torch.bfloat16, device=DEV), 128, sym=False)
 
 
+@pytest.mark.parametrize("sdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 32), ((3, 100), 20), ((64, 1024), 128),
+                                     ((2048, 7168), 128)])
+def test_int4_unpack_dequant(oracle, shape, G, sdt):
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+
+    if shape[0] > 1000 and sdt != torch.bfloat16:
+        pytest.skip("the full-size tensor is checked with bf16 scales only")
+    g = torch.Generator().manual_seed(31)
+    m, k = shape
+    packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
+    scale = torch.exp(torch.randn((m, k // G), generator=g) * 3).to(sdt)
+    got = _dequantize_tensor(packed.to(DEV), scale.to(DEV), torch.tensor(shape, dtype=torch.int32), G)
+    want = oracle.int4_unpack_dequant(packed, scale, shape, G)
+    assert got.dtype == torch.bfloat16
+    _assert_same(got, want, "dequantized values")
+
+
+def test_int4_pack_then_unpack_round_trip(oracle):
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+
+    w = W.gaussian_outliers((256, 7168), std=0.015, p_outlier=0.0005, gain=30.0, seed=4001)
+    packed, scale, _ = pack_layer(w.to(DEV), 128)
+    deq = _dequantize_tensor(packed, scale, w.shape, 128)
+    # |w - dequantized| <= scale/2 plus the bf16 roundings of the scale and of the product (each <= 7*scale*2^-9, measured against the rounded scale)
+    err = (deq.float().cpu() - w.float()).abs().reshape(256, 56, 128).amax(dim=-1)
+    assert torch.all(err <= scale.float().cpu() * 0.55 + 1e-12)
+    _assert_same(deq, oracle.int4_unpack_dequant(packed.cpu(), scale.cpu(), w.shape, 128), "round trip")
+
+
 @pytest.mark.parametrize("sym", [True, False])
 @pytest.mark.parametrize("shape,G", [((16, 256), 128), ((8, 200), 32), ((4, 128), 32), ((3, 7168), 128)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

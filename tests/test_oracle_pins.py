@@ -407,6 +407,40 @@ def test_int4_asym_known_answers(oracle):
     # rows 0..7 carry zero points 0,15,7,0,0,0,0,0 in nibbles 0,4,1,5,2,6,3,7
     assert (pzp[0, 0].item() & 0xFFFFFFFF) == (0 << 0) | (15 << 16) | (7 << 4)
 
+def torch_int4_dequantize_tensor(weight_packed, weight_scale, shape, group_size):
+    """tools/convert_kimi_int4_to_bf16.py:57-86 with compressed-tensors' unpack_from_int32 written out
+    (published algorithm: nibble i of word j -> element 8j+i, crop to the original width, subtract 8)."""
+    m, k = shape
+    unpacked = torch.zeros((weight_packed.shape[0], weight_packed.shape[1] * 8), dtype=torch.int32)
+    for i in range(8):
+        unpacked[:, i::8] = (weight_packed >> (4 * i)) & 0xF
+    weight = (unpacked[:, :k] - 8).to(torch.int8)
+    scales = torch.repeat_interleave(weight_scale.to(torch.float32), repeats=group_size, dim=1)
+    return (weight.to(torch.float32) * scales).to(torch.bfloat16).contiguous()
+
+
+@pytest.mark.parametrize("sdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 32), ((3, 100), 20), ((64, 1024), 128)])
+def test_int4_unpack_dequant_matches_torch_chain(oracle, shape, G, sdt):
+    g = torch.Generator().manual_seed(31)
+    m, k = shape
+    packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
+    scale = torch.exp(torch.randn((m, k // G), generator=g) * 3).to(sdt)
+    got = oracle.int4_unpack_dequant(packed, scale, shape, G)
+    want = torch_int4_dequantize_tensor(packed, scale, shape, G)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_int4_unpack_inverts_pack_layer(oracle):
+    # pack_layer followed by the unpacker gives q * scale in bf16 for every element (symmetric codes 1..15)
+    w = W.gaussian_outliers((16, 512), std=0.015, p_outlier=0.0005, gain=30.0, seed=4001)
+    packed, scale, _ = oracle.pack_layer(w, 128)
+    out, fscale, _ = oracle.fake_int4_quant(w, (1, 128), True)
+    deq = oracle.int4_unpack_dequant(packed, scale, w.shape, 128)
+    want = (out.float().reshape(16, 4, 128) * scale.float().unsqueeze(-1)).reshape(16, 512).to(torch.bfloat16)
+    assert torch.equal(deq.view(torch.int16), (want + 0.0).view(torch.int16))   # -0 * s: the unpacker has no -0 codes
+
+
 def test_int4_constant_rows_known_answer(oracle):
     for c in (0.5, 0.013, 3.0):
         w = torch.full((2, 128), c, dtype=torch.bfloat16)
