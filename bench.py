@@ -33,7 +33,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 + 2, "mxfp8": 2 + 1 + 1 / 32,
-                  "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16}
+                  "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16,
+                  # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
+                  "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
+                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0003 B per element)
 MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0005
@@ -148,6 +151,45 @@ def per_quantizer(gen):
     del experts
     run("C5b_fp8_dequant", "fp8_dequant", n, lambda: [weight_dequant(q, s) for q, s in quantized],
         "32 experts, FP8 block -> bf16")
+    del quantized
+    res.update(adjacent_formats(gen))
+    return res
+
+
+def adjacent_formats(gen):
+    """GB/s of the kernels either side of the path (MXFP4 pack / unpack, INT4 unpack, asymmetric INT4 pack).
+    The unpackers and the asymmetric packer are single-tensor entry points, so they are timed as direct calls on
+    eight [16384, 7168] tensors: long enough launches that the GPU, not the host, sets the pace."""
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+
+    res = {}
+    shape, count = (16384, 7168), 8
+    elems = count * shape[0] * shape[1]
+    ws = [_synth(shape, gen, std=0.015, p=0.0005, gain=30.0) for _ in range(count)]
+
+    def run(name, key, fn, note):
+        fn()
+        torch.cuda.synchronize()
+        ms = _event_ms(fn, 5)
+        gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
+        res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+                     "elements": elems, "workload": note}
+
+    batch, m4 = _record(lambda: [quantize_mxfp4(w, 32) for w in ws])
+    ms = _event_ms(batch.run, 5)
+    gbps = elems * BYTES_PER_ELEM["mxfp4"] / ms / 1e6
+    res["next_mxfp4_quant"] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+                               "elements": elems, "workload": "8 x [16384,7168] bf16, group 32, one grouped launch"}
+    del batch
+    run("next_mxfp4_dequant", "mxfp4_dequant", lambda: [dequantize_mxfp4(p, s, 32) for p, s in m4], "MXFP4 -> bf16")
+    del m4
+    i4 = [pack_layer(w, 128) for w in ws]
+    run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")
+    del i4
+    run("next_int4_g128_asym_pack", "int4_g128_asym", lambda: [pack_layer(w, 128, sym=False) for w in ws],
+        "pack_layer(sym=False), group 128")
     return res
 
 

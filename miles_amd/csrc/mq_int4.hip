@@ -246,6 +246,105 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restr
     }
 }
 
+// bf16 fast path of the asymmetric packer: LANES lanes own one group (16 bytes each, G = 8 * LANES), the data
+// stays in registers between the min/max pass and the coding pass, min and max travel through the unsigned
+// DPP reduction as order-preserving integer keys, and every rounding to bf16 is the packed hardware conversion.
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = f2u(f);
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float order_unkey(uint32_t k) {
+    return u2f(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
+}
+__device__ __forceinline__ void rd_bf16x2(float& a, float& b) {
+    const uint32_t p = hw_bf16x2(a, b);
+    a = bf16_lo(p);
+    b = bf16_hi(p);
+}
+// one 16-byte unit of one lane; LANES neighbouring lanes hold the rest of the group
+template <int LANES>
+__device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, const int64_t unit, const int t,
+                                               uint32_t* __restrict__ packed, uint16_t* __restrict__ scale_out,
+                                               uint8_t* __restrict__ zero_out) {
+    float f[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+    float mx = f[0], mn = f[0];
+#pragma unroll
+    for (int i = 1; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
+    mx = order_unkey(seg_max<LANES>(order_key(mx)));
+    mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
+    const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
+    const float sb = u2f(sw_bf16(s) << 16);
+    const float ys = 1.0f / s;
+    const float big = __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
+    const bool fast = shared_div_ok(s) && big * ys < 1e30f;
+    const float lo = __builtin_rintf(fast ? div_by_shared(mn, s, ys) : mn / s);
+    const float hi = __builtin_rintf(fast ? div_by_shared(mx, s, ys) : mx / s);
+    const float z = __builtin_fminf(__builtin_fmaxf(-lo, 0.0f), 15.0f) + 0.0f;
+    uint32_t word = 0;
+    if (fast && lo <= 0.0f && lo >= -15.0f && hi - lo <= 16.0f && sb <= 1e37f) {
+        // The zero point was not clamped, so rint(x/s) + z is an integer in [0, 16].  For such codes and every
+        // bf16 scale up to 1e37 the reference's dequantize / requantize round trip in bf16 returns the code itself
+        // (checked exhaustively on the CPU: all scales x all codes x all zero points), so the codes are final.
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            word += (uint32_t)(__builtin_rintf(div_by_shared(f[i], s, ys)) + z) << (4 * i);
+    } else {
+        // the chain as written, IEEE divisions: groups whose minimum lies above zero or far below it, huge scales
+        float q[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s) + z;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = q[i] - z;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = q[i] * sb;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = q[i] / sb;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = q[i] + z;
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            word += (uint32_t)__builtin_rintf(__builtin_fminf(__builtin_fmaxf(q[i], 0.0f), 255.0f)) << (4 * i);
+    }
+    if (live) {
+        st4(packed + unit, word);
+        if ((t & (LANES - 1)) == 0) {
+            scale_out[unit / LANES] = (uint16_t)sw_bf16(s);
+            zero_out[unit / LANES] = (uint8_t)z;
+        }
+    }
+}
+template <int LANES>
+__global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const uint16_t* __restrict__ w,
+                                                                         uint32_t* __restrict__ packed,
+                                                                         uint16_t* __restrict__ scale_out,
+                                                                         uint8_t* __restrict__ zero_out,
+                                                                         int64_t total_units) {
+    const int t = threadIdx.x;
+    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll) + t;
+    // a group is a whole number of lanes, so dead lanes never share one with live lanes; they re-read the last unit
+    u32x4 v[kI4Unroll];
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads;
+        v[i] = ld16(w + (unit < total_units ? unit : total_units - 1) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads;
+        int4_asym_unit<LANES>(v[i], unit < total_units, unit, t, packed, scale_out, zero_out);
+    }
+}
+
 // packed_zp[g, j] = sum_i zero[8j+i, g] << 4*order[i], order = {0,4,1,5,2,6,3,7}   (py:249-254)
 __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
                                                              uint32_t* __restrict__ packed_zp, int64_t M,
@@ -269,18 +368,41 @@ __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __re
 // element 8j+i, subtracts the offset 8 (compressed-tensors' unpack_from_int32), multiplies by the group's scale
 // in fp32 and rounds to bf16.  The product of a 4-bit integer and a bf16/fp16 scale is exact in fp32, so the only
 // rounding is the final one.
+#ifndef MQ_I4_UNPACK_UNROLL
+#define MQ_I4_UNPACK_UNROLL 2
+#endif
+constexpr int kI4UnpackUnroll = MQ_I4_UNPACK_UNROLL;   // words per lane, 256 lanes apart so every load and store instruction stays contiguous
 template <int SDT>
 __global__ __launch_bounds__(256) void int4_unpack_kernel(const uint32_t* __restrict__ packed,
                                                           const void* __restrict__ scale, uint16_t* __restrict__ y,
                                                           int64_t words, int group_shift) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= words) return;
-    const uint32_t word = __builtin_nontemporal_load(packed + i);
-    const float s = load_f32(scale, i >> group_shift, SDT);
-    float f[8];
+    const int64_t base = (int64_t)blockIdx.x * (256 * kI4UnpackUnroll) + threadIdx.x;
+    uint32_t word[kI4UnpackUnroll], sraw[kI4UnpackUnroll];
+    // every load is issued before the first use: lanes past the end re-read the last word instead of branching
 #pragma unroll
-    for (int k = 0; k < 8; k++) f[k] = (float)((int)((word >> (4 * k)) & 0xFu) - 8) * s;
-    st16(y + i * 8, u32x4{hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])});
+    for (int u = 0; u < kI4UnpackUnroll; u++) {
+        const int64_t i = base + u * 256 < words ? base + u * 256 : words - 1;
+        word[u] = __builtin_nontemporal_load(packed + i);
+        if (SDT == MQ_F32) sraw[u] = ((const uint32_t*)scale)[i >> group_shift];
+        else sraw[u] = ((const uint16_t*)scale)[i >> group_shift];
+    }
+#pragma unroll
+    for (int u = 0; u < kI4UnpackUnroll; u++) {
+        const int64_t i = base + u * 256;
+        float s[kI4UnpackUnroll];
+        s[u] = SDT == MQ_F32 ? u2f(sraw[u]) : SDT == MQ_BF16 ? u2f(sraw[u] << 16)
+                                                             : (float)__builtin_bit_cast(_Float16, (uint16_t)sraw[u]);
+        // even nibbles and odd nibbles as bytes: one byte-to-float conversion each
+        const uint32_t ev = word[u] & 0x0F0F0F0Fu, od = (word[u] >> 4) & 0x0F0F0F0Fu;
+        float f[8];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            f[2 * k] = ((float)((ev >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
+            f[2 * k + 1] = ((float)((od >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
+        }
+        if (i < words)
+            st16(y + i * 8, u32x4{hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])});
+    }
 }
 // any K (rows padded to whole words), any group size, any scale dtype: one lane per element
 __global__ __launch_bounds__(256) void int4_unpack_generic_kernel(const uint32_t* __restrict__ packed,
@@ -364,7 +486,17 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     int64_t blocks = (groups + 15) / 16;
     if (blocks > mq_grid_cap() * 4) blocks = mq_grid_cap() * 4;
     const int wpg = group / 8;
-    if (dtype == MQ_BF16)
+    if (dtype == MQ_BF16 && (group == 128 || group == 64 || group == 32)) {
+        const int64_t units = M * (K / 8), fblocks = (units + kI4Threads * kI4Unroll - 1) / (kI4Threads * kI4Unroll);
+        if (fblocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+        const dim3 grid((unsigned)fblocks), blk(kI4Threads);
+        if (group == 128)
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+        else if (group == 64)
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+        else
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+    } else if (dtype == MQ_BF16)
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
     else if (dtype == MQ_F16)
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
@@ -390,7 +522,7 @@ extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, 
     if (K % 8 == 0 && group % 8 == 0 && (upg & (upg - 1)) == 0 && ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0) {
         int shift = 0;
         while ((1 << shift) < upg) shift++;
-        const int64_t words = M * (K / 8), blocks = (words + 255) / 256;
+        const int64_t words = M * (K / 8), blocks = (words + 256 * kI4UnpackUnroll - 1) / (256 * kI4UnpackUnroll);
         if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
         const dim3 grid((unsigned)blocks), blk(256);
         if (scale_dtype == MQ_BF16)

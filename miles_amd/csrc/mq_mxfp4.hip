@@ -39,6 +39,25 @@ __device__ __forceinline__ uint32_t mxfp4_code(float x, float mult) {
     return mag | ((f2u(x) >> 31) << 3);
 }
 
+// Scale byte straight from the bf16 pattern of the group amax: amax = m * 2^(E-127), so amax / 6 lies in
+// (2^(E-130), 2^(E-129)] for m <= 1.5 and in (2^(E-129), 2^(E-128)) above, i.e. byte = E - 2 + (m > 1.5), floored at
+// 0 (covers zero and subnormal amax) and 254 for inf.  Identical to mxfp4_scale_byte(amax / 6.0f) for every bf16
+// pattern; no division.
+__device__ __forceinline__ uint32_t mxfp4_scale_byte_bf16(uint32_t amax_bits) {
+    const int e = (int)(amax_bits >> 7), gt = (amax_bits & 0x7Fu) > 0x40u;
+    if (e == 255) return 254u;
+    const int b = e - 2 + gt;
+    return b < 0 ? 0u : (uint32_t)b;
+}
+// The reference's thresholds send a value that sits exactly on a bound to the smaller magnitude, the hardware
+// conversion rounds ties to even.  Stepping the magnitude down by one fp32 ulp first makes the two agree: a value
+// on a bound lands just below it, and a scaled bf16 value (8 significant bits) can never be the fp32 neighbour just
+// above a bound, so nothing else moves across one.  Zero keeps its pattern (and its sign).
+__device__ __forceinline__ float step_toward_zero(float n) {
+    const uint32_t u = f2u(n);
+    return u2f(u - ((u & 0x7FFFFFFFu) != 0));
+}
+
 __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const FlatTable tab) {
     const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
@@ -59,13 +78,23 @@ __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const FlatTable 
         const int64_t unit = base + i * kM4Threads + t;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max4(hmax_u16(m2));
-        const uint32_t byte = mxfp4_scale_byte(u2f(mb << 16) / 6.0f);
+        const uint32_t byte = mxfp4_scale_byte_bf16(mb);
         const float mult = mxfp4_normalizer(byte);
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         uint32_t word = 0;
+        if (mb < 0x7F80u) {
+            float n[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) word |= mxfp4_code(f[j], mult) << (4 * j);
+            for (int j = 0; j < 8; j++) n[j] = step_toward_zero(f[j] * mult);
+            word = hw_e2m1x2<0>(n[0], n[1], word);
+            word = hw_e2m1x2<1>(n[2], n[3], word);
+            word = hw_e2m1x2<2>(n[4], n[5], word);
+            word = hw_e2m1x2<3>(n[6], n[7], word);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) word |= mxfp4_code(f[j], mult) << (4 * j);
+        }
         if (unit < total_units) {
             st4(packed + unit, word);
             if ((t & 3) == 0) scale[unit >> 2] = (uint8_t)byte;
@@ -112,19 +141,43 @@ __device__ __forceinline__ uint32_t mxfp4_decode(uint32_t code, uint32_t s) {
     return sign | (f2u(v) >> 16);
 }
 
-// flat: one lane per 4 packed bytes (8 codes -> 16 bytes of bf16); G = 8 << group_shift
+// flat: one lane per 4 packed bytes (8 codes -> 16 bytes of bf16), kM4DqUnroll such units per lane; G = 8 << group_shift.
+// Scale bytes 2..252 keep every product a normal, finite bf16 number: there the packed hardware conversion
+// (two codes per instruction, scaled by 2^(s-127)) is used; the few bytes outside that range take the software form.
+constexpr int kM4DqUnroll = 2;
+typedef __bf16 hw_bf16x2_t __attribute__((ext_vector_type(2)));
+template <int BYTE>
+__device__ __forceinline__ uint32_t hw_e2m1x2_to_bf16x2(uint32_t word, float factor) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, factor, BYTE));
+}
 __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint32_t* __restrict__ packed,
                                                             const uint8_t* __restrict__ scale,
                                                             uint16_t* __restrict__ y, int64_t units,
                                                             int group_shift) {
-    const int64_t unit = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (unit >= units) return;
-    const uint32_t word = __builtin_nontemporal_load(packed + unit);
-    const uint32_t s = scale[unit >> group_shift];
-    uint32_t c[8];
+    const int64_t base = (int64_t)blockIdx.x * (256 * kM4DqUnroll) + threadIdx.x;
+    uint32_t word[kM4DqUnroll], s[kM4DqUnroll];
 #pragma unroll
-    for (int j = 0; j < 8; j++) c[j] = mxfp4_decode((word >> (4 * j)) & 0xFu, s);
-    st16(y + unit * 8, u32x4{c[0] | (c[1] << 16), c[2] | (c[3] << 16), c[4] | (c[5] << 16), c[6] | (c[7] << 16)});
+    for (int i = 0; i < kM4DqUnroll; i++) {
+        const int64_t unit = base + i * 256 < units ? base + i * 256 : units - 1;   // past the end: re-read the last unit
+        word[i] = __builtin_nontemporal_load(packed + unit);
+        s[i] = scale[unit >> group_shift];
+    }
+#pragma unroll
+    for (int i = 0; i < kM4DqUnroll; i++) {
+        const int64_t unit = base + i * 256;
+        u32x4 o;
+        if (s[i] >= 2u && s[i] <= 252u) {
+            const float factor = u2f(s[i] << 23);
+            o = u32x4{hw_e2m1x2_to_bf16x2<0>(word[i], factor), hw_e2m1x2_to_bf16x2<1>(word[i], factor),
+                      hw_e2m1x2_to_bf16x2<2>(word[i], factor), hw_e2m1x2_to_bf16x2<3>(word[i], factor)};
+        } else {
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) c[j] = mxfp4_decode((word[i] >> (4 * j)) & 0xFu, s[i]);
+            o = u32x4{c[0] | (c[1] << 16), c[2] | (c[3] << 16), c[4] | (c[5] << 16), c[6] | (c[7] << 16)};
+        }
+        if (unit < units) st16(y + unit * 8, o);
+    }
 }
 __global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_t* __restrict__ packed,
                                                                     const uint8_t* __restrict__ scale,
@@ -190,7 +243,7 @@ extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, voi
         int shift = 0;
         while ((1 << shift) < upg) shift++;
         const int64_t units = bytes / 4;
-        const int64_t blocks = (units + 255) / 256;
+        const int64_t blocks = (units + 256 * kM4DqUnroll - 1) / (256 * kM4DqUnroll);
         if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
         hipLaunchKernelGGL(mxfp4_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)packed, scale,
                            (uint16_t*)y, units, shift);

@@ -344,6 +344,13 @@ def test_mxfp4_scale_exponent_from_bits_equals_float_log2_for_16_bit_inputs():
         e, m = u >> 23, u & 0x7FFFFF
         got = torch.where(e == 0, (m > 0x400000).to(torch.int32), torch.clamp(e + (m != 0).to(torch.int32), max=254))
         assert torch.equal(got, want.to(torch.int32))
+    # bf16 fast path: the same byte read straight off the amax pattern, byte = E - 2 + (mantissa > 1.5), no division
+    bits = torch.arange(0, 0x7F81, dtype=torch.int32)           # every finite bf16 magnitude and +inf
+    q = bits.to(torch.int16).view(torch.bfloat16).float() / 6.0
+    want = torch.ceil(torch.log2(q)).clamp_(-127, 127) + 127
+    e, gt = bits >> 7, ((bits & 0x7F) > 0x40).to(torch.int32)
+    got = torch.where(e == 255, torch.full_like(e, 254), torch.clamp(e - 2 + gt, min=0))
+    assert torch.equal(got, want.to(torch.int32))
 
 
 # ----------------------------------------------------------------------------------------------
@@ -439,6 +446,22 @@ def test_int4_unpack_inverts_pack_layer(oracle):
     deq = oracle.int4_unpack_dequant(packed, scale, w.shape, 128)
     want = (out.float().reshape(16, 4, 128) * scale.float().unsqueeze(-1)).reshape(16, 512).to(torch.bfloat16)
     assert torch.equal(deq.view(torch.int16), (want + 0.0).view(torch.int16))   # -0 * s: the unpacker has no -0 codes
+
+
+def test_int4_asym_round_trip_is_identity_for_unclamped_codes():
+    # The bf16 fast path of the asymmetric packer emits rint(x/s) + z directly when the zero point was not clamped
+    # (codes in [0, 16]) and the bf16 scale is at most 1e37.  Exhaustive over every such scale, code and zero point:
+    # the reference's chain  bf16((w1 - z) * s) / s + z -> clamp -> round  returns w1.
+    bits = torch.arange(1, 0x7F80, dtype=torch.int32).to(torch.int16)
+    sb = bits.view(torch.bfloat16)
+    sb = sb[(sb.float() >= 9.9e-6) & (sb.float() <= 1e37)]
+    for z in range(16):
+        zt = torch.tensor(float(z), dtype=torch.bfloat16)
+        for w1 in range(17):
+            w = torch.tensor(float(w1), dtype=torch.bfloat16)
+            r = ((w - zt) * sb) / sb + zt
+            code = torch.round(torch.clamp(r, 0, 255)).to(torch.uint8)
+            assert torch.all(code == w1), (z, w1)
 
 
 def test_int4_constant_rows_known_answer(oracle):
