@@ -193,6 +193,39 @@ def adjacent_formats(gen):
     return res
 
 
+def packed_payload(args, weights, fp8_cfg, steps):
+    """The same sync producing the flattened transport payload of every bucket (the reference's broadcast_packed
+    mode).  `in_place_ms`: quantizers write into the payload, only pass-through tensors are copied.
+    `flatten_after_ms`: the reference's order of work -- quantize, then copy every tensor of the bucket into the
+    payload -- with this library's own grouped copy kernel."""
+    from miles_amd.weight_update.packed_bucket import pack_bucket
+    from miles_amd.weight_update.updater import WeightUpdater
+
+    def timed(updater):
+        updater.update_weights()
+        updater.update_weights()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            updater.update_weights()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    seen = {"bytes": 0}
+    in_place = WeightUpdater(args, weights_getter=lambda: weights, model_name="qwen3", quantization_config=fp8_cfg,
+                             send_bucket=lambda b: seen.__setitem__("bytes", seen["bytes"] + b.flat.numel()),
+                             packed_buckets=True)
+    ms_in_place = timed(in_place)
+    assert in_place._plan is not None and in_place._plan.replayable
+    payload_bytes = seen["bytes"] // (steps + 2)
+    del in_place
+    after = WeightUpdater(args, weights_getter=lambda: weights, model_name="qwen3", quantization_config=fp8_cfg,
+                          send_bucket=pack_bucket)
+    ms_after = timed(after)
+    return {"in_place_ms": round(ms_in_place, 4), "flatten_after_ms": round(ms_after, 4), "payload_bytes": payload_bytes,
+            "note": "one sync = quantize + build every bucket's flat payload (embeddings and norms included)"}
+
+
 def roofline(plan, jobs_meta):
     """Time every kernel launch of one sync (same launch partition as a step) with events on the launch stream."""
     spans = []
@@ -348,6 +381,7 @@ def main():
         line["cpu_baseline"] = cpu_baseline(weights, args)
     if not a.no_extras:
         del updater, plan
+        line["packed_payload"] = packed_payload(args, weights, fp8_cfg, a.steps)
         weights.clear()
         line["per_quantizer"] = per_quantizer(gen)
     print(json.dumps(line))

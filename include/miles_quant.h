@@ -135,8 +135,11 @@ int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections,
  *   MQ_JOB_MXFP8                w             e4m3          E8M0 bytes     -                           -
  *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
  *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, -
- *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *                                                                          aux2 = fp32 weight_scale_2
+ *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
+ *   MQ_JOB_COPY                 bytes         bytes         -              -                           -
+ *     (rows * cols bytes copied verbatim: how a pass-through tensor reaches its place in a packed transport bucket,
+ *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
@@ -148,7 +151,8 @@ enum {
     MQ_JOB_MXFP8 = 3,
     MQ_JOB_INT4_PACK = 4,
     MQ_JOB_NVFP4 = 5,
-    MQ_JOB_MXFP4 = 6
+    MQ_JOB_MXFP4 = 6,
+    MQ_JOB_COPY = 7
 };
 typedef struct mq_job {
     int32_t kind;

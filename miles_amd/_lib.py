@@ -40,7 +40,8 @@ SIGNATURES = {
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 
-(JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4) = range(7)
+(JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
+ JOB_COPY) = range(8)
 
 
 class Job(_c.Structure):

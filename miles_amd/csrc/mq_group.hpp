@@ -70,6 +70,18 @@ inline bool flat_grid(FlatTable& tab, int64_t per_block) {
     return mx < 0x7FFFFFF0;
 }
 
+struct CopyJob {      // one run of bytes
+    const uint8_t* src;
+    uint8_t* dst;
+    int64_t bytes;
+};
+struct CopyTable {
+    int32_t n;
+    int32_t total;            // all chunks of the launch
+    int32_t end[kMaxGroup];   // running chunk counts, as in TileTable
+    CopyJob job[kMaxGroup];
+};
+
 // Index of the tensor that owns work item `item`: the number of running counts not above it.  The loop has
 // a fixed trip count and no early exit, so the compiler fetches the whole `end` array with a few wide scalar
 // loads and the comparison chain runs on the scalar unit: a short, latency-free prologue even for

@@ -27,6 +27,8 @@ int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
+int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
+int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
 // Upper bound on the input bytes of one NVFP4 group (amax launch + fold + quantize launch).  Measured on
 // MI355X the second read of a tensor gains nothing from the memory-side cache at any group size, so groups
@@ -52,15 +54,18 @@ static bool job_fast(const mq_job& j) {
             return mq_nvfp4_fast_ok(j.in, j.dtype, j.out) && j.cols % 16 == 0 && (j.p0 == 448 || j.p0 == 256);
         case MQ_JOB_MXFP4:
             return mq_mxfp4_fast_ok(j.in, j.dtype, j.out, j.p0);
+        case MQ_JOB_COPY:
+            return true;
         default:
             return false;
     }
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_MXFP4) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_COPY) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
+    if (j.kind == MQ_JOB_COPY) return MQ_OK;
     if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
     if (j.rows_per_block != 0) {
@@ -185,7 +190,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
             continue;
         }
         // flat kinds run on a (largest tensor) x (tensors) grid: keep the padding of a group under 25 %
-        const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST;
+        const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST && head.kind != MQ_JOB_COPY;
         int64_t j = i + 1, sum = head.rows * head.cols, mx = sum;
         while (j < n && j - i < kMaxGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
                jobs[j].cols > 0) {
@@ -232,6 +237,19 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                 rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_group(tab, st)
                      : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_group(tab, st)
                                                  : mq_int4_pack_launch_group(tab, head.p0, st);
+                break;
+            }
+            case MQ_JOB_COPY: {
+                // long aligned runs stream best from a launch of their own; everything else shares one grouped launch
+                CopyTable tab{};
+                for (int t = 0; t < cnt && rc == MQ_OK; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    const int64_t bytes = jb.rows * jb.cols;
+                    const bool aligned = (((uintptr_t)jb.in | (uintptr_t)jb.out) & 15) == 0;
+                    if (aligned && bytes >= (64 << 20)) rc = mq_copy_launch_run(jb.in, jb.out, bytes, st);
+                    else tab.job[tab.n++] = CopyJob{(const uint8_t*)jb.in, (uint8_t*)jb.out, bytes};
+                }
+                if (rc == MQ_OK && tab.n > 0) rc = mq_copy_launch_group(tab, st);
                 break;
             }
             default:

@@ -30,6 +30,7 @@ class JobBatch:
         self._array = None
         self.device = None
         self.direct_calls = 0   # kernels launched inside the block without going through the job list
+        self.constants: set[int] = set()   # addresses of result tensors whose contents never depend on the weights
 
     def __len__(self) -> int:
         return len(self._records)
@@ -66,6 +67,10 @@ class JobBatch:
 
     def input_pointers(self) -> list[int]:
         return [rec[2] for rec in self._records]
+
+    def output_pointers(self) -> set[int]:
+        """Addresses written by the recorded jobs (codes, scales, NVFP4 global scales, copy destinations)."""
+        return {rec[f] for rec in self._records for f in (3, 4, 6) if rec[f] is not None}
 
 
 def active_batch() -> JobBatch | None:
@@ -112,6 +117,15 @@ def note_direct_call() -> None:
     batch = active_batch()
     if batch is not None:
         batch.direct_calls += 1
+
+
+def note_constant(t: torch.Tensor) -> None:
+    """Called by a processor for a result tensor that is the same on every sync (a shape record, say), so that a
+    recorded batch can hand it out again without recomputing it."""
+    batch = active_batch()
+    if batch is not None:
+        batch.constants.add(t.data_ptr())
+        batch._keep.append(t)
 
 
 def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0,

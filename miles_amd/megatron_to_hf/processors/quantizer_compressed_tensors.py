@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import torch
 
+from miles_amd import launch
 from miles_amd.kernels.quant.int4_fake import pack_layer
 from miles_amd.utils.mxfp4 import quantize_mxfp4
 
@@ -38,6 +39,7 @@ def quantize_params_compressed_tensors(converted_named_params, quantization_conf
             continue
         packed, scale, zero_point = pack_layer(param, group_size, symmetric)
         shape = torch.tensor(param.shape, dtype=torch.int32, device=param.device)
+        launch.note_constant(shape)
         if zero_point is not None:
             out.append((name.replace(".weight", ".weight_zero_point"), zero_point))
         out.append((name.replace(".weight", ".weight_packed"), packed))

@@ -20,8 +20,9 @@ from collections.abc import Iterator, Mapping
 
 import torch
 
-from miles_amd import launch
+from miles_amd import _lib, launch
 from miles_amd.weight_update.bucketing import Unit
+from miles_amd.weight_update.packed_bucket import PackedBucket, layout
 from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorBase
 
 
@@ -40,8 +41,11 @@ class SyncPlan:
         self.replayable = replayable
 
     @classmethod
-    def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor]) -> "SyncPlan":
-        """Run one full sync, keeping everything needed to repeat it."""
+    def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor], *,
+               packed: bool = False) -> "SyncPlan":
+        """Run one full sync, keeping everything needed to repeat it.  With `packed`, every bucket becomes a
+        `PackedBucket`: the quantizer jobs are re-pointed at their final place in the bucket's flat payload and
+        pass-through tensors get copy jobs, so a replay produces the transport payload with no flattening pass."""
         buckets: list[Unit] = []
         marks: list[int] = []
         with launch.recording() as batch:
@@ -50,23 +54,88 @@ class SyncPlan:
                 marks.append(len(batch))   # every job of this bucket (and maybe some of the next) is recorded
         device = next((t.device for t in weights.values() if t.device.type == "cuda"), None)
         batch.device = batch.device or device
+        # every handed-out tensor must be reproduced by a replay: written by a job, a view of live parameter
+        # storage, or a declared constant (a tensor some torch op materialised would go stale)
+        spans = cls._weight_spans(weights)
+        produced = batch.output_pointers() | batch.constants
+        handed_out_ok = all(t.numel() == 0 or t.data_ptr() in produced or cls._in_spans(spans, t.data_ptr())
+                            for bucket in buckets for _, t in bucket)
+        if packed:
+            buckets, marks = cls._pack(batch, buckets, marks)
         batch.freeze()
-        replayable = batch.direct_calls == 0 and cls._inputs_alias(weights, batch)
+        replayable = batch.direct_calls == 0 and handed_out_ok and cls._inputs_alias(weights, batch)
         plan = cls(batch, buckets, marks, weights_signature(weights), replayable)
         for _ in plan.replay():     # the first execution uses the same launch partition as every replay
             pass
         return plan
 
     @staticmethod
-    def _inputs_alias(weights: Mapping[str, torch.Tensor], batch: launch.JobBatch) -> bool:
+    def _pack(batch: launch.JobBatch, buckets: list[Unit], marks: list[int]):
+        """Move every bucket into one flat payload.  A tensor that some job writes (codes, scales, NVFP4 global
+        scale) is re-homed by patching that job's pointer; anything else is copied by a job appended to the
+        bucket's range.  Returns the packed buckets and the new job marks."""
+        out_fields = (3, 4, 6)       # out, scale, aux2 of a job record
+        writers: dict[int, list[tuple[int, int]]] = {}
+        for ri, rec in enumerate(batch._records):
+            for f in out_fields:
+                if rec[f] is not None and rec[0] != _lib.JOB_COPY:
+                    writers.setdefault(rec[f], []).append((ri, f))
+        records = [list(r) for r in batch._records]
+        new_buckets: list[Unit] = []
+        copies_of: list[list[tuple]] = []
+        for bucket in buckets:      # first re-point every job (a bucket's range may hold jobs of the next bucket)
+            metas, total = layout(bucket)
+            device = bucket[0][1].device if bucket else batch.device
+            flat = torch.empty(total, dtype=torch.uint8, device=device)
+            packed = PackedBucket(flat, metas)
+            copies = []
+            for (name, old), (_, new) in zip(bucket, packed):
+                hits = writers.get(old.data_ptr()) if old.is_contiguous() and old.numel() else None
+                if hits:
+                    for ri, f in hits:
+                        records[ri][f] = new.data_ptr()
+                elif old.numel():
+                    if not old.is_contiguous():
+                        raise _lib.MilesQuantError(f"packed buckets need contiguous pass-through tensors, got {name}")
+                    nbytes = old.numel() * old.element_size()
+                    copies.append((_lib.JOB_COPY, 0, old.data_ptr(), new.data_ptr(), None, None, None, 1, nbytes, nbytes,
+                                   0, 0, 0, 0))
+                    batch._keep.append(old)
+            batch._keep.append(flat)
+            new_buckets.append(packed)
+            copies_of.append(copies)
+        new_records: list[tuple] = []
+        new_marks: list[int] = []
+        done = 0
+        for copies, mark in zip(copies_of, marks):     # then lay the list out again with each bucket's copies at its end
+            new_records.extend(tuple(r) for r in records[done:max(done, mark)])
+            done = max(done, mark)
+            new_records.extend(copies)
+            new_marks.append(len(new_records))
+        new_records.extend(tuple(r) for r in records[done:])
+        rehomed = {t.data_ptr() for bucket in buckets for _, t in bucket if t.numel() and t.data_ptr() in writers}
+        batch._keep = [t for t in batch._keep if t.data_ptr() not in rehomed]   # the first homes of re-pointed outputs
+        batch._records = new_records
+        batch._array = None
+        return new_buckets, new_marks
+
+    @staticmethod
+    def _weight_spans(weights: Mapping[str, torch.Tensor]):
         spans = sorted((t.untyped_storage().data_ptr(), t.untyped_storage().data_ptr() + t.untyped_storage().nbytes())
                        for t in weights.values())
-        starts = [s for s, _ in spans]
-        for ptr in batch.input_pointers():
-            i = bisect.bisect_right(starts, ptr) - 1
-            if i < 0 or ptr >= spans[i][1]:
-                return False
-        return True
+        return [s for s, _ in spans], spans
+
+    @staticmethod
+    def _in_spans(spans, ptr: int) -> bool:
+        starts, ranges = spans
+        i = bisect.bisect_right(starts, ptr) - 1
+        return i >= 0 and ptr < ranges[i][1]
+
+    @classmethod
+    def _inputs_alias(cls, weights: Mapping[str, torch.Tensor], batch: launch.JobBatch) -> bool:
+        """Every job input is live parameter storage or a declared constant (copy jobs move constants too)."""
+        spans = cls._weight_spans(weights)
+        return all(cls._in_spans(spans, ptr) or ptr in batch.constants for ptr in batch.input_pointers())
 
     def matches(self, weights: Mapping[str, torch.Tensor]) -> bool:
         return self.replayable and weights_signature(weights) == self.signature

@@ -19,6 +19,7 @@ import torch
 
 from miles_amd.weight_update.bucketing import Unit
 from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorDirect
+from miles_amd.weight_update.packed_bucket import pack_bucket
 from miles_amd.weight_update.sync_plan import SyncPlan
 
 
@@ -40,13 +41,15 @@ def _fp8_row_block_views_ok(args: Namespace, quantization_config: dict | None) -
 class WeightUpdater:
     def __init__(self, args: Namespace, *, weights_getter: Callable[[], Mapping[str, torch.Tensor]], model_name: str,
                  quantization_config: dict | None, send_bucket: Callable[[Unit], None],
-                 packed_weight_basenames: set[str] | None = None, use_plan: bool = True) -> None:
+                 packed_weight_basenames: set[str] | None = None, use_plan: bool = True,
+                 packed_buckets: bool = False) -> None:
         self.args = Namespace(**vars(args))
         if _fp8_row_block_views_ok(self.args, quantization_config):
             self.args.qkv_row_block_views = True
         self.weights_getter = weights_getter
         self.send_bucket = send_bucket
         self.use_plan = use_plan
+        self.packed_buckets = packed_buckets   # hand out PackedBucket payloads (the reference's broadcast_packed mode)
         self.weight_version = 0
         self._iterator = _RowBlockAwareIterator(self.args, model_name=model_name,
                                                 quantization_config=quantization_config,
@@ -71,14 +74,18 @@ class WeightUpdater:
         self._metrics["finalize_and_resume_engines"] = time.perf_counter() - t1
 
     def _iter_buckets(self, weights):
-        if not self.use_plan:
-            yield from self._iterator.iter_hf_weights(weights)
-            return
-        if self._plan is not None and self._plan.matches(weights):
+        if self.use_plan and self._plan is not None and self._plan.matches(weights):
             yield from self._plan.replay()
             return
-        self._plan = SyncPlan.record(self._iterator, weights)
-        yield from self._plan.buckets
+        if self.use_plan:
+            plan = SyncPlan.record(self._iterator, weights, packed=self.packed_buckets)
+            if plan.replayable or not self.packed_buckets:
+                self._plan = plan
+                yield from plan.buckets
+                return
+            # a packed plan re-points job outputs, which is only safe to keep when it can be replayed
+        for bucket in self._iterator.iter_hf_weights(weights):
+            yield pack_bucket(bucket) if self.packed_buckets else bucket
 
 
 class _RowBlockAwareIterator(HfWeightIteratorDirect):

@@ -216,3 +216,138 @@ def test_moe_int4_compressed_tensors_sync(oracle):
     assert [n for n, _ in flat] == [n for n, _ in want]
     for (n, g), (_, w) in zip(flat, want):
         _same(g, w, n)
+
+
+# ---------------------------------------------------------------------------------------------------
+# packed transport buckets: quantizers write straight into the flat payload
+def _payload_bytes(named):
+    return torch.cat([_bits(t).reshape(-1).view(torch.uint8) for _, t in named]) if named else torch.empty(0, dtype=torch.uint8)
+
+
+def test_packed_buckets_fp8_plan_writes_payload_in_place(oracle):
+    from miles_amd.weight_update.packed_bucket import PackedBucket
+
+    cpu = _dense_model(10)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG,
+                        send_bucket=None, packed_buckets=True)
+    got = []
+    upd.send_bucket = got.append
+    upd.update_weights()
+    torch.cuda.synchronize()
+    assert len(got) > 1 and all(isinstance(b, PackedBucket) for b in got)
+    want = _expected_fp8(oracle, cpu)
+    flat_names = [n for b in got for n, _ in b]
+    assert flat_names == [n for n, _ in want]
+    it = iter(want)
+    for b in got:
+        expect = [next(it) for _ in b]
+        for (n, g), (_, w) in zip(b, expect):
+            _same(g, w, n)
+        # the payload is the byte-for-byte concatenation of the bucket's tensors, described by the metadata
+        assert torch.equal(b.get_flattened_tensor().cpu(), _payload_bytes(expect))
+        off = 0
+        for m, (n, w) in zip(b.get_metadata(), expect):
+            assert (m.name, tuple(m.shape), m.dtype, m.start_idx, m.numel) == (n, tuple(w.shape), w.dtype, off, w.numel())
+            off = m.end_idx
+        assert off == b.flat.numel()
+        for _, t in b:      # every tensor is a view of the payload
+            assert b.flat.data_ptr() <= t.data_ptr() < b.flat.data_ptr() + max(b.flat.numel(), 1)
+    assert upd._plan is not None and upd._plan.replayable
+    # no quantizer output lives outside the payloads any more
+    payload = {(b.flat.data_ptr(), b.flat.data_ptr() + b.flat.numel()) for b in got}
+    for ptr in upd._plan.batch.output_pointers():
+        assert any(lo <= ptr < hi for lo, hi in payload)
+    # optimizer step, replay: same payload buffers, new contents
+    cpu2 = _dense_model(500)
+    for k in dev:
+        dev[k].copy_(cpu2[k])
+    first = [b.flat.data_ptr() for b in got]
+    got.clear()
+    upd.update_weights()
+    torch.cuda.synchronize()
+    assert [b.flat.data_ptr() for b in got] == first
+    it = iter(_expected_fp8(oracle, cpu2))
+    for b in got:
+        expect = [next(it) for _ in b]
+        assert torch.equal(b.flat.cpu(), _payload_bytes(expect))
+
+
+def test_packed_buckets_without_plan_and_layout_errors(oracle):
+    from miles_amd.weight_update.packed_bucket import PackedBucket, pack_bucket
+
+    cpu = _dense_model(30)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG,
+                        send_bucket=None, use_plan=False, packed_buckets=True)
+    got = []
+    upd.send_bucket = got.append
+    upd.update_weights()
+    torch.cuda.synchronize()
+    it = iter(_expected_fp8(oracle, cpu))
+    for b in got:
+        assert isinstance(b, PackedBucket)
+        assert torch.equal(b.flat.cpu(), _payload_bytes([next(it) for _ in b]))
+    # ragged sizes and unaligned pointers go through the byte path of the grouped copy
+    g = torch.Generator().manual_seed(3)
+    odd = [("a", torch.randint(0, 255, (1003,), dtype=torch.uint8, generator=g).to(DEV)[3:]),
+           ("b", torch.randint(0, 255, (40000,), dtype=torch.uint8, generator=g).to(DEV)),
+           ("c", torch.randn(0, device=DEV)),
+           ("d", torch.randint(0, 255, (17,), dtype=torch.uint8, generator=g).to(DEV))]
+    packed = pack_bucket(odd)
+    torch.cuda.synchronize()
+    assert torch.equal(packed.flat.cpu(), _payload_bytes(odd))
+    # the reference's layout rule (protocols/broadcast.py:201-205)
+    with pytest.raises(ValueError, match="Unaligned flattened weight scale: byte offset 3"):
+        pack_bucket([("w", torch.zeros(3, dtype=torch.uint8, device=DEV)), ("scale", torch.zeros(2, device=DEV))])
+
+
+def test_plan_is_not_replayed_when_a_handed_out_tensor_would_go_stale():
+    # without quantization the q/k/v tensors are fresh copies made by the name map: replaying a recorded plan would
+    # hand out last step's values, so the updater must run the full iterator every time
+    cpu = _dense_model(40)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    for packed in (False, True):
+        upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=None,
+                            send_bucket=None, packed_buckets=packed)
+        _run(upd)
+        cpu2 = _dense_model(600 + packed)
+        for k in dev:
+            dev[k].copy_(cpu2[k])
+        flat = dict(nt for b in _run(upd) for nt in b)
+        want = dict(name_maps.convert_qwen2_to_hf(ARGS, "module.module.decoder.layers.1.self_attention.linear_qkv.weight",
+                                                  cpu2["module.module.decoder.layers.1.self_attention.linear_qkv.weight"]))
+        for n, w in want.items():
+            _same(flat[n], w, n)
+
+
+def test_packed_buckets_int4_moe_two_syncs(oracle):
+    cfg = {"quant_method": "compressed-tensors", "format": "pack-quantized",
+           "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4, "type": "int"}}}}
+    basenames = {f"model.layers.{l}.mlp.experts.{e}.{p}_proj" for l in range(2) for e in range(4) for p in ("gate", "up", "down")}
+    cpu = _moe_model(50)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="kimi_k2", quantization_config=cfg, send_bucket=None,
+                        packed_weight_basenames=basenames, packed_buckets=True)
+    for seed in (50, 700):
+        src = _moe_model(seed)
+        for k in dev:
+            dev[k].copy_(src[k])
+        got = []
+        upd.send_bucket = got.append
+        upd.update_weights()
+        torch.cuda.synchronize()
+        want = []
+        for name, param in src.items():
+            for hf, t in name_maps.convert_deepseekv3_to_hf(ARGS, name, param):
+                if hf.removesuffix(".weight") in basenames:
+                    p, s, _ = oracle.pack_layer(t.contiguous(), 128)
+                    want += [(hf.replace(".weight", ".weight_packed"), p), (hf.replace(".weight", ".weight_scale"), s),
+                             (hf.replace(".weight", ".weight_shape"), torch.tensor(t.shape, dtype=torch.int32))]
+                else:
+                    want.append((hf, t))
+        it = iter(want)
+        for b in got:
+            expect = [next(it) for _ in b]
+            assert [n for n, _ in b] == [n for n, _ in expect]
+            assert torch.equal(b.flat.cpu(), _payload_bytes(expect)), f"payload of a bucket differs (seed {seed})"
