@@ -36,7 +36,7 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16,
                   # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
                   "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
-                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128}
+                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0003 B per element)
 MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0005
@@ -190,6 +190,10 @@ def adjacent_formats(gen):
     del i4
     run("next_int4_g128_asym_pack", "int4_g128_asym", lambda: [pack_layer(w, 128, sym=False) for w in ws],
         "pack_layer(sym=False), group 128")
+    from miles_amd.kernels.quant import fake_quant as fq
+    for name, fn in (("fp8", fq.fake_quant_fp8_forward), ("fp4", fq.fake_quant_fp4_forward),
+                     ("compressed_kv", fq.fake_quant_compressed_kv_forward)):
+        run(f"next_fake_quant_{name}", "fake_quant_bf16", lambda fn=fn: [fn(w) for w in ws], "bf16 in, bf16 out")
     return res
 
 

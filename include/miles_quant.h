@@ -103,6 +103,11 @@ int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, voi
 int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M, int64_t K,
                            int group, void* stream);
 
+/* fake_quant_{fp8,fp4,compressed_kv}_forward(x)       miles/kernels/quant/fake_quant.py:66-99 (kernel :25-63)
+ *   quantize + dequantize in one pass, y in the dtype of x; blocks of consecutive elements (numel % block == 0)
+ *   mode 0: e4m3, 1x32, power-of-two scale   mode 1: e2m1, 1x32, power-of-two scale   mode 2: e2m1, 1x16, e4m3 scale */
+int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, void* stream);
+
 /* NVFP4                                              miles/utils/nvfp4.py:54-114
  * The global amax travels on the device in an "amax record": MQ_NVFP4_RECORD_WORDS uint32 words made of
  * MQ_NVFP4_SECTIONS sections of MQ_NVFP4_SECTION_WORDS partial maxima (float bit patterns).  Each tensor that

@@ -1,0 +1,151 @@
+// Block fake quantization (quantize, then dequantize back to the input dtype in one pass) for gfx950.
+// Reference: miles/kernels/quant/fake_quant.py:25-99 (`_fake_quant_kernel` and its three entry points):
+//   mode 0  fp8, 1x32 blocks:  amax' = max(amax, 1e-4);        scale = ceil_pow2(amax' * f32(1/448))
+//                              q = e4m3_rne(clamp(x / scale, +-448))
+//   mode 1  fp4, 1x32 blocks:  amax' = max(amax, 6 * 2^-126);  scale = ceil_pow2(amax' * f32(1/6))
+//                              q = e2m1_rne(clamp(x / scale, +-6)), an exact zero gives +0
+//   mode 2  fp4 with e4m3 scales, 1x16 blocks ("compressed kv"):
+//                              scale = f32(e4m3_rne(min(max(amax * f32(1/6), 2^-9), 448)));  q as mode 1 with the
+//                              correctly rounded quotient x / scale
+//   out = dtype(q * scale)
+// A power-of-two scale makes x / scale exact, so it is a multiplication by the reciprocal power.  The hardware
+// conversions saturate / round exactly as clamp-then-round does for the one or two ulp by which |x / scale| can
+// exceed the format maximum.  Lanes own 8 consecutive elements; 4 (or 2) neighbouring lanes form a block.
+#include "mq_api_internal.hpp"
+#include "mq_common.hpp"
+
+namespace mq {
+
+constexpr int kFqThreads = 256;
+
+__device__ __forceinline__ float ceil_pow2_normal(float v) {   // v normal and positive
+    const uint32_t u = f2u(v);
+    return u2f(((u >> 23) + ((u & 0x7FFFFFu) != 0)) << 23);
+}
+
+template <int DT>
+__device__ __forceinline__ void fq_load8(const void* x, int64_t unit, float f[8]) {
+    if (DT == MQ_F32) {
+        const u32x4 a = ld16((const float*)x + unit * 8), b = ld16((const float*)x + unit * 8 + 4);
+        f[0] = u2f(a.x); f[1] = u2f(a.y); f[2] = u2f(a.z); f[3] = u2f(a.w);
+        f[4] = u2f(b.x); f[5] = u2f(b.y); f[6] = u2f(b.z); f[7] = u2f(b.w);
+    } else {
+        const u32x4 a = ld16((const uint16_t*)x + unit * 8);
+        const uint32_t u[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (DT == MQ_BF16) { f[2 * i] = bf16_lo(u[i]); f[2 * i + 1] = bf16_hi(u[i]); }
+            else {
+                f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] & 0xFFFFu));
+                f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] >> 16));
+            }
+        }
+    }
+}
+template <int DT>
+__device__ __forceinline__ void fq_store8(void* y, int64_t unit, const float f[8]) {
+    if (DT == MQ_F32) {
+        st16((float*)y + unit * 8, u32x4{f2u(f[0]), f2u(f[1]), f2u(f[2]), f2u(f[3])});
+        st16((float*)y + unit * 8 + 4, u32x4{f2u(f[4]), f2u(f[5]), f2u(f[6]), f2u(f[7])});
+    } else if (DT == MQ_BF16) {
+        st16((uint16_t*)y + unit * 8, u32x4{hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])});
+    } else {
+        // The compiler would fold the preceding multiplication into the conversion as fma(q, scale, +0), and adding
+        // +0 turns a -0 product into +0; the empty asm keeps the product a value of its own.
+        uint32_t p[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float a = f[2 * i], b = f[2 * i + 1];
+            asm volatile("" : "+v"(a), "+v"(b));
+            p[i] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+        }
+        st16((uint16_t*)y + unit * 8, u32x4{p[0], p[1], p[2], p[3]});
+    }
+}
+
+// MODE as above; LANES = lanes per block (4 for 1x32, 2 for 1x16)
+template <int DT, int MODE>
+__global__ __launch_bounds__(kFqThreads) void fake_quant_kernel(const void* __restrict__ x, void* __restrict__ y,
+                                                                int64_t units) {
+    constexpr int LANES = MODE == 2 ? 2 : 4;
+    const int64_t unit = (int64_t)blockIdx.x * kFqThreads + threadIdx.x;
+    const bool live = unit < units;           // a block is a whole number of lanes: dead lanes never share one with live lanes
+    float f[8];
+    fq_load8<DT>(x, live ? unit : units - 1, f);
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) m = umax(m, f2u(f[i]) & 0x7FFFFFFFu);
+    m = LANES == 4 ? group_max4(m) : group_max2(m);
+    const bool finite = m < 0x7F800000u;
+    float amax = u2f(m), scale, q[8];
+    if (MODE == 2) {
+        const float hp = __builtin_fminf(__builtin_fmaxf(amax * u2f(0x3E2AAAABu), 0.001953125f), 448.0f);
+        scale = finite ? hw_e4m3x2_decode<false>(hw_e4m3x2<false>(hp, hp, 0u)).x : sw_e4m3fn_decode(sw_e4m3fn(hp));
+        const float r = 1.0f / scale;
+        const bool fast = DT != MQ_F32;       // 16-bit numerators: the shared-divisor sequence is the exact quotient
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = fast ? div_by_shared(f[i], scale, r) : f[i] / scale;
+    } else {
+        amax = __builtin_fmaxf(amax, MODE == 0 ? 1e-4f : u2f(0x01C00000u) /* 6 * 2^-126 */);
+        scale = ceil_pow2_normal(amax * u2f(MODE == 0 ? 0x3B124925u : 0x3E2AAAABu));
+        const float r = u2f(0x7F000000u - f2u(scale));      // 2^-k for scale = 2^k
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = f[i] * r;
+    }
+    if (MODE == 0) {
+        if (finite) {
+            const uint32_t lo = hw_e4m3x4(q[0], q[1], q[2], q[3]), hi = hw_e4m3x4(q[4], q[5], q[6], q[7]);
+            const f32x2 a = hw_e4m3x2_decode<false>(lo), b = hw_e4m3x2_decode<true>(lo);
+            const f32x2 c = hw_e4m3x2_decode<false>(hi), d = hw_e4m3x2_decode<true>(hi);
+            q[0] = a.x; q[1] = a.y; q[2] = b.x; q[3] = b.y; q[4] = c.x; q[5] = c.y; q[6] = d.x; q[7] = d.y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = sw_e4m3fn_decode(sw_e4m3fn_sat(q[i]));
+        }
+    } else {
+        const bool zero[8] = {q[0] == 0.0f, q[1] == 0.0f, q[2] == 0.0f, q[3] == 0.0f,
+                              q[4] == 0.0f, q[5] == 0.0f, q[6] == 0.0f, q[7] == 0.0f};
+        uint32_t w = 0;
+        w = hw_e2m1x2<0>(q[0], q[1], w);
+        w = hw_e2m1x2<1>(q[2], q[3], w);
+        w = hw_e2m1x2<2>(q[4], q[5], w);
+        w = hw_e2m1x2<3>(q[6], q[7], w);
+        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
+        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+        q[0] = a.x; q[1] = a.y; q[2] = b.x; q[3] = b.y; q[4] = c.x; q[5] = c.y; q[6] = d.x; q[7] = d.y;
+        // an exact zero has sign 0 in the reference and comes out as +0; a negative value that rounds to zero keeps its sign
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = zero[i] ? 0.0f : q[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) q[i] = q[i] * scale;
+    if (live) fq_store8<DT>(y, unit, q);
+}
+
+}  // namespace mq
+
+using namespace mq;
+
+template <int MODE>
+static void launch_fq(const void* x, int dtype, void* y, int64_t units, hipStream_t st) {
+    const dim3 grid((unsigned)((units + kFqThreads - 1) / kFqThreads)), blk(kFqThreads);
+    if (dtype == MQ_BF16) hipLaunchKernelGGL((fake_quant_kernel<MQ_BF16, MODE>), grid, blk, 0, st, x, y, units);
+    else if (dtype == MQ_F16) hipLaunchKernelGGL((fake_quant_kernel<MQ_F16, MODE>), grid, blk, 0, st, x, y, units);
+    else hipLaunchKernelGGL((fake_quant_kernel<MQ_F32, MODE>), grid, blk, 0, st, x, y, units);
+}
+
+extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, void* stream) {
+    if (!x || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || mode < 0 || mode > 2) return mq_fail(MQ_ERR_ARG, "bad argument");
+    const int block = mode == 2 ? 16 : 32;
+    if (numel % block != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the block size");
+    if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
+    if (numel == 0) return MQ_OK;
+    const int64_t units = numel / 8;
+    if ((units + kFqThreads - 1) / kFqThreads > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    hipStream_t st = (hipStream_t)stream;
+    if (mode == 0) launch_fq<0>(x, dtype, y, units, st);
+    else if (mode == 1) launch_fq<1>(x, dtype, y, units, st);
+    else launch_fq<2>(x, dtype, y, units, st);
+    return mq_check_launch("fake quant");
+}

@@ -402,6 +402,54 @@ void mqo_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, int64_t byte
 }
 
 /* ------------------------------------------------------------------ */
+/* Block fake quantization (miles/kernels/quant/fake_quant.py:16-63)     */
+/* ------------------------------------------------------------------ */
+/* _ceil_pow2 (:16-22): exponent + (mantissa != 0), rebuilt as a power of two (inputs are normal). */
+static inline float fq_ceil_pow2(float v) {
+    uint32_t bits = f2u(v);
+    int32_t e = (int32_t)((bits >> 23) & 0xFF) - 127 + ((bits & 0x7FFFFF) != 0);
+    return u2f((uint32_t)(e + 127) << 23);
+}
+/* mode 0 fp8 1x32, mode 1 fp4 1x32 (power-of-two scales), mode 2 fp4 1x16 with an e4m3 scale (:41-62):
+ *   E4M3_SCALE: scale = f32(e4m3(min(max(amax * INV_FMAX, FLOOR), 448))); scaled = div_rn(x, scale)
+ *   else      : scale = ceil_pow2(max(amax, FLOOR) * INV_FMAX);            scaled = x / scale (exact)
+ *   scaled = clamp(scaled, -FMAX, FMAX)
+ *   FP4: q = rint(|s| / step) * step * sign(s), step 0.5 / 1 / 2 below 2 / 4 / above; sign(0) = 0
+ *   FP8: q = f32(e4m3(s))
+ *   out = dtype(q * scale)
+ * INV_FMAX is the fp32 constant nearest 1/448 or 1/6. */
+void mqo_fake_quant(const void* x, int dtype, int64_t numel, int mode, void* y) {
+    const int block = mode == 2 ? 16 : 32;
+    const float fmax_ = mode == 0 ? 448.0f : 6.0f;
+    const float inv = mode == 0 ? u2f(0x3B124925u) : u2f(0x3E2AAAABu);
+    const float floor_ = mode == 0 ? 1e-4f : mode == 1 ? u2f(0x01C00000u) : 0.001953125f;
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < numel / block; g++) {
+        float amax = 0.0f;
+        for (int j = 0; j < block; j++) amax = fmaxf(amax, fabsf(load_as_f32(x, g * block + j, dtype)));
+        float scale;
+        if (mode == 2) scale = mqo_e4m3fn_to_f32(mqo_f32_to_e4m3fn(fminf(fmaxf(amax * inv, floor_), 448.0f)));
+        else scale = fq_ceil_pow2(fmaxf(amax, floor_) * inv);
+        for (int j = 0; j < block; j++) {
+            float s = load_as_f32(x, g * block + j, dtype) / scale;
+            s = fminf(fmaxf(s, -fmax_), fmax_);
+            float q;
+            if (mode == 0) q = mqo_e4m3fn_to_f32(mqo_f32_to_e4m3fn(s));
+            else {
+                float mag = fabsf(s);
+                float step = mag < 2.0f ? 0.5f : mag < 4.0f ? 1.0f : 2.0f;
+                float sign = s > 0.0f ? 1.0f : s < 0.0f ? -1.0f : 0.0f;
+                q = rintf(mag / step) * step * sign;
+            }
+            float o = q * scale;
+            int64_t i = g * block + j;
+            if (dtype == MQ_F32) ((float*)y)[i] = o;
+            else ((uint16_t*)y)[i] = dtype == MQ_BF16 ? f32_to_bf16(o) : f32_to_f16(o);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
 /* A-3  INT4 fake quant (miles/kernels/quant/int4_fake/                 */
 /*      fake_int4_quant_cuda.cu:159-259 for (1,G); :29-91 for (1,32))   */
 /* ------------------------------------------------------------------ */

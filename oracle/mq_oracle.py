@@ -67,6 +67,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
         L.mqo_int4_unpack_dequant.restype = None
         L.mqo_int4_unpack_dequant.argtypes = [vp, vp, i32, i64, i64, i32, vp]
+        L.mqo_fake_quant.restype = None
+        L.mqo_fake_quant.argtypes = [vp, i32, i64, i32, vp]
         L.mqo_mxfp4_quant.restype = None
         L.mqo_mxfp4_quant.argtypes = [vp, i32, i64, i32, vp, vp]
         L.mqo_mxfp4_dequant.restype = None
@@ -230,6 +232,20 @@ def int4_unpack_dequant(weight_packed: torch.Tensor, weight_scale: torch.Tensor,
     assert p.shape == (M, -(-K // 8)) and K % group_size == 0 and s.numel() == M * (K // group_size)
     out = torch.empty((M, K), dtype=torch.bfloat16)
     lib().mqo_int4_unpack_dequant(p.data_ptr(), s.data_ptr(), _DTYPE[s.dtype], M, K, int(group_size), out.data_ptr())
+    return out
+
+
+# --------------------------------------------------------------------------
+# block fake quantization
+# --------------------------------------------------------------------------
+def fake_quant(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """miles/kernels/quant/fake_quant.py:66-99; kind in {"fp8", "fp4", "compressed_kv"}."""
+    _check_cpu(x)
+    mode = {"fp8": 0, "fp4": 1, "compressed_kv": 2}[kind]
+    assert x.shape[-1] % (16 if mode == 2 else 32) == 0
+    xc = x.contiguous()
+    out = torch.empty_like(xc)
+    lib().mqo_fake_quant(xc.data_ptr(), _DTYPE[xc.dtype], xc.numel(), mode, out.data_ptr())
     return out
 
 

@@ -191,9 +191,23 @@ def nvfp4() -> dict:
     return fam.save()
 
 
+def fake_quant() -> dict:
+    fam = Family("fake_quant", "torch_fake_quant_reference = the torch statement of tests/fast-gpu/kernels/quant/test_fake_quant.py:24-49",
+                 "the reference's own test statement, run by torch CPU kernels (zero signs compared by value)")
+    for dt in (torch.bfloat16, torch.float32):
+        g = torch.Generator().manual_seed(0)
+        x = (torch.randn(3, 8, 512, generator=g) * torch.logspace(-3, 3, 512)).to(dt)
+        x[0, 0, :32] = 0
+        x[1, 1, :8] = torch.tensor([448.0, -448.0, 6.0, -6.0, 3.5, 2.5, 0.75, 1.25]).to(dt)
+        for kind in ("fp8", "fp4", "compressed_kv"):
+            fam.add(f"{kind}_{str(dt).split('.')[-1]}", {"kind": kind, "dtype": str(dt).split(".")[-1], "shape": [3, 8, 512]},
+                    x=x, y=T.torch_fake_quant_reference(x, kind))
+    return fam.save()
+
+
 def main() -> None:
     manifest = {"generator": "tests/golden/make_fixtures.py", "torch": torch.__version__,
-                "families": [f() for f in (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4)]}
+                "families": [f() for f in (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4, fake_quant)]}
     with open(os.path.join(HERE, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
     total = sum(os.path.getsize(os.path.join(HERE, fam["file"])) for fam in manifest["families"])

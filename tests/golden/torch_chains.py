@@ -174,3 +174,31 @@ def torch_nvfp4(w, amax=None):
     code = code | (torch.signbit(y).to(torch.uint8) << 3)
     code = code.reshape(m, k)
     return code[:, 0::2] | (code[:, 1::2] << 4), s8.reshape(m, k // 16)
+
+
+def torch_fake_quant_reference(x, kind):
+    """The torch statement the reference's own test checks its kernels against, exactly
+    (tests/fast-gpu/kernels/quant/test_fake_quant.py:24-49): fp8 / fp4 with power-of-two scales over 32-wide blocks,
+    fp4 with e4m3 scales over 16-wide blocks ("compressed_kv")."""
+    def ceil_pow2(value):
+        mantissa, exponent = torch.frexp(value)
+        return torch.ldexp(torch.ones_like(value), torch.where(mantissa == 0.5, exponent - 1, exponent))
+
+    def round_to_fp4_grid(scaled):
+        magnitude = scaled.abs()
+        step = torch.where(magnitude < 2.0, 0.5, torch.where(magnitude < 4.0, 1.0, 2.0))
+        return torch.round(magnitude / step) * step * torch.sign(scaled)
+
+    block = 16 if kind == "compressed_kv" else 32
+    blocks = x.float().reshape(-1, block)
+    amax = blocks.abs().amax(dim=1, keepdim=True)
+    if kind == "compressed_kv":
+        scale = (amax / 6.0).clamp(2.0**-9, FP8_MAX).to(F8).float()
+        quantized = round_to_fp4_grid((blocks / scale).clamp(-6.0, 6.0))
+    elif kind == "fp4":
+        scale = ceil_pow2(amax.clamp(min=6 * 2.0**-126) / 6.0)
+        quantized = round_to_fp4_grid((blocks / scale).clamp(-6.0, 6.0))
+    else:
+        scale = ceil_pow2(amax.clamp(min=1e-4) / FP8_MAX)
+        quantized = (blocks / scale).clamp(-FP8_MAX, FP8_MAX).to(F8).float()
+    return (quantized * scale).reshape(x.shape).to(x.dtype)

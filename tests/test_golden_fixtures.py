@@ -109,6 +109,9 @@ class _OracleImpl:
     def nvfp4(self, w):
         return self.o.nvfp4_quantize_1d(w)
 
+    def fake_quant(self, x, kind):
+        return self.o.fake_quant(x, kind)
+
     def nvfp4_pair(self, a, b):
         return self.o.nvfp4_quantize_1d_pair(a, b)
 
@@ -151,6 +154,11 @@ class _HipImpl:
     def nvfp4(self, w):
         from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
         return nvfp4_quantize_1d(w)
+
+    def fake_quant(self, x, kind):
+        from miles_amd.kernels.quant import fake_quant as fq
+        return {"fp8": fq.fake_quant_fp8_forward, "fp4": fq.fake_quant_fp4_forward,
+                "compressed_kv": fq.fake_quant_compressed_kv_forward}[kind](x)
 
     def nvfp4_pair(self, a, b):
         from miles_amd.utils.nvfp4 import nvfp4_quantize_1d_pair
@@ -236,8 +244,19 @@ def _check_nvfp4(impl, case):
     _same(g, _t("nvfp4", case, "global_scale").reshape(()), f"{case} global scale")
 
 
+def _check_fake_quant(impl, case):
+    info = _info("fake_quant", case)
+    x = _t("fake_quant", case, "x", _DT[info["dtype"]]).to(impl.dev)
+    got = impl.fake_quant(x, info["kind"]).cpu()
+    want = _t("fake_quant", case, "y", _DT[info["dtype"]])
+    # the reference statement multiplies by torch.sign, which erases the sign of results that round to zero
+    assert torch.equal(got.float(), want.float()), f"{case} values"
+    nz = want != 0
+    assert torch.equal(_bits(got)[nz], _bits(want)[nz]), f"{case} bits"
+
+
 _CHECKS = [("fp8_block", _check_fp8_block), ("fp8_blockwise_cast", _check_fp8_blockwise), ("fp8_dequant", _check_fp8_dequant),
-           ("mxfp8", _check_mxfp8), ("mxfp4", _check_mxfp4), ("int4", _check_int4), ("nvfp4", _check_nvfp4)]
+           ("mxfp8", _check_mxfp8), ("mxfp4", _check_mxfp4), ("int4", _check_int4), ("nvfp4", _check_nvfp4), ("fake_quant", _check_fake_quant)]
 _PARAMS = [pytest.param(fam, fn, case, id=f"{fam}-{case}") for fam, fn in _CHECKS for case in _cases(fam)]
 
 

@@ -452,6 +452,41 @@ def test_mxfp4_grouped_jobs(oracle):
 
 
 # ---------------------------------------------------------------------------------------------------
+# block fake quantization (miles/kernels/quant/fake_quant.py)
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "compressed_kv"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fake_quant_forward(oracle, kind, dtype):
+    from miles_amd.kernels.quant import fake_quant as fq
+
+    fn = {"fp8": fq.fake_quant_fp8_forward, "fp4": fq.fake_quant_fp4_forward,
+          "compressed_kv": fq.fake_quant_compressed_kv_forward}[kind]
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(3, 37, 512, generator=g) * torch.logspace(-3, 3, 512)).to(dtype)   # the reference test's input
+    x[0, 0, :32] = 0
+    x[1, 0, :64] = torch.tensor([-0.0, 0.0] * 32).to(dtype)
+    x[1, 1, :8] = torch.tensor([448.0, -448.0, 6.0, -6.0, 3.5, 2.5, 0.75, -1e-30]).to(dtype)
+    x[1, 2, :32] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4).to(dtype)     # every fp4 tie, scale 1
+    x[2, 0, :32] = torch.finfo(dtype).max if dtype != torch.float32 else 1e38
+    got = fn(x.to(DEV))
+    assert got.dtype == dtype and got.shape == x.shape
+    _assert_same(got, oracle.fake_quant(x, kind), f"fake_quant {kind}")
+
+
+def test_fake_quant_backward_is_straight_through_and_checks_shape():
+    from miles_amd.kernels.quant import fake_quant as fq
+
+    for fn in (fq.fake_quant_fp8, fq.fake_quant_fp4, fq.fake_quant_compressed_kv):   # test_fake_quant.py:63-70
+        x = torch.randn(64, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+        grad = torch.randn_like(x)
+        fn(x).backward(grad)
+        assert torch.equal(x.grad, grad)
+    with pytest.raises(AssertionError):
+        fq.fake_quant_fp8_forward(torch.zeros(4, 48, device=DEV, dtype=torch.bfloat16))
+    # 16-wide blocks: 48 columns are fine here; 1 -> scale e4m3(1/6) = 0.171875, 1/scale = 5.8 -> 6 -> 1.03125
+    assert torch.equal(fq.fake_quant_compressed_kv_forward(torch.ones(4, 48, device=DEV)).cpu(), torch.full((4, 48), 1.03125))
+
+
+# ---------------------------------------------------------------------------------------------------
 NV_SHAPES = W.SMALL_REFERENCE_SHAPES + [(1, 16), (1, 32), (3, 48), (31, 128), (256, 256), (1024, 2048)]
 
 

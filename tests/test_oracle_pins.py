@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -351,6 +351,49 @@ def test_mxfp4_scale_exponent_from_bits_equals_float_log2_for_16_bit_inputs():
     e, gt = bits >> 7, ((bits & 0x7F) > 0x40).to(torch.int32)
     got = torch.where(e == 255, torch.full_like(e, 254), torch.clamp(e - 2 + gt, min=0))
     assert torch.equal(got, want.to(torch.int32))
+
+
+# ----------------------------------------------------------------------------------------------
+# block fake quantization (miles/kernels/quant/fake_quant.py)
+# ----------------------------------------------------------------------------------------------
+def _fake_quant_input(dtype, seed=0):
+    # the reference test's input (tests/fast-gpu/kernels/quant/test_fake_quant.py:55-60): six decades of magnitudes
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(3, 37, 512, generator=g) * torch.logspace(-3, 3, 512)).to(dtype)
+    x[0, 0, :32] = 0
+    return x
+
+
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "compressed_kv"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fake_quant_matches_the_reference_tests_torch_statement(oracle, kind, dtype):
+    for seed in (0, 1):
+        x = _fake_quant_input(dtype, seed)
+        x[1, 0, :64] = torch.tensor([-0.0, 0.0] * 32).to(dtype)
+        x[1, 1, :8] = torch.tensor([448.0, -448.0, 6.0, -6.0, 3.5, 2.5, 0.75, -1e-30]).to(dtype)
+        got = oracle.fake_quant(x, kind)
+        want = torch_fake_quant_reference(x, kind)
+        bits = torch.int32 if dtype == torch.float32 else torch.int16
+        # the reference statement multiplies by torch.sign (0 for an exact zero); compare values, then zero signs apart
+        assert torch.equal(got.float(), want.float())
+        nz = want != 0
+        assert torch.equal(got.view(bits)[nz], want.view(bits)[nz])
+
+
+def test_fake_quant_known_answers(oracle):
+    # one 32-block with amax 448: scale 1, the e4m3 grid itself
+    x = torch.tensor([448.0, 17.0, 18.0, 19.0, 21.0, 0.3, -0.3, 1e-3] + [0.0] * 24, dtype=torch.float32)
+    got = oracle.fake_quant(x, "fp8").tolist()
+    assert got[:8] == [448.0, 16.0, 18.0, 20.0, 20.0, 0.3125, -0.3125, 0.001953125]
+    # fp4: amax 6 -> scale 1; ties go to even codes, and an exact zero comes back as +0 whatever its sign
+    x = torch.tensor([6.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.0, -0.2] + [0.0] * 22, dtype=torch.float32)
+    got = oracle.fake_quant(x, "fp4")
+    assert got[:8].tolist() == [6.0, 0.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0]
+    assert got[8].item() == 0.0 and not torch.signbit(got[8]) and torch.signbit(got[9]) and got[9].item() == 0.0
+    # compressed kv: a 16-block with amax 3 -> scale e4m3(0.5) = 0.5: values land on multiples of the fp4 grid * 0.5
+    x = torch.tensor([3.0, 0.3, -1.1, 2.2] + [0.0] * 12, dtype=torch.float32)
+    assert oracle.fake_quant(x, "compressed_kv")[:4].tolist() == [3.0, 0.25, -1.0, 2.0]
+
 
 
 # ----------------------------------------------------------------------------------------------
