@@ -36,7 +36,8 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16,
                   # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
                   "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
-                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2}
+                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2,
+                  "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0003 B per element)
 MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0005
@@ -184,6 +185,9 @@ def adjacent_formats(gen):
                                "elements": elems, "workload": "8 x [16384,7168] bf16, group 32, one grouped launch"}
     del batch
     run("next_mxfp4_dequant", "mxfp4_dequant", lambda: [dequantize_mxfp4(p, s, 32) for p, s in m4], "MXFP4 -> bf16")
+    from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
+    run("next_mxfp4_to_fp8_recode", "mxfp4_to_fp8",
+        lambda: [cast_e2m1fn_to_e4m3fn(p.view(torch.int8), s) for p, s in m4], "MXFP4 -> e4m3 with 128x128 fp32 tile scales")
     del m4
     i4 = [pack_layer(w, 128) for w in ws]
     run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")

@@ -103,6 +103,12 @@ int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, voi
 int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M, int64_t K,
                            int group, void* stream);
 
+/* cast_e2m1fn_to_e4m3fn(x, scale)                     tools/convert_mxfp4_to_fp8.py:30-49
+ *   packed [out,in/2] e2m1 pairs; scale [out,in/32] E8M0 bytes; out % 128 == 0, in % 128 == 0
+ *   y [out,in] e4m3fn; tile_scale [out/128,in/128] fp32 = max scale of the tile / 64 */
+int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, void* y, float* tile_scale, int64_t out_dim,
+                          int64_t in_dim, void* stream);
+
 /* fake_quant_{fp8,fp4,compressed_kv}_forward(x)       miles/kernels/quant/fake_quant.py:66-99 (kernel :25-63)
  *   quantize + dequantize in one pass, y in the dtype of x; blocks of consecutive elements (numel % block == 0)
  *   mode 0: e4m3, 1x32, power-of-two scale   mode 1: e2m1, 1x32, power-of-two scale   mode 2: e2m1, 1x16, e4m3 scale */

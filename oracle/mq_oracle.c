@@ -449,6 +449,38 @@ void mqo_fake_quant(const void* x, int dtype, int64_t numel, int mode, void* y) 
     }
 }
 
+/* cast_e2m1fn_to_e4m3fn (tools/convert_mxfp4_to_fp8.py:30-49): per 128x128 tile
+ *   tile_scale = max(f32(scale)) / 64;  offset = f32(scale) / tile_scale;  y = e4m3(table[code] * offset)
+ * scale bytes are float8_e8m0fnu: f32 = 2^(s-127) (s = 0 is the fp32 denormal 2^-127, s = 255 NaN). */
+void mqo_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, int64_t out_dim, int64_t in_dim,
+                            uint8_t* y, float* tile_scale) {
+    static const float table[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                                    -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+    int64_t b_out = out_dim / 128, b_in = in_dim / 128, gpr = in_dim / 32;
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t ti = 0; ti < b_out; ti++)
+        for (int64_t tj = 0; tj < b_in; tj++) {
+            float top = 0.0f;
+            for (int r = 0; r < 128; r++)
+                for (int g = 0; g < 4; g++) {
+                    uint8_t sb = scale[(ti * 128 + r) * gpr + tj * 4 + g];
+                    float f = sb == 255 ? NAN : ldexpf(1.0f, (int)sb - 127);
+                    top = (f > top || f != f) ? f : top;      /* amax propagates NaN */
+                }
+            float ts = top / 64.0f;
+            tile_scale[ti * b_in + tj] = ts;
+            for (int r = 0; r < 128; r++)
+                for (int c = 0; c < 128; c++) {
+                    int64_t row = ti * 128 + r, col = tj * 128 + c;
+                    uint8_t byte = packed[row * (in_dim / 2) + col / 2];
+                    uint8_t code = (col & 1) ? (byte >> 4) : (byte & 0xF);
+                    uint8_t sb = scale[row * gpr + col / 32];
+                    float offset = (sb == 255 ? NAN : ldexpf(1.0f, (int)sb - 127)) / ts;
+                    y[row * in_dim + col] = mqo_f32_to_e4m3fn(table[code] * offset);
+                }
+        }
+}
+
 /* ------------------------------------------------------------------ */
 /* A-3  INT4 fake quant (miles/kernels/quant/int4_fake/                 */
 /*      fake_int4_quant_cuda.cu:159-259 for (1,G); :29-91 for (1,32))   */

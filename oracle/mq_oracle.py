@@ -67,6 +67,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
         L.mqo_int4_unpack_dequant.restype = None
         L.mqo_int4_unpack_dequant.argtypes = [vp, vp, i32, i64, i64, i32, vp]
+        L.mqo_mxfp4_to_fp8_block.restype = None
+        L.mqo_mxfp4_to_fp8_block.argtypes = [vp, vp, i64, i64, vp, vp]
         L.mqo_fake_quant.restype = None
         L.mqo_fake_quant.argtypes = [vp, i32, i64, i32, vp]
         L.mqo_mxfp4_quant.restype = None
@@ -275,6 +277,18 @@ def dequantize_mxfp4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, gr
     out = torch.empty((*p.shape[:-1], p.shape[-1] * 2), dtype=torch.bfloat16)
     lib().mqo_mxfp4_dequant(p.data_ptr(), s.data_ptr(), p.numel(), int(group_size), out.data_ptr())
     return out
+
+
+def cast_e2m1fn_to_e4m3fn(x: torch.Tensor, scale: torch.Tensor):
+    """tools/convert_mxfp4_to_fp8.py:30-49: int8 [out, in/2] e2m1 pairs + E8M0 [out, in/32] -> (e4m3fn [out, in], fp32 tiles)."""
+    assert x.device.type == "cpu" and x.dtype == torch.int8 and x.ndim == 2
+    out_dim, in_dim = x.size(0), x.size(1) * 2
+    assert out_dim % 128 == 0 and in_dim % 128 == 0 and tuple(scale.shape) == (out_dim, in_dim // 32)
+    p, s = x.contiguous().view(torch.uint8), scale.contiguous().view(torch.uint8)
+    y = torch.empty((out_dim, in_dim), dtype=torch.float8_e4m3fn)
+    ts = torch.empty((out_dim // 128, in_dim // 128), dtype=torch.float32)
+    lib().mqo_mxfp4_to_fp8_block(p.data_ptr(), s.data_ptr(), out_dim, in_dim, y.data_ptr(), ts.data_ptr())
+    return y, ts
 
 
 # --------------------------------------------------------------------------

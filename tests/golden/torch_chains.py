@@ -202,3 +202,18 @@ def torch_fake_quant_reference(x, kind):
         scale = ceil_pow2(amax.clamp(min=1e-4) / FP8_MAX)
         quantized = (blocks / scale).clamp(-FP8_MAX, FP8_MAX).to(F8).float()
     return (quantized * scale).reshape(x.shape).to(x.dtype)
+
+
+def torch_cast_e2m1fn_to_e4m3fn(x, scale):
+    """tools/convert_mxfp4_to_fp8.py:30-49, the reference's tensor ops in their order (scale: float8_e8m0fnu)."""
+    table = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
+    out_dim, in_dim = x.size(0), x.size(1) * 2
+    x = x.view(torch.uint8)
+    x = torch.stack([table[(x & 0x0F).long()], table[(x >> 4).long()]], dim=-1).reshape(out_dim, in_dim)
+    b_out, b_in = out_dim // 128, in_dim // 128
+    x = x.view(b_out, 128, b_in, 128).transpose(1, 2)
+    scale = scale.float().view(b_out, 128, b_in, -1).transpose(1, 2).flatten(2)
+    tile_scale = scale.amax(dim=-1, keepdim=True) / 2**6
+    offset = (scale / tile_scale).unflatten(-1, (128, -1)).repeat_interleave(32, dim=-1)
+    x = (x * offset).transpose(1, 2).reshape(out_dim, in_dim)
+    return x.to(F8), tile_scale.squeeze(-1).float()

@@ -280,3 +280,33 @@ def test_convert_mxfp4_to_bf16(tmp_path, oracle):
     index = json.loads((out / "model.safetensors.index.json").read_text())
     assert set(index["weight_map"]) == set(got)
     assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for t in got.values())
+
+
+def test_convert_mxfp4_to_fp8(tmp_path, oracle):
+    from miles_amd.tools import convert_mxfp4_to_fp8 as tool
+
+    g = torch.Generator().manual_seed(9)
+
+    def expert(seed):
+        packed = torch.randint(0, 256, (128, 128), dtype=torch.uint8, generator=g).view(torch.int8)
+        scale = torch.randint(118, 126, (128, 8), dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+        return packed, scale
+
+    (p0, s0), (p1, s1) = expert(0), expert(1)
+    shards = [{"model.layers.0.mlp.experts.0.w1.weight": p0, "model.layers.0.mlp.experts.0.w1.scale": s0,
+               "model.layers.0.mlp.experts.1.w1.weight": p1, "model.norm.weight": _rand((256,), 70)},
+              {"model.layers.0.mlp.experts.1.w1.scale": s1, "lm_head.weight": _rand((64, 256), 71)}]   # scale in another shard
+    model = _checkpoint(tmp_path, shards, {"expert_dtype": "fp4", "quantization_config": {"expert_dtype": "fp4", "quant_method": "fp8"}})
+    out = tmp_path / "fp8"
+    tool.main(str(model), str(out), "cuda")
+    got = _load_all(out)
+    for i, (p, s) in enumerate(((p0, s0), (p1, s1))):
+        y, ts = oracle.cast_e2m1fn_to_e4m3fn(p, s)
+        _same(got[f"model.layers.0.mlp.experts.{i}.w1.weight"], y, f"expert {i} codes")
+        _same(got[f"model.layers.0.mlp.experts.{i}.w1.scale"], ts, f"expert {i} tile scales")
+    _same(got["lm_head.weight"], shards[1]["lm_head.weight"], "lm_head")
+    cfg = json.loads((out / "config.json").read_text())
+    assert "expert_dtype" not in cfg and "expert_dtype" not in cfg["quantization_config"]
+    index = json.loads((out / "model.safetensors.index.json").read_text())
+    assert index["weight_map"]["model.layers.0.mlp.experts.1.w1.scale"] == index["weight_map"]["model.layers.0.mlp.experts.1.w1.weight"]
+    assert set(index["weight_map"]) == set(got) and (out / "tokenizer.json").exists()

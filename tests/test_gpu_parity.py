@@ -451,6 +451,23 @@ def test_mxfp4_grouped_jobs(oracle):
         _assert_same(p, p_o, "packed codes (grouped)")
 
 
+@pytest.mark.parametrize("shape,lo,hi", [((128, 128), 100, 140), ((256, 384), 120, 128), ((128, 256), 0, 30),
+                                         ((128, 128), 225, 255), ((2048, 7168), 110, 135)])
+def test_mxfp4_to_fp8_recode(oracle, shape, lo, hi):
+    from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
+
+    g = torch.Generator().manual_seed(41)
+    packed = torch.randint(0, 256, (shape[0], shape[1] // 2), dtype=torch.uint8, generator=g).view(torch.int8)
+    scale = torch.randint(lo, hi, (shape[0], shape[1] // 32), dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+    y, ts = cast_e2m1fn_to_e4m3fn(packed.to(DEV), scale.to(DEV))
+    y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(packed, scale)
+    assert y.dtype == torch.float8_e4m3fn and ts.dtype == torch.float32 and ts.shape == (shape[0] // 128, shape[1] // 128)
+    _assert_same(ts, ts_o, "tile scales")
+    _assert_same(y, y_o, "e4m3 codes")
+    with pytest.raises(AssertionError):
+        cast_e2m1fn_to_e4m3fn(packed[:100].to(DEV), scale[:100].to(DEV))
+
+
 # ---------------------------------------------------------------------------------------------------
 # block fake quantization (miles/kernels/quant/fake_quant.py)
 @pytest.mark.parametrize("kind", ["fp8", "fp4", "compressed_kv"])

@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -393,6 +393,26 @@ def test_fake_quant_known_answers(oracle):
     # compressed kv: a 16-block with amax 3 -> scale e4m3(0.5) = 0.5: values land on multiples of the fp4 grid * 0.5
     x = torch.tensor([3.0, 0.3, -1.1, 2.2] + [0.0] * 12, dtype=torch.float32)
     assert oracle.fake_quant(x, "compressed_kv")[:4].tolist() == [3.0, 0.25, -1.0, 2.0]
+
+
+
+def _mxfp4_checkpoint_tensor(out_dim, in_dim, seed, lo=100, hi=140):
+    g = torch.Generator().manual_seed(seed)
+    packed = torch.randint(0, 256, (out_dim, in_dim // 2), dtype=torch.uint8, generator=g).view(torch.int8)
+    scale = torch.randint(lo, hi, (out_dim, in_dim // 32), dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+    return packed, scale
+
+
+@pytest.mark.parametrize("shape,lo,hi", [((128, 128), 100, 140), ((256, 384), 120, 128), ((128, 256), 0, 30), ((128, 128), 225, 255)])
+def test_mxfp4_to_fp8_recode_matches_torch_chain(oracle, shape, lo, hi):
+    packed, scale = _mxfp4_checkpoint_tensor(*shape, seed=41, lo=lo, hi=hi)
+    y, ts = oracle.cast_e2m1fn_to_e4m3fn(packed, scale)
+    y_t, ts_t = torch_cast_e2m1fn_to_e4m3fn(packed, scale)
+    assert torch.equal(ts.view(torch.int32), ts_t.view(torch.int32)) and _same_fp8(y, y_t)
+    # lossless whenever the scales of a tile span at most 2^3 (fp4 values need e4m3's 2^-6 .. 2^8 normal range):
+    if hi - lo <= 8:
+        deq = y.float().view(shape[0] // 128, 128, shape[1] // 128, 128) * ts[:, None, :, None]
+        assert torch.equal(deq.reshape(shape).to(torch.bfloat16), oracle.dequantize_mxfp4(packed.view(torch.uint8), scale.view(torch.uint8), 32))
 
 
 
