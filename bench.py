@@ -194,6 +194,10 @@ def adjacent_formats(gen):
     del i4
     run("next_int4_g128_asym_pack", "int4_g128_asym", lambda: [pack_layer(w, 128, sym=False) for w in ws],
         "pack_layer(sym=False), group 128")
+    from miles_amd.kernels.quant.nvfp4_qdq import NVFP4QDQConfig, compute_nvfp4_amax, fused_nvfp4_qdq
+    amaxes = [compute_nvfp4_amax(w) for w in ws]
+    run("next_nvfp4_qdq", "fake_quant_bf16", lambda: [fused_nvfp4_qdq(w, a, NVFP4QDQConfig()) for w, a in zip(ws, amaxes)],
+        "fused NVFP4 quantize-dequantize given the amax, bf16 in, bf16 out")
     from miles_amd.kernels.quant import fake_quant as fq
     for name, fn in (("fp8", fq.fake_quant_fp8_forward), ("fp4", fq.fake_quant_fp4_forward),
                      ("compressed_kv", fq.fake_quant_compressed_kv_forward)):

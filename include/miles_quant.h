@@ -131,6 +131,14 @@ int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int sec
 int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
                    float* global_scale, int64_t M, int64_t K, int e4m3_max, void* stream);
 
+/* Training-forward NVFP4 fake quantization          miles/kernels/quant/nvfp4_qdq.py:1213-1229 (kernel :1067-1105)
+ * mq_nvfp4_fold: reduces the first n_sections sections of a record (written by mq_nvfp4_amax) into the amax,
+ *   stored as float bits in word MQ_NVFP4_SECTIONS * MQ_NVFP4_SECTION_WORDS of the record (compute_nvfp4_amax).
+ * mq_nvfp4_qdq: fused_nvfp4_qdq(x, amax) without Four Over Six: x bf16 / fp16, numel % 16 == 0, amax a device
+ *   fp32 scalar; y = dtype(e2m1 code * (f32(block scale) * amax / (6 * e4m3_max))) in the dtype of x. */
+int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* stream);
+int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max, void* stream);
+
 /* Batched driver: runs a list of quantization jobs on one stream, in order, with the same results as calling
  * the single-tensor entry points one by one.  Consecutive jobs of the same kind are fused into grouped
  * launches (up to 64 tensors per kernel launch, descriptors passed as kernel arguments), which is what

@@ -37,6 +37,8 @@ SIGNATURES = {
     "mq_fill_u32": [_vp, _u32, _i64, _vp],
     "mq_nvfp4_amax": [_vp, _i32, _i64, _vp, _i32, _vp],
     "mq_nvfp4_quant": [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
+    "mq_nvfp4_fold": [_vp, _i32, _i32, _vp],
+    "mq_nvfp4_qdq": [_vp, _i32, _vp, _vp, _i64, _i32, _vp],
     "mq_run_jobs": [_vp, _i64, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],

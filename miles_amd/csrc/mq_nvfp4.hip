@@ -200,6 +200,79 @@ __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __
     }
 }
 
+// ---- fused quantize + dequantize (training-forward fake quantization) -------------------------------
+// Reference: miles/kernels/quant/nvfp4_qdq.py:877-890 (standard quantize), :993-1029 (dequantize), kernel :1067-1105.
+// Given the tensor amax (a device scalar): codes and block scale exactly as the quantizer above, then
+//   final = RN(RN(f32(s8) * amax) * f32(1 / (6 * e4m3_max)));  y = dtype(RN(e2m1_value * final))
+// Two lanes own one 1x16 block; nothing but x is read and nothing but y written.
+template <int DT>
+__global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* __restrict__ x,
+                                                               const float* __restrict__ amax_ptr,
+                                                               uint16_t* __restrict__ y, int64_t total_units,
+                                                               float numer, float inv_numer) {
+    const int t = threadIdx.x;
+    const int64_t unit = (int64_t)blockIdx.x * kNvThreads + t;
+    const bool live = unit < total_units;
+    const u32x4 v = ld16(x + (live ? unit : total_units - 1) * 8);
+    const float amax = *amax_ptr;
+    const NvScales gs = nv_scales(amax, numer);
+    float f[8];
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        if (DT == MQ_BF16) { f[2 * i] = bf16_lo(u[i]); f[2 * i + 1] = bf16_hi(u[i]); }
+        else {
+            f[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] & 0xFFFFu));
+            f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[i] >> 16));
+        }
+    }
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) m = umax(m, f2u(f[i]) & 0x7FFFFFFFu);
+    m = group_max2(m);
+    const float bmax = u2f(m);
+    const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
+    float s_f, q[8];
+    if (m < 0x7F800000u && s_hp == s_hp) {
+        const uint32_t sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
+        s_f = hw_e4m3x2_decode<false>(sc).x;
+        const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
+        uint32_t word = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
+        word = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, word);
+        word = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, word);
+        word = hw_e2m1x2<3>(f[6] * inv, f[7] * inv, word);
+        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+        q[0] = a.x; q[1] = a.y; q[2] = b.x; q[3] = b.y; q[4] = c.x; q[5] = c.y; q[6] = d.x; q[7] = d.y;
+    } else {
+        const uint32_t sc = sw_e4m3fn_sat(s_hp);
+        s_f = sw_e4m3fn_decode(sc);
+        const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t c = sw_e2m1(f[j] * inv);
+            const float mag = (c & 7u) < 2u ? 0.5f * (float)(c & 7u) : u2f(0x3F000000u + ((c & 7u) << 22));
+            q[j] = (c & 8u) ? -mag : mag;
+        }
+    }
+    const float final_scale = (s_f * amax) * inv_numer;
+#pragma unroll
+    for (int j = 0; j < 8; j++) q[j] = q[j] * final_scale;
+    if (!live) return;
+    if (DT == MQ_BF16) {
+        st16(y + unit * 8, u32x4{hw_bf16x2(q[0], q[1]), hw_bf16x2(q[2], q[3]), hw_bf16x2(q[4], q[5]), hw_bf16x2(q[6], q[7])});
+    } else {
+        uint32_t p[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float a = q[2 * i], b = q[2 * i + 1];
+            asm volatile("" : "+v"(a), "+v"(b));     // keep the product apart from the conversion: a fused fma(.., +0) loses -0
+            p[i] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)a) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)b) << 16);
+        }
+        st16(y + unit * 8, u32x4{p[0], p[1], p[2], p[3]});
+    }
+}
+
 }  // namespace mq
 
 using namespace mq;
@@ -267,4 +340,34 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
                        (const uint32_t*)record, (uint8_t*)q, (uint8_t*)block_scale, blocks16);
     return mq_check_launch("nvfp4 quant");
+}
+
+extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* stream) {
+    if (!record) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (n_sections < 1 || n_sections > MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section count");
+    if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");
+    FlatTable tab{};
+    tab.n = 1;
+    tab.job[0] = FlatJob{nullptr, nullptr, nullptr, record, 0, nullptr, n_sections, 0};
+    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
+    return mq_check_launch("nvfp4 fold");
+}
+
+extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max,
+                            void* stream) {
+    if (!x || !amax || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((dtype != MQ_BF16 && dtype != MQ_F16) || numel < 0) return mq_fail(MQ_ERR_ARG, "input must be bfloat16 or float16");
+    if (numel % 16 != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of 16");
+    if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");
+    if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
+    if (numel == 0) return MQ_OK;
+    const int64_t units = numel / 8, blocks = (units + kNvThreads - 1) / kNvThreads;
+    if (blocks > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    const float numer = (float)e4m3_max * 6.0f, inv_numer = (float)(1.0 / (double)(6 * e4m3_max));
+    const dim3 grid((unsigned)blocks), blk(kNvThreads);
+    if (dtype == MQ_BF16)
+        hipLaunchKernelGGL(nvfp4_qdq_kernel<MQ_BF16>, grid, blk, 0, (hipStream_t)stream, (const uint16_t*)x, amax, (uint16_t*)y, units, numer, inv_numer);
+    else
+        hipLaunchKernelGGL(nvfp4_qdq_kernel<MQ_F16>, grid, blk, 0, (hipStream_t)stream, (const uint16_t*)x, amax, (uint16_t*)y, units, numer, inv_numer);
+    return mq_check_launch("nvfp4 qdq");
 }

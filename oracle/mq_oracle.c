@@ -700,6 +700,31 @@ void mqo_nvfp4_quant(const void* w, int dtype, int64_t M, int64_t K, float amax,
         }
 }
 
+float mqo_e2m1_to_f32(uint8_t c);
+
+/* fused_nvfp4_qdq without Four Over Six (miles/kernels/quant/nvfp4_qdq.py:877-890, 993-1029, 1067-1105):
+ * quantize exactly as mqo_nvfp4_quant, then
+ *   final = RN(RN(f32(s8) * amax) * f32(1 / (6 * e4m3_max)));  y = dtype(RN(e2m1 value * final))
+ * x bf16 or fp16, numel % 16 == 0. */
+void mqo_nvfp4_qdq(const void* x, int dtype, int64_t numel, float amax, int e4m3_max, uint16_t* y) {
+    const float inv_numer = (float)(1.0 / (double)(6 * e4m3_max));
+    int64_t nb = numel / 16;
+    uint8_t* q = (uint8_t*)malloc((size_t)numel / 2 + 1);
+    uint8_t* s8 = (uint8_t*)malloc((size_t)nb + 1);
+    mqo_nvfp4_quant(x, dtype, nb, 16, amax, e4m3_max, q, s8);
+#pragma omp parallel for schedule(static)
+    for (int64_t b = 0; b < nb; b++) {
+        float final = (mqo_e4m3fn_to_f32(s8[b]) * amax) * inv_numer;
+        for (int i = 0; i < 16; i++) {
+            uint8_t byte = q[(b * 16 + i) / 2];
+            float v = mqo_e2m1_to_f32((i & 1) ? (byte >> 4) : (byte & 0xF)) * final;
+            y[b * 16 + i] = dtype == MQ_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+        }
+    }
+    free(q);
+    free(s8);
+}
+
 /* ------------------------------------------------------------------ */
 /* decode helpers used by round-trip property tests                     */
 /* ------------------------------------------------------------------ */

@@ -69,6 +69,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_int4_unpack_dequant.argtypes = [vp, vp, i32, i64, i64, i32, vp]
         L.mqo_mxfp4_to_fp8_block.restype = None
         L.mqo_mxfp4_to_fp8_block.argtypes = [vp, vp, i64, i64, vp, vp]
+        L.mqo_nvfp4_qdq.restype = None
+        L.mqo_nvfp4_qdq.argtypes = [vp, i32, i64, f32, i32, vp]
         L.mqo_fake_quant.restype = None
         L.mqo_fake_quant.argtypes = [vp, i32, i64, i32, vp]
         L.mqo_mxfp4_quant.restype = None
@@ -364,3 +366,14 @@ def f32_to_e8m0(x: torch.Tensor) -> torch.Tensor:
 def fnv1a64(t: torch.Tensor) -> int:
     t = t.contiguous()
     return int(lib().mqo_fnv1a64(t.data_ptr(), t.numel() * t.element_size()))
+
+
+def fused_nvfp4_qdq(x: torch.Tensor, amax=None, e4m3_max: int = 448) -> torch.Tensor:
+    """miles/kernels/quant/nvfp4_qdq.py:1220-1229 (standard contract) -> tensor in the dtype of x."""
+    _check_cpu(x)
+    assert x.dtype in (torch.bfloat16, torch.float16) and x.numel() % 16 == 0
+    xc = x.contiguous()
+    a = float(nvfp4_amax(xc)) if amax is None else float(amax)
+    out = torch.empty_like(xc)
+    lib().mqo_nvfp4_qdq(xc.data_ptr(), _DTYPE[xc.dtype], xc.numel(), a, e4m3_max, out.data_ptr())
+    return out

@@ -217,3 +217,17 @@ def torch_cast_e2m1fn_to_e4m3fn(x, scale):
     offset = (scale / tile_scale).unflatten(-1, (128, -1)).repeat_interleave(32, dim=-1)
     x = (x * offset).transpose(1, 2).reshape(out_dim, in_dim)
     return x.to(F8), tile_scale.squeeze(-1).float()
+
+
+def torch_nvfp4_qdq(x, amax=None):
+    """Standard fused QDQ of miles/kernels/quant/nvfp4_qdq.py: torch_nvfp4 codes and block scales, then
+    value * RN(RN(f32(s8) * amax) * f32(1/2688)) cast to the input dtype (:993-1029)."""
+    m, k = x.shape
+    if amax is None:
+        amax = x.float().abs().max()
+    amax = torch.as_tensor(amax, dtype=torch.float32)
+    packed, s8 = torch_nvfp4(x, amax)
+    codes = torch.stack([packed & 0xF, packed >> 4], dim=-1).reshape(m, k)
+    table = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
+    final = (s8.float() * amax) * torch.tensor(1.0 / 2688.0, dtype=torch.float32)
+    return (table[codes.long()].reshape(m, k // 16, 16) * final.unsqueeze(-1)).reshape(m, k).to(x.dtype)

@@ -721,3 +721,51 @@ def test_c_abi_single_tensor_entry_points(oracle, lib):
     assert b"divisible by 32" in lib.mq_last_error()
     assert lib.mq_fp8_block_quant(None, 0, K, q.data_ptr(), s.data_ptr(), M, K, 128, 128, None) == -1
     assert L.load() is lib
+
+
+# ---------------------------------------------------------------------------------------------------
+# fused NVFP4 quantize-dequantize (miles/kernels/quant/nvfp4_qdq.py)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 16), (3, 48), (16, 64), (64, 128), (128, 1024), (2048, 7168)])
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+def test_nvfp4_qdq(oracle, shape, kind, dtype):
+    from miles_amd.kernels.quant.nvfp4_qdq import NVFP4QDQConfig, compute_nvfp4_amax, fused_nvfp4_qdq
+
+    if shape[0] > 1000 and (kind != "random" or dtype != torch.bfloat16):
+        pytest.skip("the full-size tensor is checked once")
+    x = W.reference_pattern(kind, shape, dtype=dtype, spread=12.0)
+    xd = x.to(DEV)
+    amax = compute_nvfp4_amax(xd)
+    assert amax.dtype == torch.float32 and amax.dim() == 0 and amax.item() == x.float().abs().max().item()
+    got = fused_nvfp4_qdq(xd, amax, NVFP4QDQConfig())
+    assert got.dtype == dtype and got.shape == x.shape
+    _assert_same(got, oracle.fused_nvfp4_qdq(x), "dequantized values")
+
+
+def test_nvfp4_qdq_ste_and_argument_checks(monkeypatch):
+    from miles_amd.kernels.quant import nvfp4_qdq as m
+
+    for name in ("NVTE_USE_FAST_MATH", "NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256"):
+        monkeypatch.delenv(name, raising=False)
+    x = torch.randn(64, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    x.main_grad = torch.zeros_like(x)
+    y = m.fake_nvfp4_quantization_ste(x)
+    grad = torch.randn_like(x)
+    y.backward(grad)
+    assert torch.equal(x.grad, grad) and y.main_grad is x.main_grad
+    amax = m.compute_nvfp4_amax(x)
+    with pytest.raises(TypeError, match="BF16 and FP16"):
+        m.fused_nvfp4_qdq(x.detach().float(), amax)
+    with pytest.raises(ValueError, match="K divisible by 16"):
+        m.fused_nvfp4_qdq(torch.zeros(4, 24, device=DEV, dtype=torch.bfloat16), amax)
+    with pytest.raises(ValueError, match="rank-2"):
+        m.fused_nvfp4_qdq(torch.zeros(64, device=DEV, dtype=torch.bfloat16), amax)
+    with pytest.raises(TypeError, match="exactly one FP32"):
+        m.fused_nvfp4_qdq(x.detach(), amax.double())
+    with pytest.raises(ValueError, match="only supported by Four Over Six"):
+        m.NVFP4QDQConfig(e4m3_max=256)
+    with pytest.raises(NotImplementedError):
+        m.fused_nvfp4_qdq(x.detach(), amax, m.NVFP4QDQConfig(use_4over6=True, e4m3_max=256))
+    monkeypatch.setenv("NVTE_USE_FAST_MATH", "1")
+    with pytest.raises(ValueError, match="NVTE_USE_FAST_MATH=0"):
+        m.current_nvfp4_qdq_config()

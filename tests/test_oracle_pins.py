@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -610,3 +610,15 @@ def test_nvfp4_pair_shares_one_amax(oracle):
     cq, cs, cg = oracle.nvfp4_quantize_1d(torch.cat((gate, up), dim=0))
     assert torch.equal(torch.cat((gq, uq)), cq) and _same_fp8(torch.cat((gs, us)), cs)
     assert gg.item() == ug.item() == cg.item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 16), (3, 48), (16, 64), (64, 128), (128, 1024)])
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+def test_nvfp4_qdq_matches_torch_chain(oracle, shape, kind, dtype):
+    x = W.reference_pattern(kind, shape, dtype=dtype, spread=12.0)
+    got = oracle.fused_nvfp4_qdq(x)
+    want = torch_nvfp4_qdq(x)
+    assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    if kind == "random":      # dequantized values stay within half a grid step of the input, in units of the block scale
+        assert (got.float() - x.float()).abs().max() <= x.float().abs().max() / 6.0 * 1.1
