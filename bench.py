@@ -144,6 +144,11 @@ def per_quantizer(gen):
         return out
 
     run("C5a_nvfp4", "nvfp4", n, nvfp4_all, "32 experts, gate/up paired + down, amax pass + quantize pass")
+    os.environ["NVTE_NVFP4_4OVER6"] = "weights"        # Four Over Six: two candidates per block, e4m3 max 256
+    try:
+        run("C5a_nvfp4_four_over_six", "nvfp4", n, nvfp4_all, "as C5a with NVTE_NVFP4_4OVER6=weights (MAE, e4m3 max 256)")
+    finally:
+        del os.environ["NVTE_NVFP4_4OVER6"]
     run("C5b_block_fp8", "fp8_block", n,
         lambda: [block_fp8(t, [128, 128]) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
         "32 experts, block_fp8")

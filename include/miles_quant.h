@@ -125,19 +125,25 @@ int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, vo
  * mq_nvfp4_quant: folds the record, then quantizes: w [M,K] contiguous, K % 16 == 0; q [M,K/2] (element 2i in
  *   the low nibble);
  *   block_scale [M,K/16] e4m3fn bytes; global_scale (may be NULL) receives weight_scale_2 =
- *   1 / min(e4m3_max*6/amax, FLT_MAX) as one fp32 (nvfp4.py:19-39). */
+ *   1 / min(e4m3_max*6/amax, FLT_MAX) as one fp32 (nvfp4.py:19-39).
+ * flags: MQ_NVFP4_4OVER6 selects Transformer Engine's Four Over Six block scaling (NVTE_NVFP4_4OVER6; restated in
+ *   miles/kernels/quant/nvfp4_qdq.py:893-990): every block is quantized for a maximum of 6 and of 4 and keeps the
+ *   candidate with the smaller error; MQ_NVFP4_ERR_MSE squares the error terms (NVTE_NVFP4_4OVER6_ERR_MODE=MSE),
+ *   MQ_NVFP4_ERR_FP16 uses the fp16 candidate-error form (NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH=1). */
+enum { MQ_NVFP4_4OVER6 = 1, MQ_NVFP4_ERR_MSE = 2, MQ_NVFP4_ERR_FP16 = 4 };
 int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream);
 int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream);
 int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
-                   float* global_scale, int64_t M, int64_t K, int e4m3_max, void* stream);
+                   float* global_scale, int64_t M, int64_t K, int e4m3_max, int flags, void* stream);
 
 /* Training-forward NVFP4 fake quantization          miles/kernels/quant/nvfp4_qdq.py:1213-1229 (kernel :1067-1105)
  * mq_nvfp4_fold: reduces the first n_sections sections of a record (written by mq_nvfp4_amax) into the amax,
  *   stored as float bits in word MQ_NVFP4_SECTIONS * MQ_NVFP4_SECTION_WORDS of the record (compute_nvfp4_amax).
- * mq_nvfp4_qdq: fused_nvfp4_qdq(x, amax) without Four Over Six: x bf16 / fp16, numel % 16 == 0, amax a device
+ * mq_nvfp4_qdq: fused_nvfp4_qdq(x, amax) (flags as for mq_nvfp4_quant): x bf16 / fp16, numel % 16 == 0, amax a device
  *   fp32 scalar; y = dtype(e2m1 code * (f32(block scale) * amax / (6 * e4m3_max))) in the dtype of x. */
 int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* stream);
-int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max, void* stream);
+int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max, int flags,
+                 void* stream);
 
 /* Batched driver: runs a list of quantization jobs on one stream, in order, with the same results as calling
  * the single-tensor entry points one by one.  Consecutive jobs of the same kind are fused into grouped
@@ -153,7 +159,7 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_FP8_DEQUANT          e4m3          bf16          -              aux = fp32 tile scales (in) block, -
  *   MQ_JOB_MXFP8                w             e4m3          E8M0 bytes     -                           -
  *   MQ_JOB_INT4_PACK            w             int32 words   scales (dtype) -                           group, -
- *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, -
+ *   MQ_JOB_NVFP4                w             packed e2m1   e4m3 bytes     aux = amax record,          e4m3_max, flags
  *                                                                          aux2 = fp32 weight_scale_2
  *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *   MQ_JOB_COPY                 bytes         bytes         -              -                           -

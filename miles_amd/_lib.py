@@ -36,13 +36,15 @@ SIGNATURES = {
     "mq_int4_group_quant_pack_asym": [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_fill_u32": [_vp, _u32, _i64, _vp],
     "mq_nvfp4_amax": [_vp, _i32, _i64, _vp, _i32, _vp],
-    "mq_nvfp4_quant": [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _vp],
+    "mq_nvfp4_quant": [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
     "mq_nvfp4_fold": [_vp, _i32, _i32, _vp],
-    "mq_nvfp4_qdq": [_vp, _i32, _vp, _vp, _i64, _i32, _vp],
+    "mq_nvfp4_qdq": [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _vp],
     "mq_run_jobs": [_vp, _i64, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
 }
+
+NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
  JOB_COPY) = range(8)

@@ -82,6 +82,7 @@ __global__ __launch_bounds__(256) void nvfp4_amax_generic_kernel(const void* __r
 struct NvScales {
     float enc_sixth;  // S_enc * (1/6)
     float s_dec;      // 1 / S_enc
+    float enc;        // S_enc
 };
 __device__ __forceinline__ NvScales nv_scales(float amax, float numer) {
     float enc = __builtin_fminf(numer / amax, kFltMax);
@@ -89,6 +90,7 @@ __device__ __forceinline__ NvScales nv_scales(float amax, float numer) {
     NvScales r;
     r.enc_sixth = enc * kSixth;
     r.s_dec = 1.0f / enc;
+    r.enc = enc;
     return r;
 }
 __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
@@ -102,6 +104,7 @@ __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
 constexpr int kRecAmax = MQ_NVFP4_SECTIONS * kSectionWords;   // folded amax (float bits)
 constexpr int kRecEncSixth = kRecAmax + 1;                     // S_enc * (1/6)
 constexpr int kRecSDec = kRecAmax + 2;                         // 1 / S_enc
+constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 
 // one workgroup per tensor: fold the first job.section sections of its record and publish the scales.
 // Tensors that share a record compute the same values and write them twice.
@@ -120,11 +123,97 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, fl
         rec[kRecAmax] = f2u(amax);
         rec[kRecEncSixth] = f2u(gs.enc_sixth);
         rec[kRecSDec] = f2u(gs.s_dec);
+        rec[kRecEnc] = f2u(gs.enc);
         if (job.aux2) *(float*)job.aux2 = nv_published_scale(amax, numer);
     }
 }
 
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab) {
+// ---- Four Over Six block scaling (miles/kernels/quant/nvfp4_qdq.py:893-990) --------------------------------
+// Every block is quantized twice: "map to 6" with scale6 = e4m3(min(RN(RN(bmax / 6) * S_enc), 448)) and "map to 4"
+// with scale4 = e4m3(min(RN(that product * 1.5), 448)); the candidate with the strictly smaller reconstruction
+// error wins, ties go to map-to-6.  The error is an fp32 sum over the 16 elements in element order:
+//   default   | RN(RN(RN(value * f32(scale)) * amax) / (6 * e4m3_max)) - x |   (MQ_NVFP4_ERR_MSE: its square)
+//   ERR_FP16  | f32(RN_f16(f16(value) * f16(scale))) - RN(x * S_enc) |
+struct NvCandidate {
+    uint32_t sc;     // e4m3 byte
+    uint32_t word;   // this lane's eight codes
+    float s_f;       // f32(sc)
+};
+__device__ __forceinline__ NvCandidate nv_candidate(const float f[8], float s_hp, float s_dec) {
+    NvCandidate c;
+    c.sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
+    c.s_f = hw_e4m3x2_decode<false>(c.sc).x;
+    const float inv = __builtin_fminf(1.0f / (c.s_f * s_dec), kFltMax);
+    c.word = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
+    c.word = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, c.word);
+    c.word = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, c.word);
+    c.word = hw_e2m1x2<3>(f[6] * inv, f[7] * inv, c.word);
+    return c;
+}
+__device__ __forceinline__ void nv_decode8(uint32_t word, float q[8]) {
+    const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+    const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3);
+    q[0] = a.x; q[1] = a.y; q[2] = b.x; q[3] = b.y; q[4] = c.x; q[5] = c.y; q[6] = d.x; q[7] = d.y;
+}
+// x / d for d = 2688 or 1536 with y = RN(1/d): q0 = RN(x*y); r = x - q0*d (exact in an FMA); q = RN(q0 + r*y) is the
+// correctly rounded quotient for every fp32 mantissa of x and both divisors (exhaustive CPU check, 2^23 mantissas
+// each), provided no intermediate leaves the normal range; operands outside 2^-90 .. 2^90 take the division.
+// A zero comes out as +0 whatever its sign, which no error term can see.
+__device__ __forceinline__ float div_by_numer(float x, float d, float y) {
+    const float q0 = x * y;
+    const float r = __builtin_fmaf(-q0, d, x);
+    float q = __builtin_fmaf(r, y, q0);
+    const uint32_t e = f2u(x) & 0x7F800000u;
+    if (__builtin_expect(e - 0x12000000u > 0x5A000000u && x != 0.0f, 0)) q = x / d;
+    return q;
+}
+// error terms of this lane's eight elements
+__device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandidate& c, float amax, float enc, float denom,
+                                               int flags, float term[8]) {
+    float q[8];
+    nv_decode8(c.word, q);
+    const float denom_inv = 1.0f / denom;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        float diff;
+        if (flags & MQ_NVFP4_ERR_FP16) {
+            _Float16 h = (_Float16)q[j] * (_Float16)c.s_f;        // both factors exact in fp16; one fp16 rounding
+            float hf = (float)h;
+            asm volatile("" : "+v"(hf));                          // keep the fp16 product a value of its own
+            diff = hf - f[j] * enc;
+        } else {
+            diff = div_by_numer((q[j] * c.s_f) * amax, denom, denom_inv) - f[j];
+        }
+        term[j] = (flags & MQ_NVFP4_ERR_MSE) ? diff * diff : __builtin_fabsf(diff);
+    }
+}
+// Sum of the block's sixteen terms in element order.  The even lane of the pair holds elements 0..7: its partial
+// sum from zero seeds the odd lane's accumulation, and the odd lane's total goes back to the even lane.
+__device__ __forceinline__ float nv_pair_error(const float term[8], bool odd_lane) {
+    float from_zero = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) from_zero = from_zero + term[j];
+    float seeded = u2f(dpp_u32<kDppQuadXor1>(f2u(from_zero)));
+#pragma unroll
+    for (int j = 0; j < 8; j++) seeded = seeded + term[j];
+    const float partner_total = u2f(dpp_u32<kDppQuadXor1>(f2u(seeded)));
+    return odd_lane ? seeded : partner_total;
+}
+// the winning candidate for this lane's block; bmax is the block amax (pair-uniform)
+__device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float bmax, float amax, const NvScales& gs,
+                                                        float denom, int flags, bool odd_lane) {
+    const float s6_hp = (bmax / 6.0f) * gs.enc;
+    const float s4_hp = s6_hp * 1.5f;
+    const NvCandidate c4 = nv_candidate(f, s4_hp, gs.s_dec), c6 = nv_candidate(f, s6_hp, gs.s_dec);
+    float t4[8], t6[8];
+    nv_error_terms(f, c4, amax, gs.enc, denom, flags, t4);
+    nv_error_terms(f, c6, amax, gs.enc, denom, flags, t6);
+    const float e4 = nv_pair_error(t4, odd_lane), e6 = nv_pair_error(t6, odd_lane);
+    return e4 < e6 ? c4 : c6;
+}
+
+template <int FOS>
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, int flags, float denom) {
     const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
@@ -143,6 +232,8 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     NvScales gs;
     gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
     gs.s_dec = u2f(amax_bits[kRecSDec]);
+    gs.enc = u2f(amax_bits[kRecEnc]);
+    const float amax = u2f(amax_bits[kRecAmax]);
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
@@ -153,7 +244,11 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         uint32_t sc, word;
-        if (mb < 0x7F80u && s_hp == s_hp) {
+        if (FOS) {
+            const NvCandidate c = nv_four_over_six(f, bmax, amax, gs, denom, flags, (t & 1) != 0);
+            sc = c.sc;
+            word = c.word;
+        } else if (mb < 0x7F80u && s_hp == s_hp) {
             sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
             const float s_f = hw_e4m3x2_decode<false>(sc).x;
             const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
@@ -176,18 +271,58 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     }
 }
 
+// software candidate of the one-lane-per-block kernel: codes of sixteen values and their error
+__device__ __forceinline__ float nv_candidate_sw(const float x[16], uint32_t sc, float amax, const NvScales& gs, float denom,
+                                                 int flags, uint32_t codes[16]) {
+    const float s_f = sw_e4m3fn_decode(sc);
+    const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
+    float error = 0.0f;
+    for (int j = 0; j < 16; j++) {
+        const uint32_t c = sw_e2m1(x[j] * inv);
+        codes[j] = c;
+        const float mag = (c & 7u) < 2u ? 0.5f * (float)(c & 7u) : u2f(0x3F000000u + ((c & 7u) << 22));
+        const float cand = (c & 8u) ? -mag : mag;
+        float diff;
+        if (flags & MQ_NVFP4_ERR_FP16) {
+            float hf = (float)((_Float16)cand * (_Float16)s_f);
+            asm volatile("" : "+v"(hf));
+            diff = hf - x[j] * gs.enc;
+        } else {
+            diff = ((cand * s_f) * amax) / denom - x[j];
+        }
+        error = error + ((flags & MQ_NVFP4_ERR_MSE) ? diff * diff : __builtin_fabsf(diff));
+    }
+    return error;
+}
+
 __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __restrict__ w, int dtype,
                                                                   const uint32_t* __restrict__ amax_bits,
                                                                   uint8_t* __restrict__ q, uint8_t* __restrict__ s8,
-                                                                  int64_t blocks16) {
+                                                                  int64_t blocks16, int flags, float denom) {
     NvScales gs;
     gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
     gs.s_dec = u2f(amax_bits[kRecSDec]);
+    gs.enc = u2f(amax_bits[kRecEnc]);
+    const float amax = u2f(amax_bits[kRecAmax]);
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks16; b += stride) {
         uint32_t m = 0;
         for (int j = 0; j < 16; j++) m = umax(m, f2u(load_f32(w, b * 16 + j, dtype)) & 0x7FFFFFFFu);
         const float bmax = u2f(m);
+        if (flags & MQ_NVFP4_4OVER6) {
+            float x[16];
+            for (int j = 0; j < 16; j++) x[j] = load_f32(w, b * 16 + j, dtype);
+            const float s6_hp = (bmax / 6.0f) * gs.enc, s4_hp = s6_hp * 1.5f;
+            const uint32_t sc4 = sw_e4m3fn_sat(__builtin_fminf(s4_hp, kFp8Max)), sc6 = sw_e4m3fn_sat(__builtin_fminf(s6_hp, kFp8Max));
+            uint32_t c4[16], c6[16];
+            const float e4 = nv_candidate_sw(x, sc4, amax, gs, denom, flags, c4);
+            const float e6 = nv_candidate_sw(x, sc6, amax, gs, denom, flags, c6);
+            const bool pick4 = e4 < e6;
+            s8[b] = (uint8_t)(pick4 ? sc4 : sc6);
+            for (int j = 0; j < 16; j += 2)
+                q[b * 8 + j / 2] = (uint8_t)(pick4 ? (c4[j] | (c4[j + 1] << 4)) : (c6[j] | (c6[j + 1] << 4)));
+            continue;
+        }
         const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
         const uint32_t sc = sw_e4m3fn_sat(s_hp);
         s8[b] = (uint8_t)sc;
@@ -205,11 +340,11 @@ __global__ __launch_bounds__(256) void nvfp4_quant_generic_kernel(const void* __
 // Given the tensor amax (a device scalar): codes and block scale exactly as the quantizer above, then
 //   final = RN(RN(f32(s8) * amax) * f32(1 / (6 * e4m3_max)));  y = dtype(RN(e2m1_value * final))
 // Two lanes own one 1x16 block; nothing but x is read and nothing but y written.
-template <int DT>
+template <int DT, int FOS>
 __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* __restrict__ x,
                                                                const float* __restrict__ amax_ptr,
                                                                uint16_t* __restrict__ y, int64_t total_units,
-                                                               float numer, float inv_numer) {
+                                                               float numer, float inv_numer, int flags) {
     const int t = threadIdx.x;
     const int64_t unit = (int64_t)blockIdx.x * kNvThreads + t;
     const bool live = unit < total_units;
@@ -233,7 +368,11 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* _
     const float bmax = u2f(m);
     const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
     float s_f, q[8];
-    if (m < 0x7F800000u && s_hp == s_hp) {
+    if (FOS) {
+        const NvCandidate c = nv_four_over_six(f, bmax, amax, gs, numer, flags, (t & 1) != 0);
+        s_f = c.s_f;
+        nv_decode8(c.word, q);
+    } else if (m < 0x7F800000u && s_hp == s_hp) {
         const uint32_t sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
         s_f = hw_e4m3x2_decode<false>(sc).x;
         const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
@@ -289,13 +428,15 @@ int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
 
 // tab.job[i]: w, q, s = block scales, aux = amax record, section = sections to fold, aux2 = fp32 global scale
 // out (may be null), units = numel / 8.  Launches the fold kernel, then the quantize pass.
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st) {
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStream_t st) {
     const float numer = (float)e4m3_max * 6.0f;
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     hipLaunchKernelGGL(nvfp4_fold_kernel, dim3((unsigned)tab.n), dim3(256), 0, st, tab, numer);
-    if (tab.max_blocks > 0)
-        hipLaunchKernelGGL(nvfp4_quant_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kNvThreads), 0,
-                           st, tab);
+    if (tab.max_blocks > 0) {
+        const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kNvThreads);
+        if (flags & MQ_NVFP4_4OVER6) hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<1>, grid, blk, 0, st, tab, flags, numer);
+        else hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<0>, grid, blk, 0, st, tab, flags, numer);
+    }
     return mq_check_launch("nvfp4 quant");
 }
 
@@ -316,12 +457,13 @@ extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* reco
 }
 
 extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
-                              float* global_scale, int64_t M, int64_t K, int e4m3_max, void* stream) {
+                              float* global_scale, int64_t M, int64_t K, int e4m3_max, int flags, void* stream) {
     if (!w || !record || !q || !block_scale) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (n_sections < 1 || n_sections > MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section count");
     if (K % 16 != 0) return mq_fail(MQ_ERR_ARG, "Last dim must be divisible by 16 for NVFP4");
     if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");
+    if (flags & ~(MQ_NVFP4_4OVER6 | MQ_NVFP4_ERR_MSE | MQ_NVFP4_ERR_FP16)) return mq_fail(MQ_ERR_ARG, "unknown NVFP4 flag");
     hipStream_t st = (hipStream_t)stream;
     const float numer = (float)e4m3_max * 6.0f;
     const int64_t blocks16 = M * (K / 16);
@@ -329,7 +471,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), blocks16 * 2, global_scale, n_sections, 0};
-        return mq_nvfp4_quant_launch_group(tab, e4m3_max, st);
+        return mq_nvfp4_quant_launch_group(tab, e4m3_max, flags, st);
     }
     FlatTable fold{};
     fold.n = 1;
@@ -338,7 +480,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
-                       (const uint32_t*)record, (uint8_t*)q, (uint8_t*)block_scale, blocks16);
+                       (const uint32_t*)record, (uint8_t*)q, (uint8_t*)block_scale, blocks16, flags, numer);
     return mq_check_launch("nvfp4 quant");
 }
 
@@ -354,20 +496,25 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
 }
 
 extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max,
-                            void* stream) {
+                            int flags, void* stream) {
     if (!x || !amax || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
     if ((dtype != MQ_BF16 && dtype != MQ_F16) || numel < 0) return mq_fail(MQ_ERR_ARG, "input must be bfloat16 or float16");
     if (numel % 16 != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of 16");
     if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");
     if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
+    if (flags & ~(MQ_NVFP4_4OVER6 | MQ_NVFP4_ERR_MSE | MQ_NVFP4_ERR_FP16)) return mq_fail(MQ_ERR_ARG, "unknown NVFP4 flag");
     if (numel == 0) return MQ_OK;
     const int64_t units = numel / 8, blocks = (units + kNvThreads - 1) / kNvThreads;
     if (blocks > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
     const float numer = (float)e4m3_max * 6.0f, inv_numer = (float)(1.0 / (double)(6 * e4m3_max));
     const dim3 grid((unsigned)blocks), blk(kNvThreads);
-    if (dtype == MQ_BF16)
-        hipLaunchKernelGGL(nvfp4_qdq_kernel<MQ_BF16>, grid, blk, 0, (hipStream_t)stream, (const uint16_t*)x, amax, (uint16_t*)y, units, numer, inv_numer);
-    else
-        hipLaunchKernelGGL(nvfp4_qdq_kernel<MQ_F16>, grid, blk, 0, (hipStream_t)stream, (const uint16_t*)x, amax, (uint16_t*)y, units, numer, inv_numer);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* xi = (const uint16_t*)x;
+    uint16_t* yo = (uint16_t*)y;
+    const bool fos = (flags & MQ_NVFP4_4OVER6) != 0;
+    if (dtype == MQ_BF16 && !fos) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_BF16, 0>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
+    else if (dtype == MQ_BF16) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_BF16, 1>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
+    else if (!fos) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_F16, 0>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
+    else hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_F16, 1>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
     return mq_check_launch("nvfp4 qdq");
 }

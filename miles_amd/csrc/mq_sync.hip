@@ -24,7 +24,7 @@ bool mq_int4_pack_fast_ok(const void* w, int dtype, int group);
 int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st);
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, hipStream_t st);
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
@@ -112,7 +112,7 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
             const int64_t nmx = b > mx ? b : mx;
             const bool ragged = nmx * (k - i + 1) * 4 > (bytes + b) * 5;
             if (!tied && k > i &&
-                (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 || ragged))
+                (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 || jobs[k].p1 != jobs[i].p1 || ragged))
                 break;
             mx = nmx;
             if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
@@ -143,7 +143,7 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
                 const mq_job& jb = jobs[i + t];
                 tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, sections[t], 0};
             }
-            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, st);
+            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, jobs[i].p1, st);
             if (rc) return rc;
         } else {
             for (int t = 0; t < n; t++) {
@@ -154,7 +154,7 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
                 int rc = mq_nvfp4_quant(jb.in, jb.dtype, jb.aux, sections[t], jb.out, jb.scale, (float*)jb.aux2, jb.rows,
-                                        jb.cols, jb.p0, stream);
+                                        jb.cols, jb.p0, jb.p1, stream);
                 if (rc) return rc;
             }
         }

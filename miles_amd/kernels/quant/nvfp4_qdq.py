@@ -3,8 +3,9 @@
 Mirror of the public surface of the reference's `miles/kernels/quant/nvfp4_qdq.py` (`__all__`, :1259-1266):
 `NVFP4QDQConfig` / `NVFP4QDQErrorMode` (:48-74), `current_nvfp4_qdq_config` (:93-117), `compute_nvfp4_amax`
 (:1213-1217), `fused_nvfp4_qdq` (:1220-1229) and `fake_nvfp4_quantization_ste` (:1248-1256).  The reference builds a
-CuTe-DSL kernel for Blackwell; here the standard (non Four-Over-Six) contract is one gfx950 kernel and the amax is
-the two-kernel reduction of the NVFP4 quantizer.  Four Over Six is not implemented and raises.
+CuTe-DSL kernel for Blackwell; here the contract is one gfx950 kernel and the amax is
+the two-kernel reduction of the NVFP4 quantizer.  Four Over Six (MAE / MSE, fp32 / fp16 candidate error) is a
+second instantiation of the same kernel.
 """
 
 from __future__ import annotations
@@ -116,13 +117,15 @@ def fused_nvfp4_qdq(x: torch.Tensor, amax: torch.Tensor, config: NVFP4QDQConfig 
     """Quantize to NVFP4 and dequantize again in registers; returns a detached tensor in the dtype of x."""
     if config is None:
         config = current_nvfp4_qdq_config()
-    if config.use_4over6:
-        raise NotImplementedError("Four Over Six block scaling is not implemented on gfx950")
     _validate_input(x, amax)
+    flags = 0
+    if config.use_4over6:
+        flags = _lib.NVFP4_4OVER6 | (_lib.NVFP4_ERR_MSE if config.error_mode == NVFP4QDQErrorMode.MSE else 0) \
+            | (_lib.NVFP4_ERR_FP16 if config.error_use_fast_math else 0)
     out = torch.empty_like(x)
     launch.note_direct_call()
     rc = _lib.load().mq_nvfp4_qdq(x.detach().data_ptr(), _lib.dtype_code(x, "fused_nvfp4_qdq"), amax.detach().data_ptr(),
-                                  out.data_ptr(), x.numel(), config.e4m3_max, _lib.stream_ptr(x.device))
+                                  out.data_ptr(), x.numel(), config.e4m3_max, flags, _lib.stream_ptr(x.device))
     _lib.check(rc)
     return out
 

@@ -42,10 +42,21 @@ def nvfp4_global_decode_scale_te(global_amax: torch.Tensor, nvfp4_e4m3_max: int 
     return torch.div(1.0, nvfp4_global_encode_scale_te(global_amax, nvfp4_e4m3_max))
 
 
-def _check_supported() -> int:
+def _quantizer_options() -> tuple[int, int]:
+    """(e4m3_max, flags) of the weight quantizer from Transformer Engine's environment variables: Four Over Six on or
+    off (NVTE_NVFP4_4OVER6), its error metric (NVTE_NVFP4_4OVER6_ERR_MODE, passed to NVFP4Quantizer at
+    miles/utils/nvfp4.py:72) and the fp16 candidate-error form (NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH)."""
+    flags = 0
     if _nvfp4_4over6_enabled():
-        raise NotImplementedError("NVTE_NVFP4_4OVER6 (four-over-six block scaling) is not implemented on gfx950")
-    return nvfp4_weight_e4m3_max()
+        flags |= _lib.NVFP4_4OVER6
+        mode = os.getenv("NVTE_NVFP4_4OVER6_ERR_MODE", "MAE").strip().upper()
+        if mode not in ("MAE", "MSE"):
+            raise ValueError(f"NVTE_NVFP4_4OVER6_ERR_MODE must be MAE or MSE, got {mode!r}.")
+        if mode == "MSE":
+            flags |= _lib.NVFP4_ERR_MSE
+        if os.getenv("NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH", "0").strip() == "1":
+            flags |= _lib.NVFP4_ERR_FP16
+    return nvfp4_weight_e4m3_max(), flags
 
 
 def _alloc_outputs(w: torch.Tensor):
@@ -61,13 +72,13 @@ def _alloc_outputs(w: torch.Tensor):
 def nvfp4_quantize_1d(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """weight [M, K] -> (uint8 [M, K/2], float8_e4m3fn [M, K/16], float32 [] = weight_scale_2)."""
     _lib.require_gpu(weight, "nvfp4_quantize_1d")
-    e4m3_max = _check_supported()
+    e4m3_max, flags = _quantizer_options()
     w = weight.contiguous()
     if w.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {w.shape[1]}.")
     word = torch.empty(AMAX_RECORD_WORDS, dtype=torch.int32, device=w.device)   # written by the amax pass of the job driver
     out = _alloc_outputs(w)
-    launch.submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max)
+    launch.submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max, flags)
     return out
 
 
@@ -81,7 +92,7 @@ def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
         )
     _lib.require_gpu(first, "nvfp4_quantize_1d_pair")
     _lib.require_gpu(second, "nvfp4_quantize_1d_pair")
-    e4m3_max = _check_supported()
+    e4m3_max, flags = _quantizer_options()
     a, b = first.contiguous(), second.contiguous()
     if a.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {a.shape[1]}.")
@@ -90,7 +101,7 @@ def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor):
     # two adjacent jobs on one amax word: the driver reduces both tensors before it quantizes either
     with _pair_scope() as submit:
         for w, out in zip((a, b), outs):
-            submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max)
+            submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max, flags)
     return outs
 
 

@@ -25,6 +25,10 @@
 #define MQ_BF16 0
 #define MQ_F16 1
 #define MQ_F32 2
+/* NVFP4 option flags, as in include/miles_quant.h */
+#define MQ_NVFP4_4OVER6 1
+#define MQ_NVFP4_ERR_MSE 2
+#define MQ_NVFP4_ERR_FP16 4
 
 /* ------------------------------------------------------------------ */
 /* bit-level helpers                                                    */
@@ -668,11 +672,42 @@ static inline float nvfp4_kernel_encode_scale(float amax, int e4m3_max) {
     return enc;
 }
 
+float mqo_e2m1_to_f32(uint8_t c);
+
+/* Candidate error of Four Over Six (nvfp4_qdq.py:893-953): the sum, in element order and in fp32, of
+ *   default : | RN(RN(RN(value * f32(scale)) * amax) / (6 * e4m3_max)) - x |        (or its square, MSE)
+ *   fp16    : | f32(RN_f16(f16(value) * f16(scale))) - RN(x * S_enc) |              (or its square)
+ * over the 16 elements of the block. */
+static float nvfp4_candidate_error(const float* x, const uint8_t* codes, uint8_t scale, float amax, float S_enc,
+                                   int e4m3_max, int flags) {
+    const int mse = flags & MQ_NVFP4_ERR_MSE, fp16 = flags & MQ_NVFP4_ERR_FP16;
+    const float denom = (float)(6 * e4m3_max), scale_f = mqo_e4m3fn_to_f32(scale);
+    float error = 0.0f;
+    for (int i = 0; i < 16; i++) {
+        float cand = mqo_e2m1_to_f32(codes[i]), diff;
+        if (fp16) {
+            /* both factors are exact in fp16 and their product is exact in fp32: one rounding to fp16 */
+            float prod = f16_to_f32(f32_to_f16(cand * scale_f));
+            diff = prod - x[i] * S_enc;
+        } else {
+            float dq = cand * scale_f;
+            dq = dq * amax;
+            dq = dq / denom;
+            diff = dq - x[i];
+        }
+        error = error + (mse ? diff * diff : fabsf(diff));
+    }
+    return error;
+}
+
 /* w: [M,K] contiguous, K % 16 == 0.  q: [M,K/2] (element 2i in the low
  * nibble).  s8: [M,K/16] e4m3fn bytes.  amax: global amax (for a gate/up
- * pair: over both tensors). */
-void mqo_nvfp4_quant(const void* w, int dtype, int64_t M, int64_t K, float amax,
-                     int e4m3_max, uint8_t* q, uint8_t* s8) {
+ * pair: over both tensors).
+ * flags & MQ_NVFP4_4OVER6 (nvfp4_qdq.py:956-990): two candidates per block,
+ *   scale6 = e4m3(min(RN(RN(bmax / 6) * S_enc), 448)), scale4 = e4m3(min(RN(that product * 1.5), 448)),
+ * each quantized with its own inverse; the map-to-4 candidate wins only on a strictly smaller error. */
+void mqo_nvfp4_quant_ex(const void* w, int dtype, int64_t M, int64_t K, float amax,
+                        int e4m3_max, int flags, uint8_t* q, uint8_t* s8) {
     const float sixth = u2f(0x3E2AAAABu);
     float S_enc = nvfp4_kernel_encode_scale(amax, e4m3_max);
     float S_dec = 1.0f / S_enc;                      /* nvfp4_qdq.py:1081 */
@@ -682,36 +717,54 @@ void mqo_nvfp4_quant(const void* w, int dtype, int64_t M, int64_t K, float amax,
     for (int64_t r = 0; r < M; r++)
         for (int64_t b = 0; b < nb; b++) {
             int64_t base = r * K + b * 16;
-            float bmax = 0.0f;
+            float x[16], bmax = 0.0f;
             for (int i = 0; i < 16; i++) {
-                float a = fabsf(load_as_f32(w, base + i, dtype));
+                x[i] = load_as_f32(w, base + i, dtype);
+                float a = fabsf(x[i]);
                 if (a > bmax) bmax = a;
             }
-            float s_hp = (bmax == 0.0f) ? 0.0f : bmax * enc_sixth; /* :716-743 */
-            uint8_t sc = mqo_f32_to_e4m3fn_sat(s_hp);             /* :489-511 */
-            s8[r * nb + b] = sc;
-            float s_f = mqo_e4m3fn_to_f32(sc);
-            float inv = fminf(1.0f / (s_f * S_dec), MQO_FLT_MAX); /* :870-873 */
-            for (int i = 0; i < 16; i += 2) {
-                uint8_t lo = mqo_f32_to_e2m1(load_as_f32(w, base + i, dtype) * inv);
-                uint8_t hi = mqo_f32_to_e2m1(load_as_f32(w, base + i + 1, dtype) * inv);
-                q[(base + i) / 2] = (uint8_t)(lo | (hi << 4));    /* :571-575 */
+            uint8_t sc, codes[16];
+            if (flags & MQ_NVFP4_4OVER6) {
+                float s6_hp = (bmax / 6.0f) * S_enc;
+                float s4_hp = s6_hp * 1.5f;
+                uint8_t sc4 = mqo_f32_to_e4m3fn_sat(fminf(s4_hp, 448.0f)), sc6 = mqo_f32_to_e4m3fn_sat(fminf(s6_hp, 448.0f));
+                float inv4 = fminf(1.0f / (mqo_e4m3fn_to_f32(sc4) * S_dec), MQO_FLT_MAX);
+                float inv6 = fminf(1.0f / (mqo_e4m3fn_to_f32(sc6) * S_dec), MQO_FLT_MAX);
+                uint8_t c4[16], c6[16];
+                for (int i = 0; i < 16; i++) {
+                    c4[i] = mqo_f32_to_e2m1(x[i] * inv4);
+                    c6[i] = mqo_f32_to_e2m1(x[i] * inv6);
+                }
+                float e4 = nvfp4_candidate_error(x, c4, sc4, amax, S_enc, e4m3_max, flags);
+                float e6 = nvfp4_candidate_error(x, c6, sc6, amax, S_enc, e4m3_max, flags);
+                int pick4 = e4 < e6;
+                sc = pick4 ? sc4 : sc6;
+                memcpy(codes, pick4 ? c4 : c6, 16);
+            } else {
+                float s_hp = (bmax == 0.0f) ? 0.0f : bmax * enc_sixth; /* :716-743 */
+                sc = mqo_f32_to_e4m3fn_sat(s_hp);                     /* :489-511 */
+                float inv = fminf(1.0f / (mqo_e4m3fn_to_f32(sc) * S_dec), MQO_FLT_MAX); /* :870-873 */
+                for (int i = 0; i < 16; i++) codes[i] = mqo_f32_to_e2m1(x[i] * inv);
             }
+            s8[r * nb + b] = sc;
+            for (int i = 0; i < 16; i += 2) q[(base + i) / 2] = (uint8_t)(codes[i] | (codes[i + 1] << 4)); /* :571-575 */
         }
 }
+void mqo_nvfp4_quant(const void* w, int dtype, int64_t M, int64_t K, float amax,
+                     int e4m3_max, uint8_t* q, uint8_t* s8) {
+    mqo_nvfp4_quant_ex(w, dtype, M, K, amax, e4m3_max, 0, q, s8);
+}
 
-float mqo_e2m1_to_f32(uint8_t c);
-
-/* fused_nvfp4_qdq without Four Over Six (miles/kernels/quant/nvfp4_qdq.py:877-890, 993-1029, 1067-1105):
- * quantize exactly as mqo_nvfp4_quant, then
+/* fused_nvfp4_qdq (miles/kernels/quant/nvfp4_qdq.py:877-890, 956-1029, 1067-1105):
+ * quantize exactly as mqo_nvfp4_quant_ex, then
  *   final = RN(RN(f32(s8) * amax) * f32(1 / (6 * e4m3_max)));  y = dtype(RN(e2m1 value * final))
  * x bf16 or fp16, numel % 16 == 0. */
-void mqo_nvfp4_qdq(const void* x, int dtype, int64_t numel, float amax, int e4m3_max, uint16_t* y) {
+void mqo_nvfp4_qdq(const void* x, int dtype, int64_t numel, float amax, int e4m3_max, int flags, uint16_t* y) {
     const float inv_numer = (float)(1.0 / (double)(6 * e4m3_max));
     int64_t nb = numel / 16;
     uint8_t* q = (uint8_t*)malloc((size_t)numel / 2 + 1);
     uint8_t* s8 = (uint8_t*)malloc((size_t)nb + 1);
-    mqo_nvfp4_quant(x, dtype, nb, 16, amax, e4m3_max, q, s8);
+    mqo_nvfp4_quant_ex(x, dtype, nb, 16, amax, e4m3_max, flags, q, s8);
 #pragma omp parallel for schedule(static)
     for (int64_t b = 0; b < nb; b++) {
         float final = (mqo_e4m3fn_to_f32(s8[b]) * amax) * inv_numer;

@@ -70,7 +70,9 @@ def lib() -> ctypes.CDLL:
         L.mqo_mxfp4_to_fp8_block.restype = None
         L.mqo_mxfp4_to_fp8_block.argtypes = [vp, vp, i64, i64, vp, vp]
         L.mqo_nvfp4_qdq.restype = None
-        L.mqo_nvfp4_qdq.argtypes = [vp, i32, i64, f32, i32, vp]
+        L.mqo_nvfp4_qdq.argtypes = [vp, i32, i64, f32, i32, i32, vp]
+        L.mqo_nvfp4_quant_ex.restype = None
+        L.mqo_nvfp4_quant_ex.argtypes = [vp, i32, i64, i64, f32, i32, i32, vp, vp]
         L.mqo_fake_quant.restype = None
         L.mqo_fake_quant.argtypes = [vp, i32, i64, i32, vp]
         L.mqo_mxfp4_quant.restype = None
@@ -310,8 +312,11 @@ def nvfp4_global_decode_scale(amax: float, e4m3_max: int = 448) -> float:
     return float(lib().mqo_nvfp4_global_decode_scale(amax, e4m3_max))
 
 
-def nvfp4_quantize_1d(weight: torch.Tensor, amax: float | None = None, e4m3_max: int = 448):
-    """miles/utils/nvfp4.py:54-82 -> (uint8 [M,K/2], e4m3fn [M,K/16], float32 [])."""
+NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4
+
+
+def nvfp4_quantize_1d(weight: torch.Tensor, amax: float | None = None, e4m3_max: int = 448, flags: int = 0):
+    """miles/utils/nvfp4.py:54-82 -> (uint8 [M,K/2], e4m3fn [M,K/16], float32 []).  `flags`: Four Over Six options."""
     _check_cpu(weight)
     assert weight.dim() == 2
     w = weight.contiguous()
@@ -321,15 +326,15 @@ def nvfp4_quantize_1d(weight: torch.Tensor, amax: float | None = None, e4m3_max:
         amax = nvfp4_amax(w)
     q = torch.empty((M, K // 2), dtype=torch.uint8)
     s = torch.empty((M, K // 16), dtype=torch.uint8)
-    lib().mqo_nvfp4_quant(w.data_ptr(), _DTYPE[w.dtype], M, K, amax, e4m3_max, q.data_ptr(), s.data_ptr())
+    lib().mqo_nvfp4_quant_ex(w.data_ptr(), _DTYPE[w.dtype], M, K, amax, e4m3_max, flags, q.data_ptr(), s.data_ptr())
     g = torch.tensor(nvfp4_global_decode_scale(amax, e4m3_max), dtype=torch.float32)
     return q, s.view(torch.float8_e4m3fn), g
 
 
-def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor, e4m3_max: int = 448):
+def nvfp4_quantize_1d_pair(first: torch.Tensor, second: torch.Tensor, e4m3_max: int = 448, flags: int = 0):
     """miles/utils/nvfp4.py:85-114: one amax over both tensors."""
     amax = max(nvfp4_amax(first), nvfp4_amax(second))
-    return nvfp4_quantize_1d(first, amax, e4m3_max), nvfp4_quantize_1d(second, amax, e4m3_max)
+    return nvfp4_quantize_1d(first, amax, e4m3_max, flags), nvfp4_quantize_1d(second, amax, e4m3_max, flags)
 
 
 # --------------------------------------------------------------------------
@@ -368,12 +373,12 @@ def fnv1a64(t: torch.Tensor) -> int:
     return int(lib().mqo_fnv1a64(t.data_ptr(), t.numel() * t.element_size()))
 
 
-def fused_nvfp4_qdq(x: torch.Tensor, amax=None, e4m3_max: int = 448) -> torch.Tensor:
-    """miles/kernels/quant/nvfp4_qdq.py:1220-1229 (standard contract) -> tensor in the dtype of x."""
+def fused_nvfp4_qdq(x: torch.Tensor, amax=None, e4m3_max: int = 448, flags: int = 0) -> torch.Tensor:
+    """miles/kernels/quant/nvfp4_qdq.py:1220-1229 -> tensor in the dtype of x."""
     _check_cpu(x)
     assert x.dtype in (torch.bfloat16, torch.float16) and x.numel() % 16 == 0
     xc = x.contiguous()
     a = float(nvfp4_amax(xc)) if amax is None else float(amax)
     out = torch.empty_like(xc)
-    lib().mqo_nvfp4_qdq(xc.data_ptr(), _DTYPE[xc.dtype], xc.numel(), a, e4m3_max, out.data_ptr())
+    lib().mqo_nvfp4_qdq(xc.data_ptr(), _DTYPE[xc.dtype], xc.numel(), a, e4m3_max, flags, out.data_ptr())
     return out

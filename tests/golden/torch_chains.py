@@ -231,3 +231,51 @@ def torch_nvfp4_qdq(x, amax=None):
     table = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
     final = (s8.float() * amax) * torch.tensor(1.0 / 2688.0, dtype=torch.float32)
     return (table[codes.long()].reshape(m, k // 16, 16) * final.unsqueeze(-1)).reshape(m, k).to(x.dtype)
+
+
+def torch_nvfp4_4over6(w, amax=None, e4m3_max=448, mse=False, fp16_error=False):
+    """Four Over Six block scaling (miles/kernels/quant/nvfp4_qdq.py:893-990) with fp32 tensor ops: both candidates are
+    quantized for every block, errors are accumulated element by element in fp32, map-to-4 wins on a strictly smaller
+    error.  Returns (packed codes, e4m3 block scales)."""
+    f32 = torch.float32
+    m, k = w.shape
+    x = w.float().reshape(m, k // 16, 16)
+    if amax is None:
+        amax = x.abs().max()
+    amax = torch.as_tensor(amax, dtype=f32)
+    flt_max = torch.tensor(torch.finfo(f32).max)
+    numer = torch.tensor(float(e4m3_max * 6), dtype=f32)
+    s_enc = torch.min(numer / amax, flt_max)
+    if amax == 0 or s_enc == 0:
+        s_enc = torch.tensor(1.0, dtype=f32)
+    s_dec = torch.tensor(1.0, dtype=f32) / s_enc
+    bmax = x.abs().amax(dim=-1, keepdim=True)
+    s6_hp = (bmax / torch.tensor(6.0, dtype=f32)) * s_enc
+    s4_hp = s6_hp * torch.tensor(1.5, dtype=f32)
+    table = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+
+    def candidate(s_hp):
+        s8 = s_hp.clamp(max=FP8_MAX).to(F8)
+        inv = torch.min(torch.tensor(1.0, dtype=f32) / (s8.float() * s_dec), flt_max)
+        y = x * inv
+        mag = y.abs().clamp(max=6.0)
+        step = torch.where(mag < 2.0, 0.5, torch.where(mag < 4.0, 1.0, 2.0))
+        val = torch.round(mag / step) * step
+        code = torch.bucketize(val, table).to(torch.uint8) | (torch.signbit(y).to(torch.uint8) << 3)
+        cand = torch.where(torch.signbit(y), -val, val)
+        if fp16_error:
+            diff = (cand.half() * s8.float().half()).float() - x * s_enc
+        else:
+            diff = ((cand * s8.float()) * amax) / torch.tensor(float(6 * e4m3_max), dtype=f32) - x
+        term = diff * diff if mse else diff.abs()
+        err = torch.zeros(m, k // 16, dtype=f32)
+        for i in range(16):
+            err = err + term[..., i]
+        return code, s8, err
+
+    c4, s4, e4 = candidate(s4_hp)
+    c6, s6, e6 = candidate(s6_hp)
+    pick4 = e4 < e6
+    code = torch.where(pick4.unsqueeze(-1), c4, c6).reshape(m, k)
+    s8 = torch.where(pick4.unsqueeze(-1), s4.view(torch.uint8), s6.view(torch.uint8)).view(F8)
+    return code[:, 0::2] | (code[:, 1::2] << 4), s8.reshape(m, k // 16)

@@ -707,7 +707,7 @@ def test_c_abi_single_tensor_entry_points(oracle, lib):
     g = torch.empty((), dtype=torch.float32, device=DEV)
     assert lib.mq_fill_u32(word.data_ptr(), 0x7F800000, 1280, None) == 0   # stale contents must not matter
     assert lib.mq_nvfp4_amax(d.data_ptr(), 0, M * K, word.data_ptr(), 0, None) == 0
-    assert lib.mq_nvfp4_quant(d.data_ptr(), 0, word.data_ptr(), 1, q4.data_ptr(), s8.data_ptr(), g.data_ptr(), M, K, 448,
+    assert lib.mq_nvfp4_quant(d.data_ptr(), 0, word.data_ptr(), 1, q4.data_ptr(), s8.data_ptr(), g.data_ptr(), M, K, 448, 0,
                               None) == 0
     q_o, s_o, g_o = oracle.nvfp4_quantize_1d(w)
     _assert_same(q4, q_o, "mq_nvfp4_quant codes")
@@ -764,8 +764,68 @@ def test_nvfp4_qdq_ste_and_argument_checks(monkeypatch):
         m.fused_nvfp4_qdq(x.detach(), amax.double())
     with pytest.raises(ValueError, match="only supported by Four Over Six"):
         m.NVFP4QDQConfig(e4m3_max=256)
-    with pytest.raises(NotImplementedError):
-        m.fused_nvfp4_qdq(x.detach(), amax, m.NVFP4QDQConfig(use_4over6=True, e4m3_max=256))
     monkeypatch.setenv("NVTE_USE_FAST_MATH", "1")
     with pytest.raises(ValueError, match="NVTE_USE_FAST_MATH=0"):
         m.current_nvfp4_qdq_config()
+
+
+# ---------------------------------------------------------------------------------------------------
+# NVFP4 Four Over Six block scaling (NVTE_NVFP4_4OVER6; miles/kernels/quant/nvfp4_qdq.py:893-990)
+_FOS_CASES = [(448, "MAE", False), (256, "MAE", False), (256, "MSE", False), (256, "MAE", True), (448, "MSE", True)]
+
+
+def _fos_env(monkeypatch, e4m3_max, mode, fp16):
+    monkeypatch.setenv("NVTE_NVFP4_4OVER6", "weights")
+    monkeypatch.setenv("NVTE_NVFP4_4OVER6_E4M3_USE_256", "all" if e4m3_max == 256 else "none")
+    monkeypatch.setenv("NVTE_NVFP4_4OVER6_ERR_MODE", mode)
+    monkeypatch.setenv("NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH", "1" if fp16 else "0")
+    monkeypatch.delenv("NVTE_USE_FAST_MATH", raising=False)
+
+
+@pytest.mark.parametrize("e4m3_max,mode,fp16", _FOS_CASES)
+@pytest.mark.parametrize("shape", [(1, 16), (3, 48), (64, 128), (128, 1024), (512, 7168)])
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+def test_nvfp4_four_over_six_quantizer(oracle, monkeypatch, shape, kind, e4m3_max, mode, fp16):
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    if shape[0] > 500 and kind != "random":
+        pytest.skip("the large tensor is checked on random data")
+    _fos_env(monkeypatch, e4m3_max, mode, fp16)
+    flags = oracle.NVFP4_4OVER6 | (oracle.NVFP4_ERR_MSE if mode == "MSE" else 0) | (oracle.NVFP4_ERR_FP16 if fp16 else 0)
+    w = W.reference_pattern(kind, shape, spread=12.0)
+    if kind == "random" and shape[0] > 1:
+        w[0].zero_()
+    q, s, g = nvfp4_quantize_1d(w.to(DEV))
+    q_o, s_o, g_o = oracle.nvfp4_quantize_1d(w, e4m3_max=e4m3_max, flags=flags)
+    _assert_same(s, s_o, "block scales")
+    _assert_same(q, q_o, "codes")
+    _assert_same(g, g_o, "global scale")
+    if shape == (64, 128):
+        up = 3 * W.reference_pattern("random", (32, 128), spread=12.0, seed=2)
+        (gq, gs, gg), (uq, us, ug) = nvfp4_quantize_1d_pair(w.to(DEV), up.to(DEV))
+        (gq_o, gs_o, gg_o), (uq_o, us_o, ug_o) = oracle.nvfp4_quantize_1d_pair(w, up, e4m3_max=e4m3_max, flags=flags)
+        for a, b, what in ((gq, gq_o, "pair codes"), (gs, gs_o, "pair scales"), (uq, uq_o, "pair up codes"), (us, us_o, "pair up scales"),
+                           (gg, gg_o, "pair global"), (ug, ug_o, "pair up global")):
+            _assert_same(a, b, what)
+
+
+@pytest.mark.parametrize("e4m3_max,mode,fp16", _FOS_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_nvfp4_four_over_six_qdq_and_other_dtypes(oracle, monkeypatch, dtype, e4m3_max, mode, fp16):
+    from miles_amd.kernels.quant import nvfp4_qdq as m
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    _fos_env(monkeypatch, e4m3_max, mode, fp16)
+    flags = oracle.NVFP4_4OVER6 | (oracle.NVFP4_ERR_MSE if mode == "MSE" else 0) | (oracle.NVFP4_ERR_FP16 if fp16 else 0)
+    x = W.reference_pattern("random", (96, 256), dtype=dtype, spread=12.0, seed=5)
+    x[1].zero_()
+    cfg = m.current_nvfp4_qdq_config()
+    assert cfg.use_4over6 and cfg.e4m3_max == e4m3_max and cfg.error_use_fast_math == fp16 and cfg.error_mode.name == mode
+    got = m.fused_nvfp4_qdq(x.to(DEV), m.compute_nvfp4_amax(x.to(DEV)), cfg)
+    _assert_same(got, oracle.fused_nvfp4_qdq(x, e4m3_max=e4m3_max, flags=flags), "dequantized values")
+    # fp16 / fp32 weights take the one-lane-per-block quantizer kernel
+    xf = x.float() if dtype == torch.float16 else x.half()
+    q, s, g = nvfp4_quantize_1d(xf.to(DEV))
+    q_o, s_o, g_o = oracle.nvfp4_quantize_1d(xf, e4m3_max=e4m3_max, flags=flags)
+    _assert_same(s, s_o, "block scales (generic kernel)")
+    _assert_same(q, q_o, "codes (generic kernel)")

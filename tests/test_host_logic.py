@@ -330,3 +330,20 @@ class TestDispatch:
         assert out[2][1].tolist() == [4, 32] and out[2][1].dtype == torch.int32
         with pytest.raises(AssertionError, match="packed weight names"):
             P.quantize_params(None, "x", params, cfg)
+
+
+def test_division_by_the_nvfp4_numerators_is_exact_with_one_fma_correction():
+    # Four Over Six divides every dequantized candidate by 6 * e4m3_max.  The gfx950 kernel uses
+    # q0 = x*y; r = fma(-q0, d, x); q = fma(r, y, q0) with y = RN(1/d): check it against the IEEE quotient on a
+    # large sample of mantissas here (the exhaustive sweep over all 2^23 mantissas was run once in C).
+    import numpy as np
+    rng = np.random.default_rng(1)
+    for d in (2688.0, 1536.0):
+        d32 = np.float32(d)
+        y = np.float32(1.0) / d32
+        m = rng.integers(0, 1 << 23, size=1 << 20, dtype=np.uint32)
+        x = ((np.uint32(127) << np.uint32(23)) | m).view(np.float32)
+        q0 = x * y
+        r = (-(q0.astype(np.float64) * np.float64(d32)) + x.astype(np.float64)).astype(np.float32)   # exact: the fma's value
+        q = (r.astype(np.float64) * np.float64(y) + q0.astype(np.float64)).astype(np.float32)
+        assert np.array_equal(q, x / d32)

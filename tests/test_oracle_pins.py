@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -622,3 +622,21 @@ def test_nvfp4_qdq_matches_torch_chain(oracle, shape, kind, dtype):
     assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
     if kind == "random":      # dequantized values stay within half a grid step of the input, in units of the block scale
         assert (got.float() - x.float()).abs().max() <= x.float().abs().max() / 6.0 * 1.1
+
+
+@pytest.mark.parametrize("e4m3_max,mse,fp16", [(448, False, False), (256, False, False), (256, True, False), (256, False, True),
+                                               (448, True, True)])
+@pytest.mark.parametrize("shape", [(1, 16), (3, 48), (16, 64), (64, 128), (128, 1024)])
+@pytest.mark.parametrize("kind", ["random", "boundary", "zeros", "signed_zeros", "maxes"])
+def test_nvfp4_four_over_six_matches_torch_chain(oracle, shape, kind, e4m3_max, mse, fp16):
+    w = W.reference_pattern(kind, shape, spread=12.0)
+    if kind == "random" and shape[0] > 1:
+        w[0].zero_()
+    flags = oracle.NVFP4_4OVER6 | (oracle.NVFP4_ERR_MSE if mse else 0) | (oracle.NVFP4_ERR_FP16 if fp16 else 0)
+    q, s, g = oracle.nvfp4_quantize_1d(w, e4m3_max=e4m3_max, flags=flags)
+    q_t, s_t = torch_nvfp4_4over6(w, e4m3_max=e4m3_max, mse=mse, fp16_error=fp16)
+    assert _same_fp8(s, s_t) and torch.equal(q, q_t)
+    if kind == "random" and shape[0] >= 16:
+        # both candidates are really in play, and the chosen one never has the larger error
+        q6, s6, _ = oracle.nvfp4_quantize_1d(w, e4m3_max=e4m3_max)
+        assert 0 < (s.view(torch.uint8) != s6.view(torch.uint8)).sum() < s.numel()
