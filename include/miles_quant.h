@@ -74,10 +74,11 @@ int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t* scale, in
  *   packed [bytes]; scale [2*bytes/group]; y [2*bytes] bf16 */
 int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, void* y, int64_t bytes, int group, void* stream);
 
-/* fake_int4_quant_cuda(x, (1, group), sym)           miles/kernels/quant/int4_fake/fake_int4_quant_cuda.cu:319-364
- *   x [M,N] contiguous; out [M,N], scale [M,ceil(N/group)], zero (asym only) in the dtype of x */
+/* fake_int4_quant_cuda(x, (block_m, block_n), sym)   miles/kernels/quant/int4_fake/fake_int4_quant_cuda.cu:319-364
+ *   x [M,N] contiguous; a group is a block_m x block_n tile (block_m * block_n % 32 == 0), entries past the edge
+ *   count as 0; out [M,N], scale [ceil(M/block_m), ceil(N/block_n)], zero (asym only) in the dtype of x */
 int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
-                       int group, int sym, void* stream);
+                       int block_m, int block_n, int sym, void* stream);
 
 /* pack_layer(weight, group_size, sym=True)           .../processors/quantizer_compressed_tensors.py:235-265
  *                                                    (== tools/convert_hf_to_int4_direct.py:121-151)

@@ -26,7 +26,7 @@ SIGNATURES = {
     "mq_fp8_scaled_quant": [_vp, _i32, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _vp],
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp8_quant": [_vp, _i32, _vp, _vp, _i64, _i64, _vp],
-    "mq_int4_fake_quant": [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
+    "mq_int4_fake_quant": [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp],
     "mq_int4_unpack_dequant": [_vp, _vp, _i32, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp4_to_fp8_block": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "mq_fake_quant": [_vp, _i32, _vp, _i64, _i32, _vp],

@@ -82,23 +82,24 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTa
     }
 }
 
-// One wavefront per group, lanes stride the columns: any dtype, any G, ragged last group, sym and asym.
-// PACK: additionally emit the packed int32 words (sym only, G % 8 == 0 handled by the caller).
+// One wavefront per group, lanes stride its elements: any dtype, any block (BM, BN) -- a group is a BM x BN tile of
+// the matrix, rows and columns past the edge count as 0 in the extrema -- symmetric and asymmetric.
 __global__ __launch_bounds__(256) void int4_fake_generic_kernel(const void* __restrict__ x, int dtype,
                                                                 void* __restrict__ out, void* __restrict__ scale_out,
                                                                 void* __restrict__ zero_out, int64_t M, int64_t N,
-                                                                int G, int64_t groups_per_row, int sym) {
+                                                                int BM, int BN, int64_t groups_per_row, int64_t total,
+                                                                int sym) {
     const int lane = threadIdx.x & 63;
     const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
-    const int64_t total = M * groups_per_row;
+    const int elems = BM * BN;
     for (int64_t g = wave; g < total; g += nwaves) {
-        const int64_t r = g / groups_per_row, j = g - r * groups_per_row;
-        const int64_t c0 = j * G;
+        const int64_t bi = g / groups_per_row, bj = g - bi * groups_per_row;
+        const int64_t r0 = bi * BM, c0 = bj * BN;
         float mx = -__builtin_inff(), mn = __builtin_inff();
-        for (int k = lane; k < G; k += 64) {
-            const int64_t c = c0 + k;
-            const float val = c < N ? load_f32(x, r * N + c, dtype) : 0.0f;
+        for (int k = lane; k < elems; k += 64) {
+            const int64_t r = r0 + k / BN, c = c0 + k % BN;
+            const float val = (r < M && c < N) ? load_f32(x, r * N + c, dtype) : 0.0f;
             if (sym) mx = __builtin_fmaxf(mx, __builtin_fabsf(val));
             else { mx = __builtin_fmaxf(mx, val); mn = __builtin_fminf(mn, val); }
         }
@@ -113,9 +114,9 @@ __global__ __launch_bounds__(256) void int4_fake_generic_kernel(const void* __re
             // max(-0, +0) is +0 in the reference's device code: adding +0 makes that explicit
             zero = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
         }
-        for (int k = lane; k < G; k += 64) {
-            const int64_t c = c0 + k;
-            if (c < N) {
+        for (int k = lane; k < elems; k += 64) {
+            const int64_t r = r0 + k / BN, c = c0 + k % BN;
+            if (r < M && c < N) {
                 float qv = __builtin_rintf(load_f32(x, r * N + c, dtype) / s);
                 if (!sym) qv = qv + zero;
                 store_dtype(out, r * N + c, qv, dtype);
@@ -424,17 +425,18 @@ __global__ __launch_bounds__(256) void int4_unpack_generic_kernel(const uint32_t
 using namespace mq;
 
 extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
-                                  int group, int sym, void* stream) {
+                                  int block_m, int block_n, int sym, void* stream) {
     if (!x || !out || !scale || (!sym && !zero)) return mq_fail(MQ_ERR_ARG, "null pointer");
-    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || N < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
-    if (group % 32 != 0) return mq_fail(MQ_ERR_ARG, "block_m * block_n must be divisible by 32");
+    if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || N < 0 || block_m <= 0 || block_n <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
+    if (((int64_t)block_m * block_n) % 32 != 0 || (int64_t)block_m * block_n > (1 << 24))
+        return mq_fail(MQ_ERR_ARG, "block_m * block_n must be divisible by 32");
     if (M == 0 || N == 0) return MQ_OK;
-    const int64_t gpr = (N + group - 1) / group;
-    const int64_t waves = M * gpr;
+    const int64_t gpr = (N + block_n - 1) / block_n;
+    const int64_t waves = ((M + block_m - 1) / block_m) * gpr;
     int64_t blocks = (waves + 3) / 4;
     if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
     hipLaunchKernelGGL(int4_fake_generic_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, dtype,
-                       out, scale, zero, M, N, group, gpr, sym);
+                       out, scale, zero, M, N, block_m, block_n, gpr, waves, sym);
     return mq_check_launch("int4 fake quant");
 }
 

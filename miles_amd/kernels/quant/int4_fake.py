@@ -24,16 +24,14 @@ def fake_int4_quant_cuda(x: torch.Tensor, block_size, sym: bool):
     if (block_m * block_n) % 32 != 0:
         raise RuntimeError(f"block_m * block_n ({block_m * block_n}) must be divisible by 32. "
                            f"But got a {block_m}x{block_n} block.")
-    if block_m != 1:
-        raise RuntimeError(f"only (1, G) blocks are implemented on gfx950, got {block_m}x{block_n}")
     M, N = x.shape
     xc = x.contiguous()
     out = torch.empty_like(xc)
-    scale = torch.empty((M, -(-N // block_n)), dtype=x.dtype, device=x.device)
+    scale = torch.empty((-(-M // block_m), -(-N // block_n)), dtype=x.dtype, device=x.device)
     zero = torch.empty_like(scale)  # left unwritten in symmetric mode, as in the reference
     launch.note_direct_call()
     rc = _lib.load().mq_int4_fake_quant(xc.data_ptr(), _lib.dtype_code(x, "fake_int4_quant_cuda"), out.data_ptr(),
-                                        scale.data_ptr(), zero.data_ptr(), M, N, block_n, int(bool(sym)),
+                                        scale.data_ptr(), zero.data_ptr(), M, N, block_m, block_n, int(bool(sym)),
                                         _lib.stream_ptr(x.device))
     _lib.check(rc, RuntimeError)
     return out, scale, zero

@@ -494,20 +494,22 @@ void mqo_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, int64_t
  *             zero  = clamp(-rintf(min/scale), 0, 15); out = rintf(x/scale)+zero
  * out/scale/zero are stored in the input dtype (.cu:251-254).  Columns past N
  * in a ragged last group read as 0 (.cu:209-213). */
-void mqo_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int G, int sym,
-                         void* out, void* scale_out, void* zero_out) {
+/* General block (BM, BN): a group is a BM x BN tile of the matrix, rows and columns past the edge read as 0
+ * (.cu:95-150 for (32,1), :159-259 for the rest); one scale / zero per tile, shape [ceil(M/BM), ceil(N/BN)]. */
+void mqo_int4_fake_quant_block(const void* x, int dtype, int64_t M, int64_t N, int BM, int BN, int sym,
+                               void* out, void* scale_out, void* zero_out) {
     const float SYM = 1.0f / 7.0f, ASYM = 1.0f / 15.0f;
-    int64_t ng = (N + G - 1) / G;
-#pragma omp parallel for schedule(static)
-    for (int64_t r = 0; r < M; r++)
-        for (int64_t j = 0; j < ng; j++) {
-            int64_t c0 = j * G, c1 = c0 + G < N ? c0 + G : N;
+    int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int64_t bi = 0; bi < gm; bi++)
+        for (int64_t bj = 0; bj < gn; bj++) {
             float mx = -INFINITY, mn = INFINITY;
-            for (int64_t c = c0; c < c0 + G; c++) {
-                float v = c < N ? load_as_f32(x, r * N + c, dtype) : 0.0f;
-                if (sym) mx = fmaxf(mx, fabsf(v));
-                else { mx = fmaxf(mx, v); mn = fminf(mn, v); }
-            }
+            for (int64_t r = bi * BM; r < (bi + 1) * BM; r++)
+                for (int64_t c = bj * BN; c < (bj + 1) * BN; c++) {
+                    float v = (r < M && c < N) ? load_as_f32(x, r * N + c, dtype) : 0.0f;
+                    if (sym) mx = fmaxf(mx, fabsf(v));
+                    else { mx = fmaxf(mx, v); mn = fminf(mn, v); }
+                }
             float scale, zero = 0.0f;
             if (sym) scale = fmaxf(mx * SYM, 1e-5f);
             else {
@@ -517,21 +519,26 @@ void mqo_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int G, 
                  * may return either zero) */
                 if (zero == 0.0f) zero = 0.0f;
             }
-            for (int64_t c = c0; c < c1; c++) {
-                float v = rintf(load_as_f32(x, r * N + c, dtype) / scale); /* keeps -0 */
-                if (!sym) v = v + zero;
-                if (dtype == MQ_F32) ((float*)out)[r * N + c] = v;
-                else ((uint16_t*)out)[r * N + c] = dtype == MQ_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
-            }
+            for (int64_t r = bi * BM; r < (bi + 1) * BM && r < M; r++)
+                for (int64_t c = bj * BN; c < (bj + 1) * BN && c < N; c++) {
+                    float v = rintf(load_as_f32(x, r * N + c, dtype) / scale); /* keeps -0 */
+                    if (!sym) v = v + zero;
+                    if (dtype == MQ_F32) ((float*)out)[r * N + c] = v;
+                    else ((uint16_t*)out)[r * N + c] = dtype == MQ_BF16 ? f32_to_bf16(v) : f32_to_f16(v);
+                }
+            int64_t g = bi * gn + bj;
             if (dtype == MQ_F32) {
-                ((float*)scale_out)[r * ng + j] = scale;
-                if (!sym) ((float*)zero_out)[r * ng + j] = zero;
+                ((float*)scale_out)[g] = scale;
+                if (!sym) ((float*)zero_out)[g] = zero;
             } else {
-                ((uint16_t*)scale_out)[r * ng + j] = dtype == MQ_BF16 ? f32_to_bf16(scale) : f32_to_f16(scale);
-                if (!sym)
-                    ((uint16_t*)zero_out)[r * ng + j] = dtype == MQ_BF16 ? f32_to_bf16(zero) : f32_to_f16(zero);
+                ((uint16_t*)scale_out)[g] = dtype == MQ_BF16 ? f32_to_bf16(scale) : f32_to_f16(scale);
+                if (!sym) ((uint16_t*)zero_out)[g] = dtype == MQ_BF16 ? f32_to_bf16(zero) : f32_to_f16(zero);
             }
         }
+}
+void mqo_int4_fake_quant(const void* x, int dtype, int64_t M, int64_t N, int G, int sym,
+                         void* out, void* scale_out, void* zero_out) {
+    mqo_int4_fake_quant_block(x, dtype, M, N, 1, G, sym, out, scale_out, zero_out);
 }
 
 /* pack_layer(weight, G, sym=True)

@@ -65,6 +65,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_mxfp8.argtypes = [vp, i32, i64, i64, vp, vp]
         L.mqo_int4_fake_quant.restype = None
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
+        L.mqo_int4_fake_quant_block.restype = None
+        L.mqo_int4_fake_quant_block.argtypes = [vp, i32, i64, i64, i32, i32, i32, vp, vp, vp]
         L.mqo_int4_unpack_dequant.restype = None
         L.mqo_int4_unpack_dequant.argtypes = [vp, vp, i32, i64, i64, i32, vp]
         L.mqo_mxfp4_to_fp8_block.restype = None
@@ -196,17 +198,17 @@ def mxfp8_quantize(weight: torch.Tensor):
 # INT4
 # --------------------------------------------------------------------------
 def fake_int4_quant(x: torch.Tensor, block_size, sym: bool):
-    """fake_int4_quant_cuda.cu:319-364 for block (1, G) -> (out, scale, zero) in x.dtype."""
+    """fake_int4_quant_cuda.cu:319-364 for block (BM, BN) -> (out, scale, zero) in x.dtype."""
     _check_cpu(x)
-    assert x.dim() == 2 and int(block_size[0]) == 1
+    assert x.dim() == 2
     x = x.contiguous()
-    G = int(block_size[1])
+    BM, BN = int(block_size[0]), int(block_size[1])
     M, N = x.shape
     out = torch.empty_like(x)
-    scale = torch.empty((M, ceil_div(N, G)), dtype=x.dtype)
+    scale = torch.empty((ceil_div(M, BM), ceil_div(N, BN)), dtype=x.dtype)
     zero = torch.zeros_like(scale)
-    lib().mqo_int4_fake_quant(x.data_ptr(), _DTYPE[x.dtype], M, N, G, int(sym), out.data_ptr(),
-                              scale.data_ptr(), zero.data_ptr())
+    lib().mqo_int4_fake_quant_block(x.data_ptr(), _DTYPE[x.dtype], M, N, BM, BN, int(sym), out.data_ptr(),
+                                    scale.data_ptr(), zero.data_ptr())
     return out, scale, zero
 
 

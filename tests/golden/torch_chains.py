@@ -279,3 +279,25 @@ def torch_nvfp4_4over6(w, amax=None, e4m3_max=448, mse=False, fp16_error=False):
     code = torch.where(pick4.unsqueeze(-1), c4, c6).reshape(m, k)
     s8 = torch.where(pick4.unsqueeze(-1), s4.view(torch.uint8), s6.view(torch.uint8)).view(F8)
     return code[:, 0::2] | (code[:, 1::2] << 4), s8.reshape(m, k // 16)
+
+
+def torch_fake_int4_block(x, bm, bn, sym):
+    """fake_int4_quant_cuda.cu for a general (bm, bn) block (:95-150 for (32,1), :159-259): tiles of the zero-padded
+    matrix, fp32 arithmetic, outputs in the dtype of x."""
+    m, n = x.shape
+    gm, gn = -(-m // bm), -(-n // bn)
+    xf = torch.zeros((gm * bm, gn * bn), dtype=torch.float32)
+    xf[:m, :n] = x.float()
+    t = xf.reshape(gm, bm, gn, bn)
+    if sym:
+        amax = t.abs().amax(dim=(1, 3), keepdim=True)
+        scale = torch.maximum(amax * torch.tensor(1.0 / 7.0, dtype=torch.float32), torch.tensor(1e-5, dtype=torch.float32))
+        zero = torch.zeros_like(scale)
+        out = torch.round(t / scale)
+    else:
+        mx, mn = t.amax(dim=(1, 3), keepdim=True), t.amin(dim=(1, 3), keepdim=True)
+        scale = torch.maximum((mx - mn) * torch.tensor(1.0 / 15.0, dtype=torch.float32), torch.tensor(1e-5, dtype=torch.float32))
+        zero = torch.clamp(-torch.round(mn / scale), 0.0, 15.0) + 0.0
+        out = torch.round(t / scale) + zero
+    out = out.reshape(gm * bm, gn * bn)[:m, :n]
+    return out.to(x.dtype), scale.reshape(gm, gn).to(x.dtype), zero.reshape(gm, gn).to(x.dtype)

@@ -829,3 +829,21 @@ def test_nvfp4_four_over_six_qdq_and_other_dtypes(oracle, monkeypatch, dtype, e4
     q_o, s_o, g_o = oracle.nvfp4_quantize_1d(xf, e4m3_max=e4m3_max, flags=flags)
     _assert_same(s, s_o, "block scales (generic kernel)")
     _assert_same(q, q_o, "codes (generic kernel)")
+
+
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("shape,block", [((64, 96), (32, 1)), ((70, 33), (32, 1)), ((16, 64), (4, 8)), ((18, 40), (2, 16)),
+                                          ((40, 64), (8, 32)), ((5, 200), (1, 64)), ((256, 512), (32, 1))])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fake_int4_quant_general_blocks(oracle, shape, block, sym, dtype):
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
+
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.001, gain=30.0, seed=4003, dtype=dtype)
+    w[0] = 0
+    out, scale, zero = fake_int4_quant_cuda(w.to(DEV), block, sym)
+    out_o, scale_o, zero_o = oracle.fake_int4_quant(w, block, sym)
+    assert scale.shape == (-(-shape[0] // block[0]), -(-shape[1] // block[1]))
+    _assert_same(out, out_o, "values")
+    _assert_same(scale, scale_o, "scales")
+    if not sym:
+        _assert_same(zero, zero_o, "zero points")

@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_fake_int4_block, torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -640,3 +640,19 @@ def test_nvfp4_four_over_six_matches_torch_chain(oracle, shape, kind, e4m3_max, 
         # both candidates are really in play, and the chosen one never has the larger error
         q6, s6, _ = oracle.nvfp4_quantize_1d(w, e4m3_max=e4m3_max)
         assert 0 < (s.view(torch.uint8) != s6.view(torch.uint8)).sum() < s.numel()
+
+
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("shape,block", [((64, 96), (32, 1)), ((70, 33), (32, 1)), ((16, 64), (4, 8)), ((18, 40), (2, 16)),
+                                          ((8, 96), (1, 32)), ((40, 64), (8, 32)), ((5, 200), (1, 64))])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_int4_fake_quant_general_blocks_match_torch_chain(oracle, shape, block, sym, dtype):
+    w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.001, gain=30.0, seed=4003, dtype=dtype)
+    w[0] = 0
+    out, scale, zero = oracle.fake_int4_quant(w, block, sym)
+    out_t, scale_t, zero_t = torch_fake_int4_block(w, block[0], block[1], sym)
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    assert scale.shape == (-(-shape[0] // block[0]), -(-shape[1] // block[1]))
+    assert torch.equal(out.view(bits), out_t.view(bits)) and torch.equal(scale.view(bits), scale_t.view(bits))
+    if not sym:
+        assert torch.equal(zero.view(bits), zero_t.view(bits))
