@@ -60,6 +60,12 @@ int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* s
  *   x [M,N] e4m3fn contiguous; s [ceil(M/block), ceil(N/block)] fp32; y [M,N] bf16 */
 int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block, void* stream);
 
+/* per_block_cast_to_fp8(x)                           SGLang (third party; called at .../processors/quantizer_fp8.py:139-147)
+ *   128x128 tiles, power-of-two fp32 scale 2^ceil(log2(max(amax, 1e-4) / 448)), q = e4m3(x / scale); shapes as
+ *   mq_fp8_block_quant.  Restated from the published source: parity with SGLang itself is not pinned. */
+int mq_fp8_block_quant_pow2(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
+                            void* stream);
+
 /* mxfp8_quantize(weight)                             miles/utils/mxfp8.py:51-78
  *   w [rows,K] contiguous, K % 32 == 0; q [rows,K] e4m3fn; scale [rows,K/32] E8M0 bytes */
 int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K, void* stream);
@@ -164,6 +170,7 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *                                                                          aux2 = fp32 weight_scale_2
  *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *   MQ_JOB_COPY                 bytes         bytes         -              -                           -
+ *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
  *     (rows * cols bytes copied verbatim: how a pass-through tensor reaches its place in a packed transport bucket,
  *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
@@ -178,7 +185,8 @@ enum {
     MQ_JOB_INT4_PACK = 4,
     MQ_JOB_NVFP4 = 5,
     MQ_JOB_MXFP4 = 6,
-    MQ_JOB_COPY = 7
+    MQ_JOB_COPY = 7,
+    MQ_JOB_FP8_BLOCK_POW2 = 8
 };
 typedef struct mq_job {
     int32_t kind;

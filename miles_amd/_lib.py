@@ -22,6 +22,7 @@ _vp, _i64, _i32, _f32, _u32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_float, _c.
 # symbol -> argtypes; every function returns int except the two noted below
 SIGNATURES = {
     "mq_fp8_block_quant": [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
+    "mq_fp8_block_quant_pow2": [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _vp],
     "mq_fp8_blockwise_cast": [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
     "mq_fp8_scaled_quant": [_vp, _i32, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _vp],
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
@@ -47,7 +48,7 @@ SIGNATURES = {
 NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
- JOB_COPY) = range(8)
+ JOB_COPY, JOB_FP8_BLOCK_POW2) = range(9)
 
 
 class Job(_c.Structure):

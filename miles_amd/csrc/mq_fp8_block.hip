@@ -4,6 +4,9 @@
 //                                tile has scale 0 and every byte 0xFF   (reference: tools/convert_hf_to_fp8.py:39-70)
 //   mode 1  "fp8_blockwise_cast" absmax = max(amax,1e-10), x_s = absmax/448, q = e4m3(clamp(x * (1/x_s)))
 //                                                                       (reference: miles/kernels/quant/fp8_blockwise.py:43-58)
+//   mode 2  "per_block_cast_to_fp8" (power-of-two scales) absmax = max(amax,1e-4), sf = 2^ceil(log2(absmax/448)),
+//                                q = e4m3(x * (1/sf)).  SGLang's function (third party, not in the reference tree; called at
+//                                .../processors/quantizer_fp8.py:139-147); restated from its published source
 //   dequant y = bf16(float(q) * s[i/B][j/B])                            (reference: tools/fp8_cast_bf16.py:15-40)
 //
 // Fast path (bf16, 128x128 tiles, 16-byte aligned rows): one 256-lane workgroup owns one tile.  Lane t
@@ -22,6 +25,14 @@ constexpr int kTileThreads = 512;                       // 8 wavefronts per 128x
 constexpr int kRowsPerThread = 2048 / kTileThreads;     // 16-byte row segments per lane
 constexpr int kRowStep = kTileThreads / 16;             // tile rows covered per pass of the workgroup
 constexpr int kTileWaves = kTileThreads / kWave;
+
+// 2^ceil(log2 v) for a normal positive v (the floor of 1e-4 / 448 keeps it normal): exponent, plus one when the
+// mantissa is not zero.  For bf16 / fp16 inputs this is what pow(2, ceil(log2(v))) evaluates to in floating point
+// as well: v is either an exact power of two or far from one.
+__device__ __forceinline__ float ceil_pow2_scale(float v) {
+    const uint32_t u = f2u(v);
+    return u2f(((u >> 23) + ((u & 0x7FFFFFu) != 0)) << 23);
+}
 
 template <int MODE>
 __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTable tab) {
@@ -71,7 +82,8 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
 
     float s;
     if (MODE == 0) s = amax / kFp8Max;
-    else s = (amax > 1e-10f ? amax : 1e-10f) / kFp8Max;
+    else if (MODE == 1) s = (amax > 1e-10f ? amax : 1e-10f) / kFp8Max;
+    else s = ceil_pow2_scale((amax > 1e-4f ? amax : 1e-4f) / kFp8Max);
     const float y = 1.0f / s;
     if (t == 0) job.scale[tile] = s;
 
@@ -84,7 +96,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
         }
         return;
     }
-    const bool fast_div = (MODE == 1) || shared_div_ok(s);
+    const bool fast_div = (MODE != 0) || shared_div_ok(s);
 
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; i++) {
@@ -94,7 +106,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             // |w/s| <= 448 (1 + 2^-22): no clamp is needed, the convert rounds anything up to 464 to 448
-            if (MODE == 1) f[j] = f[j] * y;
+            if (MODE != 0) f[j] = f[j] * y;
             else f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
         }
         u32x2 o;
@@ -139,9 +151,12 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
     if (MODE == 0) {
         s = amax / kFp8Max;
         y = 0.0f;
-    } else {
+    } else if (MODE == 1) {
         const float absmax = amax > 1e-10f ? amax : 1e-10f;
         s = absmax / kFp8Max;
+        y = 1.0f / s;
+    } else {
+        s = ceil_pow2_scale((amax > 1e-4f ? amax : 1e-4f) / kFp8Max);
         y = 1.0f / s;
     }
     if (t == 0) scale[tile] = s;
@@ -153,7 +168,7 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
             if (zero_tile) code = 0xFFu;
             else {
                 const float x = load_f32(w, r * sxm + c * sxn, dtype);
-                float v = MODE == 1 ? x * y : x / s;
+                float v = MODE != 0 ? x * y : x / s;
                 v = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
                 code = sw_e4m3fn(v);
             }
@@ -313,7 +328,8 @@ int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
     seal_table(tab);
     const int64_t grid = xcd_grid(tiles);
     if (mode == 0) hipLaunchKernelGGL(fp8_block128_kernel<0>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
-    else hipLaunchKernelGGL(fp8_block128_kernel<1>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    else if (mode == 1) hipLaunchKernelGGL(fp8_block128_kernel<1>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    else hipLaunchKernelGGL(fp8_block128_kernel<2>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
     return mq_check_launch("fp8 block quant");
 }
 
@@ -337,8 +353,11 @@ static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int
     if (mode == 0)
         hipLaunchKernelGGL(fp8_block_generic_kernel<0>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K, scale,
                            M, K, bm, bk, (int)tiles_k);
-    else
+    else if (mode == 1)
         hipLaunchKernelGGL(fp8_block_generic_kernel<1>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K, scale,
+                           M, K, bm, bk, (int)tiles_k);
+    else
+        hipLaunchKernelGGL(fp8_block_generic_kernel<2>, grid, blk, 0, stream, w, dtype, sxm, sxn, (uint8_t*)q, K, scale,
                            M, K, bm, bk, (int)tiles_k);
     return mq_check_launch("fp8 block quant");
 }
@@ -351,6 +370,11 @@ extern "C" int mq_fp8_block_quant(const void* w, int dtype, int64_t ldw, void* q
 extern "C" int mq_fp8_blockwise_cast(const void* x, int dtype, int64_t stride_m, int64_t stride_n, void* y, float* s,
                                      int64_t M, int64_t N, int block_m, int block_n, void* stream) {
     return fp8_block_launch(1, x, dtype, stride_m, stride_n, y, s, M, N, block_m, block_n, (hipStream_t)stream);
+}
+
+extern "C" int mq_fp8_block_quant_pow2(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
+                                       void* stream) {
+    return fp8_block_launch(2, w, dtype, ldw, 1, q, scale, M, K, kTile, kTile, (hipStream_t)stream);
 }
 
 extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws,

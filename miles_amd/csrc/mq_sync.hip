@@ -42,6 +42,7 @@ static bool job_fast(const mq_job& j) {
     switch (j.kind) {
         case MQ_JOB_FP8_BLOCK:
         case MQ_JOB_FP8_BLOCKWISE_CAST:
+        case MQ_JOB_FP8_BLOCK_POW2:
             return mq_fp8_tile_fast_ok(j.in, j.dtype, j.ld, 1, j.out, j.rows, j.cols, j.p0, j.p1) &&
                    (j.block_stride % 8) == 0;
         case MQ_JOB_FP8_DEQUANT:
@@ -62,14 +63,14 @@ static bool job_fast(const mq_job& j) {
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_COPY) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_FP8_BLOCK_POW2) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     if (j.kind == MQ_JOB_COPY) return MQ_OK;
     if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
     if (j.rows_per_block != 0) {
-        const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST;
+        const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST || j.kind == MQ_JOB_FP8_BLOCK_POW2;
         if (!fp8q || j.rows_per_block < 0 || j.rows_per_block % 128 != 0 || j.p0 != 128 || j.p1 != 128 || j.dtype != MQ_BF16)
             return mq_fail(MQ_ERR_ARG, "row-blocked input needs a bf16 FP8 128x128 job with rows_per_block % 128 == 0");
     }
@@ -83,6 +84,9 @@ static int run_single(const mq_job& j, void* stream) {
         case MQ_JOB_FP8_BLOCKWISE_CAST:
             return mq_fp8_blockwise_cast(j.in, j.dtype, j.ld, 1, j.out, (float*)j.scale, j.rows, j.cols, j.p0, j.p1,
                                          stream);
+        case MQ_JOB_FP8_BLOCK_POW2:
+            if (j.p0 != 128 || j.p1 != 128) return mq_fail(MQ_ERR_ARG, "power-of-two FP8 scales use 128x128 blocks");
+            return mq_fp8_block_quant_pow2(j.in, j.dtype, j.ld, j.out, (float*)j.scale, j.rows, j.cols, stream);
         case MQ_JOB_FP8_DEQUANT:
             return mq_fp8_block_dequant(j.in, (const float*)j.aux, j.out, j.rows, j.cols, j.p0, stream);
         case MQ_JOB_MXFP8:
@@ -190,7 +194,8 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
             continue;
         }
         // flat kinds run on a (largest tensor) x (tensors) grid: keep the padding of a group under 25 %
-        const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST && head.kind != MQ_JOB_COPY;
+        const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST &&
+                          head.kind != MQ_JOB_FP8_BLOCK_POW2 && head.kind != MQ_JOB_COPY;
         int64_t j = i + 1, sum = head.rows * head.cols, mx = sum;
         while (j < n && j - i < kMaxGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
                jobs[j].cols > 0) {
@@ -205,7 +210,8 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
         int rc = MQ_OK;
         switch (head.kind) {
             case MQ_JOB_FP8_BLOCK:
-            case MQ_JOB_FP8_BLOCKWISE_CAST: {
+            case MQ_JOB_FP8_BLOCKWISE_CAST:
+            case MQ_JOB_FP8_BLOCK_POW2: {
                 TileTable tab{};
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) {
@@ -213,7 +219,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                     tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, jb.ld, (int32_t)jb.rows, (int32_t)jb.cols, 0,
                                          (int32_t)(jb.rows_per_block / 128), jb.block_stride};
                 }
-                rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : 1, tab, st);
+                rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2, tab, st);
                 break;
             }
             case MQ_JOB_FP8_DEQUANT: {

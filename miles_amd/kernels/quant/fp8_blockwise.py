@@ -54,3 +54,32 @@ def fp8_blockwise_cast(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, 
                                                _lib.stream_ptr(x.device))
         _lib.check(rc)
     return y, s
+
+
+def per_block_cast_to_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """x [M, N] -> (float8_e4m3fn [M, N], float32 [ceil(M/128), ceil(N/128)]) with power-of-two scales.
+
+    Stands in for SGLang's `per_block_cast_to_fp8` (sglang.srt.layers.quantization.fp8_utils; imported at
+    miles/backends/megatron_utils/sglang.py:9-12 and called at .../processors/quantizer_fp8.py:139-147 when
+    NVTE_FP8_BLOCK_SCALING_FP32_SCALES=0).  Its source is not part of the reference tree; the published algorithm is
+    restated: per 128x128 tile amax = max(max|x|, 1e-4), sf = 2^ceil(log2(amax / 448)), y = e4m3(x * (1 / sf)).
+    Also accepts the row-blocked 3-D views of `fp8_blockwise_cast`.
+    """
+    _lib.require_gpu(x, "per_block_cast_to_fp8")
+    _lib.dtype_code(x, "per_block_cast_to_fp8")
+    rpb, bstride = 0, 0
+    if x.dim() == 3:
+        B, R, N = x.shape
+        if x.stride(2) == 1 and x.stride(1) == N and R % 128 == 0 and x.dtype == torch.bfloat16:
+            rpb, bstride, M, ld = R, x.stride(0), B * R, N
+        else:
+            x = x.reshape(B * R, N)
+    if x.dim() != 3:
+        assert x.dim() == 2
+        if x.stride(1) != 1 and x.shape[1] > 1:
+            x = x.contiguous()
+        (M, N), ld = x.shape, x.stride(0)
+    y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
+    s = torch.empty(ceil_div(M, 128), ceil_div(N, 128), dtype=torch.float32, device=x.device)
+    launch.submit(_lib.JOB_FP8_BLOCK_POW2, x, y, s, None, None, M, N, ld, 128, 128, rpb, bstride)
+    return y, s

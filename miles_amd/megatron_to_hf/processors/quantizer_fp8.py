@@ -15,7 +15,7 @@ import os
 
 import torch
 
-from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
 from miles_amd.tools.convert_hf_to_fp8 import tensor_fp8
 
 from ._names import parse_layer_param
@@ -123,9 +123,9 @@ def _quantize_param(args, name, weight, weight_block_size, ignored_layers, packe
             raise NotImplementedError("UE8M0 (DeepGEMM) FP8 scales come from SGLang's quant_weight_ue8m0, "
                                       "which this library does not provide")
         if os.environ.get("NVTE_FP8_BLOCK_SCALING_FP32_SCALES", "1") == "0" and list(weight_block_size) == [128, 128]:
-            raise NotImplementedError("NVTE_FP8_BLOCK_SCALING_FP32_SCALES=0 selects SGLang's per_block_cast_to_fp8 "
-                                      "(power-of-two scales), which this library does not provide")
-        qweight, scale = fp8_blockwise_cast(weight, weight_block_size)
+            qweight, scale = per_block_cast_to_fp8(weight)      # power-of-two scales, kept as fp32
+        else:
+            qweight, scale = fp8_blockwise_cast(weight, weight_block_size)
         return [(name, qweight), (name.replace(".weight", ".weight_scale_inv"), scale)]
     # per-tensor: scale = max(amax, 1e-12) / 448 with the quotient kept in the weight's dtype
     qweight, scale = tensor_fp8(weight)

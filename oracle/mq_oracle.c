@@ -301,6 +301,32 @@ void mqo_fp8_blockwise_cast(const void* x, int dtype, int64_t M, int64_t N,
     }
 }
 
+/* per_block_cast_to_fp8 (SGLang, sglang.srt.layers.quantization.fp8_utils; third party, pinned by the reference
+ * at sglang v0.5.x and absent from its tree -- PARITY UNPINNED; called at
+ * miles/backends/megatron_utils/megatron_to_hf/processors/quantizer_fp8.py:139-147).  Published algorithm:
+ *   x_amax = max|f32(x)| over the zero-padded 128x128 tile, clamped below at 1e-4
+ *   sf     = 2 ^ ceil(log2(x_amax / 448))
+ *   y      = e4m3(f32(x) * (1 / sf))
+ * x row-major with row stride ld. */
+void mqo_fp8_block_pow2(const void* x, int dtype, int64_t M, int64_t N, int64_t ld, uint8_t* y, float* S) {
+    int64_t nt = (M + 127) / 128, kt = (N + 127) / 128;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t ti = 0; ti < nt; ti++)
+        for (int64_t tj = 0; tj < kt; tj++) {
+            int64_t r0 = ti * 128, r1 = r0 + 128 < M ? r0 + 128 : M;
+            int64_t c0 = tj * 128, c1 = c0 + 128 < N ? c0 + 128 : N;
+            float amax = 0.0f;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) amax = fmaxf(amax, fabsf(load_as_f32(x, r * ld + c, dtype)));
+            if (amax < 1e-4f) amax = 1e-4f;
+            float sf = powf(2.0f, ceilf(log2f(amax / 448.0f)));
+            float inv = 1.0f / sf;
+            S[ti * kt + tj] = sf;
+            for (int64_t r = r0; r < r1; r++)
+                for (int64_t c = c0; c < c1; c++) y[r * N + c] = mqo_f32_to_e4m3fn(load_as_f32(x, r * ld + c, dtype) * inv);
+        }
+}
+
 /* ------------------------------------------------------------------ */
 /* A-5  FP8 block dequant (tools/fp8_cast_bf16.py:15-40;               */
 /*      tools/convert_mimo_v2_to_bf16.py:44-47)                        */

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_fp8_per_tensor_or_channel.argtypes = [vp, i32, i64, i64, i64, i32, f32, vp, vp]
         L.mqo_fp8_blockwise_cast.restype = None
         L.mqo_fp8_blockwise_cast.argtypes = [vp, i32, i64, i64, i64, i64, i32, i32, vp, vp]
+        L.mqo_fp8_block_pow2.restype = None
+        L.mqo_fp8_block_pow2.argtypes = [vp, i32, i64, i64, i64, vp, vp]
         L.mqo_fp8_block_dequant.restype = None
         L.mqo_fp8_block_dequant.argtypes = [vp, vp, i64, i64, i32, vp]
         L.mqo_mxfp8.restype = None
@@ -164,6 +166,17 @@ def fp8_blockwise_cast(x: torch.Tensor, block_size=None):
     s = torch.empty((ceil_div(M, bm), ceil_div(N, bn)), dtype=torch.float32)
     lib().mqo_fp8_blockwise_cast(x.data_ptr(), _DTYPE[x.dtype], M, N, x.stride(0), x.stride(1), bm, bn,
                                  y.data_ptr(), s.data_ptr())
+    return y.view(torch.float8_e4m3fn), s
+
+
+def per_block_cast_to_fp8(x: torch.Tensor):
+    """SGLang's per_block_cast_to_fp8 (power-of-two scales), restated: parity unpinned."""
+    _check_cpu(x)
+    assert x.dim() == 2 and (x.stride(1) == 1 or x.shape[1] <= 1)
+    M, N = x.shape
+    y = torch.empty((M, N), dtype=torch.uint8)
+    s = torch.empty((ceil_div(M, 128), ceil_div(N, 128)), dtype=torch.float32)
+    lib().mqo_fp8_block_pow2(x.data_ptr(), _DTYPE[x.dtype], M, N, x.stride(0), y.data_ptr(), s.data_ptr())
     return y.view(torch.float8_e4m3fn), s
 
 

@@ -301,3 +301,17 @@ def torch_fake_int4_block(x, bm, bn, sym):
         out = torch.round(t / scale) + zero
     out = out.reshape(gm * bm, gn * bn)[:m, :n]
     return out.to(x.dtype), scale.reshape(gm, gn).to(x.dtype), zero.reshape(gm, gn).to(x.dtype)
+
+
+def torch_per_block_cast_to_fp8(x):
+    """SGLang's per_block_cast_to_fp8 as published (third party; its source is not in the reference tree):
+    zero-padded 128x128 tiles, amax clamped at 1e-4, sf = 2^ceil(log2(amax / 448)), x * (1 / sf) cast to e4m3."""
+    m, n = x.shape
+    pm, pn = -(-m // 128) * 128, -(-n // 128) * 128
+    x_padded = torch.zeros((pm, pn), dtype=x.dtype)
+    x_padded[:m, :n] = x
+    x_view = x_padded.view(-1, 128, pn // 128, 128)
+    x_amax = x_view.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    sf = torch.pow(2.0, torch.ceil(torch.log2((x_amax / 448.0).abs())))
+    x_scaled = (x_view * (1.0 / sf)).to(F8)
+    return x_scaled.view_as(x_padded)[:m, :n].contiguous(), sf.view(x_view.size(0), x_view.size(2))

@@ -351,3 +351,20 @@ def test_packed_buckets_int4_moe_two_syncs(oracle):
             expect = [next(it) for _ in b]
             assert [n for n, _ in b] == [n for n, _ in expect]
             assert torch.equal(b.flat.cpu(), _payload_bytes(expect)), f"payload of a bucket differs (seed {seed})"
+
+
+def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
+    # NVTE_FP8_BLOCK_SCALING_FP32_SCALES=0 routes the block cast through per_block_cast_to_fp8 (quantizer_fp8.py:139-147)
+    monkeypatch.setenv("NVTE_FP8_BLOCK_SCALING_FP32_SCALES", "0")
+    cpu = _dense_model(60)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None)
+    for _ in range(2):      # recorded plan, then its replay
+        flat = dict(nt for b in _run(upd) for nt in b)
+        for name, param in cpu.items():
+            for hf, t in name_maps.convert_qwen2_to_hf(ARGS, name, param):
+                if hf.endswith("_proj.weight"):
+                    q, s = oracle.per_block_cast_to_fp8(t.contiguous())
+                    _same(flat[hf], q, hf)
+                    _same(flat[hf.replace(".weight", ".weight_scale_inv")], s, hf + " scale")
+    assert upd._plan is not None and upd._plan.replayable

@@ -847,3 +847,24 @@ def test_fake_int4_quant_general_blocks(oracle, shape, block, sym, dtype):
     _assert_same(scale, scale_o, "scales")
     if not sym:
         _assert_same(zero, zero_o, "zero points")
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(130, 257), (256, 384), (4096, 2560)])
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_fp8_power_of_two_scales(oracle, shape, kind):
+    from miles_amd.kernels.quant.fp8_blockwise import per_block_cast_to_fp8
+
+    if shape[0] > 1000 and kind != "random":
+        pytest.skip("the full-size tensor is checked on random data")
+    x = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    y, s = per_block_cast_to_fp8(x.to(DEV))
+    y_o, s_o = oracle.per_block_cast_to_fp8(x)
+    assert y.dtype == torch.float8_e4m3fn and s.dtype == torch.float32
+    _assert_same(s, s_o, "scales")
+    _assert_same(y, y_o, "codes")
+    if shape == (256, 384):     # fp32 input and a row-strided view take the generic kernel
+        xf = torch.cat((x.float(), x.float()), dim=1)[:, :384]
+        y2, s2 = per_block_cast_to_fp8(xf.to(DEV))
+        y2_o, s2_o = oracle.per_block_cast_to_fp8(xf)
+        _assert_same(s2, s2_o, "scales (fp32, strided)")
+        _assert_same(y2, y2_o, "codes (fp32, strided)")

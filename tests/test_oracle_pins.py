@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_fake_int4_block, torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_per_block_cast_to_fp8, torch_fake_int4_block, torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -656,3 +656,19 @@ def test_int4_fake_quant_general_blocks_match_torch_chain(oracle, shape, block, 
     assert torch.equal(out.view(bits), out_t.view(bits)) and torch.equal(scale.view(bits), scale_t.view(bits))
     if not sym:
         assert torch.equal(zero.view(bits), zero_t.view(bits))
+
+
+@pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(130, 257), (256, 384)])
+@pytest.mark.parametrize("kind", W.PATTERNS)
+def test_fp8_power_of_two_scales_match_torch_chain(oracle, shape, kind):
+    # parity with SGLang itself is unpinned (its source is not in the tree); this fixes the restated algorithm
+    x = W.reference_pattern(kind, shape, spread=512.0, amplitude=16.0)
+    y, s = oracle.per_block_cast_to_fp8(x)
+    y_t, s_t = torch_per_block_cast_to_fp8(x)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(y, y_t)
+    mant = s.view(torch.int32) & 0x7FFFFF
+    assert torch.all(mant == 0)                                   # every scale is a power of two
+    if kind == "zeros":
+        assert torch.all(s == 2.0 ** -22)                         # 2^ceil(log2(1e-4 / 448))
+    if kind == "maxes":
+        assert torch.all(y.float().abs().amax() <= 448)
