@@ -162,6 +162,22 @@ def per_quantizer(gen):
     return res
 
 
+def full_model_block_fp8(weights, elems):
+    """The whole model through the offline tool's quantizer (`block_fp8`: exact division, all-zero-tile rule) instead
+    of the sync path's `fp8_blockwise_cast`: same tensors and traffic, the variant whose bytes the reference's CPU code
+    can confirm."""
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    targets = [t for name, t in weights.items() if t.dim() == 2 and "embedding" not in name and "output_layer" not in name]
+    assert sum(t.numel() for t in targets) == elems
+    batch, outs = _record(lambda: [block_fp8(t, [128, 128]) for t in targets])
+    ms = _event_ms(batch.run, 5)
+    gbps = elems * BYTES_PER_ELEM["fp8_block"] / ms / 1e6
+    del batch, outs
+    return {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4), "elements": elems,
+            "workload": "all 36 Qwen3-4B layers (fused qkv, o, fc1, fc2 as stored), block_fp8, one job list"}
+
+
 def adjacent_formats(gen):
     """GB/s of the kernels either side of the path (MXFP4 pack / unpack, INT4 unpack, asymmetric INT4 pack).
     The unpackers and the asymmetric packer are single-tensor entry points, so they are timed as direct calls on
@@ -298,9 +314,36 @@ def cpu_baseline(weights, args, budget_s=12.0):
             break
     dt = time.perf_counter() - t0
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": round(reps * elems * BYTES_PER_ELEM["fp8_block"] / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
-            "kind": "port", "sample": f"{reps} x one Qwen3-4B layer (q,k,v,o,gate,up,down = {elems} elements) through "
-                                       f"the OpenMP C oracle's fp8_blockwise_cast, {dt:.1f} s"}
+    out = {"value": round(reps * elems * BYTES_PER_ELEM["fp8_block"] / dt / 1e9, 3), "unit": "GB/s", "cores": threads,
+           "kind": "port", "sample": f"{reps} x one Qwen3-4B layer (q,k,v,o,gate,up,down = {elems} elements) through "
+                                      f"the OpenMP C oracle's fp8_blockwise_cast, {dt:.1f} s"}
+    out["torch_cpu_op_chain"] = _torch_cpu_block_fp8(tensors[-3])
+    return out
+
+
+def _torch_cpu_block_fp8(w, budget_s=4.0):
+    """The offline tool's block_fp8 as the reference writes it -- pad, reshape to tiles, abs/max, divide, clamp, cast
+    (tools/convert_hf_to_fp8.py:39-70) -- run by PyTorch's CPU kernels on one gate_proj: the closest thing to the
+    reference's own CPU path.  Reported next to the oracle figure, not used for anything else."""
+    n, k = w.shape
+    nt, kt = -(-n // 128), -(-k // 128)
+
+    def chain():
+        padded = torch.nn.functional.pad(w, (0, kt * 128 - k, 0, nt * 128 - n), mode="constant", value=0.0)
+        tiles = padded.reshape(nt, 128, kt, 128)
+        amax = tiles.abs().max(dim=1, keepdim=True)[0].max(dim=3, keepdim=True)[0]
+        scale = amax.to(torch.float32) / 448.0
+        q = (tiles / scale).clamp(min=-448.0, max=448.0).reshape(nt * 128, kt * 128).to(torch.float8_e4m3fn)
+        return q[:n, :k], scale
+
+    chain()
+    t0, reps = time.perf_counter(), 0
+    while time.perf_counter() - t0 < budget_s:
+        chain()
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(reps * w.numel() * BYTES_PER_ELEM["fp8_block"] / dt / 1e9, 3), "unit": "GB/s",
+            "cores": torch.get_num_threads(), "sample": f"{reps} x block_fp8 op chain on gate_proj {tuple(w.shape)}, {dt:.1f} s"}
 
 
 def parity_sample(weights, args, plan):
@@ -399,8 +442,9 @@ def main():
     if not a.no_extras:
         del updater, plan
         line["packed_payload"] = packed_payload(args, weights, fp8_cfg, a.steps)
+        c2_block_fp8 = full_model_block_fp8(weights, elems)
         weights.clear()
-        line["per_quantizer"] = per_quantizer(gen)
+        line["per_quantizer"] = {"C2_block_fp8": c2_block_fp8, **per_quantizer(gen)}
     print(json.dumps(line))
 
 
