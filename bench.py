@@ -39,8 +39,8 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2,
                   "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
-# scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0003 B per element)
-MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0005
+# scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0005 B per element)
+MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0008
 
 METRIC = "HBM GB/s (% of peak) per quantizer; ms per full-model BF16->FP8 weight sync"
 DEV = "cuda:0"
