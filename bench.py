@@ -36,7 +36,7 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16,
                   # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
                   "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
-                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2,
+                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2, "act_quant": 2 + 1 + 4 / 128,
                   "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0005 B per element)
@@ -223,6 +223,11 @@ def adjacent_formats(gen):
     for name, fn in (("fp8", fq.fake_quant_fp8_forward), ("fp4", fq.fake_quant_fp4_forward),
                      ("compressed_kv", fq.fake_quant_compressed_kv_forward)):
         run(f"next_fake_quant_{name}", "fake_quant_bf16", lambda fn=fn: [fn(w) for w in ws], "bf16 in, bf16 out")
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+    run("next_act_quant_fp8_1x128", "act_quant", lambda: [act_quant(w, 128, "ue8m0") for w in ws],
+        "1x128 groups, power-of-two fp32 scales, bf16 -> e4m3 codes")
+    run("next_fp8_simulate_1x128", "fake_quant_bf16", lambda: [fp8_simulate(w, 128) for w in ws],
+        "1x128 quantize + cast back in one pass, bf16 in, bf16 out")
     return res
 
 

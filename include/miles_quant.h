@@ -121,6 +121,17 @@ int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, void* y, 
  *   mode 0: e4m3, 1x32, power-of-two scale   mode 1: e2m1, 1x32, power-of-two scale   mode 2: e2m1, 1x16, e4m3 scale */
 int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, void* stream);
 
+/* act_quant(x, block_size, scale_fmt, scale_dtype, inplace)   miles/kernels/quant/fp8_act_quant.py:110-137 (kernel :49-107)
+ *   FP8 e4m3 quantization of 1 x block groups of consecutive elements (numel % block == 0):
+ *   s = max(amax, 1e-4) * f32(1/448), code = e4m3(clamp(x / s, +-448)) with a true fp32 division.
+ *   flags: MQ_ACT_ROUND_SCALE  s rounded up to a power of two (scale_fmt given)
+ *          MQ_ACT_SCALE_E8M0   scale [numel/block] stored as E8M0 exponent bytes instead of fp32 (needs ROUND_SCALE)
+ *          MQ_ACT_INPLACE      y gets dtype(f32(code) * s) in the dtype of x instead of the codes; y may be x itself
+ *   ROUND_SCALE | INPLACE is fp8_simulate (miles_plugins/models/deepseek_v4/ops/qat.py:8-23).
+ *   Tuned for block 16 / 32 / 64 / 128 on 16-byte aligned tensors; any other block size runs a plain kernel. */
+enum { MQ_ACT_ROUND_SCALE = 1, MQ_ACT_SCALE_E8M0 = 2, MQ_ACT_INPLACE = 4 };
+int mq_fp8_act_quant(const void* x, int dtype, void* y, void* scale, int64_t numel, int block, int flags, void* stream);
+
 /* NVFP4                                              miles/utils/nvfp4.py:54-114
  * The global amax travels on the device in an "amax record": MQ_NVFP4_RECORD_WORDS uint32 words made of
  * MQ_NVFP4_SECTIONS sections of MQ_NVFP4_SECTION_WORDS partial maxima (float bit patterns).  Each tensor that

@@ -31,6 +31,7 @@ SIGNATURES = {
     "mq_int4_unpack_dequant": [_vp, _vp, _i32, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp4_to_fp8_block": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
     "mq_fake_quant": [_vp, _i32, _vp, _i64, _i32, _vp],
+    "mq_fp8_act_quant": [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _vp],
     "mq_mxfp4_quant": [_vp, _i32, _vp, _vp, _i64, _i32, _vp],
     "mq_mxfp4_dequant": [_vp, _vp, _vp, _i64, _i32, _vp],
     "mq_int4_group_quant_pack": [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp],

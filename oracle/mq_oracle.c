@@ -479,6 +479,38 @@ void mqo_fake_quant(const void* x, int dtype, int64_t numel, int mode, void* y) 
     }
 }
 
+/* act_quant (miles/kernels/quant/fp8_act_quant.py:49-137): FP8 quantization of 1 x block groups of the last
+ * dimension, the form DeepSeek-V4's activation / KV simulation uses.
+ *   amax  = max(max|x|, 1e-4)                                                        (:84)
+ *   s     = amax * f32(1/448);  round_scale: s = 2^ceil(log2(s)) read off the bits   (:85-88, :29-46)
+ *   code  = e4m3(min(max(x / s, -448), 448))      <- fp32 division                   (:100-101)
+ *   inplace: y = dtype(f32(code) * s)                                                (:90-98)
+ *   scale stored as fp32, or (power-of-two scales only) as its E8M0 exponent byte    (:102-103)
+ * flags: 1 = round_scale, 2 = E8M0 scale bytes, 4 = inplace (y has the input dtype).
+ * fp8_simulate (miles_plugins/models/deepseek_v4/ops/qat.py:8-23) = flags 1|4: the TileKernels cast-back it calls
+ * multiplies the decoded code by the scale and rounds to the output dtype, as the inplace branch does. */
+void mqo_fp8_act_quant(const void* x, int dtype, int64_t numel, int block, int flags, void* y, void* scale) {
+    const float inv = u2f(0x3B124925u);
+#pragma omp parallel for schedule(static)
+    for (int64_t g = 0; g < numel / block; g++) {
+        float amax = 0.0f;
+        for (int j = 0; j < block; j++) amax = fmaxf(amax, fabsf(load_as_f32(x, g * block + j, dtype)));
+        float s = fmaxf(amax, 1e-4f) * inv;
+        if (flags & 1) s = fq_ceil_pow2(s);
+        if (flags & 2) ((uint8_t*)scale)[g] = (uint8_t)(f2u(s) >> 23);
+        else ((float*)scale)[g] = s;
+        for (int j = 0; j < block; j++) {
+            int64_t i = g * block + j;
+            float r = load_as_f32(x, i, dtype) / s;
+            uint8_t code = mqo_f32_to_e4m3fn(fminf(fmaxf(r, -448.0f), 448.0f));
+            if (!(flags & 4)) { ((uint8_t*)y)[i] = code; continue; }
+            float o = mqo_e4m3fn_to_f32(code) * s;
+            if (dtype == MQ_F32) ((float*)y)[i] = o;
+            else ((uint16_t*)y)[i] = dtype == MQ_BF16 ? f32_to_bf16(o) : f32_to_f16(o);
+        }
+    }
+}
+
 /* cast_e2m1fn_to_e4m3fn (tools/convert_mxfp4_to_fp8.py:30-49): per 128x128 tile
  *   tile_scale = max(f32(scale)) / 64;  offset = f32(scale) / tile_scale;  y = e4m3(table[code] * offset)
  * scale bytes are float8_e8m0fnu: f32 = 2^(s-127) (s = 0 is the fp32 denormal 2^-127, s = 255 NaN). */

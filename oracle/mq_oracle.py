@@ -79,6 +79,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_nvfp4_quant_ex.argtypes = [vp, i32, i64, i64, f32, i32, i32, vp, vp]
         L.mqo_fake_quant.restype = None
         L.mqo_fake_quant.argtypes = [vp, i32, i64, i32, vp]
+        L.mqo_fp8_act_quant.restype = None
+        L.mqo_fp8_act_quant.argtypes = [vp, i32, i64, i32, i32, vp, vp]
         L.mqo_mxfp4_quant.restype = None
         L.mqo_mxfp4_quant.argtypes = [vp, i32, i64, i32, vp, vp]
         L.mqo_mxfp4_dequant.restype = None
@@ -268,6 +270,30 @@ def fake_quant(x: torch.Tensor, kind: str) -> torch.Tensor:
     out = torch.empty_like(xc)
     lib().mqo_fake_quant(xc.data_ptr(), _DTYPE[xc.dtype], xc.numel(), mode, out.data_ptr())
     return out
+
+
+def act_quant(x: torch.Tensor, block_size: int = 128, scale_fmt: str | None = None,
+              scale_dtype: torch.dtype = torch.float32, inplace: bool = False):
+    """miles/kernels/quant/fp8_act_quant.py:110-137 -> (float8_e4m3fn codes, scales), or with `inplace` the
+    quantize-dequantize result in x's dtype (returned, x is left alone)."""
+    _check_cpu(x)
+    n = x.shape[-1]
+    assert n % block_size == 0
+    e8m0 = scale_dtype == torch.float8_e8m0fnu
+    assert scale_fmt is not None or not e8m0, "E8M0 storage needs power-of-two scales"
+    z = x.contiguous()
+    y = torch.empty_like(z) if inplace else torch.empty(z.shape, dtype=torch.uint8)
+    s = torch.empty((*z.shape[:-1], n // block_size), dtype=torch.uint8 if e8m0 else torch.float32)
+    flags = (1 if scale_fmt is not None else 0) | (2 if e8m0 else 0) | (4 if inplace else 0)
+    lib().mqo_fp8_act_quant(z.data_ptr(), _DTYPE[z.dtype], z.numel(), int(block_size), flags, y.data_ptr(), s.data_ptr())
+    if e8m0:
+        s = s.view(torch.float8_e8m0fnu)
+    return y if inplace else (y.view(torch.float8_e4m3fn), s)
+
+
+def fp8_simulate(x: torch.Tensor, block_size: int) -> torch.Tensor:
+    """miles_plugins/models/deepseek_v4/ops/qat.py:8-23."""
+    return act_quant(x, block_size, "ue8m0", inplace=True)
 
 
 # --------------------------------------------------------------------------

@@ -205,9 +205,30 @@ def fake_quant() -> dict:
     return fam.save()
 
 
+def fp8_act_quant() -> dict:
+    fam = Family("fp8_act_quant", "torch_act_quant = miles/kernels/quant/fp8_act_quant.py:49-137 as torch CPU ops",
+                 "fp32 division, clamp and float8_e4m3fn cast of torch's CPU kernels (the device kernel of the reference is "
+                 "TileLang; parity with it is unpinned)")
+    for dt in (torch.bfloat16, torch.float32):
+        g = torch.Generator().manual_seed(11)
+        x = (torch.randn(6, 512, generator=g) * torch.logspace(-6, 4, 512)).to(dt)
+        x[0, :128] = 0
+        x[1, :4] = torch.tensor([448.0, -448.0, -0.0, 1e-6]).to(dt)
+        x[2, :128] = -0.0
+        name = str(dt).split(".")[-1]
+        for block in (64, 128):
+            for round_scale in (False, True):
+                y, s = T.torch_act_quant(x, block, round_scale, False)
+                qdq, _ = T.torch_act_quant(x, block, round_scale, True)
+                fam.add(f"b{block}_{'pow2' if round_scale else 'plain'}_{name}",
+                        {"block": block, "round_scale": round_scale, "dtype": name, "shape": [6, 512]},
+                        x=x, y=y, scale=s, qdq=qdq)
+    return fam.save()
+
+
 def main() -> None:
     manifest = {"generator": "tests/golden/make_fixtures.py", "torch": torch.__version__,
-                "families": [f() for f in (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4, fake_quant)]}
+                "families": [f() for f in (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4, fake_quant, fp8_act_quant)]}
     with open(os.path.join(HERE, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
     total = sum(os.path.getsize(os.path.join(HERE, fam["file"])) for fam in manifest["families"])

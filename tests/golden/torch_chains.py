@@ -315,3 +315,21 @@ def torch_per_block_cast_to_fp8(x):
     sf = torch.pow(2.0, torch.ceil(torch.log2((x_amax / 448.0).abs())))
     x_scaled = (x_view * (1.0 / sf)).to(F8)
     return x_scaled.view_as(x_padded)[:m, :n].contiguous(), sf.view(x_view.size(0), x_view.size(2))
+
+
+def torch_act_quant(x, block_size, round_scale, inplace):
+    """act_quant (miles/kernels/quant/fp8_act_quant.py:49-137) as torch CPU ops: 1 x block groups of the last
+    dimension, amax floored at 1e-4, scale = amax * f32(1/448) (round_scale: rounded up to a power of two through
+    frexp), fp32 division, clamp, e4m3 cast; `inplace` returns dtype(f32(code) * scale).  Returns (y, fp32 scales)."""
+    n = x.shape[-1]
+    xf = x.float().reshape(-1, n // block_size, block_size)
+    amax = xf.abs().amax(dim=-1, keepdim=True).clamp(min=1e-4)
+    s = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    if round_scale:
+        mant, exp = torch.frexp(s)                      # s = mant * 2^exp, mant in [0.5, 1)
+        s = torch.ldexp(torch.ones_like(s), torch.where(mant == 0.5, exp - 1, exp))
+    code = (xf / s).clamp(-448.0, 448.0).to(F8)
+    scales = s.reshape(*x.shape[:-1], n // block_size)
+    if inplace:
+        return (code.float() * s).to(x.dtype).reshape(x.shape), scales
+    return code.reshape(x.shape), scales

@@ -115,6 +115,9 @@ class _OracleImpl:
     def nvfp4_pair(self, a, b):
         return self.o.nvfp4_quantize_1d_pair(a, b)
 
+    def act_quant(self, x, block, fmt, inplace=False):
+        return self.o.act_quant(x, block, fmt, inplace=inplace)
+
 
 class _HipImpl:
     dev = DEV
@@ -163,6 +166,10 @@ class _HipImpl:
     def nvfp4_pair(self, a, b):
         from miles_amd.utils.nvfp4 import nvfp4_quantize_1d_pair
         return nvfp4_quantize_1d_pair(a, b)
+
+    def act_quant(self, x, block, fmt, inplace=False):
+        from miles_amd.kernels.quant.fp8_act_quant import act_quant
+        return act_quant(x.clone(), block, fmt, inplace=inplace)
 
 
 def _check_fp8_block(impl, case):
@@ -255,8 +262,20 @@ def _check_fake_quant(impl, case):
     assert torch.equal(_bits(got)[nz], _bits(want)[nz]), f"{case} bits"
 
 
+def _check_act_quant(impl, case):
+    info = _info("fp8_act_quant", case)
+    dt = _DT[info["dtype"]]
+    x = _t("fp8_act_quant", case, "x", dt).to(impl.dev)
+    fmt = "ue8m0" if info["round_scale"] else None
+    y, s = impl.act_quant(x, info["block"], fmt)
+    _same(s, _t("fp8_act_quant", case, "scale"), f"{case} scales")
+    _same(y.view(torch.uint8), _t("fp8_act_quant", case, "y"), f"{case} codes")
+    _same(impl.act_quant(x, info["block"], fmt, inplace=True), _t("fp8_act_quant", case, "qdq", dt), f"{case} quantize-dequantize")
+
+
 _CHECKS = [("fp8_block", _check_fp8_block), ("fp8_blockwise_cast", _check_fp8_blockwise), ("fp8_dequant", _check_fp8_dequant),
-           ("mxfp8", _check_mxfp8), ("mxfp4", _check_mxfp4), ("int4", _check_int4), ("nvfp4", _check_nvfp4), ("fake_quant", _check_fake_quant)]
+           ("mxfp8", _check_mxfp8), ("mxfp4", _check_mxfp4), ("int4", _check_int4), ("nvfp4", _check_nvfp4), ("fake_quant", _check_fake_quant),
+           ("fp8_act_quant", _check_act_quant)]
 _PARAMS = [pytest.param(fam, fn, case, id=f"{fam}-{case}") for fam, fn in _CHECKS for case in _cases(fam)]
 
 

@@ -868,3 +868,87 @@ def test_fp8_power_of_two_scales(oracle, shape, kind):
         y2_o, s2_o = oracle.per_block_cast_to_fp8(xf)
         _assert_same(s2, s2_o, "scales (fp32, strided)")
         _assert_same(y2, y2_o, "codes (fp32, strided)")
+
+
+# ---------------------------------------------------------------------------------------------------
+# act_quant / fp8_simulate (miles/kernels/quant/fp8_act_quant.py, miles_plugins/models/deepseek_v4/ops/qat.py)
+def _act_input(dtype, shape=(5, 37, 1024), seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(*shape, generator=g) * torch.logspace(-6, 4, shape[-1])).to(dtype)
+    x[0, 0, :128] = 0
+    x[0, 1, :4] = torch.tensor([448.0, -448.0, -0.0, 1e-6]).to(dtype)
+    x[0, 2, :128] = -0.0
+    x[0, 3, :128] = 2.0 ** -20
+    x[0, 4, :128] = torch.finfo(dtype).max if dtype != torch.float32 else 1e38
+    return x
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("block", [16, 32, 64, 128, 256, 8])
+@pytest.mark.parametrize("scale_fmt", [None, "ue8m0"])
+def test_act_quant_codes_scales_and_inplace(oracle, dtype, block, scale_fmt):
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+
+    x = _act_input(dtype)
+    y, s = act_quant(x.to(DEV), block, scale_fmt)
+    y_o, s_o = oracle.act_quant(x, block, scale_fmt)
+    assert y.dtype == F8 and y.shape == x.shape and s.dtype == torch.float32 and s.shape == (5, 37, 1024 // block)
+    _assert_same(s, s_o, f"act_quant scales block {block}")
+    _assert_same(y, y_o, f"act_quant codes block {block}")
+    xd = x.to(DEV)
+    out = act_quant(xd, block, scale_fmt, inplace=True)
+    assert out is xd
+    _assert_same(xd, oracle.act_quant(x, block, scale_fmt, inplace=True), f"act_quant inplace block {block}")
+    if scale_fmt is not None:
+        y8, s8 = act_quant(x.to(DEV), block, scale_fmt, scale_dtype=torch.float8_e8m0fnu)
+        assert s8.dtype == torch.float8_e8m0fnu
+        _assert_same(s8.view(torch.uint8), oracle.act_quant(x, block, scale_fmt, scale_dtype=torch.float8_e8m0fnu)[1].view(torch.uint8), "e8m0 scales")
+        _assert_same(y8, y_o, "codes with e8m0 scales")
+        src = x.to(DEV)
+        sim = fp8_simulate(src, block)
+        assert torch.equal(src.cpu(), x)                      # the input is left alone
+        _assert_same(sim, oracle.fp8_simulate(x, block), f"fp8_simulate block {block}")
+
+
+def test_act_quant_views_errors_and_straight_through(oracle):
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate_qat
+
+    x = _act_input(torch.bfloat16, shape=(2, 16, 576))
+    # the reference's callers quantize a slice of the last dimension in place (compressor.py:170): a strided view
+    xd = x.to(DEV)
+    act_quant(xd[..., :512], 64, "ue8m0", inplace=True)
+    want = x.clone()
+    want[..., :512] = oracle.act_quant(x[..., :512], 64, "ue8m0", inplace=True)
+    _assert_same(xd, want, "in-place on a slice")
+    # an unaligned base address takes the plain kernel
+    flat = torch.zeros(64 * 128 + 1, dtype=torch.bfloat16)
+    flat[1:] = x.reshape(-1)[: 64 * 128]
+    y, s = act_quant(flat.to(DEV)[1:].view(64, 128), 128)
+    y_o, s_o = oracle.act_quant(flat[1:].view(64, 128), 128)
+    _assert_same(y, y_o, "unaligned codes")
+    _assert_same(s, s_o, "unaligned scales")
+    with pytest.raises(AssertionError):
+        act_quant(torch.zeros(4, 100, device=DEV, dtype=torch.bfloat16), 64)
+    with pytest.raises(ValueError):
+        act_quant(torch.zeros(4, 128, device=DEV, dtype=torch.bfloat16), 64, scale_dtype=torch.float8_e8m0fnu)
+    kv = torch.randn(8, 256, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    grad = torch.randn_like(kv)
+    fp8_simulate_qat(kv, 64).backward(grad)
+    assert torch.equal(kv.grad, grad)
+
+
+def test_act_quant_full_size_round_trip(oracle):
+    # size-independent properties on a large activation: |qdq - x| <= scale * 2^-4 * |code| grid step, scales
+    # are powers of two, and quantizing the result again is the identity (idempotence)
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+
+    x = torch.randn(16384, 7168, device=DEV, dtype=torch.bfloat16)
+    y, s = act_quant(x, 128, "ue8m0")
+    assert torch.all((s.view(torch.int32) & 0x7FFFFF) == 0)
+    sim = fp8_simulate(x, 128)
+    again = fp8_simulate(sim, 128)
+    assert torch.equal(sim, again)
+    err = (sim.float() - x.float()).abs().view(16384, -1, 128)
+    assert torch.all(err <= s.unsqueeze(-1) * 448 * 2.0 ** -4)
+    head = x[:64].cpu()
+    _assert_same(sim[:64], oracle.fp8_simulate(head, 128), "full-size head rows")

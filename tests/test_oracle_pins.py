@@ -18,7 +18,7 @@ import pytest
 import torch
 
 from miles_amd import workloads as W
-from tests.golden.torch_chains import (torch_per_block_cast_to_fp8, torch_fake_int4_block, torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
+from tests.golden.torch_chains import (torch_act_quant, torch_per_block_cast_to_fp8, torch_fake_int4_block, torch_nvfp4_4over6, torch_nvfp4_qdq, torch_cast_e2m1fn_to_e4m3fn, torch_fake_quant_reference, torch_block_fp8, torch_dequant_fp8_block, torch_dequantize_mxfp4,
                                        torch_fake_int4_asym, torch_fake_int4_sym, torch_fp8_blockwise_cast,
                                        torch_mxfp8, torch_nvfp4, torch_pack_layer_asym_python_half,
                                        torch_pack_layer_python_half, torch_quantize_mxfp4)
@@ -672,3 +672,51 @@ def test_fp8_power_of_two_scales_match_torch_chain(oracle, shape, kind):
         assert torch.all(s == 2.0 ** -22)                         # 2^ceil(log2(1e-4 / 448))
     if kind == "maxes":
         assert torch.all(y.float().abs().amax() <= 448)
+
+
+# ---------------------------------------------------------------------------------------------------
+# act_quant / fp8_simulate (miles/kernels/quant/fp8_act_quant.py, miles_plugins/models/deepseek_v4/ops/qat.py)
+def _act_input(dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(24, 1024, generator=g) * torch.logspace(-6, 4, 1024)).to(dtype)
+    x[0, :128] = 0
+    x[1, :4] = torch.tensor([448.0, -448.0, -0.0, 1e-6]).to(dtype)
+    x[2, :128] = -0.0
+    x[3, :128] = 2.0 ** -20          # below the 1e-4 amax floor
+    return x
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("block", [16, 32, 64, 128, 256])
+@pytest.mark.parametrize("round_scale", [False, True])
+def test_act_quant_matches_torch_chain(oracle, dtype, block, round_scale):
+    x = _act_input(dtype)
+    fmt = "ue8m0" if round_scale else None
+    bits = torch.int32 if dtype == torch.float32 else torch.int16
+    y, s = oracle.act_quant(x, block, fmt)
+    y_t, s_t = torch_act_quant(x, block, round_scale, False)
+    assert y.dtype == torch.float8_e4m3fn and s.shape == (24, 1024 // block)
+    assert torch.equal(y.view(torch.uint8), y_t.view(torch.uint8)) and torch.equal(s.view(torch.int32), s_t.view(torch.int32))
+    qdq = oracle.act_quant(x, block, fmt, inplace=True)
+    qdq_t, _ = torch_act_quant(x, block, round_scale, True)
+    assert torch.equal(qdq.view(bits), qdq_t.view(bits))          # signs of zeros included
+    if round_scale:
+        y8, s8 = oracle.act_quant(x, block, fmt, scale_dtype=torch.float8_e8m0fnu)
+        assert torch.equal(s8.float(), s_t) and torch.equal(y8.view(torch.uint8), y.view(torch.uint8))
+        assert torch.equal(oracle.fp8_simulate(x, block).view(bits), qdq_t.view(bits))
+
+
+def test_act_quant_known_answers(oracle):
+    # one group of 128 with amax 448: scale 448 * f32(1/448) = 1 - 2^-24 rounds to 1.0f?  f32(1/448) is just above 1/448,
+    # so the product is 1.0000001 -> 1.0 after rounding; codes are then the values themselves
+    x = torch.zeros(1, 128)
+    x[0, :6] = torch.tensor([448.0, -1.0, 0.5, 1.0625, 2.0 ** -9, 2.0 ** -11])
+    y, s = oracle.act_quant(x, 128)
+    assert s.item() == pytest.approx(1.0, rel=1e-6)
+    assert y.float()[0, :6].tolist() == [448.0, -1.0, 0.5, 1.0, 2.0 ** -9, 0.0]      # 1.0625 is a tie -> even; 2^-11 -> 0
+    y, s = oracle.act_quant(x, 128, "ue8m0")
+    assert s.item() in (1.0, 2.0) and (s.view(torch.int32) & 0x7FFFFF).item() == 0
+    # all-zero group: the 1e-4 floor sets the scale, codes are +0
+    y, s = oracle.act_quant(torch.zeros(1, 64), 64, "ue8m0")
+    assert s.item() == 2.0 ** -22 and torch.all(y.view(torch.uint8) == 0)
+    assert oracle.act_quant(torch.zeros(1, 64), 64)[1].item() == pytest.approx(1e-4 / 448, rel=1e-6)
