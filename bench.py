@@ -162,6 +162,74 @@ def per_quantizer(gen):
     return res
 
 
+def full_configs(gen):
+    """The three MoE configurations at their full element counts, each as one whole weight sync through the driver
+    (`WeightUpdater` with a replayed plan, 512 MiB buckets): every expert of every layer at its real shape.
+    Not part of the default run (generating 58 GB of synthetic experts takes a while); `--full-configs` prints one
+    extra JSON line."""
+    from miles_amd.weight_update.updater import WeightUpdater
+
+    def moe_weights(layers, experts, ffn, hidden, std, p, gain):
+        w = {}
+        for layer in range(layers):
+            L = f"module.module.decoder.layers.{layer}."
+            for e in range(experts):
+                w[L + f"mlp.experts.linear_fc1.weight{e}"] = _synth((2 * ffn, hidden), gen, std=std, p=p, gain=gain)
+                w[L + f"mlp.experts.linear_fc2.weight{e}"] = _synth((hidden, ffn), gen, std=std, p=p, gain=gain)
+        return w
+
+    def sync(name, key, model_name, cfg, shape, note, **extra):
+        layers, experts, ffn, hidden = shape
+        weights = moe_weights(layers, experts, ffn, hidden, *((0.02, 0.0, 1.0) if key == "mxfp8" else (0.015, 0.0005, 30.0)))
+        elems = layers * experts * 3 * ffn * hidden
+        args = Namespace(hidden_size=hidden, num_attention_heads=32, num_query_groups=4, kv_channels=128, vocab_size=1000,
+                         num_layers=layers, update_weight_buffer_size=512 * 1024**2, q_lora_rank=None)
+        seen = {"buckets": 0, "tensors": 0}
+
+        def consume(bucket):
+            seen["buckets"] += 1
+            seen["tensors"] += len(bucket)
+
+        upd = WeightUpdater(args, weights_getter=lambda: weights, model_name=model_name, quantization_config=cfg,
+                            send_bucket=consume, **extra)
+        t0 = time.perf_counter()
+        upd.update_weights()
+        torch.cuda.synchronize()
+        first_s = time.perf_counter() - t0
+        assert upd._plan is not None and upd._plan.replayable, name
+        for _ in range(2):
+            upd.update_weights()
+        torch.cuda.synchronize()
+        seen.update(buckets=0, tensors=0)
+        steps = 5
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            upd.update_weights()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
+        out = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms_per_sync": round(ms, 3),
+               "elements": elems, "megatron_tensors": len(weights), "hf_tensors_per_sync": seen["tensors"] // steps,
+               "buckets_per_sync": seen["buckets"] // steps, "jobs": len(upd._plan.batch),
+               "first_sync_s": round(first_s, 2), "workload": note}
+        del upd, weights
+        return out
+
+    res = {}
+    res["C3_qwen3_30b_a3b_mxfp8"] = sync("C3", "mxfp8", "qwen3moe", {"quant_method": "mxfp8"}, (48, 128, 768, 2048),
+                                         "48 layers x 128 experts, gate/up [768,2048] down [2048,768], MXFP8 1x32 E8M0")
+    int4_cfg = {"quant_method": "compressed-tensors", "format": "pack-quantized",
+                "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4, "type": "int"}}}}
+    basenames = {f"model.layers.0.mlp.experts.{e}.{p}_proj" for e in range(384) for p in ("gate", "up", "down")}
+    res["C4_kimi_k2_int4_g128"] = sync("C4", "int4_g128", "kimi_k2", int4_cfg, (1, 384, 2048, 7168),
+                                       "384 experts, gate/up [2048,7168] down [7168,2048], INT4 group 128 packed",
+                                       packed_weight_basenames=basenames)
+    res["C5a_deepseek_v3_nvfp4"] = sync("C5a", "nvfp4", "deepseekv3", {"quant_method": "modelopt", "quant_algo": "NVFP4"},
+                                        (1, 256, 2048, 7168),
+                                        "256 experts, gate/up [2048,7168] paired + down [7168,2048], NVFP4 1x16")
+    return res
+
+
 def full_model_block_fp8(weights, elems):
     """The whole model through the offline tool's quantizer (`block_fp8`: exact division, all-zero-tile rule) instead
     of the sync path's `fp8_blockwise_cast`: same tensors and traffic, the variant whose bytes the reference's CPU code
@@ -379,6 +447,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-workload", action="store_true",
                     help="counter-collection run: three 1 GiB plain copies (calibration), three syncs, no timing")
+    ap.add_argument("--full-configs", action="store_true",
+                    help="only the three MoE configurations at full size, each as one whole sync (one JSON line)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
@@ -390,6 +460,9 @@ def main():
     _lib.load()   # fails loudly if the HIP library is not built
     gen = torch.Generator(device=DEV)
     gen.manual_seed(2001)
+    if a.full_configs:
+        print(json.dumps({"full_configs": full_configs(gen)}))
+        return
     args, weights, elems = qwen3_4b_megatron_weights(gen)
     fp8_cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
     sent = {"buckets": 0, "bytes": 0}

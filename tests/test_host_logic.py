@@ -347,3 +347,24 @@ def test_division_by_the_nvfp4_numerators_is_exact_with_one_fma_correction():
         r = (-(q0.astype(np.float64) * np.float64(d32)) + x.astype(np.float64)).astype(np.float32)   # exact: the fma's value
         q = (r.astype(np.float64) * np.float64(y) + q0.astype(np.float64)).astype(np.float32)
         assert np.array_equal(q, x / d32)
+
+
+def test_sync_plan_matches_quick_and_full_forms():
+    # the quick form (same tensor objects, same addresses) and the full signature must agree on what a parameter set is
+    from miles_amd.weight_update.sync_plan import SyncPlan, weights_signature
+
+    weights = {f"p{i}": torch.zeros(4, 8) for i in range(5)}
+    plan = SyncPlan(batch=None, buckets=[], jobs_done_at_bucket=[], signature=weights_signature(weights), replayable=True)
+    plan.remember(weights)
+    assert plan.matches(weights)
+    assert plan.matches(dict(weights))                                    # another mapping, same objects
+    assert plan.matches({k: v.view(4, 8) for k, v in weights.items()})    # other objects, same storage and shape: full form
+    assert not plan.matches({k: v.view(8, 4) for k, v in weights.items()})
+    assert not plan.matches({k: v.clone() for k, v in weights.items()})
+    assert not plan.matches({k: weights[k] for k in list(weights)[:4]})
+    assert not plan.matches({("q" + k): v for k, v in weights.items()})   # same objects under other names
+    weights["p2"].data = torch.zeros(4, 8)                                # storage swapped under the same object
+    assert not plan.matches(weights)
+    plan.replayable = False
+    plan.remember(weights)
+    assert not plan.matches(weights)
