@@ -157,34 +157,40 @@ __device__ __forceinline__ void nv_decode8(uint32_t word, float q[8]) {
 }
 // x / d for d = 2688 or 1536 with y = RN(1/d): q0 = RN(x*y); r = x - q0*d (exact in an FMA); q = RN(q0 + r*y) is the
 // correctly rounded quotient for every fp32 mantissa of x and both divisors (exhaustive CPU check, 2^23 mantissas
-// each), provided no intermediate leaves the normal range; operands outside 2^-90 .. 2^90 take the division.
-// A zero comes out as +0 whatever its sign, which no error term can see.
+// each), provided no intermediate leaves the normal range, i.e. for |x| in 2^-91 .. 2^89 (and for zero, which comes
+// out as +0 whatever its sign: no error term can see that).  The numerators here are RN(RN(value * f32(scale)) * amax)
+// with value * f32(scale) either zero or in 2^-10 .. 2688, so one test of the tensor amax covers every element:
+// nv_fast_division(amax) allows the sequence for the whole tensor, otherwise every quotient is the IEEE division.
+__device__ __forceinline__ bool nv_fast_division(float amax) {
+    const uint32_t e = f2u(amax) & 0x7F800000u;
+    return e >= 0x17800000u /* 2^-80 */ && e <= 0x65800000u /* 2^76 */;
+}
+template <bool FASTDIV>
 __device__ __forceinline__ float div_by_numer(float x, float d, float y) {
+    if (!FASTDIV) return x / d;
     const float q0 = x * y;
     const float r = __builtin_fmaf(-q0, d, x);
-    float q = __builtin_fmaf(r, y, q0);
-    const uint32_t e = f2u(x) & 0x7F800000u;
-    if (__builtin_expect(e - 0x12000000u > 0x5A000000u && x != 0.0f, 0)) q = x / d;
-    return q;
+    return __builtin_fmaf(r, y, q0);
 }
-// error terms of this lane's eight elements
+// error terms of this lane's eight elements; EM bit 0: squared error, bit 1: fp16 candidate error
+template <int EM, bool FASTDIV>
 __device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandidate& c, float amax, float enc, float denom,
-                                               int flags, float term[8]) {
+                                               float term[8]) {
     float q[8];
     nv_decode8(c.word, q);
     const float denom_inv = 1.0f / denom;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         float diff;
-        if (flags & MQ_NVFP4_ERR_FP16) {
+        if (EM & 2) {
             _Float16 h = (_Float16)q[j] * (_Float16)c.s_f;        // both factors exact in fp16; one fp16 rounding
             float hf = (float)h;
             asm volatile("" : "+v"(hf));                          // keep the fp16 product a value of its own
             diff = hf - f[j] * enc;
         } else {
-            diff = div_by_numer((q[j] * c.s_f) * amax, denom, denom_inv) - f[j];
+            diff = div_by_numer<FASTDIV>((q[j] * c.s_f) * amax, denom, denom_inv) - f[j];
         }
-        term[j] = (flags & MQ_NVFP4_ERR_MSE) ? diff * diff : __builtin_fabsf(diff);
+        term[j] = (EM & 1) ? diff * diff : __builtin_fabsf(diff);
     }
 }
 // Sum of the block's sixteen terms in element order.  The even lane of the pair holds elements 0..7: its partial
@@ -200,20 +206,24 @@ __device__ __forceinline__ float nv_pair_error(const float term[8], bool odd_lan
     return odd_lane ? seeded : partner_total;
 }
 // the winning candidate for this lane's block; bmax is the block amax (pair-uniform)
+template <int EM, bool FASTDIV>
 __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float bmax, float amax, const NvScales& gs,
-                                                        float denom, int flags, bool odd_lane) {
+                                                        float denom, bool odd_lane) {
     const float s6_hp = (bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate c4 = nv_candidate(f, s4_hp, gs.s_dec), c6 = nv_candidate(f, s6_hp, gs.s_dec);
     float t4[8], t6[8];
-    nv_error_terms(f, c4, amax, gs.enc, denom, flags, t4);
-    nv_error_terms(f, c6, amax, gs.enc, denom, flags, t6);
+    nv_error_terms<EM, FASTDIV>(f, c4, amax, gs.enc, denom, t4);
+    nv_error_terms<EM, FASTDIV>(f, c6, amax, gs.enc, denom, t6);
     const float e4 = nv_pair_error(t4, odd_lane), e6 = nv_pair_error(t6, odd_lane);
     return e4 < e6 ? c4 : c6;
 }
+// error mode of a flags word, as the EM template argument
+static inline int nv_error_mode(int flags) { return ((flags & MQ_NVFP4_ERR_MSE) ? 1 : 0) | ((flags & MQ_NVFP4_ERR_FP16) ? 2 : 0); }
 
+// FOS = 0: standard quantizer; FOS = 1 + error mode: Four Over Six
 template <int FOS>
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, int flags, float denom) {
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float denom) {
     const FlatJob& job = tab.job[blockIdx.y];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
@@ -234,6 +244,7 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     gs.s_dec = u2f(amax_bits[kRecSDec]);
     gs.enc = u2f(amax_bits[kRecEnc]);
     const float amax = u2f(amax_bits[kRecAmax]);
+    const bool fastdiv = nv_fast_division(amax);
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
@@ -245,7 +256,9 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         uint32_t sc, word;
         if (FOS) {
-            const NvCandidate c = nv_four_over_six(f, bmax, amax, gs, denom, flags, (t & 1) != 0);
+            constexpr int EM = FOS > 0 ? FOS - 1 : 0;
+            const NvCandidate c = fastdiv ? nv_four_over_six<EM, true>(f, bmax, amax, gs, denom, (t & 1) != 0)
+                                          : nv_four_over_six<EM, false>(f, bmax, amax, gs, denom, (t & 1) != 0);
             sc = c.sc;
             word = c.word;
         } else if (mb < 0x7F80u && s_hp == s_hp) {
@@ -344,7 +357,7 @@ template <int DT, int FOS>
 __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* __restrict__ x,
                                                                const float* __restrict__ amax_ptr,
                                                                uint16_t* __restrict__ y, int64_t total_units,
-                                                               float numer, float inv_numer, int flags) {
+                                                               float numer, float inv_numer) {
     const int t = threadIdx.x;
     const int64_t unit = (int64_t)blockIdx.x * kNvThreads + t;
     const bool live = unit < total_units;
@@ -369,7 +382,9 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* _
     const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
     float s_f, q[8];
     if (FOS) {
-        const NvCandidate c = nv_four_over_six(f, bmax, amax, gs, numer, flags, (t & 1) != 0);
+        constexpr int EM = FOS > 0 ? FOS - 1 : 0;
+        const NvCandidate c = nv_fast_division(amax) ? nv_four_over_six<EM, true>(f, bmax, amax, gs, numer, (t & 1) != 0)
+                                                     : nv_four_over_six<EM, false>(f, bmax, amax, gs, numer, (t & 1) != 0);
         s_f = c.s_f;
         nv_decode8(c.word, q);
     } else if (m < 0x7F800000u && s_hp == s_hp) {
@@ -434,8 +449,13 @@ int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStre
     hipLaunchKernelGGL(nvfp4_fold_kernel, dim3((unsigned)tab.n), dim3(256), 0, st, tab, numer);
     if (tab.max_blocks > 0) {
         const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kNvThreads);
-        if (flags & MQ_NVFP4_4OVER6) hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<1>, grid, blk, 0, st, tab, flags, numer);
-        else hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<0>, grid, blk, 0, st, tab, flags, numer);
+        switch ((flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0) {
+            case 0: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<0>, grid, blk, 0, st, tab, numer); break;
+            case 1: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<1>, grid, blk, 0, st, tab, numer); break;
+            case 2: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<2>, grid, blk, 0, st, tab, numer); break;
+            case 3: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<3>, grid, blk, 0, st, tab, numer); break;
+            default: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<4>, grid, blk, 0, st, tab, numer); break;
+        }
     }
     return mq_check_launch("nvfp4 quant");
 }
@@ -511,10 +531,18 @@ extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y
     hipStream_t st = (hipStream_t)stream;
     const uint16_t* xi = (const uint16_t*)x;
     uint16_t* yo = (uint16_t*)y;
-    const bool fos = (flags & MQ_NVFP4_4OVER6) != 0;
-    if (dtype == MQ_BF16 && !fos) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_BF16, 0>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
-    else if (dtype == MQ_BF16) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_BF16, 1>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
-    else if (!fos) hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_F16, 0>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
-    else hipLaunchKernelGGL((nvfp4_qdq_kernel<MQ_F16, 1>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, flags);
+    const int fos = (flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0;
+#define MQ_QDQ_LAUNCH(DT, FOS) hipLaunchKernelGGL((nvfp4_qdq_kernel<DT, FOS>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer)
+#define MQ_QDQ_SWITCH(DT)                           \
+    switch (fos) {                                  \
+        case 0: MQ_QDQ_LAUNCH(DT, 0); break;        \
+        case 1: MQ_QDQ_LAUNCH(DT, 1); break;        \
+        case 2: MQ_QDQ_LAUNCH(DT, 2); break;        \
+        case 3: MQ_QDQ_LAUNCH(DT, 3); break;        \
+        default: MQ_QDQ_LAUNCH(DT, 4); break;       \
+    }
+    if (dtype == MQ_BF16) { MQ_QDQ_SWITCH(MQ_BF16) } else { MQ_QDQ_SWITCH(MQ_F16) }
+#undef MQ_QDQ_SWITCH
+#undef MQ_QDQ_LAUNCH
     return mq_check_launch("nvfp4 qdq");
 }
