@@ -75,6 +75,9 @@ def qwen3_4b_megatron_weights(gen):
     return args, w, quantized_elems
 
 
+TIMED_ITERS = 5        # repetitions per per-quantizer measurement (1 in the counter-collection run)
+
+
 def _event_ms(fn, iters):
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -110,7 +113,7 @@ def per_quantizer(gen):
 
     def run(name, key, elems, build, note):
         batch, outs = _record(build)
-        ms = _event_ms(batch.run, 5)
+        ms = _event_ms(batch.run, TIMED_ITERS)
         gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
         res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                      "elements": elems, "workload": note}
@@ -239,7 +242,7 @@ def full_model_block_fp8(weights, elems):
     targets = [t for name, t in weights.items() if t.dim() == 2 and "embedding" not in name and "output_layer" not in name]
     assert sum(t.numel() for t in targets) == elems
     batch, outs = _record(lambda: [block_fp8(t, [128, 128]) for t in targets])
-    ms = _event_ms(batch.run, 5)
+    ms = _event_ms(batch.run, TIMED_ITERS)
     gbps = elems * BYTES_PER_ELEM["fp8_block"] / ms / 1e6
     del batch, outs
     return {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4), "elements": elems,
@@ -262,13 +265,13 @@ def adjacent_formats(gen):
     def run(name, key, fn, note):
         fn()
         torch.cuda.synchronize()
-        ms = _event_ms(fn, 5)
+        ms = _event_ms(fn, TIMED_ITERS)
         gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
         res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                      "elements": elems, "workload": note}
 
     batch, m4 = _record(lambda: [quantize_mxfp4(w, 32) for w in ws])
-    ms = _event_ms(batch.run, 5)
+    ms = _event_ms(batch.run, TIMED_ITERS)
     gbps = elems * BYTES_PER_ELEM["mxfp4"] / ms / 1e6
     res["next_mxfp4_quant"] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                                "elements": elems, "workload": "8 x [16384,7168] bf16, group 32, one grouped launch"}
@@ -447,6 +450,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-workload", action="store_true",
                     help="counter-collection run: three 1 GiB plain copies (calibration), three syncs, no timing")
+    ap.add_argument("--pmc-quantizers", action="store_true",
+                    help="counter-collection run: three 1 GiB plain copies (calibration), then every workload of the "
+                         "per-quantizer section exactly twice, no timing")
     ap.add_argument("--full-configs", action="store_true",
                     help="only the three MoE configurations at full size, each as one whole sync (one JSON line)")
     a = ap.parse_args()
@@ -462,6 +468,19 @@ def main():
     gen.manual_seed(2001)
     if a.full_configs:
         print(json.dumps({"full_configs": full_configs(gen)}))
+        return
+    if a.pmc_quantizers:
+        global TIMED_ITERS
+        TIMED_ITERS = 1
+        n = 1 << 30
+        src, dst = torch.empty(n, dtype=torch.uint8, device=DEV), torch.empty(n, dtype=torch.uint8, device=DEV)
+        src.fill_(1)
+        for _ in range(3):
+            _lib.check(_lib.load().mq_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
+        del src, dst
+        res = per_quantizer(gen)
+        print(json.dumps({"pmc_quantizers": "3 x mq_copy_bytes(1 GiB), then each workload twice",
+                          "elements": {k: v["elements"] for k, v in res.items()}}))
         return
     args, weights, elems = qwen3_4b_megatron_weights(gen)
     fp8_cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}

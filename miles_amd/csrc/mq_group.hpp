@@ -38,6 +38,18 @@ inline int64_t xcd_grid(int64_t total) {
     return ((total + unit - 1) / unit) * unit;
 }
 
+// the same dealing with a chunk length chosen at launch time (a whole row band of a matrix, say)
+__device__ __forceinline__ int32_t xcd_chunked_item(int32_t total, int32_t chunk) {
+    const int32_t bid = blockIdx.x;
+    const int32_t x = bid % kXcds, k = bid / kXcds;
+    const int32_t item = ((k / chunk) * kXcds + x) * chunk + (k % chunk);
+    return item < total ? item : -1;
+}
+inline int64_t xcd_grid_chunked(int64_t total, int64_t chunk) {
+    const int64_t unit = (int64_t)kXcds * chunk;
+    return ((total + unit - 1) / unit) * unit;
+}
+
 struct TileJob {      // one 2-D tensor cut into 128x128 tiles
     const void* w;
     void* q;

@@ -204,9 +204,10 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_
 __global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const uint8_t* __restrict__ packed,
                                                            const uint8_t* __restrict__ scale,
                                                            uint8_t* __restrict__ y, float* __restrict__ tile_scale,
-                                                           int64_t in_dim, int tiles_in, int pairs_in, int total_pairs) {
+                                                           int64_t in_dim, int tiles_in, int pairs_in, int total_pairs,
+                                                           int chunk) {
     __shared__ uint32_t wave_smax[4][2];
-    const int32_t item = xcd_contiguous_item(total_pairs);
+    const int32_t item = xcd_chunked_item(total_pairs, chunk);
     if (item < 0) return;
     const int t = threadIdx.x;
     const int64_t ti = item / pairs_in, pj = item - ti * pairs_in;
@@ -330,8 +331,13 @@ extern "C" int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale
     if ((((uintptr_t)packed | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
     if (out_dim == 0 || in_dim == 0) return MQ_OK;
     const int64_t tiles_in = in_dim / 128, pairs_in = (tiles_in + 1) / 2, pairs = (out_dim / 128) * pairs_in;
-    if (xcd_grid(pairs) > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    hipLaunchKernelGGL(mxfp4_to_fp8_kernel, dim3((unsigned)xcd_grid(pairs)), dim3(256), 0, (hipStream_t)stream, packed, scale,
-                       (uint8_t*)y, tile_scale, in_dim, (int)tiles_in, (int)pairs_in, (int)pairs);
+    // An XCD takes whole 128-row bands when there are enough of them: the band's scale bytes are one contiguous run,
+    // and dealt out in smaller pieces every 128-byte line of them was fetched by four XCDs (measured: 0.625 bytes
+    // read per element against 0.531 algorithmic).
+    const int64_t chunk = (out_dim / 128 >= 2 * kXcds && pairs_in <= 4096) ? pairs_in : MQ_XCD_CHUNK;
+    const int64_t grid = xcd_grid_chunked(pairs, chunk);
+    if (grid > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    hipLaunchKernelGGL(mxfp4_to_fp8_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, packed, scale,
+                       (uint8_t*)y, tile_scale, in_dim, (int)tiles_in, (int)pairs_in, (int)pairs, (int)chunk);
     return mq_check_launch("mxfp4 to fp8");
 }
