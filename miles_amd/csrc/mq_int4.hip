@@ -286,9 +286,17 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
         // The zero point was not clamped, so rint(x/s) + z is an integer in [0, 16].  For such codes and every
         // bf16 scale up to 1e37 the reference's dequantize / requantize round trip in bf16 returns the code itself
         // (checked exhaustively on the CPU: all scales x all codes x all zero points), so the codes are final.
+        // rint through one add of 1.5 * 2^23: the low bits of the sum's pattern are the (signed) integer.  The zero point
+        // is added as an integer afterwards (inside the float add an odd zero point would turn the ties around);
+        // everything is arithmetic modulo 2^32, like the reference's int32 sum.
+        constexpr uint32_t kMagicBits = 0x4B400000u;
+        uint32_t magic_sum = 0;
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            word += (uint32_t)(__builtin_rintf(div_by_shared(f[i], s, ys)) + z) << (4 * i);
+        for (int i = 0; i < 8; i++) {
+            word += f2u(div_by_shared(f[i], s, ys) + 12582912.0f) << (4 * i);
+            magic_sum += kMagicBits << (4 * i);
+        }
+        word = word - magic_sum + (uint32_t)z * 0x11111111u;
     } else {
         // the chain as written, IEEE divisions: groups whose minimum lies above zero or far below it, huge scales
         float q[8];
