@@ -335,14 +335,20 @@ def packed_payload(args, weights, fp8_cfg, steps):
             "note": "one sync = quantize + build every bucket's flat payload (embeddings and norms included)"}
 
 
+def _lib_max_group():
+    from miles_amd import _lib
+
+    return _lib.MAX_GROUP
+
+
 def roofline(plan, jobs_meta):
     """Time every kernel launch of one sync (same launch partition as a step) with events on the launch stream."""
     spans = []
     done = 0
-    for mark in plan.jobs_done_at_bucket:
+    for mark in plan.submission_marks():
         a = done
         while a < mark:      # mq_run_jobs fuses up to 64 consecutive same-kind jobs into one launch
-            b = min(a + 64, mark)
+            b = min(a + _lib_max_group(), mark)
             spans.append((a, b))
             a = b
         done = max(done, mark)

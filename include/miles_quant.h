@@ -214,6 +214,9 @@ typedef struct mq_job {
      * read in place.  0 / 0 = one block (plain matrix).  rows_per_block must be a multiple of the tile height. */
     int64_t rows_per_block, block_stride;
 } mq_job;
+/* Consecutive jobs of one kind (and, for the flat kernels, of similar size) are fused into launches of up to
+ * MQ_MAX_GROUP tensors, counted from the first job of the call. */
+#define MQ_MAX_GROUP 64
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 
 /* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the

@@ -100,6 +100,8 @@ static int run_single(const mq_job& j, void* stream) {
     }
 }
 
+static_assert(kMaxGroup == MQ_MAX_GROUP, "the public group size must match the launch tables");
+
 static bool same_group(const mq_job& a, const mq_job& b) {
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
 }

@@ -40,6 +40,7 @@ class SyncPlan:
         self.jobs_done_at_bucket = jobs_done_at_bucket
         self.signature = signature
         self.replayable = replayable
+        self._marks: list[int] | None = None
         self._names: list[str] = []
         self._tensors: list[torch.Tensor] = []
         self._addresses: list[int] = []
@@ -163,10 +164,38 @@ class SyncPlan:
                 return list(map(torch.Tensor.data_ptr, tensors)) == self._addresses
         return weights_signature(weights) == self.signature
 
+    # a trailing launch smaller than this many elements is topped up with the next bucket's jobs
+    SMALL_LAUNCH_ELEMENTS = 64 * 1024 * 1024
+
+    def submission_marks(self) -> list[int]:
+        """Where each bucket's submission ends: at least after the bucket's own jobs.  `mq_run_jobs` fuses up to
+        `MAX_GROUP` jobs per launch, counted from the start of a submission, so a bucket of 330 small expert tensors
+        ends in a launch of ten, which mostly ramps up and down.  When that last launch would cover fewer than
+        `SMALL_LAUNCH_ELEMENTS` elements the submission runs on into the next bucket's jobs up to the full group (the
+        plan owns every output tensor, so running ahead costs nothing; measured on the 18 432-tensor MXFP8 sync:
+        14.6 -> 14.1 ms).  Buckets of large tensors are submitted as they are -- merging their launches made the
+        Qwen3-4B FP8 sync 1 % slower.  A cut never falls between NVFP4 jobs that share an amax record."""
+        if self._marks is None:
+            records, total, done, marks = self.batch._records, len(self.batch), 0, []
+            group = _lib.MAX_GROUP
+            for mark in self.jobs_done_at_bucket:
+                if mark > done:
+                    tail = (mark - done) % group
+                    tail_elements = sum(r[7] * r[8] for r in records[mark - tail:mark])
+                    if tail and tail_elements < self.SMALL_LAUNCH_ELEMENTS:
+                        mark = min(total, mark + group - tail)
+                        while (0 < mark < total and records[mark][0] == _lib.JOB_NVFP4
+                               and records[mark - 1][0] == _lib.JOB_NVFP4 and records[mark][5] == records[mark - 1][5]):
+                            mark += 1
+                    done = mark
+                marks.append(done)
+            self._marks = marks
+        return self._marks
+
     def replay(self) -> Iterator[Unit]:
         """Re-quantize into the plan's output tensors, bucket by bucket, and yield the buckets."""
         done = 0
-        for bucket, mark in zip(self.buckets, self.jobs_done_at_bucket):
+        for bucket, mark in zip(self.buckets, self.submission_marks()):
             self.batch.run_range(done, mark)
             done = max(done, mark)
             yield bucket

@@ -368,3 +368,32 @@ def test_sync_plan_matches_quick_and_full_forms():
     plan.replayable = False
     plan.remember(weights)
     assert not plan.matches(weights)
+
+
+def test_sync_plan_tops_up_small_trailing_launches_only():
+    from miles_amd import _lib, launch
+    from miles_amd.weight_update.sync_plan import SyncPlan
+
+    def plan_with(jobs, marks):
+        batch = launch.JobBatch()
+        batch._records = jobs
+        return SyncPlan(batch=batch, buckets=[[] for _ in marks], jobs_done_at_bucket=marks, signature=(), replayable=True)
+
+    def job(kind, elements, aux=None):
+        return (kind, 1, 1, 2, 3, aux, None, 1, elements, elements, 0, 0, 0, 0)
+
+    small = [job(_lib.JOB_MXFP8, 1 << 20) for _ in range(200)]
+    # 70 small jobs: one full group and a trailing launch of 6 -> topped up to 128; the next bucket is then covered up to 128
+    assert plan_with(small, [70, 120, 200]).submission_marks() == [128, 128, 200]
+    # a submission that ends on a group boundary stays where it is
+    assert plan_with(small, [64, 200]).submission_marks() == [64, 200]
+    big = [job(_lib.JOB_FP8_BLOCKWISE_CAST, 1 << 25) for _ in range(100)]
+    assert plan_with(big, [35, 70, 100]).submission_marks() == [35, 70, 100]          # 35 x 32 Mi elements: not small
+    # NVFP4 jobs that share an amax record (a gate/up pair) are never separated by a topped-up cut
+    pairs = []
+    for p in range(100):
+        pairs += [job(_lib.JOB_NVFP4, 1 << 16, aux=1000 + p), job(_lib.JOB_NVFP4, 1 << 16, aux=1000 + p),
+                  job(_lib.JOB_NVFP4, 1 << 16, aux=5000 + p)]
+    marks = plan_with(pairs, [9, 300]).submission_marks()
+    assert marks[0] >= 64 and pairs[marks[0]][5] != pairs[marks[0] - 1][5]
+    assert marks == [65, 300]      # index 64 is the second job of a pair: the cut moves to 65
