@@ -14,6 +14,7 @@
 // exceed the format maximum.  Lanes own 8 consecutive elements; 4 (or 2) neighbouring lanes form a block.
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
+#include "mq_group.hpp"
 
 namespace mq {
 
@@ -67,9 +68,9 @@ __device__ __forceinline__ void fq_store8(void* y, int64_t unit, const float f[8
 // MODE as above; LANES = lanes per block (4 for 1x32, 2 for 1x16)
 template <int DT, int MODE>
 __global__ __launch_bounds__(kFqThreads) void fake_quant_kernel(const void* __restrict__ x, void* __restrict__ y,
-                                                                int64_t units) {
+                                                                int64_t units, int chunk) {
     constexpr int LANES = MODE == 2 ? 2 : 4;
-    const int64_t unit = (int64_t)blockIdx.x * kFqThreads + threadIdx.x;
+    const int64_t unit = xcd_chunked_block(chunk) * kFqThreads + threadIdx.x;
     const bool live = unit < units;           // a block is a whole number of lanes: dead lanes never share one with live lanes
     float f[8];
     fq_load8<DT>(x, live ? unit : units - 1, f);
@@ -201,8 +202,8 @@ __device__ __forceinline__ void act_quant_unit(const float f[8], void* y, void* 
 
 template <int DT, int LANES, bool INPLACE>
 __global__ __launch_bounds__(kFqThreads) void act_quant_kernel(const void* x, void* y, void* scale, int64_t units,
-                                                               int flags) {
-    const int64_t base = (int64_t)blockIdx.x * (kFqThreads * kActUnits<INPLACE>) + threadIdx.x;
+                                                               int flags, int chunk) {
+    const int64_t base = xcd_chunked_block(chunk) * (kFqThreads * kActUnits<INPLACE>) + threadIdx.x;
     float f[kActUnits<INPLACE>][8];
     // a group is a whole number of lanes, so dead lanes never share one with live lanes; they re-read the last unit
 #pragma unroll
@@ -245,10 +246,12 @@ using namespace mq;
 
 template <int MODE>
 static void launch_fq(const void* x, int dtype, void* y, int64_t units, hipStream_t st) {
-    const dim3 grid((unsigned)((units + kFqThreads - 1) / kFqThreads)), blk(kFqThreads);
-    if (dtype == MQ_BF16) hipLaunchKernelGGL((fake_quant_kernel<MQ_BF16, MODE>), grid, blk, 0, st, x, y, units);
-    else if (dtype == MQ_F16) hipLaunchKernelGGL((fake_quant_kernel<MQ_F16, MODE>), grid, blk, 0, st, x, y, units);
-    else hipLaunchKernelGGL((fake_quant_kernel<MQ_F32, MODE>), grid, blk, 0, st, x, y, units);
+    const int64_t blocks = (units + kFqThreads - 1) / kFqThreads;
+    const int chunk = (int)flat_chunk(blocks);
+    const dim3 grid((unsigned)flat_padded(blocks, chunk)), blk(kFqThreads);
+    if (dtype == MQ_BF16) hipLaunchKernelGGL((fake_quant_kernel<MQ_BF16, MODE>), grid, blk, 0, st, x, y, units, chunk);
+    else if (dtype == MQ_F16) hipLaunchKernelGGL((fake_quant_kernel<MQ_F16, MODE>), grid, blk, 0, st, x, y, units, chunk);
+    else hipLaunchKernelGGL((fake_quant_kernel<MQ_F32, MODE>), grid, blk, 0, st, x, y, units, chunk);
 }
 
 extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, void* stream) {
@@ -259,7 +262,7 @@ extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, i
     if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
     if (numel == 0) return MQ_OK;
     const int64_t units = numel / 8;
-    if ((units + kFqThreads - 1) / kFqThreads > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if ((units + kFqThreads - 1) / kFqThreads > 0x7FFFFF00ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
     hipStream_t st = (hipStream_t)stream;
     if (mode == 0) launch_fq<0>(x, dtype, y, units, st);
     else if (mode == 1) launch_fq<1>(x, dtype, y, units, st);
@@ -269,11 +272,13 @@ extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, i
 
 template <int DT, bool INPLACE>
 static void launch_act(const void* x, void* y, void* scale, int64_t units, int lanes, int flags, hipStream_t st) {
-    const dim3 grid((unsigned)((units + kFqThreads * kActUnits<INPLACE> - 1) / (kFqThreads * kActUnits<INPLACE>))), blk(kFqThreads);
-    if (lanes == 16) hipLaunchKernelGGL((act_quant_kernel<DT, 16, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags);
-    else if (lanes == 8) hipLaunchKernelGGL((act_quant_kernel<DT, 8, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags);
-    else if (lanes == 4) hipLaunchKernelGGL((act_quant_kernel<DT, 4, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags);
-    else hipLaunchKernelGGL((act_quant_kernel<DT, 2, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags);
+    const int64_t blocks = (units + kFqThreads * kActUnits<INPLACE> - 1) / (kFqThreads * kActUnits<INPLACE>);
+    const int chunk = 1;      // this kernel streams 1-2 % faster in plain block order (measured), unlike its neighbours
+    const dim3 grid((unsigned)flat_padded(blocks, chunk)), blk(kFqThreads);
+    if (lanes == 16) hipLaunchKernelGGL((act_quant_kernel<DT, 16, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags, chunk);
+    else if (lanes == 8) hipLaunchKernelGGL((act_quant_kernel<DT, 8, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags, chunk);
+    else if (lanes == 4) hipLaunchKernelGGL((act_quant_kernel<DT, 4, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags, chunk);
+    else hipLaunchKernelGGL((act_quant_kernel<DT, 2, INPLACE>), grid, blk, 0, st, x, y, scale, units, flags, chunk);
 }
 template <bool INPLACE>
 static void launch_act_dt(const void* x, int dtype, void* y, void* scale, int64_t units, int lanes, int flags, hipStream_t st) {
@@ -296,7 +301,7 @@ extern "C" int mq_fp8_act_quant(const void* x, int dtype, void* y, void* scale, 
     const bool shaped = block == 16 || block == 32 || block == 64 || block == 128;
     const bool aligned = ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & (inplace ? 15 : 7)) == 0 &&
                          ((flags & MQ_ACT_SCALE_E8M0) || ((uintptr_t)scale & 3) == 0);
-    if (shaped && aligned && (units + kFqThreads - 1) / kFqThreads <= 0x7FFFFFF0ll) {
+    if (shaped && aligned && (units + kFqThreads - 1) / kFqThreads <= 0x7FFFFF00ll) {
         if (inplace) launch_act_dt<true>(x, dtype, y, scale, units, block / 8, flags, st);
         else launch_act_dt<false>(x, dtype, y, scale, units, block / 8, flags, st);
     } else {

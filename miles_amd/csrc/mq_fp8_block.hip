@@ -242,13 +242,16 @@ struct DequantJob {
 struct DequantTable {
     int32_t n;
     int32_t max_blocks;
+    int32_t chunk;           // blocks per XCD chunk (xcd_chunked_block); max_blocks is a multiple of 8 * chunk
+    int32_t pad;
     DequantJob job[kMaxGroup];
 };
 
 __global__ __launch_bounds__(kDqThreads) void fp8_dequant_kernel(const DequantTable tab) {
     const DequantJob& job = tab.job[blockIdx.y];
-    const uint32_t base = blockIdx.x * (kDqThreads * kDqUnroll);
-    if (base >= job.units) return;
+    const int64_t base64 = xcd_chunked_block(tab.chunk) * (kDqThreads * kDqUnroll);
+    if (base64 >= job.units) return;
+    const uint32_t base = (uint32_t)base64;
     u32x2 in[kDqUnroll];
 #pragma unroll
     for (int i = 0; i < kDqUnroll; i++) {
@@ -422,6 +425,9 @@ int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st) {
         if (b > mx) mx = b;
     }
     if (mx == 0) return MQ_OK;
+    const int64_t chunk = flat_chunk(mx);
+    mx = flat_padded(mx, chunk);
+    tab.chunk = (int32_t)chunk;
     tab.max_blocks = (int32_t)mx;
     hipLaunchKernelGGL(fp8_dequant_kernel, dim3((unsigned)mx, (unsigned)n), dim3(kDqThreads), 0, st, tab);
     return mq_check_launch("fp8 block dequant");

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTa
     uint16_t* __restrict__ scale = (uint16_t*)job.s;
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll);
+    const int64_t base = flat_block(tab) * (kI4Threads * kI4Unroll);
     if (base >= total_units) return;
     u32x4 v[kI4Unroll];
 #pragma unroll
@@ -337,9 +337,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const u
                                                                          uint32_t* __restrict__ packed,
                                                                          uint16_t* __restrict__ scale_out,
                                                                          uint8_t* __restrict__ zero_out,
-                                                                         int64_t total_units) {
+                                                                         int64_t total_units, int chunk) {
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kI4Threads * kI4Unroll) + t;
+    const int64_t base = xcd_chunked_block(chunk) * (kI4Threads * kI4Unroll) + t;
     // a group is a whole number of lanes, so dead lanes never share one with live lanes; they re-read the last unit
     u32x4 v[kI4Unroll];
 #pragma unroll
@@ -384,8 +384,8 @@ constexpr int kI4UnpackUnroll = MQ_I4_UNPACK_UNROLL;   // words per lane, 256 la
 template <int SDT>
 __global__ __launch_bounds__(256) void int4_unpack_kernel(const uint32_t* __restrict__ packed,
                                                           const void* __restrict__ scale, uint16_t* __restrict__ y,
-                                                          int64_t words, int group_shift) {
-    const int64_t base = (int64_t)blockIdx.x * (256 * kI4UnpackUnroll) + threadIdx.x;
+                                                          int64_t words, int group_shift, int chunk) {
+    const int64_t base = xcd_chunked_block(chunk) * (256 * kI4UnpackUnroll) + threadIdx.x;
     uint32_t word[kI4UnpackUnroll], sraw[kI4UnpackUnroll];
     // every load is issued before the first use: lanes past the end re-read the last word instead of branching
 #pragma unroll
@@ -497,15 +497,18 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     if (blocks > mq_grid_cap() * 4) blocks = mq_grid_cap() * 4;
     const int wpg = group / 8;
     if (dtype == MQ_BF16 && (group == 128 || group == 64 || group == 32)) {
-        const int64_t units = M * (K / 8), fblocks = (units + kI4Threads * kI4Unroll - 1) / (kI4Threads * kI4Unroll);
+        const int64_t units = M * (K / 8);
+        int64_t fblocks = (units + kI4Threads * kI4Unroll - 1) / (kI4Threads * kI4Unroll);
+        const int chunk = (int)flat_chunk(fblocks);
+        fblocks = flat_padded(fblocks, chunk);
         if (fblocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
         const dim3 grid((unsigned)fblocks), blk(kI4Threads);
         if (group == 128)
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
         else if (group == 64)
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
         else
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units);
+            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
     } else if (dtype == MQ_BF16)
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
     else if (dtype == MQ_F16)
@@ -532,15 +535,18 @@ extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, 
     if (K % 8 == 0 && group % 8 == 0 && (upg & (upg - 1)) == 0 && ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0) {
         int shift = 0;
         while ((1 << shift) < upg) shift++;
-        const int64_t words = M * (K / 8), blocks = (words + 256 * kI4UnpackUnroll - 1) / (256 * kI4UnpackUnroll);
+        const int64_t words = M * (K / 8);
+        int64_t blocks = (words + 256 * kI4UnpackUnroll - 1) / (256 * kI4UnpackUnroll);
+        const int chunk = (int)flat_chunk(blocks);
+        blocks = flat_padded(blocks, chunk);
         if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
         const dim3 grid((unsigned)blocks), blk(256);
         if (scale_dtype == MQ_BF16)
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_BF16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_BF16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
         else if (scale_dtype == MQ_F16)
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
         else
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F32>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift);
+            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F32>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
         return mq_check_launch("int4 unpack");
     }
     int64_t blocks = (M * K + 255) / 256;

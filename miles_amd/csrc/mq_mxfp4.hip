@@ -65,7 +65,7 @@ __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const FlatTable 
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kM4Threads * kM4Unroll);
+    const int64_t base = flat_block(tab) * (kM4Threads * kM4Unroll);
     if (base >= total_units) return;
     u32x4 v[kM4Unroll];
 #pragma unroll
@@ -153,8 +153,8 @@ __device__ __forceinline__ uint32_t hw_e2m1x2_to_bf16x2(uint32_t word, float fac
 __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint32_t* __restrict__ packed,
                                                             const uint8_t* __restrict__ scale,
                                                             uint16_t* __restrict__ y, int64_t units,
-                                                            int group_shift) {
-    const int64_t base = (int64_t)blockIdx.x * (256 * kM4DqUnroll) + threadIdx.x;
+                                                            int group_shift, int chunk) {
+    const int64_t base = xcd_chunked_block(chunk) * (256 * kM4DqUnroll) + threadIdx.x;
     uint32_t word[kM4DqUnroll], s[kM4DqUnroll];
 #pragma unroll
     for (int i = 0; i < kM4DqUnroll; i++) {
@@ -310,10 +310,12 @@ extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, voi
         int shift = 0;
         while ((1 << shift) < upg) shift++;
         const int64_t units = bytes / 4;
-        const int64_t blocks = (units + 256 * kM4DqUnroll - 1) / (256 * kM4DqUnroll);
+        int64_t blocks = (units + 256 * kM4DqUnroll - 1) / (256 * kM4DqUnroll);
+        const int64_t chunk = flat_chunk(blocks);
+        blocks = flat_padded(blocks, chunk);
         if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
         hipLaunchKernelGGL(mxfp4_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)packed, scale,
-                           (uint16_t*)y, units, shift);
+                           (uint16_t*)y, units, shift, (int)chunk);
         return mq_check_launch("mxfp4 dequant");
     }
     int64_t blocks = (bytes + 255) / 256;

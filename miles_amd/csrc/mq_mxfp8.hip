@@ -40,7 +40,7 @@ __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const FlatTable 
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kMxThreads * kMxUnroll);
+    const int64_t base = flat_block(tab) * (kMxThreads * kMxUnroll);
     if (base >= total_units) return;
     u32x4 v[kMxUnroll];
 #pragma unroll

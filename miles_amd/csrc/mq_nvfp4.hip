@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
     const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = (int64_t)blockIdx.x * (kNvThreads * kNvUnroll);
+    const int64_t base = flat_block(tab) * (kNvThreads * kNvUnroll);
     if (base >= total_units) return;
     u32x4 v[kNvUnroll];
 #pragma unroll
@@ -357,9 +357,9 @@ template <int DT, int FOS>
 __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* __restrict__ x,
                                                                const float* __restrict__ amax_ptr,
                                                                uint16_t* __restrict__ y, int64_t total_units,
-                                                               float numer, float inv_numer) {
+                                                               float numer, float inv_numer, int chunk) {
     const int t = threadIdx.x;
-    const int64_t unit = (int64_t)blockIdx.x * kNvThreads + t;
+    const int64_t unit = xcd_chunked_block(chunk) * kNvThreads + t;
     const bool live = unit < total_units;
     const u32x4 v = ld16(x + (live ? unit : total_units - 1) * 8);
     const float amax = *amax_ptr;
@@ -524,7 +524,10 @@ extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y
     if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
     if (flags & ~(MQ_NVFP4_4OVER6 | MQ_NVFP4_ERR_MSE | MQ_NVFP4_ERR_FP16)) return mq_fail(MQ_ERR_ARG, "unknown NVFP4 flag");
     if (numel == 0) return MQ_OK;
-    const int64_t units = numel / 8, blocks = (units + kNvThreads - 1) / kNvThreads;
+    const int64_t units = numel / 8;
+    int64_t blocks = (units + kNvThreads - 1) / kNvThreads;
+    const int chunk = (int)flat_chunk(blocks);
+    blocks = flat_padded(blocks, chunk);
     if (blocks > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
     const float numer = (float)e4m3_max * 6.0f, inv_numer = (float)(1.0 / (double)(6 * e4m3_max));
     const dim3 grid((unsigned)blocks), blk(kNvThreads);
@@ -532,7 +535,7 @@ extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y
     const uint16_t* xi = (const uint16_t*)x;
     uint16_t* yo = (uint16_t*)y;
     const int fos = (flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0;
-#define MQ_QDQ_LAUNCH(DT, FOS) hipLaunchKernelGGL((nvfp4_qdq_kernel<DT, FOS>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer)
+#define MQ_QDQ_LAUNCH(DT, FOS) hipLaunchKernelGGL((nvfp4_qdq_kernel<DT, FOS>), grid, blk, 0, st, xi, amax, yo, units, numer, inv_numer, chunk)
 #define MQ_QDQ_SWITCH(DT)                           \
     switch (fos) {                                  \
         case 0: MQ_QDQ_LAUNCH(DT, 0); break;        \
