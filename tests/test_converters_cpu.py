@@ -128,3 +128,130 @@ def test_mxfp8_source_detection_and_scale_relabelling():
     assert MX._load_source_scale_u8(weights, "a.weight", w, {"a.weight_scale_inv": "s"}, ".", "cpu", "s")[1] is None
     with pytest.raises(ValueError, match="Expected key ending"):
         MX._strip_weight_suffix("a.bias")
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# NVFP4 checkpoint scope, the scenarios of the reference's tests/fast/test_nvfp4_scope.py with the numeric kernels
+# replaced by shape-correct stand-ins (the kernels themselves are covered by the GPU parity tests)
+LAYER_ROOTS = ("model.layers", "language_model.model.layers", "model.language_model.layers", "language_model.layers")
+
+
+@pytest.fixture
+def stand_in_quantizers(monkeypatch):
+    calls = []
+
+    def result(w):
+        rows, cols = w.shape
+        return (torch.zeros((rows, cols // 2), dtype=torch.uint8), torch.ones((rows, cols // 16)).to(torch.float8_e4m3fn),
+                torch.tensor(1.0))
+
+    monkeypatch.setattr(NV, "quantize_nvfp4", lambda w: (calls.append("single"), result(w))[1])
+    monkeypatch.setattr(NV, "nvfp4_quantize_1d_pair", lambda g, u: (calls.append("pair"), (result(g), result(u)))[1])
+    return calls
+
+
+def _run_nvfp4_conversion(tmp_path, config, shards, **kwargs):
+    src, dst = tmp_path / "src", tmp_path / "dst"
+    src.mkdir()
+    (src / "config.json").write_text(json.dumps(config))
+    for filename, tensors in shards.items():
+        safetensors.torch.save_file(tensors, src / filename)
+    NV.convert_nvfp4(str(src), str(dst), "cpu", **kwargs)
+    index = json.loads((dst / "model.safetensors.index.json").read_text())
+    out = {}
+    for filename in set(index["weight_map"].values()):
+        tensors = safetensors.torch.load_file(dst / filename)
+        assert all(index["weight_map"][n] == filename for n in tensors)
+        out.update(tensors)
+    assert set(index["weight_map"]) == set(out)
+    assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for t in out.values())
+    cfg = json.loads((dst / "config.json").read_text())
+    ignore = cfg["quantization_config"]["ignore"]
+    assert ignore == json.loads((dst / "hf_quant_config.json").read_text())["quantization"]["exclude_modules"]
+    return out, ignore, cfg
+
+
+def _kept_as_is(out, name, original, ignore):
+    assert out[name].dtype == original.dtype and torch.equal(out[name], original)
+    module = name.removesuffix(".weight")
+    assert not any(f"{module}.{s}" in out for s in ("weight_scale", "weight_scale_2", "input_scale"))
+    assert any(module == rule or module.startswith(rule.rstrip(".") + ".") for rule in ignore)
+
+
+@pytest.mark.parametrize("root", LAYER_ROOTS)
+def test_nvfp4_selector_stays_inside_the_language_decoder(root):
+    w = torch.ones((2, 16), dtype=torch.bfloat16)
+    e = ".mlp.experts.0."
+    assert NV.should_quantize(f"{root}.69{e}down_proj.weight", w, num_hidden_layers=70)
+    assert not NV.should_quantize(f"{root}.70{e}down_proj.weight", w, num_hidden_layers=70)
+    assert not NV.should_quantize(f"{root}.0.mlp.shared_experts.down_proj.weight", w)
+    assert not NV.should_quantize(f"{root}.0.mlp.shared_expert.experts.0.down_proj.weight", w)
+    assert not NV.should_quantize(f"{root}.0.mlp.down_proj.weight", w)
+    assert not NV.should_quantize(f"{root}.0{e}down_proj.weight", w, ("down_proj",))
+
+
+@pytest.mark.parametrize("root", ["model.mtp.layers", "model.mtp_layers", "mtp.layers", "visual.layers", "audio_encoder.layers",
+                                  "speech_embeddings.layers", "vision.model.layers", "model.visual.layers"])
+def test_nvfp4_selector_never_validates_other_towers(root):
+    # 7 columns would raise inside the decoder; an excluded tower must be turned away before that check
+    assert not NV.should_quantize(f"{root}.0.mlp.experts.0.gate_proj.weight", torch.ones((2, 7)))
+
+
+def test_nvfp4_multimodal_checkpoint_with_a_pair_split_over_two_shards(tmp_path, stand_in_quantizers):
+    config = {"model_type": "mimo_v2", "num_hidden_layers": 70, "num_nextn_predict_layers": 1, "vision_config": {},
+              "audio_config": {}}
+    e = ".mlp.experts.0."
+    gate, up, down = (f"model.layers.69{e}{p}.weight" for p in ("gate_proj", "up_proj", "down_proj"))
+    outside = [f"model.mtp.layers.0{e}gate_proj.weight", f"model.layers.70{e}gate_proj.weight",
+               f"visual.layers.0{e}gate_proj.weight", f"audio_encoder.layers.0{e}gate_proj.weight",
+               f"speech_embeddings.layers.0{e}gate_proj.weight", "model.mtp.layers.0.block_sparse_moe.experts.0.w1.weight",
+               "audio_encoder.layers.0.moe.experts.0.w2.weight", "model.layers.69.mlp.shared_experts.gate_proj.weight",
+               "model.layers.69.self_attn.q_proj.weight", "lm_head.weight"]
+    kept = {n: torch.full((2, 16), i + 1, dtype=torch.bfloat16) for i, n in enumerate(outside)}
+    kept["model.mtp.layers.0.mlp.experts.gate_up_proj.weight"] = torch.ones((2, 2, 16), dtype=torch.bfloat16)
+    w = torch.ones((2, 16), dtype=torch.bfloat16)
+    out, ignore, cfg = _run_nvfp4_conversion(tmp_path, config, {"a.safetensors": {gate: w, down: w.clone(), **kept},
+                                                                "b.safetensors": {up: w}})
+    assert sorted(stand_in_quantizers) == ["pair", "single"]
+    assert cfg["model_type"] == "mimo_v2" and cfg["num_hidden_layers"] == 70
+    for name in (gate, up, down):
+        module = name.removesuffix(".weight")
+        assert out[name].dtype == torch.uint8 and out[name].shape == (2, 8)
+        assert all(f"{module}.{s}" in out for s in ("weight_scale", "weight_scale_2", "input_scale"))
+        assert not any(module == rule or module.startswith(rule.rstrip(".") + ".") for rule in ignore)
+    for name, original in kept.items():
+        _kept_as_is(out, name, original, ignore)
+        if ".experts." in name:
+            assert name.split(".experts.", 1)[0] + ".experts" in ignore
+
+
+@pytest.mark.parametrize("root", LAYER_ROOTS[1:])
+def test_nvfp4_depth_comes_from_the_nested_text_config(tmp_path, stand_in_quantizers, root):
+    config = {"num_hidden_layers": 99, "text_config": {"num_hidden_layers": 3, "quantization_config": {"quant_method": "fp8"}}}
+    tensors = {f"{root}.{i}.mlp.experts.0.down_proj.weight": torch.full((2, 16), i + 1, dtype=torch.bfloat16) for i in range(4)}
+    out, ignore, cfg = _run_nvfp4_conversion(tmp_path, config, {"model.safetensors": tensors},
+                                             num_layers_at_start_in_bf16=1, num_layers_at_end_in_bf16=1)
+    assert stand_in_quantizers == ["single"]
+    nested = cfg["text_config"]["quantization_config"]
+    assert nested["ignore"] == ignore and nested["quant_algo"] == "NVFP4" and nested["quant_method"] == "modelopt"
+    for name, original in tensors.items():
+        if name == f"{root}.1.mlp.experts.0.down_proj.weight":
+            assert out[name].dtype == torch.uint8
+        else:
+            _kept_as_is(out, name, original, ignore)
+    assert {f"{root}.0.", f"{root}.2."}.issubset(ignore)
+    assert not any(rule.startswith("model.layers.") for rule in ignore)
+
+
+@pytest.mark.parametrize("prefix,eligible", [
+    ("decoder", True), ("module.module.decoder", True), ("language_model.decoder", True),
+    ("module.language_model.decoder", True), ("mtp", False), ("module.module.mtp", False), ("mtp.decoder", False),
+    ("mtp.layers.0.transformer_layer.decoder", False), ("vision_model.decoder", False), ("audio_encoder.decoder", False),
+    ("module.vision_model.decoder", False)])
+def test_runtime_nvfp4_quantizer_only_takes_the_main_language_decoder(monkeypatch, prefix, eligible):
+    from miles_amd.megatron_to_hf.processors import quantizer_nvfp4 as Q
+
+    original, converted = [], [("quantized", torch.zeros(1))]
+    monkeypatch.setattr(Q, "_quantize_moe_params", lambda *_: converted)
+    got = Q.quantize_params_nvfp4(None, f"{prefix}.layers.0.mlp.experts.linear_fc2.weight0", original, {"quant_method": "nvfp4"})
+    assert got is (converted if eligible else original)
