@@ -9,7 +9,6 @@ miles/backends/megatron_utils/megatron_to_hf/processors/quantizer_nvfp4.py: igno
 from __future__ import annotations
 
 import re
-from functools import lru_cache
 
 import torch
 
@@ -17,136 +16,133 @@ from miles_amd.utils.nvfp4 import NVFP4_GROUP_SIZE, nvfp4_quantize_1d, nvfp4_qua
 
 from ._names import in_bf16_head_or_tail, named_in_extra_high_precision, parse_layer_param
 
-GATED_PAIR_SUFFIXES = {
-    ".gate_proj.weight": "gate",
-    ".up_proj.weight": "up",
-    ".w1.weight": "gate",
-    ".w3.weight": "up",
-}
+# HF suffix -> role inside a gated MLP; the two roles of one expert share a global amax
+GATED_PAIR_SUFFIXES = {".gate_proj.weight": "gate", ".up_proj.weight": "up", ".w1.weight": "gate", ".w3.weight": "up"}
+_FLOAT_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
 
 # only the main language decoder: MTP layers and modality towers stay in high precision
 _DECODER = r"(?:module\.)*(?:language_model\.)?decoder\.layers\.(\d+)\.(.+)"
 
 
-def _as_list(value) -> list[str]:
-    if not value:
-        return []
-    return [value] if isinstance(value, str) else list(value)
+class _IgnoreRules:
+    """The `ignore` / `exclude_modules` lists of a quantization config.  A plain rule covers the module it names and
+    everything below it; a rule starting with `re:` is a regular expression matched at the start of the name."""
 
+    _cache: dict[tuple[str, ...], "_IgnoreRules"] = {}
 
-def _get_ignore_rules(quantization_config) -> list[str]:
-    rules = _as_list(quantization_config.get("ignore", []))
-    return rules + [r for r in _as_list(quantization_config.get("exclude_modules", [])) if r not in rules]
+    def __init__(self, rules: tuple[str, ...]) -> None:
+        self.plain = frozenset(r for r in rules if not r.startswith("re:"))
+        self.patterns = [re.compile(r[3:]) for r in rules if r.startswith("re:")]
 
+    @classmethod
+    def of(cls, quantization_config) -> "_IgnoreRules":
+        merged: list[str] = []
+        for key in ("ignore", "exclude_modules"):
+            value = quantization_config.get(key) or []
+            for rule in ([value] if isinstance(value, str) else value):
+                if rule not in merged:
+                    merged.append(rule)
+        key = tuple(merged)
+        if key not in cls._cache:
+            if len(cls._cache) >= 16:
+                cls._cache.clear()
+            cls._cache[key] = cls(key)
+        return cls._cache[key]
 
-@lru_cache(maxsize=16)
-def _literal_ignore_rules(ignore_rules: tuple[str, ...]) -> frozenset[str] | None:
-    """A hashable set when no rule is a regex (then matching is a walk up the dotted name)."""
-    if any(rule.startswith("re:") for rule in ignore_rules):
-        return None
-    return frozenset(ignore_rules)
+    def __bool__(self) -> bool:
+        return bool(self.plain or self.patterns)
 
-
-def _is_ignored(name: str, ignore_rules: list[str], literal_rules: frozenset[str] | None = None) -> bool:
-    if literal_rules is not None:
-        while True:
-            if name in literal_rules:
-                return True
-            name, dot, _ = name.rpartition(".")
-            if not dot:
-                return False
-    for rule in ignore_rules:
-        if rule.startswith("re:"):
-            if re.match(rule[3:], name):
-                return True
-        elif name == rule or name.startswith(f"{rule}."):
+    def covers(self, name: str) -> bool:
+        if any(p.match(name) for p in self.patterns):
             return True
-    return False
+        node = name                      # walk up the dotted path: a.b.c.weight, a.b.c, a.b, a
+        while node:
+            if node in self.plain:
+                return True
+            node = node.rpartition(".")[0]
+        return False
 
 
 def quantize_params_nvfp4(args, megatron_name, converted_named_params, quantization_config):
     assert quantization_config is not None
     assert quantization_config.get("quant_algo") == "NVFP4" or quantization_config.get("quant_method") == "nvfp4"
-    if args is not None and bool(getattr(args, "fp4_param", False) or getattr(args, "fp4_param_gather", False)):
+    if args is not None and (getattr(args, "fp4_param", False) or getattr(args, "fp4_param_gather", False)):
         raise NotImplementedError("fp4-param-gather is unsupported for Miles NVFP4 checkpoint export.")
     if named_in_extra_high_precision(args, megatron_name):
         return converted_named_params
-    p = parse_layer_param(megatron_name, decoder=_DECODER, mtp=None, anchored=True)
-    if p is None or in_bf16_head_or_tail(args, p.layer_idx):
+    where = parse_layer_param(megatron_name, decoder=_DECODER, mtp=None, anchored=True)
+    if where is None or in_bf16_head_or_tail(args, where.layer_idx):
         return converted_named_params
-    if p.routed_expert_linear in ("linear_fc1", "linear_fc2"):
-        return _quantize_moe_params(converted_named_params, _get_ignore_rules(quantization_config))
-    return converted_named_params
+    if where.routed_expert_linear not in ("linear_fc1", "linear_fc2"):
+        return converted_named_params
+    return _quantize_moe_params(converted_named_params, _IgnoreRules.of(quantization_config))
 
 
-def _quantize_moe_params(converted_named_params, ignore_rules):
-    literal_rules = _literal_ignore_rules(tuple(ignore_rules))
-    wanted = [_should_quantize_param(n, t, ignore_rules, literal_rules) for n, t in converted_named_params]
-
-    # gate/up tensors of one expert share one global amax: collect complete pairs first
-    pairs: dict[str, dict[str, tuple[str, torch.Tensor]]] = {}
-    for (name, tensor), want in zip(converted_named_params, wanted):
-        base, role = _split_gated_pair_name(name)
-        if base is None or not want:
-            continue
-        roles = pairs.setdefault(base, {})
-        if role in roles:
-            raise ValueError(f"NVFP4 requires a single complete gate/up pair per conversion batch; "
-                             f"found duplicate {role} tensor for {base}.")
-        roles[role] = (name, tensor)
-
-    paired = {}
-    for base, roles in pairs.items():
-        if set(roles) != {"gate", "up"}:
-            present = ", ".join(sorted(roles))
-            raise ValueError(f"NVFP4 requires gate/up tensors to be quantized together so they can share "
-                             f"one global amax; found only {{{present}}} for {base}.")
-        (gate_name, gate), (up_name, up) = roles["gate"], roles["up"]
-        paired[gate_name], paired[up_name] = nvfp4_quantize_1d_pair(gate, up)
-
-    out = []
-    for (name, tensor), want in zip(converted_named_params, wanted):
-        if not want:
-            out.append((name, tensor))
-            continue
-        qweight, block_scale, weight_scale_2 = paired[name] if name in paired else quantize_nvfp4(tensor)
-        out.append((name, qweight))
-        out.append((name.replace(".weight", ".weight_scale"), block_scale))
-        out.append((name.replace(".weight", ".weight_scale_2"), weight_scale_2))
-    return out
-
-
-def _should_quantize_param(name, weight, ignore_rules, literal_rules=None):
-    if ignore_rules and _is_ignored(name, ignore_rules, literal_rules):
+def _eligible(name: str, weight: torch.Tensor, rules) -> bool:
+    """A floating-point `.weight` matrix that no ignore rule covers; a last dimension that 1x16 blocks do not divide
+    is an error, not a reason to skip."""
+    if rules and rules.covers(name):
         return False
-    if not name.endswith(".weight"):
+    if not name.endswith(".weight") or weight.dtype not in _FLOAT_DTYPES or weight.dim() < 2:
         return False
-    if weight.dtype not in (torch.float16, torch.bfloat16, torch.float32) or weight.dim() < 2:
-        return False
-    if weight.shape[-1] % NVFP4_GROUP_SIZE != 0:
+    if weight.shape[-1] % NVFP4_GROUP_SIZE:
         raise ValueError(f"Last dim {weight.shape[-1]} must be divisible by {NVFP4_GROUP_SIZE} for NVFP4 ({name}).")
     return True
 
 
 def _split_gated_pair_name(name: str):
+    """(`<expert prefix>`, "gate" | "up") for a gated-MLP input projection, (None, None) for anything else."""
     for suffix, role in GATED_PAIR_SUFFIXES.items():
         if name.endswith(suffix):
             return name[: -len(suffix)], role
     return None, None
 
 
-def _quantize_nvfp4_1d(weight: torch.Tensor):
-    """1x16 tiles: (uint8 [M, K/2], float8_e4m3fn [M, K/16], float32 [])."""
-    weight = weight.contiguous()
-    if weight.shape[1] % NVFP4_GROUP_SIZE != 0:
-        raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {weight.shape[1]}.")
-    return nvfp4_quantize_1d(weight)
+def _quantize_moe_params(converted_named_params, ignore_rules):
+    """Quantize every eligible tensor of one conversion batch.  gate / up of an expert go through the paired
+    quantizer (one amax over both); a batch that holds only one of the two, or one of them twice, is refused."""
+    if not isinstance(ignore_rules, _IgnoreRules):
+        ignore_rules = _IgnoreRules(tuple(ignore_rules or ()))
+    chosen = {i for i, (name, tensor) in enumerate(converted_named_params) if _eligible(name, tensor, ignore_rules)}
+
+    by_expert: dict[str, dict[str, int]] = {}
+    for i in sorted(chosen):
+        prefix, role = _split_gated_pair_name(converted_named_params[i][0])
+        if prefix is None:
+            continue
+        slots = by_expert.setdefault(prefix, {})
+        if role in slots:
+            raise ValueError(f"NVFP4 requires a single complete gate/up pair per conversion batch; "
+                             f"found duplicate {role} tensor for {prefix}.")
+        slots[role] = i
+
+    results: dict[int, tuple] = {}
+    for prefix, slots in by_expert.items():
+        if len(slots) != 2:
+            raise ValueError(f"NVFP4 requires gate/up tensors to be quantized together so they can share "
+                             f"one global amax; found only {{{', '.join(sorted(slots))}}} for {prefix}.")
+        gate, up = slots["gate"], slots["up"]
+        results[gate], results[up] = nvfp4_quantize_1d_pair(converted_named_params[gate][1], converted_named_params[up][1])
+
+    emitted = []
+    for i, (name, tensor) in enumerate(converted_named_params):
+        if i not in chosen:
+            emitted.append((name, tensor))
+            continue
+        codes, block_scale, global_scale = results[i] if i in results else quantize_nvfp4(tensor)
+        emitted += [(name, codes), (name.replace(".weight", ".weight_scale"), block_scale),
+                    (name.replace(".weight", ".weight_scale_2"), global_scale)]
+    return emitted
 
 
 def quantize_nvfp4(weight: torch.Tensor):
-    if weight.dim() == 2:
-        return _quantize_nvfp4_1d(weight)
+    """(uint8 [.., M, K/2], float8_e4m3fn [.., M, K/16], float32 global scale) for a matrix or a stack of matrices,
+    each matrix of a stack with its own global scale."""
     if weight.dim() == 3:
-        parts = [_quantize_nvfp4_1d(weight[i]) for i in range(weight.shape[0])]
-        return tuple(torch.stack([p[k] for p in parts], dim=0) for k in range(3))
-    raise ValueError(f"Unsupported weight rank {weight.dim()} for NVFP4 quantization.")
+        per_matrix = [quantize_nvfp4(weight[i]) for i in range(weight.shape[0])]
+        return tuple(torch.stack(field, dim=0) for field in zip(*per_matrix))
+    if weight.dim() != 2:
+        raise ValueError(f"Unsupported weight rank {weight.dim()} for NVFP4 quantization.")
+    if weight.shape[1] % NVFP4_GROUP_SIZE:
+        raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {weight.shape[1]}.")
+    return nvfp4_quantize_1d(weight.contiguous())

@@ -79,44 +79,43 @@ def should_quantize(name: str, weight: torch.Tensor, skip_weight_substrings: tup
     return True
 
 
+_GROUP_DEFAULTS = {"dynamic": False, "num_bits": 4, "type": "float"}
+
+
 def _update_quantization_config(cfg: dict, ignore_list: list[str]) -> None:
-    q = cfg.get("quantization_config")
-    if not isinstance(q, dict):
-        q = {}
-    q.update(quant_algo="NVFP4", quant_method="modelopt", group_size=NVFP4_GROUP_SIZE, ignore=ignore_list)
-    q.setdefault("kv_cache_scheme", DEFAULT_KV_CACHE_SCHEME)
-    groups = q.get("config_groups")
-    if isinstance(groups, dict):
-        for group in groups.values():
-            if not isinstance(group, dict):
-                continue
+    """Stamp the NVFP4 policy on `quantization_config` (created if missing or malformed), keep what the source said
+    about the KV cache, bring every compressed-tensors style group to 1x16 float4, and repeat for a nested
+    `text_config` that carries a policy of its own (a composite config must not keep a stale one)."""
+    policy = cfg["quantization_config"] if isinstance(cfg.get("quantization_config"), dict) else {}
+    policy["quant_algo"], policy["quant_method"] = "NVFP4", "modelopt"
+    policy["group_size"], policy["ignore"] = NVFP4_GROUP_SIZE, ignore_list
+    policy.setdefault("kv_cache_scheme", DEFAULT_KV_CACHE_SCHEME)
+    groups = policy.get("config_groups")
+    for group in (groups.values() if isinstance(groups, dict) else ()):
+        if isinstance(group, dict):
             group.setdefault("targets", ["Linear"])
-            for key in ("input_activations", "weights"):
-                section = group.get(key)
-                if isinstance(section, dict):
-                    section.setdefault("dynamic", False)
-                    section.setdefault("num_bits", 4)
-                    section.setdefault("type", "float")
-                    section["group_size"] = NVFP4_GROUP_SIZE
-    cfg["quantization_config"] = q
-    text = cfg.get("text_config")
-    if isinstance(text, dict) and "quantization_config" in text:
-        _update_quantization_config(text, ignore_list)   # composite configs must not keep a stale policy
+            for side in ("input_activations", "weights"):
+                if isinstance(group.get(side), dict):
+                    for field, default in _GROUP_DEFAULTS.items():
+                        group[side].setdefault(field, default)
+                    group[side]["group_size"] = NVFP4_GROUP_SIZE
+    cfg["quantization_config"] = policy
+    nested = cfg.get("text_config")
+    if isinstance(nested, dict) and "quantization_config" in nested:
+        _update_quantization_config(nested, ignore_list)
 
 
 def _write_hf_quant_config(output_path: str, ignore_list: list[str], input_path: str) -> None:
-    src = os.path.join(input_path, "hf_quant_config.json")
-    if os.path.exists(src):
-        with open(src) as f:
+    """`hf_quant_config.json` in modelopt's layout, starting from the source's file when it has one."""
+    existing = os.path.join(input_path, "hf_quant_config.json")
+    doc = {"producer": {"name": "modelopt"}}
+    if os.path.exists(existing):
+        with open(existing) as f:
             doc = json.load(f)
-    else:
-        doc = {"producer": {"name": "modelopt"}}
-    section = doc.get("quantization")
-    if not isinstance(section, dict):
-        section = {}
-    section.update(quant_algo="NVFP4", kv_cache_quant_algo=DEFAULT_KV_CACHE_QUANT_ALGO, group_size=NVFP4_GROUP_SIZE,
-                   exclude_modules=ignore_list)
-    doc["quantization"] = section
+    block = doc["quantization"] if isinstance(doc.get("quantization"), dict) else {}
+    block["quant_algo"], block["kv_cache_quant_algo"] = "NVFP4", DEFAULT_KV_CACHE_QUANT_ALGO
+    block["group_size"], block["exclude_modules"] = NVFP4_GROUP_SIZE, ignore_list
+    doc["quantization"] = block
     with open(os.path.join(output_path, "hf_quant_config.json"), "w") as f:
         json.dump(doc, f, indent=2)
 
@@ -135,106 +134,119 @@ def _augment_ignore_list(ignore_list: list[str]) -> list[str]:
     return sorted(set(ignore_list) | extra)
 
 
-def _collect_gated_pair_locations(*, input_path, safetensors_files, device, skip_weight_substrings, num_hidden_layers):
-    """base name -> {'gate': (file, key), 'up': (file, key)} for every complete pair in the checkpoint."""
-    pairs: dict[str, dict[str, tuple[str, str]]] = {}
-    for filename in safetensors_files:
-        for key, tensor in ckpt.load_shard(input_path, filename, device).items():
-            if not should_quantize(key, tensor, skip_weight_substrings=skip_weight_substrings,
-                                   num_hidden_layers=num_hidden_layers):
-                continue
-            base, role = _split_gated_pair_name(key)
-            if base is None:
-                continue
-            roles = pairs.setdefault(base, {})
-            if role in roles:
-                raise ValueError(f"NVFP4 requires a single complete gate/up pair per converted checkpoint; "
-                                 f"found duplicate {role} tensor for {base}.")
-            roles[role] = (filename, key)
-    return {b: r for b, r in pairs.items() if set(r) == {"gate", "up"}}
+def _quantized_entries(key: str, codes, block_scale, global_scale) -> dict[str, torch.Tensor]:
+    """The four tensors a quantized `<module>.weight` becomes in a modelopt checkpoint."""
+    stem = key[: -len("weight")]
+    return {key: codes, stem + "weight_scale": block_scale, stem + "weight_scale_2": global_scale,
+            stem + "input_scale": torch.ones_like(global_scale, dtype=torch.float32)}
 
 
-def _nvfp4_quantized_entries(key, qweight, block_scale, weight_scale_2) -> dict[str, torch.Tensor]:
-    return {key: qweight, key.replace(".weight", ".weight_scale"): block_scale,
-            key.replace(".weight", ".weight_scale_2"): weight_scale_2,
-            key.replace(".weight", ".input_scale"): torch.ones_like(weight_scale_2, dtype=torch.float32)}
+class _Run:
+    """One conversion: which tensors are in scope, where the halves of every gate/up pair live, and the outputs of
+    pairs whose halves sit in different shards (quantized when the first half is met, written with each half's own
+    shard)."""
 
+    def __init__(self, src: str, dst: str, device: str, bf16_at_start: int, bf16_at_end: int, extra_skips) -> None:
+        self.src, self.dst, self.device = src, dst, device
+        self.depth = _get_num_hidden_layers(src)
+        self.bf16_prefixes = _get_bf16_layer_prefixes(self.depth, bf16_at_start, bf16_at_end)
+        self.skips = (*extra_skips, *sorted(self.bf16_prefixes))
+        self.shards = ckpt.list_shards(src)
+        self.results = ckpt.ShardResults(size_in_bytes=True)
+        self.pair_homes: dict[str, dict[str, tuple[str, str]]] = {}
+        self.pairs_done: set[str] = set()
+        self.waiting: dict[str, dict[str, dict[str, torch.Tensor]]] = {}     # shard -> key -> entries
 
-def process_file(input_path, output_path, filename, result_collector, device, num_hidden_layers,
-                 num_layers_at_start_in_bf16, num_layers_at_end_in_bf16, extra_high_precision_layers_hf,
-                 gated_pair_locations, processed_gated_pairs, deferred_quantized_entries) -> None:
-    if not filename.endswith(".safetensors"):
-        return
-    skipped: list[str] = []
-    out: dict[str, torch.Tensor] = {}
-    bf16_prefixes = _get_bf16_layer_prefixes(num_hidden_layers, num_layers_at_start_in_bf16, num_layers_at_end_in_bf16)
-    skip_substrings = (*extra_high_precision_layers_hf, *sorted(bf16_prefixes))
-    with launch.deferred():
-        for key, tensor in ckpt.load_shard(input_path, filename, device).items():
-            if key in out:
-                continue
-            parked = deferred_quantized_entries.get(filename, {}).pop(key, None)
-            if parked is not None:      # quantized earlier together with its partner from another shard
-                out.update(parked)
-                continue
-            if not should_quantize(key, tensor, skip_weight_substrings=skip_substrings, num_hidden_layers=num_hidden_layers):
-                if key.endswith(".weight"):
-                    module = key[: -len(".weight")]
-                    in_bf16_layers = [p for p in bf16_prefixes if key.startswith(p)]
-                    skipped.extend(in_bf16_layers)
-                    if ".experts." in key and in_bf16_layers:
-                        skipped.append(module.split(".experts.", 1)[0] + ".experts")   # the FusedMoE container
-                    else:
-                        skipped.append(module)
-                out[key] = tensor
-                continue
-            base, _role = _split_gated_pair_name(key)
-            if base not in gated_pair_locations:
-                out.update(_nvfp4_quantized_entries(key, *quantize_nvfp4(tensor)))
-                continue
-            if base in processed_gated_pairs:
-                raise ValueError(f"Missing deferred NVFP4 output for already processed gated pair {base}.")
-            (gate_file, gate_key), (up_file, up_key) = gated_pair_locations[base]["gate"], gated_pair_locations[base]["up"]
-            gate = tensor if key == gate_key else ckpt.load_tensor(input_path, gate_file, gate_key, device)
-            up = tensor if key == up_key else ckpt.load_tensor(input_path, up_file, up_key, device)
-            for (fname, k), result in zip(((gate_file, gate_key), (up_file, up_key)), nvfp4_quantize_1d_pair(gate, up)):
-                entries = _nvfp4_quantized_entries(k, *result)
-                if fname == filename:
-                    out.update(entries)
+    def in_scope(self, key: str, tensor: torch.Tensor) -> bool:
+        return should_quantize(key, tensor, skip_weight_substrings=self.skips, num_hidden_layers=self.depth)
+
+    def locate_pairs(self) -> None:
+        """A first pass over every shard: expert prefix -> {"gate": (shard, key), "up": (shard, key)}, complete pairs only."""
+        seen: dict[str, dict[str, tuple[str, str]]] = {}
+        for shard in self.shards:
+            for key, tensor in ckpt.load_shard(self.src, shard, self.device).items():
+                if not self.in_scope(key, tensor):
+                    continue
+                prefix, role = _split_gated_pair_name(key)
+                if prefix is None:
+                    continue
+                homes = seen.setdefault(prefix, {})
+                if role in homes:
+                    raise ValueError(f"NVFP4 requires a single complete gate/up pair per converted checkpoint; "
+                                     f"found duplicate {role} tensor for {prefix}.")
+                homes[role] = (shard, key)
+        self.pair_homes = {prefix: homes for prefix, homes in seen.items() if len(homes) == 2}
+
+    def _kept_in_high_precision(self, key: str) -> list[str]:
+        """Ignore-list entries for a `.weight` that stays as it is: its module, or for an expert of a BF16 layer the
+        layer prefix and the experts container (loaders decide per fused MoE module)."""
+        if not key.endswith(".weight"):
+            return []
+        layers = [p for p in self.bf16_prefixes if key.startswith(p)]
+        module = key[: -len(".weight")]
+        if layers and ".experts." in key:
+            return layers + [module.split(".experts.", 1)[0] + ".experts"]
+        return layers + [module]
+
+    def _quantize_pair(self, prefix: str, shard: str, key: str, tensor: torch.Tensor, out: dict) -> None:
+        if prefix in self.pairs_done:
+            raise ValueError(f"Missing deferred NVFP4 output for already processed gated pair {prefix}.")
+        homes = [self.pair_homes[prefix]["gate"], self.pair_homes[prefix]["up"]]
+        halves = [tensor if k == key else ckpt.load_tensor(self.src, f, k, self.device) for f, k in homes]
+        for (home_shard, home_key), result in zip(homes, nvfp4_quantize_1d_pair(*halves)):
+            entries = _quantized_entries(home_key, *result)
+            if home_shard == shard:
+                out.update(entries)
+            else:
+                self.waiting.setdefault(home_shard, {})[home_key] = entries
+        self.pairs_done.add(prefix)
+
+    def convert_shard(self, shard: str) -> None:
+        out: dict[str, torch.Tensor] = {}
+        ignored: list[str] = []
+        with launch.deferred():
+            for key, tensor in ckpt.load_shard(self.src, shard, self.device).items():
+                if key in out:
+                    continue
+                ready = self.waiting.get(shard, {}).pop(key, None)
+                if ready is not None:
+                    out.update(ready)
+                elif not self.in_scope(key, tensor):
+                    ignored += self._kept_in_high_precision(key)
+                    out[key] = tensor
                 else:
-                    deferred_quantized_entries.setdefault(fname, {})[k] = entries
-            processed_gated_pairs.add(base)
-    ckpt.save_shard(out, output_path, filename)
-    result_collector.add(filename, out, skipped)
+                    prefix = _split_gated_pair_name(key)[0]
+                    if prefix in self.pair_homes:
+                        self._quantize_pair(prefix, shard, key, tensor, out)
+                    else:
+                        out.update(_quantized_entries(key, *quantize_nvfp4(tensor)))
+        ckpt.save_shard(out, self.dst, shard)
+        self.results.add(shard, out, ignored)
+
+    def finish(self) -> None:
+        stranded = {shard: sorted(entries) for shard, entries in self.waiting.items() if entries}
+        if stranded:
+            raise RuntimeError(f"Unwritten deferred NVFP4 gated-pair entries: {stranded}")
+        ignore_list = _augment_ignore_list(self.results.modules_to_not_convert)
+        cfg = ckpt.read_config(self.src)
+        if cfg is not None:
+            _update_quantization_config(cfg, ignore_list)
+            ckpt.write_config(self.dst, cfg)
+        _write_hf_quant_config(self.dst, ignore_list, self.src)
+        ckpt.write_index(self.dst, self.results.weight_map, self.results.total_size)
 
 
 def convert_nvfp4(model_dir, save_dir, device, num_layers_at_start_in_bf16=0, num_layers_at_end_in_bf16=0,
                   extra_high_precision_layers_hf=()) -> None:
-    input_path, output_path = os.path.abspath(model_dir), os.path.abspath(save_dir)
-    os.makedirs(output_path, exist_ok=True)
-    ckpt.copy_side_files(input_path, output_path)
-    shards = ckpt.list_shards(input_path)
-    num_hidden_layers = _get_num_hidden_layers(input_path)
-    bf16_prefixes = _get_bf16_layer_prefixes(num_hidden_layers, num_layers_at_start_in_bf16, num_layers_at_end_in_bf16)
-    pairs = _collect_gated_pair_locations(input_path=input_path, safetensors_files=shards, device=device,
-                                          skip_weight_substrings=(*extra_high_precision_layers_hf, *sorted(bf16_prefixes)),
-                                          num_hidden_layers=num_hidden_layers)
-    done: set[str] = set()
-    parked: dict[str, dict[str, dict[str, torch.Tensor]]] = {}
-    results = ckpt.ShardResults(size_in_bytes=True)
-    for filename in shards:
-        process_file(input_path, output_path, filename, results, device, num_hidden_layers, num_layers_at_start_in_bf16,
-                     num_layers_at_end_in_bf16, tuple(extra_high_precision_layers_hf), pairs, done, parked)
-    left = {f: sorted(e) for f, e in parked.items() if e}
-    if left:
-        raise RuntimeError(f"Unwritten deferred NVFP4 gated-pair entries: {left}")
-    ignore_list = _augment_ignore_list(results.modules_to_not_convert)
-    cfg = ckpt.read_config(input_path)
-    if cfg is not None:
-        _update_quantization_config(cfg, ignore_list)
-        ckpt.write_config(output_path, cfg)
-    _write_hf_quant_config(output_path, ignore_list, input_path)
-    ckpt.write_index(output_path, results.weight_map, results.total_size)
+    src, dst = os.path.abspath(model_dir), os.path.abspath(save_dir)
+    os.makedirs(dst, exist_ok=True)
+    ckpt.copy_side_files(src, dst)
+    run = _Run(src, dst, device, num_layers_at_start_in_bf16, num_layers_at_end_in_bf16,
+               tuple(extra_high_precision_layers_hf))
+    run.locate_pairs()
+    for shard in run.shards:
+        run.convert_shard(shard)
+    run.finish()
 
 
 def main(argv=None) -> None:

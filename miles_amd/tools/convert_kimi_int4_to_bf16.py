@@ -14,8 +14,8 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import shutil
-from collections import defaultdict
 
 import torch
 from safetensors.torch import safe_open, save_file
@@ -58,82 +58,87 @@ def _dequantize_tensor(weight_packed: torch.Tensor, weight_scale: torch.Tensor, 
     return out
 
 
+_PROJECTIONS = ("gate_proj", "up_proj", "down_proj")
+_FIELDS = ("weight_packed", "weight_scale", "weight_shape")
+# <anything>.mlp.experts.<e>.<proj>.<field>, but nothing under a shared expert
+_TRIPLE_MEMBER = re.compile(r"^(?P<expert>.*\.mlp\.experts\.[^.]+)(?:\..*)?\.(?P<proj>%s)\.(?P<field>%s)$"
+                            % ("|".join(_PROJECTIONS), "|".join(_FIELDS)))
+
+
 def _is_quantized_weight_key(key: str) -> bool:
-    """Routed-expert gate/up/down tensors stored as weight_packed / weight_scale / weight_shape."""
-    if ".mlp.experts." not in key or ".shared_experts." in key:
-        return False
-    return any(key.endswith(f".{proj}.{suffix}") for proj in ("gate_proj", "up_proj", "down_proj")
-               for suffix in ("weight_packed", "weight_scale", "weight_shape"))
+    """A routed expert's gate / up / down projection stored as weight_packed / weight_scale / weight_shape."""
+    return ".shared_experts." not in key and _TRIPLE_MEMBER.match(key) is not None
 
 
 def convert_file(input_path: str, output_path: str, group_size: int, skip_existing: bool = True, device: str = "cuda"):
-    """One shard: every complete (packed, scale, shape) triple becomes `<prefix>.<proj>.weight` in bfloat16;
-    incomplete triples and all other tensors are copied."""
+    """One shard: a projection whose three fields are all present becomes `<expert>.<proj>.weight` in bfloat16;
+    everything else, fields of incomplete projections included, is carried over under its own name."""
     if skip_existing and os.path.exists(output_path):
         return
-    tensors = {}
-    experts = defaultdict(lambda: defaultdict(dict))
-    with safe_open(input_path, framework="pt", device=device) as reader:
-        for key in reader.keys():
-            tensor = reader.get_tensor(key)
-            parts = key.split(".")
-            if not _is_quantized_weight_key(key) or "experts" not in parts:
-                tensors[key] = tensor
-                continue
-            prefix = ".".join(parts[: parts.index("experts") + 2])
-            experts[prefix][parts[-2]][parts[-1]] = tensor
-    for prefix, components in experts.items():
-        for proj in ("gate_proj", "up_proj", "down_proj"):
-            data = components.get(proj, {})
-            if not {"weight_packed", "weight_scale", "weight_shape"}.issubset(data):
-                for suffix, value in data.items():
-                    tensors[f"{prefix}.{proj}.{suffix}"] = value
-                continue
-            tensors[f"{prefix}.{proj}.weight"] = _dequantize_tensor(
-                data["weight_packed"].to(torch.int32), data["weight_scale"].to(torch.float32), data["weight_shape"], group_size)
+    carried: dict[str, torch.Tensor] = {}
+    fields_of: dict[tuple[str, str], dict[str, torch.Tensor]] = {}
+    with safe_open(input_path, framework="pt", device=device) as shard:
+        for key in shard.keys():
+            member = _TRIPLE_MEMBER.match(key) if _is_quantized_weight_key(key) else None
+            if member is None:
+                carried[key] = shard.get_tensor(key)
+            else:
+                module = (key[: member.start("proj") - 1], member["proj"])        # (expert prefix, projection)
+                fields_of.setdefault(module, {})[member["field"]] = shard.get_tensor(key)
+    for (expert, proj), fields in fields_of.items():
+        if len(fields) < len(_FIELDS):
+            carried.update({f"{expert}.{proj}.{field}": value for field, value in fields.items()})
+            continue
+        carried[f"{expert}.{proj}.weight"] = _dequantize_tensor(fields["weight_packed"].to(torch.int32),
+                                                                fields["weight_scale"].to(torch.float32),
+                                                                fields["weight_shape"], group_size)
     os.makedirs(os.path.dirname(output_path), exist_ok=True)
-    save_file({k: v.cpu().contiguous() for k, v in tensors.items()}, output_path)
+    save_file({name: t.cpu().contiguous() for name, t in carried.items()}, output_path)
 
 
 def parse_args(argv=None) -> argparse.Namespace:
-    parser = argparse.ArgumentParser(description="Convert INT4 pack-quantized MoE experts to BF16 weights.")
-    parser.add_argument("--model-dir", required=True)
-    parser.add_argument("--output-dir", default=None, help="default: <model-dir>_bf16")
-    parser.add_argument("--files", nargs="+", default=None)
-    parser.add_argument("--config-path", default=None)
-    parser.add_argument("--overwrite", action="store_true")
-    return parser.parse_args(argv)
+    p = argparse.ArgumentParser(description="Convert INT4 pack-quantized MoE experts to BF16 weights.")
+    p.add_argument("--model-dir", required=True)
+    p.add_argument("--output-dir", default=None, help="default: <model-dir>_bf16")
+    p.add_argument("--files", nargs="+", default=None)
+    p.add_argument("--config-path", default=None)
+    p.add_argument("--overwrite", action="store_true")
+    return p.parse_args(argv)
+
+
+_SIDE_FILE_SUFFIXES = (".json", ".py", ".jinja", ".model")
+
+
+def _finish(model_dir: str, output_dir: str) -> None:
+    """Tokenizer / config / code files next to the shards, and an index rebuilt from the shards that were written."""
+    for name in os.listdir(model_dir):
+        if name != "model.safetensors.index.json" and (name.startswith("tokenizer") or name.endswith(_SIDE_FILE_SUFFIXES)):
+            shutil.copy2(os.path.join(model_dir, name), os.path.join(output_dir, name))
+    owner = {}
+    for name in sorted(n for n in os.listdir(output_dir) if n.endswith(".safetensors")):
+        with safe_open(os.path.join(output_dir, name), framework="pt") as shard:
+            owner.update(dict.fromkeys(shard.keys(), name))
+    with open(os.path.join(output_dir, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": owner}, f, indent=2)
 
 
 def main(argv=None) -> None:
     args = parse_args(argv)
     model_dir = os.path.abspath(args.model_dir)
-    output_dir = os.path.abspath(args.output_dir or f"{model_dir}_bf16")
     if not os.path.isdir(model_dir):
         raise FileNotFoundError(f"Model directory not found: {model_dir}")
-    _, _, group_size = _load_config(model_dir, args.config_path)
-    names = args.files or [n for n in sorted(os.listdir(model_dir)) if n.endswith(".safetensors")]
-    if not names:
+    output_dir = os.path.abspath(args.output_dir or model_dir + "_bf16")
+    group_size = _load_config(model_dir, args.config_path)[2]
+    shards = args.files or sorted(n for n in os.listdir(model_dir) if n.endswith(".safetensors"))
+    if not shards:
         print("No safetensors checkpoints found.")
         return
-    for name in names:
-        path = os.path.join(model_dir, name)
-        if os.path.isfile(path):
-            convert_file(path, os.path.join(output_dir, os.path.relpath(path, model_dir)), group_size,
+    for name in shards:
+        source = os.path.join(model_dir, name)
+        if os.path.isfile(source):
+            convert_file(source, os.path.join(output_dir, os.path.relpath(source, model_dir)), group_size,
                          skip_existing=not args.overwrite)
-    for fname in os.listdir(model_dir):
-        if fname == "model.safetensors.index.json":
-            continue
-        if fname.startswith("tokenizer") or fname.endswith((".json", ".py", ".jinja", ".model")):
-            shutil.copy2(os.path.join(model_dir, fname), os.path.join(output_dir, fname))
-    weight_map = {}
-    for fname in sorted(os.listdir(output_dir)):
-        if fname.endswith(".safetensors"):
-            with safe_open(os.path.join(output_dir, fname), framework="pt") as reader:
-                for key in reader.keys():
-                    weight_map[key] = fname
-    with open(os.path.join(output_dir, "model.safetensors.index.json"), "w") as f:
-        json.dump({"metadata": {}, "weight_map": weight_map}, f, indent=2)
+    _finish(model_dir, output_dir)
     print(f"\nSuccessful! Output saved to: {output_dir}")
 
 

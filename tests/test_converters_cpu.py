@@ -255,3 +255,68 @@ def test_runtime_nvfp4_quantizer_only_takes_the_main_language_decoder(monkeypatc
     monkeypatch.setattr(Q, "_quantize_moe_params", lambda *_: converted)
     got = Q.quantize_params_nvfp4(None, f"{prefix}.layers.0.mlp.experts.linear_fc2.weight0", original, {"quant_method": "nvfp4"})
     assert got is (converted if eligible else original)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# MiMo-V2 -> BF16: the host-side parts (names, config, head order, --keep-quant, which needs no kernel)
+def test_mimo_split_fused_qkv_restores_head_order():
+    from miles_amd.tools.convert_mimo_v2_to_bf16 import split_fused_qkv
+    from tests import mimo_fixture as MF
+
+    config = {"num_key_value_heads": 2, "swa_num_attention_heads": 8, "swa_num_key_value_heads": 4, "swa_head_dim": 3, "swa_v_head_dim": 2}
+    q, k, v = torch.randn(8 * 3, 5), torch.randn(4 * 3, 5), torch.randn(4 * 2, 5)
+    for got, want in zip(split_fused_qkv(MF.interleave(q, k, v, 2), config, is_swa=True), (q, k, v), strict=True):
+        assert torch.equal(got, want)
+    with pytest.raises(AssertionError):
+        split_fused_qkv(torch.zeros(10, 5), config, is_swa=True)
+
+
+def test_mimo_names_and_config_when_layers_and_experts_are_dropped():
+    from miles_amd.tools import convert_mimo_v2_to_bf16 as M
+    from tests import mimo_fixture as MF
+
+    assert M.output_name("lm_head.weight", {1: 0}, 2) == "lm_head.weight"
+    assert M.output_name("model.layers.0.mlp.up_proj.weight", {1: 0}, None) is None
+    assert M.output_name("model.layers.1.mlp.experts.1.up_proj.weight", {1: 0}, 2) == "model.layers.0.mlp.experts.1.up_proj.weight"
+    assert M.output_name("model.layers.1.mlp.experts.2.up_proj.weight", {1: 0}, 2) is None
+    assert M.output_name("model.layers.1.mlp.experts.2.up_proj.weight", None, None) == "model.layers.1.mlp.experts.2.up_proj.weight"
+    cfg = M.convert_config(MF.CONFIG, {1: 0}, 2, keep_quant=False)
+    assert (cfg["num_hidden_layers"], cfg["hybrid_layer_pattern"], cfg["moe_layer_freq"], cfg["n_routed_experts"]) == (1, [1], [1], 2)
+    assert "quantization_config" not in cfg and "attention_projection_layout" not in cfg
+    assert MF.CONFIG["num_hidden_layers"] == 2                                  # the input is not modified
+    kept = M.convert_config(MF.CONFIG, {1: 0}, None, keep_quant=True)
+    assert kept["quantization_config"]["ignored_layers"] == ["model.layers.0.self_attn.o_proj"]
+    with pytest.raises(AssertionError):
+        M.convert_config(MF.CONFIG, None, 1, keep_quant=False)                  # fewer experts than are routed to per token
+    with pytest.raises(AssertionError, match="experts"):
+        M.check_output({"model.layers.0.input_layernorm.weight": "f"}, cfg)            # the kept layer is the MoE layer
+    dense_only = M.convert_config(MF.CONFIG, {0: 0}, None, keep_quant=False)
+    with pytest.raises(AssertionError, match="is missing"):
+        M.check_output({"model.layers.0.input_layernorm.weight": "f"}, dense_only)
+
+
+def test_mimo_keep_quant_renumbers_and_copies_on_the_cpu(tmp_path, monkeypatch):
+    from miles_amd.tools import convert_mimo_v2_to_bf16 as M
+    from tests import mimo_fixture as MF
+
+    src, dst = tmp_path / "src", tmp_path / "dst"
+    src.mkdir()
+    MF.write(src)
+    # an interrupted side-file copy must not leave an index behind (the index is what marks a finished conversion)
+    real_copy = M.shutil.copy2
+    monkeypatch.setattr(M.shutil, "copy2", lambda *_: (_ for _ in ()).throw(OSError("interrupted auxiliary copy")))
+    with pytest.raises(OSError, match="interrupted auxiliary copy"):
+        M.main(str(src), str(dst), [1], None, keep_quant=True, device="cpu")
+    assert not (dst / "model.safetensors.index.json").exists()
+    monkeypatch.setattr(M.shutil, "copy2", real_copy)
+    M.main(str(src), str(dst), [1], None, keep_quant=True, device="cpu")
+    config = json.loads((dst / "config.json").read_text())
+    assert config["quantization_config"]["ignored_layers"] == ["model.layers.0.self_attn.o_proj"]
+    assert config["attention_projection_layout"] == "fused_qkv" and config["num_hidden_layers"] == 1
+    index = json.loads((dst / "model.safetensors.index.json").read_text())
+    out = safetensors.torch.load_file(dst / "model-00001.safetensors")
+    assert set(index["weight_map"]) == set(out)
+    assert out["model.layers.0.self_attn.qkv_proj.weight"].dtype == torch.float8_e4m3fn       # stored formats survive
+    assert out["model.layers.0.mlp.experts.3.down_proj.weight"].dtype == torch.uint8
+    assert not any(name.startswith("model.layers.1.") for name in out)
+    assert (dst / "tokenizer_config.json").read_text() == "{}"

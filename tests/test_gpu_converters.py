@@ -310,3 +310,65 @@ def test_convert_mxfp4_to_fp8(tmp_path, oracle):
     index = json.loads((out / "model.safetensors.index.json").read_text())
     assert index["weight_map"]["model.layers.0.mlp.experts.1.w1.scale"] == index["weight_map"]["model.layers.0.mlp.experts.1.w1.weight"]
     assert set(index["weight_map"]) == set(got) and (out / "tokenizer.json").exists()
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# MiMo-V2 -> BF16 (tools/convert_mimo_v2_to_bf16.py); expectations come from torch CPU ops in tests/mimo_fixture.py
+def test_mimo_dequant_mxfp4_matches_the_closed_form():
+    from miles_amd.tools.convert_mimo_v2_to_bf16 import dequant_mxfp4
+    from tests import mimo_fixture as MF
+
+    g = torch.Generator().manual_seed(3)
+    codes = torch.randint(0, 16, (8, 64), generator=g)
+    exps = torch.randint(120, 134, (8, 2), dtype=torch.uint8, generator=g)
+    want = (MF.FP4_VALUES[codes] * torch.exp2(exps.float() - 127).repeat_interleave(32, dim=1)).to(torch.bfloat16)
+    got = dequant_mxfp4(MF.pack_nibbles(codes).cuda(), exps.cuda()).cpu()
+    _same(got, want, "mxfp4 dequant")          # bit for bit, the sign of -0 codes included
+
+
+def test_mimo_fused_qkv_scales_belong_to_their_shard():
+    from miles_amd.tools.convert_mimo_v2_to_bf16 import dequant_fused_qkv
+    from tests import mimo_fixture as MF
+
+    # shards of 224 rows are not 128-aligned: each one has two scale rows of its own
+    w = torch.randn(2 * 224, 256, generator=torch.Generator().manual_seed(4))
+    halves = [MF.quantize_fp8_blocks(part) for part in w.chunk(2)]
+    q, s = torch.cat([h[0] for h in halves]), torch.cat([h[1] for h in halves])
+    assert s.shape == (4, 2)
+    got = dequant_fused_qkv(q.cuda(), s.cuda(), 2).cpu()
+    _same(got, torch.cat([MF.dequantize_fp8_blocks(*h) for h in halves]), "fused qkv")
+    assert (got.float() - w).abs().max() < 0.07 * w.abs().max()
+
+
+@pytest.mark.parametrize("layers,num_experts", [(None, None), ([1], 2)])
+def test_mimo_conversion_end_to_end(tmp_path, layers, num_experts):
+    from miles_amd.tools import convert_mimo_v2_to_bf16 as M
+    from tests import mimo_fixture as MF
+
+    src, dst = tmp_path / "src", tmp_path / "dst"
+    src.mkdir()
+    expected = MF.write(src)
+    M.main(str(src), str(dst), layers, num_experts, keep_quant=False, device="cuda")
+    config = json.loads((dst / "config.json").read_text())
+    out = _load_all(dst)
+    assert set(json.loads((dst / "model.safetensors.index.json").read_text())["weight_map"]) == set(out)
+    assert "quantization_config" not in config and "attention_projection_layout" not in config
+    assert (dst / "tokenizer_config.json").exists()
+    assert not any(n.endswith(("weight_scale", "weight_scale_inv", "qkv_proj.weight")) for n in out)
+    renumber = {old: new for new, old in enumerate(layers)} if layers else {0: 0, 1: 1}
+    experts_kept = num_experts or 4
+    assert config["num_hidden_layers"] == len(renumber) and config["n_routed_experts"] == experts_kept
+    assert config["hybrid_layer_pattern"] == config["moe_layer_freq"] == list(renumber)
+    checked = 0
+    for name, want in expected.items():
+        parts = name.split(".")
+        layer = int(parts[2])
+        if layer not in renumber or (parts[4] == "experts" and int(parts[5]) >= experts_kept):
+            continue
+        _same(out[".".join(["model", "layers", str(renumber[layer]), *parts[3:]])], want, name)
+        checked += 1
+    assert checked == (6 if 0 in renumber else 0) + 3 + 3 * experts_kept
+    moe = renumber[1]
+    assert sum(".experts." in n for n in out) == 3 * experts_kept
+    assert out[f"model.layers.{moe}.mlp.gate.weight"].shape[0] == experts_kept
+    assert out[f"model.layers.{moe}.mlp.gate.e_score_correction_bias"].dtype == torch.float32
