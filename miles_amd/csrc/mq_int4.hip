@@ -19,6 +19,7 @@
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
+#include "mq_io8.hpp"
 
 namespace mq {
 
@@ -372,6 +373,59 @@ __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __re
     }
 }
 
+// ---- fake INT4 quantization of row blocks (1, G), G = 32 / 64 / 128 ------------------------------------------------
+// The standalone form of the reference's extension (fake_int4_quant_cuda.cu:29-91 for G = 32, :159-259 otherwise):
+// `out` holds the integer codes as values of the input dtype, `scale` (and `zero`) one value per block in that dtype.
+//   symmetric:  s = max(amax * f32(1/7), 1e-5);   out = rint(x / s)
+//   asymmetric: s = max((max - min) * f32(1/15), 1e-5);   z = min(max(-rint(min / s), +0), 15);   out = rint(x / s) + z
+// Lanes own 8 consecutive elements, G / 8 neighbouring lanes a block; x / s is the exact quotient (shared-divisor
+// sequence for 16-bit inputs, the sign of a -0 numerator put back; the division itself otherwise).
+template <int DT, int LANES, bool SYM>
+__global__ __launch_bounds__(kI4Threads) void int4_fake_rows_kernel(const void* __restrict__ x, void* __restrict__ out,
+                                                                    void* __restrict__ scale_out,
+                                                                    void* __restrict__ zero_out, int64_t units, int chunk) {
+    const int64_t unit = xcd_chunked_block(chunk) * kI4Threads + threadIdx.x;
+    const bool live = unit < units;            // a block is a whole number of lanes: dead lanes never share one with live lanes
+    float f[8], q[8];
+    fq_load8<DT>(x, live ? unit : units - 1, f);
+    float mx, mn = 0.0f, s, zero = 0.0f;
+    if (SYM) {
+        mx = __builtin_fabsf(f[0]);
+#pragma unroll
+        for (int i = 1; i < 8; i++) mx = __builtin_fmaxf(mx, __builtin_fabsf(f[i]));
+        mx = u2f(seg_max<LANES>(f2u(mx)));     // non-negative floats order like their bit patterns
+        s = __builtin_fmaxf(mx * kSymCons, 1e-5f);
+    } else {
+        mx = mn = f[0];
+#pragma unroll
+        for (int i = 1; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
+        mx = order_unkey(seg_max<LANES>(order_key(mx)));
+        mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
+        s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
+        // max(-0, +0) is +0 in the reference's device code: adding +0 makes that explicit
+        zero = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
+    }
+    const float y = 1.0f / s;
+    const float top = SYM ? mx : __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
+    if (DT != MQ_F32 && shared_div_ok(s) && top * y < 1e30f) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(__builtin_copysignf(div_by_shared(f[i], s, y), f[i]));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s);
+    }
+    if (!SYM) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = q[i] + zero;
+    }
+    if (!live) return;
+    fq_store8<DT>(out, unit, q);
+    if ((threadIdx.x & (LANES - 1)) == 0) {
+        store_dtype(scale_out, unit / LANES, s, DT);
+        if (!SYM) store_dtype(zero_out, unit / LANES, zero, DT);
+    }
+}
+
 // ---- unpack + dequantize (symmetric codes) ------------------------------------------------------
 // Inverse of the symmetric pack: tools/convert_kimi_int4_to_bf16.py:57-86 unpacks nibble i of word j into
 // element 8j+i, subtracts the offset 8 (compressed-tensors' unpack_from_int32), multiplies by the group's scale
@@ -432,6 +486,26 @@ __global__ __launch_bounds__(256) void int4_unpack_generic_kernel(const uint32_t
 
 using namespace mq;
 
+template <int DT, int LANES>
+static void launch_fake_rows_sym(const void* x, void* out, void* scale, void* zero, int64_t units, bool sym, int chunk,
+                                 unsigned blocks, hipStream_t st) {
+    if (sym) hipLaunchKernelGGL((int4_fake_rows_kernel<DT, LANES, true>), dim3(blocks), dim3(kI4Threads), 0, st, x, out, scale, zero, units, chunk);
+    else hipLaunchKernelGGL((int4_fake_rows_kernel<DT, LANES, false>), dim3(blocks), dim3(kI4Threads), 0, st, x, out, scale, zero, units, chunk);
+}
+template <int DT>
+static void launch_fake_rows_dt(const void* x, void* out, void* scale, void* zero, int64_t units, int lanes, bool sym,
+                                int chunk, unsigned blocks, hipStream_t st) {
+    if (lanes == 16) launch_fake_rows_sym<DT, 16>(x, out, scale, zero, units, sym, chunk, blocks, st);
+    else if (lanes == 8) launch_fake_rows_sym<DT, 8>(x, out, scale, zero, units, sym, chunk, blocks, st);
+    else launch_fake_rows_sym<DT, 4>(x, out, scale, zero, units, sym, chunk, blocks, st);
+}
+static void launch_fake_rows(const void* x, int dtype, void* out, void* scale, void* zero, int64_t units, int lanes,
+                             bool sym, int chunk, unsigned blocks, hipStream_t st) {
+    if (dtype == MQ_BF16) launch_fake_rows_dt<MQ_BF16>(x, out, scale, zero, units, lanes, sym, chunk, blocks, st);
+    else if (dtype == MQ_F16) launch_fake_rows_dt<MQ_F16>(x, out, scale, zero, units, lanes, sym, chunk, blocks, st);
+    else launch_fake_rows_dt<MQ_F32>(x, out, scale, zero, units, lanes, sym, chunk, blocks, st);
+}
+
 extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
                                   int block_m, int block_n, int sym, void* stream) {
     if (!x || !out || !scale || (!sym && !zero)) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -439,6 +513,16 @@ extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* sca
     if (((int64_t)block_m * block_n) % 32 != 0 || (int64_t)block_m * block_n > (1 << 24))
         return mq_fail(MQ_ERR_ARG, "block_m * block_n must be divisible by 32");
     if (M == 0 || N == 0) return MQ_OK;
+    const bool rows_fast = block_m == 1 && (block_n == 32 || block_n == 64 || block_n == 128) &&
+                           N % block_n == 0 && ((((uintptr_t)x | (uintptr_t)out)) & 15) == 0 && M * (N / 8) < (1ll << 38);
+    if (rows_fast) {
+        const int64_t units = M * (N / 8);
+        int64_t blocks = (units + kI4Threads - 1) / kI4Threads;
+        const int chunk = (int)flat_chunk(blocks);
+        blocks = flat_padded(blocks, chunk);
+        launch_fake_rows(x, dtype, out, scale, zero, units, block_n / 8, sym != 0, chunk, (unsigned)blocks, (hipStream_t)stream);
+        return mq_check_launch("int4 fake quant");
+    }
     const int64_t gpr = (N + block_n - 1) / block_n;
     const int64_t waves = ((M + block_m - 1) / block_m) * gpr;
     int64_t blocks = (waves + 3) / 4;

@@ -952,3 +952,41 @@ def test_act_quant_full_size_round_trip(oracle):
     assert torch.all(err <= s.unsqueeze(-1) * 448 * 2.0 ** -4)
     head = x[:64].cpu()
     _assert_same(sim[:64], oracle.fp8_simulate(head, 128), "full-size head rows")
+
+
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("G", [32, 64, 128, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_fake_int4_quant_row_blocks_edge_values(oracle, sym, G, dtype):
+    # the row-block kernel: signed zeros, an all-zero block, a constant block (range 0 -> scale floor), blocks that are
+    # all positive / all negative (clamped zero points), magnitudes near the top of the dtype, ragged row count
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
+
+    big = {torch.bfloat16: 3.0e38, torch.float16: 6.0e4, torch.float32: 3.0e38}[dtype]
+    w = W.gaussian_outliers((37, 512), std=0.02, p_outlier=0.002, gain=25.0, seed=4100 + G, dtype=dtype)
+    w[0] = 0
+    w[1, :128] = torch.tensor([-0.0, 0.0] * 64).to(dtype)
+    w[2, :128] = 0.37
+    w[3, :128] = w[3, :128].abs() + 0.5
+    w[4, :128] = -(w[4, :128].abs()) - 0.5
+    w[5, :4] = torch.tensor([big, -big, 1e-30, -1e-30]).to(dtype)
+    w[6, :128] = torch.linspace(-7, 7, 128).to(dtype)          # exact ties of rint(x / 1)
+    out, scale, zero = fake_int4_quant_cuda(w.to(DEV), (1, G), sym)
+    out_o, scale_o, zero_o = oracle.fake_int4_quant(w, (1, G), sym)
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(out, out_o, "values")
+    if not sym:
+        _assert_same(zero, zero_o, "zero points")
+
+
+def test_fake_int4_quant_full_size_tensor(oracle):
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
+
+    w = W.c4_expert(0, 0)                                      # [2048, 7168] bf16
+    for sym in (True, False):
+        out, scale, zero = fake_int4_quant_cuda(w.to(DEV), (1, 128), sym)
+        out_o, scale_o, zero_o = oracle.fake_int4_quant(w, (1, 128), sym)
+        _assert_same(out, out_o, "values")
+        _assert_same(scale, scale_o, "scales")
+        if not sym:
+            _assert_same(zero, zero_o, "zero points")
