@@ -36,7 +36,7 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   "int4_g128": 2 + 0.5 + 2 / 128, "nvfp4": 2 + 0.5 + 1 / 16,
                   # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
                   "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
-                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2, "act_quant": 2 + 1 + 4 / 128, "fake_int4_bf16": 2 + 2 + 2 / 128,
+                  "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2, "act_quant": 2 + 1 + 4 / 128, "fake_int4_bf16": 2 + 2 + 2 / 128, "fp8_channel": 2 + 1,
                   "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0005 B per element)
@@ -286,6 +286,10 @@ def adjacent_formats(gen):
     del i4
     run("next_int4_g128_asym_pack", "int4_g128_asym", lambda: [pack_layer(w, 128, sym=False) for w in ws],
         "pack_layer(sym=False), group 128")
+    from miles_amd.tools.convert_hf_to_fp8 import channel_fp8, tensor_fp8
+    run("a2_channel_fp8", "fp8_channel", lambda: [channel_fp8(w) for w in ws], "one scale per row, rows read once")
+    run("a2_tensor_fp8", "fp8_channel", lambda: [tensor_fp8(w) for w in ws],
+        "one scale per tensor: amax pass + quantize pass (5 B/element moved, 3 counted)")
     from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
     run("a8_fake_int4_quant_1x128", "fake_int4_bf16", lambda: [fake_int4_quant_cuda(w, [1, 128], True) for w in ws],
         "fake_int4_quant_cuda(x, (1,128), sym): bf16 in, bf16 integer codes + bf16 scales out")

@@ -217,6 +217,130 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restri
         q[r * K + c] = (uint8_t)sw_e4m3fn(v);
     }
 }
+// bf16 fast paths of the two.  The quotient x / s is the exact one (shared-divisor sequence; the division itself when
+// s leaves the guarded range); the sign of a -0 numerator is taken from the input pattern.
+//
+// per channel: a row lives in the registers of ROWLANES lanes (up to 8 sixteen-byte units each), so it is read once:
+// amax across the lanes, one scale, codes.  ROWLANES = 64: four rows per workgroup, no LDS; 256: one row.
+template <int ROWLANES>
+__global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* __restrict__ w, int64_t ldw, int64_t K,
+                                                               int64_t M, float floor_v, uint8_t* __restrict__ q,
+                                                               float* __restrict__ scale) {
+    __shared__ uint32_t wave_amax[4];
+    constexpr int kRows = 256 / ROWLANES, kMaxUnits = 8;
+    const int t = threadIdx.x, lane = t % ROWLANES;
+    const int64_t row = (int64_t)blockIdx.x * kRows + t / ROWLANES;
+    const int64_t units = K / 8;
+    const bool row_ok = row < M;
+    const uint16_t* __restrict__ src = w + (row_ok ? row : M - 1) * ldw;
+    u32x4 v[kMaxUnits];
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int u = 0; u < kMaxUnits; u++) {
+        const int64_t unit = lane + (int64_t)u * ROWLANES;
+        v[u] = unit < units ? ld16(src + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v[u].x), abs2(v[u].y)), max2_u16(abs2(v[u].z), abs2(v[u].w))));
+    }
+    uint32_t m = wave_max(hmax_u16(m2));
+    if (ROWLANES == 256) {
+        if ((t & 63) == 0) wave_amax[t >> 6] = m;
+        __syncthreads();
+        m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
+    }
+    float amax = u2f(m << 16);
+    if (amax < floor_v) amax = floor_v;
+    const float s = amax / kFp8Max, y = 1.0f / s;
+    const bool fast_div = shared_div_ok(s);
+    if (!row_ok) return;
+    if (lane == 0) scale[row] = s;
+#pragma unroll
+    for (int u = 0; u < kMaxUnits; u++) {
+        const int64_t unit = lane + (int64_t)u * ROWLANES;
+        if (unit >= units) continue;
+        float f[8] = {bf16_lo(v[u].x), bf16_hi(v[u].x), bf16_lo(v[u].y), bf16_hi(v[u].y),
+                      bf16_lo(v[u].z), bf16_hi(v[u].z), bf16_lo(v[u].w), bf16_hi(v[u].w)};
+#pragma unroll
+        for (int j = 0; j < 8; j++) f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
+        u32x2 o;
+        if (m < 0x7F80u) {
+            o.x = copy_signs(hw_e4m3x4(f[0], f[1], f[2], f[3]), v[u].x, v[u].y);
+            o.y = copy_signs(hw_e4m3x4(f[4], f[5], f[6], f[7]), v[u].z, v[u].w);
+        } else {                                  // inf / NaN in the row: clamp and convert in software
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(__builtin_amdgcn_fmed3f(f[j], -kFp8Max, kFp8Max));
+            o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+        }
+        st8(q + row * K + unit * 8, o);
+    }
+}
+
+// per tensor, pass 1: every workgroup strides over 8 KiB pieces and ends with one atomic max on the bf16 amax
+__global__ __launch_bounds__(256) void fp8_tensor_amax_bf16_kernel(const uint16_t* __restrict__ w, int64_t units,
+                                                                   uint32_t* __restrict__ amax_bits) {
+    __shared__ uint32_t wave_amax[4];
+    const int t = threadIdx.x;
+    uint32_t m2 = 0;
+    for (int64_t base = (int64_t)blockIdx.x * 512; base < units; base += (int64_t)gridDim.x * 512) {
+        const int64_t a = base + t, b = base + 256 + t;
+        const u32x4 va = a < units ? ld16(w + a * 8) : u32x4{0u, 0u, 0u, 0u};
+        const u32x4 vb = b < units ? ld16(w + b * 8) : u32x4{0u, 0u, 0u, 0u};
+        m2 = max2_u16(m2, max2_u16(max2_u16(abs2(va.x), abs2(va.y)), max2_u16(abs2(va.z), abs2(va.w))));
+        m2 = max2_u16(m2, max2_u16(max2_u16(abs2(vb.x), abs2(vb.y)), max2_u16(abs2(vb.z), abs2(vb.w))));
+    }
+    const uint32_t m = wave_max(hmax_u16(m2));
+    if ((t & 63) == 0) wave_amax[t >> 6] = m;
+    __syncthreads();
+    if (t == 0) atomicMax(amax_bits, umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3])) << 16);
+}
+// per tensor, pass 2: flat.  torch divides by a zero-dimensional scale in the weight's dtype, so the quotient is
+// rounded to bf16 before it is clamped and converted.
+__global__ __launch_bounds__(256) void fp8_tensor_quant_bf16_kernel(const uint16_t* __restrict__ w,
+                                                                    const uint32_t* __restrict__ amax_bits, float floor_v,
+                                                                    uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                                    int64_t units, int chunk) {
+    const int64_t base = xcd_chunked_block(chunk) * 512 + threadIdx.x;
+    u32x4 v[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int64_t unit = base + i * 256;
+        v[i] = ld16(w + (unit < units ? unit : units - 1) * 8);
+    }
+    const uint32_t abits = amax_bits[0];
+    float amax = u2f(abits);
+    if (amax < floor_v) amax = floor_v;
+    const float s = amax / kFp8Max, y = 1.0f / s;
+    const bool fast_div = shared_div_ok(s);
+    if (base == 0) scale[0] = s;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int64_t unit = base + i * 256;
+        float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                      bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+#pragma unroll
+        for (int j = 0; j < 8; j++) f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {           // the rounding to bf16
+            const uint32_t p = hw_bf16x2(f[j], f[j + 1]);
+            f[j] = bf16_lo(p);
+            f[j + 1] = bf16_hi(p);
+        }
+        u32x2 o;
+        if (abits < 0x7F800000u) {
+            o.x = copy_signs(hw_e4m3x4(f[0], f[1], f[2], f[3]), v[i].x, v[i].y);
+            o.y = copy_signs(hw_e4m3x4(f[4], f[5], f[6], f[7]), v[i].z, v[i].w);
+        } else {
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(__builtin_amdgcn_fmed3f(f[j], -kFp8Max, kFp8Max));
+            o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+        }
+        if (unit < units) st8(q + unit * 8, o);
+    }
+}
+
 __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -387,6 +511,29 @@ extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* 
     if (M == 0 || K == 0) return MQ_OK;
     if (M > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many rows");
     hipStream_t st = (hipStream_t)stream;
+    const bool aligned = dtype == MQ_BF16 && K % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
+    if (aligned && per_channel && K / 8 <= 2048) {
+        const uint16_t* wi = (const uint16_t*)w;
+        if (K / 8 <= 256)
+            hipLaunchKernelGGL(fp8_channel_bf16_kernel<64>, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, st, wi, ldw, K, M,
+                               floor_in_dtype, (uint8_t*)q, scale);
+        else
+            hipLaunchKernelGGL(fp8_channel_bf16_kernel<256>, dim3((unsigned)M), dim3(256), 0, st, wi, ldw, K, M,
+                               floor_in_dtype, (uint8_t*)q, scale);
+        return mq_check_launch("fp8 scaled quant");
+    }
+    if (aligned && !per_channel && ldw == K && M * (K / 8) < (1ll << 38)) {
+        const int64_t units = M * (K / 8);
+        int64_t blocks = (units + 511) / 512;
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)amax_ws, 0u, 1);
+        hipLaunchKernelGGL(fp8_tensor_amax_bf16_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, st,
+                           (const uint16_t*)w, units, (uint32_t*)amax_ws);
+        const int chunk = (int)flat_chunk(blocks);
+        blocks = flat_padded(blocks, chunk);
+        hipLaunchKernelGGL(fp8_tensor_quant_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint16_t*)w,
+                           (const uint32_t*)amax_ws, floor_in_dtype, (uint8_t*)q, scale, units, chunk);
+        return mq_check_launch("fp8 scaled quant");
+    }
     if (!per_channel) hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)amax_ws, 0u, 1);
     hipLaunchKernelGGL(fp8_row_amax_kernel, dim3((unsigned)M), dim3(256), 0, st, w, dtype, ldw, K,
                        (uint32_t*)amax_ws, per_channel);

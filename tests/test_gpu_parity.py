@@ -136,6 +136,38 @@ def test_tensor_and_channel_fp8(oracle, dtype):
     _assert_same(q, q_o, "channel codes")
 
 
+@pytest.mark.parametrize("shape", [(64, 2048), (37, 7168), (5, 16384), (3, 16392), (130, 264), (2048, 7168)])
+def test_tensor_and_channel_fp8_bf16_row_kernels(oracle, shape):
+    # the bf16 kernels: rows held by one wavefront (K <= 2048), by a workgroup (K <= 16384), longer rows on the plain
+    # kernels; an all-zero row, a row of signed zeros, a row below the 1e-12 floor, format-sized magnitudes
+    from miles_amd.tools.convert_hf_to_fp8 import quant_fp8
+
+    w = W.gaussian_outliers(shape, std=0.02, p_outlier=0.001, gain=25.0, seed=1300 + shape[1], dtype=torch.bfloat16)
+    w[0] = 0
+    w[1, :64] = torch.tensor([-0.0, 0.0] * 32, dtype=torch.bfloat16)
+    w[2] = 1e-20
+    w[2, 5] = -3e-20
+    for strategy, ref in (("tensor", oracle.tensor_fp8), ("channel", oracle.channel_fp8)):
+        q, s = quant_fp8(w.to(DEV), strategy)
+        q_o, s_o = ref(w)
+        _assert_same(s, s_o, f"{strategy} scale")
+        _assert_same(q, q_o, f"{strategy} codes")
+    big = w.clone()
+    big[1, 7] = 3e38                               # one huge value: every other quotient underflows, signs must survive
+    q, s = quant_fp8(big.to(DEV), "tensor")
+    q_o, s_o = oracle.tensor_fp8(big)
+    _assert_same(s, s_o, "tensor scale, huge amax")
+    _assert_same(q, q_o, "tensor codes, huge amax")
+    # rows taken from a wider matrix (row stride != K): per channel reads them in place
+    wide = W.gaussian_outliers((shape[0], shape[1] + 64), std=0.02, p_outlier=0.001, gain=25.0, seed=77, dtype=torch.bfloat16)
+    view = wide.to(DEV)[:, : shape[1]]
+    for strategy, ref in (("tensor", oracle.tensor_fp8), ("channel", oracle.channel_fp8)):
+        q, s = quant_fp8(view, strategy)
+        q_o, s_o = ref(wide[:, : shape[1]].contiguous())
+        _assert_same(s, s_o, f"{strategy} scale, strided rows")
+        _assert_same(q, q_o, f"{strategy} codes, strided rows")
+
+
 # ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape", FP8_SHAPES)
 @pytest.mark.parametrize("kind", W.PATTERNS)
