@@ -86,6 +86,38 @@ __global__ __launch_bounds__(kFqThreads) void fake_quant_kernel(const void* __re
 }
 
 
+// Tensors that do not start on a 16-byte boundary: one lane per block, element-wise accesses, software conversions.
+__global__ __launch_bounds__(256) void fake_quant_generic_kernel(const void* __restrict__ x, int dtype,
+                                                                 void* __restrict__ y, int64_t blocks, int mode) {
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const int n = mode == 2 ? 16 : 32;
+    float amax = 0.0f;
+    for (int j = 0; j < n; j++) amax = __builtin_fmaxf(amax, __builtin_fabsf(load_f32(x, b * n + j, dtype)));
+    float scale;
+    if (mode == 2) {
+        const float hp = __builtin_fminf(__builtin_fmaxf(amax * u2f(0x3E2AAAABu), 0.001953125f), 448.0f);
+        scale = sw_e4m3fn_decode(sw_e4m3fn(hp));
+    } else {
+        amax = __builtin_fmaxf(amax, mode == 0 ? 1e-4f : u2f(0x01C00000u));
+        scale = ceil_pow2_normal(amax * u2f(mode == 0 ? 0x3B124925u : 0x3E2AAAABu));
+    }
+    const float top = mode == 0 ? 448.0f : 6.0f;
+    for (int j = 0; j < n; j++) {
+        const float v = __builtin_fminf(__builtin_fmaxf(load_f32(x, b * n + j, dtype) / scale, -top), top);
+        float q;
+        if (mode == 0) q = sw_e4m3fn_decode(sw_e4m3fn_sat(v));
+        else {
+            const uint32_t c = sw_e2m1(v);
+            const float mag = (c & 7u) < 2u ? 0.5f * (float)(c & 7u) : u2f(0x3F000000u + ((c & 7u) << 22));
+            q = v == 0.0f ? 0.0f : ((c & 8u) ? -mag : mag);     // an exact zero gives +0, a value rounded to zero keeps its sign
+        }
+        float o = q * scale;
+        asm volatile("" : "+v"(o));            // keep the product apart from the fp16 conversion (see fq_store8)
+        store_dtype(y, b * n + j, o, dtype);
+    }
+}
+
 // ---- act_quant: FP8 codes + one scale per 1 x block group of consecutive elements -------------------------------
 // Reference: miles/kernels/quant/fp8_act_quant.py:49-137 (`act_quant_kernel`, `act_quant`):
 //   amax' = max(amax, 1e-4);  s = amax' * f32(1/448), with MQ_ACT_ROUND_SCALE rounded up to a power of two
@@ -220,8 +252,14 @@ extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, i
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || mode < 0 || mode > 2) return mq_fail(MQ_ERR_ARG, "bad argument");
     const int block = mode == 2 ? 16 : 32;
     if (numel % block != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the block size");
-    if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
     if (numel == 0) return MQ_OK;
+    if ((((uintptr_t)x | (uintptr_t)y) & 15) != 0) {
+        const int64_t blocks = numel / block;
+        if ((blocks + 255) / 256 > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+        hipLaunchKernelGGL(fake_quant_generic_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, x, dtype, y, blocks, mode);
+        return mq_check_launch("fake quant");
+    }
     const int64_t units = numel / 8;
     if ((units + kFqThreads - 1) / kFqThreads > 0x7FFFFF00ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
     hipStream_t st = (hipStream_t)stream;

@@ -190,13 +190,21 @@ __device__ __forceinline__ void load8(const void* p, int64_t word, float f[8]) {
     }
 }
 
+// the same for a tensor that does not start on a 16-byte boundary: element by element
+template <int DT>
+__device__ __forceinline__ void load8_any(const void* p, int64_t word, float f[8], bool aligned) {
+    if (aligned) { load8<DT>(p, word, f); return; }
+#pragma unroll
+    for (int i = 0; i < 8; i++) f[i] = load_f32(p, word * 8 + i, DT);
+}
+
 // 16 lanes own one group; a lane handles the 8-element words lane, lane+16, ... of it.
 template <int DT>
 __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restrict__ w,
                                                              uint32_t* __restrict__ packed,
                                                              void* __restrict__ scale_out,
                                                              uint8_t* __restrict__ zero_out, int64_t total_groups,
-                                                             int words_per_group) {
+                                                             int words_per_group, bool aligned) {
     const int lane = threadIdx.x & 15;
     const int64_t team = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int64_t nteams = ((int64_t)gridDim.x * blockDim.x) >> 4;
@@ -210,7 +218,7 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restr
         float f[8];
         if (live)
             for (int k = lane; k < words_per_group; k += 16) {
-                load8<DT>(w, word0 + k, f);
+                load8_any<DT>(w, word0 + k, f, aligned);
 #pragma unroll
                 for (int i = 0; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
             }
@@ -227,7 +235,7 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restr
         const float big = __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
         const bool fast = DT != MQ_F32 && shared_div_ok(s) && shared_div_ok(sb) && big * ys < 1e30f;
         for (int k = lane; k < words_per_group; k += 16) {
-            load8<DT>(w, word0 + k, f);
+            load8_any<DT>(w, word0 + k, f, aligned);
             uint32_t word = 0;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -573,14 +581,14 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (K % group != 0 || group % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and the group size of 8");
     if (M % 8 != 0) return mq_fail(MQ_ERR_ARG, "asymmetric packing needs a multiple of 8 rows");
-    if (((uintptr_t)w % 16) != 0) return mq_fail(MQ_ERR_ARG, "weight must be 16-byte aligned");
+    const bool aligned = ((uintptr_t)w % 16) == 0;
     if (M == 0 || K == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
     const int64_t gpr = K / group, groups = M * gpr;
     int64_t blocks = (groups + 15) / 16;
     if (blocks > mq_grid_cap() * 4) blocks = mq_grid_cap() * 4;
     const int wpg = group / 8;
-    if (dtype == MQ_BF16 && (group == 128 || group == 64 || group == 32)) {
+    if (aligned && dtype == MQ_BF16 && (group == 128 || group == 64 || group == 32)) {
         const int64_t units = M * (K / 8);
         int64_t fblocks = (units + kI4Threads * kI4Unroll - 1) / (kI4Threads * kI4Unroll);
         const int chunk = (int)flat_chunk(fblocks);
@@ -594,11 +602,11 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
         else
             hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
     } else if (dtype == MQ_BF16)
-        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     else if (dtype == MQ_F16)
-        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     else
-        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F32>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg);
+        hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F32>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     int rc = mq_check_launch("int4 asymmetric pack");
     if (rc != MQ_OK) return rc;
     const int64_t zp_words = gpr * (M / 8);

@@ -1,0 +1,173 @@
+"""Seeded random shapes, dtypes and placements for every quantizer, against the oracle.
+
+The shape lists of the other GPU tests come from the reference's tests and from the benchmark configurations; this file
+adds what they do not enumerate: odd row counts, column counts at every residue the API allows, tensors that start in
+the middle of a larger allocation (so the 16-byte-aligned kernels and the plain ones both get exercised), fp16 and
+fp32 inputs, and values spread over many binades.  Everything is deterministic: the case list is generated from a
+fixed seed at collection time.
+"""
+
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F8 = torch.float8_e4m3fn
+_DTYPES = (torch.bfloat16, torch.bfloat16, torch.float16, torch.float32)     # bf16 twice as likely
+
+
+def _bits(t):
+    t = t.detach().cpu().contiguous()
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32}[t.element_size()])
+
+
+def _same(got, want, what):
+    g, w = _bits(got), _bits(want)
+    assert g.shape == w.shape, f"{what}: shape {tuple(g.shape)} vs {tuple(w.shape)}"
+    if not torch.equal(g, w):
+        bad = (g != w).nonzero()
+        i = tuple(bad[0].tolist())
+        raise AssertionError(f"{what}: {bad.shape[0]} of {g.numel()} differ; first at {i}: got {g[i].item()} want {w[i].item()}")
+
+
+def _tensor(seed, shape, dtype, offset):
+    """Values over ~12 binades with a few zeros; on the device the tensor starts `offset` elements into its storage."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g) * torch.exp2(torch.randint(-8, 4, shape, generator=g).float())
+    x = torch.where(torch.rand(shape, generator=g) < 0.02, torch.zeros(()), x).to(dtype)
+    n = x.numel()
+    flat = torch.zeros(n + offset, dtype=dtype, device=DEV)
+    flat[offset:] = x.reshape(-1).to(DEV)
+    return x, flat[offset:].view(shape)
+
+
+def _cases(name, count, columns_multiple_of, max_rows=300, max_cols=1100):
+    rng = random.Random(f"miles-quant-{name}")
+    out = []
+    for i in range(count):
+        rows = rng.choice([1, 2, 3, 5, 31, 64, 127, 128, 129, 200, rng.randint(1, max_rows)])
+        cols = columns_multiple_of * rng.randint(1, max(1, max_cols // columns_multiple_of))
+        dtype = rng.choice(_DTYPES)
+        offset = rng.choice([0, 0, 0, 1, 3, 8, 24])          # elements: 0 keeps the allocator's 256-byte alignment
+        out.append(pytest.param(i, (rows, cols), dtype, offset, id=f"{name}{i}-{rows}x{cols}-{str(dtype)[6:]}-o{offset}"))
+    return out
+
+
+@pytest.mark.parametrize("seed,shape,dtype,offset", _cases("fp8", 40, 1))
+def test_random_fp8_block_and_blockwise(oracle, seed, shape, dtype, offset):
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+
+    x, xd = _tensor(1000 + seed, shape, dtype, offset)
+    for name, fn, ref in (("block_fp8", lambda t: block_fp8(t, [128, 128]), lambda t: oracle.block_fp8(t, (128, 128))),
+                          ("fp8_blockwise_cast", fp8_blockwise_cast, oracle.fp8_blockwise_cast)):
+        q, s = fn(xd)
+        q_o, s_o = ref(x)
+        _same(s, s_o, f"{name} scales")
+        _same(q, q_o, f"{name} codes")
+    if dtype == torch.bfloat16:
+        q, s = per_block_cast_to_fp8(xd)
+        q_o, s_o = oracle.per_block_cast_to_fp8(x)
+        _same(s, s_o, "power-of-two scales")
+        _same(q, q_o, "power-of-two codes")
+        _same(weight_dequant(q.contiguous(), s.contiguous()), oracle.weight_dequant(q_o, s_o), "dequant")
+    for strategy, ref in (("tensor", oracle.tensor_fp8), ("channel", oracle.channel_fp8)):
+        q, s = quant_fp8(xd, strategy)
+        q_o, s_o = ref(x)
+        _same(s, s_o, f"{strategy} scale")
+        _same(q, q_o, f"{strategy} codes")
+
+
+@pytest.mark.parametrize("seed,shape,dtype,offset", _cases("mx", 40, 32))
+def test_random_mxfp8_mxfp4_and_row_block_fake_quant(oracle, seed, shape, dtype, offset):
+    from miles_amd.kernels.quant import fake_quant as fq
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+
+    x, xd = _tensor(2000 + seed, shape, dtype, offset)
+    q, s = mxfp8_quantize(xd)
+    q_o, s_o = oracle.mxfp8_quantize(x)
+    _same(s, s_o, "mxfp8 scales")
+    _same(q, q_o, "mxfp8 codes")
+    p, s4 = quantize_mxfp4(xd, 32)
+    p_o, s4_o = oracle.quantize_mxfp4(x, 32)
+    _same(s4, s4_o, "mxfp4 scales")
+    _same(p, p_o, "mxfp4 codes")
+    _same(dequantize_mxfp4(p, s4, 32), oracle.dequantize_mxfp4(p_o, s4_o, 32), "mxfp4 dequant")
+    for kind, fn in (("fp8", fq.fake_quant_fp8_forward), ("fp4", fq.fake_quant_fp4_forward),
+                     ("compressed_kv", fq.fake_quant_compressed_kv_forward)):
+        _same(fn(xd), oracle.fake_quant(x, kind), f"fake_quant {kind}")
+    for fmt in (None, "ue8m0"):
+        y, sc = act_quant(xd, 32, fmt)
+        y_o, sc_o = oracle.act_quant(x, 32, fmt)
+        if shape[1] % 64 == 0:
+            _same(act_quant(xd, 64, fmt)[0], oracle.act_quant(x, 64, fmt)[0], f"act_quant codes, block 64 {fmt}")
+        _same(sc, sc_o, f"act_quant scales {fmt}")
+        _same(y, y_o, f"act_quant codes {fmt}")
+    _same(fp8_simulate(xd, 32), oracle.fp8_simulate(x, 32), "fp8_simulate")
+
+
+@pytest.mark.parametrize("seed,shape,dtype,offset", _cases("int4", 40, 128, max_cols=1600))
+def test_random_int4(oracle, seed, shape, dtype, offset):
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda, pack_layer
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+
+    x, xd = _tensor(3000 + seed, shape, dtype, offset)
+    G = (32, 64, 128)[seed % 3]
+    for sym in (True, False):
+        out, scale, zero = fake_int4_quant_cuda(xd.contiguous(), (1, G), sym)
+        out_o, scale_o, zero_o = oracle.fake_int4_quant(x, (1, G), sym)
+        _same(scale, scale_o, f"fake int4 scales sym={sym}")
+        _same(out, out_o, f"fake int4 values sym={sym}")
+        if not sym:
+            _same(zero, zero_o, "fake int4 zero points")
+    if dtype == torch.float32:
+        return                                  # pack_layer is defined on 16-bit weights
+    packed, scale, _ = pack_layer(xd, G)
+    packed_o, scale_o, _ = oracle.pack_layer(x, G)
+    _same(scale, scale_o, "pack_layer scales")
+    _same(packed, packed_o, "pack_layer words")
+    _same(_dequantize_tensor(packed, scale, shape, G), oracle.int4_unpack_dequant(packed_o, scale_o, shape, G), "unpack")
+    if shape[0] % 8 == 0:
+        got = pack_layer(xd, G, sym=False)
+        want = oracle.pack_layer(x, G, sym=False)
+        for g, w, what in zip(got, want, ("asym words", "asym scales", "asym packed zero points")):
+            _same(g, w, what)
+
+
+@pytest.mark.parametrize("seed,shape,dtype,offset", _cases("nv", 40, 16))
+def test_random_nvfp4(oracle, monkeypatch, seed, shape, dtype, offset):
+    from miles_amd.kernels.quant.nvfp4_qdq import NVFP4QDQConfig, compute_nvfp4_amax, fused_nvfp4_qdq
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    x, xd = _tensor(4000 + seed, shape, dtype, offset)
+    if seed % 4 == 3:      # Four Over Six, alternating error modes, through the environment switches the reference reads
+        monkeypatch.setenv("NVTE_NVFP4_4OVER6", "weights")
+        monkeypatch.setenv("NVTE_NVFP4_4OVER6_ERR_MODE", "MSE" if seed % 8 == 7 else "MAE")
+        flags = 1 | (2 if seed % 8 == 7 else 0)
+        q, s, g = nvfp4_quantize_1d(xd)
+        q_o, s_o, g_o = oracle.nvfp4_quantize_1d(x, e4m3_max=256, flags=flags)
+        _same(g, g_o, "global scale (4/6)")
+        _same(s, s_o, "block scales (4/6)")
+        _same(q, q_o, "codes (4/6)")
+        return
+    q, s, g = nvfp4_quantize_1d(xd)
+    q_o, s_o, g_o = oracle.nvfp4_quantize_1d(x)
+    _same(g, g_o, "global scale")
+    _same(s, s_o, "block scales")
+    _same(q, q_o, "codes")
+    y, yd = _tensor(4500 + seed, shape, dtype, offset)
+    for got, want in zip(nvfp4_quantize_1d_pair(xd, yd), oracle.nvfp4_quantize_1d_pair(x, y)):
+        for a, b, what in zip(got, want, ("pair codes", "pair block scales", "pair global scale")):
+            _same(a, b, what)
+    if dtype != torch.float32:
+        amax = compute_nvfp4_amax(xd)
+        if xd.data_ptr() % 16:
+            with pytest.raises(ValueError, match="16-byte-aligned"):      # the reference's contract (nvfp4_qdq.py:1147-1149)
+                fused_nvfp4_qdq(xd, amax, NVFP4QDQConfig())
+        else:
+            _same(fused_nvfp4_qdq(xd, amax, NVFP4QDQConfig()), oracle.fused_nvfp4_qdq(x), "fused qdq")
