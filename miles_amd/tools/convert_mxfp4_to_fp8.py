@@ -35,6 +35,8 @@ def cast_e2m1fn_to_e4m3fn(x: torch.Tensor, scale: torch.Tensor) -> tuple[torch.T
     if scale.element_size() != 1:
         raise _lib.MilesQuantError(f"cast_e2m1fn_to_e4m3fn expects one-byte E8M0 scales, got {scale.dtype}")
     packed, sbytes = x.contiguous(), scale.contiguous().view(torch.uint8)
+    if packed.data_ptr() % 16:        # the kernel reads whole 16-byte pieces: a view that starts mid-allocation is moved first
+        packed = packed.clone()
     y = torch.empty((out_dim, in_dim), dtype=torch.float8_e4m3fn, device=x.device)
     tile_scale = torch.empty((out_dim // 128, in_dim // 128), dtype=torch.float32, device=x.device)
     launch.note_direct_call()

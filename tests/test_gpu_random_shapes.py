@@ -171,3 +171,21 @@ def test_random_nvfp4(oracle, monkeypatch, seed, shape, dtype, offset):
                 fused_nvfp4_qdq(xd, amax, NVFP4QDQConfig())
         else:
             _same(fused_nvfp4_qdq(xd, amax, NVFP4QDQConfig()), oracle.fused_nvfp4_qdq(x), "fused qdq")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_mxfp4_to_fp8(oracle, seed):
+    from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
+
+    rng = random.Random(f"miles-quant-recode-{seed}")
+    out_dim, in_dim, offset = 128 * rng.randint(1, 3), 128 * rng.randint(1, 5), rng.choice([0, 1, 16, 40])
+    g = torch.Generator().manual_seed(5000 + seed)
+    packed = torch.randint(-128, 128, (out_dim, in_dim // 2), dtype=torch.int8, generator=g)
+    scale = torch.randint(100, 140, (out_dim, in_dim // 32), dtype=torch.uint8, generator=g)
+    scale[0, 0] = 0                                            # 2^-127: far below the tile maximum
+    flat = torch.zeros(packed.numel() + offset, dtype=torch.int8, device=DEV)
+    flat[offset:] = packed.reshape(-1).to(DEV)
+    y, ts = cast_e2m1fn_to_e4m3fn(flat[offset:].view(out_dim, in_dim // 2), scale.to(DEV).view(torch.float8_e8m0fnu))
+    y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(packed, scale.view(torch.float8_e8m0fnu))
+    _same(ts, ts_o, "tile scales")
+    _same(y, y_o, "codes")
