@@ -103,6 +103,10 @@ class SyncPlan:
             copies = []
             for (name, old), (_, new) in zip(bucket, packed):
                 hits = writers.get(old.data_ptr()) if old.is_contiguous() and old.numel() else None
+                # codes written by a quantizer need their slot on a 16-byte boundary for the tuned kernels (a row-blocked
+                # FP8 job has no other kernel at all); a slot that follows, say, a 12-byte scale grid is filled by a copy
+                if hits and new.data_ptr() % 16 and any(f == 3 for _, f in hits):
+                    hits = None
                 if hits:
                     for ri, f in hits:
                         records[ri][f] = new.data_ptr()
@@ -125,7 +129,9 @@ class SyncPlan:
             new_records.extend(copies)
             new_marks.append(len(new_records))
         new_records.extend(tuple(r) for r in records[done:])
-        rehomed = {t.data_ptr() for bucket in buckets for _, t in bucket if t.numel() and t.data_ptr() in writers}
+        still_written = {rec[f] for rec in records for f in out_fields if rec[f] is not None}
+        rehomed = {t.data_ptr() for bucket in buckets for _, t in bucket
+                   if t.numel() and t.data_ptr() in writers and t.data_ptr() not in still_written}
         batch._keep = [t for t in batch._keep if t.data_ptr() not in rehomed]   # the first homes of re-pointed outputs
         batch._records = new_records
         batch._array = None
@@ -145,9 +151,11 @@ class SyncPlan:
 
     @classmethod
     def _inputs_alias(cls, weights: Mapping[str, torch.Tensor], batch: launch.JobBatch) -> bool:
-        """Every job input is live parameter storage or a declared constant (copy jobs move constants too)."""
+        """Every job input is live parameter storage, a declared constant (copy jobs move constants too), or
+        something a job of the list writes (a copy that moves quantizer output into a misaligned payload slot)."""
         spans = cls._weight_spans(weights)
-        return all(cls._in_spans(spans, ptr) or ptr in batch.constants for ptr in batch.input_pointers())
+        produced = batch.output_pointers()
+        return all(cls._in_spans(spans, ptr) or ptr in batch.constants or ptr in produced for ptr in batch.input_pointers())
 
     def matches(self, weights: Mapping[str, torch.Tensor]) -> bool:
         """True when `weights` is the parameter set the plan was recorded on.  Between RL steps the mapping holds
