@@ -450,3 +450,96 @@ def test_random_dense_models_sync_and_replay(oracle, seed, packed):
             break                                   # the follow-up case happens to have other shapes: nothing to copy into
         for k in dev:
             dev[k].copy_(cpu[k])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# randomly shaped MoE layers through the driver, in the three expert formats
+def _random_moe_case(seed):
+    import random
+    from argparse import Namespace
+
+    rng = random.Random(f"miles-moe-{seed}")
+    experts = rng.choice([1, 2, 3, 8])
+    hidden = 128 * rng.randint(1, 3)
+    ffn = 128 * rng.randint(1, 3)
+    layers = rng.randint(1, 2)
+    args = Namespace(hidden_size=hidden, num_attention_heads=4, num_query_groups=2, kv_channels=64, vocab_size=1000, num_layers=layers,
+                     update_weight_buffer_size=rng.choice([1 << 16, 1 << 19, 1 << 22]), q_lora_rank=None)
+    p, k = {}, 0
+    for layer in range(layers):
+        L = f"module.module.decoder.layers.{layer}."
+        p[L + "mlp.router.weight"] = W.gaussian_outliers((experts, hidden), std=0.02, p_outlier=0, gain=1, seed=7000 + 10 * seed + layer)
+        for e in range(experts):
+            k += 1
+            p[L + f"mlp.experts.linear_fc1.weight{e}"] = W.student_t_rows((2 * ffn, hidden), std=0.02, seed=7100 + 100 * seed + 2 * k)
+            p[L + f"mlp.experts.linear_fc2.weight{e}"] = W.student_t_rows((hidden, ffn), std=0.02, seed=7101 + 100 * seed + 2 * k)
+    return args, p, experts, layers
+
+
+def _moe_expected(oracle, fmt, args, params, basenames):
+    want = []
+    for name, param in params.items():
+        if fmt == "mxfp8":
+            for hf, t in name_maps.convert_qwen3moe_to_hf(args, name, param):
+                if "experts" in hf:
+                    q, s = oracle.mxfp8_quantize(t.contiguous())
+                    want += [(hf, q), (hf.replace(".weight", ".weight_scale_inv"), s)]
+                else:
+                    want.append((hf, t))
+            continue
+        hf = name_maps.convert_deepseekv3_to_hf(args, name, param)
+        if fmt == "nvfp4" and "linear_fc1" in name:
+            (gn, g), (un, u) = hf
+            for n, (q, s, gl) in zip((gn, un), oracle.nvfp4_quantize_1d_pair(g.contiguous(), u.contiguous())):
+                want += [(n, q), (n.replace(".weight", ".weight_scale"), s), (n.replace(".weight", ".weight_scale_2"), gl)]
+        elif fmt == "nvfp4" and "linear_fc2" in name:
+            n, t = hf[0]
+            q, s, gl = oracle.nvfp4_quantize_1d(t)
+            want += [(n, q), (n.replace(".weight", ".weight_scale"), s), (n.replace(".weight", ".weight_scale_2"), gl)]
+        elif fmt == "int4":
+            for n, t in hf:
+                if n.removesuffix(".weight") in basenames:
+                    packed, scale, _ = oracle.pack_layer(t.contiguous(), 128)
+                    want += [(n.replace(".weight", ".weight_packed"), packed), (n.replace(".weight", ".weight_scale"), scale),
+                             (n.replace(".weight", ".weight_shape"), torch.tensor(t.shape, dtype=torch.int32))]
+                else:
+                    want.append((n, t))
+        else:
+            want += hf
+    return want
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("fmt", ["mxfp8", "nvfp4", "int4"])
+@pytest.mark.parametrize("packed", [False, True])
+def test_random_moe_models_sync_and_replay(oracle, seed, fmt, packed):
+    args, cpu, experts, layers = _random_moe_case(seed)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    basenames = {f"model.layers.{l}.mlp.experts.{e}.{p}_proj" for l in range(layers) for e in range(experts) for p in ("gate", "up", "down")}
+    model, cfg, extra = {
+        "mxfp8": ("qwen3moe", {"quant_method": "mxfp8"}, {}),
+        "nvfp4": ("deepseekv3", {"quant_method": "modelopt", "quant_algo": "NVFP4"}, {}),
+        "int4": ("kimi_k2", {"quant_method": "compressed-tensors", "format": "pack-quantized",
+                             "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4, "type": "int"}}}},
+                 {"packed_weight_basenames": basenames}),
+    }[fmt]
+    upd = WeightUpdater(args, weights_getter=lambda: dev, model_name=model, quantization_config=cfg, send_bucket=None,
+                        packed_buckets=packed, **extra)
+    for round_ in range(3):
+        buckets = []
+        upd.send_bucket = buckets.append
+        upd.update_weights()
+        torch.cuda.synchronize()
+        flat = [nt for b in buckets for nt in b]
+        want = _moe_expected(oracle, fmt, args, cpu, basenames)
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} (sync {round_})")
+        if packed:
+            for b in buckets:
+                assert torch.equal(b.flat.cpu(), _payload_bytes(list(b)))
+        cpu = {k: W.student_t_rows(tuple(v.shape), std=0.03, seed=8000 + 37 * seed + round_ * 1000 + i) if v.dim() == 2 and "router" not in k else v
+               for i, (k, v) in enumerate(cpu.items())}
+        for k in dev:
+            dev[k].copy_(cpu[k])
+    assert upd._plan is not None and upd._plan.replayable
