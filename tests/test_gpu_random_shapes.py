@@ -189,3 +189,50 @@ def test_random_mxfp4_to_fp8(oracle, seed):
     y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(packed, scale.view(torch.float8_e8m0fnu))
     _same(ts, ts_o, "tile scales")
     _same(y, y_o, "codes")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_job_lists_in_one_submission(oracle, seed):
+    """150 jobs of mixed kinds and sizes recorded in random order and submitted with one call: the native driver has to cut
+    the list into launches by kind, size class, NVFP4 pairing and group limit, and every job must come out as if alone."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    rng = random.Random(f"miles-jobs-{seed}")
+    kinds = ["cast", "block", "mxfp8", "int4", "nvfp4", "pair", "mxfp4"]
+    plan = []
+    for i in range(150):
+        kind = rng.choice(kinds) if rng.random() < 0.5 or not plan else plan[-1][0]       # runs of one kind and switches
+        shape = (rng.choice([1, 8, 64, 128, 200, 384]), 128 * rng.randint(1, 6))
+        plan.append((kind, shape, i))
+    cpu, dev = {}, {}
+    for kind, shape, i in plan:
+        for tag in ("a", "b") if kind == "pair" else ("a",):
+            g = torch.Generator().manual_seed(6000 + 1000 * seed + 2 * i + (tag == "b"))
+            cpu[i, tag] = (torch.randn(shape, generator=g) * 0.05).to(torch.bfloat16)
+            dev[i, tag] = cpu[i, tag].to(DEV)
+    results = {}
+    with launch.deferred() as batch:
+        for kind, shape, i in plan:
+            x = dev[i, "a"]
+            results[i] = {"cast": lambda: fp8_blockwise_cast(x), "block": lambda: block_fp8(x, [128, 128]),
+                          "mxfp8": lambda: mxfp8_quantize(x), "int4": lambda: pack_layer(x, 128)[:2],
+                          "nvfp4": lambda: nvfp4_quantize_1d(x), "mxfp4": lambda: quantize_mxfp4(x, 32),
+                          "pair": lambda: nvfp4_quantize_1d_pair(x, dev[i, "b"])}[kind]()
+        assert len(batch) == sum(2 if k == "pair" else 1 for k, _, _ in plan)
+    for kind, shape, i in plan:
+        x = cpu[i, "a"]
+        want = {"cast": lambda: oracle.fp8_blockwise_cast(x), "block": lambda: oracle.block_fp8(x, (128, 128)),
+                "mxfp8": lambda: oracle.mxfp8_quantize(x), "int4": lambda: oracle.pack_layer(x, 128)[:2],
+                "nvfp4": lambda: oracle.nvfp4_quantize_1d(x), "mxfp4": lambda: oracle.quantize_mxfp4(x, 32),
+                "pair": lambda: oracle.nvfp4_quantize_1d_pair(x, cpu[i, "b"])}[kind]()
+        got = results[i]
+        if kind == "pair":
+            got, want = [t for half in got for t in half], [t for half in want for t in half]
+        for j, (g_, w_) in enumerate(zip(got, want)):
+            _same(g_, w_, f"job {i} ({kind} {shape}) output {j}")
