@@ -543,7 +543,7 @@ def main():
 
     plan = updater._plan
     assert plan is not None and plan.replayable, "the benchmark expects the replayable plan path"
-    jobs_meta = [rec[7] * rec[8] for rec in plan.batch._records]     # rows * cols of every job
+    jobs_meta = [rec[7] * rec[8] for rec in plan.batch.records]     # rows * cols of every job
     line = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -42,6 +42,30 @@ class JobBatch:
         self._keep.extend(keep)
         self._array = None
 
+    # Field positions of a job record (the order of `mq_job` in include/miles_quant.h).
+    KIND, DTYPE, IN, OUT, SCALE, AUX, AUX2, ROWS, COLS, LD, P0, P1, ROWS_PER_BLOCK, BLOCK_STRIDE = range(14)
+
+    @property
+    def records(self) -> list[tuple]:
+        """The recorded jobs, in submission order (read-only view for planners; use `replace_records` to change them)."""
+        return self._records
+
+    def replace_records(self, records: list[tuple], keep: list[torch.Tensor] | None = None) -> None:
+        """Swap in an edited job list (a planner re-pointing outputs, adding copy jobs); `keep` replaces the tensors
+        the batch holds alive."""
+        self._records = list(records)
+        if keep is not None:
+            self._keep = list(keep)
+        self._array = None
+
+    def hold(self, tensor: torch.Tensor) -> None:
+        """Keep a tensor alive for as long as the batch exists."""
+        self._keep.append(tensor)
+
+    @property
+    def held(self) -> list[torch.Tensor]:
+        return self._keep
+
     def freeze(self):
         """Materialise the ctypes job array (done once; `run` can then be repeated)."""
         if self._array is None:
@@ -125,7 +149,7 @@ def note_constant(t: torch.Tensor) -> None:
     batch = active_batch()
     if batch is not None:
         batch.constants.add(t.data_ptr())
-        batch._keep.append(t)
+        batch.hold(t)
 
 
 def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0,

@@ -88,11 +88,11 @@ class SyncPlan:
         bucket's range.  Returns the packed buckets and the new job marks."""
         out_fields = (3, 4, 6)       # out, scale, aux2 of a job record
         writers: dict[int, list[tuple[int, int]]] = {}
-        for ri, rec in enumerate(batch._records):
+        for ri, rec in enumerate(batch.records):
             for f in out_fields:
                 if rec[f] is not None and rec[0] != _lib.JOB_COPY:
                     writers.setdefault(rec[f], []).append((ri, f))
-        records = [list(r) for r in batch._records]
+        records = [list(r) for r in batch.records]
         new_buckets: list[Unit] = []
         copies_of: list[list[tuple]] = []
         for bucket in buckets:      # first re-point every job (a bucket's range may hold jobs of the next bucket)
@@ -116,8 +116,8 @@ class SyncPlan:
                     nbytes = old.numel() * old.element_size()
                     copies.append((_lib.JOB_COPY, 0, old.data_ptr(), new.data_ptr(), None, None, None, 1, nbytes, nbytes,
                                    0, 0, 0, 0))
-                    batch._keep.append(old)
-            batch._keep.append(flat)
+                    batch.hold(old)
+            batch.hold(flat)
             new_buckets.append(packed)
             copies_of.append(copies)
         new_records: list[tuple] = []
@@ -132,9 +132,8 @@ class SyncPlan:
         still_written = {rec[f] for rec in records for f in out_fields if rec[f] is not None}
         rehomed = {t.data_ptr() for bucket in buckets for _, t in bucket
                    if t.numel() and t.data_ptr() in writers and t.data_ptr() not in still_written}
-        batch._keep = [t for t in batch._keep if t.data_ptr() not in rehomed]   # the first homes of re-pointed outputs
-        batch._records = new_records
-        batch._array = None
+        # drop the first homes of re-pointed outputs
+        batch.replace_records(new_records, keep=[t for t in batch.held if t.data_ptr() not in rehomed])
         return new_buckets, new_marks
 
     @staticmethod
@@ -184,7 +183,7 @@ class SyncPlan:
         14.6 -> 14.1 ms).  Buckets of large tensors are submitted as they are -- merging their launches made the
         Qwen3-4B FP8 sync 1 % slower.  A cut never falls between NVFP4 jobs that share an amax record."""
         if self._marks is None:
-            records, total, done, marks = self.batch._records, len(self.batch), 0, []
+            records, total, done, marks = self.batch.records, len(self.batch), 0, []
             group = _lib.MAX_GROUP
             for mark in self.jobs_done_at_bucket:
                 if mark > done:

@@ -258,7 +258,7 @@ def test_packed_buckets_fp8_plan_writes_payload_in_place(oracle):
     # quantizer outputs live in the payloads; the only ones outside are codes whose slot is not 16-byte aligned (it
     # follows a scale grid of odd size), and those reach the payload through a copy job
     payload = {(b.flat.data_ptr(), b.flat.data_ptr() + b.flat.numel()) for b in got}
-    copied_from = {rec[2] for rec in upd._plan.batch._records if rec[0] == _lib.JOB_COPY}
+    copied_from = {rec[2] for rec in upd._plan.batch.records if rec[0] == _lib.JOB_COPY}
     outputs = upd._plan.batch.output_pointers()
     outside = [ptr for ptr in outputs if not any(lo <= ptr < hi for lo, hi in payload)]
     assert all(ptr in copied_from for ptr in outside) and len(outside) < len(outputs) / 2

@@ -376,7 +376,7 @@ def test_sync_plan_tops_up_small_trailing_launches_only():
 
     def plan_with(jobs, marks):
         batch = launch.JobBatch()
-        batch._records = jobs
+        batch.replace_records(jobs)
         return SyncPlan(batch=batch, buckets=[[] for _ in marks], jobs_done_at_bucket=marks, signature=(), replayable=True)
 
     def job(kind, elements, aux=None):
