@@ -56,6 +56,14 @@ int mq_fp8_blockwise_cast(const void* x, int dtype, int64_t stride_m, int64_t st
 int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws, int64_t M,
                         int64_t K, int per_channel, float floor_in_dtype, void* stream);
 
+/* transform_scale_ue8m0(sf, mn)                      .../processors/quantizer_fp8.py:141-142 (SGLang; DeepGEMM layout)
+ *   sf  [batch, tile_rows, kb] fp32 power-of-two tile scales of a [mn, 128*kb] weight, tile_rows >= ceil(mn/128)
+ *   out [batch, ceil(kb/4), align(mn,4)] int32: out[b,j,r] = sum_e exponent_byte(sf[b, r/128, 4j+e]) << 8e,
+ *   zero where r >= mn or 4j+e >= kb; the caller views it transposed as [batch, mn, ceil(kb/4)]
+ *   row_major != 0: out is that view made contiguous instead, [batch, mn, ceil(kb/4)] with no padding rows */
+int mq_ue8m0_pack_scales(const float* sf, int32_t* out, int64_t batch, int64_t mn, int64_t kb, int64_t tile_rows,
+                         int row_major, void* stream);
+
 /* weight_dequant(x, s, block_size)                   tools/fp8_cast_bf16.py:30-40
  *   x [M,N] e4m3fn contiguous; s [ceil(M/block), ceil(N/block)] fp32; y [M,N] bf16 */
 int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block, void* stream);
@@ -181,9 +189,12 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *                                                                          aux2 = fp32 weight_scale_2
  *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *   MQ_JOB_COPY                 bytes         bytes         -              -                           -
- *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
  *     (rows * cols bytes copied verbatim: how a pass-through tensor reaches its place in a packed transport bucket,
  *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208)
+ *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
+ *   MQ_JOB_UE8M0_PACK           fp32 tiles    int32 words   -              -                           batch, tile_rows
+ *     (mq_ue8m0_pack_scales with mn = rows, kb = cols, row_major = ld; its input is usually the scale output of an
+ *      earlier job)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
@@ -197,7 +208,8 @@ enum {
     MQ_JOB_NVFP4 = 5,
     MQ_JOB_MXFP4 = 6,
     MQ_JOB_COPY = 7,
-    MQ_JOB_FP8_BLOCK_POW2 = 8
+    MQ_JOB_FP8_BLOCK_POW2 = 8,
+    MQ_JOB_UE8M0_PACK = 9
 };
 typedef struct mq_job {
     int32_t kind;

@@ -25,6 +25,7 @@ SIGNATURES = {
     "mq_fp8_block_quant_pow2": [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _vp],
     "mq_fp8_blockwise_cast": [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
     "mq_fp8_scaled_quant": [_vp, _i32, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _vp],
+    "mq_ue8m0_pack_scales": [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp8_quant": [_vp, _i32, _vp, _vp, _i64, _i64, _vp],
     "mq_int4_fake_quant": [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp],
@@ -50,7 +51,7 @@ MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensor
 NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
- JOB_COPY, JOB_FP8_BLOCK_POW2) = range(9)
+ JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK) = range(10)
 
 
 class Job(_c.Structure):

@@ -580,6 +580,52 @@ int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st) {
     return mq_check_launch("fp8 block dequant");
 }
 
+// One lane per output word.  ROW_MAJOR = false: DeepGEMM's layout [batch][ceil(kb/4)][align(mn,4)], consecutive lanes
+// take consecutive rows; true: the same words as a contiguous [batch][mn][ceil(kb/4)] array (what `.contiguous()` makes
+// of the transposed view, e.g. inside a flattened transport payload).
+template <bool ROW_MAJOR>
+__global__ __launch_bounds__(256) void ue8m0_pack_scales_kernel(const float* __restrict__ sf, uint32_t* __restrict__ out,
+                                                                int64_t total, int64_t mn, int64_t amn, int64_t kb,
+                                                                int64_t kw, int64_t tile_rows) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        int64_t r, j, b;
+        if (ROW_MAJOR) {
+            j = i % kw;
+            r = (i / kw) % mn;
+            b = i / (kw * mn);
+        } else {
+            r = i % amn;
+            j = (i / amn) % kw;
+            b = i / (amn * kw);
+        }
+        uint32_t word = 0;
+        if (r < mn) {
+            const float* row = sf + (b * tile_rows + r / 128) * kb;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (4 * j + e < kb) word |= ((__float_as_uint(row[4 * j + e]) >> 23) & 0xFFu) << (8 * e);
+        }
+        out[i] = word;
+    }
+}
+
+extern "C" int mq_ue8m0_pack_scales(const float* sf, int32_t* out, int64_t batch, int64_t mn, int64_t kb,
+                                    int64_t tile_rows, int row_major, void* stream) {
+    if (!sf || !out) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (batch < 0 || mn < 0 || kb < 0 || tile_rows < (mn + 127) / 128) return mq_fail(MQ_ERR_ARG, "bad shape");
+    const int64_t amn = (mn + 3) / 4 * 4, kw = (kb + 3) / 4, total = batch * kw * (row_major ? mn : amn);
+    if (total == 0) return MQ_OK;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > mq_grid_cap()) blocks = mq_grid_cap();
+    const dim3 grid((unsigned)blocks), blk(256);
+    if (row_major)
+        hipLaunchKernelGGL(ue8m0_pack_scales_kernel<true>, grid, blk, 0, (hipStream_t)stream, sf, (uint32_t*)out, total, mn, amn, kb, kw, tile_rows);
+    else
+        hipLaunchKernelGGL(ue8m0_pack_scales_kernel<false>, grid, blk, 0, (hipStream_t)stream, sf, (uint32_t*)out, total, mn, amn, kb, kw, tile_rows);
+    return mq_check_launch("ue8m0 scale pack");
+}
+
 extern "C" int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block,
                                     void* stream) {
     if (!x || !s || !y) return mq_fail(MQ_ERR_ARG, "null pointer");

@@ -63,10 +63,12 @@ static bool job_fast(const mq_job& j) {
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_FP8_BLOCK_POW2) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_UE8M0_PACK) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     if (j.kind == MQ_JOB_COPY) return MQ_OK;
+    if (j.kind == MQ_JOB_UE8M0_PACK)
+        return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
     if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
     if (j.rows_per_block != 0) {
@@ -95,6 +97,8 @@ static int run_single(const mq_job& j, void* stream) {
             return mq_int4_group_quant_pack(j.in, j.dtype, (int32_t*)j.out, j.scale, j.rows, j.cols, j.p0, stream);
         case MQ_JOB_MXFP4:
             return mq_mxfp4_quant(j.in, j.dtype, (uint8_t*)j.out, (uint8_t*)j.scale, j.rows * j.cols, j.p0, stream);
+        case MQ_JOB_UE8M0_PACK:
+            return mq_ue8m0_pack_scales((const float*)j.in, (int32_t*)j.out, j.p0, j.rows, j.cols, j.p1, j.ld != 0, stream);
         default:
             return mq_fail(MQ_ERR_ARG, "unknown job kind");
     }

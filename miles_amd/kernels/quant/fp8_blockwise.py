@@ -83,3 +83,41 @@ def per_block_cast_to_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     s = torch.empty(ceil_div(M, 128), ceil_div(N, 128), dtype=torch.float32, device=x.device)
     launch.submit(_lib.JOB_FP8_BLOCK_POW2, x, y, s, None, None, M, N, ld, 128, 128, rpb, bstride)
     return y, s
+
+
+def quant_weight_ue8m0(weight_dequant: torch.Tensor, weight_block_size) -> tuple[torch.Tensor, torch.Tensor]:
+    """bf16 [..., n, k] -> (float8_e4m3fn [..., n, k], float32 [..., ceil(n/128), ceil(k/128)] power-of-two scales).
+
+    Stands in for SGLang's `quant_weight_ue8m0` (imported at miles/backends/megatron_utils/sglang.py:13-20, called
+    at .../processors/quantizer_fp8.py:141): `per_block_cast_to_fp8` over the weight flattened to [-1, k].  SGLang's
+    source is not part of the reference tree; the published algorithm is restated.
+    """
+    assert list(weight_block_size) == [128, 128]
+    assert weight_dequant.dtype == torch.bfloat16
+    *batch_dims, n, k = weight_dequant.shape
+    out_w, out_s = per_block_cast_to_fp8(weight_dequant.view((-1, k)))
+    return out_w.view((*batch_dims, n, k)), out_s.view((*batch_dims, ceil_div(n, 128), ceil_div(k, 128)))
+
+
+def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:
+    """float32 [(b,) ceil(mn/128), kb] tile scales -> int32 [(b,) mn, ceil(kb/4)] with strides (1, align(mn, 4)).
+
+    Stands in for SGLang's `transform_scale_ue8m0` (.../processors/quantizer_fp8.py:142): every weight row gets the
+    scales of its tile row (`index_select(-2, arange(mn) // 128)`), then DeepGEMM's
+    `get_mn_major_tma_aligned_packed_ue8m0_tensor`: the exponent byte of each scale, four neighbours along k in one
+    int32 (lowest byte first, zero padded), rows contiguous in memory and padded to a multiple of 4.  Restated from
+    the published algorithm; neither library is part of the reference tree.
+    """
+    _lib.require_gpu(sf, "transform_scale_ue8m0")
+    assert sf.dtype == torch.float32 and sf.dim() in (2, 3)
+    squeeze = sf.dim() == 2
+    if squeeze:
+        sf = sf.unsqueeze(0)
+    b, tile_rows, kb = sf.shape
+    if ceil_div(mn, 128) > tile_rows:
+        raise IndexError(f"index out of range: {mn} rows need {ceil_div(mn, 128)} tile rows of scales, got {tile_rows}")
+    sf = sf.contiguous()            # no copy for the scales a quantizer just produced (they may not be computed yet)
+    storage = torch.empty((b, ceil_div(kb, 4), ceil_div(mn, 4) * 4), dtype=torch.int32, device=sf.device)
+    launch.submit(_lib.JOB_UE8M0_PACK, sf, storage, None, None, None, mn, kb, 0, b, tile_rows)
+    packed = storage.mT[:, :mn, :]
+    return packed.squeeze(0) if squeeze else packed

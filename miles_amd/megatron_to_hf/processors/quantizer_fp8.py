@@ -4,9 +4,9 @@ Same interface and decisions as the reference's
 miles/backends/megatron_utils/megatron_to_hf/processors/quantizer_fp8.py:
 `quantize_params_fp8` (:16-128) decides from the Megatron parameter name, `_quantize_param` (:131-159)
 quantizes one HF tensor and names its scale.  The 128x128 cast is the gfx950 kernel behind
-`fp8_blockwise_cast`; the power-of-two-scale variants the reference takes from SGLang
-(`quant_weight_ue8m0`, `per_block_cast_to_fp8`) are third-party code that is not part of this library and
-raise if a configuration asks for them.
+`fp8_blockwise_cast`; the power-of-two-scale variants the reference takes from SGLang (`per_block_cast_to_fp8`,
+`quant_weight_ue8m0` + `transform_scale_ue8m0`) are third-party code outside the reference tree, restated here from
+their published algorithms.
 """
 
 from __future__ import annotations
@@ -15,7 +15,8 @@ import os
 
 import torch
 
-from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+from miles_amd.kernels.quant.fp8_blockwise import (fp8_blockwise_cast, per_block_cast_to_fp8, quant_weight_ue8m0,
+                                                   transform_scale_ue8m0)
 from miles_amd.tools.convert_hf_to_fp8 import tensor_fp8
 
 from ._names import parse_layer_param
@@ -120,9 +121,12 @@ def _quantize_param(args, name, weight, weight_block_size, ignored_layers, packe
     if weight_block_size is not None:
         scale_format = _get_scale_format(args, name, weight_block_size)
         if scale_format == "ue8m0":
-            raise NotImplementedError("UE8M0 (DeepGEMM) FP8 scales come from SGLang's quant_weight_ue8m0, "
-                                      "which this library does not provide")
-        if os.environ.get("NVTE_FP8_BLOCK_SCALING_FP32_SCALES", "1") == "0" and list(weight_block_size) == [128, 128]:
+            if weight.dim() == 3 and getattr(args, "qkv_row_block_views", False):
+                qweight, scale = per_block_cast_to_fp8(weight)      # a [groups, rows, hidden] view standing for a matrix
+            else:
+                qweight, scale = quant_weight_ue8m0(weight, weight_block_size=weight_block_size)
+            scale = transform_scale_ue8m0(scale, mn=qweight.shape[-2])
+        elif os.environ.get("NVTE_FP8_BLOCK_SCALING_FP32_SCALES", "1") == "0" and list(weight_block_size) == [128, 128]:
             qweight, scale = per_block_cast_to_fp8(weight)      # power-of-two scales, kept as fp32
         else:
             qweight, scale = fp8_blockwise_cast(weight, weight_block_size)

@@ -39,9 +39,11 @@ def _dequantize_tensor(weight_packed: torch.Tensor, weight_scale: torch.Tensor, 
     else:
         shape = tuple(weight_shape)
     _lib.require_gpu(weight_packed, "_dequantize_tensor")
-    if group_size <= 0:
-        raise NotImplementedError("per-element scales (group_size <= 0) are not implemented on gfx950")
     M, K = shape
+    if group_size <= 0:                 # one scale per element (:75-76): the same kernel with groups of one column
+        if weight_scale.numel() != M * K:
+            raise ValueError(f"Scale shape {tuple(weight_scale.shape)} incompatible with weight shape {shape}")
+        weight_scale, group_size = weight_scale.reshape(M, K), 1
     packed = weight_packed.contiguous()
     if packed.dtype != torch.int32 or tuple(packed.shape) != (M, -(-K // 8)):
         raise ValueError(f"Packed shape {tuple(packed.shape)} / dtype {packed.dtype} incompatible with weight shape {shape}")

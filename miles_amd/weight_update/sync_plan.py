@@ -103,6 +103,13 @@ class SyncPlan:
             copies = []
             for (name, old), (_, new) in zip(bucket, packed):
                 hits = writers.get(old.data_ptr()) if old.is_contiguous() and old.numel() else None
+                if not old.is_contiguous() and old.numel():
+                    # the transposed view of packed UE8M0 scales: its job can write the contiguous form straight into the slot
+                    packers = [ri for ri, f in writers.get(old.data_ptr(), ()) if records[ri][launch.JobBatch.KIND] == _lib.JOB_UE8M0_PACK]
+                    if packers and new.data_ptr() % 4 == 0:
+                        for ri in packers:
+                            records[ri][launch.JobBatch.OUT], records[ri][launch.JobBatch.LD] = new.data_ptr(), 1
+                        continue
                 # codes written by a quantizer need their slot on a 16-byte boundary for the tuned kernels (a row-blocked
                 # FP8 job has no other kernel at all); a slot that follows, say, a 12-byte scale grid is filled by a copy
                 if hits and new.data_ptr() % 16 and any(f == 3 for _, f in hits):

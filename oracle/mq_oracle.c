@@ -331,6 +331,26 @@ void mqo_fp8_block_pow2(const void* x, int dtype, int64_t M, int64_t N, int64_t 
 /* A-5  FP8 block dequant (tools/fp8_cast_bf16.py:15-40;               */
 /*      tools/convert_mimo_v2_to_bf16.py:44-47)                        */
 /* ------------------------------------------------------------------ */
+/* SGLang's transform_scale_ue8m0 (called at quantizer_fp8.py:142; third party, not in the reference tree; restated
+ * from DeepGEMM's published get_mn_major_tma_aligned_packed_ue8m0_tensor): weight row r takes the scales of tile
+ * row r/128; byte = (bits(sf) >> 23) & 255; four neighbours along k share one int32, lowest byte first, missing
+ * ones zero; storage is [batch][ceil(kb/4)][align(mn,4)] (rows contiguous), rows >= mn zero.  Parity unpinned. */
+void mqo_ue8m0_pack_scales(const float* sf, int64_t batch, int64_t mn, int64_t kb, int32_t* out) {
+    int64_t amn = (mn + 3) / 4 * 4, kw = (kb + 3) / 4, tile_rows = (mn + 127) / 128;
+    for (int64_t b = 0; b < batch; b++)
+        for (int64_t j = 0; j < kw; j++)
+            for (int64_t r = 0; r < amn; r++) {
+                uint32_t word = 0;
+                for (int e = 0; e < 4 && r < mn; e++) {
+                    if (4 * j + e >= kb) break;
+                    uint32_t bits;
+                    memcpy(&bits, sf + (b * tile_rows + r / 128) * kb + 4 * j + e, 4);
+                    word |= ((bits >> 23) & 0xFFu) << (8 * e);
+                }
+                out[(b * kw + j) * amn + r] = (int32_t)word;
+            }
+}
+
 /* y[i,j] = bf16_rne( f32(e4m3(x[i,j])) * s[i/B, j/B] ) */
 void mqo_fp8_block_dequant(const uint8_t* x, const float* s, int64_t M, int64_t N,
                            int block, uint16_t* y) {

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.mqo_fp8_per_tensor_or_channel.argtypes = [vp, i32, i64, i64, i64, i32, f32, vp, vp]
         L.mqo_fp8_blockwise_cast.restype = None
         L.mqo_fp8_blockwise_cast.argtypes = [vp, i32, i64, i64, i64, i64, i32, i32, vp, vp]
+        L.mqo_ue8m0_pack_scales.restype = None
+        L.mqo_ue8m0_pack_scales.argtypes = [vp, i64, i64, i64, vp]
         L.mqo_fp8_block_pow2.restype = None
         L.mqo_fp8_block_pow2.argtypes = [vp, i32, i64, i64, i64, vp, vp]
         L.mqo_fp8_block_dequant.restype = None
@@ -182,6 +184,20 @@ def per_block_cast_to_fp8(x: torch.Tensor):
     return y.view(torch.float8_e4m3fn), s
 
 
+def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:
+    """SGLang's transform_scale_ue8m0 (DeepGEMM packed UE8M0 layout), restated: parity unpinned.
+    float32 [(b,) ceil(mn/128), kb] -> int32 [(b,) mn, ceil(kb/4)] with strides (1, align(mn, 4))."""
+    _check_cpu(sf)
+    assert sf.dtype == torch.float32 and sf.dim() in (2, 3)
+    squeeze = sf.dim() == 2
+    sf3 = (sf.unsqueeze(0) if squeeze else sf)[:, : ceil_div(mn, 128)].contiguous()
+    b, _, kb = sf3.shape
+    storage = torch.empty((b, ceil_div(kb, 4), ceil_div(mn, 4) * 4), dtype=torch.int32)
+    lib().mqo_ue8m0_pack_scales(sf3.data_ptr(), b, mn, kb, storage.data_ptr())
+    packed = storage.mT[:, :mn, :]
+    return packed.squeeze(0) if squeeze else packed
+
+
 def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128) -> torch.Tensor:
     """tools/fp8_cast_bf16.py:30-40 -> bf16 [M,N]."""
     assert x.is_contiguous() and s.is_contiguous() and x.dim() == 2 and s.dim() == 2
@@ -251,6 +267,8 @@ def int4_unpack_dequant(weight_packed: torch.Tensor, weight_scale: torch.Tensor,
     assert weight_packed.device.type == "cpu" and weight_packed.dtype == torch.int32
     _check_cpu(weight_scale)
     M, K = (int(v) for v in (weight_shape.view(-1).tolist() if isinstance(weight_shape, torch.Tensor) else weight_shape))
+    if group_size <= 0:                 # :75-76, one scale per element
+        weight_scale, group_size = weight_scale.reshape(M, K), 1
     p, s = weight_packed.contiguous(), weight_scale.contiguous()
     assert p.shape == (M, -(-K // 8)) and K % group_size == 0 and s.numel() == M * (K // group_size)
     out = torch.empty((M, K), dtype=torch.bfloat16)

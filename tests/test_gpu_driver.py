@@ -374,6 +374,37 @@ def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
     assert upd._plan is not None and upd._plan.replayable
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_dense_fp8_sync_with_packed_ue8m0_scales(oracle, packed):
+    # DeepGEMM requantization (quantizer_fp8.py:140-142): power-of-two tile scales, then four exponent bytes per int32
+    # in a row-contiguous layout; the packer consumes the scales of a job recorded just before it
+    import copy
+    args = copy.copy(ARGS)
+    args.deepgemm_weight_requant_ue8m0 = True
+    cpu = _dense_model(61)
+    for name in list(cpu):      # an MLP width of 640 gives down_proj five tile columns: two words per row, a strided view
+        if name.endswith("mlp.linear_fc1.weight"):
+            cpu[name] = W.gaussian_outliers((2 * 640, 256), std=0.02, p_outlier=0.001, gain=20.0, seed=611)
+        elif name.endswith("mlp.linear_fc2.weight"):
+            cpu[name] = W.gaussian_outliers((256, 640), std=0.02, p_outlier=0.001, gain=20.0, seed=612)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(args, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None,
+                        packed_buckets=packed)
+    for _ in range(3):      # recorded plan, then two replays
+        flat = dict(nt for b in _run(upd) for nt in b)
+        for name, param in cpu.items():
+            for hf, t in name_maps.convert_qwen2_to_hf(args, name, param):
+                if hf.endswith("_proj.weight"):
+                    q, s = oracle.per_block_cast_to_fp8(t.contiguous())
+                    want = oracle.transform_scale_ue8m0(s, t.shape[0])
+                    got = flat[hf.replace(".weight", ".weight_scale_inv")]
+                    _same(flat[hf], q, hf)
+                    assert got.dtype == torch.int32 and got.shape == want.shape, hf
+                    assert torch.equal(got.cpu(), want), hf + " packed scale"
+                    assert got.is_contiguous() if packed else got.stride() == want.stride(), hf
+    assert upd._plan is not None and upd._plan.replayable
+
+
 # ---------------------------------------------------------------------------------------------------------------------
 # randomly shaped dense models through the whole driver (seeded; shapes the fixed models above do not reach: head
 # sizes that rule the in-place q/k/v views out, hidden sizes off the 128 grid, buffer sizes that cut anywhere)

@@ -348,6 +348,24 @@ def test_int4_unpack_dequant(oracle, shape, G, sdt):
     _assert_same(got, want, "dequantized values")
 
 
+@pytest.mark.parametrize("flat", [False, True])
+@pytest.mark.parametrize("shape", [(5, 44), (64, 1024)])
+def test_int4_unpack_dequant_per_element_scales(oracle, shape, flat):
+    # group_size <= 0 means one scale per weight, given in the weight's shape or flattened
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+
+    g = torch.Generator().manual_seed(33)
+    m, k = shape
+    packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
+    scale = torch.exp(torch.randn((m, k), generator=g) * 3).to(torch.bfloat16)
+    if flat:
+        scale = scale.reshape(-1)
+    got = _dequantize_tensor(packed.to(DEV), scale.to(DEV), shape, 0)
+    _assert_same(got, oracle.int4_unpack_dequant(packed, scale, shape, 0), "per-element scales")
+    with pytest.raises(ValueError, match="incompatible"):
+        _dequantize_tensor(packed.to(DEV), scale.to(DEV)[..., :-1], shape, -1)
+
+
 def test_int4_pack_then_unpack_round_trip(oracle):
     from miles_amd.kernels.quant.int4_fake import pack_layer
     from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
@@ -900,6 +918,48 @@ def test_fp8_power_of_two_scales(oracle, shape, kind):
         y2_o, s2_o = oracle.per_block_cast_to_fp8(xf)
         _assert_same(s2, s2_o, "scales (fp32, strided)")
         _assert_same(y2, y2_o, "codes (fp32, strided)")
+
+
+@pytest.mark.parametrize("shape,mn", [((1, 1), 1), ((2, 5), 200), ((3, 4), 384), ((3, 2, 7), 130), ((1, 3, 8), 128),
+                                      ((2, 4), 250), ((76, 20), 9728), ((4, 3), 300)])
+def test_transform_scale_ue8m0(oracle, shape, mn):
+    from miles_amd.kernels.quant.fp8_blockwise import transform_scale_ue8m0
+
+    g = torch.Generator().manual_seed(43)
+    sf = torch.exp2(torch.randint(-40, 20, shape, generator=g).float())
+    got, want = transform_scale_ue8m0(sf.to(DEV), mn), oracle.transform_scale_ue8m0(sf, mn)
+    assert got.dtype == torch.int32 and got.shape == want.shape and got.stride() == want.stride()
+    assert torch.equal(got.cpu(), want)
+    # the padding rows of the storage are written too (zeros), as in the published construction
+    amn, kw = -(-mn // 4) * 4, got.shape[-1]
+    batch = got.shape[0] if got.dim() == 3 else 1
+    whole = torch.as_strided(got, (batch, amn, kw), (kw * amn, 1, amn), got.storage_offset())
+    assert torch.all(whole[:, mn:, :] == 0)
+    with pytest.raises(IndexError):
+        transform_scale_ue8m0(sf.to(DEV), 128 * shape[-2] + 1)
+    # the contiguous form of the same words (what a flattened payload holds)
+    from miles_amd import _lib
+    sfd = sf.to(DEV).reshape(batch, shape[-2], shape[-1])
+    dense = torch.full((batch, mn, kw), -1, dtype=torch.int32, device=DEV)
+    _lib.check(_lib.load().mq_ue8m0_pack_scales(sfd.data_ptr(), dense.data_ptr(), batch, mn, shape[-1], shape[-2], 1,
+                                                _lib.stream_ptr(dense.device)))
+    assert torch.equal(dense.cpu().reshape(want.shape), want.contiguous())
+
+
+@pytest.mark.parametrize("shape", [(256, 384), (130, 257), (3, 256, 128), (2, 2, 128, 256)])
+def test_quant_weight_ue8m0(oracle, shape):
+    from miles_amd.kernels.quant.fp8_blockwise import quant_weight_ue8m0
+
+    x = W.reference_pattern("random", (int(torch.tensor(shape[:-1]).prod()), shape[-1]), spread=512.0, amplitude=16.0)
+    y, s = quant_weight_ue8m0(x.view(shape).to(DEV), [128, 128])
+    y_o, s_o = oracle.per_block_cast_to_fp8(x)
+    assert y.shape == shape and s.shape == (*shape[:-2], -(-shape[-2] // 128), -(-shape[-1] // 128))
+    _assert_same(y.view(-1, shape[-1]), y_o, "codes")
+    _assert_same(s.reshape(s_o.shape), s_o, "scales")
+    with pytest.raises(AssertionError):
+        quant_weight_ue8m0(x.to(DEV), [128, 64])
+    with pytest.raises(AssertionError):
+        quant_weight_ue8m0(x.float().to(DEV), [128, 128])
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -485,7 +485,10 @@ def torch_int4_dequantize_tensor(weight_packed, weight_scale, shape, group_size)
     for i in range(8):
         unpacked[:, i::8] = (weight_packed >> (4 * i)) & 0xF
     weight = (unpacked[:, :k] - 8).to(torch.int8)
-    scales = torch.repeat_interleave(weight_scale.to(torch.float32), repeats=group_size, dim=1)
+    if group_size > 0:
+        scales = torch.repeat_interleave(weight_scale.to(torch.float32), repeats=group_size, dim=1)
+    else:
+        scales = weight_scale.to(torch.float32).reshape_as(weight)
     return (weight.to(torch.float32) * scales).to(torch.bfloat16).contiguous()
 
 
@@ -498,6 +501,20 @@ def test_int4_unpack_dequant_matches_torch_chain(oracle, shape, G, sdt):
     scale = torch.exp(torch.randn((m, k // G), generator=g) * 3).to(sdt)
     got = oracle.int4_unpack_dequant(packed, scale, shape, G)
     want = torch_int4_dequantize_tensor(packed, scale, shape, G)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("flat", [False, True])
+def test_int4_unpack_dequant_per_element_scales(oracle, flat):
+    # group_size <= 0: the scale tensor has one entry per weight, in the weight's shape or flattened (:75-82)
+    g = torch.Generator().manual_seed(32)
+    m, k = 5, 44
+    packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
+    scale = torch.exp(torch.randn((m, k), generator=g) * 3).to(torch.bfloat16)
+    if flat:
+        scale = scale.reshape(-1)
+    got = oracle.int4_unpack_dequant(packed, scale, (m, k), 0)
+    want = torch_int4_dequantize_tensor(packed, scale, (m, k), 0)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
@@ -720,3 +737,41 @@ def test_act_quant_known_answers(oracle):
     y, s = oracle.act_quant(torch.zeros(1, 64), 64, "ue8m0")
     assert s.item() == 2.0 ** -22 and torch.all(y.view(torch.uint8) == 0)
     assert oracle.act_quant(torch.zeros(1, 64), 64)[1].item() == pytest.approx(1e-4 / 448, rel=1e-6)
+
+
+def torch_transform_scale_ue8m0(sf, mn):
+    """SGLang's transform_scale_ue8m0 as published: broadcast tile rows to weight rows, then DeepGEMM's torch form of
+    get_mn_major_tma_aligned_packed_ue8m0_tensor (exponent bytes, pad, reinterpret 4 bytes as int32, transpose)."""
+    sf = sf.index_select(-2, torch.arange(mn) // 128)
+    exps = (sf.view(torch.int32) >> 23).to(torch.uint8)
+    squeeze = sf.dim() == 2
+    if squeeze:
+        exps = exps.unsqueeze(0)
+    b, _, k = exps.shape
+    amn, ak = -(-mn // 4) * 4, -(-k // 4) * 4
+    padded = torch.zeros((b, amn, ak), dtype=torch.uint8)
+    padded[:, :mn, :k] = exps
+    words = padded.view(-1).view(torch.int32).view(b, amn, ak // 4)
+    transposed = torch.zeros((b, ak // 4, amn), dtype=torch.int32).mT
+    transposed[:, :, :] = words
+    out = transposed[:, :mn, :]
+    return out.squeeze(0) if squeeze else out
+
+
+@pytest.mark.parametrize("shape,mn", [((1, 1), 1), ((2, 5), 200), ((3, 4), 384), ((3, 2, 7), 130), ((1, 3, 8), 128),
+                                      ((2, 4), 250)])
+def test_transform_scale_ue8m0_matches_torch_chain(oracle, shape, mn):
+    g = torch.Generator().manual_seed(41)
+    sf = torch.exp2(torch.randint(-40, 20, shape, generator=g).float())
+    got, want = oracle.transform_scale_ue8m0(sf, mn), torch_transform_scale_ue8m0(sf, mn)
+    assert got.shape == want.shape and got.stride() == want.stride() and got.dtype == torch.int32
+    assert torch.equal(got, want)
+
+
+def test_transform_scale_ue8m0_known_answer(oracle):
+    # 2^e has exponent byte e + 127; five scales along k fill one word and the lowest byte of the next
+    sf = torch.tensor([[1.0, 2.0, 0.5, 4.0, 2.0 ** -126]])
+    out = oracle.transform_scale_ue8m0(sf, 3)
+    assert out.shape == (3, 2) and out.stride() == (1, 4)
+    assert [v & 0xFFFFFFFF for v in out[:, 0].tolist()] == [127 | 128 << 8 | 126 << 16 | 129 << 24] * 3
+    assert out[:, 1].tolist() == [1] * 3
