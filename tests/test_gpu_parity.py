@@ -819,6 +819,23 @@ def test_nvfp4_qdq_ste_and_argument_checks(monkeypatch):
         m.current_nvfp4_qdq_config()
 
 
+def test_nvfp4_fake_qat_switch_on_grouped_weights(oracle, monkeypatch):
+    # miles/utils/nvfp4_fake_qat.py:10-23: one configuration for the whole list, every weight through the fused q-dq
+    from miles_amd.utils import nvfp4_fake_qat as qat
+
+    for name in ("NVTE_USE_FAST_MATH", "NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256"):
+        monkeypatch.delenv(name, raising=False)
+    cpu = [W.gaussian_outliers((64, 256), std=0.02, p_outlier=0.001, gain=20.0, seed=970 + i) for i in range(3)]
+    weights = [torch.nn.Parameter(w.to(DEV)) for w in cpu]
+    monkeypatch.setenv(qat.NVFP4_FAKE_QAT_FLAG, "1")
+    out = qat.maybe_fake_quantize_nvfp4_weight_tensors(weights)
+    assert len(out) == 3 and all(o.requires_grad for o in out)
+    for o, w in zip(out, cpu):
+        _assert_same(o.detach(), oracle.fused_nvfp4_qdq(w), "fake-quantized weight")
+    sum(o.float().sum() for o in out).backward()
+    assert all(torch.equal(w.grad, torch.ones_like(w)) for w in weights)
+
+
 # ---------------------------------------------------------------------------------------------------
 # NVFP4 Four Over Six block scaling (NVTE_NVFP4_4OVER6; miles/kernels/quant/nvfp4_qdq.py:893-990)
 _FOS_CASES = [(448, "MAE", False), (256, "MAE", False), (256, "MSE", False), (256, "MAE", True), (448, "MSE", True)]

@@ -397,3 +397,32 @@ def test_sync_plan_tops_up_small_trailing_launches_only():
     marks = plan_with(pairs, [9, 300]).submission_marks()
     assert marks[0] >= 64 and pairs[marks[0]][5] != pairs[marks[0] - 1][5]
     assert marks == [65, 300]      # index 64 is the second job of a pair: the cut moves to 65
+
+
+# ---------------------------------------------------------------------------------------------------
+# NVFP4 fake-QAT switch (miles/utils/nvfp4_fake_qat.py; the reference's TestNVFP4FakeQATAdapter)
+def test_nvfp4_fake_qat_switch_off_returns_the_same_list(monkeypatch):
+    from miles_amd.utils import nvfp4_fake_qat as qat
+
+    weights = [torch.nn.Parameter(torch.empty(4, 16))]
+    for value in ("0", "true", ""):
+        monkeypatch.setenv(qat.NVFP4_FAKE_QAT_FLAG, value)
+        assert qat.maybe_fake_quantize_nvfp4_weight_tensors(weights) is weights
+    monkeypatch.delenv(qat.NVFP4_FAKE_QAT_FLAG)
+    assert qat.maybe_fake_quantize_nvfp4_weight_tensors(weights) is weights
+
+
+def test_nvfp4_fake_qat_switch_on_reads_the_configuration_once(monkeypatch):
+    from miles_amd.kernels.quant import nvfp4_qdq
+    from miles_amd.utils import nvfp4_fake_qat as qat
+
+    weights = [torch.nn.Parameter(torch.empty(4, 16)) for _ in range(3)]
+    images = [torch.empty_like(w) for w in weights]
+    config, seen, reads = object(), [], []
+    monkeypatch.setattr(nvfp4_qdq, "current_nvfp4_qdq_config", lambda: reads.append(1) or config)
+    monkeypatch.setattr(nvfp4_qdq, "fake_nvfp4_quantization_ste", lambda w, c: seen.append((w, c)) or images[len(seen) - 1])
+    monkeypatch.setenv(qat.NVFP4_FAKE_QAT_FLAG, "1")
+    out = qat.maybe_fake_quantize_nvfp4_weight_tensors(weights)
+    assert len(reads) == 1 and len(out) == 3
+    assert all(o is i for o, i in zip(out, images))
+    assert all(w is got_w and c is config for w, (got_w, c) in zip(weights, seen))
