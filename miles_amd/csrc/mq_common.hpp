@@ -112,6 +112,10 @@ __device__ __forceinline__ uint32_t sw_e4m3fn(float x) {
     uint32_t code = (a >> 20) - (120u << 3);
     return sign | (code > 0x7Fu ? 0x7Fu : code);
 }
+// clamp that leaves NaN alone, like torch.clamp (v_med3_f32 alone would return the lower bound for a NaN)
+__device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
+    return v != v ? v : __builtin_amdgcn_fmed3f(v, lo, hi);
+}
 // saturating form: |x| >= 448 and inf -> 0x7E | sign, NaN -> 0x7F
 __device__ __forceinline__ uint32_t sw_e4m3fn_sat(float x) {
     uint32_t u = f2u(x), a = u & 0x7FFFFFFFu;

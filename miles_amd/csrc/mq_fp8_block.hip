@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
             else {
                 const float x = load_f32(w, r * sxm + c * sxn, dtype);
                 float v = MODE != 0 ? x * y : x / s;
-                v = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+                v = clamp_keep_nan(v, -kFp8Max, kFp8Max);
                 code = sw_e4m3fn(v);
             }
             q[r * ldq + c] = (uint8_t)code;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restri
     for (int64_t c = t; c < K; c += 256) {
         float v = load_f32(w, r * ldw + c, dtype) / s;
         if (!per_channel) v = round_to_dtype(v, dtype);
-        v = __builtin_amdgcn_fmed3f(v, -kFp8Max, kFp8Max);
+        v = clamp_keep_nan(v, -kFp8Max, kFp8Max);
         q[r * K + c] = (uint8_t)sw_e4m3fn(v);
     }
 }
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* _
         } else {                                  // inf / NaN in the row: clamp and convert in software
             uint32_t c[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(__builtin_amdgcn_fmed3f(f[j], -kFp8Max, kFp8Max));
+            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(clamp_keep_nan(f[j], -kFp8Max, kFp8Max));
             o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
             o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
         }
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256) void fp8_tensor_quant_bf16_kernel(const uint16
         } else {
             uint32_t c[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(__builtin_amdgcn_fmed3f(f[j], -kFp8Max, kFp8Max));
+            for (int j = 0; j < 8; j++) c[j] = sw_e4m3fn(clamp_keep_nan(f[j], -kFp8Max, kFp8Max));
             o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
             o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
         }

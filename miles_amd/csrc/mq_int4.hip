@@ -11,7 +11,8 @@
 //                           code = rintf(x/scale_f32) + 8 in [1,15]; eight codes per int32, element 8j+i in bits
 //                           4i..4i+3; scale stored as bf16.  The bf16 round trip that pack_layer performs
 //                           (w = q*scale_b, q' = round(w/scale_b)) returns q for every |q| <= 7 and every scale
-//                           below 4.8e37, so the codes come straight from the fp32 quotient.
+//                           below 4.8e37, so the codes come straight from the fp32 quotient; groups with a larger
+//                           scale or a non-finite element run the round trip as written.
 //
 // Packed fast path (bf16, G = 8 * LANES): LANES lanes own one group, 16 bytes each; the group amax is a DPP
 // max over the LANES-lane segment; x/scale uses the shared-divisor sequence (3 FMA-class ops per element,
@@ -43,6 +44,40 @@ __device__ __forceinline__ uint32_t seg_max(uint32_t v) {
 // nibble = (rint(q) + 8) & 15 taken from the low bits of q + (1.5*2^23 + 8)
 __device__ __forceinline__ uint32_t code_bits(float q) { return f2u(q + 12582920.0f); }
 
+// The fused form of the packed kernel relies on the round trip q -> bf16(q * scale_b) -> bf16(. / scale_b) being the
+// identity.  It is for every group maximum below the largest finite bf16 (all maxima x all codes checked on the CPU);
+// at that maximum 7 * scale_b overflows, and an infinity or a NaN breaks it too.  This function runs the chain as
+// written for one unit: NaN skipped by the group maximum as the reference's fmaxf reduction does, codes above 15
+// carrying into the next nibble as in its int32 sum.
+template <int LANES>
+__device__ __forceinline__ void int4_pack_chain_unit(const u32x4 v, const int64_t unit, const bool live,
+                                                               const int t, uint32_t* __restrict__ packed,
+                                                               uint16_t* __restrict__ scale) {
+    const float f[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t a = f2u(f[j]) & 0x7FFFFFFFu;
+        m = umax(m, a > 0x7F800000u ? 0u : a);
+    }
+    const float s = __builtin_fmaxf(u2f(seg_max<LANES>(m)) * kSymCons, 1e-5f);
+    const float sb = u2f(sw_bf16(s) << 16);
+    uint32_t word = 0;
+#pragma unroll 1
+    for (int j = 0; j < 8; j++) {
+        const uint32_t pair = j < 2 ? v.x : j < 4 ? v.y : j < 6 ? v.z : v.w;
+        const float x = (j & 1) ? bf16_hi(pair) : bf16_lo(pair);
+        const float q0 = u2f(sw_bf16(__builtin_rintf(x / s)) << 16);
+        const float wv = u2f(sw_bf16(q0 * sb) << 16);
+        const float rv = clamp_keep_nan(u2f(sw_bf16(wv / sb) << 16), -128.0f, 127.0f);
+        word += (uint32_t)(((int)__builtin_rintf(rv) + 8) & 0xFF) << (4 * j);
+    }
+    if (live) {
+        st4(packed + unit, word);
+        if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
+    }
+}
+
 template <int LANES>
 __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTable tab) {
     const FlatJob& job = tab.job[blockIdx.y];
@@ -59,11 +94,13 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTa
         const int64_t unit = base + i * kI4Threads + t;
         v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
     }
+    uint32_t top = 0;
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
         const int64_t unit = base + i * kI4Threads + t;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = seg_max<LANES>(hmax_u16(m2));
+        top = umax(top, mb);
         const float amax = u2f(mb << 16);
         const float s = __builtin_fmaxf(amax * kSymCons, 1e-5f);
         const float y = 1.0f / s;
@@ -80,6 +117,15 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTa
             st4(packed + unit, word);
             if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
         }
+    }
+    // A group holding the largest finite bf16, an infinity or a NaN is outside the fused form: a wavefront that met one
+    // writes all of its groups again through the written-out chain (a scalar branch after the common path, which
+    // therefore stays one straight instruction stream; the later store of a lane to the same address wins).
+    if (__builtin_amdgcn_ballot_w64(top >= 0x7F7Fu) == 0) return;
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads + t;
+        int4_pack_chain_unit<LANES>(v[i], unit, unit < total_units, t, packed, scale);
     }
 }
 
@@ -151,8 +197,8 @@ __global__ __launch_bounds__(256) void int4_pack_generic_kernel(const void* __re
             const float sb = round_to_dtype(s, dtype);
             const float wv = round_to_dtype(q0 * sb, dtype);
             float rv = round_to_dtype(wv / sb, dtype);
-            rv = __builtin_fminf(__builtin_fmaxf(rv, -128.0f), 127.0f);
-            const int qi = (int)__builtin_rintf(rv);
+            rv = clamp_keep_nan(rv, -128.0f, 127.0f);
+            const int qi = (int)__builtin_rintf(rv);                     // NaN converts to 0
             word += (uint32_t)((qi + 8) & 0xFF) << (4 * k);
             if (c == g0) store_dtype(scale_out, r * gpr + c / G, s, dtype);
         }
@@ -242,9 +288,10 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restr
                 const float q = fast ? div_by_shared(f[i], s, ys) : f[i] / s;
                 const float w1 = round_to_dtype(__builtin_rintf(q) + z, DT);
                 const float w2 = round_to_dtype(round_to_dtype(w1 - z, DT) * sb, DT);
-                const float d = fast ? div_by_shared(w2, sb, yb) : w2 / sb;
+                // w1 * sb may have overflowed the dtype: the sequence needs a finite numerator
+                const float d = (fast && __builtin_fabsf(w2) < __builtin_inff()) ? div_by_shared(w2, sb, yb) : w2 / sb;
                 float r = round_to_dtype(round_to_dtype(d, DT) + z, DT);
-                r = __builtin_fminf(__builtin_fmaxf(r, 0.0f), 255.0f);
+                r = clamp_keep_nan(r, 0.0f, 255.0f);
                 word += (uint32_t)__builtin_rintf(r) << (4 * i);
             }
             packed[word0 + k] = word;
@@ -280,6 +327,8 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
     float mx = f[0], mn = f[0];
 #pragma unroll
     for (int i = 1; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
+    mx = mx != mx ? -__builtin_inff() : mx;         // eight NaNs in one lane: the group reduction skips them
+    mn = mn != mn ? __builtin_inff() : mn;
     mx = order_unkey(seg_max<LANES>(order_key(mx)));
     mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
     const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
@@ -331,7 +380,7 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
         for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            word += (uint32_t)__builtin_rintf(__builtin_fminf(__builtin_fmaxf(q[i], 0.0f), 255.0f)) << (4 * i);
+            word += (uint32_t)__builtin_rintf(clamp_keep_nan(q[i], 0.0f, 255.0f)) << (4 * i);
     }
     if (live) {
         st4(packed + unit, word);
@@ -401,12 +450,15 @@ __global__ __launch_bounds__(kI4Threads) void int4_fake_rows_kernel(const void* 
         mx = __builtin_fabsf(f[0]);
 #pragma unroll
         for (int i = 1; i < 8; i++) mx = __builtin_fmaxf(mx, __builtin_fabsf(f[i]));
+        mx = mx != mx ? 0.0f : mx;             // eight NaNs in one lane: fmaxf over the group skips them
         mx = u2f(seg_max<LANES>(f2u(mx)));     // non-negative floats order like their bit patterns
         s = __builtin_fmaxf(mx * kSymCons, 1e-5f);
     } else {
         mx = mn = f[0];
 #pragma unroll
         for (int i = 1; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
+        mx = mx != mx ? -__builtin_inff() : mx;     // eight NaNs in one lane: the group reduction skips them
+        mn = mn != mn ? __builtin_inff() : mn;
         mx = order_unkey(seg_max<LANES>(order_key(mx)));
         mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
         s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);

@@ -236,3 +236,126 @@ def test_random_job_lists_in_one_submission(oracle, seed):
             got, want = [t for half in got for t in half], [t for half in want for t in half]
         for j, (g_, w_) in enumerate(zip(got, want)):
             _same(g_, w_, f"job {i} ({kind} {shape}) output {j}")
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# non-finite and extreme values scattered over random data: NaN of both signs, infinities, signed zeros, the largest and
+# the smallest magnitudes of the dtype, whole rows of zeros / NaN / one infinity
+def _special_tensor(seed, shape, dtype, non_finite):
+    g = torch.Generator().manual_seed(seed)
+    rows, cols = shape
+    x = (torch.randn(shape, generator=g) * torch.exp2(torch.randint(-6, 6, shape, generator=g).float())).to(dtype)
+    fi = torch.finfo(dtype)
+    pool = torch.tensor([0.0, -0.0, fi.max, -fi.max, fi.tiny, -fi.tiny, fi.smallest_normal * 0.5, 448.0, 464.0, 480.0, 6.0, 5.0,
+                         1e-10, 7.0], dtype=torch.float32).to(dtype)
+    hits = torch.rand(shape, generator=g) < 0.01
+    picks = pool[torch.randint(0, pool.numel(), shape, generator=g)]
+    x = torch.where(hits, picks, x)
+    x[1 % rows] = 0.0
+    x[3 % rows, : cols // 2] = 0.0
+    x[5 % rows] = -0.0
+    x[6 % rows, cols // 2:] = fi.max
+    if non_finite:      # a few poisoned places only, so that most tiles / rows / blocks stay finite
+        x[2 % rows] = float("nan")
+        x[4 % rows, cols // 3] = float("inf")
+        x[7 % rows, 5] = -float("inf")
+        x[7 % rows, cols - 3] = float("nan")
+        bits = x.view(torch.int16 if dtype != torch.float32 else torch.int32)
+        bits[7 % rows, cols - 3] |= (-0x8000 if dtype != torch.float32 else -0x80000000)        # a NaN with the sign bit set
+        x[(rows - 1), 17 % cols] = float("nan")
+        x[(rows - 1), 18 % cols] = float("inf")
+    return x
+
+
+def _same_float(got, want, what):
+    """Bit equality except that any NaN matches any NaN, for outputs held in a floating-point type of two bytes or more."""
+    g, w = got.detach().cpu().contiguous(), want.detach().cpu().contiguous()
+    assert g.shape == w.shape and g.dtype == w.dtype, f"{what}: {tuple(g.shape)} {g.dtype} vs {tuple(w.shape)} {w.dtype}"
+    gn, wn = torch.isnan(g.float()), torch.isnan(w.float())
+    assert torch.equal(gn, wn), f"{what}: NaN in different places ({int(gn.sum())} vs {int(wn.sum())})"
+    _same(torch.where(gn, torch.zeros((), dtype=g.dtype), g), torch.where(wn, torch.zeros((), dtype=w.dtype), w), what)
+
+
+def _same_any(got, want, what):
+    if got.is_floating_point() and got.element_size() >= 2:
+        _same_float(got, want, what)
+    elif got.dtype == F8:       # the two NaN codes 0x7F / 0xFF count as one: which sign a NaN carries is the host FPU's choice
+        g, w = _bits(got).clone(), _bits(want).clone()
+        g[(g & 0x7F) == 0x7F] = 0x7F
+        w[(w & 0x7F) == 0x7F] = 0x7F
+        _same(g, w, what)
+    else:
+        _same(got, want, what)
+
+
+@pytest.mark.parametrize("non_finite", [False, True], ids=["finite", "nonfinite"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
+@pytest.mark.parametrize("seed", range(4))
+def test_random_special_values(oracle, monkeypatch, seed, dtype, non_finite):
+    from miles_amd.kernels.quant import fake_quant as fq
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda, pack_layer
+    from miles_amd.kernels.quant.nvfp4_qdq import NVFP4QDQConfig, compute_nvfp4_amax, fused_nvfp4_qdq
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    for name in ("NVTE_USE_FAST_MATH", "NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256"):
+        monkeypatch.delenv(name, raising=False)
+    shape = [(136, 384), (64, 1024), (8, 256), (200, 128)][seed]
+    x = _special_tensor(7000 + seed, shape, dtype, non_finite)
+    xd = x.to(DEV)
+    failures = []
+
+    def check(what, got, want):
+        got, want = (got, want) if isinstance(got, (tuple, list)) else ((got,), (want,))
+        for i, (g_, w_) in enumerate(zip(got, want)):
+            if g_ is None and w_ is None:
+                continue
+            try:
+                _same_any(g_, w_, f"{what}[{i}]")
+            except AssertionError as e:
+                failures.append(str(e))
+
+    # Functions whose reference is a chain of torch floating-point ops, or CUDA code whose fmaxf / fminf reductions skip
+    # NaN by definition, have a defined result for non-finite input and are held to it.  The rest of the list runs on
+    # finite data only: there the reference's result for a NaN or an infinity hangs on a float -> integer conversion of
+    # NaN (undefined in torch), on which NaN rule its Triton / TileLang compiler picks for max and clamp, or on a
+    # third-party kernel outside the reference tree.
+    check("block_fp8", block_fp8(xd, [128, 128]), oracle.block_fp8(x, (128, 128)))
+    check("tensor_fp8", quant_fp8(xd, "tensor"), oracle.tensor_fp8(x))
+    check("channel_fp8", quant_fp8(xd, "channel"), oracle.channel_fp8(x))
+    for sym in (True, False):
+        got = fake_int4_quant_cuda(xd, (1, 128), sym)
+        want = oracle.fake_int4_quant(x, (1, 128), sym)
+        check(f"fake_int4 sym={sym}", got[: 2 if sym else 3], want[: 2 if sym else 3])
+    if dtype == torch.bfloat16:
+        q_o, s_o = oracle.block_fp8(x, (128, 128))
+        check("weight_dequant", weight_dequant(q_o.to(DEV), s_o.to(DEV)), oracle.weight_dequant(q_o, s_o))
+    if non_finite:
+        assert not failures, "\n".join(failures)
+        return
+    check("fp8_blockwise_cast", fp8_blockwise_cast(xd), oracle.fp8_blockwise_cast(x))
+    check("mxfp8", mxfp8_quantize(xd), oracle.mxfp8_quantize(x))
+    p, s4 = quantize_mxfp4(xd, 32)
+    p_o, s4_o = oracle.quantize_mxfp4(x, 32)
+    check("mxfp4", (p, s4), (p_o, s4_o))
+    check("mxfp4 dequant", dequantize_mxfp4(p_o.to(DEV), s4_o.to(DEV), 32), oracle.dequantize_mxfp4(p_o, s4_o, 32))
+    check("nvfp4", nvfp4_quantize_1d(xd), oracle.nvfp4_quantize_1d(x))
+    for kind, fn in (("fp8", fq.fake_quant_fp8_forward), ("fp4", fq.fake_quant_fp4_forward),
+                     ("compressed_kv", fq.fake_quant_compressed_kv_forward)):
+        check(f"fake_quant {kind}", fn(xd), oracle.fake_quant(x, kind))
+    for fmt in (None, "ue8m0"):
+        check(f"act_quant {fmt}", act_quant(xd, 128, fmt), oracle.act_quant(x, 128, fmt))
+    check("fp8_simulate", fp8_simulate(xd, 128), oracle.fp8_simulate(x, 128))
+    if dtype != torch.float32:
+        check("pack_layer", pack_layer(xd, 128)[:2], oracle.pack_layer(x, 128)[:2])
+        check("pack_layer asym", pack_layer(xd, 128, sym=False), oracle.pack_layer(x, 128, sym=False))
+        check("nvfp4 qdq", fused_nvfp4_qdq(xd, compute_nvfp4_amax(xd), NVFP4QDQConfig()), oracle.fused_nvfp4_qdq(x))
+    if dtype == torch.bfloat16:
+        q_o, s_o = oracle.per_block_cast_to_fp8(x)
+        check("per_block_cast_to_fp8", per_block_cast_to_fp8(xd), (q_o, s_o))
+    assert not failures, "\n".join(failures)
