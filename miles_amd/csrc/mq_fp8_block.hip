@@ -78,6 +78,53 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
     m = 0;
 #pragma unroll
     for (int k = 0; k < kTileWaves; k++) m = umax(m, wave_amax[k]);
+    if (MODE != 0 && m >= 0x7F80u) {
+        // An infinity or a NaN in the tile (rare, and uniform over the workgroup).  Mode 1: Triton's max, maximum and
+        // clamp return the operand that is not NaN, so the tile maximum skips NaN and a NaN product clamps to -448.
+        // Mode 2: torch's amax hands a NaN on, 2^ceil(log2(.)) of inf / NaN is inf / NaN, and nothing clamps.
+        float sx;
+        if (MODE == 1) {
+            uint32_t mf = 0;
+#pragma unroll
+            for (int i = 0; i < kRowsPerThread; i++) {
+                const uint32_t u[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t lo = u[k] & 0x7FFFu, hi = (u[k] >> 16) & 0x7FFFu;
+                    mf = umax(mf, umax(lo > 0x7F80u ? 0u : lo, hi > 0x7F80u ? 0u : hi));
+                }
+            }
+            mf = wave_max(mf);
+            __syncthreads();                    // every wavefront has read the first set of maxima
+            if ((t & (kWave - 1)) == 0) wave_amax[t >> 6] = mf;
+            __syncthreads();
+            mf = 0;
+#pragma unroll
+            for (int k = 0; k < kTileWaves; k++) mf = umax(mf, wave_amax[k]);
+            const float finite_max = u2f(mf << 16);
+            sx = (finite_max > 1e-10f ? finite_max : 1e-10f) / kFp8Max;
+        } else {
+            sx = u2f(m > 0x7F80u ? 0x7FC00000u : 0x7F800000u);
+        }
+        const float yx = 1.0f / sx;
+        if (t == 0) job.scale[tile] = sx;
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; i++) {
+            const int64_t r = row0 + kRowStep * i;
+            const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                                bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float p = f[j] * yx;
+                if (MODE == 1) p = __builtin_fminf(__builtin_fmaxf(p, -kFp8Max), kFp8Max);
+                c[j] = sw_e4m3fn(p);
+            }
+            if (col_ok && r < M)
+                st8(q + r * K + col, u32x2{c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24)});
+        }
+        return;
+    }
     const float amax = u2f(m << 16);
 
     float s;
@@ -140,7 +187,10 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
     uint32_t m = 0;
     for (int idx = t; idx < n; idx += kGenThreads) {
         const int64_t r = r0 + idx / bk, c = c0 + idx % bk;
-        if (r < M && c < K) m = umax(m, f2u(load_f32(w, r * sxm + c * sxn, dtype)) & 0x7FFFFFFFu);
+        if (r < M && c < K) {
+            const uint32_t a = f2u(load_f32(w, r * sxm + c * sxn, dtype)) & 0x7FFFFFFFu;
+            m = umax(m, (MODE == 1 && a > 0x7F800000u) ? 0u : a);      // Triton's max skips NaN, torch's amax hands it on
+        }
     }
     m = wave_max(m);
     if ((t & (kWave - 1)) == 0) wave_amax[t >> 6] = m;
@@ -156,7 +206,7 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
         s = absmax / kFp8Max;
         y = 1.0f / s;
     } else {
-        s = ceil_pow2_scale((amax > 1e-4f ? amax : 1e-4f) / kFp8Max);
+        s = m >= 0x7F800000u ? amax : ceil_pow2_scale((amax > 1e-4f ? amax : 1e-4f) / kFp8Max);   // inf / NaN stay
         y = 1.0f / s;
     }
     if (t == 0) scale[tile] = s;
@@ -169,7 +219,8 @@ __global__ __launch_bounds__(kGenThreads) void fp8_block_generic_kernel(const vo
             else {
                 const float x = load_f32(w, r * sxm + c * sxn, dtype);
                 float v = MODE != 0 ? x * y : x / s;
-                v = clamp_keep_nan(v, -kFp8Max, kFp8Max);
+                if (MODE == 0) v = clamp_keep_nan(v, -kFp8Max, kFp8Max);                              // torch.clamp
+                else if (MODE == 1) v = __builtin_fminf(__builtin_fmaxf(v, -kFp8Max), kFp8Max);        // tl.clamp: NaN -> -448
                 code = sw_e4m3fn(v);
             }
             q[r * ldq + c] = (uint8_t)code;

@@ -270,7 +270,10 @@ void mqo_fp8_per_tensor_or_channel(const void* w, int dtype, int64_t M, int64_t 
 /*   absmax = max( max|f32(x)| over tile , 1e-10f )      (:51)
  *   x_s    = absmax / 448   ; s_inv = 1 / x_s           (:52-53) IEEE division
  *   y      = e4m3( clamp(f32(x) * s_inv, -448, 448) )   (:54)
- * strides in elements for x; y contiguous; S contiguous. */
+ * strides in elements for x; y contiguous; S contiguous.
+ * NaN: tl.max, tl.maximum and tl.clamp are called without propagate_nan, i.e. they lower to the maxnum / minnum
+ * operations that return the operand which is not NaN: the tile maximum skips NaN elements and a NaN product leaves
+ * the clamp as max(NaN, -448) = -448. */
 void mqo_fp8_blockwise_cast(const void* x, int dtype, int64_t M, int64_t N,
                             int64_t sxm, int64_t sxn, int bm, int bn,
                             uint8_t* y, float* S) {
@@ -293,8 +296,7 @@ void mqo_fp8_blockwise_cast(const void* x, int dtype, int64_t M, int64_t N,
             for (int64_t r = r0; r < r1; r++)
                 for (int64_t c = c0; c < c1; c++) {
                     float v = load_as_f32(x, r * sxm + c * sxn, dtype) * s_inv;
-                    if (v < -448.0f) v = -448.0f;
-                    if (v > 448.0f) v = 448.0f;
+                    v = fminf(fmaxf(v, -448.0f), 448.0f);
                     y[r * N + c] = mqo_f32_to_e4m3fn(v);
                 }
         }
@@ -317,7 +319,10 @@ void mqo_fp8_block_pow2(const void* x, int dtype, int64_t M, int64_t N, int64_t 
             int64_t c0 = tj * 128, c1 = c0 + 128 < N ? c0 + 128 : N;
             float amax = 0.0f;
             for (int64_t r = r0; r < r1; r++)
-                for (int64_t c = c0; c < c1; c++) amax = fmaxf(amax, fabsf(load_as_f32(x, r * ld + c, dtype)));
+                for (int64_t c = c0; c < c1; c++) {
+                    float a = fabsf(load_as_f32(x, r * ld + c, dtype));
+                    if (a > amax || a != a) amax = a;                  /* torch's amax hands a NaN on */
+                }
             if (amax < 1e-4f) amax = 1e-4f;
             float sf = powf(2.0f, ceilf(log2f(amax / 448.0f)));
             float inv = 1.0f / sf;
