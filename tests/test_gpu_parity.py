@@ -1099,3 +1099,46 @@ def test_fake_int4_quant_full_size_tensor(oracle):
         _assert_same(scale, scale_o, "scales")
         if not sym:
             _assert_same(zero, zero_o, "zero points")
+
+
+# ---------------------------------------------------------------------------------------------------
+# several host threads at once: the converters call the quantizers from a ThreadPoolExecutor
+# (tools/convert_hf_to_fp8.py:175-184, tools/convert_hf_to_int4_direct.py:220-236)
+def test_quantizers_from_concurrent_host_threads(oracle):
+    from concurrent.futures import ThreadPoolExecutor
+
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    cpu = [W.gaussian_outliers((128 + 8 * i, 256), std=0.02, p_outlier=0.001, gain=20.0, seed=900 + i) for i in range(8)]
+    dev = [w.to(DEV) for w in cpu]
+    torch.cuda.synchronize()
+
+    def work(i):
+        x = dev[i]
+        out = {}
+        for rep in range(10):
+            out["block"] = block_fp8(x, [128, 128])
+            out["tensor"] = quant_fp8(x, "tensor")
+            out["mxfp8"] = mxfp8_quantize(x)
+            out["nvfp4"] = nvfp4_quantize_1d(x)
+            with launch.deferred() as batch:       # batches are per thread: only this thread's two jobs land here
+                out["cast"] = fp8_blockwise_cast(x)
+                out["int4"] = pack_layer(x, 128)[:2]
+                assert len(batch) == 2
+        torch.cuda.synchronize()
+        return out
+
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        results = list(pool.map(work, range(8)))
+    for i, out in enumerate(results):
+        x = cpu[i]
+        want = {"block": oracle.block_fp8(x, (128, 128)), "tensor": oracle.tensor_fp8(x), "mxfp8": oracle.mxfp8_quantize(x),
+                "nvfp4": oracle.nvfp4_quantize_1d(x), "cast": oracle.fp8_blockwise_cast(x), "int4": oracle.pack_layer(x, 128)[:2]}
+        for name, got in out.items():
+            for j, (g_, w_) in enumerate(zip(got, want[name])):
+                _assert_same(g_, w_, f"thread {i} {name} output {j}")
