@@ -1142,3 +1142,47 @@ def test_quantizers_from_concurrent_host_threads(oracle):
         for name, got in out.items():
             for j, (g_, w_) in enumerate(zip(got, want[name])):
                 _assert_same(g_, w_, f"thread {i} {name} output {j}")
+
+
+# ---------------------------------------------------------------------------------------------------
+# more than 2^31 elements in one tensor: every offset computed by the kernels has to be 64-bit.  The tensor is one
+# [4096, 8192] block repeated down the rows, and every quantizer here works on row-local groups (tiles of 128 rows,
+# row segments), so each repetition must come out as the block alone does; NVFP4 shares one amax, equal by construction.
+def test_tensors_beyond_2_to_31_elements(oracle):
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    reps, block_rows, cols, tail = 64, 4096, 8192, 128
+    base_cpu = W.gaussian_outliers((block_rows, cols), std=0.02, p_outlier=0.001, gain=20.0, seed=31)
+    base = base_cpu.to(DEV)
+    rows = reps * block_rows + tail
+    assert rows * cols > 2**31
+    x = torch.empty((rows, cols), dtype=torch.bfloat16, device=DEV)
+    x[: reps * block_rows].view(reps, block_rows, cols).copy_(base.unsqueeze(0).expand(reps, -1, -1))
+    x[reps * block_rows:] = base[:tail]
+
+    def repeats(full, small, what):
+        full, small = full.view(torch.uint8) if full.element_size() == 1 else full, small.view(torch.uint8) if small.element_size() == 1 else small
+        per = small.shape[0]
+        body = full[: reps * per].view(reps, *small.shape)
+        assert bool((body == small.unsqueeze(0)).all()), f"{what}: a repetition differs from the block alone"
+        assert torch.equal(full[reps * per:], small[: full.shape[0] - reps * per]), f"{what}: tail differs"
+
+    for name, fn in (("fp8_blockwise_cast", fp8_blockwise_cast), ("block_fp8", lambda t: block_fp8(t, [128, 128])),
+                     ("mxfp8", mxfp8_quantize), ("int4", lambda t: pack_layer(t, 128)[:2]),
+                     ("mxfp4", lambda t: quantize_mxfp4(t, 32)), ("nvfp4", lambda t: nvfp4_quantize_1d(t)[:2])):
+        big, small = fn(x), fn(base)
+        for j, (b_, s_) in enumerate(zip(big, small)):
+            repeats(b_, s_, f"{name} output {j}")
+        if name == "fp8_blockwise_cast":
+            q_o, s_o = oracle.fp8_blockwise_cast(base_cpu)
+            _assert_same(small[0], q_o, "block codes")
+            _assert_same(small[1], s_o, "block scales")
+            repeats(weight_dequant(big[0], big[1]), weight_dequant(small[0], small[1]), "weight_dequant")
+        del big, small
+    torch.cuda.synchronize()
