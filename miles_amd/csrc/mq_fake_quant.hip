@@ -248,7 +248,7 @@ static void launch_fq(const void* x, int dtype, void* y, int64_t units, hipStrea
 }
 
 extern "C" int mq_fake_quant(const void* x, int dtype, void* y, int64_t numel, int mode, void* stream) {
-    if (!x || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!x || !y) && numel != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || mode < 0 || mode > 2) return mq_fail(MQ_ERR_ARG, "bad argument");
     const int block = mode == 2 ? 16 : 32;
     if (numel % block != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the block size");
@@ -288,7 +288,7 @@ static void launch_act_dt(const void* x, int dtype, void* y, void* scale, int64_
 
 extern "C" int mq_fp8_act_quant(const void* x, int dtype, void* y, void* scale, int64_t numel, int block, int flags,
                                 void* stream) {
-    if (!x || !y || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!x || !y || !scale) && numel != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || block <= 0 || (flags & ~7) != 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (numel % block != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the block size");
     if ((flags & MQ_ACT_SCALE_E8M0) && !(flags & MQ_ACT_ROUND_SCALE))

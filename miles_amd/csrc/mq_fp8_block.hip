@@ -513,7 +513,7 @@ int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
 
 static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int64_t sxn, void* q, float* scale,
                             int64_t M, int64_t K, int bm, int bk, hipStream_t stream) {
-    if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !q || !scale) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (M < 0 || K < 0 || bm <= 0 || bk <= 0) return mq_fail(MQ_ERR_ARG, "bad shape or block size");
     if (dtype < MQ_BF16 || dtype > MQ_F32) return mq_fail(MQ_ERR_ARG, "unsupported dtype");
     if (M == 0 || K == 0) return MQ_OK;
@@ -557,7 +557,8 @@ extern "C" int mq_fp8_block_quant_pow2(const void* w, int dtype, int64_t ldw, vo
 
 extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws,
                                    int64_t M, int64_t K, int per_channel, float floor_in_dtype, void* stream) {
-    if (!w || !q || !scale || !amax_ws) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !q) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!scale || !amax_ws) && (M != 0 || !per_channel)) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (M == 0 || K == 0) return MQ_OK;
     if (M > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many rows");
@@ -663,7 +664,7 @@ __global__ __launch_bounds__(256) void ue8m0_pack_scales_kernel(const float* __r
 
 extern "C" int mq_ue8m0_pack_scales(const float* sf, int32_t* out, int64_t batch, int64_t mn, int64_t kb,
                                     int64_t tile_rows, int row_major, void* stream) {
-    if (!sf || !out) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!sf || !out) && batch != 0 && mn != 0 && kb != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (batch < 0 || mn < 0 || kb < 0 || tile_rows < (mn + 127) / 128) return mq_fail(MQ_ERR_ARG, "bad shape");
     const int64_t amn = (mn + 3) / 4 * 4, kw = (kb + 3) / 4, total = batch * kw * (row_major ? mn : amn);
     if (total == 0) return MQ_OK;
@@ -679,7 +680,7 @@ extern "C" int mq_ue8m0_pack_scales(const float* sf, int32_t* out, int64_t batch
 
 extern "C" int mq_fp8_block_dequant(const void* x, const float* s, void* y, int64_t M, int64_t N, int block,
                                     void* stream) {
-    if (!x || !s || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!x || !s || !y) && M != 0 && N != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (M < 0 || N < 0 || block <= 0) return mq_fail(MQ_ERR_ARG, "bad shape or block size");
     if (M == 0 || N == 0) return MQ_OK;
     const int64_t tiles_n = (N + block - 1) / block;

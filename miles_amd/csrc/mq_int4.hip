@@ -568,7 +568,7 @@ static void launch_fake_rows(const void* x, int dtype, void* out, void* scale, v
 
 extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* scale, void* zero, int64_t M, int64_t N,
                                   int block_m, int block_n, int sym, void* stream) {
-    if (!x || !out || !scale || (!sym && !zero)) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!x || !out || !scale || (!sym && !zero)) && M != 0 && N != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || N < 0 || block_m <= 0 || block_n <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (((int64_t)block_m * block_n) % 32 != 0 || (int64_t)block_m * block_n > (1 << 24))
         return mq_fail(MQ_ERR_ARG, "block_m * block_n must be divisible by 32");
@@ -608,7 +608,7 @@ int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st) {
 
 extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packed, void* scale, int64_t M, int64_t K,
                                         int group, void* stream) {
-    if (!w || !packed || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !packed || !scale) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (K % group != 0 || K % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and of 8");
     if (M == 0 || K == 0) return MQ_OK;
@@ -629,7 +629,7 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
 
 extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
                                              int32_t* packed_zp, int64_t M, int64_t K, int group, void* stream) {
-    if (!w || !packed || !scale || !zero || !packed_zp) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !packed || !scale || !zero || !packed_zp) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (K % group != 0 || group % 8 != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size and the group size of 8");
     if (M % 8 != 0) return mq_fail(MQ_ERR_ARG, "asymmetric packing needs a multiple of 8 rows");
@@ -670,7 +670,7 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
 
 extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M,
                                       int64_t K, int group, void* stream) {
-    if (!packed || !scale || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!packed || !scale || !y) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (scale_dtype < MQ_BF16 || scale_dtype > MQ_F32 || M < 0 || K < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (K % group != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size");
     if (M == 0 || K == 0) return MQ_OK;

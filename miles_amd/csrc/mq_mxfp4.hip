@@ -274,7 +274,7 @@ int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st) {
 
 extern "C" int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t* scale, int64_t numel, int group,
                               void* stream) {
-    if (!w || !packed || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !packed || !scale) && numel != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (numel % group != 0 || numel % 2 != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the group size and of 2");
     if (numel == 0) return MQ_OK;
@@ -299,7 +299,7 @@ extern "C" int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t
 
 extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, void* y, int64_t bytes, int group,
                                 void* stream) {
-    if (!packed || !scale || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!packed || !scale || !y) && bytes != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (bytes < 0 || group <= 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if ((2 * bytes) % group != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the group size");
     if (bytes == 0) return MQ_OK;
@@ -327,7 +327,7 @@ extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, voi
 
 extern "C" int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, void* y, float* tile_scale,
                                      int64_t out_dim, int64_t in_dim, void* stream) {
-    if (!packed || !scale || !y || !tile_scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!packed || !scale || !y || !tile_scale) && out_dim != 0 && in_dim != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (out_dim < 0 || in_dim < 0 || out_dim % 128 != 0 || in_dim % 128 != 0)
         return mq_fail(MQ_ERR_ARG, "both dimensions must be multiples of 128");
     if ((((uintptr_t)packed | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");

@@ -111,7 +111,7 @@ int mq_mxfp8_launch_group(FlatTable& tab, hipStream_t st) {
 
 extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K,
                               void* stream) {
-    if (!w || !q || !scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w || !q || !scale) && rows != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || rows < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (K % 32 != 0) return mq_fail(MQ_ERR_ARG, "Last dim must be divisible by 32 for MXFP8.");
     if (rows == 0 || K == 0) return MQ_OK;

@@ -461,7 +461,7 @@ int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStre
 }
 
 extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream) {
-    if (!w || !record) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if ((!w && numel != 0) || !record) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (section < 0 || section >= MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section");
     hipStream_t st = (hipStream_t)stream;
@@ -478,7 +478,7 @@ extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* reco
 
 extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
                               float* global_scale, int64_t M, int64_t K, int e4m3_max, int flags, void* stream) {
-    if (!w || !record || !q || !block_scale) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (((!w || !q || !block_scale) && M != 0 && K != 0) || !record) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (n_sections < 1 || n_sections > MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section count");
     if (K % 16 != 0) return mq_fail(MQ_ERR_ARG, "Last dim must be divisible by 16 for NVFP4");
@@ -517,7 +517,7 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
 
 extern "C" int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t numel, int e4m3_max,
                             int flags, void* stream) {
-    if (!x || !amax || !y) return mq_fail(MQ_ERR_ARG, "null pointer");
+    if (((!x || !y) && numel != 0) || !amax) return mq_fail(MQ_ERR_ARG, "null pointer");
     if ((dtype != MQ_BF16 && dtype != MQ_F16) || numel < 0) return mq_fail(MQ_ERR_ARG, "input must be bfloat16 or float16");
     if (numel % 16 != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of 16");
     if (e4m3_max != 448 && e4m3_max != 256) return mq_fail(MQ_ERR_ARG, "e4m3_max must be 448 or 256");

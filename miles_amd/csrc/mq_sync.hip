@@ -64,12 +64,13 @@ static bool job_fast(const mq_job& j) {
 
 static int check_job(const mq_job& j) {
     if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_UE8M0_PACK) return mq_fail(MQ_ERR_ARG, "unknown job kind");
-    if (!j.in || !j.out) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
+    const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
+    if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
     if (j.kind == MQ_JOB_COPY) return MQ_OK;
     if (j.kind == MQ_JOB_UE8M0_PACK)
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
-    if (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
+    if (!empty && (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale)) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
     if (j.rows_per_block != 0) {
         const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST || j.kind == MQ_JOB_FP8_BLOCK_POW2;

@@ -48,6 +48,11 @@ def block_fp8(weight: torch.Tensor, block_size):
 def _scaled_fp8(weight: torch.Tensor, per_channel: bool):
     _lib.require_gpu(weight, "channel_fp8" if per_channel else "tensor_fp8")
     n, k = weight.shape
+    # the reference reduces with weight.abs().max() / .amax(dim=1): torch refuses a reduction over nothing
+    if not per_channel and weight.numel() == 0:
+        raise RuntimeError("max(): Expected reduction dim to be specified for input.numel() == 0. Specify the reduction dim with the 'dim' argument.")
+    if per_channel and k == 0:
+        raise RuntimeError("amax(): Expected reduction dim 1 to have non-zero size.")
     w = weight if weight.stride(1) == 1 else weight.contiguous()
     q = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((n, 1) if per_channel else (1,), dtype=torch.float32, device=w.device)

@@ -1186,3 +1186,58 @@ def test_tensors_beyond_2_to_31_elements(oracle):
             repeats(weight_dequant(big[0], big[1]), weight_dequant(small[0], small[1]), "weight_dequant")
         del big, small
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------------------
+# empty tensors (no rows, or no columns): torch hands them a null data pointer; every wrapper returns outputs of the
+# shapes the reference's torch code would, and the reductions torch refuses over nothing raise the same way
+@pytest.mark.parametrize("shape", [(0, 256), (4, 0)])
+def test_empty_tensors(oracle, shape):
+    from miles_amd.kernels.quant import fake_quant as fq
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda, pack_layer
+    from miles_amd.kernels.quant.nvfp4_qdq import compute_nvfp4_amax
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    x = torch.empty(shape, dtype=torch.bfloat16, device=DEV)
+    xc = x.cpu()
+    for name, got, want in (
+            ("block_fp8", block_fp8(x, [128, 128]), oracle.block_fp8(xc, (128, 128))),
+            ("fp8_blockwise_cast", fp8_blockwise_cast(x), oracle.fp8_blockwise_cast(xc)),
+            ("per_block_cast_to_fp8", per_block_cast_to_fp8(x), oracle.per_block_cast_to_fp8(xc)),
+            ("mxfp4", quantize_mxfp4(x, 32), oracle.quantize_mxfp4(xc, 32)),
+            ("pack_layer", pack_layer(x, 128)[:2], oracle.pack_layer(xc, 128)[:2]),
+            ("fake_int4", fake_int4_quant_cuda(x, (1, 128), False), oracle.fake_int4_quant(xc, (1, 128), False)),
+            ("nvfp4", nvfp4_quantize_1d(x), oracle.nvfp4_quantize_1d(xc)),
+            ("fake_quant", (fq.fake_quant_fp8_forward(x),), (oracle.fake_quant(xc, "fp8"),)),
+            ("act_quant", act_quant(x, 128), oracle.act_quant(xc, 128)),
+            ("fp8_simulate", (fp8_simulate(x, 128),), (oracle.fp8_simulate(xc, 128),))):
+        for j, (g_, w_) in enumerate(zip(got, want)):
+            assert g_.shape == w_.shape and g_.dtype == w_.dtype, f"{name} output {j}: {tuple(g_.shape)} {g_.dtype}"
+            _assert_same(g_, w_, f"{name} output {j}")       # 0-dim NVFP4 global scale: the value of an all-zero tensor
+    q, s = mxfp8_quantize(x)
+    assert q.shape == shape and q.dtype == torch.float8_e4m3fn and s.shape == (shape[0], shape[1] // 32) and s.dtype == torch.uint8
+    a, b = nvfp4_quantize_1d_pair(x, x.clone())
+    assert a[0].shape == (shape[0], shape[1] // 2) and b[1].shape == (shape[0], shape[1] // 16) and torch.equal(a[2], b[2])
+    p, s4 = quantize_mxfp4(x, 32)
+    assert dequantize_mxfp4(p, s4, 32).shape == shape
+    if shape[0] == 0:
+        q8, s8 = block_fp8(x, [128, 128])
+        assert weight_dequant(q8, s8).shape == shape
+        cq, cs = quant_fp8(x, "channel")
+        assert cq.shape == shape and cs.shape == (0, 1)
+        packed, scale, zp = pack_layer(x, 128, sym=False)
+        assert packed.shape == (0, 32) and scale.shape == (0, 2) and zp.shape == (2, 0)
+    else:
+        with pytest.raises(RuntimeError, match="non-zero size"):
+            quant_fp8(x, "channel")
+    with pytest.raises(RuntimeError, match="numel\\(\\) == 0"):
+        quant_fp8(x, "tensor")
+    with pytest.raises(ValueError, match="empty tensor"):
+        compute_nvfp4_amax(x)
+    torch.cuda.synchronize()
