@@ -359,3 +359,65 @@ def test_random_special_values(oracle, monkeypatch, seed, dtype, non_finite):
         check("pack_layer asym", pack_layer(xd, 128, sym=False), oracle.pack_layer(x, 128, sym=False))
         check("nvfp4 qdq", fused_nvfp4_qdq(xd, compute_nvfp4_amax(xd), NVFP4QDQConfig()), oracle.fused_nvfp4_qdq(x))
     assert not failures, "\n".join(failures)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# strided and N-dimensional views: the reference's functions take them (they call .contiguous() or index by stride), so
+# each must give what the contiguous copy gives
+_VIEWS = {
+    "transposed": lambda t: t.t(),
+    "column_slice": lambda t: t[:, 128:384],
+    "every_other_row": lambda t: t[::2],
+    "every_other_column": lambda t: t[:, ::2],
+    "3d": lambda t: t.view(2, 128, 512),
+    "4d": lambda t: t.view(2, 2, 64, 512),
+    "1d": lambda t: t.reshape(-1)[:1024],
+}
+
+
+@pytest.mark.parametrize("view", list(_VIEWS))
+def test_strided_and_nd_views(oracle, view):
+    from miles_amd.kernels.quant import fake_quant as fq
+    from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+    from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda, pack_layer
+    from miles_amd.kernels.quant.nvfp4_qdq import NVFP4QDQConfig, compute_nvfp4_amax, fused_nvfp4_qdq
+    from miles_amd.megatron_to_hf.processors.quantizer_nvfp4 import quantize_nvfp4
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, quant_fp8
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    g = torch.Generator().manual_seed(8000)
+    base = (torch.randn(256, 512, generator=g) * 0.05).to(torch.bfloat16)
+    xc, xd = _VIEWS[view](base), _VIEWS[view](base.to(DEV))
+    cc = xc.contiguous()
+    rows = cc.reshape(-1, cc.shape[-1])
+
+    def check(what, got, want):
+        got, want = (got, want) if isinstance(got, (tuple, list)) else ((got,), (want,))
+        for j, (g_, w_) in enumerate(zip(got, want)):
+            if g_ is not None:
+                _same(g_, w_.reshape(g_.shape), f"{what} output {j} on a {view} view")
+
+    if xc.dim() == 2:
+        check("block_fp8", block_fp8(xd, [128, 128]), oracle.block_fp8(cc, (128, 128)))
+        check("fp8_blockwise_cast", fp8_blockwise_cast(xd), oracle.fp8_blockwise_cast(cc))
+        check("per_block_cast_to_fp8", per_block_cast_to_fp8(xd), oracle.per_block_cast_to_fp8(cc))
+        check("tensor_fp8", quant_fp8(xd, "tensor"), oracle.tensor_fp8(cc))
+        check("channel_fp8", quant_fp8(xd, "channel"), oracle.channel_fp8(cc))
+        check("pack_layer", pack_layer(xd, 128)[:2], oracle.pack_layer(cc, 128)[:2])
+        check("pack_layer asym", pack_layer(xd, 128, sym=False), oracle.pack_layer(cc, 128, sym=False))
+        check("fake_int4", fake_int4_quant_cuda(xd, (1, 128), True)[:2], oracle.fake_int4_quant(cc, (1, 128), True)[:2])
+        check("nvfp4", nvfp4_quantize_1d(xd), oracle.nvfp4_quantize_1d(cc))
+        if not xd.is_contiguous():
+            with pytest.raises(ValueError, match="contiguous"):      # the reference's contract for the fused q-dq
+                fused_nvfp4_qdq(xd, compute_nvfp4_amax(xd), NVFP4QDQConfig())
+    check("mxfp8", mxfp8_quantize(xd), oracle.mxfp8_quantize(rows))
+    check("mxfp4", quantize_mxfp4(xd, 32), oracle.quantize_mxfp4(rows, 32))
+    check("fake_quant", fq.fake_quant_fp8_forward(xd), oracle.fake_quant(rows, "fp8"))
+    check("act_quant", act_quant(xd, 128), oracle.act_quant(rows, 128))
+    check("fp8_simulate", fp8_simulate(xd, 128), oracle.fp8_simulate(rows, 128))
+    if xc.dim() == 3:
+        want = tuple(torch.stack(f) for f in zip(*[oracle.nvfp4_quantize_1d(cc[i]) for i in range(cc.shape[0])]))
+        check("quantize_nvfp4 on a stack", quantize_nvfp4(xd), want)
