@@ -465,6 +465,25 @@ def parity_sample(weights, args, plan):
     return f"ok ({checked} tensors of layer 0 byte-identical to the oracle)"
 
 
+def stream_ceilings():
+    """What plain streaming kernels reach on this GPU at the read : write mixes of the quantizers, measured with torch's own
+    elementwise kernels on 4 GiB operands (no part of the product): the yardstick for the per-quantizer fractions."""
+    n = 1 << 31
+    x = torch.empty(n, dtype=torch.bfloat16, device=DEV).normal_()
+    y = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    q = torch.empty(n, dtype=torch.float8_e4m3fn, device=DEV)
+    res = {}
+    for name, fn, nbytes in (("fill_write_only", lambda: y.fill_(1.0), 2 * n),
+                             ("copy_bf16_1r_1w", lambda: y.copy_(x), 4 * n),
+                             ("cast_bf16_to_fp8_2r_1w", lambda: q.copy_(x), 3 * n),
+                             ("cast_fp8_to_bf16_1r_2w", lambda: y.copy_(q), 3 * n)):
+        fn()
+        torch.cuda.synchronize()
+        ms = min(_event_ms(fn, 5) for _ in range(3))
+        res[name] = {"GBps": round(nbytes / ms / 1e6, 1), "ms": round(ms, 4)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -477,6 +496,8 @@ def main():
     ap.add_argument("--pmc-quantizers", action="store_true",
                     help="counter-collection run: three 1 GiB plain copies (calibration), then every workload of the "
                          "per-quantizer section exactly twice, no timing")
+    ap.add_argument("--stream-ceilings", action="store_true",
+                    help="only torch's fill / copy / cast kernels on 4 GiB operands: what plain streaming reaches here (one JSON line)")
     ap.add_argument("--full-configs", action="store_true",
                     help="only the three MoE configurations at full size, each as one whole sync (one JSON line)")
     a = ap.parse_args()
@@ -490,6 +511,9 @@ def main():
     _lib.load()   # fails loudly if the HIP library is not built
     gen = torch.Generator(device=DEV)
     gen.manual_seed(2001)
+    if a.stream_ceilings:
+        print(json.dumps({"stream_ceilings": stream_ceilings()}))
+        return
     if a.full_configs:
         print(json.dumps({"full_configs": full_configs(gen)}))
         return
