@@ -32,6 +32,10 @@ def weights_signature(weights: Mapping[str, torch.Tensor]) -> tuple:
     return tuple((name, t.data_ptr(), tuple(t.shape), t.dtype) for name, t in weights.items())
 
 
+class _NotPackable(Exception):
+    """A bucket holds a tensor that can be neither produced in place in a flat payload nor byte-copied into it."""
+
+
 class SyncPlan:
     def __init__(self, batch: launch.JobBatch, buckets: list[Unit], jobs_done_at_bucket: list[int],
                  signature: tuple, replayable: bool) -> None:
@@ -71,10 +75,14 @@ class SyncPlan:
         produced = batch.output_pointers() | batch.constants
         handed_out_ok = all(t.numel() == 0 or t.data_ptr() in produced or cls._in_spans(spans, t.data_ptr())
                             for bucket in buckets for _, t in bucket)
+        packable = True
         if packed:
-            buckets, marks = cls._pack(batch, buckets, marks)
+            try:
+                buckets, marks = cls._pack(batch, buckets, marks)
+            except _NotPackable:
+                packable = False       # the updater flattens such buckets after the fact (one extra copy), every sync
         batch.freeze()
-        replayable = batch.direct_calls == 0 and handed_out_ok and cls._inputs_alias(weights, batch)
+        replayable = batch.direct_calls == 0 and handed_out_ok and packable and cls._inputs_alias(weights, batch)
         plan = cls(batch, buckets, marks, weights_signature(weights), replayable)
         plan.remember(weights)
         for _ in plan.replay():     # the first execution uses the same launch partition as every replay
@@ -119,7 +127,7 @@ class SyncPlan:
                         records[ri][f] = new.data_ptr()
                 elif old.numel():
                     if not old.is_contiguous():
-                        raise _lib.MilesQuantError(f"packed buckets need contiguous pass-through tensors, got {name}")
+                        raise _NotPackable(f"{name} is a strided pass-through tensor: it needs a gathering copy")
                     nbytes = old.numel() * old.element_size()
                     copies.append((_lib.JOB_COPY, 0, old.data_ptr(), new.data_ptr(), None, None, None, 1, nbytes, nbytes,
                                    0, 0, 0, 0))

@@ -55,6 +55,7 @@ class WeightUpdater:
                                                 quantization_config=quantization_config,
                                                 packed_weight_basenames=packed_weight_basenames)
         self._plan: SyncPlan | None = None
+        self._packed_plan_refused = False
         self._metrics: dict[str, float] = {}
 
     def pop_metrics(self) -> dict[str, float]:
@@ -77,13 +78,15 @@ class WeightUpdater:
         if self.use_plan and self._plan is not None and self._plan.matches(weights):
             yield from self._plan.replay()
             return
-        if self.use_plan:
+        if self.use_plan and not self._packed_plan_refused:
             plan = SyncPlan.record(self._iterator, weights, packed=self.packed_buckets)
             if plan.replayable or not self.packed_buckets:
                 self._plan = plan
                 yield from plan.buckets
                 return
-            # a packed plan re-points job outputs, which is only safe to keep when it can be replayed
+            # a packed plan re-points job outputs, which is only safe to keep when it can be replayed; a model that
+            # cannot be planned this way is not tried again (recording runs the whole sync once for nothing)
+            self._packed_plan_refused = True
         for bucket in self._iterator.iter_hf_weights(weights):
             yield pack_bucket(bucket) if self.packed_buckets else bucket
 

@@ -306,6 +306,61 @@ def test_packed_buckets_without_plan_and_layout_errors(oracle):
         pack_bucket([("w", torch.zeros(3, dtype=torch.uint8, device=DEV)), ("scale", torch.zeros(2, device=DEV))])
 
 
+def _mixed_bucket():
+    """The tensor mix of the reference's wire-format test (tests/fast/backends/training_utils/weight_update/
+    test_broadcast_packed.py:41-50): transposed and strided views, an e4m3 vector, a 0-dim scalar, an empty tensor."""
+    return [("expert.weight", torch.arange(16, dtype=torch.uint8).reshape(2, 8).T),
+            ("expert.weight_scale", torch.tensor([0, 128, 126, 255], dtype=torch.uint8).view(torch.float8_e4m3fn)),
+            ("expert.weight_scale_2", torch.tensor(-0.0, dtype=torch.float32)),
+            ("dense.weight", torch.arange(8, dtype=torch.bfloat16).reshape(2, 4).T),
+            ("strided_bf16.weight", torch.arange(8, dtype=torch.bfloat16)[::2]),
+            ("strided_fp32.weight", torch.arange(8, dtype=torch.float32)[::2]),
+            ("empty", torch.empty((0, 2), dtype=torch.float32))]
+
+
+def test_pack_bucket_keeps_mixed_dtype_bytes_scalar_shapes_and_strided_views():
+    from miles_amd.weight_update.packed_bucket import pack_bucket
+
+    cpu = _mixed_bucket()
+    packed = pack_bucket([(n, t.to(DEV)) for n, t in cpu])
+    torch.cuda.synchronize()
+    assert [n for n, _ in packed] == [n for n, _ in cpu]
+    for (_, want), (_, got), meta in zip(cpu, packed, packed.get_metadata()):
+        assert got.shape == want.shape and got.dtype == want.dtype and got.is_contiguous()
+        assert meta.numel == want.numel() and meta.end_idx - meta.start_idx == want.numel() * want.element_size()
+        assert torch.equal(got.cpu().flatten().view(torch.uint8), want.contiguous().flatten().view(torch.uint8))
+    assert torch.equal(packed.get_flattened_tensor().cpu(), _payload_bytes(cpu))
+    assert [t.shape for _, t in packed.reconstruct_tensors()] == [t.shape for _, t in cpu]
+
+
+def test_packed_sync_of_a_model_with_strided_pass_through_tensors_falls_back_to_flattening(monkeypatch):
+    # a strided view cannot be byte-copied into a payload slot by a job: the plan is refused once and every sync flattens
+    # its buckets after the fact, still current after the weights change in place
+    from miles_amd.weight_update.packed_bucket import PackedBucket
+
+    base = torch.arange(64, dtype=torch.bfloat16, device=DEV).reshape(8, 8)
+    weights = {"w": base}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: weights, model_name="qwen3", quantization_config=None, send_bucket=None,
+                        packed_buckets=True)
+    calls = []
+
+    def fake_iter(ws):
+        calls.append(1)
+        yield [("a.weight", ws["w"].t()), ("b.weight", ws["w"][:, ::2]), ("c.weight", ws["w"])]
+
+    monkeypatch.setattr(upd._iterator, "iter_hf_weights", fake_iter)
+    for step in range(3):
+        got = []
+        upd.send_bucket = got.append
+        upd.update_weights()
+        torch.cuda.synchronize()
+        assert len(got) == 1 and isinstance(got[0], PackedBucket)
+        want = [("a.weight", base.t().cpu()), ("b.weight", base[:, ::2].cpu()), ("c.weight", base.cpu())]
+        assert torch.equal(got[0].flat.cpu(), _payload_bytes(want)), f"sync {step}"
+        base.add_(1)
+    assert upd._plan is None and len(calls) == 4       # recorded once (refused), then one pass per sync
+
+
 def test_plan_is_not_replayed_when_a_handed_out_tensor_would_go_stale():
     # without quantization the q/k/v tensors are fresh copies made by the name map: replaying a recorded plan would
     # hand out last step's values, so the updater must run the full iterator every time
