@@ -117,9 +117,16 @@ def per_quantizer(gen):
 
     res = {}
 
-    def run(name, key, elems, build, note):
+    def run(name, key, elems, build, note, prepare=None, before_each=None):
         batch, outs = _record(build)
-        ms = _best_ms(batch.run)
+        if prepare is not None:
+            prepare(batch)
+        fn = batch.run
+        if before_each is not None:
+            def fn():
+                before_each()
+                batch.run()
+        ms = _best_ms(fn)
         gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
         res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                      "elements": elems, "workload": note}
@@ -152,10 +159,28 @@ def per_quantizer(gen):
             out.append(nvfp4_quantize_1d(fc2))
         return out
 
-    run("C5a_nvfp4", "nvfp4", n, nvfp4_all, "32 experts, gate/up paired + down, amax pass + quantize pass")
+    # NVFP4 as the sync driver runs it: the first sync of a model takes two passes (amax, then quantize); every later sync
+    # quantizes in one pass with the amax its records kept and repeats only the tensors whose amax moved
+    run("C5a_nvfp4", "nvfp4", n, nvfp4_all,
+        "32 experts, gate/up paired + down; steady-state sync: one pass with the amax carried over from the previous sync "
+        "(checked on the way; here no amax moves)", prepare=lambda b: b.carry_nvfp4_amax())
+    run("C5a_nvfp4_first_sync", "nvfp4", n, nvfp4_all, "as C5a, first sync of a model: amax pass + quantize pass")
+    firsts = [t.view(-1)[:1] for fc1, fc2 in experts for t in (fc1, fc2)]
+    for f in firsts:
+        f.fill_(1.0)            # the largest element of every tensor (of every gate/up pair), toggled below
+    toggle = [4.0]
+
+    def move_every_amax():
+        torch._foreach_mul_(firsts, toggle[0])
+        toggle[0] = 1.0 / toggle[0]
+
+    run("C5a_nvfp4_every_amax_moved", "nvfp4", n, nvfp4_all,
+        "as C5a, worst case of the carried amax: every tensor's amax differs from the last sync's, so each is quantized twice",
+        prepare=lambda b: b.carry_nvfp4_amax(), before_each=move_every_amax)
     os.environ["NVTE_NVFP4_4OVER6"] = "weights"        # Four Over Six: two candidates per block, e4m3 max 256
     try:
-        run("C5a_nvfp4_four_over_six", "nvfp4", n, nvfp4_all, "as C5a with NVTE_NVFP4_4OVER6=weights (MAE, e4m3 max 256)")
+        run("C5a_nvfp4_four_over_six", "nvfp4", n, nvfp4_all,
+            "as C5a (steady state) with NVTE_NVFP4_4OVER6=weights (MAE, e4m3 max 256)", prepare=lambda b: b.carry_nvfp4_amax())
     finally:
         del os.environ["NVTE_NVFP4_4OVER6"]
     run("C5b_block_fp8", "fp8_block", n,

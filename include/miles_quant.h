@@ -156,7 +156,9 @@ int mq_fp8_act_quant(const void* x, int dtype, void* y, void* scale, int64_t num
  *   miles/kernels/quant/nvfp4_qdq.py:893-990): every block is quantized for a maximum of 6 and of 4 and keeps the
  *   candidate with the smaller error; MQ_NVFP4_ERR_MSE squares the error terms (NVTE_NVFP4_4OVER6_ERR_MODE=MSE),
  *   MQ_NVFP4_ERR_FP16 uses the fp16 candidate-error form (NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH=1). */
-enum { MQ_NVFP4_4OVER6 = 1, MQ_NVFP4_ERR_MSE = 2, MQ_NVFP4_ERR_FP16 = 4 };
+enum { MQ_NVFP4_4OVER6 = 1, MQ_NVFP4_ERR_MSE = 2, MQ_NVFP4_ERR_FP16 = 4,
+       /* jobs of mq_run_jobs only: see the NVFP4 note there */
+       MQ_NVFP4_CARRY_AMAX = 8 };
 int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream);
 int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream);
 int mq_nvfp4_quant(const void* w, int dtype, const void* record, int n_sections, void* q, void* block_scale,
@@ -198,7 +200,12 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
- * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list. */
+ * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list.
+ * MQ_NVFP4_CARRY_AMAX in p1 (no counterpart in the reference): a caller that submits the same job list again, amax
+ * records included and untouched in between, after at least one submission without the flag, may set it on bf16
+ * jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
+ * submission, collects the new amax on the way, and quantizes a tensor a second time only if its amax changed
+ * (results are identical either way; a weight tensor's amax rarely moves between two syncs). */
 enum {
     MQ_JOB_FP8_BLOCK = 0,
     MQ_JOB_FP8_BLOCKWISE_CAST = 1,

@@ -49,6 +49,7 @@ SIGNATURES = {
 
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs
 NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
+NVFP4_CARRY_AMAX = 8                                      # MQ_NVFP4_CARRY_AMAX: NVFP4 jobs of a re-submitted list only
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
  JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK) = range(10)

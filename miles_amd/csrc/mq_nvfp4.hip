@@ -105,26 +105,49 @@ constexpr int kRecAmax = MQ_NVFP4_SECTIONS * kSectionWords;   // folded amax (fl
 constexpr int kRecEncSixth = kRecAmax + 1;                     // S_enc * (1/6)
 constexpr int kRecSDec = kRecAmax + 2;                         // 1 / S_enc
 constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
+constexpr int kRecRedo = kRecAmax + 4;                         // carried-over amax turned out stale: quantize again
 
-// one workgroup per tensor: fold the first job.section sections of its record and publish the scales.
-// Tensors that share a record compute the same values and write them twice.
+// Fold kernel, one workgroup per tensor.
+// MODE 0 (single calls): fold the first job.section sections of the record and publish the scales.  Tensors that share
+//   a record compute the same values and write them twice.
+// MODE 1 / 2 (the job driver): job.section is the tensor's place inside its record and job.pad the number of tensors
+//   sharing it; they sit next to each other in the table.  Only the workgroup of the last one works: it folds all their
+//   sections, writes every one's global scale and then clears the sections, so that the next sync may collect its
+//   partial maxima with atomic max (see the carried-over amax below).  MODE 2 additionally checks the amax and scales
+//   the record held before against the new ones: all four words equal means the codes just written with the old values
+//   are final (kRecRedo = 0); otherwise the new values are stored and kRecRedo = 1 asks for a second quantization.
+template <int MODE>
 __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, float numer) {
     __shared__ uint32_t lds4[4];
-    const FlatJob& job = tab.job[blockIdx.x];
+    const int ji = blockIdx.x;
+    const FlatJob& job = tab.job[ji];
+    const int sections = MODE == 0 ? job.section : job.pad;
+    if (MODE != 0 && job.section != job.pad - 1) return;
     uint32_t* rec = (uint32_t*)job.aux;
     uint32_t m = 0;
-    for (int i = threadIdx.x; i < job.section * kSectionWords; i += 256) m = umax(m, rec[i]);
+    for (int i = threadIdx.x; i < sections * kSectionWords; i += 256) m = umax(m, rec[i]);
     m = wave_max(m);
     if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = m;
     __syncthreads();
+    if (MODE != 0)
+        for (int i = threadIdx.x; i < sections * kSectionWords; i += 256) rec[i] = 0;
     if (threadIdx.x == 0) {
         const float amax = u2f(umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3])));
         const NvScales gs = nv_scales(amax, numer);
+        if (MODE == 2)
+            rec[kRecRedo] = !(rec[kRecAmax] == f2u(amax) && rec[kRecEncSixth] == f2u(gs.enc_sixth) &&
+                              rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
         rec[kRecAmax] = f2u(amax);
         rec[kRecEncSixth] = f2u(gs.enc_sixth);
         rec[kRecSDec] = f2u(gs.s_dec);
         rec[kRecEnc] = f2u(gs.enc);
-        if (job.aux2) *(float*)job.aux2 = nv_published_scale(amax, numer);
+        const float published = nv_published_scale(amax, numer);
+        if (MODE == 0) {
+            if (job.aux2) *(float*)job.aux2 = published;
+        } else {
+            for (int k = 0; k < sections; k++)
+                if (tab.job[ji - k].aux2) *(float*)tab.job[ji - k].aux2 = published;
+        }
     }
 }
 
@@ -221,18 +244,15 @@ __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float 
 // error mode of a flags word, as the EM template argument
 static inline int nv_error_mode(int flags) { return ((flags & MQ_NVFP4_ERR_MSE) ? 1 : 0) | ((flags & MQ_NVFP4_ERR_FP16) ? 2 : 0); }
 
+// kNvThreads * kNvUnroll units starting at `base` of one tensor; returns the largest |element| this lane saw (bf16 bits)
 // FOS = 0: standard quantizer; FOS = 1 + error mode: Four Over Six
 template <int FOS>
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float denom) {
-    const FlatJob& job = tab.job[blockIdx.y];
+__device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
     const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
     const int64_t total_units = job.units;
-    const int t = threadIdx.x;
-    const int64_t base = flat_block(tab) * (kNvThreads * kNvUnroll);
-    if (base >= total_units) return;
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
@@ -245,11 +265,13 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     gs.enc = u2f(amax_bits[kRecEnc]);
     const float amax = u2f(amax_bits[kRecAmax]);
     const bool fastdiv = nv_fast_division(amax);
+    uint32_t seen = 0;
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
         const int64_t unit = base + i * kNvThreads + t;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max2(hmax_u16(m2));
+        seen = umax(seen, mb);
         const float bmax = u2f(mb << 16);
         const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
@@ -280,6 +302,41 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
         if (unit < total_units) {
             st4(q + unit, word);
             if ((t & 1) == 0) s8[unit >> 1] = (uint8_t)sc;
+        }
+    }
+    return seen;
+}
+
+// Carried-over amax.  A weight tensor's amax rarely changes from one sync to the next (the largest element has to move
+// to another bf16 value), and the amax record of a replayed job list still holds the last sync's amax and scales.
+// PASS 1 quantizes with those in a single read of the tensor and collects this sync's partial maxima on the way (one
+// atomic max per workgroup into the tensor's section, cleared by the previous fold); the fold kernel then compares, and
+// PASS 2, a small grid striding over the blocks, quantizes again only the tensors whose amax did change.
+// PASS 0 is the second pass of the plain two-pass form (amax kernel, fold, quantize).
+template <int FOS, int PASS>
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float denom) {
+    const FlatJob& job = tab.job[blockIdx.y];
+    const int t = threadIdx.x;
+    constexpr int64_t kPerBlock = kNvThreads * kNvUnroll;
+    if (PASS == 2) {
+        if (((const uint32_t*)job.aux)[kRecRedo] == 0) return;
+        for (int64_t base = (int64_t)blockIdx.x * kPerBlock; base < job.units; base += (int64_t)gridDim.x * kPerBlock)
+            nvfp4_quant_units<FOS>(job, base, t, denom);
+        return;
+    }
+    const int64_t base = flat_block(tab) * kPerBlock;
+    if (base >= job.units) return;
+    uint32_t seen = nvfp4_quant_units<FOS>(job, base, t, denom);
+    if (PASS == 1) {
+        __shared__ uint32_t wave_seen[kNvThreads / 64];
+        seen = wave_max(seen);
+        if ((t & 63) == 0) wave_seen[t >> 6] = seen;
+        __syncthreads();
+        if (t == 0) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int k = 0; k < kNvThreads / 64; k++) m = umax(m, wave_seen[k]);
+            atomicMax((uint32_t*)job.aux + job.section * kSectionWords + (blockIdx.x & (kSectionWords - 1)), m << 16);
         }
     }
 }
@@ -441,22 +498,41 @@ int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
     return mq_check_launch("nvfp4 amax");
 }
 
-// tab.job[i]: w, q, s = block scales, aux = amax record, section = sections to fold, aux2 = fp32 global scale
-// out (may be null), units = numel / 8.  Launches the fold kernel, then the quantize pass.
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStream_t st) {
+template <int PASS>
+static void launch_nvfp4_quant(const FlatTable& tab, int flags, float numer, dim3 grid, hipStream_t st) {
+    const dim3 blk(kNvThreads);
+    switch ((flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0) {
+        case 0: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS>), grid, blk, 0, st, tab, numer); break;
+        case 1: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<1, PASS>), grid, blk, 0, st, tab, numer); break;
+        case 2: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<2, PASS>), grid, blk, 0, st, tab, numer); break;
+        case 3: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<3, PASS>), grid, blk, 0, st, tab, numer); break;
+        default: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<4, PASS>), grid, blk, 0, st, tab, numer); break;
+    }
+}
+
+// tab.job[i]: w, q, s = block scales, aux = amax record, aux2 = fp32 global scale out (may be null), units = numel / 8.
+// mode 0 (single calls): section = sections to fold; fold, then quantize.
+// mode 1 (job driver, after its amax launch): section = place of the tensor inside its record, pad = tensors sharing the
+//   record (adjacent entries); fold once per record, clear the sections, quantize.
+// mode 2 (job driver, carried-over amax; the sections were cleared by the previous sync's fold): quantize with the
+//   record's old scales while collecting the new partial maxima, fold and compare, quantize again where they differ.
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st) {
     const float numer = (float)e4m3_max * 6.0f;
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3((unsigned)tab.n), dim3(256), 0, st, tab, numer);
-    if (tab.max_blocks > 0) {
-        const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kNvThreads);
-        switch ((flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0) {
-            case 0: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<0>, grid, blk, 0, st, tab, numer); break;
-            case 1: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<1>, grid, blk, 0, st, tab, numer); break;
-            case 2: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<2>, grid, blk, 0, st, tab, numer); break;
-            case 3: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<3>, grid, blk, 0, st, tab, numer); break;
-            default: hipLaunchKernelGGL(nvfp4_quant_bf16_kernel<4>, grid, blk, 0, st, tab, numer); break;
+    const dim3 folds((unsigned)tab.n), blk(256);
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n);
+    if (mode == 2) {
+        if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
+        hipLaunchKernelGGL(nvfp4_fold_kernel<2>, folds, blk, 0, st, tab, numer);
+        if (tab.max_blocks > 0) {
+            const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
+            launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)tab.n), st);
         }
+        return mq_check_launch("nvfp4 quant (carried-over amax)");
     }
+    if (mode == 1) hipLaunchKernelGGL(nvfp4_fold_kernel<1>, folds, blk, 0, st, tab, numer);
+    else hipLaunchKernelGGL(nvfp4_fold_kernel<0>, folds, blk, 0, st, tab, numer);
+    if (tab.max_blocks > 0) launch_nvfp4_quant<0>(tab, flags, numer, grid, st);
     return mq_check_launch("nvfp4 quant");
 }
 
@@ -491,12 +567,12 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), blocks16 * 2, global_scale, n_sections, 0};
-        return mq_nvfp4_quant_launch_group(tab, e4m3_max, flags, st);
+        return mq_nvfp4_quant_launch_group(tab, e4m3_max, flags, 0, st);
     }
     FlatTable fold{};
     fold.n = 1;
     fold.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), 0, global_scale, n_sections, 0};
-    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3(1), dim3(256), 0, st, fold, numer);
+    hipLaunchKernelGGL(nvfp4_fold_kernel<0>, dim3(1), dim3(256), 0, st, fold, numer);
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
@@ -511,7 +587,7 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
     FlatTable tab{};
     tab.n = 1;
     tab.job[0] = FlatJob{nullptr, nullptr, nullptr, record, 0, nullptr, n_sections, 0};
-    hipLaunchKernelGGL(nvfp4_fold_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
+    hipLaunchKernelGGL(nvfp4_fold_kernel<0>, dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
     return mq_check_launch("nvfp4 fold");
 }
 

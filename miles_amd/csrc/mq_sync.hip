@@ -24,7 +24,7 @@ bool mq_int4_pack_fast_ok(const void* w, int dtype, int group);
 int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st);
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, hipStream_t st);
+int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
@@ -141,20 +141,27 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
         bool all_fast = true;
         for (int t = 0; t < n; t++) all_fast &= job_fast(jobs[i + t]);
         if (all_fast) {
+            // MQ_NVFP4_CARRY_AMAX (set by a caller that replays this very list, records included, after a first plain
+            // run): one pass with last sync's amax instead of the amax pass; every job of the chunk must ask for it
+            bool carry = true;
+            for (int t = 0; t < n; t++) carry &= (jobs[i + t].p1 & MQ_NVFP4_CARRY_AMAX) != 0;
             FlatTable tab{};
             tab.n = n;
+            int rc = MQ_OK;
+            if (!carry) {
+                for (int t = 0; t < n; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    const int64_t numel = jb.rows * jb.cols;
+                    tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8, nullptr, section[t], 0};
+                }
+                rc = mq_nvfp4_amax_launch_group(tab, st);
+                if (rc) return rc;
+            }
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
-                const int64_t numel = jb.rows * jb.cols;
-                tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8, nullptr, section[t], 0};
+                tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, section[t], sections[t]};
             }
-            int rc = mq_nvfp4_amax_launch_group(tab, st);
-            if (rc) return rc;
-            for (int t = 0; t < n; t++) {
-                const mq_job& jb = jobs[i + t];
-                tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, sections[t], 0};
-            }
-            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, jobs[i].p1, st);
+            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, jobs[i].p1 & ~MQ_NVFP4_CARRY_AMAX, carry ? 2 : 1, st);
             if (rc) return rc;
         } else {
             for (int t = 0; t < n; t++) {
@@ -165,7 +172,7 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
                 int rc = mq_nvfp4_quant(jb.in, jb.dtype, jb.aux, sections[t], jb.out, jb.scale, (float*)jb.aux2, jb.rows,
-                                        jb.cols, jb.p0, jb.p1, stream);
+                                        jb.cols, jb.p0, jb.p1 & ~MQ_NVFP4_CARRY_AMAX, stream);
                 if (rc) return rc;
             }
         }

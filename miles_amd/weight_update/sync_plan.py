@@ -45,6 +45,7 @@ class SyncPlan:
         self.signature = signature
         self.replayable = replayable
         self._marks: list[int] | None = None
+        self._completed = 0         # full replays so far
         self._names: list[str] = []
         self._tensors: list[torch.Tensor] = []
         self._addresses: list[int] = []
@@ -221,6 +222,11 @@ class SyncPlan:
             self.batch.run_range(done, mark)
             done = max(done, mark)
             yield bucket
+        self._completed += 1
+        if self._completed == 1:
+            # every amax record now holds this model's values: later replays quantize NVFP4 tensors in one pass with
+            # them and repeat a tensor only when its amax moved
+            self.batch.carry_nvfp4_amax()
 
     def replay_all(self) -> list[Unit]:
         """Whole model in one submission (fewest launches); returns every bucket."""

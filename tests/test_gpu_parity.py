@@ -1241,3 +1241,60 @@ def test_empty_tensors(oracle, shape):
     with pytest.raises(ValueError, match="empty tensor"):
         compute_nvfp4_amax(x)
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------------------
+# NVFP4 with the amax carried over from the previous run of the same job list: one pass when the amax did not move,
+# a second quantization of exactly the tensors whose amax did -- the results must never depend on which happened
+@pytest.mark.parametrize("four_over_six", [False, True])
+def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
+    from miles_amd import launch
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    for name in ("NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256", "NVTE_NVFP4_4OVER6_ERR_MODE"):
+        monkeypatch.delenv(name, raising=False)
+    kw = {}
+    if four_over_six:
+        monkeypatch.setenv("NVTE_NVFP4_4OVER6", "weights")
+        kw = {"e4m3_max": 256, "flags": 1}
+    shapes = [(256, 512), (384, 1024), (100, 256), (64, 2048), (512, 512), (128, 7168)]
+    cpu = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=1200 + i) for i, s in enumerate(shapes)]
+    pair_cpu = [W.gaussian_outliers((320, 768), std=0.02, p_outlier=0.001, gain=20.0, seed=1250 + i) for i in range(2)]
+    dev, pair_dev = [w.to(DEV) for w in cpu], [w.to(DEV) for w in pair_cpu]
+    with launch.recording() as batch:
+        outs = [nvfp4_quantize_1d(w) for w in dev[:3]]
+        pair_out = nvfp4_quantize_1d_pair(*pair_dev)
+        outs += [nvfp4_quantize_1d(w) for w in dev[3:]]
+    batch.device = torch.device(DEV)
+
+    def check(what):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, (w, got) in enumerate(zip(dev, outs)):
+            for j, (g_, w_) in enumerate(zip(got, oracle.nvfp4_quantize_1d(w.cpu(), **kw))):
+                _assert_same(g_, w_, f"{what}: tensor {i} output {j}")
+        want = oracle.nvfp4_quantize_1d_pair(pair_dev[0].cpu(), pair_dev[1].cpu(), **kw)
+        for half in range(2):
+            for j, (g_, w_) in enumerate(zip(pair_out[half], want[half])):
+                _assert_same(g_, w_, f"{what}: pair half {half} output {j}")
+
+    check("first run (two passes)")
+    assert batch.carry_nvfp4_amax() == len(shapes) + 2
+    check("same weights (every amax carried)")
+    check("same weights again")
+    for w in dev + pair_dev:                       # new values everywhere, every amax as before
+        top = w.abs().flatten().argmax()
+        keep = w.flatten()[top].clone()
+        w.mul_(0.75)
+        w.view(-1)[top] = keep
+    check("changed data, same amax")
+    dev[1].mul_(3.0)                               # these amax move: tensor 1 up, tensor 4 down, the pair through its second half
+    dev[4].mul_(0.25)
+    pair_dev[1].mul_(5.0)
+    check("three amax moved")
+    check("and stayed")
+    dev[2].zero_()                                 # amax 0
+    dev[0].view(-1)[7] = float("inf")              # amax inf
+    check("zero tensor and an infinity")
+    dev[0].view(-1)[7] = 1.0
+    check("back to finite")
