@@ -172,7 +172,16 @@ def test_moe_nvfp4_sync_pairs_share_amax(oracle):
     dev = {k: v.to(DEV) for k, v in cpu.items()}
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="deepseekv3",
                         quantization_config={"quant_method": "modelopt", "quant_algo": "NVFP4"}, send_bucket=None)
-    for round_ in range(2):
+    # round 0 records the plan (amax pass + quantize pass); later rounds replay it with the amax carried over: round 1 on
+    # new weights (every amax moved), round 2 on the same weights (none moved), round 3 with one expert's amax moved
+    changed = _moe_model(41)
+    one_moved = {k: v.clone() for k, v in changed.items()}
+    moved_name = next(k for k in one_moved if "linear_fc1" in k)
+    one_moved[moved_name].mul_(2.0)
+    rounds = [cpu, changed, changed, one_moved]
+    for round_, cpu in enumerate(rounds):
+        for k in dev:
+            dev[k].copy_(cpu[k])
         flat = [nt for b in _run(upd) for nt in b]
         want = []
         for name, param in cpu.items():
@@ -190,10 +199,8 @@ def test_moe_nvfp4_sync_pairs_share_amax(oracle):
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
             _same(g, w, f"{n} round {round_}")
-        cpu = _moe_model(41)
-        for k in dev:
-            dev[k].copy_(cpu[k])
     assert upd._plan.replayable
+    assert any(r[upd._plan.batch.P1] & 8 for r in upd._plan.batch.records), "replays should carry the amax over"
 
 
 def test_moe_int4_compressed_tensors_sync(oracle):
