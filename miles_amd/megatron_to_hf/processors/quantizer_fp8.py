@@ -13,8 +13,6 @@ from __future__ import annotations
 
 import os
 
-import torch
-
 from miles_amd.kernels.quant.fp8_blockwise import (fp8_blockwise_cast, per_block_cast_to_fp8, quant_weight_ue8m0,
                                                    transform_scale_ue8m0)
 from miles_amd.tools.convert_hf_to_fp8 import tensor_fp8
