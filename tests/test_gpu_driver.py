@@ -437,6 +437,35 @@ def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
 
 
 @pytest.mark.parametrize("packed", [False, True])
+def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
+    # no weight_block_size in the config: the per-tensor branch (quantizer_fp8.py:153-158), scale name `.weight_scale`.
+    # Its two-pass quantizer is launched directly, so the sync cannot be planned: every sync runs the whole iterator.
+    cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic"}
+    cpu = _dense_model(62)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=cfg, send_bucket=None,
+                        packed_buckets=packed)
+    for round_ in range(3):
+        flat = [nt for b in _run(upd) for nt in b]
+        want = []
+        for name, param in cpu.items():
+            if "word_embeddings" in name or "output_layer" in name:
+                param = param[:1000]
+            for hf, t in name_maps.convert_qwen2_to_hf(ARGS, name, param):
+                if hf.endswith("_proj.weight"):
+                    q, sc = oracle.tensor_fp8(t.contiguous())
+                    want += [(hf, q), (hf.replace(".weight", ".weight_scale"), sc)]
+                else:
+                    want.append((hf, t))
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} round {round_}")
+        cpu = _dense_model(63 + round_)
+        for k in dev:
+            dev[k].copy_(cpu[k])
+
+
+@pytest.mark.parametrize("packed", [False, True])
 def test_dense_fp8_sync_with_packed_ue8m0_scales(oracle, packed):
     # DeepGEMM requantization (quantizer_fp8.py:140-142): power-of-two tile scales, then four exponent bytes per int32
     # in a row-contiguous layout; the packer consumes the scales of a job recorded just before it
