@@ -163,7 +163,7 @@ def per_quantizer(gen):
     # quantizes in one pass with the amax its records kept and repeats only the tensors whose amax moved
     run("C5a_nvfp4", "nvfp4", n, nvfp4_all,
         "32 experts, gate/up paired + down; steady-state sync: one pass with the amax carried over from the previous sync "
-        "(checked on the way; here no amax moves)", prepare=lambda b: b.carry_nvfp4_amax())
+        "(checked on the way; here no amax moves)", prepare=lambda b: b.carry_amax())
     run("C5a_nvfp4_first_sync", "nvfp4", n, nvfp4_all, "as C5a, first sync of a model: amax pass + quantize pass")
     firsts = [t.view(-1)[:1] for fc1, fc2 in experts for t in (fc1, fc2)]
     for f in firsts:
@@ -176,11 +176,11 @@ def per_quantizer(gen):
 
     run("C5a_nvfp4_every_amax_moved", "nvfp4", n, nvfp4_all,
         "as C5a, worst case of the carried amax: every tensor's amax differs from the last sync's, so each is quantized twice",
-        prepare=lambda b: b.carry_nvfp4_amax(), before_each=move_every_amax)
+        prepare=lambda b: b.carry_amax(), before_each=move_every_amax)
     os.environ["NVTE_NVFP4_4OVER6"] = "weights"        # Four Over Six: two candidates per block, e4m3 max 256
     try:
         run("C5a_nvfp4_four_over_six", "nvfp4", n, nvfp4_all,
-            "as C5a (steady state) with NVTE_NVFP4_4OVER6=weights (MAE, e4m3 max 256)", prepare=lambda b: b.carry_nvfp4_amax())
+            "as C5a (steady state) with NVTE_NVFP4_4OVER6=weights (MAE, e4m3 max 256)", prepare=lambda b: b.carry_amax())
     finally:
         del os.environ["NVTE_NVFP4_4OVER6"]
     run("C5b_block_fp8", "fp8_block", n,
@@ -319,8 +319,20 @@ def adjacent_formats(gen):
         "pack_layer(sym=False), group 128")
     from miles_amd.tools.convert_hf_to_fp8 import channel_fp8, tensor_fp8
     run("a2_channel_fp8", "fp8_channel", lambda: [channel_fp8(w) for w in ws], "one scale per row, rows read once")
-    run("a2_tensor_fp8", "fp8_channel", lambda: [tensor_fp8(w) for w in ws],
-        "one scale per tensor: amax pass + quantize pass (5 B/element moved, 3 counted)")
+    # per-tensor FP8 is a job of the batched driver: timed as a replayed job list, like the sync path runs it
+    batch, outs = _record(lambda: [tensor_fp8(w) for w in ws])
+    ms = _best_ms(batch.run)
+    gbps = elems * BYTES_PER_ELEM["fp8_channel"] / ms / 1e6
+    res["a2_tensor_fp8_first_sync"] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+                                       "elements": elems, "workload": "one scale per tensor, first sync of a model: amax pass + "
+                                       "quantize pass (5 B/element moved, 3 counted)"}
+    batch.carry_amax()
+    ms = _best_ms(batch.run)
+    gbps = elems * BYTES_PER_ELEM["fp8_channel"] / ms / 1e6
+    res["a2_tensor_fp8"] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
+                            "elements": elems, "workload": "one scale per tensor, steady-state sync: one pass with the amax "
+                            "carried over from the previous sync (checked on the way; here no amax moves)"}
+    del batch, outs
     from miles_amd.kernels.quant.int4_fake import fake_int4_quant_cuda
     run("a8_fake_int4_quant_1x128", "fake_int4_bf16", lambda: [fake_int4_quant_cuda(w, [1, 128], True) for w in ws],
         "fake_int4_quant_cuda(x, (1,128), sym): bf16 in, bf16 integer codes + bf16 scales out")

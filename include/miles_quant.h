@@ -195,15 +195,18 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208)
  *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
  *   MQ_JOB_UE8M0_PACK           fp32 tiles    int32 words   -              -                           batch, tile_rows
+ *   MQ_JOB_FP8_TENSOR           w[rows,cols]  e4m3          fp32 [1]       aux = amax record           floor bits, flags
+ *     (tensor_fp8 / the per-tensor branch of the sync path, see mq_fp8_scaled_quant: bf16, contiguous, cols % 8 == 0,
+ *      16-byte aligned input; p0 = bit pattern of 1e-12 rounded to the weight dtype; p1 = 0 or MQ_NVFP4_CARRY_AMAX)
  *     (mq_ue8m0_pack_scales with mn = rows, kb = cols, row_major = ld; its input is usually the scale output of an
  *      earlier job)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
  * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list.
- * MQ_NVFP4_CARRY_AMAX in p1 (no counterpart in the reference): a caller that submits the same job list again, amax
- * records included and untouched in between, after at least one submission without the flag, may set it on bf16
- * jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
+ * MQ_NVFP4_CARRY_AMAX in p1 of NVFP4 and FP8_TENSOR jobs (no counterpart in the reference): a caller that submits the
+ * same job list again, amax records included and untouched in between, after at least one submission without the
+ * flag, may set it on bf16 jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
  * submission, collects the new amax on the way, and quantizes a tensor a second time only if its amax changed
  * (results are identical either way; a weight tensor's amax rarely moves between two syncs). */
 enum {
@@ -216,7 +219,8 @@ enum {
     MQ_JOB_MXFP4 = 6,
     MQ_JOB_COPY = 7,
     MQ_JOB_FP8_BLOCK_POW2 = 8,
-    MQ_JOB_UE8M0_PACK = 9
+    MQ_JOB_UE8M0_PACK = 9,
+    MQ_JOB_FP8_TENSOR = 10
 };
 typedef struct mq_job {
     int32_t kind;

@@ -127,6 +127,13 @@ inline bool flat_grid(FlatTable& tab, int64_t per_block) {
     return mx < 0x7FFFFFF0;
 }
 
+// The amax record of the quantizers that need a whole-tensor maximum (NVFP4, per-tensor FP8): kRecordSections
+// sections of kSectionWords partial maxima (float bit patterns), then the folded amax and what is derived from it.
+constexpr int kSectionWords = 256;      // MQ_NVFP4_SECTION_WORDS: workgroups of an amax pass per tensor
+constexpr int kRecordSections = 4;      // MQ_NVFP4_SECTIONS
+constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (float bits)
+constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
+
 struct CopyJob {      // one run of bytes
     const uint8_t* src;
     uint8_t* dst;

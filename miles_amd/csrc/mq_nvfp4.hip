@@ -26,7 +26,7 @@ constexpr int kNvThreads = 256;
 constexpr int kNvUnroll = MQ_NV_UNROLL;
 constexpr float kSixth = 0.16666667163372040f;  // 0x3E2AAAAB
 
-constexpr int kSectionWords = MQ_NVFP4_SECTION_WORDS;   // = workgroups of the amax pass per tensor
+static_assert(kSectionWords == MQ_NVFP4_SECTION_WORDS && kRecordSections == MQ_NVFP4_SECTIONS, "record layout");
 #ifndef MQ_AMAX_UNROLL
 #define MQ_AMAX_UNROLL 4
 #endif
@@ -101,11 +101,9 @@ __device__ __forceinline__ float nv_published_scale(float amax, float numer) {
 }
 
 // words of a record behind its sections
-constexpr int kRecAmax = MQ_NVFP4_SECTIONS * kSectionWords;   // folded amax (float bits)
 constexpr int kRecEncSixth = kRecAmax + 1;                     // S_enc * (1/6)
 constexpr int kRecSDec = kRecAmax + 2;                         // 1 / S_enc
 constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
-constexpr int kRecRedo = kRecAmax + 4;                         // carried-over amax turned out stale: quantize again
 
 // Fold kernel, one workgroup per tensor.
 // MODE 0 (single calls): fold the first job.section sections of the record and publish the scales.  Tensors that share

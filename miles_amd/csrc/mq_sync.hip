@@ -6,6 +6,8 @@
 // list order.
 #include <vector>
 
+#include <string.h>
+
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -27,6 +29,8 @@ int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
+bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
+int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -57,13 +61,15 @@ static bool job_fast(const mq_job& j) {
             return mq_mxfp4_fast_ok(j.in, j.dtype, j.out, j.p0);
         case MQ_JOB_COPY:
             return true;
+        case MQ_JOB_FP8_TENSOR:
+            return mq_fp8_tensor_fast_ok(j.in, j.dtype, j.out, j.rows, j.cols, j.ld);
         default:
             return false;
     }
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_UE8M0_PACK) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_FP8_TENSOR) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
@@ -72,6 +78,10 @@ static int check_job(const mq_job& j) {
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
     if (!empty && (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale)) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
+    if (j.kind == MQ_JOB_FP8_TENSOR) {
+        if (!j.aux || !j.scale) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 job without an amax record or a scale pointer");
+        if (!empty && !job_fast(j)) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 jobs take contiguous bf16 tensors (cols % 8 == 0, 16-byte aligned)");
+    }
     if (j.rows_per_block != 0) {
         const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST || j.kind == MQ_JOB_FP8_BLOCK_POW2;
         if (!fp8q || j.rows_per_block < 0 || j.rows_per_block % 128 != 0 || j.p0 != 128 || j.p1 != 128 || j.dtype != MQ_BF16)
@@ -109,6 +119,31 @@ static_assert(kMaxGroup == MQ_MAX_GROUP, "the public group size must match the l
 
 static bool same_group(const mq_job& a, const mq_job& b) {
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
+}
+
+// per-tensor FP8 run [i, j): chunks of up to kMaxGroup tensors of similar size with the same floor and flags
+static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
+    while (i < j) {
+        FlatTable tab{};
+        int64_t k = i, sum = 0, mx = 0;
+        while (k < j && k - i < kMaxGroup && jobs[k].p0 == jobs[i].p0 && jobs[k].p1 == jobs[i].p1) {
+            const int64_t e = jobs[k].rows * jobs[k].cols;
+            const int64_t nmx = e > mx ? e : mx;
+            if (k > i && nmx * (k - i + 1) * 4 > (sum + e) * 5) break;       // padding of the 2-D grid under 25 %
+            tab.job[k - i] = FlatJob{jobs[k].in, jobs[k].out, jobs[k].scale, jobs[k].aux, e / 8, nullptr, 0, 1};
+            sum += e;
+            mx = nmx;
+            k++;
+        }
+        tab.n = (int)(k - i);
+        const uint32_t floor_bits = (uint32_t)jobs[i].p0;
+        float floor_v;
+        memcpy(&floor_v, &floor_bits, 4);
+        int rc = mq_fp8_tensor_launch_group(tab, floor_v, (jobs[i].p1 & MQ_NVFP4_CARRY_AMAX) != 0, (hipStream_t)stream);
+        if (rc) return rc;
+        i = k;
+    }
+    return MQ_OK;
 }
 
 // NVFP4 run [i, j): all jobs fast or not, processed as amax-phase then quantize-phase per chunk
@@ -191,10 +226,10 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
     int64_t i = 0;
     while (i < n) {
         const mq_job& head = jobs[i];
-        if (head.kind == MQ_JOB_NVFP4) {
+        if (head.kind == MQ_JOB_NVFP4 || head.kind == MQ_JOB_FP8_TENSOR) {
             int64_t j = i + 1;
-            while (j < n && jobs[j].kind == MQ_JOB_NVFP4) j++;
-            int rc = run_nvfp4(jobs, i, j, stream);
+            while (j < n && jobs[j].kind == head.kind) j++;
+            int rc = head.kind == MQ_JOB_NVFP4 ? run_nvfp4(jobs, i, j, stream) : run_fp8_tensor(jobs, i, j, stream);
             if (rc) return rc;
             i = j;
             continue;

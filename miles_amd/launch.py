@@ -58,21 +58,23 @@ class JobBatch:
             self._keep = list(keep)
         self._array = None
 
-    def carry_nvfp4_amax(self) -> int:
-        """After this list has run once: let later runs of the same list quantize NVFP4 tensors in one pass with the
-        amax their record kept from the run before (MQ_NVFP4_CARRY_AMAX; the driver checks the amax on the way and
-        quantizes a tensor again if it moved, so results do not change).  Only done when every NVFP4 job of the list
-        is one the packed kernels take (bf16, 16-byte aligned input, 4-byte aligned codes), so that every record goes
-        through the same driver path on every run.  Returns the number of jobs flagged."""
+    def carry_amax(self) -> int:
+        """After this list has run once: let later runs of the same list quantize NVFP4 and per-tensor FP8 tensors in
+        one pass with the amax their record kept from the run before (MQ_NVFP4_CARRY_AMAX; the driver checks the amax on
+        the way and quantizes a tensor again if it moved, so results do not change).  NVFP4 jobs are only flagged when
+        every one of the list is one the packed kernels take (bf16, 16-byte aligned input, 4-byte aligned codes), so
+        that every record goes through the same driver path on every run; per-tensor FP8 jobs always are.
+        Returns the number of jobs flagged."""
         nv = [r for r in self._records if r[self.KIND] == _lib.JOB_NVFP4]
-        fit = all(r[self.DTYPE] == _lib.DTYPE_CODE[torch.bfloat16] and (r[self.IN] or 0) % 16 == 0
-                  and (r[self.OUT] or 0) % 4 == 0 and r[self.COLS] % 16 == 0 for r in nv)
-        if not nv or not fit:
-            return 0
-        self._records = [r[: self.P1] + (r[self.P1] | _lib.NVFP4_CARRY_AMAX,) + r[self.P1 + 1:]
-                         if r[self.KIND] == _lib.JOB_NVFP4 else r for r in self._records]
-        self._array = None
-        return len(nv)
+        nv_fit = bool(nv) and all(r[self.DTYPE] == _lib.DTYPE_CODE[torch.bfloat16] and (r[self.IN] or 0) % 16 == 0
+                                  and (r[self.OUT] or 0) % 4 == 0 and r[self.COLS] % 16 == 0 for r in nv)
+        kinds = {_lib.JOB_FP8_TENSOR} | ({_lib.JOB_NVFP4} if nv_fit else set())
+        flagged = sum(r[self.KIND] in kinds for r in self._records)
+        if flagged:
+            self._records = [r[: self.P1] + (r[self.P1] | _lib.NVFP4_CARRY_AMAX,) + r[self.P1 + 1:]
+                             if r[self.KIND] in kinds else r for r in self._records]
+            self._array = None
+        return flagged
 
     def hold(self, tensor: torch.Tensor) -> None:
         """Keep a tensor alive for as long as the batch exists."""

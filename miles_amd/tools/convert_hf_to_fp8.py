@@ -45,6 +45,9 @@ def block_fp8(weight: torch.Tensor, block_size):
     return q, scale
 
 
+_AMAX_RECORD_WORDS = 1280   # MQ_NVFP4_RECORD_WORDS: partial maxima of a tensor on the device, then its folded amax
+
+
 def _scaled_fp8(weight: torch.Tensor, per_channel: bool):
     _lib.require_gpu(weight, "channel_fp8" if per_channel else "tensor_fp8")
     n, k = weight.shape
@@ -56,9 +59,15 @@ def _scaled_fp8(weight: torch.Tensor, per_channel: bool):
     w = weight if weight.stride(1) == 1 else weight.contiguous()
     q = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((n, 1) if per_channel else (1,), dtype=torch.float32, device=w.device)
+    floor = float(torch.tensor(1e-12, dtype=w.dtype).float())  # clamp(min=1e-12) acts in the weight dtype
+    if not per_channel and w.dtype == torch.bfloat16 and w.is_contiguous() and k % 8 == 0 and w.data_ptr() % 16 == 0:
+        # a job of the batched driver (grouped launches, replayable): amax record as for NVFP4
+        record = torch.empty(_AMAX_RECORD_WORDS, dtype=torch.int32, device=w.device)
+        floor_bits = int(torch.tensor(floor, dtype=torch.float32).view(torch.int32))
+        launch.submit(_lib.JOB_FP8_TENSOR, w, q, scale, record, None, n, k, k, floor_bits, 0)
+        return q, scale
     ws = torch.empty(max(n, 1), dtype=torch.int32, device=w.device)
     launch.note_direct_call()
-    floor = float(torch.tensor(1e-12, dtype=w.dtype).float())  # clamp(min=1e-12) acts in the weight dtype
     rc = _lib.load().mq_fp8_scaled_quant(w.data_ptr(), _lib.dtype_code(w, "fp8"), w.stride(0), q.data_ptr(),
                                          scale.data_ptr(), ws.data_ptr(), n, k, int(per_channel), floor,
                                          _lib.stream_ptr(w.device))

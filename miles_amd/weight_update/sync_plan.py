@@ -226,7 +226,7 @@ class SyncPlan:
         if self._completed == 1:
             # every amax record now holds this model's values: later replays quantize NVFP4 tensors in one pass with
             # them and repeat a tensor only when its amax moved
-            self.batch.carry_nvfp4_amax()
+            self.batch.carry_amax()
 
     def replay_all(self) -> list[Unit]:
         """Whole model in one submission (fewest launches); returns every bucket."""

@@ -439,13 +439,15 @@ def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
 @pytest.mark.parametrize("packed", [False, True])
 def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
     # no weight_block_size in the config: the per-tensor branch (quantizer_fp8.py:153-158), scale name `.weight_scale`.
-    # Its two-pass quantizer is launched directly, so the sync cannot be planned: every sync runs the whole iterator.
+    # Every quantizer call is a job of the batched driver; the plan itself is not replayed for this model, because q / k / v
+    # of the fused attention weight are regrouped into fresh tensors by the name map (in-place row-block views exist for
+    # the 128x128 quantizers only)
     cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic"}
     cpu = _dense_model(62)
     dev = {k: v.to(DEV) for k, v in cpu.items()}
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=cfg, send_bucket=None,
                         packed_buckets=packed)
-    for round_ in range(3):
+    for round_ in range(4):
         flat = [nt for b in _run(upd) for nt in b]
         want = []
         for name, param in cpu.items():
@@ -460,9 +462,11 @@ def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
             _same(g, w, f"{n} round {round_}")
-        cpu = _dense_model(63 + round_)
-        for k in dev:
-            dev[k].copy_(cpu[k])
+        if round_ != 1:             # rounds 1 and 2 see the same weights: no amax moves between them
+            cpu = _dense_model(63 + round_)
+            for k in dev:
+                dev[k].copy_(cpu[k])
+    assert upd._plan is None or not upd._plan.replayable
 
 
 @pytest.mark.parametrize("packed", [False, True])

@@ -1279,7 +1279,7 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
                 _assert_same(g_, w_, f"{what}: pair half {half} output {j}")
 
     check("first run (two passes)")
-    assert batch.carry_nvfp4_amax() == len(shapes) + 2
+    assert batch.carry_amax() == len(shapes) + 2
     check("same weights (every amax carried)")
     check("same weights again")
     for w in dev + pair_dev:                       # new values everywhere, every amax as before
@@ -1298,3 +1298,52 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
     check("zero tensor and an infinity")
     dev[0].view(-1)[7] = 1.0
     check("back to finite")
+
+
+def test_tensor_fp8_jobs_grouped_and_with_carried_amax(oracle):
+    # per-tensor FP8 as a job of the batched driver: several tensors per launch, and later runs of the same list with the
+    # amax carried over (one pass, a second quantization only where the amax moved)
+    from miles_amd import launch
+    from miles_amd.tools.convert_hf_to_fp8 import quant_fp8
+
+    shapes = [(256, 512), (100, 264), (3, 8), (1024, 1024), (64, 7168), (129, 1000)]
+    cpu = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=1300 + i) for i, s in enumerate(shapes)]
+    dev = [w.to(DEV) for w in cpu]
+    with launch.recording() as batch:
+        outs = [quant_fp8(w, "tensor") for w in dev]
+    assert len(batch) == len(shapes) and batch.direct_calls == 0
+    batch.device = torch.device(DEV)
+
+    def check(what):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, (w, (q, sc)) in enumerate(zip(dev, outs)):
+            q_o, s_o = oracle.tensor_fp8(w.cpu())
+            _assert_same(sc, s_o, f"{what}: tensor {i} scale")
+            _assert_same(q, q_o, f"{what}: tensor {i} codes")
+
+    check("first run (two passes)")
+    assert batch.carry_amax() == len(shapes)
+    check("same weights")
+    for w in dev:                                    # new values, every amax as before
+        top = w.abs().flatten().argmax()
+        keep = w.flatten()[top].clone()
+        w.mul_(0.5)
+        w.view(-1)[top] = keep
+    check("changed data, same amax")
+    dev[0].mul_(3.0)
+    dev[3].mul_(0.125)
+    check("two amax moved")
+    dev[2].zero_()                                   # amax below the 1e-12 floor
+    dev[4].view(-1)[5] = float("nan")                # NaN amax: scale and every code NaN
+    check("zero tensor and a NaN")
+    dev[4].view(-1)[5] = 0.5
+    check("back to finite")
+    # tensors the packed kernels do not take still go through the direct two-pass entry point
+    odd = torch.randn(16, 12, device=DEV).to(torch.bfloat16)
+    with launch.recording() as b2:
+        q, sc = quant_fp8(odd, "tensor")
+    assert len(b2) == 0 and b2.direct_calls == 1
+    q_o, s_o = oracle.tensor_fp8(odd.cpu())
+    _assert_same(sc, s_o, "odd width scale")
+    _assert_same(q, q_o, "odd width codes")
