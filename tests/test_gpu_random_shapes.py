@@ -198,13 +198,13 @@ def test_random_job_lists_in_one_submission(oracle, seed):
     from miles_amd import launch
     from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
     from miles_amd.kernels.quant.int4_fake import pack_layer
-    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8, tensor_fp8
     from miles_amd.utils.mxfp4 import quantize_mxfp4
     from miles_amd.utils.mxfp8 import mxfp8_quantize
     from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
 
     rng = random.Random(f"miles-jobs-{seed}")
-    kinds = ["cast", "block", "mxfp8", "int4", "nvfp4", "pair", "mxfp4"]
+    kinds = ["cast", "block", "mxfp8", "int4", "nvfp4", "pair", "mxfp4", "tensor"]
     plan = []
     for i in range(150):
         kind = rng.choice(kinds) if rng.random() < 0.5 or not plan else plan[-1][0]       # runs of one kind and switches
@@ -223,14 +223,14 @@ def test_random_job_lists_in_one_submission(oracle, seed):
             results[i] = {"cast": lambda: fp8_blockwise_cast(x), "block": lambda: block_fp8(x, [128, 128]),
                           "mxfp8": lambda: mxfp8_quantize(x), "int4": lambda: pack_layer(x, 128)[:2],
                           "nvfp4": lambda: nvfp4_quantize_1d(x), "mxfp4": lambda: quantize_mxfp4(x, 32),
-                          "pair": lambda: nvfp4_quantize_1d_pair(x, dev[i, "b"])}[kind]()
+                          "tensor": lambda: tensor_fp8(x), "pair": lambda: nvfp4_quantize_1d_pair(x, dev[i, "b"])}[kind]()
         assert len(batch) == sum(2 if k == "pair" else 1 for k, _, _ in plan)
     for kind, shape, i in plan:
         x = cpu[i, "a"]
         want = {"cast": lambda: oracle.fp8_blockwise_cast(x), "block": lambda: oracle.block_fp8(x, (128, 128)),
                 "mxfp8": lambda: oracle.mxfp8_quantize(x), "int4": lambda: oracle.pack_layer(x, 128)[:2],
                 "nvfp4": lambda: oracle.nvfp4_quantize_1d(x), "mxfp4": lambda: oracle.quantize_mxfp4(x, 32),
-                "pair": lambda: oracle.nvfp4_quantize_1d_pair(x, cpu[i, "b"])}[kind]()
+                "tensor": lambda: oracle.tensor_fp8(x), "pair": lambda: oracle.nvfp4_quantize_1d_pair(x, cpu[i, "b"])}[kind]()
         got = results[i]
         if kind == "pair":
             got, want = [t for half in got for t in half], [t for half in want for t in half]
