@@ -217,7 +217,7 @@ def test_random_job_lists_in_one_submission(oracle, seed):
             cpu[i, tag] = (torch.randn(shape, generator=g) * 0.05).to(torch.bfloat16)
             dev[i, tag] = cpu[i, tag].to(DEV)
     results = {}
-    with launch.deferred() as batch:
+    with launch.recording() as batch:
         for kind, shape, i in plan:
             x = dev[i, "a"]
             results[i] = {"cast": lambda: fp8_blockwise_cast(x), "block": lambda: block_fp8(x, [128, 128]),
@@ -225,6 +225,29 @@ def test_random_job_lists_in_one_submission(oracle, seed):
                           "nvfp4": lambda: nvfp4_quantize_1d(x), "mxfp4": lambda: quantize_mxfp4(x, 32),
                           "tensor": lambda: tensor_fp8(x), "pair": lambda: nvfp4_quantize_1d_pair(x, dev[i, "b"])}[kind]()
         assert len(batch) == sum(2 if k == "pair" else 1 for k, _, _ in plan)
+    batch.device = torch.device(DEV)
+    batch.run()
+    _check_job_list(oracle, plan, cpu, results, "first submission")
+    # the same list again with the amax of the NVFP4 / per-tensor FP8 jobs carried over: unchanged inputs, then every third
+    # tensor doubled (its amax moves) and every fourth replaced by new values under the old maximum
+    batch.carry_amax()
+    batch.run()
+    _check_job_list(oracle, plan, cpu, results, "second submission, same inputs")
+    for n, (key, x) in enumerate(sorted(dev.items())):
+        if n % 3 == 0:
+            x.mul_(2.0)
+        elif n % 4 == 0:
+            top = x.abs().flatten().argmax()
+            keep = x.flatten()[top].clone()
+            x.mul_(0.5)
+            x.view(-1)[top] = keep
+        cpu[key] = x.cpu()
+    batch.run()
+    _check_job_list(oracle, plan, cpu, results, "third submission, changed inputs")
+
+
+def _check_job_list(oracle, plan, cpu, results, what):
+    torch.cuda.synchronize()
     for kind, shape, i in plan:
         x = cpu[i, "a"]
         want = {"cast": lambda: oracle.fp8_blockwise_cast(x), "block": lambda: oracle.block_fp8(x, (128, 128)),
@@ -235,7 +258,7 @@ def test_random_job_lists_in_one_submission(oracle, seed):
         if kind == "pair":
             got, want = [t for half in got for t in half], [t for half in want for t in half]
         for j, (g_, w_) in enumerate(zip(got, want)):
-            _same(g_, w_, f"job {i} ({kind} {shape}) output {j}")
+            _same(g_, w_, f"{what}: job {i} ({kind} {shape}) output {j}")
 
 
 # ---------------------------------------------------------------------------------------------------------------------
