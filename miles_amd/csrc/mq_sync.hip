@@ -121,6 +121,20 @@ static bool same_group(const mq_job& a, const mq_job& b) {
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
 }
 
+// Copy jobs of one launch run in no particular order: a job that reads what an earlier job of the group writes (a
+// regrouped tensor that is then copied into a payload), or writes what one reads or writes, has to start a new group.
+static bool copy_depends_on_group(const mq_job* jobs, int64_t first, int64_t candidate) {
+    const mq_job& c = jobs[candidate];
+    const uintptr_t cin = (uintptr_t)c.in, cout = (uintptr_t)c.out, cb = (uintptr_t)(c.rows * c.cols);
+    for (int64_t t = first; t < candidate; t++) {
+        const uintptr_t tin = (uintptr_t)jobs[t].in, tout = (uintptr_t)jobs[t].out, tb = (uintptr_t)(jobs[t].rows * jobs[t].cols);
+        const bool reads_written = cin < tout + tb && tout < cin + cb;
+        const bool writes_touched = (cout < tout + tb && tout < cout + cb) || (cout < tin + tb && tin < cout + cb);
+        if (reads_written || writes_touched) return true;
+    }
+    return false;
+}
+
 // per-tensor FP8 run [i, j): chunks of up to kMaxGroup tensors of similar size with the same floor and flags
 static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
     while (i < j) {
@@ -251,6 +265,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
             const int64_t e = jobs[j].rows * jobs[j].cols;
             const int64_t nmx = e > mx ? e : mx;
             if (flat && nmx * (j - i + 1) * 4 > (sum + e) * 5) break;
+            if (head.kind == MQ_JOB_COPY && copy_depends_on_group(jobs, i, j)) break;
             sum += e;
             mx = nmx;
             j++;

@@ -368,9 +368,29 @@ def test_packed_sync_of_a_model_with_strided_pass_through_tensors_falls_back_to_
     assert upd._plan is None and len(calls) == 4       # recorded once (refused), then one pass per sync
 
 
-def test_plan_is_not_replayed_when_a_handed_out_tensor_would_go_stale():
-    # without quantization the q/k/v tensors are fresh copies made by the name map: replaying a recorded plan would
-    # hand out last step's values, so the updater must run the full iterator every time
+def test_copy_jobs_that_depend_on_each_other_run_in_order():
+    # one submission: a -> b, b -> c, then c -> a shifted by 16 bytes (overlapping its own source's neighbour); copy jobs of
+    # one launch run in no order, so the driver has to cut the launches at each dependency
+    from miles_amd import launch
+    from miles_amd.weight_update.packed_bucket import submit_copy
+
+    g = torch.Generator().manual_seed(77)
+    a = torch.randint(0, 255, (4096,), dtype=torch.uint8, generator=g).to(DEV)
+    b, c = torch.zeros_like(a), torch.zeros_like(a)
+    before = a.cpu().clone()
+    with launch.deferred() as batch:
+        submit_copy(a, b)
+        submit_copy(b, c)
+        submit_copy(c[:4080], a[16:])
+        assert len(batch) == 3
+    torch.cuda.synchronize()
+    assert torch.equal(b.cpu(), before) and torch.equal(c.cpu(), before)
+    assert torch.equal(a.cpu()[16:], before[:4080]) and torch.equal(a.cpu()[:16], before[:16])
+
+
+def test_unquantized_sync_hands_out_current_regrouped_qkv():
+    # without quantization q / k / v are regrouped copies of the fused attention weight: the copies are jobs of the plan,
+    # so a replay refreshes them (a tensor a torch op had materialised would hand out last step's values)
     cpu = _dense_model(40)
     dev = {k: v.to(DEV) for k, v in cpu.items()}
     for packed in (False, True):
@@ -385,6 +405,7 @@ def test_plan_is_not_replayed_when_a_handed_out_tensor_would_go_stale():
                                                   cpu2["module.module.decoder.layers.1.self_attention.linear_qkv.weight"]))
         for n, w in want.items():
             _same(flat[n], w, n)
+        assert upd._plan is not None and upd._plan.replayable
 
 
 def test_packed_buckets_int4_moe_two_syncs(oracle):
@@ -439,9 +460,8 @@ def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
 @pytest.mark.parametrize("packed", [False, True])
 def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
     # no weight_block_size in the config: the per-tensor branch (quantizer_fp8.py:153-158), scale name `.weight_scale`.
-    # Every quantizer call is a job of the batched driver; the plan itself is not replayed for this model, because q / k / v
-    # of the fused attention weight are regrouped into fresh tensors by the name map (in-place row-block views exist for
-    # the 128x128 quantizers only)
+    # Every quantizer call is a job of the batched driver and q / k / v are regrouped by copy jobs, so the sync is planned
+    # and replayed, from the second replay on with the amax carried over
     cfg = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic"}
     cpu = _dense_model(62)
     dev = {k: v.to(DEV) for k, v in cpu.items()}
@@ -466,7 +486,8 @@ def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
             cpu = _dense_model(63 + round_)
             for k in dev:
                 dev[k].copy_(cpu[k])
-    assert upd._plan is None or not upd._plan.replayable
+    assert upd._plan is not None and upd._plan.replayable
+    assert any(r[upd._plan.batch.KIND] == 10 and r[upd._plan.batch.P1] & 8 for r in upd._plan.batch.records)
 
 
 @pytest.mark.parametrize("packed", [False, True])
