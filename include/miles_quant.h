@@ -198,6 +198,9 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_FP8_TENSOR           w[rows,cols]  e4m3          fp32 [1]       aux = amax record           floor bits, flags
  *     (tensor_fp8 / the per-tensor branch of the sync path, see mq_fp8_scaled_quant: bf16, contiguous, cols % 8 == 0,
  *      16-byte aligned input; p0 = bit pattern of 1e-12 rounded to the weight dtype; p1 = 0 or MQ_NVFP4_CARRY_AMAX)
+ *   MQ_JOB_INT4_PACK_ASYM       w             int32 words   scales (dtype) aux = uint8 zero points,    group, -
+ *                                                                          aux2 = int32 packed_zp
+ *     (mq_int4_group_quant_pack_asym, one tensor per launch pair)
  *     (mq_ue8m0_pack_scales with mn = rows, kb = cols, row_major = ld; its input is usually the scale output of an
  *      earlier job)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
@@ -220,7 +223,8 @@ enum {
     MQ_JOB_COPY = 7,
     MQ_JOB_FP8_BLOCK_POW2 = 8,
     MQ_JOB_UE8M0_PACK = 9,
-    MQ_JOB_FP8_TENSOR = 10
+    MQ_JOB_FP8_TENSOR = 10,
+    MQ_JOB_INT4_PACK_ASYM = 11
 };
 typedef struct mq_job {
     int32_t kind;

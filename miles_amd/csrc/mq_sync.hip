@@ -69,7 +69,7 @@ static bool job_fast(const mq_job& j) {
 }
 
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_FP8_TENSOR) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_INT4_PACK_ASYM) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
@@ -78,6 +78,7 @@ static int check_job(const mq_job& j) {
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
     if (!empty && (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale)) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
+    if (j.kind == MQ_JOB_INT4_PACK_ASYM && !empty && (!j.aux || !j.aux2)) return mq_fail(MQ_ERR_ARG, "asymmetric INT4 job without zero-point outputs");
     if (j.kind == MQ_JOB_FP8_TENSOR) {
         if (!j.aux || !j.scale) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 job without an amax record or a scale pointer");
         if (!empty && !job_fast(j)) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 jobs take contiguous bf16 tensors (cols % 8 == 0, 16-byte aligned)");
@@ -108,6 +109,9 @@ static int run_single(const mq_job& j, void* stream) {
             return mq_int4_group_quant_pack(j.in, j.dtype, (int32_t*)j.out, j.scale, j.rows, j.cols, j.p0, stream);
         case MQ_JOB_MXFP4:
             return mq_mxfp4_quant(j.in, j.dtype, (uint8_t*)j.out, (uint8_t*)j.scale, j.rows * j.cols, j.p0, stream);
+        case MQ_JOB_INT4_PACK_ASYM:
+            return mq_int4_group_quant_pack_asym(j.in, j.dtype, (int32_t*)j.out, j.scale, (uint8_t*)j.aux, (int32_t*)j.aux2,
+                                                 j.rows, j.cols, j.p0, stream);
         case MQ_JOB_UE8M0_PACK:
             return mq_ue8m0_pack_scales((const float*)j.in, (int32_t*)j.out, j.p0, j.rows, j.cols, j.p1, j.ld != 0, stream);
         default:

@@ -74,9 +74,6 @@ def _pack_layer_asym(weight: torch.Tensor, group_size: int):
     scale = torch.empty((M, groups), dtype=w.dtype, device=w.device)
     zero = torch.empty((M, groups), dtype=torch.uint8, device=w.device)
     packed_zp = torch.empty((groups, M // 8), dtype=torch.int32, device=w.device)
-    launch.note_direct_call()
-    rc = _lib.load().mq_int4_group_quant_pack_asym(w.data_ptr(), _lib.dtype_code(w, "pack_layer"), packed.data_ptr(),
-                                                   scale.data_ptr(), zero.data_ptr(), packed_zp.data_ptr(), M, K,
-                                                   group_size, _lib.stream_ptr(w.device))
-    _lib.check(rc, RuntimeError)
+    _lib.dtype_code(w, "pack_layer")
+    launch.submit(_lib.JOB_INT4_PACK_ASYM, w, packed, scale, zero, packed_zp, M, K, K, int(group_size), 0)
     return packed, scale, packed_zp

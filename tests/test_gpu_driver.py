@@ -226,6 +226,37 @@ def test_moe_int4_compressed_tensors_sync(oracle):
         _same(g, w, n)
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_moe_int4_asymmetric_sync_is_planned_and_replayed(oracle, packed):
+    # symmetric: False adds zero points (quantizer_compressed_tensors.py:286-301); the asymmetric packer is a job too
+    cfg = {"quant_method": "compressed-tensors", "format": "pack-quantized",
+           "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": False, "num_bits": 4, "type": "int"}}}}
+    basenames = {f"model.layers.{l}.mlp.experts.{e}.{p}_proj" for l in range(2) for e in range(4) for p in ("gate", "up", "down")}
+    cpu = _moe_model(55)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="kimi_k2", quantization_config=cfg, send_bucket=None,
+                        packed_weight_basenames=basenames, packed_buckets=packed)
+    for round_ in range(3):
+        flat = [nt for b in _run(upd) for nt in b]
+        want = []
+        for name, param in cpu.items():
+            for hf, t in name_maps.convert_deepseekv3_to_hf(ARGS, name, param):
+                if hf.removesuffix(".weight") in basenames:
+                    p_, s_, z_ = oracle.pack_layer(t.contiguous(), 128, sym=False)
+                    want += [(hf.replace(".weight", ".weight_zero_point"), z_),      # the reference's order (:296-301)
+                             (hf.replace(".weight", ".weight_packed"), p_), (hf.replace(".weight", ".weight_scale"), s_),
+                             (hf.replace(".weight", ".weight_shape"), torch.tensor(t.shape, dtype=torch.int32))]
+                else:
+                    want.append((hf, t))
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} round {round_}")
+        cpu = _moe_model(56 + round_)
+        for k in dev:
+            dev[k].copy_(cpu[k])
+    assert upd._plan is not None and upd._plan.replayable
+
+
 # ---------------------------------------------------------------------------------------------------
 # packed transport buckets: quantizers write straight into the flat payload
 def _payload_bytes(named):
