@@ -102,6 +102,10 @@ class SyncPlan:
                 if rec[f] is not None and rec[0] != _lib.JOB_COPY:
                     writers.setdefault(rec[f], []).append((ri, f))
         records = [list(r) for r in batch.records]
+        # byte copies recorded by a name map (regrouped q / k / v): [destination, record index, bytes], by destination
+        gathers = sorted((rec[3], ri, rec[7] * rec[8]) for ri, rec in enumerate(batch.records)
+                         if rec[0] == _lib.JOB_COPY and rec[3] is not None)
+        gather_starts = [g[0] for g in gathers]
         new_buckets: list[Unit] = []
         copies_of: list[list[tuple]] = []
         for bucket in buckets:      # first re-point every job (a bucket's range may hold jobs of the next bucket)
@@ -123,6 +127,20 @@ class SyncPlan:
                 # FP8 job has no other kernel at all); a slot that follows, say, a 12-byte scale grid is filled by a copy
                 if hits and new.data_ptr() % 16 and any(f == 3 for _, f in hits):
                     hits = None
+                if not hits and old.is_contiguous() and old.numel():
+                    # a tensor that copy jobs assemble piece by piece is assembled in its payload slot instead
+                    lo, nbytes = old.data_ptr(), old.numel() * old.element_size()
+                    first = bisect.bisect_left(gather_starts, lo)
+                    pieces, end = [], lo
+                    for dst, ri, size in gathers[first:]:
+                        if dst != end or dst >= lo + nbytes:
+                            break
+                        pieces.append(ri)
+                        end = dst + size
+                    if pieces and end == lo + nbytes:
+                        for ri in pieces:
+                            records[ri][3] += new.data_ptr() - lo
+                        continue
                 if hits:
                     for ri, f in hits:
                         records[ri][f] = new.data_ptr()

@@ -437,6 +437,8 @@ def test_unquantized_sync_hands_out_current_regrouped_qkv():
         for n, w in want.items():
             _same(flat[n], w, n)
         assert upd._plan is not None and upd._plan.replayable
+        if packed:      # q / k / v are assembled in their payload slots: 12 gathering copies, 19 pass-through copies, none twice
+            assert len(upd._plan.batch) == 31
 
 
 def test_packed_buckets_int4_moe_two_syncs(oracle):
