@@ -185,8 +185,23 @@ def convert_qwen3moe_to_hf(args, name, param):
 
 
 def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
+    """Swap the two 64-wide halves along `dim` (size 128).  On the GPU the two halves of every leading index are byte-copy
+    jobs, so a recorded sync repeats the swap on the current weights; elsewhere a torch concatenation."""
     a, b = t.split(64, dim=dim)
-    return torch.cat([b, a], dim=dim)
+    if t.device.type != "cuda" or not t.is_contiguous():
+        return torch.cat([b, a], dim=dim)
+    from miles_amd.weight_update.packed_bucket import submit_copy
+
+    out = torch.empty_like(t)
+    first, second = out.split(64, dim=dim)
+    lead = 1
+    for size in t.shape[:dim]:
+        lead *= size
+    for src, dst in ((b, first), (a, second)):
+        src, dst = src.reshape(lead, -1), dst.reshape(lead, -1)      # views: each leading index owns one contiguous run
+        for i in range(lead):
+            submit_copy(src[i], dst[i])
+    return out
 
 
 def _dsv3_indexer(args, layer: str, rest: str, param: torch.Tensor):

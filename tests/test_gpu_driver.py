@@ -723,3 +723,35 @@ def test_random_moe_models_sync_and_replay(oracle, seed, fmt, packed):
         for k in dev:
             dev[k].copy_(cpu[k])
     assert upd._plan is not None and upd._plan.replayable
+
+
+def test_dsa_indexer_half_rotation_is_replayable():
+    # DeepSeek's DSA indexer with rope interleave swaps the two 64-channel halves of each 128-wide head: copy jobs on the
+    # GPU (the torch concatenation of the CPU path would hand out stale values on replay)
+    from argparse import Namespace
+
+    from miles_amd import launch
+
+    args = Namespace(**vars(ARGS), indexer_rope_interleave=True)
+    g = torch.Generator().manual_seed(91)
+    cpu = {"self_attention.wq_b.weight": torch.randn(4 * 128, 96, generator=g).to(torch.bfloat16),
+           "self_attention.wk.weight": torch.randn(128, 256, generator=g).to(torch.bfloat16),
+           "self_attention.k_norm.weight": torch.randn(128, generator=g).to(torch.bfloat16),
+           "self_attention.k_norm.bias": torch.randn(128, generator=g).to(torch.bfloat16)}
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    name = "module.module.decoder.layers.0."
+    with launch.recording() as batch:
+        got = {k: name_maps.convert_deepseekv3_to_hf(args, name + k, v) for k, v in dev.items()}
+    assert batch.direct_calls == 0 and len(batch) == 2 * 4 + 2 + 2 + 2
+    batch.device = torch.device(DEV)
+    for round_ in range(2):
+        batch.run()
+        torch.cuda.synchronize()
+        for k, v in cpu.items():
+            (want_name, want), = name_maps.convert_deepseekv3_to_hf(args, name + k, v)      # torch path on the CPU
+            (got_name, got_t), = got[k]
+            assert got_name == want_name
+            _same(got_t, want, f"{k} round {round_}")
+        for k in cpu:
+            cpu[k] = (cpu[k].float() * 1.5 + 0.25).to(torch.bfloat16)
+            dev[k].copy_(cpu[k])
