@@ -75,7 +75,7 @@ def _head_dim(args) -> int:
     return kv if kv is not None else args.hidden_size // args.num_attention_heads
 
 
-def _gather_groups(parts: torch.Tensor, shape) -> torch.Tensor:
+def gather_groups(parts: torch.Tensor, shape) -> torch.Tensor:
     """`parts` [groups, ...] is a strided selection of each group's rows (or elements) whose per-group piece is
     contiguous; returns the pieces back to back as a tensor of `shape`.  On the GPU the regrouping is one byte-copy job
     per group instead of a torch copy, so a recorded sync can repeat it on the current weights (a replayed plan hands
@@ -101,7 +101,7 @@ def _split_qkv_weight(args, layer: str, param: torch.Tensor):
         # weight; the FP8 kernel reads the row blocks in place and the regrouping copy disappears
         return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", t.flatten(1, 2))
                 for n, t in (("q", q), ("k", k), ("v", v))]
-    return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", _gather_groups(t, (-1, args.hidden_size)))
+    return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", gather_groups(t, (-1, args.hidden_size)))
             for n, t in (("q", q), ("k", k), ("v", v))]
 
 
@@ -110,7 +110,7 @@ def _split_qkv_bias(args, layer: str, param: torch.Tensor):
     q_per_group = args.num_attention_heads // groups
     hd = _head_dim(args)
     q, k, v = torch.split(param.view(groups, -1), [q_per_group * hd, hd, hd], dim=1)
-    return [(f"model.layers.{layer}.self_attn.{n}_proj.bias", _gather_groups(t, (-1,)))
+    return [(f"model.layers.{layer}.self_attn.{n}_proj.bias", gather_groups(t, (-1,)))
             for n, t in (("q", q), ("k", k), ("v", v))]
 
 

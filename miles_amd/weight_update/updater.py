@@ -17,6 +17,7 @@ from collections.abc import Callable, Mapping
 
 import torch
 
+from miles_amd.megatron_to_hf import name_maps
 from miles_amd.weight_update.bucketing import Unit
 from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorDirect
 from miles_amd.weight_update.packed_bucket import pack_bucket
@@ -100,5 +101,5 @@ class _RowBlockAwareIterator(HfWeightIteratorDirect):
             for unit in units:
                 for i, (name, t) in enumerate(unit):
                     if t.dim() == 3 and name.endswith(("q_proj.weight", "k_proj.weight", "v_proj.weight")):
-                        unit[i] = (name, t.reshape(-1, t.shape[-1]))
+                        unit[i] = (name, name_maps.gather_groups(t, (-1, t.shape[-1])))
         return units

@@ -130,6 +130,15 @@ def test_modules_to_not_convert_keep_bf16_and_2d_shape(oracle):
                                               cpu["module.module.decoder.layers.1.self_attention.linear_qkv.weight"]))
     _same(k1, want["model.layers.1.self_attn.k_proj.weight"], "unquantized k_proj")
     assert flat["model.layers.1.self_attn.q_proj.weight"].dtype == F8
+    # the regrouped bf16 k_proj is produced by copy jobs: the plan is replayed and hands out current values
+    assert upd._plan is not None and upd._plan.replayable
+    cpu2 = _dense_model(21)
+    for k in dev:
+        dev[k].copy_(cpu2[k])
+    flat = dict(nt for b in _run(upd) for nt in b)
+    want = dict(name_maps.convert_qwen2_to_hf(ARGS, "module.module.decoder.layers.1.self_attention.linear_qkv.weight",
+                                              cpu2["module.module.decoder.layers.1.self_attention.linear_qkv.weight"]))
+    _same(flat["model.layers.1.self_attn.k_proj.weight"], want["model.layers.1.self_attn.k_proj.weight"], "k_proj after a step")
 
 
 def _moe_model(seed, experts=4, ffn=128, hidden=256):
