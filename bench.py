@@ -503,8 +503,11 @@ def parity_sample(weights, args, plan):
 
 
 def stream_ceilings():
-    """What plain streaming kernels reach on this GPU at the read : write mixes of the quantizers, measured with torch's own
-    elementwise kernels on 4 GiB operands (no part of the product): the yardstick for the per-quantizer fractions."""
+    """What plain streaming kernels reach on this GPU: torch's own elementwise kernels on 4 GiB operands, and the
+    library's byte-copy job (one 16-byte unit per lane, no loop) on the same buffers: yardsticks for the per-quantizer
+    fractions."""
+    from miles_amd.weight_update.packed_bucket import submit_copy
+
     n = 1 << 31
     x = torch.empty(n, dtype=torch.bfloat16, device=DEV).normal_()
     y = torch.empty(n, dtype=torch.bfloat16, device=DEV)
@@ -512,6 +515,7 @@ def stream_ceilings():
     res = {}
     for name, fn, nbytes in (("fill_write_only", lambda: y.fill_(1.0), 2 * n),
                              ("copy_bf16_1r_1w", lambda: y.copy_(x), 4 * n),
+                             ("library_copy_job_1r_1w", lambda: submit_copy(x, y), 4 * n),
                              ("cast_bf16_to_fp8_2r_1w", lambda: q.copy_(x), 3 * n),
                              ("cast_fp8_to_bf16_1r_2w", lambda: y.copy_(q), 3 * n)):
         fn()
