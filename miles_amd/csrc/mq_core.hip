@@ -31,11 +31,6 @@ __global__ void fill_u32_n_kernel(uint32_t* p, uint32_t v, int64_t n) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) p[i] = v;
 }
-__global__ __launch_bounds__(256) void copy16_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, int64_t n16) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (; i < n16; i += stride) dst[i] = src[i];
-}
 // Grouped byte copies: a workgroup moves one 16 KiB chunk (four 16-byte units per lane) of one of up to 64 runs.
 // Runs whose pointers are 16-byte aligned use 16-byte accesses with a byte tail; the others go byte by byte.
 constexpr int kCopyUnits = 4;
@@ -110,10 +105,5 @@ extern "C" int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* s
     if (!src || !dst || nbytes < 0 || (nbytes % 16) || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16))
         return mq_fail(MQ_ERR_ARG, "copy needs 16-byte aligned pointers and size");
     if (nbytes == 0) return MQ_OK;
-    const int64_t n16 = nbytes / 16;
-    int64_t blocks = (n16 + 255) / 256;
-    if (blocks > 256 * 32) blocks = 256 * 32;
-    hipLaunchKernelGGL(mq::copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const mq::u32x4*)src, (mq::u32x4*)dst, n16);
-    return mq_check_launch("copy");
+    return mq_copy_launch_run(src, dst, nbytes, (hipStream_t)stream);
 }
