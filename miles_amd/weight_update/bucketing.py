@@ -35,53 +35,82 @@ def _validate(groups: list[AtomicUpdateGroup]) -> None:
     assert len(set(keys)) == len(keys), f"Duplicate atomic update group keys: {keys}"
 
 
+class _PendingGroups:
+    """Members of atomic groups seen so far, keyed by (name prefix, group key), until their group is complete."""
+
+    def __init__(self, groups: list[AtomicUpdateGroup]) -> None:
+        self.groups = groups
+        self.open: dict[tuple[str, str], list[Unit | None]] = {}
+        self.matched: set[str] = set()
+
+    def locate(self, unit: Unit):
+        """(group, member index, name prefix) of the one suffix this unit's names end in, or None."""
+        found = []
+        for name, _tensor in unit:
+            for group in self.groups:
+                for index, suffix in enumerate(group.suffixes):
+                    if name.endswith(suffix):
+                        found.append((group, index, name[: len(name) - len(suffix)]))
+        assert len(found) <= 1, f"Unit {[n for n, _ in unit]} matches multiple atomic group suffixes"
+        return found[0] if found else None
+
+    def place(self, unit: Unit, group: AtomicUpdateGroup, index: int, prefix: str) -> Unit | None:
+        """Store the member; the merged unit (members in suffix order) once the last one is in."""
+        self.matched.add(group.key)
+        key = (prefix, group.key)
+        members = self.open.setdefault(key, [None] * len(group.suffixes))
+        assert members[index] is None, f"Duplicate member in atomic update group: {prefix}{group.suffixes[index]}"
+        members[index] = unit
+        if any(m is None for m in members):
+            return None
+        del self.open[key]
+        merged: Unit = []
+        for member in members:
+            merged.extend(member)
+        return merged
+
+    def finish(self) -> None:
+        assert not self.open, f"Incomplete atomic update groups at end of stream: {sorted(self.open)}"
+        for group in self.groups:
+            assert group.optional or group.key in self.matched, \
+                f"Atomic update group {group.key} matched no params (suffixes {group.suffixes})"
+
+
 def assemble_atomic_update_groups(hf_param_units: Iterable[Unit],
                                   atomic_update_groups: list[AtomicUpdateGroup]) -> Iterator[Unit]:
     """Merge the units whose members end in a group's suffixes into one unit per name prefix (members in
     suffix order, each member's other tensors -- its scales -- riding along); pass other units through."""
     _validate(atomic_update_groups)
-    waiting: dict[tuple[str, str], list[Unit | None]] = {}
-    seen_keys: set[str] = set()
+    pending = _PendingGroups(atomic_update_groups)
     for unit in hf_param_units:
         if not unit:
             continue
-        hits = [(g, idx, name[: -len(suffix)])
-                for name, _t in unit
-                for g in atomic_update_groups
-                for idx, suffix in enumerate(g.suffixes)
-                if name.endswith(suffix)]
-        assert len(hits) <= 1, f"Unit {[n for n, _ in unit]} matches multiple atomic group suffixes"
-        if not hits:
+        where = pending.locate(unit)
+        if where is None:
             yield unit
             continue
-        group, idx, prefix = hits[0]
-        seen_keys.add(group.key)
-        slots = waiting.setdefault((prefix, group.key), [None] * len(group.suffixes))
-        assert slots[idx] is None, f"Duplicate member in atomic update group: {prefix}{group.suffixes[idx]}"
-        slots[idx] = unit
-        if all(s is not None for s in slots):
-            del waiting[(prefix, group.key)]
-            yield [named for member in slots for named in member]
-    assert not waiting, f"Incomplete atomic update groups at end of stream: {sorted(waiting)}"
-    for g in atomic_update_groups:
-        assert g.optional or g.key in seen_keys, \
-            f"Atomic update group {g.key} matched no params (suffixes {g.suffixes})"
+        merged = pending.place(unit, *where)
+        if merged is not None:
+            yield merged
+    pending.finish()
 
 
 def pack_units_by_size(hf_param_units: Iterable[Unit], max_bytes: int) -> Iterator[Unit]:
     """Greedy buckets: a bucket closes when adding the next unit would reach `max_bytes`; a unit larger
     than `max_bytes` gets a bucket of its own."""
-    bucket: Unit = []
-    size = 0
+    open_bucket: Unit = []
+    held = 0
     for unit in hf_param_units:
-        unit_bytes = sum(t.nbytes for _n, t in unit)
-        if bucket and size + unit_bytes >= max_bytes:
-            yield bucket
-            bucket, size = [], 0
-        bucket.extend(unit)
-        size += unit_bytes
-    if bucket:
-        yield bucket
+        incoming = 0
+        for _name, tensor in unit:
+            incoming += tensor.nbytes
+        if open_bucket and held + incoming >= max_bytes:
+            yield open_bucket
+            open_bucket, held = [], 0
+        open_bucket += unit
+        held += incoming
+    if open_bucket:
+        yield open_bucket
 
 
 # ---- per-model atomic groups --------------------------------------------------------------------------
