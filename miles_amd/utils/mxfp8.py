@@ -14,28 +14,30 @@ from miles_amd import _lib, launch
 
 MXFP8_GROUP_SIZE = 32
 
-MXFP8_SKIP_WEIGHT_SUBSTRINGS = (
-    "layernorm", "embed", "router", "mlp.gate.", "norm", "lm_head", "eh_proj", "weights_proj", "head.", "wo_a",
-    "ffn.gate.", "compressor.",
-)
+# name fragments of tensors that stay in high precision whatever their shape
+MXFP8_SKIP_WEIGHT_SUBSTRINGS = tuple(
+    "layernorm embed router mlp.gate. norm lm_head eh_proj weights_proj head. wo_a ffn.gate. compressor.".split())
 
-MXFP8_SOURCE_FP8_DTYPES = (torch.float8_e4m3fn,) + (
-    (torch.float8_e4m3fnuz,) if hasattr(torch, "float8_e4m3fnuz") else ()
-)
+MXFP8_SOURCE_FP8_DTYPES = tuple(getattr(torch, n) for n in ("float8_e4m3fn", "float8_e4m3fnuz") if hasattr(torch, n))
+
+_HIGH_PRECISION_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
 
 
 def should_use_mxfp8(name: str, shape: tuple[int, ...], dtype: torch.dtype, *,
                      skip_substrings: tuple[str, ...] = MXFP8_SKIP_WEIGHT_SUBSTRINGS,
                      allow_source_fp8: bool = False, packed_mxfp4_experts: bool = False) -> bool:
-    """Whether a checkpoint tensor is stored as MXFP8 in the rollout layout."""
-    if not name.endswith(".weight"):
+    """Whether a checkpoint tensor is stored as MXFP8 in the rollout layout: a `.weight` matrix outside the skip list
+    whose last dimension splits into 1x32 groups (for packed MXFP4 experts the stored byte holds two weights, and the
+    dtype is not looked at); FP8 sources only count when the caller re-scales them."""
+    is_matrix_weight = name.endswith(".weight") and len(shape) >= 2
+    if not is_matrix_weight or any(fragment in name for fragment in skip_substrings):
         return False
-    if any(s in name for s in skip_substrings) or len(shape) < 2:
+    width = shape[-1] * (2 if packed_mxfp4_experts else 1)
+    if width % MXFP8_GROUP_SIZE:
         return False
     if packed_mxfp4_experts:
-        return (2 * shape[-1]) % MXFP8_GROUP_SIZE == 0  # two e2m1 weights per stored byte
-    ok_dtypes = (torch.float16, torch.bfloat16, torch.float32) + (MXFP8_SOURCE_FP8_DTYPES if allow_source_fp8 else ())
-    return dtype in ok_dtypes and shape[-1] % MXFP8_GROUP_SIZE == 0
+        return True
+    return dtype in _HIGH_PRECISION_DTYPES or (allow_source_fp8 and dtype in MXFP8_SOURCE_FP8_DTYPES)
 
 
 def mxfp8_quantize(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
