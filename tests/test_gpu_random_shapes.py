@@ -7,6 +7,7 @@ fp32 inputs, and values spread over many binades.  Everything is deterministic: 
 fixed seed at collection time.
 """
 
+import os
 import random
 
 import pytest
@@ -43,10 +44,14 @@ def _tensor(seed, shape, dtype, offset):
     return x, flat[offset:].view(shape)
 
 
+# MQ_RANDOM_SCALE=10 runs ten times as many random cases (the extra ones continue the same seeded sequence)
+_SCALE = max(1, int(os.environ.get("MQ_RANDOM_SCALE", "1")))
+
+
 def _cases(name, count, columns_multiple_of, max_rows=300, max_cols=1100):
     rng = random.Random(f"miles-quant-{name}")
     out = []
-    for i in range(count):
+    for i in range(count * _SCALE):
         rows = rng.choice([1, 2, 3, 5, 31, 64, 127, 128, 129, 200, rng.randint(1, max_rows)])
         cols = columns_multiple_of * rng.randint(1, max(1, max_cols // columns_multiple_of))
         dtype = rng.choice(_DTYPES)
@@ -313,7 +318,7 @@ def _same_any(got, want, what):
 
 @pytest.mark.parametrize("non_finite", [False, True], ids=["finite", "nonfinite"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(4 * _SCALE))
 def test_random_special_values(oracle, monkeypatch, seed, dtype, non_finite):
     from miles_amd.kernels.quant import fake_quant as fq
     from miles_amd.kernels.quant.fp8_act_quant import act_quant, fp8_simulate
@@ -328,7 +333,7 @@ def test_random_special_values(oracle, monkeypatch, seed, dtype, non_finite):
 
     for name in ("NVTE_USE_FAST_MATH", "NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256"):
         monkeypatch.delenv(name, raising=False)
-    shape = [(136, 384), (64, 1024), (8, 256), (200, 128)][seed]
+    shape = [(136, 384), (64, 1024), (8, 256), (200, 128)][seed % 4]
     x = _special_tensor(7000 + seed, shape, dtype, non_finite)
     xd = x.to(DEV)
     failures = []
