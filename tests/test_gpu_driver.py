@@ -1,6 +1,7 @@
 """End-to-end sync driver on the GPU: Megatron-named parameters -> WeightUpdater -> buckets of quantized HF
 tensors, compared tensor by tensor with the oracle applied to the HF tensors the name maps produce."""
 
+import os
 from argparse import Namespace
 
 import pytest
@@ -15,6 +16,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 F8 = torch.float8_e4m3fn
 
+_SCALE = max(1, int(os.environ.get("MQ_RANDOM_SCALE", "1")))     # multiplies the seeded random model cases
 ARGS = Namespace(hidden_size=256, num_attention_heads=4, num_query_groups=2, kv_channels=128, vocab_size=1000,
                  num_layers=2, update_weight_buffer_size=1 << 20, q_lora_rank=None)
 FP8_CFG = {"quant_method": "fp8", "fmt": "e4m3", "activation_scheme": "dynamic", "weight_block_size": [128, 128]}
@@ -601,7 +603,7 @@ def _random_dense_case(seed):
     return args, p
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(10 * _SCALE))
 @pytest.mark.parametrize("packed", [False, True])
 def test_random_dense_models_sync_and_replay(oracle, seed, packed):
     args, cpu = _random_dense_case(seed)
@@ -698,7 +700,7 @@ def _moe_expected(oracle, fmt, args, params, basenames):
     return want
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(6 * _SCALE))
 @pytest.mark.parametrize("fmt", ["mxfp8", "nvfp4", "int4"])
 @pytest.mark.parametrize("packed", [False, True])
 def test_random_moe_models_sync_and_replay(oracle, seed, fmt, packed):
