@@ -50,3 +50,23 @@ def test_wrappers_refuse_cpu_tensors():
                      (nvfp4_quantize_1d, (w,))]:
         with pytest.raises(_lib.MilesQuantError, match="GPU"):
             fn(*args)
+
+
+def test_python_constants_match_the_header():
+    """Job kinds, flags and record sizes are written down twice (C header, ctypes side): they must agree."""
+    from miles_amd import _lib
+    from miles_amd.tools.convert_hf_to_fp8 import _AMAX_RECORD_WORDS
+    from miles_amd.utils.nvfp4 import AMAX_RECORD_WORDS
+
+    text = open(os.path.join(ROOT, "include", "miles_quant.h")).read()
+    enums = {name: int(value) for name, value in re.findall(r"\b(MQ_[A-Z0-9_]+)\s*=\s*(\d+)", text)}
+    defines = {name: value for name, value in re.findall(r"#define\s+(MQ_[A-Z0-9_]+)\s+(\S.*)", text)}
+    kinds = {k[len("MQ_JOB_"):]: v for k, v in enums.items() if k.startswith("MQ_JOB_")}
+    assert kinds and all(getattr(_lib, "JOB_" + k) == v for k, v in kinds.items())
+    assert len(kinds) == len({getattr(_lib, n) for n in dir(_lib) if n.startswith("JOB_")})
+    for name in ("NVFP4_4OVER6", "NVFP4_ERR_MSE", "NVFP4_ERR_FP16", "NVFP4_CARRY_AMAX"):
+        assert getattr(_lib, name) == enums["MQ_" + name]
+    assert _lib.MAX_GROUP == int(defines["MQ_MAX_GROUP"])
+    words = int(defines["MQ_NVFP4_SECTION_WORDS"]) * (int(defines["MQ_NVFP4_SECTIONS"]) + 1)
+    assert AMAX_RECORD_WORDS == _AMAX_RECORD_WORDS == words
+    assert (_lib.MQ_BF16, _lib.MQ_F16, _lib.MQ_F32) == (enums["MQ_BF16"], enums["MQ_F16"], enums["MQ_F32"])
