@@ -2,15 +2,19 @@
 
 from __future__ import annotations
 
-from .name_maps import convert_deepseekv3_to_hf, convert_qwen2_to_hf, convert_qwen3moe_to_hf
+from .name_maps import (convert_deepseekv3_to_hf, convert_glm4_to_hf, convert_llama_to_hf, convert_qwen2_to_hf,
+                        convert_qwen3moe_to_hf)
 from .processors import quantize_params, remove_padding
 
 # substring of the lower-cased model name -> converter; first match wins, order as in the reference's
 # _convert_to_hf_core (megatron_to_hf/__init__.py:37-83) for the families implemented here
 _CONVERTERS = (
     (("glm4moelite", "deepseekv3", "glmmoedsa", "glm_moe_dsa", "kimi_k2", "kimik2"), convert_deepseekv3_to_hf),
+    (("glm4moe",), None),          # GLM-4 MoE has a map of its own in the reference; not built here
+    (("glm4",), convert_glm4_to_hf),
     (("qwen3moe",), convert_qwen3moe_to_hf),
     (("qwen2", "qwen3"), convert_qwen2_to_hf),
+    (("llama",), convert_llama_to_hf),
 )
 
 
@@ -18,6 +22,8 @@ def _convert_to_hf_core(args, model_name, name, param):
     lowered = model_name.lower()
     for keys, fn in _CONVERTERS:
         if any(k in lowered for k in keys):
+            if fn is None:
+                break
             return fn(args, name, param)
     raise ValueError(f"Unsupported model: {lowered}")
 

@@ -170,6 +170,42 @@ def convert_qwen2_to_hf(args, name, param):
     raise ValueError(f"Unknown parameter name: {name}")
 
 
+# Llama (reference: megatron_to_hf/llama.py:5-53): the dense layer without q / k norms, biases or a separate
+# input_layernorm entry.  GLM-4 (reference: megatron_to_hf/glm4.py): gate and up stay fused as gate_up_proj, q / k / v
+# biases exist, and the two sandwich norms keep their Megatron names.
+_LLAMA_RENAMES = dict(_COMMON_RENAMES)
+_GLM4_RENAMES = {
+    "self_attention.linear_proj.weight": "self_attn.o_proj.weight",
+    "mlp.linear_fc2.weight": "mlp.down_proj.weight",
+    "mlp.linear_fc1.weight": "mlp.gate_up_proj.weight",
+    "self_attention.linear_qkv.layer_norm_weight": "input_layernorm.weight",
+    "mlp.linear_fc1.layer_norm_weight": "post_attention_layernorm.weight",
+    "self_attention.q_layernorm.weight": "self_attn.q_norm.weight",
+    "self_attention.k_layernorm.weight": "self_attn.k_norm.weight",
+    "post_self_attn_layernorm.weight": "post_self_attn_layernorm.weight",
+    "post_mlp_layernorm.weight": "post_mlp_layernorm.weight",
+}
+
+
+def _convert_dense_family(args, name, param, renames, *, qkv_bias: bool):
+    if name in _TOP_LEVEL:
+        return [(_TOP_LEVEL[name], param)]
+    m = _DECODER.match(name)
+    if m and (qkv_bias or m.group(2) != "self_attention.linear_qkv.bias"):
+        out = _dense_layer(args, m.group(1), m.group(2), param, renames)
+        if out is not None:
+            return out
+    raise ValueError(f"Unknown parameter name: {name}")
+
+
+def convert_llama_to_hf(args, name, param):
+    return _convert_dense_family(args, name, param, _LLAMA_RENAMES, qkv_bias=False)
+
+
+def convert_glm4_to_hf(args, name, param):
+    return _convert_dense_family(args, name, param, _GLM4_RENAMES, qkv_bias=True)
+
+
 def convert_qwen3moe_to_hf(args, name, param):
     if name in _TOP_LEVEL:
         return [(_TOP_LEVEL[name], param)]

@@ -119,6 +119,82 @@ def test_dense_fp8_sync_matches_oracle_and_replays(oracle, use_plan):
         _same(g, w, n + " (new storage)")
 
 
+def _family_model(family, seed):
+    """The dense model above renamed for another family: Llama has no q/k norms and names the second norm
+    `pre_mlp_layernorm`; GLM-4 adds a norm after attention and after the MLP and a bias on the fused q/k/v."""
+    p = _dense_model(seed)
+    for layer in range(2):
+        L = f"module.module.decoder.layers.{layer}."
+        if family == "llama":
+            del p[L + "self_attention.q_layernorm.weight"], p[L + "self_attention.k_layernorm.weight"]
+            p[L + "pre_mlp_layernorm.weight"] = p.pop(L + "mlp.linear_fc1.layer_norm_weight")
+        else:
+            p[L + "self_attention.linear_qkv.bias"] = W.gaussian_outliers((1024,), std=0.02, p_outlier=0.0, gain=1.0, seed=seed + 90 + layer)
+            p[L + "post_self_attn_layernorm.weight"] = W.gaussian_outliers((256,), std=0.02, p_outlier=0.0, gain=1.0, seed=seed + 70 + layer)
+            p[L + "post_mlp_layernorm.weight"] = W.gaussian_outliers((256,), std=0.02, p_outlier=0.0, gain=1.0, seed=seed + 80 + layer)
+    return p
+
+
+def _family_expected(oracle, family, cpu):
+    """HF names written out by hand (megatron_to_hf/llama.py:6-44, glm4.py:6-60), weights of *_proj cast per tile."""
+    out = []
+
+    def emit(name, t):
+        if name.endswith("_proj.weight"):
+            q, s = oracle.fp8_blockwise_cast(t.contiguous())
+            out.extend([(name, q), (name.replace(".weight", ".weight_scale_inv"), s)])
+        else:
+            out.append((name, t))
+
+    def qkv(t):
+        g = t.view(2, 4, 128, *t.shape[1:])
+        return g[:, :2].reshape(512, *t.shape[1:]), g[:, 2].reshape(256, *t.shape[1:]), g[:, 3].reshape(256, *t.shape[1:])
+
+    for name, t in cpu.items():
+        if "decoder.layers." not in name:
+            hf = {"embedding.word_embeddings.weight": "model.embed_tokens.weight", "output_layer.weight": "lm_head.weight",
+                  "decoder.final_layernorm.weight": "model.norm.weight"}[name[len("module.module."):]]
+            emit(hf, t[:1000] if t.dim() == 2 else t)
+            continue
+        layer, rest = name[len("module.module.decoder.layers."):].split(".", 1)
+        H = f"model.layers.{layer}."
+        if rest in ("self_attention.linear_qkv.weight", "self_attention.linear_qkv.bias"):
+            for proj, part in zip("qkv", qkv(t)):
+                emit(f"{H}self_attn.{proj}_proj.{rest.rsplit('.', 1)[1]}", part)
+        elif rest == "mlp.linear_fc1.weight" and family == "llama":
+            emit(H + "mlp.gate_proj.weight", t[:384])
+            emit(H + "mlp.up_proj.weight", t[384:])
+        else:
+            emit(H + {"mlp.linear_fc1.weight": "mlp.gate_up_proj.weight", "mlp.linear_fc2.weight": "mlp.down_proj.weight",
+                      "self_attention.linear_proj.weight": "self_attn.o_proj.weight",
+                      "self_attention.linear_qkv.layer_norm_weight": "input_layernorm.weight",
+                      "mlp.linear_fc1.layer_norm_weight": "post_attention_layernorm.weight",
+                      "pre_mlp_layernorm.weight": "post_attention_layernorm.weight",
+                      "self_attention.q_layernorm.weight": "self_attn.q_norm.weight",
+                      "self_attention.k_layernorm.weight": "self_attn.k_norm.weight",
+                      "post_self_attn_layernorm.weight": "post_self_attn_layernorm.weight",
+                      "post_mlp_layernorm.weight": "post_mlp_layernorm.weight"}[rest], t)
+    return out
+
+
+@pytest.mark.parametrize("family,model_name", [("llama", "Llama-3.1-8B"), ("glm4", "glm4")])
+def test_llama_and_glm4_fp8_sync_and_replay(oracle, family, model_name):
+    cpu = _family_model(family, 40)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name=model_name, quantization_config=FP8_CFG, send_bucket=None)
+    for sync, seed in enumerate((40, 41, 42)):
+        if sync:
+            cpu = _family_model(family, seed)
+            for k in dev:
+                dev[k].copy_(cpu[k])
+        flat = [nt for b in _run(upd) for nt in b]
+        want = _family_expected(oracle, family, cpu)
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{family} sync {sync}: {n}")
+    assert upd._plan is not None and upd._plan.replayable
+
+
 def test_modules_to_not_convert_keep_bf16_and_2d_shape(oracle):
     cpu = _dense_model(20)
     dev = {k: v.to(DEV) for k, v in cpu.items()}

@@ -426,3 +426,49 @@ def test_nvfp4_fake_qat_switch_on_reads_the_configuration_once(monkeypatch):
     assert len(reads) == 1 and len(out) == 3
     assert all(o is i for o, i in zip(out, images))
     assert all(w is got_w and c is config for w, (got_w, c) in zip(weights, seen))
+
+
+# ---------------------------------------------------------------------------------------------------
+# Llama and GLM-4 dense name maps (megatron_to_hf/llama.py, glm4.py)
+def test_llama_and_glm4_name_maps():
+    from argparse import Namespace
+
+    from miles_amd.megatron_to_hf import convert_to_hf, name_maps
+
+    args = Namespace(hidden_size=64, num_attention_heads=4, num_query_groups=2, kv_channels=16, vocab_size=100)
+    L = "module.module.decoder.layers.3."
+    qkv = torch.arange(2 * (2 + 1 + 1) * 16 * 64, dtype=torch.float32).reshape(-1, 64)
+    fc1 = torch.arange(2 * 24 * 64, dtype=torch.float32).reshape(48, 64)
+
+    names = lambda out: [n for n, _ in out]
+    llama = name_maps.convert_llama_to_hf
+    assert names(llama(args, L + "self_attention.linear_qkv.weight", qkv)) == [
+        f"model.layers.3.self_attn.{p}_proj.weight" for p in "qkv"]
+    q, k, v = (t for _, t in llama(args, L + "self_attention.linear_qkv.weight", qkv))
+    grouped = qkv.view(2, 4, 16, 64)
+    assert torch.equal(q, grouped[:, :2].reshape(-1, 64)) and torch.equal(k, grouped[:, 2].reshape(-1, 64))
+    assert torch.equal(v, grouped[:, 3].reshape(-1, 64))
+    gate_up = llama(args, L + "mlp.linear_fc1.weight", fc1)
+    assert names(gate_up) == ["model.layers.3.mlp.gate_proj.weight", "model.layers.3.mlp.up_proj.weight"]
+    assert torch.equal(gate_up[0][1], fc1[:24]) and torch.equal(gate_up[1][1], fc1[24:])
+    assert names(llama(args, L + "pre_mlp_layernorm.weight", fc1[0])) == ["model.layers.3.post_attention_layernorm.weight"]
+    assert names(llama(args, "module.module.output_layer.weight", fc1)) == ["lm_head.weight"]
+    for unknown in ("self_attention.linear_qkv.bias", "self_attention.q_layernorm.weight", "input_layernorm.weight"):
+        with pytest.raises(ValueError, match="Unknown parameter name"):
+            llama(args, L + unknown, fc1[0])
+
+    glm4 = name_maps.convert_glm4_to_hf
+    fused = glm4(args, L + "mlp.linear_fc1.weight", fc1)
+    assert names(fused) == ["model.layers.3.mlp.gate_up_proj.weight"] and fused[0][1] is fc1      # gate and up stay fused
+    assert names(glm4(args, L + "post_self_attn_layernorm.weight", fc1[0])) == ["model.layers.3.post_self_attn_layernorm.weight"]
+    assert names(glm4(args, L + "post_mlp_layernorm.weight", fc1[0])) == ["model.layers.3.post_mlp_layernorm.weight"]
+    assert names(glm4(args, L + "self_attention.linear_qkv.bias", torch.arange(128.0))) == [
+        f"model.layers.3.self_attn.{p}_proj.bias" for p in "qkv"]
+    with pytest.raises(ValueError, match="Unknown parameter name"):
+        glm4(args, L + "pre_mlp_layernorm.weight", fc1[0])
+
+    # dispatch by model name: glm4 before qwen*, llama last; GLM-4 MoE is a different map and is refused, not mis-mapped
+    assert names(convert_to_hf(args, "Llama-3.1-8B", L + "mlp.linear_fc2.weight", fc1)) == ["model.layers.3.mlp.down_proj.weight"]
+    assert names(convert_to_hf(args, "glm4", L + "mlp.linear_fc1.weight", fc1)) == ["model.layers.3.mlp.gate_up_proj.weight"]
+    with pytest.raises(ValueError, match="Unsupported model"):
+        convert_to_hf(args, "glm4moe", L + "mlp.linear_fc1.weight", fc1)
