@@ -2,17 +2,20 @@
 
 from __future__ import annotations
 
-from .name_maps import (convert_deepseekv3_to_hf, convert_glm4_to_hf, convert_llama_to_hf, convert_qwen2_to_hf,
-                        convert_qwen3moe_to_hf)
+from .name_maps import (convert_deepseekv3_to_hf, convert_glm4_to_hf, convert_glm4moe_to_hf, convert_llama_to_hf,
+                        convert_qwen2_to_hf, convert_qwen3moe_to_hf)
 from .processors import quantize_params, remove_padding
 
 # substring of the lower-cased model name -> converter; first match wins, order as in the reference's
-# _convert_to_hf_core (megatron_to_hf/__init__.py:37-83) for the families implemented here
+# _convert_to_hf_core (megatron_to_hf/__init__.py:37-83).  A family whose map is not built here keeps its place in the
+# order with None, so that its name is refused and not taken by a later, shorter key ("qwen3next" contains "qwen3").
 _CONVERTERS = (
+    (("glm5_next", "glm5next"), None),
     (("glm4moelite", "deepseekv3", "glmmoedsa", "glm_moe_dsa", "kimi_k2", "kimik2"), convert_deepseekv3_to_hf),
-    (("glm4moe",), None),          # GLM-4 MoE has a map of its own in the reference; not built here
+    (("glm4moe",), convert_glm4moe_to_hf),
     (("glm4",), convert_glm4_to_hf),
     (("qwen3moe",), convert_qwen3moe_to_hf),
+    (("qwen3next", "qwen3_8_next", "qwen4_exp", "qwen3.8_next", "qwen3_5", "qwen3_6"), None),
     (("qwen2", "qwen3"), convert_qwen2_to_hf),
     (("llama",), convert_llama_to_hf),
 )

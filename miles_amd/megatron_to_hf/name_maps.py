@@ -220,6 +220,48 @@ def convert_qwen3moe_to_hf(args, name, param):
     raise ValueError(f"Unknown parameter name: {name}")
 
 
+def _mtp_layer(args, name: str, param: torch.Tensor, convert):
+    """A multi-token-prediction layer is numbered after the decoder layers; its own four tensors are renamed here, the
+    transformer layer inside it goes back through `convert` under that number."""
+    m = _MTP.match(name)
+    if not m:
+        return None
+    layer = int(m.group(1)) + args.num_layers
+    rest = m.group(2)
+    direct = {"eh_proj.weight": "eh_proj.weight", "enorm.weight": "enorm.weight", "hnorm.weight": "hnorm.weight",
+              "final_layernorm.weight": "shared_head.norm.weight"}
+    if rest in direct:
+        return [(f"model.layers.{layer}.{direct[rest]}", param)]
+    inner = f"module.module.decoder.layers.{layer}.{rest}".replace("transformer_layer.", "").replace("mtp_model_layer.", "")
+    return convert(args, inner, param)
+
+
+_GLM4MOE_RENAMES = {
+    **_QWEN3MOE_RENAMES,
+    "post_self_attn_layernorm.weight": "post_self_attn_layernorm.weight",
+    "post_mlp_layernorm.weight": "post_mlp_layernorm.weight",
+}
+
+
+def convert_glm4moe_to_hf(args, name, param):
+    """GLM-4 MoE (reference: megatron_to_hf/glm4moe.py:6-139): routed and shared experts split into gate / up / down,
+    q / k / v regrouped, the norms after attention and after the MLP kept, MTP layers numbered after the decoder's."""
+    if name in _TOP_LEVEL:
+        return [(_TOP_LEVEL[name], param)]
+    m = _DECODER.match(name)
+    if m:
+        layer, rest = m.groups()
+        out = (_routed_expert(name, layer, rest, param)
+               or _shared_expert(name, layer, rest, param, "shared_experts", gate_key=False)
+               or _dense_layer(args, layer, rest, param, _GLM4MOE_RENAMES))
+        if out is not None:
+            return out
+    out = _mtp_layer(args, name, param, convert_glm4moe_to_hf)
+    if out is not None:
+        return out
+    raise ValueError(f"Unknown parameter name: {name}")
+
+
 def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
     """Swap the two 64-wide halves along `dim` (size 128).  On the GPU the two halves of every leading index are byte-copy
     jobs, so a recorded sync repeats the swap on the current weights; elsewhere a torch concatenation."""
@@ -275,15 +317,7 @@ def convert_deepseekv3_to_hf(args, name, param):
             out = _dense_layer(args, layer, rest, param, _DSV3_RENAMES)
         if out is not None:
             return out
-    m = _MTP.match(name)
-    if m:
-        layer = int(m.group(1)) + args.num_layers
-        rest = m.group(2)
-        direct = {"eh_proj.weight": "eh_proj.weight", "enorm.weight": "enorm.weight", "hnorm.weight": "hnorm.weight",
-                  "final_layernorm.weight": "shared_head.norm.weight"}
-        if rest in direct:
-            return [(f"model.layers.{layer}.{direct[rest]}", param)]
-        inner = f"module.module.decoder.layers.{layer}.{rest}".replace("transformer_layer.", "").replace(
-            "mtp_model_layer.", "")
-        return convert_deepseekv3_to_hf(args, inner, param)
+    out = _mtp_layer(args, name, param, convert_deepseekv3_to_hf)
+    if out is not None:
+        return out
     raise ValueError(f"Unknown parameter name: {name}")

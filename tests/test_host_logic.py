@@ -470,5 +470,40 @@ def test_llama_and_glm4_name_maps():
     # dispatch by model name: glm4 before qwen*, llama last; GLM-4 MoE is a different map and is refused, not mis-mapped
     assert names(convert_to_hf(args, "Llama-3.1-8B", L + "mlp.linear_fc2.weight", fc1)) == ["model.layers.3.mlp.down_proj.weight"]
     assert names(convert_to_hf(args, "glm4", L + "mlp.linear_fc1.weight", fc1)) == ["model.layers.3.mlp.gate_up_proj.weight"]
-    with pytest.raises(ValueError, match="Unsupported model"):
-        convert_to_hf(args, "glm4moe", L + "mlp.linear_fc1.weight", fc1)
+    for other_family in ("qwen3next", "Qwen3_5-MoE", "glm5_next", "mimo"):      # maps not built here: refused, never mis-mapped
+        with pytest.raises(ValueError, match="Unsupported model"):
+            convert_to_hf(args, other_family, L + "mlp.linear_fc1.weight", fc1)
+
+
+def test_glm4moe_name_map():
+    from argparse import Namespace
+
+    from miles_amd.megatron_to_hf import convert_to_hf
+
+    args = Namespace(hidden_size=64, num_attention_heads=4, num_query_groups=2, kv_channels=16, vocab_size=100, num_layers=5)
+    names = lambda name, t: [n for n, _ in convert_to_hf(args, "glm4moe", name, t)]
+    L = "module.module.decoder.layers.2."
+    w = torch.arange(48 * 64, dtype=torch.float32).reshape(48, 64)
+    assert names(L + "mlp.experts.linear_fc1.weight7", w) == [
+        "model.layers.2.mlp.experts.7.gate_proj.weight", "model.layers.2.mlp.experts.7.up_proj.weight"]
+    assert names(L + "mlp.experts.linear_fc2.weight7", w) == ["model.layers.2.mlp.experts.7.down_proj.weight"]
+    assert names(L + "mlp.shared_experts.linear_fc1.weight", w) == [
+        "model.layers.2.mlp.shared_experts.gate_proj.weight", "model.layers.2.mlp.shared_experts.up_proj.weight"]
+    assert names(L + "mlp.shared_experts.linear_fc2.weight", w) == ["model.layers.2.mlp.shared_experts.down_proj.weight"]
+    assert names(L + "mlp.router.weight", w) == ["model.layers.2.mlp.gate.weight"]
+    assert names(L + "mlp.router.expert_bias", w[0]) == ["model.layers.2.mlp.gate.e_score_correction_bias"]
+    assert names(L + "post_self_attn_layernorm.weight", w[0]) == ["model.layers.2.post_self_attn_layernorm.weight"]
+    assert names(L + "post_mlp_layernorm.weight", w[0]) == ["model.layers.2.post_mlp_layernorm.weight"]
+    assert names(L + "mlp.linear_fc1.weight", w) == ["model.layers.2.mlp.gate_proj.weight", "model.layers.2.mlp.up_proj.weight"]
+    assert names(L + "self_attention.linear_qkv.bias", torch.arange(128.0)) == [
+        f"model.layers.2.self_attn.{p}_proj.bias" for p in "qkv"]
+    # MTP layers come after the decoder's, and the transformer layer inside one goes through the same map
+    M = "module.module.mtp.layers.1."
+    assert names(M + "eh_proj.weight", w) == ["model.layers.6.eh_proj.weight"]
+    assert names(M + "final_layernorm.weight", w[0]) == ["model.layers.6.shared_head.norm.weight"]
+    assert names(M + "transformer_layer.mlp.experts.linear_fc2.weight3", w) == ["model.layers.6.mlp.experts.3.down_proj.weight"]
+    assert names(M + "transformer_layer.self_attention.linear_proj.weight", w) == ["model.layers.6.self_attn.o_proj.weight"]
+    for bad in (L + "mlp.shared_experts.gate_weight", L + "mlp.experts.linear_fc3.weight0", L + "input_layernorm.weight",
+                "module.module.unknown.weight"):
+        with pytest.raises(ValueError, match="Unknown"):
+            names(bad, w)
