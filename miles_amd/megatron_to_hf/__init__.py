@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 from .name_maps import (convert_deepseekv3_to_hf, convert_glm4_to_hf, convert_glm4moe_to_hf, convert_llama_to_hf,
-                        convert_qwen2_to_hf, convert_qwen3moe_to_hf)
+                        convert_mimo_to_hf, convert_qwen2_to_hf, convert_qwen3moe_to_hf)
 from .processors import quantize_params, remove_padding
 
 # substring of the lower-cased model name -> converter; first match wins, order as in the reference's
@@ -11,13 +11,16 @@ from .processors import quantize_params, remove_padding
 # order with None, so that its name is refused and not taken by a later, shorter key ("qwen3next" contains "qwen3").
 _CONVERTERS = (
     (("glm5_next", "glm5next"), None),
+    (("kimi_k25", "kimi_k3", "kimivl"), None),      # ahead of "kimi_k2" below, which is a key of this table only
     (("glm4moelite", "deepseekv3", "glmmoedsa", "glm_moe_dsa", "kimi_k2", "kimik2"), convert_deepseekv3_to_hf),
     (("glm4moe",), convert_glm4moe_to_hf),
     (("glm4",), convert_glm4_to_hf),
     (("qwen3moe",), convert_qwen3moe_to_hf),
     (("qwen3next", "qwen3_8_next", "qwen4_exp", "qwen3.8_next", "qwen3_5", "qwen3_6"), None),
     (("qwen2", "qwen3"), convert_qwen2_to_hf),
+    (("deepseekv41", "deepseekv4", "inkling"), None),
     (("llama",), convert_llama_to_hf),
+    (("mimo",), convert_mimo_to_hf),
 )
 
 

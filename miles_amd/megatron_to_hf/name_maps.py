@@ -263,15 +263,16 @@ def convert_glm4moe_to_hf(args, name, param):
 
 
 def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
-    """Swap the two 64-wide halves along `dim` (size 128).  On the GPU the two halves of every leading index are byte-copy
-    jobs, so a recorded sync repeats the swap on the current weights; elsewhere a torch concatenation."""
-    a, b = t.split(64, dim=dim)
+    """Swap the two halves along `dim` (64 + 64 channels of a DSA indexer head, the two input halves of MiMo's MTP
+    projection).  On the GPU the two halves of every leading index are byte-copy jobs, so a recorded sync repeats the
+    swap on the current weights; elsewhere a torch concatenation."""
+    a, b = t.chunk(2, dim=dim)
     if t.device.type != "cuda" or not t.is_contiguous():
         return torch.cat([b, a], dim=dim)
     from miles_amd.weight_update.packed_bucket import submit_copy
 
     out = torch.empty_like(t)
-    first, second = out.split(64, dim=dim)
+    first, second = out.chunk(2, dim=dim)
     lead = 1
     for size in t.shape[:dim]:
         lead *= size
@@ -280,6 +281,30 @@ def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
         for i in range(lead):
             submit_copy(src[i], dst[i])
     return out
+
+
+_MIMO_MTP_DIRECT = {"enorm.weight": "token_layernorm.weight", "hnorm.weight": "hidden_layernorm.weight",
+                    "eh_proj.weight": "input_proj.weight", "final_layernorm.weight": "final_layernorm.weight"}
+
+
+def convert_mimo_to_hf(args, name, param):
+    """MiMo (reference: megatron_to_hf/mimo.py:6-75): the Qwen2 map, plus MTP layers that HF keeps under
+    `model.mtp_layers.<i>` with their own numbering; the MTP input projection swaps its two column halves."""
+    if "mtp" not in name:
+        return convert_qwen2_to_hf(args, name, param)
+    m = _MTP.match(name)
+    if not m:
+        raise ValueError(f"Invalid MTP parameter name: {name}")
+    layer, rest = m.groups()
+    if rest in _MIMO_MTP_DIRECT:
+        if rest == "eh_proj.weight":
+            param = _rotate_halves(param, 1)
+        return [(f"model.mtp_layers.{layer}.{_MIMO_MTP_DIRECT[rest]}", param)]
+    for prefix in ("transformer_layer.", "mtp_model_layer."):
+        if rest.startswith(prefix):
+            inner = convert_qwen2_to_hf(args, f"module.module.decoder.layers.{layer}.{rest[len(prefix):]}", param)
+            return [(hf.replace(f"model.layers.{layer}", f"model.mtp_layers.{layer}"), t) for hf, t in inner]
+    raise ValueError(f"Unknown MTP component: {rest} in {name}")
 
 
 def _dsv3_indexer(args, layer: str, rest: str, param: torch.Tensor):

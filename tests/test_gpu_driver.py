@@ -842,3 +842,42 @@ def test_dsa_indexer_half_rotation_is_replayable():
         for k in cpu:
             cpu[k] = (cpu[k].float() * 1.5 + 0.25).to(torch.bfloat16)
             dev[k].copy_(cpu[k])
+
+
+def test_mimo_mtp_sync_swaps_projection_halves_and_replays(oracle):
+    # MiMo = the dense map + MTP layers under model.mtp_layers.<i>; the MTP input projection swaps its column halves
+    # (megatron_to_hf/mimo.py:41-43), as copy jobs on the GPU so that a replayed sync sees the current weights
+    def model(seed):
+        p = _dense_model(seed)
+        M = "module.module.mtp.layers.0."
+        g = torch.Generator().manual_seed(seed)
+        p[M + "enorm.weight"] = torch.randn(256, generator=g).to(torch.bfloat16)
+        p[M + "hnorm.weight"] = torch.randn(256, generator=g).to(torch.bfloat16)
+        p[M + "eh_proj.weight"] = (torch.randn(256, 512, generator=g) * 0.02).to(torch.bfloat16)
+        p[M + "transformer_layer.mlp.linear_fc2.weight"] = (torch.randn(256, 384, generator=g) * 0.02).to(torch.bfloat16)
+        p[M + "final_layernorm.weight"] = torch.randn(256, generator=g).to(torch.bfloat16)
+        return p
+
+    cpu = model(60)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="mimo", quantization_config=FP8_CFG, send_bucket=None)
+    for sync, seed in enumerate((60, 61, 62)):
+        if sync:
+            cpu = model(seed)
+            for k in dev:
+                dev[k].copy_(cpu[k])
+        got = dict(nt for b in _run(upd) for nt in b)
+        M = "module.module.mtp.layers.0."
+        eh = cpu[M + "eh_proj.weight"]
+        # eh_proj is not among the linears the FP8 processor quantizes (quantizer_fp8.py:84-103): bf16, halves swapped
+        _same(got["model.mtp_layers.0.input_proj.weight"], torch.cat([eh[:, 256:], eh[:, :256]], dim=1), f"input_proj sync {sync}")
+        assert "model.mtp_layers.0.input_proj.weight_scale_inv" not in got
+        q, s = oracle.fp8_blockwise_cast(cpu[M + "transformer_layer.mlp.linear_fc2.weight"])
+        _same(got["model.mtp_layers.0.mlp.down_proj.weight"], q, f"mtp down_proj sync {sync}")
+        _same(got["model.mtp_layers.0.mlp.down_proj.weight_scale_inv"], s, f"mtp down_proj scales sync {sync}")
+        for mg, hf in (("enorm", "token_layernorm"), ("hnorm", "hidden_layernorm"), ("final_layernorm", "final_layernorm")):
+            _same(got[f"model.mtp_layers.0.{hf}.weight"], cpu[M + mg + ".weight"], f"{hf} sync {sync}")
+        want_dense = _expected_fp8(oracle, {k: v for k, v in cpu.items() if ".mtp." not in k})
+        for n, w in want_dense:
+            _same(got[n], w, f"{n} sync {sync}")
+    assert upd._plan is not None and upd._plan.replayable

@@ -470,7 +470,7 @@ def test_llama_and_glm4_name_maps():
     # dispatch by model name: glm4 before qwen*, llama last; GLM-4 MoE is a different map and is refused, not mis-mapped
     assert names(convert_to_hf(args, "Llama-3.1-8B", L + "mlp.linear_fc2.weight", fc1)) == ["model.layers.3.mlp.down_proj.weight"]
     assert names(convert_to_hf(args, "glm4", L + "mlp.linear_fc1.weight", fc1)) == ["model.layers.3.mlp.gate_up_proj.weight"]
-    for other_family in ("qwen3next", "Qwen3_5-MoE", "glm5_next", "mimo"):      # maps not built here: refused, never mis-mapped
+    for other_family in ("qwen3next", "Qwen3_5-MoE", "glm5_next", "deepseekv4", "kimi_k3", "kimi_k25", "kimivl"):      # maps not built here: refused, never mis-mapped
         with pytest.raises(ValueError, match="Unsupported model"):
             convert_to_hf(args, other_family, L + "mlp.linear_fc1.weight", fc1)
 
@@ -507,3 +507,30 @@ def test_glm4moe_name_map():
                 "module.module.unknown.weight"):
         with pytest.raises(ValueError, match="Unknown"):
             names(bad, w)
+
+
+def test_mimo_name_map():
+    from argparse import Namespace
+
+    from miles_amd.megatron_to_hf import convert_to_hf
+
+    args = Namespace(hidden_size=64, num_attention_heads=4, num_query_groups=2, kv_channels=16, vocab_size=100, num_layers=5)
+    conv = lambda name, t: convert_to_hf(args, "MiMo-7B", name, t)
+    w = torch.arange(64 * 128, dtype=torch.float32).reshape(64, 128)
+    M = "module.module.mtp.layers.0."
+    (name, swapped), = conv(M + "eh_proj.weight", w)
+    assert name == "model.mtp_layers.0.input_proj.weight"
+    assert torch.equal(swapped[:, :64], w[:, 64:]) and torch.equal(swapped[:, 64:], w[:, :64])
+    assert [n for n, _ in conv(M + "enorm.weight", w[0])] == ["model.mtp_layers.0.token_layernorm.weight"]
+    assert [n for n, _ in conv(M + "hnorm.weight", w[0])] == ["model.mtp_layers.0.hidden_layernorm.weight"]
+    assert [n for n, _ in conv(M + "final_layernorm.weight", w[0])] == ["model.mtp_layers.0.final_layernorm.weight"]
+    assert [n for n, _ in conv(M + "transformer_layer.mlp.linear_fc1.weight", w)] == [
+        "model.mtp_layers.0.mlp.gate_proj.weight", "model.mtp_layers.0.mlp.up_proj.weight"]
+    assert [n for n, _ in conv(M + "mtp_model_layer.self_attention.linear_proj.weight", w)] == [
+        "model.mtp_layers.0.self_attn.o_proj.weight"]
+    assert [n for n, _ in conv("module.module.decoder.layers.4.self_attention.q_layernorm.weight", w[0])] == [
+        "model.layers.4.self_attn.q_norm.weight"]
+    with pytest.raises(ValueError, match="Unknown MTP component"):
+        conv(M + "something_else.weight", w)
+    with pytest.raises(ValueError, match="Invalid MTP parameter name"):
+        conv("module.module.mtp.weight", w)
