@@ -56,7 +56,20 @@ int mq_fp8_blockwise_cast(const void* x, int dtype, int64_t stride_m, int64_t st
 int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws, int64_t M,
                         int64_t K, int per_channel, float floor_in_dtype, void* stream);
 
-/* transform_scale_ue8m0(sf, mn)                      .../processors/quantizer_fp8.py:141-142 (SGLang; DeepGEMM layout)
+/* mq_fp8_scaled_quant without the workspace argument.  No counterpart in the reference: it is for callers that
+ * cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  The amax workspace is a static device array of MQ_FP8_STATIC_MAX_ROWS words (1 MiB, held by every
+ * GPU the library runs on until the process ends); the call allocates nothing.  Results are those of
+ * mq_fp8_scaled_quant.  per_channel != 0 with M > MQ_FP8_STATIC_MAX_ROWS is refused with MQ_ERR_ARG.
+ * The device that is current at the call must be the one holding the tensors.  Every call on a GPU shares that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two host threads) race on it.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress); make that call (M = 0 is enough) before
+ * starting a graph capture. */
+#define MQ_FP8_STATIC_MAX_ROWS 262144
+int mq_fp8_scaled_quant_static(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
+                               int per_channel, float floor_in_dtype, void* stream);
+
+/* transform_scale_ue8m0(sf, mn)                     .../processors/quantizer_fp8.py:141-142 (SGLang; DeepGEMM layout)
  *   sf  [batch, tile_rows, kb] fp32 power-of-two tile scales of a [mn, 128*kb] weight, tile_rows >= ceil(mn/128)
  *   out [batch, ceil(kb/4), align(mn,4)] int32: out[b,j,r] = sum_e exponent_byte(sf[b, r/128, 4j+e]) << 8e,
  *   zero where r >= mn or 4j+e >= kb; the caller views it transposed as [batch, mn, ceil(kb/4)]

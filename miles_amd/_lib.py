@@ -25,6 +25,7 @@ SIGNATURES = {
     "mq_fp8_block_quant_pow2": [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _vp],
     "mq_fp8_blockwise_cast": [_vp, _i32, _i64, _i64, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
     "mq_fp8_scaled_quant": [_vp, _i32, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, _vp],
+    "mq_fp8_scaled_quant_static": [_vp, _i32, _i64, _vp, _vp, _i64, _i64, _i32, _f32, _vp],
     "mq_ue8m0_pack_scales": [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp8_quant": [_vp, _i32, _vp, _vp, _i64, _i64, _vp],

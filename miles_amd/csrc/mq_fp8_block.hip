@@ -9,11 +9,13 @@
 //                                .../processors/quantizer_fp8.py:139-147); restated from its published source
 //   dequant y = bf16(float(q) * s[i/B][j/B])                            (reference: tools/fp8_cast_bf16.py:15-40)
 //
-// Fast path (bf16, 128x128 tiles, 16-byte aligned rows): one 256-lane workgroup owns one tile.  Lane t
-// loads eight 16-byte row segments (rows t/16 + 16 i, columns 8 (t%16) ..+8) so that sixteen lanes read one
-// contiguous 256-byte tile row; the 64 values stay in registers, the tile amax is reduced with DPP inside each
-// wavefront and through four LDS words across the wavefronts, and the tile is quantized from registers:
+// Fast path (bf16, 128x128 tiles, 16-byte aligned rows): one 512-lane workgroup (eight wavefronts) owns one tile.
+// Lane t loads four 16-byte row segments (rows t/16 + 32 i, columns 8 (t%16) ..+8) so that sixteen lanes read one
+// contiguous 256-byte tile row; the 32 values stay in registers, the tile amax is reduced with DPP inside each
+// wavefront and through eight LDS words across the wavefronts, and the tile is quantized from registers:
 // HBM traffic is one read of the input and one write of the codes and scale.
+#include <mutex>
+
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -555,8 +557,8 @@ extern "C" int mq_fp8_block_quant_pow2(const void* w, int dtype, int64_t ldw, vo
     return fp8_block_launch(2, w, dtype, ldw, 1, q, scale, M, K, kTile, kTile, (hipStream_t)stream);
 }
 
-extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws,
-                                   int64_t M, int64_t K, int per_channel, float floor_in_dtype, void* stream) {
+static int fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws, int64_t M,
+                            int64_t K, int per_channel, float floor_in_dtype, void* stream) {
     if ((!w || !q) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if ((!scale || !amax_ws) && (M != 0 || !per_channel)) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (dtype < MQ_BF16 || dtype > MQ_F32 || M < 0 || K < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
@@ -592,6 +594,52 @@ extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* 
     hipLaunchKernelGGL(fp8_row_quant_kernel, dim3((unsigned)M), dim3(256), 0, st, w, dtype, ldw, K,
                        (const uint32_t*)amax_ws, floor_in_dtype, per_channel, (uint8_t*)q, scale);
     return mq_check_launch("fp8 scaled quant");
+}
+
+extern "C" int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* scale, void* amax_ws,
+                                   int64_t M, int64_t K, int per_channel, float floor_in_dtype, void* stream) {
+    return fp8_scaled_quant(w, dtype, ldw, q, scale, amax_ws, M, K, per_channel, floor_in_dtype, stream);
+}
+
+// ---- the same quantizer for callers that cannot allocate ------------------------------------------------------
+// The amax workspace (one word per tensor, or one per row with per-channel scales) lives in a file-scope device
+// array instead of coming from the caller.  `scratch` names the array in host code only as a symbol: its address in
+// device memory differs per GPU and is looked up once per device with hipGetSymbolAddress; kernels and fills get
+// that address, never the symbol.
+static __device__ __align__(256) uint32_t scratch[MQ_FP8_STATIC_MAX_ROWS];
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_lock;
+static uint32_t* g_scratch_ptr[kMaxDevices];      // device address of `scratch` on each GPU, 0 until first use there
+
+// address of `scratch` on the current device, or null with the error text set
+static uint32_t* scratch_on_current_device() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        mq_fail(MQ_ERR_HIP, "mq_fp8_scaled_quant_static: no current device (or a device index above 63)");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            mq_fail(MQ_ERR_HIP, "mq_fp8_scaled_quant_static: hipGetSymbolAddress failed for the amax workspace");
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = (uint32_t*)p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+extern "C" int mq_fp8_scaled_quant_static(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M,
+                                          int64_t K, int per_channel, float floor_in_dtype, void* stream) {
+    if (per_channel && M > MQ_FP8_STATIC_MAX_ROWS)
+        return mq_fail(MQ_ERR_ARG, "mq_fp8_scaled_quant_static: per-channel scales take at most MQ_FP8_STATIC_MAX_ROWS "
+                                   "(262144) rows; use mq_fp8_scaled_quant with a workspace of its own");
+    uint32_t* ws = scratch_on_current_device();
+    if (!ws) return MQ_ERR_HIP;
+    return fp8_scaled_quant(w, dtype, ldw, q, scale, ws, M, K, per_channel, floor_in_dtype, stream);
 }
 
 bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block) {
