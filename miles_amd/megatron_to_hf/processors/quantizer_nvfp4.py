@@ -139,8 +139,18 @@ def quantize_nvfp4(weight: torch.Tensor):
     """(uint8 [.., M, K/2], float8_e4m3fn [.., M, K/16], float32 global scale) for a matrix or a stack of matrices,
     each matrix of a stack with its own global scale."""
     if weight.dim() == 3:
-        per_matrix = [quantize_nvfp4(weight[i]) for i in range(weight.shape[0])]
-        return tuple(torch.stack(field, dim=0) for field in zip(*per_matrix))
+        # The stacked results are allocated first and every matrix's job writes its slices: inside a deferred or
+        # recorded batch the jobs have not run when this function returns, so nothing may be gathered from
+        # per-matrix results here (a torch.stack would copy buffers that are still uninitialised).
+        n, rows, cols = weight.shape
+        if cols % NVFP4_GROUP_SIZE:
+            raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {cols}.")
+        codes = torch.empty((n, rows, cols // 2), dtype=torch.uint8, device=weight.device)
+        block_scale = torch.empty((n, rows, cols // NVFP4_GROUP_SIZE), dtype=torch.float8_e4m3fn, device=weight.device)
+        global_scale = torch.empty((n,), dtype=torch.float32, device=weight.device)
+        for i in range(n):
+            nvfp4_quantize_1d(weight[i], out=(codes[i], block_scale[i], global_scale[i]))
+        return codes, block_scale, global_scale
     if weight.dim() != 2:
         raise ValueError(f"Unsupported weight rank {weight.dim()} for NVFP4 quantization.")
     if weight.shape[1] % NVFP4_GROUP_SIZE:

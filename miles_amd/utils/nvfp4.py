@@ -69,15 +69,23 @@ def _alloc_outputs(w: torch.Tensor):
     return q, block_scale, global_scale
 
 
-def nvfp4_quantize_1d(weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """weight [M, K] -> (uint8 [M, K/2], float8_e4m3fn [M, K/16], float32 [] = weight_scale_2)."""
+def nvfp4_quantize_1d(weight: torch.Tensor, *, out=None) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """weight [M, K] -> (uint8 [M, K/2], float8_e4m3fn [M, K/16], float32 [] = weight_scale_2).
+    `out` (not in the reference): three contiguous tensors of those shapes to write into, e.g. one matrix's slices
+    of stacked outputs, so that a caller inside a deferred batch never has to read results before the batch runs."""
     _lib.require_gpu(weight, "nvfp4_quantize_1d")
     e4m3_max, flags = _quantizer_options()
     w = weight.contiguous()
     if w.shape[1] % NVFP4_GROUP_SIZE != 0:
         raise ValueError(f"NVFP4 requires K divisible by {NVFP4_GROUP_SIZE}, got {w.shape[1]}.")
     word = torch.empty(AMAX_RECORD_WORDS, dtype=torch.int32, device=w.device)   # written by the amax pass of the job driver
-    out = _alloc_outputs(w)
+    if out is None:
+        out = _alloc_outputs(w)
+    else:
+        _lib.dtype_code(w, "nvfp4")
+        want = ((w.shape[0], w.shape[1] // 2), (w.shape[0], w.shape[1] // NVFP4_GROUP_SIZE), ())
+        if any(tuple(t.shape) != shape or not t.is_contiguous() for t, shape in zip(out, want)):
+            raise ValueError("nvfp4_quantize_1d: `out` tensors must be contiguous and shaped like the results")
     launch.submit(_lib.JOB_NVFP4, w, out[0], out[1], word, out[2], w.shape[0], w.shape[1], w.shape[1], e4m3_max, flags)
     return out
 

@@ -154,6 +154,27 @@ def test_convert_nvfp4_pairs_across_shards(oracle, tmp_path):
     assert index["model.layers.0.mlp.experts.2.gate_proj.weight"] == "model-00000-of-00002.safetensors"
 
 
+def test_convert_nvfp4_stacked_expert_weight(oracle, tmp_path):
+    """A checkpoint that stores its routed experts as one 3-D tensor: every matrix of the stack is quantized with its
+    own global scale.  The converter works inside a deferred batch, so the stacked results must be written by the jobs
+    themselves (nothing may be gathered before the batch has run)."""
+    from miles_amd.tools.convert_hf_to_nvfp4 import convert_nvfp4
+
+    stack = torch.stack([_rand((256, 96), 60 + e) * (1.0 + e) for e in range(4)])
+    shards = [{"model.layers.0.mlp.experts.down_proj.weight": stack, "model.layers.0.mlp.gate.weight": _rand((4, 256), 70)}]
+    model = _checkpoint(tmp_path, shards)
+    out = tmp_path / "nvfp4"
+    convert_nvfp4(str(model), str(out), device="cuda:0")
+    got = _load_all(out)
+    want = [oracle.nvfp4_quantize_1d(stack[e].contiguous()) for e in range(4)]
+    base = "model.layers.0.mlp.experts.down_proj"
+    _same(got[base + ".weight"], torch.stack([w[0] for w in want]), "stacked codes")
+    _same(got[base + ".weight_scale"], torch.stack([w[1] for w in want]), "stacked block scales")
+    _same(got[base + ".weight_scale_2"], torch.stack([w[2] for w in want]), "stacked global scales")
+    assert got[base + ".weight_scale_2"].unique().numel() == 4
+    assert torch.equal(got[base + ".input_scale"], torch.ones(4))
+
+
 def test_convert_mxfp8_from_bf16_and_from_pow2_fp8(oracle, tmp_path):
     from miles_amd.tools.convert_hf_to_mxfp8 import convert_mxfp8
 

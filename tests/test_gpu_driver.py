@@ -881,3 +881,34 @@ def test_mimo_mtp_sync_swaps_projection_halves_and_replays(oracle):
         for n, w in want_dense:
             _same(got[n], w, f"{n} sync {sync}")
     assert upd._plan is not None and upd._plan.replayable
+
+
+def test_quantize_nvfp4_on_a_stack_inside_a_batch_and_replayed(oracle):
+    """A 3-D weight (a stack of expert matrices) quantized inside a deferred batch: the stacked outputs are written by
+    the jobs, so they hold the results once the batch has run, and a recorded batch re-run after an in-place weight
+    change produces the new results at the same addresses."""
+    from miles_amd import launch
+    from miles_amd.megatron_to_hf.processors.quantizer_nvfp4 import quantize_nvfp4
+
+    def expected(cpu):
+        per = [oracle.nvfp4_quantize_1d(cpu[i].contiguous()) for i in range(cpu.shape[0])]
+        return tuple(torch.stack(f) for f in zip(*per))
+
+    cpu = torch.stack([W.gaussian_outliers((64, 128), std=0.02 * (i + 1), p_outlier=0.01, gain=20.0, seed=300 + i)
+                       for i in range(3)])
+    dev = cpu.to(DEV)
+    with launch.deferred():
+        got = quantize_nvfp4(dev)
+    torch.cuda.synchronize()
+    for g, w, what in zip(got, expected(cpu), ("codes", "block scales", "global scales")):
+        _same(g, w, f"deferred stack {what}")
+    with launch.recording() as batch:
+        got = quantize_nvfp4(dev)
+    batch.device = torch.device(DEV)
+    batch.run()
+    cpu2 = torch.stack([W.gaussian_outliers((64, 128), std=0.05, p_outlier=0.0, gain=1.0, seed=400 + i) for i in range(3)])
+    dev.copy_(cpu2)
+    batch.run()
+    torch.cuda.synchronize()
+    for g, w, what in zip(got, expected(cpu2), ("codes", "block scales", "global scales")):
+        _same(g, w, f"replayed stack {what}")

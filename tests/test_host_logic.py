@@ -186,8 +186,12 @@ def fake_kernels(monkeypatch):
     def nv_outputs(w):
         return torch.zeros(w.shape[0], w.shape[1] // 2, dtype=torch.uint8), torch.zeros(w.shape[0], w.shape[1] // 16), torch.ones(())
 
-    def fake_nv(w):
+    def fake_nv(w, *, out=None):
         calls.append(("nvfp4", tuple(w.shape)))
+        if out is not None:                       # a stack's matrices are written into slices of the stacked outputs
+            assert [tuple(t.shape) for t in out] == [(w.shape[0], w.shape[1] // 2), (w.shape[0], w.shape[1] // 16), ()]
+            out[2].fill_(1.0)
+            return out
         return nv_outputs(w)
 
     def fake_pair(a, b):
