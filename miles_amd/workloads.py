@@ -130,3 +130,95 @@ def c5_expert(expert: int, which: int, seed: int = 5001):
     """DeepSeek-V3-shaped expert: gate/up [2048,7168], down [7168,2048]; N(0,0.02)."""
     shape = (2048, 7168) if which < 2 else (7168, 2048)
     return gaussian_outliers(shape, std=0.02, p_outlier=0.0, gain=1.0, seed=seed + expert * 3 + which)
+
+
+# ---- the same configurations generated on the GPU ---------------------------------------------------------
+# Whole models are too large to generate on the CPU in reasonable time (3.6e9 to 2.9e10 elements): these build the
+# Megatron-named parameter sets of the benchmark configurations on the device with a seeded device generator.  A
+# checker that needs the same bits on the host copies the tensors back.
+def device_gaussian_outliers(shape, gen, *, std=0.02, p_outlier=0.001, gain=20.0):
+    """bf16 N(0, std) with a fraction p_outlier of entries multiplied by gain."""
+    x = torch.randn(shape, generator=gen, device=gen.device, dtype=torch.float32) * std
+    if p_outlier > 0:
+        x = torch.where(torch.rand(shape, generator=gen, device=gen.device) < p_outlier, x * gain, x)
+    return x.to(torch.bfloat16)
+
+
+def device_student_t_rows(shape, gen, *, std=0.02):
+    """bf16 std*randn scaled per row by |t|, t ~ Student-t(3) (= z / sqrt(chi2_3 / 3)): heavy-tailed row magnitudes."""
+    m, _ = shape
+    x = torch.randn(shape, generator=gen, device=gen.device, dtype=torch.float32) * std
+    z = torch.randn((m, 1), generator=gen, device=gen.device, dtype=torch.float32)
+    chi2 = (torch.randn((m, 3), generator=gen, device=gen.device, dtype=torch.float32) ** 2).sum(dim=1, keepdim=True)
+    return (x * (z / torch.sqrt(chi2 / 3.0)).abs()).to(torch.bfloat16)
+
+
+def qwen3_4b_megatron(gen, *, layers=QWEN3_4B["layers"], buffer_bytes=512 * 1024**2):
+    """Megatron-named parameters of Qwen3-4B (hidden 2560, 32 q heads / 8 kv groups of 128, ffn 9728, `layers` decoder
+    layers, embeddings and norms included) -> (args, weights, number of elements the FP8 sync quantizes)."""
+    from argparse import Namespace
+
+    h, heads, groups, hd, ffn, vocab = 2560, 32, 8, 128, 9728, 151936
+    dev = gen.device
+    w = {"module.module.embedding.word_embeddings.weight": device_gaussian_outliers((vocab, h), gen, p_outlier=0)}
+    for i in range(layers):
+        L = f"module.module.decoder.layers.{i}."
+        w[L + "self_attention.linear_qkv.layer_norm_weight"] = torch.ones(h, device=dev, dtype=torch.bfloat16)
+        w[L + "self_attention.linear_qkv.weight"] = device_gaussian_outliers(((heads + 2 * groups) * hd, h), gen)
+        w[L + "self_attention.q_layernorm.weight"] = torch.ones(hd, device=dev, dtype=torch.bfloat16)
+        w[L + "self_attention.k_layernorm.weight"] = torch.ones(hd, device=dev, dtype=torch.bfloat16)
+        w[L + "self_attention.linear_proj.weight"] = device_gaussian_outliers((h, heads * hd), gen)
+        w[L + "mlp.linear_fc1.layer_norm_weight"] = torch.ones(h, device=dev, dtype=torch.bfloat16)
+        w[L + "mlp.linear_fc1.weight"] = device_gaussian_outliers((2 * ffn, h), gen)
+        w[L + "mlp.linear_fc2.weight"] = device_gaussian_outliers((h, ffn), gen)
+    w["module.module.decoder.final_layernorm.weight"] = torch.ones(h, device=dev, dtype=torch.bfloat16)
+    args = Namespace(hidden_size=h, num_attention_heads=heads, num_query_groups=groups, kv_channels=hd,
+                     vocab_size=vocab, num_layers=layers, update_weight_buffer_size=buffer_bytes, q_lora_rank=None)
+    quantized_elems = layers * (heads * hd * h + 2 * groups * hd * h + h * heads * hd + 3 * ffn * h)
+    return args, w, quantized_elems
+
+
+# the three MoE configurations: model name of the name map, quantization config, (layers, experts, ffn, hidden) and the
+# distribution of the expert weights
+MOE_CONFIGS = {
+    "C3": dict(model_name="qwen3moe", cfg={"quant_method": "mxfp8"}, shape=(48, 128, 768, 2048), dist="student_t"),
+    "C4": dict(model_name="kimi_k2",
+               cfg={"quant_method": "compressed-tensors", "format": "pack-quantized",
+                    "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4,
+                                                              "type": "int"}}}},
+               shape=(1, 384, 2048, 7168), dist="outliers_0.015"),
+    "C5a": dict(model_name="deepseekv3", cfg={"quant_method": "modelopt", "quant_algo": "NVFP4"},
+                shape=(1, 256, 2048, 7168), dist="gaussian_0.02"),
+}
+
+
+def device_expert_tensor(shape, gen, dist: str):
+    if dist == "student_t":
+        return device_student_t_rows(shape, gen, std=0.02)
+    if dist == "outliers_0.015":
+        return device_gaussian_outliers(shape, gen, std=0.015, p_outlier=0.0005, gain=30.0)
+    if dist == "gaussian_0.02":
+        return device_gaussian_outliers(shape, gen, std=0.02, p_outlier=0.0)
+    raise ValueError(dist)
+
+
+def moe_megatron(gen, *, layers, experts, ffn, hidden, dist, buffer_bytes=512 * 1024**2):
+    """Megatron-named routed-expert parameters (fused gate/up `linear_fc1` [2*ffn, hidden], `linear_fc2` [hidden, ffn])
+    -> (args, weights, elements)."""
+    from argparse import Namespace
+
+    w = {}
+    for layer in range(layers):
+        L = f"module.module.decoder.layers.{layer}."
+        for e in range(experts):
+            w[L + f"mlp.experts.linear_fc1.weight{e}"] = device_expert_tensor((2 * ffn, hidden), gen, dist)
+            w[L + f"mlp.experts.linear_fc2.weight{e}"] = device_expert_tensor((hidden, ffn), gen, dist)
+    args = Namespace(hidden_size=hidden, num_attention_heads=32, num_query_groups=4, kv_channels=128, vocab_size=1000,
+                     num_layers=layers, update_weight_buffer_size=buffer_bytes, q_lora_rank=None)
+    return args, w, layers * experts * 3 * ffn * hidden
+
+
+def int4_packed_basenames(layers: int, experts: int) -> set[str]:
+    """The module names a compressed-tensors checkpoint stores packed: every routed expert projection."""
+    return {f"model.layers.{l}.mlp.experts.{e}.{p}_proj" for l in range(layers) for e in range(experts)
+            for p in ("gate", "up", "down")}
