@@ -14,7 +14,7 @@ The JSON line also carries
                 events on the launch stream; peak = 8 TB/s HBM
   cpu_baseline  the CPU oracle (bit-exact port) timed on the host cores on a bounded sample of the workload
   per_quantizer GB/s of every quantizer on its BASELINE.json configuration shape (not part of `value`)
-  parity        a sample of the step's outputs compared byte for byte with the oracle
+  parity        every tensor one sync hands out compared with the oracle (fingerprints of all, bytes of a sample)
 """
 
 from __future__ import annotations
@@ -48,31 +48,16 @@ DEV = "cuda:0"
 
 def _synth(shape, gen, *, std=0.02, p=0.001, gain=20.0):
     """bf16 N(0, std) with a fraction p of entries multiplied by gain, generated on the GPU."""
-    x = torch.randn(shape, generator=gen, device=DEV, dtype=torch.float32) * std
-    if p > 0:
-        x = torch.where(torch.rand(shape, generator=gen, device=DEV) < p, x * gain, x)
-    return x.to(torch.bfloat16)
+    from miles_amd import workloads as W
+
+    return W.device_gaussian_outliers(shape, gen, std=std, p_outlier=p, gain=gain)
 
 
 def qwen3_4b_megatron_weights(gen):
     """Megatron-named parameters of Qwen3-4B: hidden 2560, 32 q heads / 8 kv groups of 128, ffn 9728, 36 layers."""
-    h, heads, groups, hd, ffn, layers, vocab = 2560, 32, 8, 128, 9728, 36, 151936
-    w = {"module.module.embedding.word_embeddings.weight": _synth((vocab, h), gen, p=0)}
-    for i in range(layers):
-        L = f"module.module.decoder.layers.{i}."
-        w[L + "self_attention.linear_qkv.layer_norm_weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
-        w[L + "self_attention.linear_qkv.weight"] = _synth(((heads + 2 * groups) * hd, h), gen)
-        w[L + "self_attention.q_layernorm.weight"] = torch.ones(hd, device=DEV, dtype=torch.bfloat16)
-        w[L + "self_attention.k_layernorm.weight"] = torch.ones(hd, device=DEV, dtype=torch.bfloat16)
-        w[L + "self_attention.linear_proj.weight"] = _synth((h, heads * hd), gen)
-        w[L + "mlp.linear_fc1.layer_norm_weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
-        w[L + "mlp.linear_fc1.weight"] = _synth((2 * ffn, h), gen)
-        w[L + "mlp.linear_fc2.weight"] = _synth((h, ffn), gen)
-    w["module.module.decoder.final_layernorm.weight"] = torch.ones(h, device=DEV, dtype=torch.bfloat16)
-    args = Namespace(hidden_size=h, num_attention_heads=heads, num_query_groups=groups, kv_channels=hd,
-                     vocab_size=vocab, num_layers=layers, update_weight_buffer_size=512 * 1024**2, q_lora_rank=None)
-    quantized_elems = layers * (heads * hd * h + 2 * groups * hd * h + h * heads * hd + 3 * ffn * h)
-    return args, w, quantized_elems
+    from miles_amd import workloads as W
+
+    return W.qwen3_4b_megatron(gen)
 
 
 TIMED_ITERS = 5        # repetitions per per-quantizer measurement (1 in the counter-collection run)
@@ -114,6 +99,7 @@ def per_quantizer(gen):
     from miles_amd.tools.fp8_cast_bf16 import weight_dequant
     from miles_amd.utils.mxfp8 import mxfp8_quantize
     from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+    from miles_amd import workloads as W
 
     res = {}
 
@@ -139,18 +125,21 @@ def per_quantizer(gen):
         lambda: [block_fp8(t, [128, 128]) for m in mlp for t in m], "8 x Qwen3-4B MLP (gate, up, down), block_fp8")
     del mlp
     # C3: Qwen3-30B-A3B experts, MXFP8; 2 layers of 128 experts
-    experts = [(_synth((1536, 2048), gen, p=0), _synth((2048, 768), gen, p=0)) for _ in range(256)]
+    experts = [(W.device_student_t_rows((1536, 2048), gen), W.device_student_t_rows((2048, 768), gen)) for _ in range(256)]
     run("C3_mxfp8", "mxfp8", 256 * 3 * 768 * 2048,
         lambda: [mxfp8_quantize(t) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
-        "2 layers x 128 experts (gate, up [768,2048], down [2048,768])")
+        "2 layers x 128 experts (gate, up [768,2048], down [2048,768]), 0.02 N(0,1) x Student-t(3) row scales")
     del experts
-    # C4 / C5: Kimi-K2- / DeepSeek-V3-shaped experts, 32 experts
+    # C4: Kimi-K2-shaped experts, 32 of them, N(0, 0.015) + 0.05 % outliers x 30
     experts = [(_synth((4096, 7168), gen, std=0.015, p=0.0005, gain=30.0), _synth((7168, 2048), gen, std=0.015, p=0.0005, gain=30.0))
                for _ in range(32)]
     n = 32 * 3 * 2048 * 7168
     run("C4_int4_g128_pack", "int4_g128", n,
         lambda: [pack_layer(t, 128) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
         "32 experts (gate, up [2048,7168], down [7168,2048]), pack_layer group 128")
+    del experts
+    # C5: DeepSeek-V3-shaped experts, 32 of them, N(0, 0.02)
+    experts = [(_synth((4096, 7168), gen, p=0), _synth((7168, 2048), gen, p=0)) for _ in range(32)]
 
     def nvfp4_all():
         out = []
@@ -165,6 +154,7 @@ def per_quantizer(gen):
         "32 experts, gate/up paired + down; steady-state sync: one pass with the amax carried over from the previous sync "
         "(checked on the way; here no amax moves)", prepare=lambda b: b.carry_amax())
     run("C5a_nvfp4_first_sync", "nvfp4", n, nvfp4_all, "as C5a, first sync of a model: amax pass + quantize pass")
+    res.update(nvfp4_after_update(gen, experts, nvfp4_all, n))
     firsts = [t.view(-1)[:1] for fc1, fc2 in experts for t in (fc1, fc2)]
     for f in firsts:
         f.fill_(1.0)            # the largest element of every tensor (of every gate/up pair), toggled below
@@ -196,72 +186,110 @@ def per_quantizer(gen):
     return res
 
 
+def nvfp4_after_update(gen, experts, build, elems):
+    """NVFP4 syncs with a training step between them.  fp32 master weights take an Adam-sized step (every element moves
+    by lr x a unit-variance direction) and are rounded to bf16 in place; the sync after each step is timed on its own
+    (events around the job list) and the amax records say how many tensors had to be quantized in the second pass.
+    A weight's bf16 value changes when its master crosses a rounding boundary, so with lr = 1e-6 (an RL fine-tuning
+    rate) about one element in a hundred changes per step and a tensor's amax only now and then."""
+    from miles_amd import _lib
+
+    tensors = [t for fc1, fc2 in experts for t in (fc1, fc2)]
+    out = {}
+    for lr, label in ((1e-6, "lr1e-6"), (1e-4, "lr1e-4")):
+        masters = [t.float() for t in tensors]
+        batch, outs = _record(build)
+        batch.carry_amax()
+        batch.run()
+        torch.cuda.synchronize()
+        total_ms, redone, records, changed, steps = 0.0, 0, 0, 0.0, 8
+        for _ in range(steps):
+            before = tensors[0].clone()
+            for m, t in zip(masters, tensors):
+                m.add_(torch.randn(m.shape, generator=gen, device=DEV), alpha=lr)
+                t.copy_(m)
+            changed += (tensors[0] != before).float().mean().item()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            batch.run()
+            e1.record()
+            torch.cuda.synchronize()
+            total_ms += e0.elapsed_time(e1)
+            recs = torch.stack([r[_lib.RECORD_REDO_WORD] for r in batch.amax_records()])
+            redone += int(recs.sum().item())
+            records += recs.numel()
+        ms = total_ms / steps
+        gbps = elems * BYTES_PER_ELEM["nvfp4"] / ms / 1e6
+        out[f"C5a_nvfp4_after_update_{label}"] = {
+            "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4), "elements": elems,
+            "fraction_of_tensors_quantized_in_the_second_pass": round(redone / max(records, 1), 4),
+            "fraction_of_bf16_values_changed_per_step": round(changed / steps, 4),
+            "workload": f"as C5a, {steps} syncs each after an optimizer step of size lr = {lr:g} on fp32 master weights "
+                        "(unit-variance direction), rounded to bf16 in place"}
+        for m, t in zip(masters, tensors):
+            del m
+        del masters, batch, outs
+    return out
+
+
 def full_configs(gen):
-    """The three MoE configurations at their full element counts, each as one whole weight sync through the driver
-    (`WeightUpdater` with a replayed plan, 512 MiB buckets): every expert of every layer at its real shape.
-    Not part of the default run (generating 58 GB of synthetic experts takes a while); `--full-configs` prints one
-    extra JSON line."""
+    """The three MoE configurations at their full element counts and on their own data distributions, each as one whole
+    weight sync through the driver (`WeightUpdater` with a replayed plan, 512 MiB buckets): every expert of every layer
+    at its real shape.  Timed like the headline: K syncs between two events on the launch stream and a wall clock."""
+    from miles_amd import workloads as W
     from miles_amd.weight_update.updater import WeightUpdater
 
-    def moe_weights(layers, experts, ffn, hidden, std, p, gain):
-        w = {}
-        for layer in range(layers):
-            L = f"module.module.decoder.layers.{layer}."
-            for e in range(experts):
-                w[L + f"mlp.experts.linear_fc1.weight{e}"] = _synth((2 * ffn, hidden), gen, std=std, p=p, gain=gain)
-                w[L + f"mlp.experts.linear_fc2.weight{e}"] = _synth((hidden, ffn), gen, std=std, p=p, gain=gain)
-        return w
-
-    def sync(name, key, model_name, cfg, shape, note, **extra):
-        layers, experts, ffn, hidden = shape
-        weights = moe_weights(layers, experts, ffn, hidden, *((0.02, 0.0, 1.0) if key == "mxfp8" else (0.015, 0.0005, 30.0)))
-        elems = layers * experts * 3 * ffn * hidden
-        args = Namespace(hidden_size=hidden, num_attention_heads=32, num_query_groups=4, kv_channels=128, vocab_size=1000,
-                         num_layers=layers, update_weight_buffer_size=512 * 1024**2, q_lora_rank=None)
+    def sync(key, fmt, note):
+        conf = W.MOE_CONFIGS[key]
+        layers, experts, ffn, hidden = conf["shape"]
+        args, weights, elems = W.moe_megatron(gen, layers=layers, experts=experts, ffn=ffn, hidden=hidden, dist=conf["dist"])
+        extra = {"packed_weight_basenames": W.int4_packed_basenames(layers, experts)} if fmt == "int4_g128" else {}
         seen = {"buckets": 0, "tensors": 0}
 
         def consume(bucket):
             seen["buckets"] += 1
             seen["tensors"] += len(bucket)
 
-        upd = WeightUpdater(args, weights_getter=lambda: weights, model_name=model_name, quantization_config=cfg,
-                            send_bucket=consume, **extra)
+        torch.cuda.synchronize()
+        resident = torch.cuda.memory_allocated()
+        upd = WeightUpdater(args, weights_getter=lambda: weights, model_name=conf["model_name"],
+                            quantization_config=conf["cfg"], send_bucket=consume, **extra)
         t0 = time.perf_counter()
         upd.update_weights()
         torch.cuda.synchronize()
         first_s = time.perf_counter() - t0
-        assert upd._plan is not None and upd._plan.replayable, name
-        for _ in range(2):
+        assert upd._plan is not None and upd._plan.replayable, key
+        for _ in range(3):
             upd.update_weights()
         torch.cuda.synchronize()
         seen.update(buckets=0, tensors=0)
         steps = 5
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        e0.record()
         for _ in range(steps):
             upd.update_weights()
+        e1.record()
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / steps * 1e3
-        gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
+        gpu_ms = e0.elapsed_time(e1) / steps
+        gbps = elems * BYTES_PER_ELEM[fmt] / ms / 1e6
         out = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms_per_sync": round(ms, 3),
-               "elements": elems, "megatron_tensors": len(weights), "hf_tensors_per_sync": seen["tensors"] // steps,
-               "buckets_per_sync": seen["buckets"] // steps, "jobs": len(upd._plan.batch),
-               "first_sync_s": round(first_s, 2), "workload": note}
+               "gpu_ms_per_sync": round(gpu_ms, 3), "elements": elems, "megatron_tensors": len(weights),
+               "hf_tensors_per_sync": seen["tensors"] // steps, "buckets_per_sync": seen["buckets"] // steps,
+               "jobs": len(upd._plan.batch), "first_sync_s": round(first_s, 2),
+               "sync_output_bytes_resident": torch.cuda.memory_allocated() - resident, "workload": note}
         del upd, weights
         return out
 
-    res = {}
-    res["C3_qwen3_30b_a3b_mxfp8"] = sync("C3", "mxfp8", "qwen3moe", {"quant_method": "mxfp8"}, (48, 128, 768, 2048),
-                                         "48 layers x 128 experts, gate/up [768,2048] down [2048,768], MXFP8 1x32 E8M0")
-    int4_cfg = {"quant_method": "compressed-tensors", "format": "pack-quantized",
-                "config_groups": {"group_0": {"weights": {"group_size": 128, "symmetric": True, "num_bits": 4, "type": "int"}}}}
-    basenames = {f"model.layers.0.mlp.experts.{e}.{p}_proj" for e in range(384) for p in ("gate", "up", "down")}
-    res["C4_kimi_k2_int4_g128"] = sync("C4", "int4_g128", "kimi_k2", int4_cfg, (1, 384, 2048, 7168),
-                                       "384 experts, gate/up [2048,7168] down [7168,2048], INT4 group 128 packed",
-                                       packed_weight_basenames=basenames)
-    res["C5a_deepseek_v3_nvfp4"] = sync("C5a", "nvfp4", "deepseekv3", {"quant_method": "modelopt", "quant_algo": "NVFP4"},
-                                        (1, 256, 2048, 7168),
-                                        "256 experts, gate/up [2048,7168] paired + down [7168,2048], NVFP4 1x16")
-    return res
+    return {
+        "C3_full": sync("C3", "mxfp8", "Qwen3-30B-A3B: 48 layers x 128 experts, gate/up [768,2048] down [2048,768], MXFP8 1x32 "
+                                       "E8M0, rows 0.02 N(0,1) x |Student-t(3)|"),
+        "C4_full": sync("C4", "int4_g128", "Kimi-K2-shaped: 384 experts, gate/up [2048,7168] down [7168,2048], INT4 group 128 "
+                                           "packed, N(0,0.015) + 0.05% x30"),
+        "C5a_full": sync("C5a", "nvfp4", "DeepSeek-V3-shaped: 256 experts, gate/up [2048,7168] paired + down [7168,2048], "
+                                         "NVFP4 1x16, N(0,0.02); steady state (amax carried over, none moved)"),
+    }
 
 
 def full_model_block_fp8(weights, elems):
@@ -385,47 +413,33 @@ def packed_payload(args, weights, fp8_cfg, steps):
             "note": "one sync = quantize + build every bucket's flat payload (embeddings and norms included)"}
 
 
-def _lib_max_group():
+def launches_per_sync(plan):
+    """Kernel launches of one replayed sync: every submission of the plan is cut into launches of up to MAX_GROUP
+    consecutive jobs of one kind (the headline sync has only FP8 128x128 jobs)."""
     from miles_amd import _lib
 
-    return _lib.MAX_GROUP
-
-
-def roofline(plan, jobs_meta):
-    """Average duration of the kernel launches of a sync (same launch partition as a step), from events on the launch
-    stream."""
-    spans = []
-    done = 0
+    n, done = 0, 0
     for mark in plan.submission_marks():
-        a = done
-        while a < mark:      # mq_run_jobs fuses up to 64 consecutive same-kind jobs into one launch
-            b = min(a + _lib_max_group(), mark)
-            spans.append((a, b))
-            a = b
+        n += -(-(mark - done) // _lib.MAX_GROUP) if mark > done else 0
         done = max(done, mark)
-    # One event pair around the launches of a whole sync: the launches run back to back on one stream, so the elapsed
-    # time over their count is the average launch duration plus the gap between launches (it can only understate the
-    # kernel).  A pair around every single launch adds about 5 us of dispatch latency to each (221 us against the
-    # 216 us of the kernel trace).
-    total_ms, total_bytes = 0.0, 0.0
-    reps = 10
-    for _ in range(reps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for a, b in spans:
-            plan.batch.run_range(a, b)
-        e1.record()
-        e1.synchronize()
-        total_ms += e0.elapsed_time(e1)
-        total_bytes += sum(sum(jobs_meta[a:b]) for a, b in spans) * BYTES_PER_ELEM["fp8_block"]
-    launches = reps * len(spans)
-    achieved = total_bytes / total_ms / 1e6
-    elems_per_launch = total_bytes / BYTES_PER_ELEM["fp8_block"] / launches
-    traffic = round(MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems_per_launch)
+    return n
+
+
+def roofline(plan, elems, steps, gpu_ms):
+    """The dominant kernel over the timed region itself: `gpu_ms` is the time between two events recorded on the launch
+    stream around the `steps` timed syncs.  The launches run back to back on that one stream, so the elapsed time over
+    their count is the average launch duration plus the gap to the next launch: it can only understate the kernel, and
+    launches_per_sync x avg_launch_us <= ms_per_step holds by construction (the wall clock contains the event span)."""
+    launches = launches_per_sync(plan)
+    avg_us = gpu_ms * 1e3 / (steps * launches)
+    bytes_per_launch = elems * BYTES_PER_ELEM["fp8_block"] / launches
+    achieved = bytes_per_launch / avg_us / 1e3
     return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-            "launches_per_sync": len(spans), "avg_launch_us": round(total_ms / launches * 1e3, 2),
-            "algorithmic_bytes_per_launch": round(total_bytes / launches)}
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": round(MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems / launches),
+            "launches_per_sync": launches, "avg_launch_us": round(avg_us, 2),
+            "algorithmic_bytes_per_launch": round(bytes_per_launch),
+            "timed_with": f"one event pair on the launch stream around the {steps} timed syncs ({steps * launches} launches)"}
 
 
 def cpu_baseline(weights, args, budget_s=12.0):
@@ -483,23 +497,29 @@ def _torch_cpu_block_fp8(w, budget_s=4.0):
             "cores": torch.get_num_threads(), "sample": f"{reps} x block_fp8 op chain on gate_proj {tuple(w.shape)}, {dt:.1f} s"}
 
 
-def parity_sample(weights, args, plan):
-    """Byte-compare layer 0's quantized tensors of the timed sync with the oracle."""
-    from miles_amd.megatron_to_hf import name_maps
+def parity_whole_sync(weights, args, updater):
+    """Every tensor one sync hands out (252 quantized weights with their scales, embeddings and norms) against the
+    oracle applied to the same weights: names and order, a 64-bit fingerprint of every tensor, full bytes of the first,
+    the last and every 17th."""
     from oracle import mq_oracle
+    from tests import sync_expectations as E
 
-    got = {n: t for bucket in plan.buckets for n, t in bucket}
-    checked = 0
-    for rest in ("self_attention.linear_qkv.weight", "mlp.linear_fc1.weight", "mlp.linear_fc2.weight"):
-        name = "module.module.decoder.layers.0." + rest
-        for hf, t in name_maps.convert_qwen2_to_hf(args, name, weights[name].cpu()):
-            q, s = mq_oracle.fp8_blockwise_cast(t.contiguous())
-            ok = torch.equal(got[hf].cpu().view(torch.uint8), q.view(torch.uint8)) and \
-                torch.equal(got[hf.replace(".weight", ".weight_scale_inv")].cpu(), s)
-            if not ok:
-                raise SystemExit(f"PARITY FAILURE: {hf} differs from the oracle")
-            checked += 1
-    return f"ok ({checked} tensors of layer 0 byte-identical to the oracle)"
+    mq_oracle.build()
+    want = E.expected_dense_fp8(mq_oracle, args, {k: v.cpu() for k, v in weights.items()})
+    got = []
+    consumer, updater.send_bucket = updater.send_bucket, lambda bucket: got.extend((n, t.cpu()) for n, t in bucket)
+    try:
+        updater.update_weights()
+        torch.cuda.synchronize()
+    finally:
+        updater.send_bucket = consumer
+    try:
+        stats = E.compare_streams(mq_oracle, got, want, "timed sync")
+    except AssertionError as exc:
+        raise SystemExit(f"PARITY FAILURE: {exc}") from None
+    quantized = sum(n.endswith("_proj.weight") for n, _ in want)
+    return (f"ok ({quantized} quantized tensors + their scales + {stats['tensors'] - 2 * quantized} pass-through tensors of the "
+            f"whole sync: every 64-bit fingerprint equal to the oracle's, {stats['byte_compared']} tensors compared byte for byte)")
 
 
 def stream_ceilings():
@@ -540,7 +560,8 @@ def main():
     ap.add_argument("--stream-ceilings", action="store_true",
                     help="only torch's fill / copy / cast kernels on 4 GiB operands: what plain streaming reaches here (one JSON line)")
     ap.add_argument("--full-configs", action="store_true",
-                    help="only the three MoE configurations at full size, each as one whole sync (one JSON line)")
+                    help="only the three MoE configurations at full size, each as one whole sync (one JSON line; the "
+                         "default run includes them under per_quantizer)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
@@ -581,7 +602,11 @@ def main():
 
     updater = WeightUpdater(args, weights_getter=lambda: weights, model_name="qwen3", quantization_config=fp8_cfg,
                             send_bucket=consume)
+    torch.cuda.synchronize()
+    plan_bytes = torch.cuda.memory_allocated()
     updater.update_weights()          # builds the plan (first sync pays the per-parameter Python work)
+    torch.cuda.synchronize()
+    plan_bytes = torch.cuda.memory_allocated() - plan_bytes      # device memory the sync's outputs occupy from now on
     if a.pmc_workload:
         n = 1 << 30
         src, dst = torch.empty(n, dtype=torch.uint8, device=DEV), torch.empty(n, dtype=torch.uint8, device=DEV)
@@ -603,40 +628,47 @@ def main():
         updater.update_weights()
     torch.cuda.synchronize()
     sent.update(buckets=0, bytes=0)
+    # the timed region: K syncs between two wall-clock reads, and inside them between two events on the launch stream
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(a.steps):
         updater.update_weights()
+    e1.record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    gpu_ms = e0.elapsed_time(e1)
     ms_per_step = dt / a.steps * 1e3
     algorithmic_bytes = elems * BYTES_PER_ELEM["fp8_block"]
     value = algorithmic_bytes / (dt / a.steps) / 1e9
 
     plan = updater._plan
     assert plan is not None and plan.replayable, "the benchmark expects the replayable plan path"
-    jobs_meta = [rec[7] * rec[8] for rec in plan.batch.records]     # rows * cols of every job
+    assert all(rec[0] == _lib.JOB_FP8_BLOCKWISE_CAST for rec in plan.batch.records), "the headline sync runs one kernel only"
     line = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32", "io_dtypes": "bf16 in -> float8_e4m3fn codes + fp32 tile scales out (arithmetic in fp32)",
+        "data": "synthetic",
         "config": {"workload": "configs[1]: full Qwen3-4B weight sync to FP8 e4m3 128x128 block scales, 36 layers "
                                "(q[4096,2560] k/v[1024,2560] o[2560,4096] gate/up[9728,2560] down[2560,9728]), bf16 "
                                "N(0,0.02) + 0.1% x20 outliers, embeddings and norms passed through as bf16",
                    "quantizer": "fp8_blockwise_cast (sync path)", "quantized_elements": elems,
                    "algorithmic_bytes": round(algorithmic_bytes), "buckets_per_sync": sent["buckets"] // max(a.steps, 1),
-                   "bucket_bytes": args.update_weight_buffer_size},
+                   "bucket_bytes": args.update_weight_buffer_size, "gpus": "one GPU; no second GPU is used or measured"},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-        "roofline": roofline(plan, jobs_meta),
-        "parity": parity_sample(weights, args, plan),
+        "roofline": roofline(plan, elems, a.steps, gpu_ms),
+        "sync_output_bytes_resident": plan_bytes,
+        "parity": parity_whole_sync(weights, args, updater),
     }
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(weights, args)
     if not a.no_extras:
         del updater, plan
-        line["packed_payload"] = packed_payload(args, weights, fp8_cfg, a.steps)
+        line["packed_payload"] = packed_payload(args, weights, fp8_cfg, min(a.steps, 20))
         c2_block_fp8 = full_model_block_fp8(weights, elems)
         weights.clear()
-        line["per_quantizer"] = {"C2_block_fp8": c2_block_fp8, **per_quantizer(gen)}
+        line["per_quantizer"] = {"C2_block_fp8": c2_block_fp8, **per_quantizer(gen), **full_configs(gen)}
     print(json.dumps(line))
 
 

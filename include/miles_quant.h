@@ -29,6 +29,12 @@ extern "C" {
 #define MQ_NVFP4_SECTION_WORDS 256
 #define MQ_NVFP4_SECTIONS 4
 #define MQ_NVFP4_RECORD_WORDS (MQ_NVFP4_SECTION_WORDS * (MQ_NVFP4_SECTIONS + 1))
+/* words of an amax record behind its sections: the folded amax (float bits), three scale factors derived from it,
+ * then two state words of the carried-over amax (see MQ_NVFP4_CARRY_AMAX): REDO is 1 when the last carried submission
+ * quantized the tensor in its second pass, VOLATILE is 1 when the amax moved on the last carried submission */
+#define MQ_NVFP4_RECORD_AMAX_WORD (MQ_NVFP4_SECTION_WORDS * MQ_NVFP4_SECTIONS)
+#define MQ_NVFP4_RECORD_REDO_WORD (MQ_NVFP4_RECORD_AMAX_WORD + 4)
+#define MQ_NVFP4_RECORD_VOLATILE_WORD (MQ_NVFP4_RECORD_AMAX_WORD + 5)
 
 enum { MQ_BF16 = 0, MQ_F16 = 1, MQ_F32 = 2 };
 enum { MQ_OK = 0, MQ_ERR_ARG = -1, MQ_ERR_HIP = -2, MQ_ERR_UNSUPPORTED = -3 };
@@ -224,7 +230,10 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  * same job list again, amax records included and untouched in between, after at least one submission without the
  * flag, may set it on bf16 jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
  * submission, collects the new amax on the way, and quantizes a tensor a second time only if its amax changed
- * (results are identical either way; a weight tensor's amax rarely moves between two syncs). */
+ * (results are identical either way; a weight tensor's amax rarely moves between two syncs).  A tensor whose amax did
+ * change is marked volatile in its record: on the next submission the single pass only collects its amax and the
+ * second pass quantizes it (what the plain two-pass form costs), and it returns to the single pass once its amax
+ * has stayed the same for one submission. */
 enum {
     MQ_JOB_FP8_BLOCK = 0,
     MQ_JOB_FP8_BLOCKWISE_CAST = 1,

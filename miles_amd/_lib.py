@@ -51,6 +51,8 @@ SIGNATURES = {
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs
 NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
 NVFP4_CARRY_AMAX = 8                                      # MQ_NVFP4_CARRY_AMAX: NVFP4 jobs of a re-submitted list only
+# words of an amax record behind its four sections of 256 partial maxima (MQ_NVFP4_RECORD_*_WORD)
+RECORD_AMAX_WORD, RECORD_REDO_WORD, RECORD_VOLATILE_WORD = 1024, 1028, 1029
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
  JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM) = range(12)

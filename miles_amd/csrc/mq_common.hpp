@@ -82,14 +82,17 @@ __device__ __forceinline__ uint32_t wave_max(uint32_t v) {
 }
 
 // ---- exact division by a divisor shared by many elements -------------------------------------
-// q = RN(w / s) from y = RN(1/s):  q0 = RN(w*y); e = w - q0*s (exact in an FMA); q = RN(q0 + e*y).
+// q = RN(w / s) from y = RN(1/s):  q0 = RN(w*y); e = q0*s - w (exact in an FMA); q = RN(q0 - e*y).
 // For a numerator with at most 11 significant bits (bf16, fp16) this equals the correctly rounded
 // quotient for every divisor mantissa (exhaustive check: 2^23 divisors x all numerator mantissas),
 // provided no intermediate under/overflows; callers guard the exponent range of s.
+// The residual is taken as q0*s - w and subtracted (a source negation, free on v_fma_f32) rather than
+// w - q0*s added: for a zero numerator the first form gives e = +0 and q = q0 - (+0) = q0, which keeps
+// the sign of a -0 numerator as the division itself does; the second form would return +0 for -0.
 __device__ __forceinline__ float div_by_shared(float w, float s, float y) {
     float q0 = w * y;
-    float e = __builtin_fmaf(-q0, s, w);
-    return __builtin_fmaf(e, y, q0);
+    float e = __builtin_fmaf(q0, s, -w);
+    return __builtin_fmaf(-e, y, q0);
 }
 // divisor range in which div_by_shared is used; outside it kernels fall back to operator/
 __device__ __forceinline__ bool shared_div_ok(float s) {
@@ -155,12 +158,6 @@ __device__ __forceinline__ uint32_t hw_e4m3x2(float a, float b, uint32_t old) {
 __device__ __forceinline__ uint32_t hw_e4m3x4(float a, float b, float c, float d) {
     uint32_t r = hw_e4m3x2<false>(a, b, 0u);
     return hw_e4m3x2<true>(c, d, r);
-}
-// replace the sign bits of four e4m3 bytes by the sign bits of four bf16 values held in (a, b)
-// (a = elements 0,1; b = elements 2,3)
-__device__ __forceinline__ uint32_t copy_signs(uint32_t codes, uint32_t a, uint32_t b) {
-    const uint32_t hi_bytes = __builtin_amdgcn_perm(b, a, 0x07050301u);  // bytes 1,3 of a then 1,3 of b
-    return (codes & 0x7F7F7F7Fu) | (hi_bytes & 0x80808080u);
 }
 // two e4m3 bytes (low or high half of w) -> two floats
 template <bool HI>

@@ -151,7 +151,7 @@ __device__ __forceinline__ void act_quant_unit(const float f[8], void* y, void* 
     } else if (DT != MQ_F32 && finite && shared_div_ok(s)) {
         const float r = 1.0f / s;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = __builtin_copysignf(div_by_shared(f[i], s, r), f[i]);
+        for (int i = 0; i < 8; i++) q[i] = div_by_shared(f[i], s, r);
     } else {
         if (flags & MQ_ACT_ROUND_SCALE) s = ceil_pow2_normal(s);
 #pragma unroll

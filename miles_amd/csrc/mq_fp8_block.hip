@@ -161,12 +161,6 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
         u32x2 o;
         o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
         o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
-        if (MODE == 0) {
-            // the shared-divisor sequence returns +0 for a -0 numerator; the quotient's sign is the
-            // numerator's, so take the four sign bits straight from the bf16 inputs
-            o.x = copy_signs(o.x, v[i].x, v[i].y);
-            o.y = copy_signs(o.y, v[i].z, v[i].w);
-        }
         if (col_ok && r < M) st8(q + r * K + col, o);
     }
 }
@@ -270,8 +264,8 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restri
         q[r * K + c] = (uint8_t)sw_e4m3fn(v);
     }
 }
-// bf16 fast paths of the two.  The quotient x / s is the exact one (shared-divisor sequence; the division itself when
-// s leaves the guarded range); the sign of a -0 numerator is taken from the input pattern.
+// bf16 fast paths of the two.  The quotient x / s is the exact one (shared-divisor sequence, which keeps the sign of a
+// -0 numerator; the division itself when s leaves the guarded range).
 //
 // per channel: a row lives in the registers of ROWLANES lanes (up to 8 sixteen-byte units each), so it is read once:
 // amax across the lanes, one scale, codes.  ROWLANES = 64: four rows per workgroup, no LDS; 256: one row.
@@ -316,8 +310,8 @@ __global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* _
         for (int j = 0; j < 8; j++) f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
         u32x2 o;
         if (m < 0x7F80u) {
-            o.x = copy_signs(hw_e4m3x4(f[0], f[1], f[2], f[3]), v[u].x, v[u].y);
-            o.y = copy_signs(hw_e4m3x4(f[4], f[5], f[6], f[7]), v[u].z, v[u].w);
+            o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
+            o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
         } else {                                  // inf / NaN in the row: clamp and convert in software
             uint32_t c[8];
 #pragma unroll
@@ -381,8 +375,8 @@ __global__ __launch_bounds__(256) void fp8_tensor_quant_bf16_kernel(const uint16
         }
         u32x2 o;
         if (abits < 0x7F800000u) {
-            o.x = copy_signs(hw_e4m3x4(f[0], f[1], f[2], f[3]), v[i].x, v[i].y);
-            o.y = copy_signs(hw_e4m3x4(f[4], f[5], f[6], f[7]), v[i].z, v[i].w);
+            o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
+            o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
         } else {
             uint32_t c[8];
 #pragma unroll

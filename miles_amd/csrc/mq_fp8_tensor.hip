@@ -8,7 +8,10 @@
 // with NVFP4 (256 partial maxima per tensor, plain stores), a fold kernel (one workgroup per tensor: amax, scale out,
 // sections cleared) and the flat quantize kernel.  Later runs of the same list carry the amax over like NVFP4 does:
 // pass 1 quantizes with the amax the record kept, collecting the new partial maxima with one atomic max per workgroup;
-// the fold compares; pass 2 quantizes again only the tensors whose amax moved.
+// the fold compares; pass 2 quantizes again only the tensors whose amax moved.  A tensor whose amax moved takes the
+// two-pass form on the next run (pass 1 only collects its amax) and returns to the single pass once the amax has held.
+#include <stdlib.h>
+
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -31,7 +34,16 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const FlatTable ta
     __syncthreads();
     if (threadIdx.x == 0) {
         m = umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3]));
-        if (MODE == 2) rec[kRecRedo] = rec[kRecAmax] != m;
+        if (MODE == 2) {
+            // a record whose amax moved is marked volatile: the next carried run only collects its amax in the single
+            // pass and quantizes in the second one (the two-pass cost instead of two quantizations), until it holds still
+            const bool moved = rec[kRecAmax] != m;
+            rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;
+            rec[kRecVolatile] = moved ? 1u : 0u;
+        } else {
+            rec[kRecRedo] = 0;
+            rec[kRecVolatile] = 0;
+        }
         rec[kRecAmax] = m;
         float amax = u2f(m);
         if (amax < floor_v) amax = floor_v;          // a NaN amax stays NaN, as torch's clamp leaves it
@@ -71,8 +83,8 @@ __device__ __forceinline__ uint32_t fp8_tensor_quant_units(const FlatJob& job, c
         }
         u32x2 o;
         if (abits < 0x7F800000u) {
-            o.x = copy_signs(hw_e4m3x4(f[0], f[1], f[2], f[3]), v[i].x, v[i].y);
-            o.y = copy_signs(hw_e4m3x4(f[4], f[5], f[6], f[7]), v[i].z, v[i].w);
+            o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
+            o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
         } else {                                   // inf / NaN amax: clamp and convert in software
             uint32_t c[8];
 #pragma unroll
@@ -100,7 +112,20 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Flat
     }
     const int64_t base = flat_block(tab) * kPerBlock;
     if (base >= job.units) return;
-    uint32_t seen = fp8_tensor_quant_units(job, base, t, floor_v);
+    uint32_t seen;
+    if (PASS == 1 && ((const uint32_t*)job.aux)[kRecVolatile] != 0) {
+        const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+        uint32_t m2 = 0;
+#pragma unroll
+        for (int i = 0; i < kFtUnroll; i++) {
+            const int64_t unit = base + i * kFtThreads + t;
+            const u32x4 v = unit < job.units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+            m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+        }
+        seen = hmax_u16(m2);
+    } else {
+        seen = fp8_tensor_quant_units(job, base, t, floor_v);
+    }
     if (PASS == 1) {
         __shared__ uint32_t wave_seen[kFtThreads / 64];
         seen = wave_max(seen);
@@ -143,7 +168,8 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
         if (tab.max_blocks > 0) hipLaunchKernelGGL(fp8_tensor_quant_kernel<1>, grid, dim3(kFtThreads), 0, st, tab, floor_v);
         hipLaunchKernelGGL(fp8_tensor_fold_kernel<2>, folds, blk, 0, st, tab, floor_v);
         if (tab.max_blocks > 0) {
-            const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
+            static const int redo_cap = getenv("MQ_NV_REDO_BLOCKS") ? atoi(getenv("MQ_NV_REDO_BLOCKS")) : kSectionWords;
+            const unsigned redo = tab.max_blocks < redo_cap ? (unsigned)tab.max_blocks : (unsigned)redo_cap;
             hipLaunchKernelGGL(fp8_tensor_quant_kernel<2>, dim3(redo, (unsigned)tab.n), dim3(kFtThreads), 0, st, tab, floor_v);
         }
         return mq_check_launch("fp8 per-tensor quant (carried-over amax)");

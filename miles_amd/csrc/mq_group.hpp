@@ -133,6 +133,7 @@ constexpr int kSectionWords = 256;      // MQ_NVFP4_SECTION_WORDS: workgroups of
 constexpr int kRecordSections = 4;      // MQ_NVFP4_SECTIONS
 constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (float bits)
 constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
+constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last run: the next carried run collects the amax first
 
 struct CopyJob {      // one run of bytes
     const uint8_t* src;

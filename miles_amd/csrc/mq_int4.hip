@@ -469,7 +469,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_fake_rows_kernel(const void* 
     const float top = SYM ? mx : __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
     if (DT != MQ_F32 && shared_div_ok(s) && top * y < 1e30f) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(__builtin_copysignf(div_by_shared(f[i], s, y), f[i]));
+        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(div_by_shared(f[i], s, y));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s);

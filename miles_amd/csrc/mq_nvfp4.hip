@@ -13,6 +13,8 @@
 // Pass 2 (mq_nvfp4_quant) reads those two factors with a scalar load; two lanes own one 16-element block
 // (16 bytes each), the block amax is one DPP step, and each lane emits four bytes of codes.  A gate/up pair
 // writes two sections of one record.
+#include <stdlib.h>
+
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -114,6 +116,10 @@ constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 //   partial maxima with atomic max (see the carried-over amax below).  MODE 2 additionally checks the amax and scales
 //   the record held before against the new ones: all four words equal means the codes just written with the old values
 //   are final (kRecRedo = 0); otherwise the new values are stored and kRecRedo = 1 asks for a second quantization.
+//   A record whose amax moved is marked volatile (kRecVolatile): on the next carried sync the single pass only collects
+//   its partial maxima (no codes are written with an amax that is likely stale again) and the second pass quantizes it
+//   with the fresh amax -- the cost of the plain two-pass form, instead of two full quantizations.  The mark is dropped
+//   as soon as the amax has held still for one sync.
 template <int MODE>
 __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, float numer) {
     __shared__ uint32_t lds4[4];
@@ -132,9 +138,15 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, fl
     if (threadIdx.x == 0) {
         const float amax = u2f(umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3])));
         const NvScales gs = nv_scales(amax, numer);
-        if (MODE == 2)
-            rec[kRecRedo] = !(rec[kRecAmax] == f2u(amax) && rec[kRecEncSixth] == f2u(gs.enc_sixth) &&
-                              rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
+        if (MODE == 2) {
+            const bool moved = !(rec[kRecAmax] == f2u(amax) && rec[kRecEncSixth] == f2u(gs.enc_sixth) &&
+                                 rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
+            rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;     // a volatile record has no codes yet
+            rec[kRecVolatile] = moved ? 1u : 0u;
+        } else if (MODE == 1) {
+            rec[kRecRedo] = 0;
+            rec[kRecVolatile] = 0;
+        }
         rec[kRecAmax] = f2u(amax);
         rec[kRecEncSixth] = f2u(gs.enc_sixth);
         rec[kRecSDec] = f2u(gs.s_dec);
@@ -305,6 +317,20 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
     return seen;
 }
 
+// the largest |element| (bf16 bits) this lane sees in kNvThreads * kNvUnroll units starting at `base`: what the single
+// pass does for a record marked volatile
+__device__ __forceinline__ uint32_t nvfp4_amax_units(const FlatJob& job, const int64_t base, const int t) {
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t m2 = 0;
+#pragma unroll
+    for (int i = 0; i < kNvUnroll; i++) {
+        const int64_t unit = base + i * kNvThreads + t;
+        const u32x4 v = unit < job.units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        m2 = max2_u16(m2, max2_u16(max2_u16(abs2(v.x), abs2(v.y)), max2_u16(abs2(v.z), abs2(v.w))));
+    }
+    return hmax_u16(m2);
+}
+
 // Carried-over amax.  A weight tensor's amax rarely changes from one sync to the next (the largest element has to move
 // to another bf16 value), and the amax record of a replayed job list still holds the last sync's amax and scales.
 // PASS 1 quantizes with those in a single read of the tensor and collects this sync's partial maxima on the way (one
@@ -324,7 +350,9 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Flat
     }
     const int64_t base = flat_block(tab) * kPerBlock;
     if (base >= job.units) return;
-    uint32_t seen = nvfp4_quant_units<FOS>(job, base, t, denom);
+    uint32_t seen;
+    if (PASS == 1 && ((const uint32_t*)job.aux)[kRecVolatile] != 0) seen = nvfp4_amax_units(job, base, t);
+    else seen = nvfp4_quant_units<FOS>(job, base, t, denom);
     if (PASS == 1) {
         __shared__ uint32_t wave_seen[kNvThreads / 64];
         seen = wave_max(seen);
@@ -523,7 +551,8 @@ int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mod
         if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
         hipLaunchKernelGGL(nvfp4_fold_kernel<2>, folds, blk, 0, st, tab, numer);
         if (tab.max_blocks > 0) {
-            const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
+            static const int redo_cap = getenv("MQ_NV_REDO_BLOCKS") ? atoi(getenv("MQ_NV_REDO_BLOCKS")) : kSectionWords;
+            const unsigned redo_blocks = tab.max_blocks < redo_cap ? (unsigned)tab.max_blocks : (unsigned)redo_cap;
             launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)tab.n), st);
         }
         return mq_check_launch("nvfp4 quant (carried-over amax)");

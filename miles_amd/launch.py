@@ -76,6 +76,18 @@ class JobBatch:
             self._array = None
         return flagged
 
+    def amax_records(self) -> list[torch.Tensor]:
+        """The amax records of the NVFP4 and per-tensor FP8 jobs, one per tensor or gate/up pair, in job order (int32
+        tensors; words `_lib.RECORD_AMAX_WORD`, `RECORD_REDO_WORD`, `RECORD_VOLATILE_WORD` hold the folded amax and
+        the state of the carried-over amax after a run)."""
+        by_address = {t.data_ptr(): t for t in self._keep}
+        seen, out = set(), []
+        for r in self._records:
+            if r[self.KIND] in (_lib.JOB_NVFP4, _lib.JOB_FP8_TENSOR) and r[self.AUX] not in seen:
+                seen.add(r[self.AUX])
+                out.append(by_address[r[self.AUX]])
+        return out
+
     def hold(self, tensor: torch.Tensor) -> None:
         """Keep a tensor alive for as long as the batch exists."""
         self._keep.append(tensor)

@@ -69,4 +69,8 @@ def test_python_constants_match_the_header():
     assert _lib.MAX_GROUP == int(defines["MQ_MAX_GROUP"])
     words = int(defines["MQ_NVFP4_SECTION_WORDS"]) * (int(defines["MQ_NVFP4_SECTIONS"]) + 1)
     assert AMAX_RECORD_WORDS == _AMAX_RECORD_WORDS == words
+    amax_word = int(defines["MQ_NVFP4_SECTION_WORDS"]) * int(defines["MQ_NVFP4_SECTIONS"])
+    assert defines["MQ_NVFP4_RECORD_REDO_WORD"] == "(MQ_NVFP4_RECORD_AMAX_WORD + 4)"
+    assert defines["MQ_NVFP4_RECORD_VOLATILE_WORD"] == "(MQ_NVFP4_RECORD_AMAX_WORD + 5)"
+    assert (_lib.RECORD_AMAX_WORD, _lib.RECORD_REDO_WORD, _lib.RECORD_VOLATILE_WORD) == (amax_word, amax_word + 4, amax_word + 5)
     assert (_lib.MQ_BF16, _lib.MQ_F16, _lib.MQ_F32) == (enums["MQ_BF16"], enums["MQ_F16"], enums["MQ_F32"])

@@ -1278,9 +1278,18 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
             for j, (g_, w_) in enumerate(zip(pair_out[half], want[half])):
                 _assert_same(g_, w_, f"{what}: pair half {half} output {j}")
 
+    from miles_amd import _lib
+
+    def state():
+        """(second pass ran, marked volatile) per record, in job order: tensors 0-2, the pair, tensors 3-5"""
+        recs = [r.cpu() for r in batch.amax_records()]
+        return [int(r[_lib.RECORD_REDO_WORD]) for r in recs], [int(r[_lib.RECORD_VOLATILE_WORD]) for r in recs]
+
     check("first run (two passes)")
     assert batch.carry_amax() == len(shapes) + 2
+    assert len(batch.amax_records()) == len(shapes) + 1
     check("same weights (every amax carried)")
+    assert state() == ([0] * 7, [0] * 7)
     check("same weights again")
     for w in dev + pair_dev:                       # new values everywhere, every amax as before
         top = w.abs().flatten().argmax()
@@ -1288,11 +1297,23 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
         w.mul_(0.75)
         w.view(-1)[top] = keep
     check("changed data, same amax")
+    assert state() == ([0] * 7, [0] * 7)
     dev[1].mul_(3.0)                               # these amax move: tensor 1 up, tensor 4 down, the pair through its second half
     dev[4].mul_(0.25)
     pair_dev[1].mul_(5.0)
     check("three amax moved")
+    moved = [0, 1, 0, 1, 0, 1, 0]                  # records: tensors 0, 1, 2, the pair, tensors 3, 4, 5
+    assert state() == (moved, moved)               # quantized twice, and marked: the next run collects their amax first
     check("and stayed")
+    assert state() == (moved, [0] * 7)             # the marked ones took the two-pass form once more, then settled
+    check("settled")
+    assert state() == ([0] * 7, [0] * 7)
+    dev[1].mul_(0.5)
+    check("tensor 1 moved")
+    dev[1].mul_(0.5)
+    dev[3].mul_(2.0)
+    check("tensor 1 moved again while marked, tensor 3 for the first time")
+    assert state() == ([0, 1, 0, 0, 1, 0, 0], [0, 1, 0, 0, 1, 0, 0])
     dev[2].zero_()                                 # amax 0
     dev[0].view(-1)[7] = float("inf")              # amax inf
     check("zero tensor and an infinity")

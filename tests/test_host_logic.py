@@ -538,3 +538,27 @@ def test_mimo_name_map():
         conv(M + "something_else.weight", w)
     with pytest.raises(ValueError, match="Invalid MTP parameter name"):
         conv("module.module.mtp.weight", w)
+
+
+def test_shared_divisor_division_is_exact_and_keeps_the_sign_of_zero():
+    # The FP8 / INT4 kernels divide many elements by one scale s with y = RN(1/s):
+    #   q0 = x*y; e = fma(q0, s, -x); q = fma(-e, y, q0)
+    # For bf16 / fp16 numerators this must be the IEEE quotient, signed zeros included (the exhaustive sweep over all
+    # 2^23 divisor mantissas x all numerator mantissas was run once in C; this is a large sample plus the zero cases).
+    # The two FMAs are evaluated in float64: the residual e is exactly representable, and q0 - e*y has fewer than 53
+    # significant bits between its largest and smallest term, so float64 holds both results before the one rounding.
+    import numpy as np
+    rng = np.random.default_rng(7)
+    n = 1 << 21
+    s = ((rng.integers(90, 170, size=n, dtype=np.uint32) << np.uint32(23)) | rng.integers(0, 1 << 23, size=n, dtype=np.uint32)).view(np.float32)
+    xm = rng.integers(0, 1 << 10, size=n, dtype=np.uint32) << np.uint32(13)          # up to 11 significant bits
+    x = ((rng.integers(0, 2, size=n, dtype=np.uint32) << np.uint32(31)) | (rng.integers(100, 150, size=n, dtype=np.uint32) << np.uint32(23)) | xm).view(np.float32)
+    x[:1024:2] = np.float32(-0.0)
+    x[1:1024:2] = np.float32(0.0)
+    y = np.float32(1.0) / s
+    q0 = x * y
+    e = (q0.astype(np.float64) * s.astype(np.float64) - x.astype(np.float64)).astype(np.float32)
+    q = (q0.astype(np.float64) - e.astype(np.float64) * y.astype(np.float64)).astype(np.float32)
+    want = x / s
+    assert np.array_equal(q.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(np.signbit(q[:1024]), np.signbit(x[:1024])) and not q[:1024].any()
