@@ -3,19 +3,23 @@
 The shapes, names and addresses of a training model's parameters do not change between RL steps, so the
 per-parameter Python work of a sync (name mapping, quantizer dispatch, output allocation, bucketing) only
 has to happen once.  `SyncPlan.record` runs the iterator once under `launch.recording()`: every quantizer
-call allocates its outputs and records its job; the plan keeps the job list, the output tensors and the
-buckets.  `SyncPlan.replay` then re-runs the jobs -- a handful of `mq_run_jobs` calls, each a few grouped
-kernel launches -- and hands out the same buckets again, now holding the freshly quantized values.
+call allocates its outputs and records its job; the plan keeps the job list and the buckets.
+`SyncPlan.replay` then runs the jobs -- a handful of `mq_run_jobs` calls, each a few grouped kernel launches --
+and hands out the buckets, holding the freshly quantized values.
+
+Memory: the outputs live in a ring of arenas, one bucket per arena (`plan_memory.Placement`), not in one buffer
+per tensor, so a plan holds `ring` x the largest bucket (about `update_weight_buffer_size` each) however large the
+model is -- the bound the reference keeps by producing, sending and dropping one bucket at a time
+(miles/backends/training_utils/weight_update/updater.py:150-160).  A bucket is valid from the moment it is handed
+out until the consumer returns from it; work the consumer queued on the launch stream is ordered before the reuse.
 
 Replay is only valid when every kernel input aliases live parameter storage (views such as gate/up chunks or
 row-blocked q/k/v are fine; a name map that materialises a copy is not): `replayable` says so, and the
-updater falls back to the full iterator when it is False.  The plan owns its output tensors: a bucket's
-contents are valid until the next replay.
+updater falls back to the full iterator when it is False.
 """
 
 from __future__ import annotations
 
-import bisect
 import operator
 from collections.abc import Iterator, Mapping
 
@@ -23,8 +27,8 @@ import torch
 
 from miles_amd import _lib, launch
 from miles_amd.weight_update.bucketing import Unit
-from miles_amd.weight_update.packed_bucket import PackedBucket, layout
 from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorBase
+from miles_amd.weight_update.plan_memory import Placement
 
 
 def weights_signature(weights: Mapping[str, torch.Tensor]) -> tuple:
@@ -32,18 +36,16 @@ def weights_signature(weights: Mapping[str, torch.Tensor]) -> tuple:
     return tuple((name, t.data_ptr(), tuple(t.shape), t.dtype) for name, t in weights.items())
 
 
-class _NotPackable(Exception):
-    """A bucket holds a tensor that can be neither produced in place in a flat payload nor byte-copied into it."""
-
-
 class SyncPlan:
     def __init__(self, batch: launch.JobBatch, buckets: list[Unit], jobs_done_at_bucket: list[int],
-                 signature: tuple, replayable: bool) -> None:
+                 signature: tuple, replayable: bool, ring: int | None = None, arena_bytes: int = 0) -> None:
         self.batch = batch
         self.buckets = buckets
         self.jobs_done_at_bucket = jobs_done_at_bucket
         self.signature = signature
         self.replayable = replayable
+        self.ring = ring or max(len(buckets), 1)     # arenas the buckets rotate through
+        self.arena_bytes = arena_bytes              # device memory the plan's outputs occupy
         self._marks: list[int] | None = None
         self._completed = 0         # full replays so far
         self._names: list[str] = []
@@ -58,137 +60,32 @@ class SyncPlan:
 
     @classmethod
     def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor], *,
-               packed: bool = False) -> "SyncPlan":
-        """Run one full sync, keeping everything needed to repeat it.  With `packed`, every bucket becomes a
-        `PackedBucket`: the quantizer jobs are re-pointed at their final place in the bucket's flat payload and
-        pass-through tensors get copy jobs, so a replay produces the transport payload with no flattening pass."""
-        buckets: list[Unit] = []
-        marks: list[int] = []
+               packed: bool = False, ring: int | None = 2) -> "SyncPlan":
+        """Run the per-parameter work of one full sync, keeping everything needed to repeat it.  Nothing is
+        executed here: `replay()` produces the buckets, the first time as every later time.
+
+        Every tensor a job writes gets its place in one of `ring` output arenas (bucket k in arena k mod ring, None:
+        an arena per bucket), so the plan holds `ring` buckets' worth of output memory whatever the size of the model
+        (`plan_memory.Placement`).  With `packed`, every bucket becomes a `PackedBucket`: the quantizer jobs are
+        pointed at their final place in the bucket's flat payload and pass-through tensors get copy jobs, so a
+        replay produces the transport payload with no flattening pass."""
         with launch.recording() as batch:
+            batch.device = next((t.device for t in weights.values() if t.device.type == "cuda"), None)
+            placement = Placement(batch, weights, packed=packed, ring=ring)
             for bucket in iterator.iter_hf_weights(weights):
-                buckets.append(bucket)
-                marks.append(len(batch))   # every job of this bucket (and maybe some of the next) is recorded
-        device = next((t.device for t in weights.values() if t.device.type == "cuda"), None)
-        batch.device = batch.device or device
-        # every handed-out tensor must be reproduced by a replay: written by a job, a view of live parameter
-        # storage, or a declared constant (a tensor some torch op materialised would go stale)
-        spans = cls._weight_spans(weights)
-        produced = batch.output_pointers() | batch.constants
-        handed_out_ok = all(t.numel() == 0 or t.data_ptr() in produced or cls._in_spans(spans, t.data_ptr())
-                            for bucket in buckets for _, t in bucket)
-        packable = True
-        if packed:
-            try:
-                buckets, marks = cls._pack(batch, buckets, marks)
-            except _NotPackable:
-                packable = False       # the updater flattens such buckets after the fact (one extra copy), every sync
+                placement.take(bucket)       # every job of this bucket (and maybe some of the next) is recorded
+            del bucket
+        buckets, marks, ring, arena_bytes = placement.finish()
         batch.freeze()
-        replayable = batch.direct_calls == 0 and handed_out_ok and packable and cls._inputs_alias(weights, batch)
-        plan = cls(batch, buckets, marks, weights_signature(weights), replayable)
+        # a replay reproduces the sync only if no kernel bypassed the job list, every job input is live parameter
+        # storage, a declared constant or made by a job, and every handed-out tensor is one of those too (a tensor
+        # that some torch op materialised would go stale)
+        replayable = (batch.direct_calls == 0 and placement.handed_out_ok and placement.packable
+                      and placement.inputs_alias)
+        plan = cls(batch, buckets, marks, weights_signature(weights), replayable, ring, arena_bytes)
+        plan.packable = placement.packable
         plan.remember(weights)
-        for _ in plan.replay():     # the first execution uses the same launch partition as every replay
-            pass
         return plan
-
-    @staticmethod
-    def _pack(batch: launch.JobBatch, buckets: list[Unit], marks: list[int]):
-        """Move every bucket into one flat payload.  A tensor that some job writes (codes, scales, NVFP4 global
-        scale) is re-homed by patching that job's pointer; anything else is copied by a job appended to the
-        bucket's range.  Returns the packed buckets and the new job marks."""
-        out_fields = (3, 4, 6)       # out, scale, aux2 of a job record
-        writers: dict[int, list[tuple[int, int]]] = {}
-        for ri, rec in enumerate(batch.records):
-            for f in out_fields:
-                if rec[f] is not None and rec[0] != _lib.JOB_COPY:
-                    writers.setdefault(rec[f], []).append((ri, f))
-        records = [list(r) for r in batch.records]
-        # byte copies recorded by a name map (regrouped q / k / v): [destination, record index, bytes], by destination
-        gathers = sorted((rec[3], ri, rec[7] * rec[8]) for ri, rec in enumerate(batch.records)
-                         if rec[0] == _lib.JOB_COPY and rec[3] is not None)
-        gather_starts = [g[0] for g in gathers]
-        new_buckets: list[Unit] = []
-        copies_of: list[list[tuple]] = []
-        for bucket in buckets:      # first re-point every job (a bucket's range may hold jobs of the next bucket)
-            metas, total = layout(bucket)
-            device = bucket[0][1].device if bucket else batch.device
-            flat = torch.empty(total, dtype=torch.uint8, device=device)
-            packed = PackedBucket(flat, metas)
-            copies = []
-            for (name, old), (_, new) in zip(bucket, packed):
-                hits = writers.get(old.data_ptr()) if old.is_contiguous() and old.numel() else None
-                if not old.is_contiguous() and old.numel():
-                    # the transposed view of packed UE8M0 scales: its job can write the contiguous form straight into the slot
-                    packers = [ri for ri, f in writers.get(old.data_ptr(), ()) if records[ri][launch.JobBatch.KIND] == _lib.JOB_UE8M0_PACK]
-                    if packers and new.data_ptr() % 4 == 0:
-                        for ri in packers:
-                            records[ri][launch.JobBatch.OUT], records[ri][launch.JobBatch.LD] = new.data_ptr(), 1
-                        continue
-                # codes written by a quantizer need their slot on a 16-byte boundary for the tuned kernels (a row-blocked
-                # FP8 job has no other kernel at all); a slot that follows, say, a 12-byte scale grid is filled by a copy
-                if hits and new.data_ptr() % 16 and any(f == 3 for _, f in hits):
-                    hits = None
-                if not hits and old.is_contiguous() and old.numel():
-                    # a tensor that copy jobs assemble piece by piece is assembled in its payload slot instead
-                    lo, nbytes = old.data_ptr(), old.numel() * old.element_size()
-                    first = bisect.bisect_left(gather_starts, lo)
-                    pieces, end = [], lo
-                    for dst, ri, size in gathers[first:]:
-                        if dst != end or dst >= lo + nbytes:
-                            break
-                        pieces.append(ri)
-                        end = dst + size
-                    if pieces and end == lo + nbytes:
-                        for ri in pieces:
-                            records[ri][3] += new.data_ptr() - lo
-                        continue
-                if hits:
-                    for ri, f in hits:
-                        records[ri][f] = new.data_ptr()
-                elif old.numel():
-                    if not old.is_contiguous():
-                        raise _NotPackable(f"{name} is a strided pass-through tensor: it needs a gathering copy")
-                    nbytes = old.numel() * old.element_size()
-                    copies.append((_lib.JOB_COPY, 0, old.data_ptr(), new.data_ptr(), None, None, None, 1, nbytes, nbytes,
-                                   0, 0, 0, 0))
-                    batch.hold(old)
-            batch.hold(flat)
-            new_buckets.append(packed)
-            copies_of.append(copies)
-        new_records: list[tuple] = []
-        new_marks: list[int] = []
-        done = 0
-        for copies, mark in zip(copies_of, marks):     # then lay the list out again with each bucket's copies at its end
-            new_records.extend(tuple(r) for r in records[done:max(done, mark)])
-            done = max(done, mark)
-            new_records.extend(copies)
-            new_marks.append(len(new_records))
-        new_records.extend(tuple(r) for r in records[done:])
-        still_written = {rec[f] for rec in records for f in out_fields if rec[f] is not None}
-        rehomed = {t.data_ptr() for bucket in buckets for _, t in bucket
-                   if t.numel() and t.data_ptr() in writers and t.data_ptr() not in still_written}
-        # drop the first homes of re-pointed outputs
-        batch.replace_records(new_records, keep=[t for t in batch.held if t.data_ptr() not in rehomed])
-        return new_buckets, new_marks
-
-    @staticmethod
-    def _weight_spans(weights: Mapping[str, torch.Tensor]):
-        spans = sorted((t.untyped_storage().data_ptr(), t.untyped_storage().data_ptr() + t.untyped_storage().nbytes())
-                       for t in weights.values())
-        return [s for s, _ in spans], spans
-
-    @staticmethod
-    def _in_spans(spans, ptr: int) -> bool:
-        starts, ranges = spans
-        i = bisect.bisect_right(starts, ptr) - 1
-        return i >= 0 and ptr < ranges[i][1]
-
-    @classmethod
-    def _inputs_alias(cls, weights: Mapping[str, torch.Tensor], batch: launch.JobBatch) -> bool:
-        """Every job input is live parameter storage, a declared constant (copy jobs move constants too), or
-        something a job of the list writes (a copy that moves quantizer output into a misaligned payload slot)."""
-        spans = cls._weight_spans(weights)
-        produced = batch.output_pointers()
-        return all(cls._in_spans(spans, ptr) or ptr in batch.constants or ptr in produced for ptr in batch.input_pointers())
 
     def matches(self, weights: Mapping[str, torch.Tensor]) -> bool:
         """True when `weights` is the parameter set the plan was recorded on.  Between RL steps the mapping holds
@@ -213,8 +110,8 @@ class SyncPlan:
         `MAX_GROUP` jobs per launch, counted from the start of a submission, so a bucket of 330 small expert tensors
         ends in a launch of ten, which mostly ramps up and down.  When that last launch would cover fewer than
         `SMALL_LAUNCH_ELEMENTS` elements the submission runs on into the next bucket's jobs up to the full group (the
-        plan owns every output tensor, so running ahead costs nothing; measured on the 18 432-tensor MXFP8 sync:
-        14.6 -> 14.1 ms).  Buckets of large tensors are submitted as they are -- merging their launches made the
+        next bucket's outputs live in another arena, so running ahead by less than `ring` buckets is safe; measured on
+        the 18 432-tensor MXFP8 sync: 14.6 -> 14.1 ms).  Buckets of large tensors are submitted as they are -- merging their launches made the
         Qwen3-4B FP8 sync 1 % slower.  A cut never falls between NVFP4 jobs that share an amax record."""
         if self._marks is None:
             records, total, done, marks = self.batch.records, len(self.batch), 0, []
@@ -224,7 +121,9 @@ class SyncPlan:
                     tail = (mark - done) % group
                     tail_elements = sum(r[7] * r[8] for r in records[mark - tail:mark])
                     if tail and tail_elements < self.SMALL_LAUNCH_ELEMENTS:
-                        mark = min(total, mark + group - tail)
+                        # bucket k + ring writes the arena of bucket k, which the consumer is about to read
+                        ahead = self.jobs_done_at_bucket[min(len(marks) + self.ring - 1, len(self.jobs_done_at_bucket) - 1)]
+                        mark = max(mark, min(total, mark + group - tail, ahead))
                         while (0 < mark < total and records[mark][0] == _lib.JOB_NVFP4
                                and records[mark - 1][0] == _lib.JOB_NVFP4 and records[mark][5] == records[mark - 1][5]):
                             mark += 1
@@ -246,7 +145,3 @@ class SyncPlan:
             # them and repeat a tensor only when its amax moved
             self.batch.carry_amax()
 
-    def replay_all(self) -> list[Unit]:
-        """Whole model in one submission (fewest launches); returns every bucket."""
-        self.batch.run()
-        return self.buckets

@@ -5,8 +5,9 @@ Single-process form of the reference's `WeightUpdater.update_weights`
 transfer protocols of the reference are outside this path; what remains is the loop
 `for bucket in iterator.iter_hf_weights(weights): protocol.send_bucket(bucket)` wrapped in the same two
 wall-clock spans ("update_weights_implementation", "finalize_and_resume_engines").  `send_bucket` is any
-callable taking a list of (hf_name, tensor).  After the first sync the recorded `SyncPlan` is replayed as long
-as the parameter set is unchanged.
+callable taking a list of (hf_name, tensor); as in the reference, a bucket belongs to the consumer only until
+`send_bucket` returns (its memory is reused for a later bucket).  After the first sync the recorded `SyncPlan` is
+replayed as long as the parameter set is unchanged.
 """
 
 from __future__ import annotations
@@ -43,7 +44,7 @@ class WeightUpdater:
     def __init__(self, args: Namespace, *, weights_getter: Callable[[], Mapping[str, torch.Tensor]], model_name: str,
                  quantization_config: dict | None, send_bucket: Callable[[Unit], None],
                  packed_weight_basenames: set[str] | None = None, use_plan: bool = True,
-                 packed_buckets: bool = False) -> None:
+                 packed_buckets: bool = False, plan_arenas: int | None = 2) -> None:
         self.args = Namespace(**vars(args))
         if _fp8_row_block_views_ok(self.args, quantization_config):
             self.args.qkv_row_block_views = True
@@ -51,12 +52,15 @@ class WeightUpdater:
         self.send_bucket = send_bucket
         self.use_plan = use_plan
         self.packed_buckets = packed_buckets   # hand out PackedBucket payloads (the reference's broadcast_packed mode)
+        # output arenas of a recorded sync: bucket k lives in arena k mod plan_arenas and is valid until `send_bucket`
+        # returns from it (the reference drops a bucket after sending it); None keeps every bucket in an arena of its own
+        self.plan_arenas = plan_arenas
         self.weight_version = 0
         self._iterator = _RowBlockAwareIterator(self.args, model_name=model_name,
                                                 quantization_config=quantization_config,
                                                 packed_weight_basenames=packed_weight_basenames)
         self._plan: SyncPlan | None = None
-        self._packed_plan_refused = False
+        self._plan_refused = False
         self._metrics: dict[str, float] = {}
 
     def pop_metrics(self) -> dict[str, float]:
@@ -79,15 +83,18 @@ class WeightUpdater:
         if self.use_plan and self._plan is not None and self._plan.matches(weights):
             yield from self._plan.replay()
             return
-        if self.use_plan and not self._packed_plan_refused:
-            plan = SyncPlan.record(self._iterator, weights, packed=self.packed_buckets)
-            if plan.replayable or not self.packed_buckets:
+        if self.use_plan and not self._plan_refused:
+            self._plan = None                      # a plan for another parameter set: let its arenas go first
+            plan = SyncPlan.record(self._iterator, weights, packed=self.packed_buckets, ring=self.plan_arenas)
+            if plan.replayable:
                 self._plan = plan
-                yield from plan.buckets
+                yield from plan.replay()
                 return
-            # a packed plan re-points job outputs, which is only safe to keep when it can be replayed; a model that
-            # cannot be planned this way is not tried again (recording runs the whole sync once for nothing)
-            self._packed_plan_refused = True
+            # A sync that a replay cannot reproduce (a kernel outside the job list, a tensor some torch op materialised,
+            # a bucket that cannot be laid out as a payload) streams through the iterator, this time and every later
+            # time: recording it again would repeat the per-parameter work of a whole sync for nothing.
+            self._plan_refused = True
+            del plan
         for bucket in self._iterator.iter_hf_weights(weights):
             yield pack_bucket(bucket) if self.packed_buckets else bucket
 

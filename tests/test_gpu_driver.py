@@ -74,9 +74,19 @@ def _expected_fp8(oracle, cpu_params):
     return out
 
 
+def _snapshot(bucket):
+    """What a consumer must do to keep a bucket past its own send: copy it (the sync reuses the memory for a later
+    bucket).  A packed bucket is copied as one payload."""
+    from miles_amd.weight_update.packed_bucket import PackedBucket
+
+    if isinstance(bucket, PackedBucket):
+        return PackedBucket(bucket.flat.clone(), bucket.metadata)
+    return [(n, t.clone()) for n, t in bucket]
+
+
 def _run(updater):
     got = []
-    updater.send_bucket = lambda bucket: got.append(list(bucket))
+    updater.send_bucket = lambda bucket: got.append(_snapshot(bucket))
     updater.update_weights()
     torch.cuda.synchronize()
     return got
@@ -104,10 +114,10 @@ def test_dense_fp8_sync_matches_oracle_and_replays(oracle, use_plan):
     cpu2 = _dense_model(500)
     for k in dev:
         dev[k].copy_(cpu2[k])
+    plan = upd._plan
     buckets2 = _run(upd)
     if use_plan:
-        assert upd._plan is not None and upd._plan.replayable
-        assert buckets2[0][0][1].data_ptr() == buckets[0][0][1].data_ptr()   # replay reuses the plan's outputs
+        assert upd._plan is plan and plan is not None and plan.replayable      # the same plan, replayed
     want2 = _expected_fp8(oracle, cpu2)
     for (n, g), (_, w) in zip([nt for b in buckets2 for nt in b], want2):
         _same(g, w, n + " (second sync)")
@@ -355,8 +365,9 @@ def test_packed_buckets_fp8_plan_writes_payload_in_place(oracle):
 
     cpu = _dense_model(10)
     dev = {k: v.to(DEV) for k, v in cpu.items()}
+    # plan_arenas=None: every bucket keeps an arena of its own, so all of them can be looked at after the sync
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG,
-                        send_bucket=None, packed_buckets=True)
+                        send_bucket=None, packed_buckets=True, plan_arenas=None)
     got = []
     upd.send_bucket = got.append
     upd.update_weights()
@@ -410,7 +421,7 @@ def test_packed_buckets_without_plan_and_layout_errors(oracle):
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG,
                         send_bucket=None, use_plan=False, packed_buckets=True)
     got = []
-    upd.send_bucket = got.append
+    upd.send_bucket = lambda b: got.append(_snapshot(b))
     upd.update_weights()
     torch.cuda.synchronize()
     it = iter(_expected_fp8(oracle, cpu))
@@ -476,7 +487,7 @@ def test_packed_sync_of_a_model_with_strided_pass_through_tensors_falls_back_to_
     monkeypatch.setattr(upd._iterator, "iter_hf_weights", fake_iter)
     for step in range(3):
         got = []
-        upd.send_bucket = got.append
+        upd.send_bucket = lambda b: got.append(_snapshot(b))
         upd.update_weights()
         torch.cuda.synchronize()
         assert len(got) == 1 and isinstance(got[0], PackedBucket)
@@ -541,7 +552,7 @@ def test_packed_buckets_int4_moe_two_syncs(oracle):
         for k in dev:
             dev[k].copy_(src[k])
         got = []
-        upd.send_bucket = got.append
+        upd.send_bucket = lambda b: got.append(_snapshot(b))
         upd.update_weights()
         torch.cuda.synchronize()
         want = []
@@ -700,7 +711,7 @@ def test_random_dense_models_sync_and_replay(oracle, seed, packed):
 
     for round_ in range(3):                       # recording sync, then two replays with changed weights in between
         buckets = []
-        upd.send_bucket = buckets.append
+        upd.send_bucket = lambda b: buckets.append(_snapshot(b))
         upd.update_weights()
         torch.cuda.synchronize()
         flat = [nt for b in buckets for nt in b]
@@ -794,7 +805,7 @@ def test_random_moe_models_sync_and_replay(oracle, seed, fmt, packed):
                         packed_buckets=packed, **extra)
     for round_ in range(3):
         buckets = []
-        upd.send_bucket = buckets.append
+        upd.send_bucket = lambda b: buckets.append(_snapshot(b))
         upd.update_weights()
         torch.cuda.synchronize()
         flat = [nt for b in buckets for nt in b]
