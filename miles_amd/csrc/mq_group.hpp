@@ -54,12 +54,26 @@ struct TileJob {      // one 2-D tensor cut into 128x128 tiles
     const void* w;
     void* q;
     float* scale;
-    int64_t ldw;      // input row stride, elements
+    int32_t ldw;              // input row stride, elements (below 2^24)
     int32_t M, K;
-    int32_t tiles_k;
-    int32_t tiles_per_block;  // tile rows per input row block (row-blocked inputs), 0 = plain matrix
-    int64_t block_stride;     // elements between the first rows of consecutive row blocks
+    int32_t block_stride;     // elements between the first rows of consecutive row blocks (row-blocked inputs)
+    int32_t tiles_per_block;  // tile rows per input row block, 0 = plain matrix
+    uint32_t magic_k, magic_b;  // tile_div constants for division by the tiles per row and by tiles_per_block
+    uint32_t shifts;            // their shifts: the first in bits 0-7, the second in bits 8-15
 };
+// n / d for any 32-bit n from constants made on the host for a divisor d >= 2 (round-up multiply-high method):
+// t = mulhi(magic, n); n / d = (t + ((n - t) >> 1)) >> shift.  Both values are uniform over a workgroup, so the three
+// operations run on the scalar unit.
+inline void tile_div_magic(uint32_t d, uint32_t& magic, uint32_t& shift) {
+    uint32_t l = 0;
+    while ((1ull << l) < d) l++;                 // ceil(log2 d) >= 1
+    magic = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+    shift = l - 1;
+}
+__device__ __forceinline__ uint32_t tile_div(uint32_t n, uint32_t magic, uint32_t shift) {
+    const uint32_t t = __umulhi(magic, n);
+    return (t + ((n - t) >> 1)) >> shift;
+}
 struct TileTable {
     int32_t n;
     int32_t total;            // all work items of the launch
@@ -157,14 +171,17 @@ struct JobRef {
 };
 template <class Table>
 __device__ __forceinline__ JobRef find_job(const Table& tab, int32_t item) {
-    JobRef r{0, 0};
+    // `item` is uniform over the workgroup, and so is everything here: the count is kept on the scalar unit with a
+    // compare and an add-with-carry per entry.  (Left to the compiler the chain ended up on the vector unit -- two
+    // vector operations per entry, or, with the descriptor selected inside the loop, a vector multiply-add per entry
+    // to build its address: a quarter to a half of the vector work of a whole 128x128 tile.)
+    int32_t ji = 0;
 #pragma unroll
     for (int i = 0; i < kMaxGroup - 1; i++) {
-        const bool past = item >= tab.end[i];
-        r.ji += past ? 1 : 0;
-        r.start = past ? tab.end[i] : r.start;
+        const int32_t e = tab.end[i];
+        asm("s_cmp_ge_i32 %1, %2\n\ts_addc_u32 %0, %0, 0" : "+s"(ji) : "s"(item), "s"(e) : "scc");
     }
-    return r;
+    return JobRef{ji, ji > 0 ? tab.end[ji - 1] : 0};
 }
 // host side: after end[0..n) holds the running counts, record the total and pad the rest of `end`
 template <class Table>

@@ -48,7 +48,8 @@ static bool job_fast(const mq_job& j) {
         case MQ_JOB_FP8_BLOCKWISE_CAST:
         case MQ_JOB_FP8_BLOCK_POW2:
             return mq_fp8_tile_fast_ok(j.in, j.dtype, j.ld, 1, j.out, j.rows, j.cols, j.p0, j.p1) &&
-                   (j.block_stride % 8) == 0;
+                   (j.block_stride % 8) == 0 && j.block_stride >= 0 && j.block_stride <= 0x7FFFFFFF &&
+                   j.rows_per_block / 128 <= 0x7FFFFFFF;
         case MQ_JOB_FP8_DEQUANT:
             return mq_fp8_dequant_fast_ok(j.in, j.out, j.rows, j.cols, j.p0);
         case MQ_JOB_MXFP8:
@@ -254,7 +255,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
         }
         if (head.rows == 0 || head.cols == 0) { i++; continue; }
         if (!job_fast(head)) {
-            if (head.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "row-blocked input is not 16-byte aligned");
+            if (head.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "row-blocked input must be 16-byte aligned, with fewer than 2^24 columns and a block stride below 2^31 elements");
             int rc = run_single(head, stream);
             if (rc) return rc;
             i++;
@@ -284,8 +285,8 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) {
                     const mq_job& jb = jobs[i + t];
-                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, jb.ld, (int32_t)jb.rows, (int32_t)jb.cols, 0,
-                                         (int32_t)(jb.rows_per_block / 128), jb.block_stride};
+                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, (int32_t)jb.ld, (int32_t)jb.rows, (int32_t)jb.cols,
+                                         (int32_t)jb.block_stride, (int32_t)(jb.rows_per_block / 128), 0, 0, 0};
                 }
                 rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2, tab, st);
                 break;
