@@ -245,6 +245,7 @@ class Placement:
         # the first homes of this bucket's outputs are free again (nothing was ever written there)
         for s in owned + [s for s in touched if not s.written_by and not s.read_by]:
             self._storages.pop(s.ptr, None)
+            s.tensors = []                           # (records still point at the bookkeeping object: drop the memory itself)
         self._starts = None
         self.bucket_specs.append(specs)
         self.copies.append(copies)

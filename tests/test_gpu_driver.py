@@ -923,3 +923,86 @@ def test_quantize_nvfp4_on_a_stack_inside_a_batch_and_replayed(oracle):
     torch.cuda.synchronize()
     for g, w, what in zip(got, expected(cpu2), ("codes", "block scales", "global scales")):
         _same(g, w, f"replayed stack {what}")
+
+
+def test_plan_outputs_rotate_through_two_arenas(oracle):
+    """A recorded sync holds two buckets' worth of output memory, whatever the number of buckets: bucket k lives in arena
+    k mod 2.  A consumer that queues its reads of bucket k on the launch stream (no host synchronisation) gets the right
+    bytes although bucket k + 2 overwrites the same memory later in the same sync."""
+    cpu = _dense_model(60)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    args = Namespace(**{**vars(ARGS), "update_weight_buffer_size": 1 << 18})        # small buckets: six or more of them
+    upd = WeightUpdater(args, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None)
+    seen, copies = [], []
+
+    def consume(bucket):
+        # address range of the job-written tensors of this bucket, and stream-ordered copies of everything in it
+        made = [t for n, t in bucket if t.dtype in (F8, torch.float32)]
+        if made:      # a bucket of pass-through tensors only (the embedding) hands out views of the parameters
+            seen.append((len(copies), min(t.data_ptr() for t in made), max(t.data_ptr() + t.nbytes for t in made),
+                         sum(t.nbytes for t in made)))
+        copies.append([(n, t.clone()) for n, t in bucket])
+
+    for round_ in range(2):
+        seen.clear(), copies.clear()
+        upd.send_bucket = consume
+        upd.update_weights()
+        torch.cuda.synchronize()
+        flat = [nt for b in copies for nt in b]
+        want = _expected_fp8(oracle, cpu)
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} (sync {round_})")
+        cpu = _dense_model(61)
+        for k in dev:
+            dev[k].copy_(cpu[k])
+    plan = upd._plan
+    assert plan is not None and plan.replayable and plan.ring == 2 and len(seen) >= 4
+    largest = max(nbytes for _, _, _, nbytes in seen)
+    assert plan.arena_bytes <= 2 * (largest + 256 * 64), "two arenas of the largest bucket (plus alignment padding)"
+    assert torch.cuda.memory_allocated() - before - sum(t.nbytes for b in copies for _, t in b) <= plan.arena_bytes + (1 << 20)
+    starts = {}
+    for k, lo, hi, _ in seen:                  # buckets of the same parity share an arena, neighbours never overlap
+        assert starts.setdefault(k % 2, lo) == lo
+    for (k, lo, hi, _), (k2, lo2, hi2, _) in zip(seen, seen[1:]):
+        if k2 == k + 1:
+            assert hi <= lo2 or hi2 <= lo
+    assert len(starts) == 2
+    # an arena per bucket on request: every bucket of the sync stays valid until the next sync
+    keep = WeightUpdater(args, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None,
+                         plan_arenas=None)
+    held = []
+    keep.send_bucket = held.append
+    keep.update_weights()
+    torch.cuda.synchronize()
+    for (n, g), (_, w) in zip([nt for b in held for nt in b], _expected_fp8(oracle, cpu)):
+        _same(g, w, f"{n} (an arena per bucket)")
+    assert keep._plan.ring == len(held)
+
+
+def test_recording_a_sync_holds_no_more_than_a_few_buckets():
+    """While a sync is recorded nothing is executed and every bucket's first output buffers are released as soon as the
+    bucket has its place in an arena: the peak stays near the arenas' size instead of the size of all outputs."""
+    from miles_amd import workloads as Wl
+
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(9)
+    args, weights, elems = Wl.moe_megatron(gen, layers=1, experts=48, ffn=2048, hidden=7168, dist="gaussian_0.02",
+                                           buffer_bytes=64 << 20)
+    conf = Wl.MOE_CONFIGS["C4"]
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    upd = WeightUpdater(args, weights_getter=lambda: weights, model_name=conf["model_name"], quantization_config=conf["cfg"],
+                        send_bucket=lambda b: None, packed_weight_basenames=Wl.int4_packed_basenames(1, 48))
+    upd.update_weights()
+    torch.cuda.synchronize()
+    outputs = elems * (0.5 + 2 / 128)              # packed words + bf16 scales of the whole model
+    plan = upd._plan
+    assert plan is not None and plan.replayable and len(plan.buckets) >= 8
+    assert plan.arena_bytes <= 2 * (64 << 20) + (4 << 20)
+    peak = torch.cuda.max_memory_allocated() - base
+    assert peak <= plan.arena_bytes + 3 * (64 << 20), f"recording peaked at {peak} bytes for {outputs:.0f} bytes of outputs"
+    assert outputs > 5 * plan.arena_bytes
