@@ -10,8 +10,6 @@
 // pass 1 quantizes with the amax the record kept, collecting the new partial maxima with one atomic max per workgroup;
 // the fold compares; pass 2 quantizes again only the tensors whose amax moved.  A tensor whose amax moved takes the
 // two-pass form on the next run (pass 1 only collects its amax) and returns to the single pass once the amax has held.
-#include <stdlib.h>
-
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -168,8 +166,7 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
         if (tab.max_blocks > 0) hipLaunchKernelGGL(fp8_tensor_quant_kernel<1>, grid, dim3(kFtThreads), 0, st, tab, floor_v);
         hipLaunchKernelGGL(fp8_tensor_fold_kernel<2>, folds, blk, 0, st, tab, floor_v);
         if (tab.max_blocks > 0) {
-            static const int redo_cap = getenv("MQ_NV_REDO_BLOCKS") ? atoi(getenv("MQ_NV_REDO_BLOCKS")) : kSectionWords;
-            const unsigned redo = tab.max_blocks < redo_cap ? (unsigned)tab.max_blocks : (unsigned)redo_cap;
+            const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             hipLaunchKernelGGL(fp8_tensor_quant_kernel<2>, dim3(redo, (unsigned)tab.n), dim3(kFtThreads), 0, st, tab, floor_v);
         }
         return mq_check_launch("fp8 per-tensor quant (carried-over amax)");

@@ -13,8 +13,6 @@
 // Pass 2 (mq_nvfp4_quant) reads those two factors with a scalar load; two lanes own one 16-element block
 // (16 bytes each), the block amax is one DPP step, and each lane emits four bytes of codes.  A gate/up pair
 // writes two sections of one record.
-#include <stdlib.h>
-
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -551,8 +549,7 @@ int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mod
         if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
         hipLaunchKernelGGL(nvfp4_fold_kernel<2>, folds, blk, 0, st, tab, numer);
         if (tab.max_blocks > 0) {
-            static const int redo_cap = getenv("MQ_NV_REDO_BLOCKS") ? atoi(getenv("MQ_NV_REDO_BLOCKS")) : kSectionWords;
-            const unsigned redo_blocks = tab.max_blocks < redo_cap ? (unsigned)tab.max_blocks : (unsigned)redo_cap;
+            const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)tab.n), st);
         }
         return mq_check_launch("nvfp4 quant (carried-over amax)");
