@@ -268,6 +268,20 @@ typedef struct mq_job {
 #define MQ_MAX_GROUP 64
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 
+/* mq_run_jobs with the per-tensor descriptors of its launches kept in device memory (no counterpart in the reference; for
+ * callers that submit one job list again and again, as a replayed weight sync does).  The kernel arguments of a launch
+ * hold MQ_MAX_GROUP descriptors at most; a model of thousands of small tensors (the 18 432 expert matrices of a
+ * Qwen3-30B-A3B sync, 3 MB each) then drains and refills the chip every 64 tensors.  With a table a launch of the
+ * MXFP8, MXFP4 and symmetric INT4 jobs covers up to MQ_TABLE_GROUP tensors; every other job kind runs as in mq_run_jobs.
+ * mq_job_table_fill writes n entries of MQ_JOB_TABLE_ENTRY_BYTES bytes into host memory, entry i for jobs[i]; the
+ * caller copies them to device memory (any 8-byte aligned address) and passes that address, together with the same
+ * jobs, to mq_run_jobs_tabled.  A call may cover a sub-range of the list: pass jobs + k, n' and the address of entry k.
+ * The table must not change while a submitted call may still run; a NULL table makes the call mq_run_jobs. */
+#define MQ_JOB_TABLE_ENTRY_BYTES 56
+#define MQ_TABLE_GROUP 8192
+int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table);
+int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, void* stream);
+
 /* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the
  * software round-to-nearest-even forms over every fp32 bit pattern.  counts: 8 uint64 on the device
  * (cleared by the call): [0] e4m3 mismatches for |x| <= 448, [1] NaN inputs whose e4m3 code is not

@@ -44,11 +44,14 @@ SIGNATURES = {
     "mq_nvfp4_fold": [_vp, _i32, _i32, _vp],
     "mq_nvfp4_qdq": [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _vp],
     "mq_run_jobs": [_vp, _i64, _vp],
+    "mq_job_table_fill": [_vp, _i64, _vp],
+    "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
 }
 
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs
+TABLE_ENTRY_BYTES, TABLE_GROUP = 56, 8192                 # MQ_JOB_TABLE_ENTRY_BYTES, MQ_TABLE_GROUP (mq_run_jobs_tabled)
 NVFP4_4OVER6, NVFP4_ERR_MSE, NVFP4_ERR_FP16 = 1, 2, 4     # flags of mq_nvfp4_quant / mq_nvfp4_qdq
 NVFP4_CARRY_AMAX = 8                                      # MQ_NVFP4_CARRY_AMAX: NVFP4 jobs of a re-submitted list only
 # words of an amax record behind its four sections of 256 partial maxima (MQ_NVFP4_RECORD_*_WORD)

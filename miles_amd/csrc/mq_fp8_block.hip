@@ -23,7 +23,10 @@
 namespace mq {
 
 constexpr int kTile = 128;
-constexpr int kTileThreads = 512;                       // 8 wavefronts per 128x128 tile
+#ifndef MQ_TILE_THREADS
+#define MQ_TILE_THREADS 512
+#endif
+constexpr int kTileThreads = MQ_TILE_THREADS;            // 8 wavefronts per 128x128 tile
 constexpr int kRowsPerThread = 2048 / kTileThreads;     // 16-byte row segments per lane
 constexpr int kRowStep = kTileThreads / 16;             // tile rows covered per pass of the workgroup
 constexpr int kTileWaves = kTileThreads / kWave;
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTa
             // The first quarter of the tile is waited for before the other three are requested.  With all four loads
             // of every lane in flight at once the sync ran 0.5 - 1.2 % slower (alternating runs on one GPU): the
             // memory queues are full either way, and the narrower front of requests keeps more of them on open pages.
-            if (i == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (i == 0 && kRowsPerThread > 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     } else {
         const uint32_t c = col_ok ? c0 : 0u;

@@ -114,7 +114,20 @@ __device__ __forceinline__ int64_t xcd_chunked_block(int32_t chunk) {
     const int32_t bid = blockIdx.x, x = bid % kXcds, k = bid / kXcds;
     return (int64_t)((k / chunk) * kXcds + x) * chunk + (k % chunk);
 }
-__device__ __forceinline__ int64_t flat_block(const FlatTable& tab) { return xcd_chunked_block(tab.chunk); }
+// The same descriptors kept in device memory by a caller that submits one job list again and again: a launch is then not
+// bound to the kMaxGroup tensors that fit the kernel arguments.  A model of thousands of small tensors (MoE experts of
+// 3 MB) otherwise pays a launch boundary -- the chip draining and filling again, about 4 us -- per 64 of them, 8 % of
+// such a sync.  Kernels are templates over the two forms and read their descriptor with scalar loads either way.
+struct FlatRef {
+    const FlatJob* job;       // device memory, one entry per tensor of the launch (blockIdx.y)
+    int32_t chunk;
+    int32_t max_blocks;
+};
+constexpr int kTableGroup = 8192;         // tensors per launch of the device-table form (gridDim.y stays below 65 536)
+template <class Table>
+__device__ __forceinline__ const FlatJob& flat_job(const Table& tab) { return tab.job[blockIdx.y]; }
+template <class Table>
+__device__ __forceinline__ int64_t flat_block(const Table& tab) { return xcd_chunked_block(tab.chunk); }
 // largest power-of-two chunk (up to MQ_FLAT_CHUNK) whose grid padding stays under 3 % of `blocks` workgroups
 inline int64_t flat_chunk(int64_t blocks) {
     int64_t chunk = 1;
@@ -138,6 +151,15 @@ inline bool flat_grid(FlatTable& tab, int64_t per_block) {
     mx = flat_padded(mx, chunk);
     tab.chunk = (int32_t)chunk;
     tab.max_blocks = (int32_t)mx;
+    return mx < 0x7FFFFFF0;
+}
+// the same for a device table whose largest tensor has `max_units` units
+inline bool flat_grid(FlatRef& ref, int64_t max_units, int64_t per_block) {
+    int64_t mx = (max_units + per_block - 1) / per_block;
+    const int64_t chunk = flat_chunk(mx);
+    mx = flat_padded(mx, chunk);
+    ref.chunk = (int32_t)chunk;
+    ref.max_blocks = (int32_t)mx;
     return mx < 0x7FFFFFF0;
 }
 

@@ -78,9 +78,9 @@ __device__ __forceinline__ void int4_pack_chain_unit(const u32x4 v, const int64_
     }
 }
 
-template <int LANES>
-__global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const FlatTable tab) {
-    const FlatJob& job = tab.job[blockIdx.y];
+template <int LANES, class Table>
+__global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table tab) {
+    const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
     uint16_t* __restrict__ scale = (uint16_t*)job.s;
@@ -600,9 +600,20 @@ int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st) {
     if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
     dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kI4Threads);
-    if (group == 128) hipLaunchKernelGGL(int4_pack_bf16_kernel<16>, grid, blk, 0, st, tab);
-    else if (group == 64) hipLaunchKernelGGL(int4_pack_bf16_kernel<8>, grid, blk, 0, st, tab);
-    else hipLaunchKernelGGL(int4_pack_bf16_kernel<4>, grid, blk, 0, st, tab);
+    if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, FlatTable>), grid, blk, 0, st, tab);
+    else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, FlatTable>), grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, FlatTable>), grid, blk, 0, st, tab);
+    return mq_check_launch("int4 pack");
+}
+
+int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st) {
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (ref.max_blocks == 0 || n == 0) return MQ_OK;
+    dim3 grid((unsigned)ref.max_blocks, (unsigned)n), blk(kI4Threads);
+    if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, FlatRef>), grid, blk, 0, st, ref);
+    else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, FlatRef>), grid, blk, 0, st, ref);
+    else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, FlatRef>), grid, blk, 0, st, ref);
     return mq_check_launch("int4 pack");
 }
 

@@ -58,8 +58,9 @@ __device__ __forceinline__ float step_toward_zero(float n) {
     return u2f(u - ((u & 0x7FFFFFFFu) != 0));
 }
 
-__global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const FlatTable tab) {
-    const FlatJob& job = tab.job[blockIdx.y];
+template <class Table>
+__global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const Table tab) {
+    const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
@@ -268,7 +269,15 @@ bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group) {
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st) {
     if (!flat_grid(tab, kM4Threads * kM4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp4_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kM4Threads), 0, st, tab);
+    hipLaunchKernelGGL(mxfp4_bf16_kernel<FlatTable>, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kM4Threads), 0, st, tab);
+    return mq_check_launch("mxfp4 quant");
+}
+
+int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kM4Threads * kM4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (ref.max_blocks == 0 || n == 0) return MQ_OK;
+    hipLaunchKernelGGL(mxfp4_bf16_kernel<FlatRef>, dim3((unsigned)ref.max_blocks, (unsigned)n), dim3(kM4Threads), 0, st, ref);
     return mq_check_launch("mxfp4 quant");
 }
 

@@ -32,9 +32,10 @@ __device__ __forceinline__ float e8m0_inverse(uint32_t e) {
     return u2f((254u - e) << 23);
 }
 
-__global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const FlatTable tab) {
+template <class Table>
+__global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab) {
     const float inv448 = u2f(0x3B124925u);
-    const FlatJob& job = tab.job[blockIdx.y];
+    const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint8_t* __restrict__ q = (uint8_t*)job.q;
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
@@ -105,7 +106,16 @@ bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q) {
 int mq_mxfp8_launch_group(FlatTable& tab, hipStream_t st) {
     if (!flat_grid(tab, kMxThreads * kMxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp8_bf16_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kMxThreads), 0, st, tab);
+    hipLaunchKernelGGL(mxfp8_bf16_kernel<FlatTable>, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kMxThreads), 0, st, tab);
+    return mq_check_launch("mxfp8 quant");
+}
+
+// n descriptors in device memory; max_units: the largest tensor's 16-byte units
+int mq_mxfp8_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kMxThreads * kMxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (ref.max_blocks == 0 || n == 0) return MQ_OK;
+    hipLaunchKernelGGL(mxfp8_bf16_kernel<FlatRef>, dim3((unsigned)ref.max_blocks, (unsigned)n), dim3(kMxThreads), 0, st, ref);
     return mq_check_launch("mxfp8 quant");
 }
 

@@ -31,6 +31,9 @@ bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
 int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
+int mq_mxfp8_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
+int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
+int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -121,6 +124,13 @@ static int run_single(const mq_job& j, void* stream) {
 }
 
 static_assert(kMaxGroup == MQ_MAX_GROUP, "the public group size must match the launch tables");
+static_assert(sizeof(FlatJob) == MQ_JOB_TABLE_ENTRY_BYTES && kTableGroup == MQ_TABLE_GROUP, "the public table entry must match FlatJob");
+
+// job kinds whose grouped launch can read its descriptors from a device table
+static bool table_kind(int kind) { return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK; }
+static FlatJob flat_entry(const mq_job& jb) {
+    return FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8, nullptr, 0, 0};
+}
 
 static bool same_group(const mq_job& a, const mq_job& b) {
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
@@ -235,8 +245,21 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
     return mq_check_launch("nvfp4 group");
 }
 
-extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
+extern "C" int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table) {
+    if (n < 0 || (n > 0 && (!jobs || !host_table))) return mq_fail(MQ_ERR_ARG, "bad job list");
+    for (int64_t i = 0; i < n; i++) {
+        const FlatJob e = table_kind(jobs[i].kind) ? flat_entry(jobs[i]) : FlatJob{};
+        memcpy((char*)host_table + i * sizeof(FlatJob), &e, sizeof(FlatJob));
+    }
+    return MQ_OK;
+}
+
+extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) { return mq_run_jobs_tabled(jobs, n, nullptr, stream); }
+
+extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, void* stream) {
     if (n < 0 || (n > 0 && !jobs)) return mq_fail(MQ_ERR_ARG, "bad job list");
+    if ((uintptr_t)device_table % 8 != 0) return mq_fail(MQ_ERR_ARG, "job table must be 8-byte aligned");
+    const FlatJob* table = (const FlatJob*)device_table;
     hipStream_t st = (hipStream_t)stream;
     for (int64_t i = 0; i < n; i++) {
         int rc = check_job(jobs[i]);
@@ -264,8 +287,10 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
         // flat kinds run on a (largest tensor) x (tensors) grid: keep the padding of a group under 25 %
         const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST &&
                           head.kind != MQ_JOB_FP8_BLOCK_POW2 && head.kind != MQ_JOB_COPY;
+        const bool tabled = table != nullptr && table_kind(head.kind);
+        const int64_t group_cap = tabled ? kTableGroup : kMaxGroup;
         int64_t j = i + 1, sum = head.rows * head.cols, mx = sum;
-        while (j < n && j - i < kMaxGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
+        while (j < n && j - i < group_cap && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
                jobs[j].cols > 0) {
             const int64_t e = jobs[j].rows * jobs[j].cols;
             const int64_t nmx = e > mx ? e : mx;
@@ -303,12 +328,15 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) {
             case MQ_JOB_MXFP8:
             case MQ_JOB_MXFP4:
             case MQ_JOB_INT4_PACK: {
+                if (tabled && cnt > kMaxGroup) {        // small groups keep the kernel-argument form (no pointer chase)
+                    rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_table(table + i, cnt, mx / 8, st)
+                         : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_table(table + i, cnt, mx / 8, st)
+                                                     : mq_int4_pack_launch_table(table + i, cnt, mx / 8, head.p0, st);
+                    break;
+                }
                 FlatTable tab{};
                 tab.n = cnt;
-                for (int t = 0; t < cnt; t++) {
-                    const mq_job& jb = jobs[i + t];
-                    tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8};
-                }
+                for (int t = 0; t < cnt; t++) tab.job[t] = flat_entry(jobs[i + t]);
                 rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_group(tab, st)
                      : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_group(tab, st)
                                                  : mq_int4_pack_launch_group(tab, head.p0, st);

@@ -28,6 +28,7 @@ class JobBatch:
         self._records: list[tuple] = []
         self._keep: list[torch.Tensor] = []
         self._array = None
+        self._table = None      # device copy of the launch descriptors (see freeze)
         self.device = None
         self.direct_calls = 0   # kernels launched inside the block without going through the job list
         self.constants: set[int] = set()   # addresses of result tensors whose contents never depend on the weights
@@ -96,14 +97,30 @@ class JobBatch:
     def held(self) -> list[torch.Tensor]:
         return self._keep
 
+    # job kinds whose grouped launches can take their descriptors from a device table (mq_run_jobs_tabled)
+    _TABLE_KINDS = (_lib.JOB_MXFP8, _lib.JOB_MXFP4, _lib.JOB_INT4_PACK)
+
     def freeze(self):
-        """Materialise the ctypes job array (done once; `run` can then be repeated)."""
+        """Materialise the ctypes job array (done once; `run` can then be repeated).  A list with more jobs of a
+        table kind than one launch's kernel arguments hold (MoE experts by the thousand) also gets its descriptors
+        copied to device memory, so that `run` is not cut into launches of 64 tensors."""
         if self._array is None:
             arr = (_lib.Job * len(self._records))()
             for i, rec in enumerate(self._records):
                 arr[i] = _lib.Job(*rec)
             self._array = arr
+            self._table = None
+            if self.device is not None and sum(r[self.KIND] in self._TABLE_KINDS for r in self._records) > _lib.MAX_GROUP:
+                host = torch.empty(len(self._records) * _lib.TABLE_ENTRY_BYTES, dtype=torch.uint8)
+                _lib.check(_lib.load().mq_job_table_fill(arr, len(self._records), host.data_ptr()))
+                self._table = host.to(self.device)
         return self._array
+
+    def launch_group(self, index: int) -> int:
+        """How many consecutive jobs one launch can cover at job `index`: `TABLE_GROUP` for a table kind of a frozen
+        batch that keeps a device table, `MAX_GROUP` otherwise."""
+        tabled = self._table is not None and self._records[index][self.KIND] in self._TABLE_KINDS
+        return _lib.TABLE_GROUP if tabled else _lib.MAX_GROUP
 
     def run(self, stream: int | None = None) -> None:
         self.run_range(0, len(self._records), stream)
@@ -117,7 +134,8 @@ class JobBatch:
         if stream is None:
             stream = _lib.stream_ptr(self.device)
         ptr = ctypes.byref(arr, start * ctypes.sizeof(_lib.Job))
-        _lib.check(_lib.load().mq_run_jobs(ptr, stop - start, stream))
+        table = None if self._table is None else self._table.data_ptr() + start * _lib.TABLE_ENTRY_BYTES
+        _lib.check(_lib.load().mq_run_jobs_tabled(ptr, stop - start, table, stream))
 
     def input_pointers(self) -> list[int]:
         return [rec[2] for rec in self._records]

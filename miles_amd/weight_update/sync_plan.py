@@ -115,9 +115,10 @@ class SyncPlan:
         Qwen3-4B FP8 sync 1 % slower.  A cut never falls between NVFP4 jobs that share an amax record."""
         if self._marks is None:
             records, total, done, marks = self.batch.records, len(self.batch), 0, []
-            group = _lib.MAX_GROUP
+            self.batch.freeze()
             for mark in self.jobs_done_at_bucket:
                 if mark > done:
+                    group = self.batch.launch_group(mark - 1)     # with a device table a bucket's experts are one launch
                     tail = (mark - done) % group
                     tail_elements = sum(r[7] * r[8] for r in records[mark - tail:mark])
                     if tail and tail_elements < self.SMALL_LAUNCH_ELEMENTS:

@@ -67,6 +67,7 @@ def test_python_constants_match_the_header():
     for name in ("NVFP4_4OVER6", "NVFP4_ERR_MSE", "NVFP4_ERR_FP16", "NVFP4_CARRY_AMAX"):
         assert getattr(_lib, name) == enums["MQ_" + name]
     assert _lib.MAX_GROUP == int(defines["MQ_MAX_GROUP"])
+    assert (_lib.TABLE_ENTRY_BYTES, _lib.TABLE_GROUP) == (int(defines["MQ_JOB_TABLE_ENTRY_BYTES"]), int(defines["MQ_TABLE_GROUP"]))
     words = int(defines["MQ_NVFP4_SECTION_WORDS"]) * (int(defines["MQ_NVFP4_SECTIONS"]) + 1)
     assert AMAX_RECORD_WORDS == _AMAX_RECORD_WORDS == words
     amax_word = int(defines["MQ_NVFP4_SECTION_WORDS"]) * int(defines["MQ_NVFP4_SECTIONS"])

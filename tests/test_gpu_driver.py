@@ -1006,3 +1006,68 @@ def test_recording_a_sync_holds_no_more_than_a_few_buckets():
     peak = torch.cuda.max_memory_allocated() - base
     assert peak <= plan.arena_bytes + 3 * (64 << 20), f"recording peaked at {peak} bytes for {outputs:.0f} bytes of outputs"
     assert outputs > 5 * plan.arena_bytes
+
+
+@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4"])
+def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
+    """More than MQ_MAX_GROUP jobs of a table kind: the batch copies their descriptors to device memory and one launch
+    covers the lot.  Shapes vary inside the 25 % band that keeps a group together, with a few far outside it (which
+    cut the group), an FP8 tile job in the middle, and the list is also submitted in two ranges that start mid-table."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.megatron_to_hf.processors.quantizer_compressed_tensors import pack_layer
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+
+    g = torch.Generator().manual_seed(77)
+    shapes = [(int(torch.randint(52, 64, (1,), generator=g)), 256) for _ in range(150)]
+    shapes[40], shapes[41], shapes[120] = (8, 128), (300, 256), (1, 128)
+    ws = [W.student_t_rows(s, std=0.02, seed=7700 + i) for i, s in enumerate(shapes)]
+    dev = [w.to(DEV) for w in ws]
+    tile_w = W.gaussian_outliers((256, 384), std=0.02, p_outlier=0.001, gain=20.0, seed=7)
+
+    def quantize(w):
+        if fmt == "mxfp8":
+            return mxfp8_quantize(w)
+        if fmt == "mxfp4":
+            return quantize_mxfp4(w, 32)
+        return pack_layer(w, 128)[:2]
+
+    def expected(w):
+        if fmt == "mxfp8":
+            return oracle.mxfp8_quantize(w)
+        if fmt == "mxfp4":
+            return oracle.quantize_mxfp4(w, 32)
+        return oracle.pack_layer(w, 128)[:2]
+
+    with launch.recording() as batch:
+        outs = [quantize(w) for w in dev[:75]]
+        tile_out = fp8_blockwise_cast(tile_w.to(DEV))
+        outs += [quantize(w) for w in dev[75:]]
+    batch.freeze()
+    assert batch._table is not None and batch._table.numel() == len(batch) * _lib.TABLE_ENTRY_BYTES
+
+    def check(what):
+        torch.cuda.synchronize()
+        for i, (w, out) in enumerate(zip(ws, outs)):
+            for k, (got, want) in enumerate(zip(out, expected(w))):
+                _same(got, want, f"{fmt} tensor {i} {tuple(w.shape)} output {k} ({what})")
+        for got, want in zip(tile_out, oracle.fp8_blockwise_cast(tile_w)):
+            _same(got, want, f"fp8 tile job between the {fmt} jobs ({what})")
+
+    def poison():
+        for out in (*outs, tile_out):
+            for t in out:
+                t.view(torch.uint8).fill_(0x5A)
+
+    batch.run()
+    check("one submission")
+    poison()
+    batch.run_range(0, 70)
+    batch.run_range(70, len(batch))
+    check("two ranges")
+    # the same list through the kernel-argument form
+    poison()
+    batch._table = None
+    batch.run()
+    check("without the table")
