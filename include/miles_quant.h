@@ -211,7 +211,10 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_MXFP4                w             packed e2m1   E8M0 bytes     -                           group, -
  *   MQ_JOB_COPY                 bytes         bytes         -              -                           -
  *     (rows * cols bytes copied verbatim: how a pass-through tensor reaches its place in a packed transport bucket,
- *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208)
+ *      the flattened payload of miles/backends/training_utils/weight_update/protocols/broadcast.py:191-208.  With
+ *      rows > 1 the job is a 2-D copy of rows runs of cols bytes each: source runs ld bytes apart, destination runs
+ *      block_stride bytes apart (0: back to back) -- one job regroups the q rows of a fused QKV weight or swaps the
+ *      column halves of a matrix; both pitches must be at least cols)
  *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
  *   MQ_JOB_UE8M0_PACK           fp32 tiles    int32 words   -              -                           batch, tile_rows
  *   MQ_JOB_FP8_TENSOR           w[rows,cols]  e4m3          fp32 [1]       aux = amax record           floor bits, flags

@@ -39,8 +39,11 @@ __global__ __launch_bounds__(256) void copy_group_kernel(const CopyTable tab) {
     const int32_t item = blockIdx.x;
     const JobRef r = find_job(tab, item);
     const CopyJob& job = tab.job[r.ji];
-    const int64_t off0 = (int64_t)(item - r.start) * kCopyChunk;
-    const bool aligned = (((uintptr_t)job.src | (uintptr_t)job.dst) & 15) == 0;
+    const int32_t local = item - r.start, row = local / job.chunks_per_row;
+    const int64_t off0 = (int64_t)(local - row * job.chunks_per_row) * kCopyChunk;
+    const uint8_t* __restrict__ src = job.src + row * job.src_pitch;
+    uint8_t* __restrict__ dst = job.dst + row * job.dst_pitch;
+    const bool aligned = (((uintptr_t)src | (uintptr_t)dst) & 15) == 0;
     if (aligned) {
         u32x4 v[kCopyUnits];
         bool full[kCopyUnits];
@@ -48,17 +51,17 @@ __global__ __launch_bounds__(256) void copy_group_kernel(const CopyTable tab) {
         for (int u = 0; u < kCopyUnits; u++) {
             const int64_t o = off0 + (u * 256 + threadIdx.x) * 16;
             full[u] = o + 16 <= job.bytes;
-            if (full[u]) v[u] = ld16(job.src + o);
+            if (full[u]) v[u] = ld16(src + o);
         }
 #pragma unroll
         for (int u = 0; u < kCopyUnits; u++) {
             const int64_t o = off0 + (u * 256 + threadIdx.x) * 16;
-            if (full[u]) st16(job.dst + o, v[u]);
-            else for (int64_t b = o; b < job.bytes && b < o + 16; b++) job.dst[b] = job.src[b];
+            if (full[u]) st16(dst + o, v[u]);
+            else for (int64_t b = o; b < job.bytes && b < o + 16; b++) dst[b] = src[b];
         }
     } else {
         const int64_t stop = off0 + kCopyChunk < job.bytes ? off0 + kCopyChunk : job.bytes;
-        for (int64_t b = off0 + threadIdx.x; b < stop; b += 256) job.dst[b] = job.src[b];
+        for (int64_t b = off0 + threadIdx.x; b < stop; b += 256) dst[b] = src[b];
     }
 }
 // one long aligned run: one 16-byte unit per lane, no table (the access pattern that streams fastest on MI355X)
@@ -81,7 +84,12 @@ int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st
 int mq_copy_launch_group(mq::CopyTable& tab, hipStream_t st) {
     int64_t run = 0;
     for (int i = 0; i < tab.n; i++) {
-        run += (tab.job[i].bytes + mq::kCopyChunk - 1) / mq::kCopyChunk;
+        // chunks_per_row holds the row count on entry (0 or 1: a plain run)
+        const int64_t rows = tab.job[i].chunks_per_row > 1 ? tab.job[i].chunks_per_row : 1;
+        const int64_t per_row = (tab.job[i].bytes + mq::kCopyChunk - 1) / mq::kCopyChunk;
+        if (per_row > 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "copy group too large");
+        tab.job[i].chunks_per_row = per_row > 0 ? (int32_t)per_row : 1;
+        run += rows * per_row;
         if (run > 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "copy group too large");
         tab.end[i] = (int32_t)run;
     }

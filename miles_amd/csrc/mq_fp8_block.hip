@@ -430,7 +430,10 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 // 1 KiB of consecutive output per store instruction.  Row and column of a unit come from a multiply-high
 // division by the row length (exact for every 32-bit unit index), not from an integer divide.
 constexpr int kDqThreads = 256;
-constexpr int kDqUnroll = 2;
+#ifndef MQ_DQ_UNROLL
+#define MQ_DQ_UNROLL 2
+#endif
+constexpr int kDqUnroll = MQ_DQ_UNROLL;
 struct DequantJob {
     const uint8_t* x;
     const float* s;

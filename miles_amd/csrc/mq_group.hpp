@@ -171,10 +171,13 @@ constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (f
 constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
 constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last run: the next carried run collects the amax first
 
-struct CopyJob {      // one run of bytes
+struct CopyJob {      // rows of `bytes` bytes each (one row: a plain run), chunks_per_row chunks of the copy kernel per row
     const uint8_t* src;
     uint8_t* dst;
     int64_t bytes;
+    int64_t src_pitch, dst_pitch;
+    int32_t chunks_per_row;
+    int32_t pad;
 };
 struct CopyTable {
     int32_t n;

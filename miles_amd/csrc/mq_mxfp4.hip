@@ -145,7 +145,10 @@ __device__ __forceinline__ uint32_t mxfp4_decode(uint32_t code, uint32_t s) {
 // flat: one lane per 4 packed bytes (8 codes -> 16 bytes of bf16), kM4DqUnroll such units per lane; G = 8 << group_shift.
 // Scale bytes 2..252 keep every product a normal, finite bf16 number: there the packed hardware conversion
 // (two codes per instruction, scaled by 2^(s-127)) is used; the few bytes outside that range take the software form.
-constexpr int kM4DqUnroll = 2;
+#ifndef MQ_M4DQ_UNROLL
+#define MQ_M4DQ_UNROLL 2
+#endif
+constexpr int kM4DqUnroll = MQ_M4DQ_UNROLL;
 typedef __bf16 hw_bf16x2_t __attribute__((ext_vector_type(2)));
 template <int BYTE>
 __device__ __forceinline__ uint32_t hw_e2m1x2_to_bf16x2(uint32_t word, float factor) {

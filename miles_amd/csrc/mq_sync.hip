@@ -72,12 +72,17 @@ static bool job_fast(const mq_job& j) {
     }
 }
 
+static int64_t copy_dst_pitch(const mq_job& j);
 static int check_job(const mq_job& j) {
     if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_INT4_PACK_ASYM) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
-    if (j.kind == MQ_JOB_COPY) return MQ_OK;
+    if (j.kind == MQ_JOB_COPY) {
+        if (j.rows > 1 && (j.ld < j.cols || copy_dst_pitch(j) < j.cols || j.rows > 0x7FFFFFF0))
+            return mq_fail(MQ_ERR_ARG, "rows of a copy job overlap");
+        return MQ_OK;
+    }
     if (j.kind == MQ_JOB_UE8M0_PACK)
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
     if (!empty && (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale)) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
@@ -138,13 +143,21 @@ static bool same_group(const mq_job& a, const mq_job& b) {
 
 // Copy jobs of one launch run in no particular order: a job that reads what an earlier job of the group writes (a
 // regrouped tensor that is then copied into a payload), or writes what one reads or writes, has to start a new group.
+// A copy job is `rows` rows of `cols` bytes; with more than one row the source rows are `ld` bytes apart and the
+// destination rows `block_stride` bytes (0: back to back).  Its footprints are taken as the whole span of the rows.
+static int64_t copy_dst_pitch(const mq_job& j) { return j.block_stride != 0 ? j.block_stride : j.cols; }
+static uintptr_t copy_span(const mq_job& j, int64_t pitch) {
+    return (uintptr_t)(j.rows > 1 ? (j.rows - 1) * pitch + j.cols : j.rows * j.cols);
+}
 static bool copy_depends_on_group(const mq_job* jobs, int64_t first, int64_t candidate) {
     const mq_job& c = jobs[candidate];
-    const uintptr_t cin = (uintptr_t)c.in, cout = (uintptr_t)c.out, cb = (uintptr_t)(c.rows * c.cols);
+    const uintptr_t cin = (uintptr_t)c.in, cout = (uintptr_t)c.out;
+    const uintptr_t cib = copy_span(c, c.ld), cob = copy_span(c, copy_dst_pitch(c));
     for (int64_t t = first; t < candidate; t++) {
-        const uintptr_t tin = (uintptr_t)jobs[t].in, tout = (uintptr_t)jobs[t].out, tb = (uintptr_t)(jobs[t].rows * jobs[t].cols);
-        const bool reads_written = cin < tout + tb && tout < cin + cb;
-        const bool writes_touched = (cout < tout + tb && tout < cout + cb) || (cout < tin + tb && tin < cout + cb);
+        const uintptr_t tin = (uintptr_t)jobs[t].in, tout = (uintptr_t)jobs[t].out;
+        const uintptr_t tib = copy_span(jobs[t], jobs[t].ld), tob = copy_span(jobs[t], copy_dst_pitch(jobs[t]));
+        const bool reads_written = cin < tout + tob && tout < cin + cib;
+        const bool writes_touched = (cout < tout + tob && tout < cout + cob) || (cout < tin + tib && tin < cout + cob);
         if (reads_written || writes_touched) return true;
     }
     return false;
@@ -349,8 +362,11 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                     const mq_job& jb = jobs[i + t];
                     const int64_t bytes = jb.rows * jb.cols;
                     const bool aligned = (((uintptr_t)jb.in | (uintptr_t)jb.out) & 15) == 0;
-                    if (aligned && bytes >= (64 << 20)) rc = mq_copy_launch_run(jb.in, jb.out, bytes, st);
-                    else tab.job[tab.n++] = CopyJob{(const uint8_t*)jb.in, (uint8_t*)jb.out, bytes};
+                    const bool one_run = jb.rows == 1 || (jb.ld == jb.cols && copy_dst_pitch(jb) == jb.cols);
+                    if (one_run && aligned && bytes >= (64 << 20)) rc = mq_copy_launch_run(jb.in, jb.out, bytes, st);
+                    else if (one_run) tab.job[tab.n++] = CopyJob{(const uint8_t*)jb.in, (uint8_t*)jb.out, bytes, 0, 0, 1, 0};
+                    else tab.job[tab.n++] = CopyJob{(const uint8_t*)jb.in, (uint8_t*)jb.out, jb.cols, jb.ld, copy_dst_pitch(jb),
+                                                    (int32_t)jb.rows, 0};
                 }
                 if (rc == MQ_OK && tab.n > 0) rc = mq_copy_launch_group(tab, st);
                 break;

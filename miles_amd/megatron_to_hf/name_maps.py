@@ -96,9 +96,13 @@ def _split_qkv_weight(args, layer: str, param: torch.Tensor):
     q_per_group = args.num_attention_heads // groups
     grouped = param.view(groups, -1, _head_dim(args), args.hidden_size)
     q, k, v = torch.split(grouped, [q_per_group, 1, 1], dim=1)
-    if getattr(args, "qkv_row_block_views", False):
-        # opt-in of the batched sync driver: hand q / k / v on as [groups, rows, hidden] VIEWS of the fused
-        # weight; the FP8 kernel reads the row blocks in place and the regrouping copy disappears
+    # opt-in of the batched sync driver: hand q / k / v on as [groups, rows, hidden] VIEWS of the fused weight; the
+    # FP8 kernel reads the row blocks in place and the regrouping copy disappears.  Only the tuned kernel reads such
+    # views, and it takes contiguous bf16 storage that starts on a 16-byte boundary: a parameter carved out of a flat
+    # buffer at an odd offset, or of another dtype, is regrouped with copy jobs like everywhere else.
+    in_place = (getattr(args, "qkv_row_block_views", False) and param.dtype == torch.bfloat16 and param.is_contiguous()
+                and param.data_ptr() % 16 == 0)
+    if in_place:
         return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", t.flatten(1, 2))
                 for n, t in (("q", q), ("k", k), ("v", v))]
     return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", gather_groups(t, (-1, args.hidden_size)))
@@ -264,12 +268,12 @@ def convert_glm4moe_to_hf(args, name, param):
 
 def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
     """Swap the two halves along `dim` (64 + 64 channels of a DSA indexer head, the two input halves of MiMo's MTP
-    projection).  On the GPU the two halves of every leading index are byte-copy jobs, so a recorded sync repeats the
-    swap on the current weights; elsewhere a torch concatenation."""
+    projection).  On the GPU each half is one 2-D byte-copy job, so a recorded sync repeats the swap on
+    the current weights; elsewhere a torch concatenation."""
     a, b = t.chunk(2, dim=dim)
     if t.device.type != "cuda" or not t.is_contiguous():
         return torch.cat([b, a], dim=dim)
-    from miles_amd.weight_update.packed_bucket import submit_copy
+    from miles_amd.weight_update.packed_bucket import submit_copy_rows
 
     out = torch.empty_like(t)
     first, second = out.chunk(2, dim=dim)
@@ -277,9 +281,8 @@ def _rotate_halves(t: torch.Tensor, dim: int) -> torch.Tensor:
     for size in t.shape[:dim]:
         lead *= size
     for src, dst in ((b, first), (a, second)):
-        src, dst = src.reshape(lead, -1), dst.reshape(lead, -1)      # views: each leading index owns one contiguous run
-        for i in range(lead):
-            submit_copy(src[i], dst[i])
+        # views: each leading index owns one contiguous run, and the runs are one row pitch apart -- one 2-D copy job
+        submit_copy_rows(src.reshape(lead, -1), dst.reshape(lead, -1))
     return out
 
 

@@ -87,3 +87,22 @@ def submit_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     _lib.require_gpu(src, "packed bucket copy")
     if nbytes:
         launch.submit(_lib.JOB_COPY, src, dst, None, None, None, 1, nbytes, nbytes)
+
+
+def submit_copy_rows(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Record (or run) one 2-D byte copy between two [rows, n] views whose rows are contiguous runs (any row stride of
+    at least a row): the strided form of a copy job, one job where `submit_copy` would need one per row."""
+    if src.shape != dst.shape or src.dim() != 2 or src.dtype != dst.dtype:
+        raise _lib.MilesQuantError("2-D copy between tensors of different shapes")
+    rows, n = src.shape
+    size = src.element_size()
+    if not rows or not n:
+        return
+    if n > 1 and (src.stride(1) != 1 or dst.stride(1) != 1):
+        raise _lib.MilesQuantError("2-D copy needs contiguous rows")
+    _lib.require_gpu(src, "packed bucket copy")
+    src_pitch = src.stride(0) * size if rows > 1 else n * size
+    dst_pitch = dst.stride(0) * size if rows > 1 else n * size
+    if src_pitch < n * size or dst_pitch < n * size:
+        raise _lib.MilesQuantError("2-D copy with overlapping rows")
+    launch.submit(_lib.JOB_COPY, src, dst, None, None, None, rows, n * size, src_pitch, block_stride=dst_pitch)

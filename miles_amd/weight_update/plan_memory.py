@@ -264,7 +264,10 @@ class Placement:
                 continue
             for ri, f in s.written_by:
                 if recorded[ri][_F.KIND] == _lib.JOB_COPY:
-                    gathers.append((recorded[ri][f], ri, recorded[ri][_F.ROWS] * recorded[ri][_F.COLS], s))
+                    rec = recorded[ri]
+                    # (a 2-D copy whose destination rows lie apart fills no single run: its tensor is copied afterwards)
+                    if rec[_F.ROWS] == 1 or rec[_F.BLOCK_STRIDE] in (0, rec[_F.COLS]):
+                        gathers.append((rec[f], ri, rec[_F.ROWS] * rec[_F.COLS], s))
                 else:
                     writers.setdefault(recorded[ri][f], []).append((ri, f, s))
         gathers = sorted({g[:3]: g for g in gathers}.values(), key=lambda g: g[0])

@@ -840,7 +840,7 @@ def test_dsa_indexer_half_rotation_is_replayable():
     name = "module.module.decoder.layers.0."
     with launch.recording() as batch:
         got = {k: name_maps.convert_deepseekv3_to_hf(args, name + k, v) for k, v in dev.items()}
-    assert batch.direct_calls == 0 and len(batch) == 2 * 4 + 2 + 2 + 2
+    assert batch.direct_calls == 0 and len(batch) == 4 * 2         # each rotation: one 2-D copy job per half
     batch.device = torch.device(DEV)
     for round_ in range(2):
         batch.run()
@@ -1071,3 +1071,84 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     batch._table = None
     batch.run()
     check("without the table")
+
+
+@pytest.mark.parametrize("odd", ["offset", "fp16"])
+def test_fused_qkv_that_the_tuned_kernel_cannot_read_in_place_is_regrouped(oracle, odd):
+    """Row-blocked q / k / v views are switched on per model, by shape.  A fused qkv parameter that starts two bytes into
+    a flat buffer, or a model held in fp16, is outside what the tile kernel reads in place: the name map regroups it
+    with copy jobs instead, and the sync stays correct and replayable."""
+    cpu = _dense_model(31)
+    if odd == "fp16":
+        cpu = {k: v.to(torch.float16) for k, v in cpu.items()}
+    dev = {}
+    for k, v in cpu.items():
+        if odd == "offset" and k.endswith("linear_qkv.weight"):
+            flat = torch.empty(v.numel() + 1, dtype=v.dtype, device=DEV)
+            dev[k] = flat[1:].view(v.shape).copy_(v)
+            assert dev[k].data_ptr() % 16 == 2
+        else:
+            dev[k] = v.to(DEV)
+    upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG,
+                        send_bucket=None)
+    assert upd.args.qkv_row_block_views
+    for label in ("first sync", "replay"):
+        flat = [nt for b in _run(upd) for nt in b]
+        want = _expected_fp8(oracle, cpu)
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} ({label})")
+        assert upd._plan is not None and upd._plan.replayable
+        cpu = {k: (v.float() * 0.5).to(v.dtype) for k, v in cpu.items()}
+        for k in dev:
+            dev[k].copy_(cpu[k])
+
+
+@pytest.mark.parametrize("rows,row_bytes,src_pitch,dst_pitch,offset", [
+    (64, 8192, 16384, 8192, 0), (37, 100, 131, 257, 0), (1, 5000, 5000, 5000, 0), (9, 40000, 40016, 50000, 0),
+    (16, 4096, 8192, 8192, 3), (300, 16, 48, 16, 0), (5, 16384, 16384, 32768, 0)])
+def test_copy_jobs_with_row_pitches(rows, row_bytes, src_pitch, dst_pitch, offset):
+    """The 2-D form of a copy job: rows of bytes at one pitch in the source and another in the destination; what lies
+    between the destination rows stays untouched.  Run alone and as members of one grouped launch."""
+    from miles_amd import launch
+    from miles_amd.weight_update.packed_bucket import submit_copy_rows
+
+    g = torch.Generator().manual_seed(rows * 7 + row_bytes)
+
+    def case():
+        src = torch.randint(0, 256, (rows * src_pitch + offset,), dtype=torch.uint8, generator=g).to(DEV)
+        dst = torch.full((rows * dst_pitch + offset,), 0xA5, dtype=torch.uint8, device=DEV)
+        sv = src[offset:].view(rows, src_pitch)[:, :row_bytes]
+        dv = dst[offset:].view(rows, dst_pitch)[:, :row_bytes]
+        return src, dst, sv, dv
+
+    def check(src, dst, sv, dv, what):
+        want = torch.full_like(dst, 0xA5)
+        want[offset:].view(rows, dst_pitch)[:, :row_bytes] = sv
+        assert torch.equal(dst, want), what
+
+    one = case()
+    submit_copy_rows(one[2], one[3])
+    torch.cuda.synchronize()
+    check(*one, "single job")
+    many = [case() for _ in range(5)]
+    with launch.deferred():
+        for _, _, sv, dv in many:
+            submit_copy_rows(sv, dv)
+    torch.cuda.synchronize()
+    for c in many:
+        check(*c, "grouped jobs")
+
+
+def test_a_2d_copy_that_reads_what_an_earlier_copy_wrote_runs_after_it():
+    from miles_amd import launch
+    from miles_amd.weight_update.packed_bucket import submit_copy, submit_copy_rows
+
+    a = torch.arange(64 * 64, dtype=torch.int32, device=DEV).view(64, 64)
+    b = torch.zeros_like(a)
+    c = torch.zeros(64, 32, dtype=torch.int32, device=DEV)
+    with launch.deferred():
+        submit_copy(a.view(-1), b.view(-1))
+        submit_copy_rows(b[:, 32:], c)                      # reads rows of b: must see what the first job wrote
+    torch.cuda.synchronize()
+    assert torch.equal(c, a[:, 32:])

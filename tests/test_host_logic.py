@@ -133,12 +133,20 @@ class TestNameMaps:
 
     def test_row_block_views_opt_in(self):
         args = Namespace(**vars(QWEN_ARGS), qkv_row_block_views=True)
-        qkv = torch.randn((4 + 2 * 2) * 16, 64)
-        out = name_maps.convert_qwen2_to_hf(args, "module.module.decoder.layers.0.self_attention.linear_qkv.weight", qkv)
-        ref = name_maps.convert_qwen2_to_hf(QWEN_ARGS, "module.module.decoder.layers.0.self_attention.linear_qkv.weight", qkv)
+        name = "module.module.decoder.layers.0.self_attention.linear_qkv.weight"
+        qkv = torch.randn((4 + 2 * 2) * 16, 64).to(torch.bfloat16)
+        out = name_maps.convert_qwen2_to_hf(args, name, qkv)
+        ref = name_maps.convert_qwen2_to_hf(QWEN_ARGS, name, qkv)
         for (n, view), (n2, copy) in zip(out, ref):
             assert n == n2 and view.dim() == 3 and view.untyped_storage().data_ptr() == qkv.untyped_storage().data_ptr()
             assert torch.equal(view.reshape(-1, 64), copy)
+        # what the tile kernel cannot read in place is regrouped as without the opt-in: another dtype, or storage that
+        # starts off a 16-byte boundary
+        flat = torch.empty(qkv.numel() + 1, dtype=torch.bfloat16)
+        for odd in (qkv.float(), flat[1:].view(qkv.shape).copy_(qkv)):
+            got = name_maps.convert_qwen2_to_hf(args, name, odd)
+            for (n, t), (n2, copy) in zip(got, ref):
+                assert n == n2 and t.dim() == 2 and torch.equal(t.to(torch.bfloat16), copy)
 
     def test_moe_experts(self):
         fc1 = torch.randn(32, 64)
