@@ -222,7 +222,8 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      16-byte aligned input; p0 = bit pattern of 1e-12 rounded to the weight dtype; p1 = 0 or MQ_NVFP4_CARRY_AMAX)
  *   MQ_JOB_INT4_PACK_ASYM       w             int32 words   scales (dtype) aux = uint8 zero points,    group, -
  *                                                                          aux2 = int32 packed_zp
- *     (mq_int4_group_quant_pack_asym, one tensor per launch pair)
+ *     (mq_int4_group_quant_pack_asym; bf16 tensors on a 16-byte boundary with groups of 32 / 64 / 128 share their two
+ *      launches, codes and then packed zero points, with up to MQ_MAX_GROUP tensors)
  *     (mq_ue8m0_pack_scales with mn = rows, kb = cols, row_major = ld; its input is usually the scale output of an
  *      earlier job)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
@@ -275,7 +276,7 @@ int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
  * callers that submit one job list again and again, as a replayed weight sync does).  The kernel arguments of a launch
  * hold MQ_MAX_GROUP descriptors at most; a model of thousands of small tensors (the 18 432 expert matrices of a
  * Qwen3-30B-A3B sync, 3 MB each) then drains and refills the chip every 64 tensors.  With a table a launch of the
- * MXFP8, MXFP4 and symmetric INT4 jobs covers up to MQ_TABLE_GROUP tensors; every other job kind runs as in mq_run_jobs.
+ * MXFP8, MXFP4 and INT4 jobs (symmetric and asymmetric) covers up to MQ_TABLE_GROUP tensors; every other job kind runs as in mq_run_jobs.
  * mq_job_table_fill writes n entries of MQ_JOB_TABLE_ENTRY_BYTES bytes into host memory, entry i for jobs[i]; the
  * caller copies them to device memory (any 8-byte aligned address) and passes that address, together with the same
  * jobs, to mq_run_jobs_tabled.  A call may cover a sub-range of the list: pass jobs + k, n' and the address of entry k.

@@ -390,14 +390,20 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
         }
     }
 }
-template <int LANES>
-__global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const uint16_t* __restrict__ w,
-                                                                         uint32_t* __restrict__ packed,
-                                                                         uint16_t* __restrict__ scale_out,
-                                                                         uint8_t* __restrict__ zero_out,
-                                                                         int64_t total_units, int chunk) {
+// job: w, q = packed codes, s = scales, aux = zero points (one byte per group, read again by the zero-point packer),
+// aux2 = packed zero points, units, section = groups per row
+template <int LANES, class Table>
+__global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const Table tab) {
+    const FlatJob& job = flat_job(tab);
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ packed = (uint32_t*)job.q;
+    uint16_t* __restrict__ scale_out = (uint16_t*)job.s;
+    uint8_t* __restrict__ zero_out = (uint8_t*)job.aux;
+    const int64_t total_units = job.units;
     const int t = threadIdx.x;
-    const int64_t base = xcd_chunked_block(chunk) * (kI4Threads * kI4Unroll) + t;
+    const int64_t first = flat_block(tab) * (kI4Threads * kI4Unroll);
+    if (first >= total_units) return;
+    const int64_t base = first + t;
     // a group is a whole number of lanes, so dead lanes never share one with live lanes; they re-read the last unit
     u32x4 v[kI4Unroll];
 #pragma unroll
@@ -413,10 +419,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const u
 }
 
 // packed_zp[g, j] = sum_i zero[8j+i, g] << 4*order[i], order = {0,4,1,5,2,6,3,7}   (py:249-254)
-__global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
-                                                             uint32_t* __restrict__ packed_zp, int64_t M,
-                                                             int64_t groups_per_row) {
-    const int64_t rows8 = M / 8, total = groups_per_row * rows8;
+__device__ __forceinline__ void int4_zero_pack(const uint8_t* __restrict__ zero, uint32_t* __restrict__ packed_zp,
+                                               const int64_t rows8, const int64_t groups_per_row) {
+    const int64_t total = groups_per_row * rows8;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const int64_t g = i / rows8, j = i - g * rows8;
@@ -428,6 +433,20 @@ __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __re
         }
         packed_zp[i] = word;
     }
+}
+__global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
+                                                             uint32_t* __restrict__ packed_zp, int64_t M,
+                                                             int64_t groups_per_row) {
+    int4_zero_pack(zero, packed_zp, M / 8, groups_per_row);
+}
+// the zero points of a group of tensors (descriptors as for int4_pack_asym_bf16_kernel): blockIdx.y selects the tensor;
+// a tensor of `units` 16-byte units has units / units_per_group groups, groups_per_row of them in each row
+template <class Table>
+__global__ __launch_bounds__(256) void int4_zero_pack_group_kernel(const Table tab, int units_per_group) {
+    const FlatJob& job = flat_job(tab);
+    const int64_t groups_per_row = job.section;
+    if (groups_per_row <= 0) return;
+    int4_zero_pack((const uint8_t*)job.aux, (uint32_t*)job.aux2, job.units / units_per_group / groups_per_row / 8, groups_per_row);
 }
 
 // ---- fake INT4 quantization of row blocks (1, G), G = 32 / 64 / 128 ------------------------------------------------
@@ -638,6 +657,41 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
     return mq_check_launch("int4 pack");
 }
 
+bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M) {
+    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32) && M % 8 == 0;
+}
+
+// The two launches of an asymmetric pack for a group of tensors: codes + scales + zero points, then the zero points
+// packed eight rows to a word.  max_units: the largest tensor's 16-byte units.
+template <class Table>
+static int int4_pack_asym_launch(const Table& tab, int n, int64_t max_units, int group, hipStream_t st) {
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)n), blk(kI4Threads);
+    if (group == 128) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<16, Table>), grid, blk, 0, st, tab);
+    else if (group == 64) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<8, Table>), grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<4, Table>), grid, blk, 0, st, tab);
+    int rc = mq_check_launch("int4 asymmetric pack");
+    if (rc != MQ_OK) return rc;
+    const int64_t zp_words = max_units / group;             // (K / group) * (M / 8) words per tensor
+    int64_t zblocks = (zp_words + 255) / 256;
+    if (zblocks > mq_grid_cap()) zblocks = mq_grid_cap();
+    if (zblocks < 1) zblocks = 1;
+    hipLaunchKernelGGL(int4_zero_pack_group_kernel<Table>, dim3((unsigned)zblocks, (unsigned)n), dim3(256), 0, st, tab, group / 8);
+    return mq_check_launch("int4 zero-point pack");
+}
+int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st) {
+    if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) return MQ_OK;
+    int64_t max_units = 0;
+    for (int i = 0; i < tab.n; i++) max_units = tab.job[i].units > max_units ? tab.job[i].units : max_units;
+    return int4_pack_asym_launch(tab, tab.n, max_units, group, st);
+}
+int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st) {
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (ref.max_blocks == 0 || n == 0) return MQ_OK;
+    return int4_pack_asym_launch(ref, n, max_units, group, st);
+}
+
 extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
                                              int32_t* packed_zp, int64_t M, int64_t K, int group, void* stream) {
     if ((!w || !packed || !scale || !zero || !packed_zp) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -651,19 +705,11 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     int64_t blocks = (groups + 15) / 16;
     if (blocks > mq_grid_cap() * 4) blocks = mq_grid_cap() * 4;
     const int wpg = group / 8;
-    if (aligned && dtype == MQ_BF16 && (group == 128 || group == 64 || group == 32)) {
-        const int64_t units = M * (K / 8);
-        int64_t fblocks = (units + kI4Threads * kI4Unroll - 1) / (kI4Threads * kI4Unroll);
-        const int chunk = (int)flat_chunk(fblocks);
-        fblocks = flat_padded(fblocks, chunk);
-        if (fblocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
-        const dim3 grid((unsigned)fblocks), blk(kI4Threads);
-        if (group == 128)
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<16>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
-        else if (group == 64)
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<8>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
-        else
-            hipLaunchKernelGGL(int4_pack_asym_bf16_kernel<4>, grid, blk, 0, st, (const uint16_t*)w, (uint32_t*)packed, (uint16_t*)scale, zero, units, chunk);
+    if (mq_int4_pack_asym_fast_ok(w, dtype, group, M)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = FlatJob{w, packed, scale, zero, M * (K / 8), packed_zp, (int32_t)gpr, 0};
+        return mq_int4_pack_asym_launch_group(tab, group, st);
     } else if (dtype == MQ_BF16)
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     else if (dtype == MQ_F16)

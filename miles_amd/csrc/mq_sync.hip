@@ -34,6 +34,9 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
 int mq_mxfp8_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
+bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M);
+int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st);
+int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -59,6 +62,8 @@ static bool job_fast(const mq_job& j) {
             return mq_mxfp8_fast_ok(j.in, j.dtype, j.out) && j.cols % 32 == 0;
         case MQ_JOB_INT4_PACK:
             return mq_int4_pack_fast_ok(j.in, j.dtype, j.p0) && j.cols % j.p0 == 0 && j.cols % 8 == 0;
+        case MQ_JOB_INT4_PACK_ASYM:
+            return mq_int4_pack_asym_fast_ok(j.in, j.dtype, j.p0, j.rows) && j.cols % j.p0 == 0;
         case MQ_JOB_NVFP4:
             return mq_nvfp4_fast_ok(j.in, j.dtype, j.out) && j.cols % 16 == 0 && (j.p0 == 448 || j.p0 == 256);
         case MQ_JOB_MXFP4:
@@ -132,8 +137,12 @@ static_assert(kMaxGroup == MQ_MAX_GROUP, "the public group size must match the l
 static_assert(sizeof(FlatJob) == MQ_JOB_TABLE_ENTRY_BYTES && kTableGroup == MQ_TABLE_GROUP, "the public table entry must match FlatJob");
 
 // job kinds whose grouped launch can read its descriptors from a device table
-static bool table_kind(int kind) { return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK; }
+static bool table_kind(int kind) {
+    return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK || kind == MQ_JOB_INT4_PACK_ASYM;
+}
 static FlatJob flat_entry(const mq_job& jb) {
+    if (jb.kind == MQ_JOB_INT4_PACK_ASYM)       // zero points, packed zero points, groups per row
+        return FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, jb.p0 > 0 ? (int32_t)(jb.cols / jb.p0) : 0, 0};
     return FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8, nullptr, 0, 0};
 }
 
@@ -340,19 +349,22 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
             }
             case MQ_JOB_MXFP8:
             case MQ_JOB_MXFP4:
-            case MQ_JOB_INT4_PACK: {
+            case MQ_JOB_INT4_PACK:
+            case MQ_JOB_INT4_PACK_ASYM: {
                 if (tabled && cnt > kMaxGroup) {        // small groups keep the kernel-argument form (no pointer chase)
-                    rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_table(table + i, cnt, mx / 8, st)
-                         : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_table(table + i, cnt, mx / 8, st)
-                                                     : mq_int4_pack_launch_table(table + i, cnt, mx / 8, head.p0, st);
+                    rc = head.kind == MQ_JOB_MXFP8       ? mq_mxfp8_launch_table(table + i, cnt, mx / 8, st)
+                         : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_table(table + i, cnt, mx / 8, st)
+                         : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_table(table + i, cnt, mx / 8, head.p0, st)
+                                                         : mq_int4_pack_asym_launch_table(table + i, cnt, mx / 8, head.p0, st);
                     break;
                 }
                 FlatTable tab{};
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) tab.job[t] = flat_entry(jobs[i + t]);
-                rc = head.kind == MQ_JOB_MXFP8   ? mq_mxfp8_launch_group(tab, st)
-                     : head.kind == MQ_JOB_MXFP4 ? mq_mxfp4_launch_group(tab, st)
-                                                 : mq_int4_pack_launch_group(tab, head.p0, st);
+                rc = head.kind == MQ_JOB_MXFP8       ? mq_mxfp8_launch_group(tab, st)
+                     : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_group(tab, st)
+                     : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_group(tab, head.p0, st)
+                                                     : mq_int4_pack_asym_launch_group(tab, head.p0, st);
                 break;
             }
             case MQ_JOB_COPY: {

@@ -77,17 +77,24 @@ def _head_dim(args) -> int:
 
 def gather_groups(parts: torch.Tensor, shape) -> torch.Tensor:
     """`parts` [groups, ...] is a strided selection of each group's rows (or elements) whose per-group piece is
-    contiguous; returns the pieces back to back as a tensor of `shape`.  On the GPU the regrouping is one byte-copy job
-    per group instead of a torch copy, so a recorded sync can repeat it on the current weights (a replayed plan hands
+    contiguous; returns the pieces back to back as a tensor of `shape`.  On the GPU the regrouping is one 2-D byte-copy
+    job (one job per group where the pieces cannot be seen as rows of one view) instead of a torch copy, so a recorded sync can repeat it on the current weights (a replayed plan hands
     out the same output tensor, refreshed by the job)."""
     if parts.device.type != "cuda":
         return parts.reshape(shape)
-    from miles_amd.weight_update.packed_bucket import submit_copy
+    from miles_amd.weight_update.packed_bucket import submit_copy, submit_copy_rows
 
     out = torch.empty(parts.numel(), dtype=parts.dtype, device=parts.device).view(shape)
     flat = out.view(parts.shape[0], -1)
-    for g in range(parts.shape[0]):
-        submit_copy(parts[g].reshape(-1), flat[g])
+    try:
+        rows = parts.view(parts.shape[0], -1)      # the groups' pieces one group pitch apart: a single 2-D copy job
+    except RuntimeError:
+        rows = None
+    if rows is not None and parts.numel():
+        submit_copy_rows(rows, flat)
+    else:
+        for g in range(parts.shape[0]):
+            submit_copy(parts[g].reshape(-1), flat[g])
     return out
 
 

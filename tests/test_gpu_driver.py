@@ -535,8 +535,8 @@ def test_unquantized_sync_hands_out_current_regrouped_qkv():
         for n, w in want.items():
             _same(flat[n], w, n)
         assert upd._plan is not None and upd._plan.replayable
-        if packed:      # q / k / v are assembled in their payload slots: 12 gathering copies, 19 pass-through copies, none twice
-            assert len(upd._plan.batch) == 31
+        if packed:      # q / k / v are assembled in their payload slots: 6 gathering 2-D copies, 19 pass-through copies, none twice
+            assert len(upd._plan.batch) == 25
 
 
 def test_packed_buckets_int4_moe_two_syncs(oracle):
@@ -1008,7 +1008,7 @@ def test_recording_a_sync_holds_no_more_than_a_few_buckets():
     assert outputs > 5 * plan.arena_bytes
 
 
-@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4"])
+@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4", "int4_asym"])
 def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     """More than MQ_MAX_GROUP jobs of a table kind: the batch copies their descriptors to device memory and one launch
     covers the lot.  Shapes vary inside the 25 % band that keeps a group together, with a few far outside it (which
@@ -1022,6 +1022,8 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     g = torch.Generator().manual_seed(77)
     shapes = [(int(torch.randint(52, 64, (1,), generator=g)), 256) for _ in range(150)]
     shapes[40], shapes[41], shapes[120] = (8, 128), (300, 256), (1, 128)
+    if fmt == "int4_asym":          # packed zero points take eight rows to a word
+        shapes = [((r + 7) // 8 * 8, k) for r, k in shapes]
     ws = [W.student_t_rows(s, std=0.02, seed=7700 + i) for i, s in enumerate(shapes)]
     dev = [w.to(DEV) for w in ws]
     tile_w = W.gaussian_outliers((256, 384), std=0.02, p_outlier=0.001, gain=20.0, seed=7)
@@ -1031,14 +1033,14 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
             return mxfp8_quantize(w)
         if fmt == "mxfp4":
             return quantize_mxfp4(w, 32)
-        return pack_layer(w, 128)[:2]
+        return pack_layer(w, 128, sym=fmt == "int4")[:3 if fmt == "int4_asym" else 2]
 
     def expected(w):
         if fmt == "mxfp8":
             return oracle.mxfp8_quantize(w)
         if fmt == "mxfp4":
             return oracle.quantize_mxfp4(w, 32)
-        return oracle.pack_layer(w, 128)[:2]
+        return oracle.pack_layer(w, 128, sym=fmt == "int4")[:3 if fmt == "int4_asym" else 2]
 
     with launch.recording() as batch:
         outs = [quantize(w) for w in dev[:75]]
