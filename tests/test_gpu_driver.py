@@ -1154,3 +1154,27 @@ def test_a_2d_copy_that_reads_what_an_earlier_copy_wrote_runs_after_it():
         submit_copy_rows(b[:, 32:], c)                      # reads rows of b: must see what the first job wrote
     torch.cuda.synchronize()
     assert torch.equal(c, a[:, 32:])
+
+
+def test_snapshot_publisher_writes_the_quantized_model(oracle, tmp_path):
+    """The export entry of the weight iterator: shards on disk hold what the sync would have sent."""
+    import json
+
+    import safetensors.torch
+
+    from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorDirect
+    from miles_amd.weight_update.snapshot_publisher import SnapshotPublisher
+
+    cpu = _dense_model(77)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    iterator = HfWeightIteratorDirect(ARGS, model_name="qwen3", quantization_config=FP8_CFG)
+    SnapshotPublisher(iterator).write_model(tmp_path, weights=dev, hf_checkpoint=str(tmp_path / "absent"))
+    index = json.loads((tmp_path / "model.safetensors.index.json").read_text())
+    got = {}
+    for shard in sorted(set(index["weight_map"].values())):
+        got.update(safetensors.torch.load_file(tmp_path / shard))
+    want = _expected_fp8(oracle, cpu)
+    assert list(index["weight_map"]) == [n for n, _ in want]
+    for n, w in want:
+        _same(got[n], w, n)
+    assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for _, t in want)

@@ -570,3 +570,54 @@ def test_shared_divisor_division_is_exact_and_keeps_the_sign_of_zero():
     want = x / s
     assert np.array_equal(q.view(np.uint32), want.view(np.uint32))
     assert np.array_equal(np.signbit(q[:1024]), np.signbit(x[:1024])) and not q[:1024].any()
+
+
+# ---------------------------------------------------------------------------------------------------
+# quantized snapshot export (miles/backends/training_utils/weight_update/snapshot_publisher.py:62-99)
+def test_snapshot_publisher_writes_shards_index_and_metadata(tmp_path):
+    import json
+
+    import safetensors.torch
+
+    from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorDirect
+    from miles_amd.weight_update.snapshot_publisher import SnapshotPublisher
+
+    args = Namespace(**vars(QWEN_ARGS), update_weight_buffer_size=20000)
+    L = "module.module.decoder.layers.0."
+    weights = {"module.module.embedding.word_embeddings.weight": torch.randn(100, 64).to(torch.bfloat16),
+               L + "self_attention.linear_proj.weight": torch.randn(64, 64).to(torch.bfloat16),
+               L + "mlp.linear_fc1.weight": torch.randn(64, 64).to(torch.bfloat16),
+               L + "mlp.linear_fc2.weight": torch.randn(64, 32).to(torch.bfloat16),
+               "module.module.decoder.final_layernorm.weight": torch.randn(64).to(torch.bfloat16)}
+    base = tmp_path / "base"
+    base.mkdir()
+    (base / "config.json").write_text('{"model_type": "qwen3"}')
+    (base / "tokenizer.json").write_text("{}")
+    (base / "model.safetensors.index.json").write_text('{"weight_map": {"stale": "x"}}')
+    (base / "model-00001-of-00001.safetensors").write_bytes(b"not copied")
+    out = tmp_path / "snapshot"
+    out.mkdir()
+    iterator = HfWeightIteratorDirect(args, model_name="qwen3", quantization_config=None)
+    SnapshotPublisher(iterator).write_model(out, weights=weights, hf_checkpoint=str(base))
+
+    index = json.loads((out / "model.safetensors.index.json").read_text())
+    shards = sorted(p.name for p in out.glob("model-*.safetensors"))
+    assert len(shards) > 1 and shards[0] == "model-00001.safetensors" and set(index["weight_map"].values()) == set(shards)
+    assert sorted(p.name for p in out.iterdir() if not p.name.startswith("model")) == ["config.json", "tokenizer.json"]
+    got = {}
+    for shard in shards:
+        got.update(safetensors.torch.load_file(out / shard))
+    want = {}
+    for name, param in weights.items():
+        want.update(dict(name_maps.convert_qwen2_to_hf(args, name, param)))
+    assert set(got) == set(want) == set(index["weight_map"])
+    for name, t in want.items():
+        assert torch.equal(got[name], t.contiguous())
+    assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for t in want.values())
+    # a base checkpoint that is not a local directory: the shards and the index are still written
+    out2 = tmp_path / "snapshot2"
+    out2.mkdir()
+    SnapshotPublisher(iterator).write_model(out2, weights=weights, hf_checkpoint="Qwen/Qwen3-4B")
+    assert (out2 / "model.safetensors.index.json").exists() and not (out2 / "config.json").exists()
+    with pytest.raises(AssertionError, match="produced no weights"):
+        SnapshotPublisher(iterator).write_model(out2, weights={}, hf_checkpoint=str(base))
