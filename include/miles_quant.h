@@ -276,7 +276,8 @@ int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
  * callers that submit one job list again and again, as a replayed weight sync does).  The kernel arguments of a launch
  * hold MQ_MAX_GROUP descriptors at most; a model of thousands of small tensors (the 18 432 expert matrices of a
  * Qwen3-30B-A3B sync, 3 MB each) then drains and refills the chip every 64 tensors.  With a table a launch of the
- * MXFP8, MXFP4 and INT4 jobs (symmetric and asymmetric) covers up to MQ_TABLE_GROUP tensors; every other job kind runs as in mq_run_jobs.
+ * MXFP8, MXFP4, INT4 (symmetric and asymmetric) and 128x128 FP8 jobs covers up to MQ_TABLE_GROUP tensors of similar size;
+ * every other job kind, and FP8 jobs of mixed shapes, run as in mq_run_jobs.
  * mq_job_table_fill writes n entries of MQ_JOB_TABLE_ENTRY_BYTES bytes into host memory, entry i for jobs[i]; the
  * caller copies them to device memory (any 8-byte aligned address) and passes that address, together with the same
  * jobs, to mq_run_jobs_tabled.  A call may cover a sub-range of the list: pass jobs + k, n' and the address of entry k.

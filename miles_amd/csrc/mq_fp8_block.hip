@@ -45,14 +45,30 @@ __device__ __forceinline__ float ceil_pow2_scale(float v) {
 // output.  A lane adds 32-bit offsets to those bases.  Interior tiles take a path with no bounds tests at all; edge
 // tiles load from clamped (always valid) addresses and zero what lies outside, so that in both cases the four loads of
 // a lane are issued back to back.
-template <int MODE>
-__global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const TileTable tab) {
-    __shared__ uint32_t wave_amax[kTileWaves];
+// which tensor and which of its tiles a workgroup works on: searched in the running counts of a kernel-argument table, or
+// read off the two-dimensional grid of a device table (the workgroup then leaves if its tensor has fewer tiles)
+struct TilePick {
+    int32_t ji;         // index into tab.job
+    int32_t tile;       // -1: nothing to do
+};
+__device__ __forceinline__ TilePick pick_tile(const TileTable& tab) {
     const int32_t item = xcd_contiguous_item(tab.total);
-    if (item < 0) return;
+    if (item < 0) return TilePick{0, -1};
     const JobRef ref = find_job(tab, item);
-    const TileJob& job = tab.job[ref.ji];
-    const uint32_t tile = (uint32_t)(item - ref.start);
+    return TilePick{ref.ji, item - ref.start};
+}
+__device__ __forceinline__ TilePick pick_tile(const TileRef& tab) {
+    const TileJob& job = tab.job[blockIdx.y];
+    const int32_t tiles = ((job.M + kTile - 1) / kTile) * ((job.K + kTile - 1) / kTile);
+    return TilePick{(int32_t)blockIdx.y, xcd_contiguous_item(tiles)};
+}
+template <int MODE, class Table>
+__global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table tab) {
+    __shared__ uint32_t wave_amax[kTileWaves];
+    const TilePick pick = pick_tile(tab);
+    if (pick.tile < 0) return;
+    const TileJob& job = tab.job[pick.ji];
+    const uint32_t tile = (uint32_t)pick.tile;
     const uint32_t M = (uint32_t)job.M, K = (uint32_t)job.K, ldw = (uint32_t)job.ldw;
     const uint32_t tiles_k = (K + kTile - 1) / kTile;
     uint32_t ti = tile, tj = 0;
@@ -524,26 +540,43 @@ bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, con
            sxm < (1 << 24);
 }
 
+// fills the division constants of a descriptor whose w, q, scale, ldw, M, K and row blocks are set; returns its tile count
+int64_t mq_fp8_tile_job_finish(TileJob& j) {
+    const uint32_t tiles_k = (uint32_t)((j.K + kTile - 1) / kTile);
+    uint32_t shift_k = 0, shift_b = 0;
+    if (tiles_k > 1) tile_div_magic(tiles_k, j.magic_k, shift_k);
+    if (j.tiles_per_block > 1) tile_div_magic((uint32_t)j.tiles_per_block, j.magic_b, shift_b);
+    j.shifts = shift_k | (shift_b << 8);
+    return (int64_t)((j.M + kTile - 1) / kTile) * tiles_k;
+}
+
+// n finished descriptors in device memory; max_tiles: the largest tensor's tile count
+int mq_fp8_tile_launch_table(int mode, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st) {
+    if (n == 0 || max_tiles == 0) return MQ_OK;
+    const int64_t gx = xcd_grid(max_tiles);
+    if (gx >= 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "too many tiles");
+    const TileRef ref{device_jobs};
+    const dim3 grid((unsigned)gx, (unsigned)n), blk(kTileThreads);
+    if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, TileRef>), grid, blk, 0, st, ref);
+    else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, TileRef>), grid, blk, 0, st, ref);
+    else hipLaunchKernelGGL((fp8_block128_kernel<2, TileRef>), grid, blk, 0, st, ref);
+    return mq_check_launch("fp8 block quant");
+}
+
 // tab.job[i] filled by the caller (w, q, scale, ldw, M, K, row blocks); fills the division constants and `end`, launches
 int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
     int64_t tiles = 0;
     for (int i = 0; i < tab.n; i++) {
-        TileJob& j = tab.job[i];
-        const uint32_t tiles_k = (uint32_t)((j.K + kTile - 1) / kTile);
-        uint32_t shift_k = 0, shift_b = 0;
-        if (tiles_k > 1) tile_div_magic(tiles_k, j.magic_k, shift_k);
-        if (j.tiles_per_block > 1) tile_div_magic((uint32_t)j.tiles_per_block, j.magic_b, shift_b);
-        j.shifts = shift_k | (shift_b << 8);
-        tiles += (int64_t)((j.M + kTile - 1) / kTile) * tiles_k;
+        tiles += mq_fp8_tile_job_finish(tab.job[i]);
         if (tiles >= 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "too many tiles");
         tab.end[i] = (int32_t)tiles;
     }
     if (tiles == 0) return MQ_OK;
     seal_table(tab);
     const int64_t grid = xcd_grid(tiles);
-    if (mode == 0) hipLaunchKernelGGL(fp8_block128_kernel<0>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
-    else if (mode == 1) hipLaunchKernelGGL(fp8_block128_kernel<1>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
-    else hipLaunchKernelGGL(fp8_block128_kernel<2>, dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    else hipLaunchKernelGGL((fp8_block128_kernel<2, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
     return mq_check_launch("fp8 block quant");
 }
 

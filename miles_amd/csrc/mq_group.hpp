@@ -81,6 +81,13 @@ struct TileTable {
     TileJob job[kMaxGroup];
 };
 
+// Tile descriptors in device memory (see FlatRef below): tensors of similar tile counts on a two-dimensional grid,
+// blockIdx.y the tensor and blockIdx.x the tile (gridDim.x is the largest count, rounded up for the XCD dealing), so no
+// search is needed however many tensors the launch covers.
+struct TileRef {
+    const TileJob* job;
+};
+
 struct FlatJob {      // one tensor seen as a flat run of 16-byte input units
     const void* w;
     void* q;

@@ -18,6 +18,8 @@ using namespace mq;
 bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, const void* q, int64_t M, int64_t K,
                          int bm, int bk);
 int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st);
+int64_t mq_fp8_tile_job_finish(TileJob& j);
+int mq_fp8_tile_launch_table(int mode, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st);
 bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block);
 int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st);
 bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q);
@@ -134,12 +136,22 @@ static int run_single(const mq_job& j, void* stream) {
 }
 
 static_assert(kMaxGroup == MQ_MAX_GROUP, "the public group size must match the launch tables");
-static_assert(sizeof(FlatJob) == MQ_JOB_TABLE_ENTRY_BYTES && kTableGroup == MQ_TABLE_GROUP, "the public table entry must match FlatJob");
+static_assert(sizeof(FlatJob) == MQ_JOB_TABLE_ENTRY_BYTES && sizeof(TileJob) == MQ_JOB_TABLE_ENTRY_BYTES &&
+              kTableGroup == MQ_TABLE_GROUP, "the public table entry must match FlatJob and TileJob");
 
-// job kinds whose grouped launch can read its descriptors from a device table
-static bool table_kind(int kind) {
-    return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK || kind == MQ_JOB_INT4_PACK_ASYM;
+// job kinds whose grouped launch can read its descriptors from a device table: the flat kernels and the FP8 tile kernel
+static bool tile_kind(int kind) {
+    return kind == MQ_JOB_FP8_BLOCK || kind == MQ_JOB_FP8_BLOCKWISE_CAST || kind == MQ_JOB_FP8_BLOCK_POW2;
 }
+static bool table_kind(int kind) {
+    return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK || kind == MQ_JOB_INT4_PACK_ASYM ||
+           tile_kind(kind);
+}
+static TileJob tile_entry(const mq_job& jb) {
+    return TileJob{jb.in, jb.out, (float*)jb.scale, (int32_t)jb.ld, (int32_t)jb.rows, (int32_t)jb.cols,
+                   (int32_t)jb.block_stride, (int32_t)(jb.rows_per_block / 128), 0, 0, 0};
+}
+static int64_t tiles_of(const mq_job& jb) { return ((jb.rows + 127) / 128) * ((jb.cols + 127) / 128); }
 static FlatJob flat_entry(const mq_job& jb) {
     if (jb.kind == MQ_JOB_INT4_PACK_ASYM)       // zero points, packed zero points, groups per row
         return FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, jb.p0 > 0 ? (int32_t)(jb.cols / jb.p0) : 0, 0};
@@ -270,8 +282,15 @@ static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
 extern "C" int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table) {
     if (n < 0 || (n > 0 && (!jobs || !host_table))) return mq_fail(MQ_ERR_ARG, "bad job list");
     for (int64_t i = 0; i < n; i++) {
-        const FlatJob e = table_kind(jobs[i].kind) ? flat_entry(jobs[i]) : FlatJob{};
-        memcpy((char*)host_table + i * sizeof(FlatJob), &e, sizeof(FlatJob));
+        char* slot = (char*)host_table + i * MQ_JOB_TABLE_ENTRY_BYTES;
+        if (tile_kind(jobs[i].kind) && job_fast(jobs[i])) {
+            TileJob e = tile_entry(jobs[i]);
+            mq_fp8_tile_job_finish(e);
+            memcpy(slot, &e, sizeof(e));
+        } else {
+            const FlatJob e = table_kind(jobs[i].kind) && !tile_kind(jobs[i].kind) ? flat_entry(jobs[i]) : FlatJob{};
+            memcpy(slot, &e, sizeof(e));
+        }
     }
     return MQ_OK;
 }
@@ -310,7 +329,29 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
         const bool flat = head.kind != MQ_JOB_FP8_BLOCK && head.kind != MQ_JOB_FP8_BLOCKWISE_CAST &&
                           head.kind != MQ_JOB_FP8_BLOCK_POW2 && head.kind != MQ_JOB_COPY;
         const bool tabled = table != nullptr && table_kind(head.kind);
-        const int64_t group_cap = tabled ? kTableGroup : kMaxGroup;
+        if (tabled && tile_kind(head.kind)) {
+            // tile jobs of similar tile counts (an MoE layer's experts) beyond what the kernel arguments hold: one launch
+            // on a (largest tile count) x (tensors) grid; mixed shapes keep the searched form below, 64 tensors at a time
+            int64_t j = i + 1, sum = tiles_of(head), mx = sum;
+            while (j < n && j - i < kTableGroup && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
+                   jobs[j].cols > 0) {
+                const int64_t e = tiles_of(jobs[j]);
+                const int64_t nmx = e > mx ? e : mx;
+                if (nmx * (j - i + 1) * 4 > (sum + e) * 5) break;
+                sum += e;
+                mx = nmx;
+                j++;
+            }
+            // (tensors of 256 tiles and more fill a searched launch of 64 well enough, and run 1-2 % faster in that form)
+            if (j - i > kMaxGroup && mx < 256) {
+                const int mode = head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2;
+                int rc = mq_fp8_tile_launch_table(mode, (const TileJob*)table + i, (int)(j - i), mx, st);
+                if (rc) return rc;
+                i = j;
+                continue;
+            }
+        }
+        const int64_t group_cap = tabled && !tile_kind(head.kind) ? kTableGroup : kMaxGroup;
         int64_t j = i + 1, sum = head.rows * head.cols, mx = sum;
         while (j < n && j - i < group_cap && same_group(head, jobs[j]) && job_fast(jobs[j]) && jobs[j].rows > 0 &&
                jobs[j].cols > 0) {
@@ -332,8 +373,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) {
                     const mq_job& jb = jobs[i + t];
-                    tab.job[t] = TileJob{jb.in, jb.out, (float*)jb.scale, (int32_t)jb.ld, (int32_t)jb.rows, (int32_t)jb.cols,
-                                         (int32_t)jb.block_stride, (int32_t)(jb.rows_per_block / 128), 0, 0, 0};
+                    tab.job[t] = tile_entry(jb);
                 }
                 rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2, tab, st);
                 break;

@@ -1008,7 +1008,7 @@ def test_recording_a_sync_holds_no_more_than_a_few_buckets():
     assert outputs > 5 * plan.arena_bytes
 
 
-@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4", "int4_asym"])
+@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4", "int4_asym", "fp8", "block_fp8"])
 def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     """More than MQ_MAX_GROUP jobs of a table kind: the batch copies their descriptors to device memory and one launch
     covers the lot.  Shapes vary inside the 25 % band that keeps a group together, with a few far outside it (which
@@ -1016,6 +1016,7 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     from miles_amd import launch
     from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
     from miles_amd.megatron_to_hf.processors.quantizer_compressed_tensors import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
     from miles_amd.utils.mxfp4 import quantize_mxfp4
     from miles_amd.utils.mxfp8 import mxfp8_quantize
 
@@ -1024,11 +1025,18 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     shapes[40], shapes[41], shapes[120] = (8, 128), (300, 256), (1, 128)
     if fmt == "int4_asym":          # packed zero points take eight rows to a word
         shapes = [((r + 7) // 8 * 8, k) for r, k in shapes]
+    if fmt in ("fp8", "block_fp8"):  # 128x128 tiles: two row tiles by three column tiles, the last of each partial
+        shapes = [(130 + (r * 7 + i) % 120, 264 + 8 * (i % 3)) for i, (r, k) in enumerate(shapes)]
+        shapes[40], shapes[41], shapes[120], shapes[130] = (8, 128), (1300, 256), (1, 8), (256, 384)
     ws = [W.student_t_rows(s, std=0.02, seed=7700 + i) for i, s in enumerate(shapes)]
     dev = [w.to(DEV) for w in ws]
     tile_w = W.gaussian_outliers((256, 384), std=0.02, p_outlier=0.001, gain=20.0, seed=7)
 
     def quantize(w):
+        if fmt == "fp8":
+            return fp8_blockwise_cast(w)
+        if fmt == "block_fp8":
+            return block_fp8(w, [128, 128])
         if fmt == "mxfp8":
             return mxfp8_quantize(w)
         if fmt == "mxfp4":
@@ -1036,6 +1044,10 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
         return pack_layer(w, 128, sym=fmt == "int4")[:3 if fmt == "int4_asym" else 2]
 
     def expected(w):
+        if fmt == "fp8":
+            return oracle.fp8_blockwise_cast(w)
+        if fmt == "block_fp8":
+            return oracle.block_fp8(w, (128, 128))
         if fmt == "mxfp8":
             return oracle.mxfp8_quantize(w)
         if fmt == "mxfp4":
