@@ -129,6 +129,10 @@ def per_quantizer(gen):
     run("C3_mxfp8", "mxfp8", 256 * 3 * 768 * 2048,
         lambda: [mxfp8_quantize(t) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
         "2 layers x 128 experts (gate, up [768,2048], down [2048,768]), 0.02 N(0,1) x Student-t(3) row scales")
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    run("next_fp8_cast_small_experts", "fp8_block", 256 * 3 * 768 * 2048,
+        lambda: [fp8_blockwise_cast(t) for fc1, fc2 in experts for t in (*fc1.chunk(2, dim=0), fc2)],
+        "the same 768 expert matrices through the sync path's FP8 128x128 quantizer (one launch over a device table)")
     del experts
     # C4: Kimi-K2-shaped experts, 32 of them, N(0, 0.015) + 0.05 % outliers x 30
     experts = [(_synth((4096, 7168), gen, std=0.015, p=0.0005, gain=30.0), _synth((7168, 2048), gen, std=0.015, p=0.0005, gain=30.0))
@@ -434,7 +438,7 @@ def roofline(plan, elems, steps, gpu_ms):
     avg_us = gpu_ms * 1e3 / (steps * launches)
     bytes_per_launch = elems * BYTES_PER_ELEM["fp8_block"] / launches
     achieved = bytes_per_launch / avg_us / 1e3
-    return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+    return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1, mq::TileTable>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems / launches),
             "launches_per_sync": launches, "avg_launch_us": round(avg_us, 2),

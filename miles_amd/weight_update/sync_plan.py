@@ -51,12 +51,14 @@ class SyncPlan:
         self._names: list[str] = []
         self._tensors: list[torch.Tensor] = []
         self._addresses: list[int] = []
+        self._numels: list[int] = []
 
     def remember(self, weights: Mapping[str, torch.Tensor]) -> None:
         """Keep the parameter objects themselves, for the quick form of `matches`."""
         self._names = list(weights)
         self._tensors = list(weights.values())
         self._addresses = [t.data_ptr() for t in self._tensors]
+        self._numels = [t.numel() for t in self._tensors]
 
     @classmethod
     def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor], *,
@@ -91,15 +93,16 @@ class SyncPlan:
         """True when `weights` is the parameter set the plan was recorded on.  Between RL steps the mapping holds
         the very same tensor objects, so the usual answer costs one identity pass and one address per tensor (0.5 ms
         for 12 288 expert tensors, against 5 ms for the full signature, which builds a shape tuple per tensor).
-        The quick form takes the shapes of unchanged objects at unchanged addresses as unchanged: an in-place
-        `set_` / `resize_` that keeps the address would go unnoticed.  Anything else (other objects, other
+        The quick form takes the shapes of unchanged objects at unchanged addresses with unchanged element counts as
+        unchanged: an in-place `set_` that keeps address and size but changes the shape would go unnoticed.  Anything else (other objects, other
         names, another count) is decided by the full signature."""
         if not self.replayable:
             return False
         if len(weights) == len(self._tensors):
             tensors = list(weights.values())
             if all(map(operator.is_, tensors, self._tensors)) and list(weights) == self._names:
-                return list(map(torch.Tensor.data_ptr, tensors)) == self._addresses
+                return (list(map(torch.Tensor.data_ptr, tensors)) == self._addresses
+                        and list(map(torch.Tensor.numel, tensors)) == self._numels)
         return weights_signature(weights) == self.signature
 
     # a trailing launch smaller than this many elements is topped up with the next bucket's jobs

@@ -377,6 +377,10 @@ def test_sync_plan_matches_quick_and_full_forms():
     assert not plan.matches({("q" + k): v for k, v in weights.items()})   # same objects under other names
     weights["p2"].data = torch.zeros(4, 8)                                # storage swapped under the same object
     assert not plan.matches(weights)
+    plan.remember(weights)
+    assert plan.matches(weights)
+    weights["p3"].resize_(2, 8)                                           # same object, same address, fewer elements
+    assert not plan.matches(weights)
     plan.replayable = False
     plan.remember(weights)
     assert not plan.matches(weights)
