@@ -546,6 +546,31 @@ def stream_ceilings():
         torch.cuda.synchronize()
         ms = min(_event_ms(fn, 5) for _ in range(3))
         res[name] = {"GBps": round(nbytes / ms / 1e6, 1), "ms": round(ms, 4)}
+    del q
+    # the library's probes: kernels that only move bytes, in the access shapes of the quantizers (2 GiB on the larger side)
+    from miles_amd import _lib
+    lib, stream, big = _lib.load(), _lib.stream_ptr(x.device), 1 << 31
+    FLAT_2_1, FLAT_1_2, LOOP_2_1, TILE_2_1, TILE_READ, TILE_WRITE = range(6)
+
+    def probe(name, shape, param, moved):
+        def fn():
+            _lib.check(lib.mq_stream_probe(shape, x.data_ptr(), y.data_ptr(), big, param, stream))
+        fn()
+        torch.cuda.synchronize()
+        ms = min(_event_ms(fn, 10) for _ in range(3))
+        res[name] = {"GBps": round(moved / ms / 1e6, 1), "ms": round(ms, 4)}
+
+    for units in (1, 2, 4, 8):
+        probe(f"flat_2r_1w_{units}_units_per_lane", FLAT_2_1, units, big * 3 // 2)
+    for groups in (2048, 16384, 65536, 262144):
+        probe(f"loop_2r_1w_{groups}_workgroups", LOOP_2_1, groups, big * 3 // 2)
+    for units in (1, 2):
+        probe(f"flat_1r_2w_{units}_units_per_lane", FLAT_1_2, units, big * 3 // 2)
+    for k in (2048, 2560, 4096, 5120, 7168, 8192, 9728):
+        elems = (big // 2 // k // 128 * 128) * k
+        probe(f"tile128_2r_1w_K{k}", TILE_2_1, k, elems * 3)
+        probe(f"tile128_read_only_K{k}", TILE_READ, k, elems * 2)
+        probe(f"tile128_write_only_K{k}", TILE_WRITE, k, elems)
     return res
 
 

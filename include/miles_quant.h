@@ -299,6 +299,18 @@ int mq_selftest_convert(uint64_t* counts, void* stream);
 /* Plain 16-byte-per-lane copy used to calibrate achievable HBM bandwidth and rocprof counters. */
 int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
 
+/* Streaming probes (no counterpart in the reference; measurement only): kernels that only move bytes in the access
+ * shapes of the quantizers, to calibrate what a shape reaches on a GPU.  nbytes counts the larger side; dst must hold
+ * nbytes as well (the probes write at most that).
+ *   MQ_PROBE_FLAT_2_1   16 bytes read, 8 written per unit, one-shot workgroups; param = units per lane (1, 2, 4, 8)
+ *   MQ_PROBE_FLAT_1_2   8 bytes read, 16 written per unit; param = units per lane
+ *   MQ_PROBE_LOOP_2_1   the 2:1 mix as a grid of param workgroups striding over the buffer (param % 512 == 0)
+ *   MQ_PROBE_TILE_2_1 / _READ / _WRITE   128 x 128 tiles of a row-major matrix of 2-byte elements, param = its row
+ *                       length K; both sides, the reads alone, the writes alone */
+enum { MQ_PROBE_FLAT_2_1 = 0, MQ_PROBE_FLAT_1_2 = 1, MQ_PROBE_LOOP_2_1 = 2, MQ_PROBE_TILE_2_1 = 3, MQ_PROBE_TILE_READ = 4,
+       MQ_PROBE_TILE_WRITE = 5 };
+int mq_stream_probe(int shape, const void* src, void* dst, int64_t nbytes, int64_t param, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

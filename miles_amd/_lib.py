@@ -48,6 +48,7 @@ SIGNATURES = {
     "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
+    "mq_stream_probe": [_i32, _vp, _vp, _i64, _i64, _vp],
 }
 
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs

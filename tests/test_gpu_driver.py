@@ -1190,3 +1190,20 @@ def test_snapshot_publisher_writes_the_quantized_model(oracle, tmp_path):
     for n, w in want:
         _same(got[n], w, n)
     assert index["metadata"]["total_size"] == sum(t.numel() * t.element_size() for _, t in want)
+
+
+def test_stream_probes_run_and_refuse_bad_arguments():
+    """The measurement-only probes: every shape runs on a small buffer, stays inside it, and refuses what it cannot take."""
+    lib = _lib.load()
+    nbytes = 3 * 128 * 1024 * 2 + 4096                   # a [384, 1024] matrix of 2-byte elements and a little more
+    src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=DEV)
+    guard = 4096
+    dst = torch.full((nbytes + guard,), 0xA5, dtype=torch.uint8, device=DEV)
+    stream = _lib.stream_ptr(src.device)
+    for shape, param in ((0, 1), (0, 2), (0, 4), (0, 8), (1, 1), (1, 2), (2, 512), (3, 1024), (4, 1024), (5, 1024), (3, 128)):
+        assert lib.mq_stream_probe(shape, src.data_ptr(), dst.data_ptr(), nbytes, param, stream) == 0, (shape, param)
+    torch.cuda.synchronize()
+    assert bool((dst[nbytes:] == 0xA5).all())
+    for shape, param, size in ((0, 3, nbytes), (2, 100, nbytes), (3, 100, nbytes), (9, 1, nbytes), (0, 2, nbytes + 8), (3, 1 << 30, nbytes)):
+        assert lib.mq_stream_probe(shape, src.data_ptr(), dst.data_ptr(), size, param, stream) != 0, (shape, param, size)
+    assert lib.mq_stream_probe(0, None, dst.data_ptr(), nbytes, 2, stream) != 0
