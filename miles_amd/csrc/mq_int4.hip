@@ -107,15 +107,25 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         const bool fast = shared_div_ok(s);
+        // |x / s| <= 7 (1 + 2^-23), so the pattern of q + (1.5 * 2^23 + 8) is 0x4B400000 + nibble: the eight patterns
+        // are summed at their nibble's place (one shift-add each, modulo 2^32) and what the high bits added up to is
+        // taken off once.  (A wavefront that met an infinity, a NaN or the largest bf16 writes its words again below.)
+        constexpr uint32_t kMagicSum = 0x4B400000u + (0x4B400000u << 4) + (0x4B400000u << 8);     // further shifts: 0
         uint32_t word = 0;
+        if (__builtin_amdgcn_ballot_w64(!fast) == 0) {         // every scale of the wavefront in range: one straight run
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float qv = fast ? div_by_shared(f[j], s, y) : f[j] / s;
-            word |= (code_bits(qv) & 0xFu) << (4 * j);
+            for (int j = 0; j < 8; j++) word += code_bits(div_by_shared(f[j], s, y)) << (4 * j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float qv = fast ? div_by_shared(f[j], s, y) : f[j] / s;
+                word += code_bits(qv) << (4 * j);
+            }
         }
+        word -= kMagicSum;
         if (unit < total_units) {
             st4(packed + unit, word);
-            if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
+            if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)hw_bf16x2(s, 0.0f);
         }
     }
     // A group holding the largest finite bf16, an infinity or a NaN is outside the fused form: a wavefront that met one
