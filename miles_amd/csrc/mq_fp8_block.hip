@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
         tj = tile - ti * tiles_k;
     }
     // row-blocked input: the tile's rows sit in block ti / tiles_per_block, at the same offset inside it
-    const uint16_t* __restrict__ wt = (const uint16_t*)job.w;
+    const uint16_t* __restrict__ wt = (const uint16_t*)load_global_ptr(&job.w);
     uint32_t wti = ti;
     if (job.tiles_per_block > 0) {
         const uint32_t tpb = (uint32_t)job.tiles_per_block;
@@ -86,7 +86,8 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
         wti = ti - blk * tpb;
     }
     wt += (int64_t)wti * kTile * ldw + (int64_t)tj * kTile;
-    uint8_t* __restrict__ qt = (uint8_t*)job.q + (int64_t)ti * kTile * K + (int64_t)tj * kTile;
+    uint8_t* __restrict__ qt = (uint8_t*)load_global_ptr(&job.q) + (int64_t)ti * kTile * K + (int64_t)tj * kTile;
+    float* __restrict__ tile_scales = load_global_ptr(&job.scale);
     const uint32_t rows_left = M - ti * kTile, cols_left = K - tj * kTile;     // both at least 1
     const bool full = rows_left >= (uint32_t)kTile && cols_left >= (uint32_t)kTile;
 
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
             sx = u2f(m > 0x7F80u ? 0x7FC00000u : 0x7F800000u);
         }
         const float yx = 1.0f / sx;
-        if (t == 0) job.scale[tile] = sx;
+        if (t == 0) tile_scales[tile] = sx;
 #pragma unroll 1
         for (int i = 0; i < kRowsPerThread; i++) {
             const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
     else if (MODE == 1) s = (amax > 1e-10f ? amax : 1e-10f) / kFp8Max;
     else s = ceil_pow2_scale((amax > 1e-4f ? amax : 1e-4f) / kFp8Max);
     const float y = 1.0f / s;
-    if (t == 0) job.scale[tile] = s;
+    if (t == 0) tile_scales[tile] = s;
 
     if (MODE == 0 && !(amax > 0.0f) && amax == amax) {
         // all-zero tile: 0/0 on every element; the reference's CPU result is the negative NaN code

@@ -20,8 +20,8 @@ constexpr int kFtThreads = 256;
 constexpr int kFtUnroll = 2;
 
 // job.s = fp32 scale output, job.aux = amax record (section 0)
-template <int MODE>   // 1: fold and clear; 2: also compare with the amax the record held
-__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const FlatTable tab, float floor_v) {
+template <int MODE, class Table>   // 1: fold and clear; 2: also compare with the amax the record held
+__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, float floor_v) {
     __shared__ uint32_t lds4[4];
     const FlatJob& job = tab.job[blockIdx.x];
     uint32_t* rec = (uint32_t*)job.aux;
@@ -97,9 +97,9 @@ __device__ __forceinline__ uint32_t fp8_tensor_quant_units(const FlatJob& job, c
 
 // PASS 0: second pass of the two-pass form; 1: single pass with the carried-over amax, new partial maxima collected;
 // 2: grid-stride second quantization of the tensors whose amax moved
-template <int PASS>
-__global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const FlatTable tab, float floor_v) {
-    const FlatJob& job = tab.job[blockIdx.y];
+template <int PASS, class Table>
+__global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Table tab, float floor_v) {
+    const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const int t = threadIdx.x;
     constexpr int64_t kPerBlock = kFtThreads * kFtUnroll;
     if (PASS == 2) {
@@ -145,10 +145,29 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Flat
 using namespace mq;
 
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
+int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st);
 
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld) {
     return dtype == MQ_BF16 && cols % 8 == 0 && ld == cols && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 &&
            rows * (cols / 8) < (1ll << 38);
+}
+
+// fold + quantize (+ second pass) over a table whose grid is known
+template <class Table>
+static int fp8_tensor_launch(const Table& tab, int n, float floor_v, bool carry, hipStream_t st) {
+    const dim3 folds((unsigned)n), blk(256), grid((unsigned)tab.max_blocks, (unsigned)n);
+    if (carry) {
+        if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<1, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
+        hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v);
+        if (tab.max_blocks > 0) {
+            const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
+            hipLaunchKernelGGL((fp8_tensor_quant_kernel<2, Table>), dim3(redo, (unsigned)n), dim3(kFtThreads), 0, st, tab, floor_v);
+        }
+        return mq_check_launch("fp8 per-tensor quant (carried-over amax)");
+    }
+    hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v);
+    if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<0, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
+    return mq_check_launch("fp8 per-tensor quant");
 }
 
 // tab.job[i]: w, q, s = fp32 scale out, aux = amax record, units = numel / 8.  carry: see the file header.
@@ -163,17 +182,16 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
         if (rc) return rc;
     }
     if (!flat_grid(tab, kFtThreads * kFtUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    const dim3 folds((unsigned)tab.n), blk(256), grid((unsigned)tab.max_blocks, (unsigned)tab.n);
-    if (carry) {
-        if (tab.max_blocks > 0) hipLaunchKernelGGL(fp8_tensor_quant_kernel<1>, grid, dim3(kFtThreads), 0, st, tab, floor_v);
-        hipLaunchKernelGGL(fp8_tensor_fold_kernel<2>, folds, blk, 0, st, tab, floor_v);
-        if (tab.max_blocks > 0) {
-            const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
-            hipLaunchKernelGGL(fp8_tensor_quant_kernel<2>, dim3(redo, (unsigned)tab.n), dim3(kFtThreads), 0, st, tab, floor_v);
-        }
-        return mq_check_launch("fp8 per-tensor quant (carried-over amax)");
+    return fp8_tensor_launch(tab, tab.n, floor_v, carry, st);
+}
+// the same over n descriptors of a device table (section 0 in every entry); max_units: the largest tensor's units
+int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st) {
+    if (n == 0) return MQ_OK;
+    if (!carry) {
+        int rc = mq_nvfp4_amax_launch_table(device_jobs, n, st);
+        if (rc) return rc;
     }
-    hipLaunchKernelGGL(fp8_tensor_fold_kernel<1>, folds, blk, 0, st, tab, floor_v);
-    if (tab.max_blocks > 0) hipLaunchKernelGGL(fp8_tensor_quant_kernel<0>, grid, dim3(kFtThreads), 0, st, tab, floor_v);
-    return mq_check_launch("fp8 per-tensor quant");
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kFtThreads * kFtUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    return fp8_tensor_launch(ref, n, floor_v, carry, st);
 }

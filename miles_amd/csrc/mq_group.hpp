@@ -131,8 +131,22 @@ struct FlatRef {
     int32_t max_blocks;
 };
 constexpr int kTableGroup = 8192;         // tensors per launch of the device-table form (gridDim.y stays below 65 536)
+// the descriptor of this workgroup's tensor, copied into registers (a descriptor in device memory must not be read
+// again after the kernel's own stores) with its pointers loaded as global ones (see load_global_ptr)
 template <class Table>
-__device__ __forceinline__ const FlatJob& flat_job(const Table& tab) { return tab.job[blockIdx.y]; }
+__device__ __forceinline__ FlatJob flat_job(const Table& tab) {
+    const FlatJob& src = tab.job[blockIdx.y];
+    FlatJob j;
+    j.w = load_global_ptr(&src.w);
+    j.q = load_global_ptr(&src.q);
+    j.s = load_global_ptr(&src.s);
+    j.aux = load_global_ptr(&src.aux);
+    j.units = src.units;
+    j.aux2 = load_global_ptr(&src.aux2);
+    j.section = src.section;
+    j.pad = src.pad;
+    return j;
+}
 template <class Table>
 __device__ __forceinline__ int64_t flat_block(const Table& tab) { return xcd_chunked_block(tab.chunk); }
 // largest power-of-two chunk (up to MQ_FLAT_CHUNK) whose grid padding stays under 3 % of `blocks` workgroups

@@ -13,6 +13,8 @@
 // Pass 2 (mq_nvfp4_quant) reads those two factors with a scalar load; two lanes own one 16-element block
 // (16 bytes each), the block amax is one DPP step, and each lane emits four bytes of codes.  A gate/up pair
 // writes two sections of one record.
+#include <type_traits>
+
 #include "mq_api_internal.hpp"
 #include "mq_common.hpp"
 #include "mq_group.hpp"
@@ -37,12 +39,15 @@ constexpr int kAmaxUnroll = MQ_AMAX_UNROLL;             // 16-byte units per lan
 
 // grid (kSectionWords, tensors): workgroup b of a tensor strides over its 16 KiB chunks and writes word b of
 // the section.  job.units counts whole 16-byte units; job.s carries the element count for the sub-unit tail.
-__global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const FlatTable tab) {
+// (descriptors of a device table are in the quantizer's form, whose tensors are whole units: no tail, and job.s is the
+// block-scale pointer there)
+template <class Table>
+__global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const Table tab) {
     __shared__ uint32_t wave_amax[4];
-    const FlatJob& job = tab.job[blockIdx.y];
+    const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ section = (uint32_t*)job.aux + job.section * kSectionWords;
-    const int64_t n16 = job.units, numel = (int64_t)(uintptr_t)job.s;
+    const int64_t n16 = job.units, numel = std::is_same<Table, FlatRef>::value ? n16 * 8 : (int64_t)(uintptr_t)job.s;
     const int t = threadIdx.x;
     uint32_t m2 = 0;
     for (int64_t base = (int64_t)blockIdx.x * (256 * kAmaxUnroll); base < n16; base += (int64_t)kSectionWords * 256 * kAmaxUnroll) {
@@ -118,8 +123,8 @@ constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 //   its partial maxima (no codes are written with an amax that is likely stale again) and the second pass quantizes it
 //   with the fresh amax -- the cost of the plain two-pass form, instead of two full quantizations.  The mark is dropped
 //   as soon as the amax has held still for one sync.
-template <int MODE>
-__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const FlatTable tab, float numer) {
+template <int MODE, class Table>
+__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer) {
     __shared__ uint32_t lds4[4];
     const int ji = blockIdx.x;
     const FlatJob& job = tab.job[ji];
@@ -335,9 +340,9 @@ __device__ __forceinline__ uint32_t nvfp4_amax_units(const FlatJob& job, const i
 // atomic max per workgroup into the tensor's section, cleared by the previous fold); the fold kernel then compares, and
 // PASS 2, a small grid striding over the blocks, quantizes again only the tensors whose amax did change.
 // PASS 0 is the second pass of the plain two-pass form (amax kernel, fold, quantize).
-template <int FOS, int PASS>
-__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const FlatTable tab, float denom) {
-    const FlatJob& job = tab.job[blockIdx.y];
+template <int FOS, int PASS, class Table>
+__global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Table tab, float denom) {
+    const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const int t = threadIdx.x;
     constexpr int64_t kPerBlock = kNvThreads * kNvUnroll;
     if (PASS == 2) {
@@ -520,20 +525,54 @@ bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q) {
 
 // tab.job[i]: w, aux = amax record, section, units = numel / 8, s = (void*)numel
 int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
-    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel, dim3(kSectionWords, (unsigned)tab.n), dim3(256), 0, st, tab);
+    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel<FlatTable>, dim3(kSectionWords, (unsigned)tab.n), dim3(256), 0, st, tab);
+    return mq_check_launch("nvfp4 amax");
+}
+// the same over n descriptors of a device table (the quantizer's form: whole units, section = place inside the record)
+int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st) {
+    if (n == 0) return MQ_OK;
+    const FlatRef ref{device_jobs, 0, 0};
+    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel<FlatRef>, dim3(kSectionWords, (unsigned)n), dim3(256), 0, st, ref);
     return mq_check_launch("nvfp4 amax");
 }
 
-template <int PASS>
-static void launch_nvfp4_quant(const FlatTable& tab, int flags, float numer, dim3 grid, hipStream_t st) {
+template <int PASS, class Table>
+static void launch_nvfp4_quant(const Table& tab, int flags, float numer, dim3 grid, hipStream_t st) {
     const dim3 blk(kNvThreads);
-    switch ((flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0) {
-        case 0: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS>), grid, blk, 0, st, tab, numer); break;
-        case 1: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<1, PASS>), grid, blk, 0, st, tab, numer); break;
-        case 2: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<2, PASS>), grid, blk, 0, st, tab, numer); break;
-        case 3: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<3, PASS>), grid, blk, 0, st, tab, numer); break;
-        default: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<4, PASS>), grid, blk, 0, st, tab, numer); break;
+    // Four Over Six keeps to launches of kernel-argument tables (its five error modes are not built in the other form)
+    const int fos = (flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0;
+    if constexpr (std::is_same<Table, FlatRef>::value) {
+        hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table>), grid, blk, 0, st, tab, numer);
+    } else {
+        switch (fos) {
+            case 0: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+            case 1: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<1, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+            case 2: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<2, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+            case 3: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<3, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+            default: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<4, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+        }
     }
+}
+
+// fold + quantize (+ second pass) over a table whose grid is known: tab.chunk / tab.max_blocks are set
+template <class Table>
+static int nvfp4_quant_launch(const Table& tab, int n, int e4m3_max, int flags, int mode, hipStream_t st) {
+    const float numer = (float)e4m3_max * 6.0f;
+    const dim3 folds((unsigned)n), blk(256);
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)n);
+    if (mode == 2) {
+        if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
+        hipLaunchKernelGGL((nvfp4_fold_kernel<2, Table>), folds, blk, 0, st, tab, numer);
+        if (tab.max_blocks > 0) {
+            const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
+            launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)n), st);
+        }
+        return mq_check_launch("nvfp4 quant (carried-over amax)");
+    }
+    if (mode == 1) hipLaunchKernelGGL((nvfp4_fold_kernel<1, Table>), folds, blk, 0, st, tab, numer);
+    else hipLaunchKernelGGL((nvfp4_fold_kernel<0, Table>), folds, blk, 0, st, tab, numer);
+    if (tab.max_blocks > 0) launch_nvfp4_quant<0>(tab, flags, numer, grid, st);
+    return mq_check_launch("nvfp4 quant");
 }
 
 // tab.job[i]: w, q, s = block scales, aux = amax record, aux2 = fp32 global scale out (may be null), units = numel / 8.
@@ -543,23 +582,15 @@ static void launch_nvfp4_quant(const FlatTable& tab, int flags, float numer, dim
 // mode 2 (job driver, carried-over amax; the sections were cleared by the previous sync's fold): quantize with the
 //   record's old scales while collecting the new partial maxima, fold and compare, quantize again where they differ.
 int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st) {
-    const float numer = (float)e4m3_max * 6.0f;
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    const dim3 folds((unsigned)tab.n), blk(256);
-    const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n);
-    if (mode == 2) {
-        if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
-        hipLaunchKernelGGL(nvfp4_fold_kernel<2>, folds, blk, 0, st, tab, numer);
-        if (tab.max_blocks > 0) {
-            const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
-            launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)tab.n), st);
-        }
-        return mq_check_launch("nvfp4 quant (carried-over amax)");
-    }
-    if (mode == 1) hipLaunchKernelGGL(nvfp4_fold_kernel<1>, folds, blk, 0, st, tab, numer);
-    else hipLaunchKernelGGL(nvfp4_fold_kernel<0>, folds, blk, 0, st, tab, numer);
-    if (tab.max_blocks > 0) launch_nvfp4_quant<0>(tab, flags, numer, grid, st);
-    return mq_check_launch("nvfp4 quant");
+    return nvfp4_quant_launch(tab, tab.n, e4m3_max, flags, mode, st);
+}
+// modes 1 and 2 over n descriptors of a device table (standard block scaling only); max_units: the largest tensor's units
+int mq_nvfp4_quant_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode, hipStream_t st) {
+    FlatRef ref{device_jobs, 0, 0};
+    if (!flat_grid(ref, max_units, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (n == 0) return MQ_OK;
+    return nvfp4_quant_launch(ref, n, e4m3_max, 0, mode, st);
 }
 
 extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream) {
@@ -598,7 +629,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
     FlatTable fold{};
     fold.n = 1;
     fold.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), 0, global_scale, n_sections, 0};
-    hipLaunchKernelGGL(nvfp4_fold_kernel<0>, dim3(1), dim3(256), 0, st, fold, numer);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, st, fold, numer);
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
@@ -613,7 +644,7 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
     FlatTable tab{};
     tab.n = 1;
     tab.job[0] = FlatJob{nullptr, nullptr, nullptr, record, 0, nullptr, n_sections, 0};
-    hipLaunchKernelGGL(nvfp4_fold_kernel<0>, dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
     return mq_check_launch("nvfp4 fold");
 }
 

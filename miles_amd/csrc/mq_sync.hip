@@ -33,6 +33,9 @@ bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
 int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
+int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st);
+int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st);
+int mq_nvfp4_quant_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode, hipStream_t st);
 int mq_mxfp8_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
@@ -145,7 +148,16 @@ static bool tile_kind(int kind) {
 }
 static bool table_kind(int kind) {
     return kind == MQ_JOB_MXFP8 || kind == MQ_JOB_MXFP4 || kind == MQ_JOB_INT4_PACK || kind == MQ_JOB_INT4_PACK_ASYM ||
-           tile_kind(kind);
+           kind == MQ_JOB_FP8_TENSOR || kind == MQ_JOB_NVFP4 || tile_kind(kind);
+}
+// NVFP4 jobs that share an amax record are neighbours in the list: the place of job t among them, and how many they are
+static void nvfp4_sections(const mq_job* jobs, int64_t n, int64_t t, int& section, int& sections) {
+    section = 0;
+    for (int64_t b = t; b > 0 && section < 2 * MQ_NVFP4_SECTIONS && jobs[b - 1].kind == MQ_JOB_NVFP4 && jobs[b - 1].aux == jobs[t].aux; b--)
+        section++;
+    sections = section + 1;
+    for (int64_t f = t + 1; f < n && sections < 2 * MQ_NVFP4_SECTIONS && jobs[f].kind == MQ_JOB_NVFP4 && jobs[f].aux == jobs[t].aux; f++)
+        sections++;
 }
 static TileJob tile_entry(const mq_job& jb) {
     return TileJob{jb.in, jb.out, (float*)jb.scale, (int32_t)jb.ld, (int32_t)jb.rows, (int32_t)jb.cols,
@@ -155,6 +167,8 @@ static int64_t tiles_of(const mq_job& jb) { return ((jb.rows + 127) / 128) * ((j
 static FlatJob flat_entry(const mq_job& jb) {
     if (jb.kind == MQ_JOB_INT4_PACK_ASYM)       // zero points, packed zero points, groups per row
         return FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, jb.p0 > 0 ? (int32_t)(jb.cols / jb.p0) : 0, 0};
+    if (jb.kind == MQ_JOB_FP8_TENSOR)           // amax record, one section
+        return FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, nullptr, 0, 1};
     return FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8, nullptr, 0, 0};
 }
 
@@ -185,24 +199,32 @@ static bool copy_depends_on_group(const mq_job* jobs, int64_t first, int64_t can
 }
 
 // per-tensor FP8 run [i, j): chunks of up to kMaxGroup tensors of similar size with the same floor and flags
-static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
+// (`table`: the device descriptors of jobs[0..), or null)
+static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, const FlatJob* table, void* stream) {
+    const int64_t cap = table ? kTableGroup : kMaxGroup;
     while (i < j) {
-        FlatTable tab{};
         int64_t k = i, sum = 0, mx = 0;
-        while (k < j && k - i < kMaxGroup && jobs[k].p0 == jobs[i].p0 && jobs[k].p1 == jobs[i].p1) {
+        while (k < j && k - i < cap && jobs[k].p0 == jobs[i].p0 && jobs[k].p1 == jobs[i].p1) {
             const int64_t e = jobs[k].rows * jobs[k].cols;
             const int64_t nmx = e > mx ? e : mx;
             if (k > i && nmx * (k - i + 1) * 4 > (sum + e) * 5) break;       // padding of the 2-D grid under 25 %
-            tab.job[k - i] = FlatJob{jobs[k].in, jobs[k].out, jobs[k].scale, jobs[k].aux, e / 8, nullptr, 0, 1};
             sum += e;
             mx = nmx;
             k++;
         }
-        tab.n = (int)(k - i);
         const uint32_t floor_bits = (uint32_t)jobs[i].p0;
         float floor_v;
         memcpy(&floor_v, &floor_bits, 4);
-        int rc = mq_fp8_tensor_launch_group(tab, floor_v, (jobs[i].p1 & MQ_NVFP4_CARRY_AMAX) != 0, (hipStream_t)stream);
+        const bool carry = (jobs[i].p1 & MQ_NVFP4_CARRY_AMAX) != 0;
+        int rc;
+        if (k - i > kMaxGroup) {
+            rc = mq_fp8_tensor_launch_table(table + i, (int)(k - i), mx / 8, floor_v, carry, (hipStream_t)stream);
+        } else {
+            FlatTable tab{};
+            tab.n = (int)(k - i);
+            for (int64_t t = i; t < k; t++) tab.job[t - i] = flat_entry(jobs[t]);
+            rc = mq_fp8_tensor_launch_group(tab, floor_v, carry, (hipStream_t)stream);
+        }
         if (rc) return rc;
         i = k;
     }
@@ -210,42 +232,74 @@ static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, void* stream
 }
 
 // NVFP4 run [i, j): all jobs fast or not, processed as amax-phase then quantize-phase per chunk
-static int run_nvfp4(const mq_job* jobs, int64_t i, int64_t j, void* stream) {
+// (`table`: the device descriptors of jobs[0..), or null; n_all: length of the whole list, for the section lookup)
+static int run_nvfp4(const mq_job* jobs, int64_t n_all, int64_t i, int64_t j, const FlatJob* table, void* stream) {
     hipStream_t st = (hipStream_t)stream;
     while (i < j) {
         // a chunk ends at the group / byte limit, but never between two jobs that share an amax word
-        int64_t k = i, bytes = 0, mx = 0;
-        while (k < j) {
-            const bool tied = k > i && jobs[k].aux == jobs[k - 1].aux;
-            const int64_t b = jobs[k].rows * jobs[k].cols * (jobs[k].dtype == MQ_F32 ? 4 : 2);
-            const int64_t nmx = b > mx ? b : mx;
-            const bool ragged = nmx * (k - i + 1) * 4 > (bytes + b) * 5;
-            if (!tied && k > i &&
-                (k - i >= kMaxGroup - 1 || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 || jobs[k].p1 != jobs[i].p1 || ragged))
-                break;
-            mx = nmx;
-            if (k - i >= kMaxGroup) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
-            bytes += b;
-            k++;
+        auto form = [&](int64_t cap) {
+            int64_t k = i, bytes = 0, mx = 0;
+            while (k < j) {
+                int64_t r = k + 1;                               // the jobs of one record: k .. r-1
+                while (r < j && jobs[r].aux == jobs[k].aux) r++;
+                int64_t b = 0, nmx = mx;
+                for (int64_t t = k; t < r; t++) {
+                    const int64_t bt = jobs[t].rows * jobs[t].cols * (jobs[t].dtype == MQ_F32 ? 4 : 2);
+                    b += bt;
+                    nmx = bt > nmx ? bt : nmx;
+                }
+                const bool ragged = nmx * (r - i) * 4 > (bytes + b) * 5;
+                if (k > i && (r - i > cap || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 ||
+                              jobs[k].p1 != jobs[i].p1 || ragged))
+                    break;
+                mx = nmx;
+                bytes += b;
+                k = r;
+            }
+            return k;
+        };
+        auto all_fast_in = [&](int64_t k) {
+            for (int64_t t = i; t < k; t++)
+                if (!job_fast(jobs[t])) return false;
+            return true;
+        };
+        // a device table lifts the limit for standard block scaling when every job takes the packed kernels
+        const bool standard = (jobs[i].p1 & (MQ_NVFP4_4OVER6 | MQ_NVFP4_ERR_MSE | MQ_NVFP4_ERR_FP16)) == 0;
+        int64_t k = form(table && standard ? kTableGroup : kMaxGroup);
+        bool all_fast = all_fast_in(k);
+        if (k - i > kMaxGroup && !all_fast) {
+            k = form(kMaxGroup);
+            all_fast = all_fast_in(k);
         }
         const int n = (int)(k - i);
-        // section of each job inside its record, and how many sections the record ends up with
-        int section[kMaxGroup], sections[kMaxGroup];
-        for (int t = 0; t < n; t++) section[t] = (t > 0 && jobs[i + t].aux == jobs[i + t - 1].aux) ? section[t - 1] + 1 : 0;
-        for (int t = n - 1; t >= 0; t--)
-            sections[t] = (t + 1 < n && jobs[i + t + 1].aux == jobs[i + t].aux) ? sections[t + 1] : section[t] + 1;
-        for (int t = 0; t < n; t++)
-            if (section[t] >= MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
-        bool all_fast = true;
-        for (int t = 0; t < n; t++) all_fast &= job_fast(jobs[i + t]);
+        const bool from_table = table && standard && all_fast && n > kMaxGroup;
+        if (n > kMaxGroup && !from_table) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
+        std::vector<int> section(n), sections(n);
+        for (int t = 0; t < n; t++) {
+            nvfp4_sections(jobs, n_all, i + t, section[t], sections[t]);
+            if (sections[t] > MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "too many NVFP4 jobs share one amax record");
+        }
         if (all_fast) {
             // MQ_NVFP4_CARRY_AMAX (set by a caller that replays this very list, records included, after a first plain
             // run): one pass with last sync's amax instead of the amax pass; every job of the chunk must ask for it
             bool carry = true;
             for (int t = 0; t < n; t++) carry &= (jobs[i + t].p1 & MQ_NVFP4_CARRY_AMAX) != 0;
+            int rc = MQ_OK;
+            if (from_table) {
+                int64_t max_units = 0;
+                for (int t = 0; t < n; t++) {
+                    const int64_t u = jobs[i + t].rows * jobs[i + t].cols / 8;
+                    max_units = u > max_units ? u : max_units;
+                }
+                if (!carry) rc = mq_nvfp4_amax_launch_table(table + i, n, st);
+                if (rc) return rc;
+                rc = mq_nvfp4_quant_launch_table(table + i, n, max_units, jobs[i].p0, carry ? 2 : 1, st);
+                if (rc) return rc;
+                i = k;
+                continue;
+            }
             FlatTable tab{};
             tab.n = n;
-            int rc = MQ_OK;
             if (!carry) {
                 for (int t = 0; t < n; t++) {
                     const mq_job& jb = jobs[i + t];
@@ -287,6 +341,12 @@ extern "C" int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table
             TileJob e = tile_entry(jobs[i]);
             mq_fp8_tile_job_finish(e);
             memcpy(slot, &e, sizeof(e));
+        } else if (jobs[i].kind == MQ_JOB_NVFP4) {
+            const mq_job& jb = jobs[i];
+            int section, sections;
+            nvfp4_sections(jobs, n, i, section, sections);
+            const FlatJob e{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, section, sections};
+            memcpy(slot, &e, sizeof(e));
         } else {
             const FlatJob e = table_kind(jobs[i].kind) && !tile_kind(jobs[i].kind) ? flat_entry(jobs[i]) : FlatJob{};
             memcpy(slot, &e, sizeof(e));
@@ -312,7 +372,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
         if (head.kind == MQ_JOB_NVFP4 || head.kind == MQ_JOB_FP8_TENSOR) {
             int64_t j = i + 1;
             while (j < n && jobs[j].kind == head.kind) j++;
-            int rc = head.kind == MQ_JOB_NVFP4 ? run_nvfp4(jobs, i, j, stream) : run_fp8_tensor(jobs, i, j, stream);
+            int rc = head.kind == MQ_JOB_NVFP4 ? run_nvfp4(jobs, n, i, j, table, stream) : run_fp8_tensor(jobs, i, j, table, stream);
             if (rc) return rc;
             i = j;
             continue;

@@ -99,7 +99,7 @@ class JobBatch:
 
     # job kinds whose grouped launches can take their descriptors from a device table (mq_run_jobs_tabled)
     _TABLE_KINDS = (_lib.JOB_MXFP8, _lib.JOB_MXFP4, _lib.JOB_INT4_PACK, _lib.JOB_INT4_PACK_ASYM, _lib.JOB_FP8_BLOCK,
-                    _lib.JOB_FP8_BLOCKWISE_CAST, _lib.JOB_FP8_BLOCK_POW2)
+                    _lib.JOB_FP8_BLOCKWISE_CAST, _lib.JOB_FP8_BLOCK_POW2, _lib.JOB_NVFP4, _lib.JOB_FP8_TENSOR)
 
     def freeze(self):
         """Materialise the ctypes job array (done once; `run` can then be repeated).  A list with more jobs of a

@@ -1207,3 +1207,62 @@ def test_stream_probes_run_and_refuse_bad_arguments():
     for shape, param, size in ((0, 3, nbytes), (2, 100, nbytes), (3, 100, nbytes), (9, 1, nbytes), (0, 2, nbytes + 8), (3, 1 << 30, nbytes)):
         assert lib.mq_stream_probe(shape, src.data_ptr(), dst.data_ptr(), size, param, stream) != 0, (shape, param, size)
     assert lib.mq_stream_probe(0, None, dst.data_ptr(), nbytes, 2, stream) != 0
+
+
+@pytest.mark.parametrize("fmt", ["nvfp4", "tensor_fp8"])
+def test_amax_quantizers_over_a_device_table_first_run_carried_and_moved(oracle, fmt):
+    """NVFP4 (pairs sharing a record and single tensors) and per-tensor FP8 with more jobs than one launch's kernel
+    arguments hold: the amax pass, the fold and the quantizer read their descriptors from the device table; then the
+    carried-over form on unchanged weights, and after some amaxes moved."""
+    from miles_amd import launch
+    from miles_amd.tools.convert_hf_to_fp8 import tensor_fp8
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    g = torch.Generator().manual_seed(91)
+    shapes = [(int(torch.randint(52, 64, (1,), generator=g)), 256) for _ in range(120)]
+    shapes[60] = (300, 256)                       # far outside the band of the others: cuts the group
+    cpu = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=9100 + i) for i, s in enumerate(shapes)]
+    pairs_cpu = [[W.gaussian_outliers((56, 256), std=0.02, p_outlier=0.001, gain=20.0, seed=9500 + 2 * i + h) for h in range(2)]
+                 for i in range(30)]
+    dev = [w.to(DEV) for w in cpu]
+    pairs_dev = [[w.to(DEV) for w in p] for p in pairs_cpu]
+    with launch.recording() as batch:
+        if fmt == "nvfp4":
+            outs, pair_outs = [], []
+            for i, w in enumerate(dev):
+                outs.append(nvfp4_quantize_1d(w))
+                if i % 4 == 0:
+                    pair_outs.append(nvfp4_quantize_1d_pair(*pairs_dev[i // 4]))
+        else:
+            outs, pair_outs = [tensor_fp8(w) for w in dev], []
+    batch.freeze()
+    assert batch._table is not None and len(batch) > _lib.MAX_GROUP
+
+    def check(what):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, (w, got) in enumerate(zip(dev, outs)):
+            want = oracle.nvfp4_quantize_1d(w.cpu()) if fmt == "nvfp4" else oracle.tensor_fp8(w.cpu())
+            for k, (g_, w_) in enumerate(zip(got, want)):
+                _same(g_, w_, f"{what}: tensor {i} output {k}")
+        for i, got in enumerate(pair_outs):
+            want = oracle.nvfp4_quantize_1d_pair(pairs_dev[i][0].cpu(), pairs_dev[i][1].cpu())
+            for half in range(2):
+                for k, (g_, w_) in enumerate(zip(got[half], want[half])):
+                    _same(g_, w_, f"{what}: pair {i} half {half} output {k}")
+
+    check("first run")
+    assert batch.carry_amax() == len(batch)
+    batch.freeze()
+    assert batch._table is not None
+    check("carried, unchanged weights")
+    for i in (3, 50, 119):
+        dev[i].mul_(3.0)
+    if pair_outs:
+        pairs_dev[7][1].mul_(0.25)
+        pairs_dev[20][0].mul_(4.0)
+    check("some amaxes moved")
+    check("and stayed (the marked records take two passes once more)")
+    check("settled")
+    redo = torch.stack([r[_lib.RECORD_REDO_WORD] for r in batch.amax_records()]).cpu()
+    assert int(redo.sum()) == 0
