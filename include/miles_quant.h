@@ -296,6 +296,13 @@ int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, 
  * its first operand in the low nibble.  The kernels rely on [0], [2], [3], [4], [7] being zero. */
 int mq_selftest_convert(uint64_t* counts, void* stream);
 
+/* Reciprocal self-test (no counterpart in the reference).  The INT4 packers divide a group's elements by its scale
+ * through y = 1/scale, taken from the hardware reciprocal and one Newton step instead of an IEEE division; the codes are
+ * only right if y is the correctly rounded reciprocal.  count: one uint64 on the device (cleared by the call) = divisors
+ * of both signs in [2^-91, 2^90], the range in which the kernels use y, for which it differs from 1.0f / scale.
+ * The kernels rely on it being zero. */
+int mq_selftest_reciprocal(uint64_t* count, void* stream);
+
 /* Plain 16-byte-per-lane copy used to calibrate achievable HBM bandwidth and rocprof counters. */
 int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
 

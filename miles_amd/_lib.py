@@ -47,6 +47,7 @@ SIGNATURES = {
     "mq_job_table_fill": [_vp, _i64, _vp],
     "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
     "mq_selftest_convert": [_vp, _vp],
+    "mq_selftest_reciprocal": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],
     "mq_stream_probe": [_i32, _vp, _vp, _i64, _i64, _vp],
 }

@@ -94,6 +94,15 @@ __device__ __forceinline__ float div_by_shared(float w, float s, float y) {
     float e = __builtin_fmaf(q0, s, -w);
     return __builtin_fmaf(-e, y, q0);
 }
+// y = RN(1/s) for div_by_shared: the hardware reciprocal (within one ulp) and one Newton step, three instructions where
+// the IEEE division 1.0f / s takes eleven.  On gfx950 the result equals that division for every divisor in the range
+// of shared_div_ok (mq_selftest_reciprocal compares them over the whole range on the device); outside that range the
+// callers do not use y.
+__device__ __forceinline__ float recip_shared(float s) {
+    const float r = __builtin_amdgcn_rcpf(s);
+    const float e = __builtin_fmaf(-s, r, 1.0f);
+    return __builtin_fmaf(e, r, r);
+}
 // divisor range in which div_by_shared is used; outside it kernels fall back to operator/
 __device__ __forceinline__ bool shared_div_ok(float s) {
     uint32_t a = f2u(s) & 0x7FFFFFFFu;

@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
         top = umax(top, mb);
         const float amax = u2f(mb << 16);
         const float s = __builtin_fmaxf(amax * kSymCons, 1e-5f);
-        const float y = 1.0f / s;
+        const float y = recip_shared(s);
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         const bool fast = shared_div_ok(s);
@@ -313,9 +313,10 @@ __global__ __launch_bounds__(256) void int4_pack_asym_kernel(const void* __restr
     }
 }
 
-// bf16 fast path of the asymmetric packer: LANES lanes own one group (16 bytes each, G = 8 * LANES), the data
-// stays in registers between the min/max pass and the coding pass, min and max travel through the unsigned
-// DPP reduction as order-preserving integer keys, and every rounding to bf16 is the packed hardware conversion.
+// bf16 fast path of the asymmetric packer: LANES lanes own one group (16 bytes each, G = 8 * LANES) and the data
+// stays in registers between the min/max pass and the coding pass.  In the written-out chain min and max travel
+// through the unsigned DPP reduction as order-preserving integer keys, and every rounding to bf16 is the packed
+// hardware conversion.
 __device__ __forceinline__ uint32_t order_key(float f) {
     const uint32_t u = f2u(f);
     return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
@@ -328,7 +329,9 @@ __device__ __forceinline__ void rd_bf16x2(float& a, float& b) {
     a = bf16_lo(p);
     b = bf16_hi(p);
 }
-// one 16-byte unit of one lane; LANES neighbouring lanes hold the rest of the group
+// One 16-byte unit of one lane, LANES neighbouring lanes hold the rest of the group: the chain as written, with IEEE
+// divisions.  The packed kernel sends here the wavefronts that met a group outside its fused form (minimum above zero
+// or far below it, huge scales, infinities, NaN).
 template <int LANES>
 __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, const int64_t unit, const int t,
                                                uint32_t* __restrict__ packed, uint16_t* __restrict__ scale_out,
@@ -343,55 +346,32 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
     mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
     const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
     const float sb = u2f(sw_bf16(s) << 16);
-    const float ys = 1.0f / s;
-    const float big = __builtin_fmaxf(__builtin_fabsf(mx), __builtin_fabsf(mn));
-    const bool fast = shared_div_ok(s) && big * ys < 1e30f;
-    const float lo = __builtin_rintf(fast ? div_by_shared(mn, s, ys) : mn / s);
-    const float hi = __builtin_rintf(fast ? div_by_shared(mx, s, ys) : mx / s);
-    const float z = __builtin_fminf(__builtin_fmaxf(-lo, 0.0f), 15.0f) + 0.0f;
+    const float z = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
     uint32_t word = 0;
-    if (fast && lo <= 0.0f && lo >= -15.0f && hi - lo <= 16.0f && sb <= 1e37f) {
-        // The zero point was not clamped, so rint(x/s) + z is an integer in [0, 16].  For such codes and every
-        // bf16 scale up to 1e37 the reference's dequantize / requantize round trip in bf16 returns the code itself
-        // (checked exhaustively on the CPU: all scales x all codes x all zero points), so the codes are final.
-        // rint through one add of 1.5 * 2^23: the low bits of the sum's pattern are the (signed) integer.  The zero point
-        // is added as an integer afterwards (inside the float add an odd zero point would turn the ties around);
-        // everything is arithmetic modulo 2^32, like the reference's int32 sum.
-        constexpr uint32_t kMagicBits = 0x4B400000u;
-        uint32_t magic_sum = 0;
+    float q[8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            word += f2u(div_by_shared(f[i], s, ys) + 12582912.0f) << (4 * i);
-            magic_sum += kMagicBits << (4 * i);
-        }
-        word = word - magic_sum + (uint32_t)z * 0x11111111u;
-    } else {
-        // the chain as written, IEEE divisions: groups whose minimum lies above zero or far below it, huge scales
-        float q[8];
+    for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s) + z;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s) + z;
+    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i++) q[i] = q[i] - z;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = q[i] - z;
+    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i++) q[i] = q[i] * sb;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = q[i] * sb;
+    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i++) q[i] = q[i] / sb;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = q[i] / sb;
+    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i++) q[i] = q[i] + z;
 #pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = q[i] + z;
+    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
-#pragma unroll
-        for (int i = 0; i < 8; i++)
-            word += (uint32_t)__builtin_rintf(clamp_keep_nan(q[i], 0.0f, 255.0f)) << (4 * i);
-    }
+    for (int i = 0; i < 8; i++)
+        word += (uint32_t)__builtin_rintf(clamp_keep_nan(q[i], 0.0f, 255.0f)) << (4 * i);
     if (live) {
         st4(packed + unit, word);
         if ((t & (LANES - 1)) == 0) {
@@ -400,8 +380,40 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
         }
     }
 }
+// Max of `mx` and min of `mn` over aligned groups of LANES lanes, for floats that are not NaN.  Written as instructions:
+// through the builtins every step costs a move, a quieting of the moved value and the max itself.  A DPP operand must
+// have been written two issue slots earlier (whatever the compiler put in front of the block included), so the block
+// opens with two idle slots and the two chains alternate with one idle slot per step.
+#define MQ_EXTREMA_STEP(ctrl)                                                \
+    "v_max_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t"        \
+    "v_min_f32_dpp %1, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
+template <int LANES>
+__device__ __forceinline__ void seg_extrema(float& mx, float& mn) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16, "group of 32, 64 or 128 elements");
+    if (LANES == 4)
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+                     : "+v"(mx), "+v"(mn));
+    else if (LANES == 8)
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+                     "s_nop 0\n\t" MQ_EXTREMA_STEP("row_half_mirror")
+                     : "+v"(mx), "+v"(mn));
+    else
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+                     "s_nop 0\n\t" MQ_EXTREMA_STEP("row_half_mirror") "s_nop 0\n\t" MQ_EXTREMA_STEP("row_mirror")
+                     : "+v"(mx), "+v"(mn));
+}
+#undef MQ_EXTREMA_STEP
 // job: w, q = packed codes, s = scales, aux = zero points (one byte per group, read again by the zero-point packer),
 // aux2 = packed zero points, units, section = groups per row
+//
+// Every group first runs the fused form as one straight instruction stream: scale and zero point from the group's
+// extrema, codes = rint(x / s) + z through the shared-divisor sequence.  The form is final when the scale is in the
+// range of that sequence, the zero point was not clamped (lo = rint(min / s) in [-15, 0]) and bf16(s) <= 1e37: then
+// every rint(x / s) + z is an integer in [0, 16] -- (max - min) / s <= 15 (1 + 2^-22) because s >= RN(RN(max - min) / 15),
+// and two roundings to integer lie at most one further apart than their arguments -- and for such codes the reference's
+// dequantize / requantize round trip in bf16 returns the code itself (checked exhaustively on the CPU: all scales x
+// all codes x all zero points).  A wavefront that met any other group (minimum above zero or far below it, huge or
+// non-finite values) writes its groups again through int4_asym_unit, the chain as written; the later store wins.
 template <int LANES, class Table>
 __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const Table tab) {
     const FlatJob& job = flat_job(tab);
@@ -421,6 +433,53 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
         const int64_t unit = base + i * kI4Threads;
         v[i] = ld16(w + (unit < total_units ? unit : total_units - 1) * 8);
     }
+    bool odd = false;
+    uint32_t word[kI4Unroll], sb[kI4Unroll], z[kI4Unroll];
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
+                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        float mx = f[0], mn = f[0];
+#pragma unroll
+        for (int j = 1; j < 8; j++) { mx = __builtin_fmaxf(mx, f[j]); mn = __builtin_fminf(mn, f[j]); }
+        // a NaN element is skipped by the extrema but is not coded like a number: its wavefront takes the chain below,
+        // whatever the fused form makes of the group (fcmp unordered takes two elements at a time)
+        const bool nan = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]) | (f[4] != f[4]) |
+                         (f[5] != f[5]) | (f[6] != f[6]) | (f[7] != f[7]);
+        seg_extrema<LANES>(mx, mn);
+        const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
+        const float ys = recip_shared(s);
+        sb[i] = hw_bf16x2(s, 0.0f);
+        // The zero point unclamped: lo = rint(min / s) in [-15, 0].  Every quotient of the group then lies within +-16,
+        // far from the range limits of the shared-divisor sequence, and bf16(s) <= 2^90 (1 + 2^-8) is far below 1e37.
+        // One infinite extremum makes s infinite, which shared_div_ok refuses; a group of equal infinities has the
+        // floor scale and lo = NaN, which fails both comparisons.
+        const float lo = __builtin_rintf(div_by_shared(mn, s, ys));
+        z[i] = (uint32_t)(int)(0.0f - lo);
+        odd |= !shared_div_ok(s) | !(lo <= 0.0f) | !(lo >= -15.0f) | nan;
+        // rint through one add of 1.5 * 2^23: the low bits of the sum's pattern are the (signed) integer.  The zero point
+        // is added as an integer afterwards (inside the float add an odd zero point would turn the ties around);
+        // everything is arithmetic modulo 2^32, like the reference's int32 sum.
+        constexpr uint32_t kMagicSum = 0x4B400000u + (0x4B400000u << 4) + (0x4B400000u << 8);     // further shifts: 0
+        uint32_t sum = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) sum += f2u(div_by_shared(f[j], s, ys) + 12582912.0f) << (4 * j);
+        word[i] = sum - kMagicSum + z[i] * 0x11111111u;
+    }
+    // all stores after all loads have been used: a store between them would have to complete before the next unit's
+    // data counts as arrived (loads and stores return in order)
+#pragma unroll
+    for (int i = 0; i < kI4Unroll; i++) {
+        const int64_t unit = base + i * kI4Threads;
+        if (unit < total_units) {
+            st4(packed + unit, word[i]);
+            if ((t & (LANES - 1)) == 0) {
+                scale_out[unit / LANES] = (uint16_t)sb[i];
+                zero_out[unit / LANES] = (uint8_t)z[i];
+            }
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64(odd) == 0) return;
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
         const int64_t unit = base + i * kI4Threads;
@@ -429,34 +488,62 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
 }
 
 // packed_zp[g, j] = sum_i zero[8j+i, g] << 4*order[i], order = {0,4,1,5,2,6,3,7}   (py:249-254)
-__device__ __forceinline__ void int4_zero_pack(const uint8_t* __restrict__ zero, uint32_t* __restrict__ packed_zp,
-                                               const int64_t rows8, const int64_t groups_per_row) {
-    const int64_t total = groups_per_row * rows8;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int64_t g = i / rows8, j = i - g * rows8;
+// `zero` is [rows, groups_per_row] bytes and the packed words are its transpose, eight rows to a word.  A workgroup
+// takes a tile of 256 rows x 64 groups through LDS: the bytes are read along the rows (neighbouring lanes, neighbouring
+// bytes) and the words written along j (32 consecutive words of one group per half wavefront).
+constexpr int kZpRows = 256, kZpCols = 64, kZpPitch = kZpCols + 2;
+__host__ __device__ __forceinline__ int64_t int4_zero_tiles(int64_t rows8, int64_t groups_per_row) {
+    return ((rows8 * 8 + kZpRows - 1) / kZpRows) * ((groups_per_row + kZpCols - 1) / kZpCols);
+}
+__device__ __forceinline__ void int4_zero_pack_tile(const uint8_t* __restrict__ zero, uint32_t* __restrict__ packed_zp,
+                                                    const int64_t rows8, const int64_t groups_per_row, const int64_t tile,
+                                                    uint8_t* lds) {
+    const int64_t col_tiles = (groups_per_row + kZpCols - 1) / kZpCols;
+    const int64_t row0 = (tile / col_tiles) * kZpRows, g0 = (tile % col_tiles) * kZpCols;
+    const int64_t rows = rows8 * 8;
+    const int t = threadIdx.x;
+    {
+        const int c = t & (kZpCols - 1);
+        const bool col_live = g0 + c < groups_per_row;
+#pragma unroll 8
+        for (int r = t / kZpCols; r < kZpRows; r += 256 / kZpCols) {
+            const bool live = col_live && row0 + r < rows;
+            lds[r * kZpPitch + c] = live ? zero[(row0 + r) * groups_per_row + g0 + c] : (uint8_t)0;
+        }
+    }
+    __syncthreads();
+    const int j = t & (kZpRows / 8 - 1);
+    const int64_t jj = row0 / 8 + j;
+    if (jj >= rows8) return;
+#pragma unroll
+    for (int g = t / (kZpRows / 8); g < kZpCols; g += 256 / (kZpRows / 8)) {
+        if (g0 + g >= groups_per_row) break;
         uint32_t word = 0;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const int nib = (k >> 1) + 4 * (k & 1);
-            word += (uint32_t)zero[(j * 8 + k) * groups_per_row + g] << (4 * nib);
+            word += (uint32_t)lds[(j * 8 + k) * kZpPitch + g] << (4 * nib);
         }
-        packed_zp[i] = word;
+        packed_zp[(g0 + g) * rows8 + jj] = word;
     }
 }
 __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
                                                              uint32_t* __restrict__ packed_zp, int64_t M,
                                                              int64_t groups_per_row) {
-    int4_zero_pack(zero, packed_zp, M / 8, groups_per_row);
+    __shared__ uint8_t lds[kZpRows * kZpPitch];
+    int4_zero_pack_tile(zero, packed_zp, M / 8, groups_per_row, blockIdx.x, lds);
 }
 // the zero points of a group of tensors (descriptors as for int4_pack_asym_bf16_kernel): blockIdx.y selects the tensor;
 // a tensor of `units` 16-byte units has units / units_per_group groups, groups_per_row of them in each row
 template <class Table>
 __global__ __launch_bounds__(256) void int4_zero_pack_group_kernel(const Table tab, int units_per_group) {
+    __shared__ uint8_t lds[kZpRows * kZpPitch];
     const FlatJob& job = flat_job(tab);
     const int64_t groups_per_row = job.section;
     if (groups_per_row <= 0) return;
-    int4_zero_pack((const uint8_t*)job.aux, (uint32_t*)job.aux2, job.units / units_per_group / groups_per_row / 8, groups_per_row);
+    const int64_t rows8 = job.units / units_per_group / groups_per_row / 8;
+    if (blockIdx.x >= int4_zero_tiles(rows8, groups_per_row)) return;
+    int4_zero_pack_tile((const uint8_t*)job.aux, (uint32_t*)job.aux2, rows8, groups_per_row, blockIdx.x, lds);
 }
 
 // ---- fake INT4 quantization of row blocks (1, G), G = 32 / 64 / 128 ------------------------------------------------
@@ -671,35 +758,42 @@ bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M) {
     return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32) && M % 8 == 0;
 }
 
+// tiles of the zero-point packer for a [rows, cols] tensor with groups of `group` elements
+int64_t mq_int4_zero_tiles(int64_t rows, int64_t cols, int group) { return int4_zero_tiles(rows / 8, cols / group); }
+
 // The two launches of an asymmetric pack for a group of tensors: codes + scales + zero points, then the zero points
-// packed eight rows to a word.  max_units: the largest tensor's 16-byte units.
+// packed eight rows to a word.  max_tiles: the most tiles the second launch has to cover in one tensor.
 template <class Table>
-static int int4_pack_asym_launch(const Table& tab, int n, int64_t max_units, int group, hipStream_t st) {
+static int int4_pack_asym_launch(const Table& tab, int n, int64_t max_tiles, int group, hipStream_t st) {
     const dim3 grid((unsigned)tab.max_blocks, (unsigned)n), blk(kI4Threads);
     if (group == 128) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<16, Table>), grid, blk, 0, st, tab);
     else if (group == 64) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<8, Table>), grid, blk, 0, st, tab);
     else hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<4, Table>), grid, blk, 0, st, tab);
     int rc = mq_check_launch("int4 asymmetric pack");
     if (rc != MQ_OK) return rc;
-    const int64_t zp_words = max_units / group;             // (K / group) * (M / 8) words per tensor
-    int64_t zblocks = (zp_words + 255) / 256;
-    if (zblocks > mq_grid_cap()) zblocks = mq_grid_cap();
-    if (zblocks < 1) zblocks = 1;
-    hipLaunchKernelGGL(int4_zero_pack_group_kernel<Table>, dim3((unsigned)zblocks, (unsigned)n), dim3(256), 0, st, tab, group / 8);
+    hipLaunchKernelGGL(int4_zero_pack_group_kernel<Table>, dim3((unsigned)max_tiles, (unsigned)n), dim3(256), 0, st, tab, group / 8);
     return mq_check_launch("int4 zero-point pack");
 }
 int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st) {
     if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    int64_t max_units = 0;
-    for (int i = 0; i < tab.n; i++) max_units = tab.job[i].units > max_units ? tab.job[i].units : max_units;
-    return int4_pack_asym_launch(tab, tab.n, max_units, group, st);
+    int64_t max_tiles = 1;
+    for (int i = 0; i < tab.n; i++) {
+        const int64_t gpr = tab.job[i].section;
+        if (gpr <= 0) continue;
+        const int64_t tiles = int4_zero_tiles(tab.job[i].units / (group / 8) / gpr / 8, gpr);
+        max_tiles = tiles > max_tiles ? tiles : max_tiles;
+    }
+    if (max_tiles >= 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    return int4_pack_asym_launch(tab, tab.n, max_tiles, group, st);
 }
-int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st) {
+// max_units: the largest tensor's 16-byte units; max_zero_tiles: the largest mq_int4_zero_tiles of the tensors
+int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int64_t max_zero_tiles, int group,
+                                   hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
-    if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll) || max_zero_tiles >= 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (ref.max_blocks == 0 || n == 0) return MQ_OK;
-    return int4_pack_asym_launch(ref, n, max_units, group, st);
+    return int4_pack_asym_launch(ref, n, max_zero_tiles < 1 ? 1 : max_zero_tiles, group, st);
 }
 
 extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
@@ -728,9 +822,8 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_F32>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     int rc = mq_check_launch("int4 asymmetric pack");
     if (rc != MQ_OK) return rc;
-    const int64_t zp_words = gpr * (M / 8);
-    int64_t zblocks = (zp_words + 255) / 256;
-    if (zblocks > mq_grid_cap()) zblocks = mq_grid_cap();
+    const int64_t zblocks = int4_zero_tiles(M / 8, gpr);
+    if (zblocks >= 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
     hipLaunchKernelGGL(int4_zero_pack_kernel, dim3((unsigned)zblocks), dim3(256), 0, st, zero, (uint32_t*)packed_zp, M, gpr);
     return mq_check_launch("int4 zero-point pack");
 }

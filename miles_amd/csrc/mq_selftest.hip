@@ -54,7 +54,28 @@ __global__ __launch_bounds__(256) void selftest_kernel(uint64_t* counts) {
     }
 }
 
+// every divisor in the range of the shared-divisor sequence: refined hardware reciprocal against the IEEE division
+__global__ __launch_bounds__(256) void selftest_reciprocal_kernel(uint64_t* count) {
+    const uint32_t tid = blockIdx.x * blockDim.x + threadIdx.x;   // 2^20 lanes
+    for (uint32_t it = 0; it < 4096; it++) {
+        const uint32_t bits = it * (1u << 20) + tid;
+        const float s = u2f(bits);
+        float want = 1.0f / s;
+        asm volatile("" : "+v"(want));
+        tally(count, 0, shared_div_ok(s) && f2u(recip_shared(s)) != f2u(want));
+    }
+}
+
 }  // namespace mq
+
+extern "C" int mq_selftest_reciprocal(uint64_t* count, void* stream) {
+    if (!count) return mq_fail(MQ_ERR_ARG, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    int rc = mq_fill_u32(count, 0u, 2, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(mq::selftest_reciprocal_kernel, dim3(4096), dim3(256), 0, st, count);
+    return mq_check_launch("selftest reciprocal");
+}
 
 extern "C" int mq_selftest_convert(uint64_t* counts, void* stream) {
     if (!counts) return mq_fail(MQ_ERR_ARG, "null pointer");

@@ -41,7 +41,9 @@ int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, 
 int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
 bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M);
 int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st);
-int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
+int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int64_t max_zero_tiles, int group,
+                                   hipStream_t st);
+int64_t mq_int4_zero_tiles(int64_t rows, int64_t cols, int group);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -452,10 +454,16 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
             case MQ_JOB_INT4_PACK:
             case MQ_JOB_INT4_PACK_ASYM: {
                 if (tabled && cnt > kMaxGroup) {        // small groups keep the kernel-argument form (no pointer chase)
+                    int64_t zero_tiles = 0;
+                    if (head.kind == MQ_JOB_INT4_PACK_ASYM)
+                        for (int t = 0; t < cnt; t++) {
+                            const int64_t tiles = mq_int4_zero_tiles(jobs[i + t].rows, jobs[i + t].cols, head.p0);
+                            zero_tiles = tiles > zero_tiles ? tiles : zero_tiles;
+                        }
                     rc = head.kind == MQ_JOB_MXFP8       ? mq_mxfp8_launch_table(table + i, cnt, mx / 8, st)
                          : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_table(table + i, cnt, mx / 8, st)
                          : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_table(table + i, cnt, mx / 8, head.p0, st)
-                                                         : mq_int4_pack_asym_launch_table(table + i, cnt, mx / 8, head.p0, st);
+                                                         : mq_int4_pack_asym_launch_table(table + i, cnt, mx / 8, zero_tiles, head.p0, st);
                     break;
                 }
                 FlatTable tab{};

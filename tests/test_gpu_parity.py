@@ -52,6 +52,13 @@ def test_hardware_converts_agree_with_software_rne(lib):
     assert c[7] == 0, "packed e2m1 convert nibble order"
 
 
+def test_refined_hardware_reciprocal_is_the_ieee_quotient(lib):
+    count = torch.ones(1, dtype=torch.int64, device=DEV)
+    assert lib.mq_selftest_reciprocal(count.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert count.item() == 0, "v_rcp_f32 + one Newton step differs from 1.0f / s inside the shared-divisor range"
+
+
 # ---------------------------------------------------------------------------------------------------
 FP8_SHAPES = W.SMALL_REFERENCE_SHAPES + [(130, 264), (1, 8), (127, 136), (200, 1000), (5, 3)]
 
@@ -316,6 +323,39 @@ def test_int4_pack_layer_asymmetric(oracle, shape, G, dtype):
     packed_o, scale_o, zp_o = oracle.pack_layer(w, G, sym=False)
     assert packed.dtype == torch.int32 and scale.dtype == dtype and zp.dtype == torch.int32
     assert zp.shape == (shape[1] // G, shape[0] // 8)
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(zp, zp_o, "packed zero points")
+    _assert_same(packed, packed_o, "packed")
+
+
+@pytest.mark.parametrize("G", [32, 64, 128])
+def test_int4_pack_layer_asymmetric_shifted_groups(oracle, G):
+    """Groups shifted so that rint(min / scale) sweeps from below -15 to above 0: the fused form of the packed kernel
+    ends exactly at an unclamped zero point, and both neighbours (zero point clamped at 15 or at 0) take the written-out
+    chain; huge and tiny scales and an infinite extremum sit next to ordinary groups of the same wavefront."""
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    rows, cols = 64, 2048
+    gen = torch.Generator().manual_seed(4201)
+    w = torch.randn(rows, cols, generator=gen) * 0.02
+    groups = w.view(rows, cols // G, G)
+    span = groups.amax(-1, keepdim=True) - groups.amin(-1, keepdim=True)
+    # group minimum at -(k / 15) * span for k from -4 to 20 in steps of 0.25, plus half-way cases
+    k = (torch.arange(rows * (cols // G), dtype=torch.float32).view(rows, cols // G, 1) % 97) * 0.25 - 4.0
+    groups += -groups.amin(-1, keepdim=True) - k / 15.0 * span
+    w = groups.reshape(rows, cols).to(torch.bfloat16)
+    w[5, :G] *= 2.0 ** 100          # scale beyond the range of the shared-divisor sequence
+    w[6, :G] *= 2.0 ** -100
+    w[7, 3] = float("inf")
+    w[8, 5] = float("-inf")
+    w[9, 7] = float("nan")
+    w[10, G:2 * G] = 3.3e38         # bf16(scale) above 1e37 with an all-equal group next to it
+    w[11, :G] = torch.linspace(-3.3e38, 3.3e38, G).to(torch.bfloat16)
+    w[12, :G] = float("inf")        # equal infinities: the range is NaN and the scale falls to its floor
+    w[13, G:2 * G] = float("-inf")
+    w[14, :G] = float("nan")
+    packed, scale, zp = pack_layer(w.to(DEV), G, sym=False)
+    packed_o, scale_o, zp_o = oracle.pack_layer(w, G, sym=False)
     _assert_same(scale, scale_o, "scales")
     _assert_same(zp, zp_o, "packed zero points")
     _assert_same(packed, packed_o, "packed")
