@@ -314,8 +314,8 @@ def full_model_block_fp8(weights, elems):
 
 def adjacent_formats(gen):
     """GB/s of the kernels either side of the path (MXFP4 pack / unpack, INT4 unpack, asymmetric INT4 pack).
-    The unpackers and the asymmetric packer are single-tensor entry points, so they are timed as direct calls on
-    eight [16384, 7168] tensors: long enough launches that the GPU, not the host, sets the pace."""
+    The unpackers are single-tensor entry points, so they are timed as direct calls on eight [16384, 7168] tensors:
+    long enough launches that the GPU, not the host, sets the pace; the packers and the re-coder are job lists."""
     from miles_amd.kernels.quant.int4_fake import pack_layer
     from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
     from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
@@ -341,14 +341,18 @@ def adjacent_formats(gen):
     del batch
     run("next_mxfp4_dequant", "mxfp4_dequant", lambda: [dequantize_mxfp4(p, s, 32) for p, s in m4], "MXFP4 -> bf16")
     from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
-    run("next_mxfp4_to_fp8_recode", "mxfp4_to_fp8",
-        lambda: [cast_e2m1fn_to_e4m3fn(p.view(torch.int8), s) for p, s in m4], "MXFP4 -> e4m3 with 128x128 fp32 tile scales")
-    del m4
+    # the converter submits a shard's casts together (launch.deferred), so the line is a job list too
+    batch, outs = _record(lambda: [cast_e2m1fn_to_e4m3fn(p.view(torch.int8), s) for p, s in m4])
+    run("next_mxfp4_to_fp8_recode", "mxfp4_to_fp8", batch.run,
+        "MXFP4 -> e4m3 with 128x128 fp32 tile scales, one grouped launch (single calls: 0.65 of peak at this size)")
+    del batch, outs, m4
     i4 = [pack_layer(w, 128) for w in ws]
     run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")
     del i4
-    run("next_int4_g128_asym_pack", "int4_g128_asym", lambda: [pack_layer(w, 128, sym=False) for w in ws],
-        "pack_layer(sym=False), group 128")
+    batch, outs = _record(lambda: [pack_layer(w, 128, sym=False) for w in ws])
+    run("next_int4_g128_asym_pack", "int4_g128_asym", batch.run,
+        "pack_layer(sym=False), group 128, as the sync path runs it: one job list, two grouped launches")
+    del batch, outs
     from miles_amd.tools.convert_hf_to_fp8 import channel_fp8, tensor_fp8
     run("a2_channel_fp8", "fp8_channel", lambda: [channel_fp8(w) for w in ws], "one scale per row, rows read once")
     # per-tensor FP8 is a job of the batched driver: timed as a replayed job list, like the sync path runs it

@@ -226,6 +226,9 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      launches, codes and then packed zero points, with up to MQ_MAX_GROUP tensors)
  *     (mq_ue8m0_pack_scales with mn = rows, kb = cols, row_major = ld; its input is usually the scale output of an
  *      earlier job)
+ *   MQ_JOB_MXFP4_TO_FP8         e2m1 pairs    e4m3          fp32 tiles     aux = E8M0 bytes (in)       -
+ *     (mq_mxfp4_to_fp8_block with out_dim = rows, in_dim = cols, both multiples of 128: the experts of a checkpoint
+ *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
@@ -250,7 +253,8 @@ enum {
     MQ_JOB_FP8_BLOCK_POW2 = 8,
     MQ_JOB_UE8M0_PACK = 9,
     MQ_JOB_FP8_TENSOR = 10,
-    MQ_JOB_INT4_PACK_ASYM = 11
+    MQ_JOB_INT4_PACK_ASYM = 11,
+    MQ_JOB_MXFP4_TO_FP8 = 12
 };
 typedef struct mq_job {
     int32_t kind;
@@ -276,8 +280,9 @@ int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
  * callers that submit one job list again and again, as a replayed weight sync does).  The kernel arguments of a launch
  * hold MQ_MAX_GROUP descriptors at most; a model of thousands of small tensors (the 18 432 expert matrices of a
  * Qwen3-30B-A3B sync, 3 MB each) then drains and refills the chip every 64 tensors.  With a table a launch of the
- * MXFP8, MXFP4, INT4 (symmetric and asymmetric) and 128x128 FP8 jobs covers up to MQ_TABLE_GROUP tensors of similar size;
- * every other job kind, and FP8 jobs of mixed shapes, run as in mq_run_jobs.
+ * MXFP8, MXFP4, INT4 (symmetric and asymmetric), NVFP4 (standard block scaling), per-tensor FP8 and 128x128 FP8 jobs
+ * covers up to MQ_TABLE_GROUP tensors of similar size; every other job kind, Four Over Six NVFP4 jobs and FP8 jobs of
+ * mixed shapes run as in mq_run_jobs.
  * mq_job_table_fill writes n entries of MQ_JOB_TABLE_ENTRY_BYTES bytes into host memory, entry i for jobs[i]; the
  * caller copies them to device memory (any 8-byte aligned address) and passes that address, together with the same
  * jobs, to mq_run_jobs_tabled.  A call may cover a sub-range of the list: pass jobs + k, n' and the address of entry k.

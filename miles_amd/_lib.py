@@ -60,7 +60,7 @@ NVFP4_CARRY_AMAX = 8                                      # MQ_NVFP4_CARRY_AMAX:
 RECORD_AMAX_WORD, RECORD_REDO_WORD, RECORD_VOLATILE_WORD = 1024, 1028, 1029
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
- JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM) = range(12)
+ JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM, JOB_MXFP4_TO_FP8) = range(13)
 
 
 class Job(_c.Structure):

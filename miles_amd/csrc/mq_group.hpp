@@ -184,6 +184,21 @@ inline bool flat_grid(FlatRef& ref, int64_t max_units, int64_t per_block) {
     return mx < 0x7FFFFFF0;
 }
 
+// one MXFP4 tensor re-coded as FP8 with 128 x 128 scales: a workgroup takes a pair of tiles, neighbours along `in`
+struct RecodeJob {
+    const uint8_t* packed;    // [out, in / 2] e2m1 pairs
+    const uint8_t* scale;     // [out, in / 32] E8M0 bytes
+    uint8_t* y;               // [out, in] e4m3
+    float* tile_scale;        // [out / 128, in / 128]
+    int64_t in_dim;
+    int32_t tiles_in, pairs_in, total_pairs;
+    int32_t chunk;            // tile pairs an XCD takes in a row
+};
+struct RecodeTable {
+    int32_t n;
+    RecodeJob job[kMaxGroup];
+};
+
 // The amax record of the quantizers that need a whole-tensor maximum (NVFP4, per-tensor FP8): kRecordSections
 // sections of kSectionWords partial maxima (float bit patterns), then the folded amax and what is derived from it.
 constexpr int kSectionWords = 256;      // MQ_NVFP4_SECTION_WORDS: workgroups of an amax pass per tensor

@@ -205,14 +205,19 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_
 // 128-byte line coming in and 256 contiguous bytes going out, and every load and store instruction of a wavefront is a
 // run of consecutive 8- or 16-byte pieces.  A lane owns the same 16 columns of 8 rows; two neighbouring lanes share a
 // 1x32 group and its scale byte.
-__global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const uint8_t* __restrict__ packed,
-                                                           const uint8_t* __restrict__ scale,
-                                                           uint8_t* __restrict__ y, float* __restrict__ tile_scale,
-                                                           int64_t in_dim, int tiles_in, int pairs_in, int total_pairs,
-                                                           int chunk) {
+// blockIdx.y selects the tensor of a launch of up to kMaxGroup of them (a checkpoint shard's experts); the grid's x
+// extent is the largest tensor's, and a tensor deals its own tile pairs to the XCDs in its own chunk length.
+__global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const RecodeTable tab) {
     __shared__ uint32_t wave_smax[4][2];
-    const int32_t item = xcd_chunked_item(total_pairs, chunk);
+    const RecodeJob& job = tab.job[blockIdx.y];
+    const int32_t item = xcd_chunked_item(job.total_pairs, job.chunk);
     if (item < 0) return;
+    const uint8_t* __restrict__ packed = job.packed;
+    const uint8_t* __restrict__ scale = job.scale;
+    uint8_t* __restrict__ y = job.y;
+    float* __restrict__ tile_scale = job.tile_scale;
+    const int64_t in_dim = job.in_dim;
+    const int tiles_in = job.tiles_in, pairs_in = job.pairs_in;
     const int t = threadIdx.x;
     const int64_t ti = item / pairs_in, pj = item - ti * pairs_in;
     const int64_t groups_per_row = in_dim / 32;
@@ -337,21 +342,39 @@ extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, voi
     return mq_check_launch("mxfp4 dequant");
 }
 
-extern "C" int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, void* y, float* tile_scale,
-                                     int64_t out_dim, int64_t in_dim, void* stream) {
+// fills one descriptor; the shape checks of mq_mxfp4_to_fp8_block
+int mq_mxfp4_to_fp8_job(RecodeJob& job, const void* packed, const void* scale, void* y, void* tile_scale, int64_t out_dim,
+                        int64_t in_dim) {
     if ((!packed || !scale || !y || !tile_scale) && out_dim != 0 && in_dim != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
     if (out_dim < 0 || in_dim < 0 || out_dim % 128 != 0 || in_dim % 128 != 0)
         return mq_fail(MQ_ERR_ARG, "both dimensions must be multiples of 128");
     if ((((uintptr_t)packed | (uintptr_t)y) & 15) != 0) return mq_fail(MQ_ERR_ARG, "tensors must be 16-byte aligned");
-    if (out_dim == 0 || in_dim == 0) return MQ_OK;
     const int64_t tiles_in = in_dim / 128, pairs_in = (tiles_in + 1) / 2, pairs = (out_dim / 128) * pairs_in;
     // An XCD takes whole 128-row bands when there are enough of them: the band's scale bytes are one contiguous run,
     // and dealt out in smaller pieces every 128-byte line of them was fetched by four XCDs (measured: 0.625 bytes
     // read per element against 0.531 algorithmic).
     const int64_t chunk = (out_dim / 128 >= 2 * kXcds && pairs_in <= 4096) ? pairs_in : MQ_XCD_CHUNK;
-    const int64_t grid = xcd_grid_chunked(pairs, chunk);
-    if (grid > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    hipLaunchKernelGGL(mxfp4_to_fp8_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, packed, scale,
-                       (uint8_t*)y, tile_scale, in_dim, (int)tiles_in, (int)pairs_in, (int)pairs, (int)chunk);
+    if (xcd_grid_chunked(pairs, chunk) > 0x7FFFFFF0ll) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    job = RecodeJob{(const uint8_t*)packed, (const uint8_t*)scale, (uint8_t*)y, (float*)tile_scale, in_dim,
+                    (int32_t)tiles_in, (int32_t)pairs_in, (int32_t)pairs, (int32_t)chunk};
+    return MQ_OK;
+}
+int mq_mxfp4_to_fp8_launch_group(const RecodeTable& tab, hipStream_t st) {
+    int64_t grid = 0;
+    for (int i = 0; i < tab.n; i++) {
+        const int64_t g = xcd_grid_chunked(tab.job[i].total_pairs, tab.job[i].chunk);
+        grid = g > grid ? g : grid;
+    }
+    if (grid == 0 || tab.n == 0) return MQ_OK;
+    hipLaunchKernelGGL(mxfp4_to_fp8_kernel, dim3((unsigned)grid, (unsigned)tab.n), dim3(256), 0, st, tab);
     return mq_check_launch("mxfp4 to fp8");
+}
+
+extern "C" int mq_mxfp4_to_fp8_block(const uint8_t* packed, const uint8_t* scale, void* y, float* tile_scale,
+                                     int64_t out_dim, int64_t in_dim, void* stream) {
+    RecodeTable tab{};
+    tab.n = 1;
+    int rc = mq_mxfp4_to_fp8_job(tab.job[0], packed, scale, y, tile_scale, out_dim, in_dim);
+    if (rc != MQ_OK) return rc;
+    return mq_mxfp4_to_fp8_launch_group(tab, (hipStream_t)stream);
 }

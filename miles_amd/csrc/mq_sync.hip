@@ -44,6 +44,9 @@ int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st);
 int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int64_t max_zero_tiles, int group,
                                    hipStream_t st);
 int64_t mq_int4_zero_tiles(int64_t rows, int64_t cols, int group);
+int mq_mxfp4_to_fp8_job(RecodeJob& job, const void* packed, const void* scale, void* y, void* tile_scale, int64_t out_dim,
+                        int64_t in_dim);
+int mq_mxfp4_to_fp8_launch_group(const RecodeTable& tab, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -79,6 +82,8 @@ static bool job_fast(const mq_job& j) {
             return true;
         case MQ_JOB_FP8_TENSOR:
             return mq_fp8_tensor_fast_ok(j.in, j.dtype, j.out, j.rows, j.cols, j.ld);
+        case MQ_JOB_MXFP4_TO_FP8:
+            return true;               // check_job has refused what the kernel does not take
         default:
             return false;
     }
@@ -86,7 +91,7 @@ static bool job_fast(const mq_job& j) {
 
 static int64_t copy_dst_pitch(const mq_job& j);
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_INT4_PACK_ASYM) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_MXFP4_TO_FP8) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
@@ -97,6 +102,11 @@ static int check_job(const mq_job& j) {
     }
     if (j.kind == MQ_JOB_UE8M0_PACK)
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
+    if (j.kind == MQ_JOB_MXFP4_TO_FP8) {
+        if (j.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "bad MXFP4 to FP8 job");
+        RecodeJob probe;
+        return mq_mxfp4_to_fp8_job(probe, j.in, j.aux, j.out, j.scale, j.rows, j.cols);
+    }
     if (!empty && (j.kind == MQ_JOB_FP8_DEQUANT ? !j.aux : !j.scale)) return mq_fail(MQ_ERR_ARG, "job without a scale pointer");
     if (j.kind == MQ_JOB_NVFP4 && !j.aux) return mq_fail(MQ_ERR_ARG, "NVFP4 job without an amax record");
     if (j.kind == MQ_JOB_INT4_PACK_ASYM && !empty && (!j.aux || !j.aux2)) return mq_fail(MQ_ERR_ARG, "asymmetric INT4 job without zero-point outputs");
@@ -135,6 +145,8 @@ static int run_single(const mq_job& j, void* stream) {
                                                  j.rows, j.cols, j.p0, stream);
         case MQ_JOB_UE8M0_PACK:
             return mq_ue8m0_pack_scales((const float*)j.in, (int32_t*)j.out, j.p0, j.rows, j.cols, j.p1, j.ld != 0, stream);
+        case MQ_JOB_MXFP4_TO_FP8:
+            return mq_mxfp4_to_fp8_block((const uint8_t*)j.in, (const uint8_t*)j.aux, j.out, (float*)j.scale, j.rows, j.cols, stream);
         default:
             return mq_fail(MQ_ERR_ARG, "unknown job kind");
     }
@@ -473,6 +485,16 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                      : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_group(tab, st)
                      : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_group(tab, head.p0, st)
                                                      : mq_int4_pack_asym_launch_group(tab, head.p0, st);
+                break;
+            }
+            case MQ_JOB_MXFP4_TO_FP8: {
+                RecodeTable tab{};
+                tab.n = cnt;
+                for (int t = 0; t < cnt && rc == MQ_OK; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    rc = mq_mxfp4_to_fp8_job(tab.job[t], jb.in, jb.aux, jb.out, jb.scale, jb.rows, jb.cols);
+                }
+                if (rc == MQ_OK) rc = mq_mxfp4_to_fp8_launch_group(tab, st);
                 break;
             }
             case MQ_JOB_COPY: {

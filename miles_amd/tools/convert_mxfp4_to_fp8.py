@@ -39,10 +39,8 @@ def cast_e2m1fn_to_e4m3fn(x: torch.Tensor, scale: torch.Tensor) -> tuple[torch.T
         packed = packed.clone()
     y = torch.empty((out_dim, in_dim), dtype=torch.float8_e4m3fn, device=x.device)
     tile_scale = torch.empty((out_dim // 128, in_dim // 128), dtype=torch.float32, device=x.device)
-    launch.note_direct_call()
-    rc = _lib.load().mq_mxfp4_to_fp8_block(packed.data_ptr(), sbytes.data_ptr(), y.data_ptr(), tile_scale.data_ptr(),
-                                           out_dim, in_dim, _lib.stream_ptr(x.device))
-    _lib.check(rc)
+    # a job of the batched driver: inside `launch.deferred()` the casts of a whole shard share grouped launches
+    launch.submit(_lib.JOB_MXFP4_TO_FP8, packed, y, tile_scale, sbytes, None, out_dim, in_dim, in_dim)
     return y, tile_scale
 
 
@@ -86,17 +84,18 @@ def main(model_dir: str, save_dir: str, device: str = "cuda") -> None:
     for shard_name in shard_names:
         state = load_file(str(src / shard_name), device=device)
         converted = {}
-        for name, tensor in state.items():
-            if name in fp4_scales:
-                continue            # re-emitted next to its weight
-            if name not in fp4_weights:
-                converted[name] = tensor
-                continue
-            scale_name = scale_of[name]
-            scale = state[scale_name] if scale_name in state else \
-                load_file(str(src / weight_map[scale_name]), device=device)[scale_name]
-            converted[name], converted[scale_name] = cast_e2m1fn_to_e4m3fn(tensor, scale)
-            weight_map[scale_name] = shard_name
+        with launch.deferred():     # the shard's casts are submitted together when the block ends
+            for name, tensor in state.items():
+                if name in fp4_scales:
+                    continue            # re-emitted next to its weight
+                if name not in fp4_weights:
+                    converted[name] = tensor
+                    continue
+                scale_name = scale_of[name]
+                scale = state[scale_name] if scale_name in state else \
+                    load_file(str(src / weight_map[scale_name]), device=device)[scale_name]
+                converted[name], converted[scale_name] = cast_e2m1fn_to_e4m3fn(tensor, scale)
+                weight_map[scale_name] = shard_name
         save_file(converted, str(dst / shard_name))
     (dst / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}, indent=2) + "\n")
     assert fp4_weights, "no packed-fp4 expert weights found; is this already an FP8 checkpoint?"

@@ -558,6 +558,42 @@ def test_mxfp4_to_fp8_recode(oracle, shape, lo, hi):
         cast_e2m1fn_to_e4m3fn(packed[:100].to(DEV), scale[:100].to(DEV))
 
 
+def test_mxfp4_to_fp8_recode_grouped(oracle):
+    """A shard's experts re-coded inside `launch.deferred()`: tensors of different shapes share grouped launches
+    (the larger ones set the grid, a single-pair tensor rides along), bytes as from single calls."""
+    from miles_amd import launch
+    from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
+
+    g = torch.Generator().manual_seed(43)
+    shapes = [(256, 512), (256, 384), (128, 128), (384, 256), (256, 512), (2048, 7168), (7168, 2048), (128, 256)]
+    ins = []
+    for shape in shapes:
+        packed = torch.randint(0, 256, (shape[0], shape[1] // 2), dtype=torch.uint8, generator=g).view(torch.int8)
+        scale = torch.randint(100, 140, (shape[0], shape[1] // 32), dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+        ins.append((packed, scale))
+    dev = [(p.to(DEV), s.to(DEV)) for p, s in ins]
+    with launch.deferred() as batch:
+        outs = [cast_e2m1fn_to_e4m3fn(p, s) for p, s in dev]
+    assert len(batch) == len(shapes) and batch.direct_calls == 0
+    for (p, s), (y, ts) in zip(ins, outs):
+        y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(p, s)
+        _assert_same(ts, ts_o, "tile scales (grouped)")
+        _assert_same(y, y_o, "e4m3 codes (grouped)")
+
+
+def test_mxfp4_to_fp8_job_argument_checks(lib):
+    from miles_amd import _lib
+
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
+    def job(rows, cols, offset=0):
+        return (_lib.Job * 1)(_lib.Job(_lib.JOB_MXFP4_TO_FP8, 0, buf.data_ptr() + offset, buf.data_ptr(), buf.data_ptr(),
+                                       buf.data_ptr(), None, rows, cols, cols, 0, 0, 0, 0))
+    assert lib.mq_run_jobs(job(128, 128), 1, None) == 0
+    assert lib.mq_run_jobs(job(100, 128), 1, None) != 0          # rows not a multiple of 128
+    assert lib.mq_run_jobs(job(128, 128, offset=8), 1, None) != 0  # packed codes off a 16-byte boundary
+    torch.cuda.synchronize()
+
+
 # ---------------------------------------------------------------------------------------------------
 # block fake quantization (miles/kernels/quant/fake_quant.py)
 @pytest.mark.parametrize("kind", ["fp8", "fp4", "compressed_kv"])
