@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
 // `zero` is [rows, groups_per_row] bytes and the packed words are its transpose, eight rows to a word.  A workgroup
 // takes a tile of 256 rows x 64 groups through LDS: the bytes are read along the rows (neighbouring lanes, neighbouring
 // bytes) and the words written along j (32 consecutive words of one group per half wavefront).
-constexpr int kZpRows = 256, kZpCols = 64, kZpPitch = kZpCols + 2;
+constexpr int kZpRows = 256, kZpCols = 64, kZpPitch = kZpCols + 4;
 __host__ __device__ __forceinline__ int64_t int4_zero_tiles(int64_t rows8, int64_t groups_per_row) {
     return ((rows8 * 8 + kZpRows - 1) / kZpRows) * ((groups_per_row + kZpCols - 1) / kZpCols);
 }
@@ -502,7 +502,20 @@ __device__ __forceinline__ void int4_zero_pack_tile(const uint8_t* __restrict__ 
     const int64_t row0 = (tile / col_tiles) * kZpRows, g0 = (tile % col_tiles) * kZpCols;
     const int64_t rows = rows8 * 8;
     const int t = threadIdx.x;
-    {
+    if ((groups_per_row & 3) == 0 && ((uintptr_t)zero & 3) == 0) {
+        // four bytes per lane and every load of the tile issued before the first is used: one memory round trip
+        const int c = (t & 15) * 4;
+        const bool col_live = g0 + c < groups_per_row;
+        uint32_t v[kZpRows / 16];
+#pragma unroll
+        for (int i = 0; i < kZpRows / 16; i++) {
+            const int r = (t >> 4) + 16 * i;
+            const bool live = col_live && row0 + r < rows;
+            v[i] = live ? *(const uint32_t*)(zero + (row0 + r) * groups_per_row + g0 + c) : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < kZpRows / 16; i++) *(uint32_t*)(lds + ((t >> 4) + 16 * i) * kZpPitch + c) = v[i];
+    } else {
         const int c = t & (kZpCols - 1);
         const bool col_live = g0 + c < groups_per_row;
 #pragma unroll 8
@@ -530,14 +543,14 @@ __device__ __forceinline__ void int4_zero_pack_tile(const uint8_t* __restrict__ 
 __global__ __launch_bounds__(256) void int4_zero_pack_kernel(const uint8_t* __restrict__ zero,
                                                              uint32_t* __restrict__ packed_zp, int64_t M,
                                                              int64_t groups_per_row) {
-    __shared__ uint8_t lds[kZpRows * kZpPitch];
+    __shared__ __align__(4) uint8_t lds[kZpRows * kZpPitch];
     int4_zero_pack_tile(zero, packed_zp, M / 8, groups_per_row, blockIdx.x, lds);
 }
 // the zero points of a group of tensors (descriptors as for int4_pack_asym_bf16_kernel): blockIdx.y selects the tensor;
 // a tensor of `units` 16-byte units has units / units_per_group groups, groups_per_row of them in each row
 template <class Table>
 __global__ __launch_bounds__(256) void int4_zero_pack_group_kernel(const Table tab, int units_per_group) {
-    __shared__ uint8_t lds[kZpRows * kZpPitch];
+    __shared__ __align__(4) uint8_t lds[kZpRows * kZpPitch];
     const FlatJob& job = flat_job(tab);
     const int64_t groups_per_row = job.section;
     if (groups_per_row <= 0) return;
