@@ -344,7 +344,7 @@ def adjacent_formats(gen):
     # the converter submits a shard's casts together (launch.deferred), so the line is a job list too
     batch, outs = _record(lambda: [cast_e2m1fn_to_e4m3fn(p.view(torch.int8), s) for p, s in m4])
     run("next_mxfp4_to_fp8_recode", "mxfp4_to_fp8", batch.run,
-        "MXFP4 -> e4m3 with 128x128 fp32 tile scales, one grouped launch (single calls: 0.65 of peak at this size)")
+        "MXFP4 -> e4m3 with 128x128 fp32 tile scales, one job list: tile scales, then a flat stream (single calls: 0.65 of peak at this size)")
     del batch, outs, m4
     i4 = [pack_layer(w, 128) for w in ws]
     run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")

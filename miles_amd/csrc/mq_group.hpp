@@ -192,7 +192,10 @@ struct RecodeJob {
     float* tile_scale;        // [out / 128, in / 128]
     int64_t in_dim;
     int32_t tiles_in, pairs_in, total_pairs;
-    int32_t chunk;            // tile pairs an XCD takes in a row
+    int32_t chunk;            // tile pairs an XCD takes in a row (tile form)
+    // flat form: 16-element units, tile_div constants for units per row, XCD run length of the flat grid
+    uint32_t units, magic_upr, shift_upr;
+    int32_t flat_chunk;
 };
 struct RecodeTable {
     int32_t n;

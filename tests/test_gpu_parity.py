@@ -579,6 +579,19 @@ def test_mxfp4_to_fp8_recode_grouped(oracle):
         y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(p, s)
         _assert_same(ts, ts_o, "tile scales (grouped)")
         _assert_same(y, y_o, "e4m3 codes (grouped)")
+    # scale bytes off a 4-byte boundary: the group falls back to the one-launch tile form
+    odd = []
+    for p, s in ins[:3]:
+        flat = torch.zeros(s.numel() + 1, dtype=torch.uint8, device=DEV)
+        flat[1:] = s.view(torch.uint8).reshape(-1).to(DEV)
+        odd.append((p.to(DEV), flat[1:].view(s.shape).view(torch.float8_e8m0fnu)))
+    assert all(s.data_ptr() % 4 == 1 for _, s in odd)
+    with launch.deferred():
+        outs = [cast_e2m1fn_to_e4m3fn(p, s) for p, s in odd]
+    for (p, s), (y, ts) in zip(ins[:3], outs):
+        y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(p, s)
+        _assert_same(ts, ts_o, "tile scales (grouped, unaligned scales)")
+        _assert_same(y, y_o, "e4m3 codes (grouped, unaligned scales)")
 
 
 def test_mxfp4_to_fp8_job_argument_checks(lib):
