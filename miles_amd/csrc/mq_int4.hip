@@ -85,14 +85,20 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
     uint16_t* __restrict__ scale = (uint16_t*)job.s;
     const int64_t total_units = job.units;
-    const int t = threadIdx.x;
+    const uint32_t t = threadIdx.x;
     const int64_t base = flat_block(tab) * (kI4Threads * kI4Unroll);
     if (base >= total_units) return;
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset
+    const int64_t left = total_units - base;
+    const uint32_t rem = left < kI4Threads * kI4Unroll ? (uint32_t)left : (uint32_t)(kI4Threads * kI4Unroll);
+    const uint16_t* __restrict__ w0 = w + base * 8;
+    uint32_t* __restrict__ packed0 = packed + base;
+    uint16_t* __restrict__ scale0 = scale + base / LANES;        // `base` is a multiple of the lanes per group
     u32x4 v[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
-        const int64_t unit = base + i * kI4Threads + t;
-        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        const uint32_t off = t + i * kI4Threads;
+        v[i] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
     }
     uint32_t top = 0;
 #pragma unroll
@@ -123,9 +129,10 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
             }
         }
         word -= kMagicSum;
-        if (unit < total_units) {
-            st4(packed + unit, word);
-            if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)hw_bf16x2(s, 0.0f);
+        const uint32_t off = t + i * kI4Threads;
+        if (off < rem) {
+            st4(packed0 + off, word);
+            if ((t & (LANES - 1)) == 0) scale0[off / LANES] = (uint16_t)hw_bf16x2(s, 0.0f);
         }
     }
     // A group holding the largest finite bf16, an infinity or a NaN is outside the fused form: a wavefront that met one
@@ -384,24 +391,31 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
 // through the builtins every step costs a move, a quieting of the moved value and the max itself.  A DPP operand must
 // have been written two issue slots earlier (whatever the compiler put in front of the block included), so the block
 // opens with two idle slots and the two chains alternate with one idle slot per step.
+#define MQ_EXTREMA_FIRST(ctrl)                                               \
+    "v_max_f32_dpp %0, %2, %2 " ctrl " row_mask:0xf bank_mask:0xf\n\t"        \
+    "v_min_f32_dpp %1, %3, %3 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
 #define MQ_EXTREMA_STEP(ctrl)                                                \
     "v_max_f32_dpp %0, %0, %0 " ctrl " row_mask:0xf bank_mask:0xf\n\t"        \
     "v_min_f32_dpp %1, %1, %1 " ctrl " row_mask:0xf bank_mask:0xf\n\t"
 template <int LANES>
 __device__ __forceinline__ void seg_extrema(float& mx, float& mn) {
     static_assert(LANES == 4 || LANES == 8 || LANES == 16, "group of 32, 64 or 128 elements");
+    float gx, gn;          // results in registers of their own: tied operands made the compiler copy the inputs first
     if (LANES == 4)
-        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
-                     : "+v"(mx), "+v"(mn));
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_FIRST("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+                     : "=&v"(gx), "=&v"(gn) : "v"(mx), "v"(mn));
     else if (LANES == 8)
-        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_FIRST("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
                      "s_nop 0\n\t" MQ_EXTREMA_STEP("row_half_mirror")
-                     : "+v"(mx), "+v"(mn));
+                     : "=&v"(gx), "=&v"(gn) : "v"(mx), "v"(mn));
     else
-        asm volatile("s_nop 1\n\t" MQ_EXTREMA_STEP("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
+        asm volatile("s_nop 1\n\t" MQ_EXTREMA_FIRST("quad_perm:[1,0,3,2]") "s_nop 0\n\t" MQ_EXTREMA_STEP("quad_perm:[2,3,0,1]")
                      "s_nop 0\n\t" MQ_EXTREMA_STEP("row_half_mirror") "s_nop 0\n\t" MQ_EXTREMA_STEP("row_mirror")
-                     : "+v"(mx), "+v"(mn));
+                     : "=&v"(gx), "=&v"(gn) : "v"(mx), "v"(mn));
+    mx = gx;
+    mn = gn;
 }
+#undef MQ_EXTREMA_FIRST
 #undef MQ_EXTREMA_STEP
 // job: w, q = packed codes, s = scales, aux = zero points (one byte per group, read again by the zero-point packer),
 // aux2 = packed zero points, units, section = groups per row
@@ -422,18 +436,25 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
     uint16_t* __restrict__ scale_out = (uint16_t*)job.s;
     uint8_t* __restrict__ zero_out = (uint8_t*)job.aux;
     const int64_t total_units = job.units;
-    const int t = threadIdx.x;
+    const uint32_t t = threadIdx.x;
     const int64_t first = flat_block(tab) * (kI4Threads * kI4Unroll);
     if (first >= total_units) return;
-    const int64_t base = first + t;
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset
+    const int64_t left = total_units - first;
+    const uint32_t rem = left < kI4Threads * kI4Unroll ? (uint32_t)left : (uint32_t)(kI4Threads * kI4Unroll);
+    const uint16_t* __restrict__ w0 = w + first * 8;
+    uint32_t* __restrict__ packed0 = packed + first;
+    uint16_t* __restrict__ scale0 = scale_out + first / LANES;        // `first` is a multiple of the lanes per group
+    uint8_t* __restrict__ zero0 = zero_out + first / LANES;
     // a group is a whole number of lanes, so dead lanes never share one with live lanes; they re-read the last unit
     u32x4 v[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
-        const int64_t unit = base + i * kI4Threads;
-        v[i] = ld16(w + (unit < total_units ? unit : total_units - 1) * 8);
+        const uint32_t off = t + i * kI4Threads;
+        v[i] = ld16(w0 + (off < rem ? off : rem - 1) * 8u);
     }
-    bool odd = false;
+    // wavefronts with a group outside the fused form: the tests are collected as wavefront masks (scalar registers)
+    uint64_t odd = 0;
     uint32_t word[kI4Unroll], sb[kI4Unroll], z[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
@@ -443,9 +464,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
 #pragma unroll
         for (int j = 1; j < 8; j++) { mx = __builtin_fmaxf(mx, f[j]); mn = __builtin_fminf(mn, f[j]); }
         // a NaN element is skipped by the extrema but is not coded like a number: its wavefront takes the chain below,
-        // whatever the fused form makes of the group (fcmp unordered takes two elements at a time)
-        const bool nan = (f[0] != f[0]) | (f[1] != f[1]) | (f[2] != f[2]) | (f[3] != f[3]) | (f[4] != f[4]) |
-                         (f[5] != f[5]) | (f[6] != f[6]) | (f[7] != f[7]);
+        // whatever the fused form makes of the group (an unordered compare takes two elements at a time)
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) odd |= __builtin_amdgcn_ballot_w64(!(f[j] == f[j]) || !(f[j + 1] == f[j + 1]));
         seg_extrema<LANES>(mx, mn);
         const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
         const float ys = recip_shared(s);
@@ -456,7 +477,9 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
         // floor scale and lo = NaN, which fails both comparisons.
         const float lo = __builtin_rintf(div_by_shared(mn, s, ys));
         z[i] = (uint32_t)(int)(0.0f - lo);
-        odd |= !shared_div_ok(s) | !(lo <= 0.0f) | !(lo >= -15.0f) | nan;
+        odd |= __builtin_amdgcn_ballot_w64(!shared_div_ok(s));
+        odd |= __builtin_amdgcn_ballot_w64(!(lo <= 0.0f));
+        odd |= __builtin_amdgcn_ballot_w64(!(lo >= -15.0f));
         // rint through one add of 1.5 * 2^23: the low bits of the sum's pattern are the (signed) integer.  The zero point
         // is added as an integer afterwards (inside the float add an odd zero point would turn the ties around);
         // everything is arithmetic modulo 2^32, like the reference's int32 sum.
@@ -464,22 +487,25 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
         uint32_t sum = 0;
 #pragma unroll
         for (int j = 0; j < 8; j++) sum += f2u(div_by_shared(f[j], s, ys) + 12582912.0f) << (4 * j);
-        word[i] = sum - kMagicSum + z[i] * 0x11111111u;
+        // z in every nibble (z <= 15 where the word is kept): z * 0x11 in the low byte, the byte copied to all four
+        const uint32_t zz = __builtin_amdgcn_perm(0u, z[i] | (z[i] << 4), 0u);
+        word[i] = sum - kMagicSum + zz;
     }
     // all stores after all loads have been used: a store between them would have to complete before the next unit's
     // data counts as arrived (loads and stores return in order)
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
-        const int64_t unit = base + i * kI4Threads;
-        if (unit < total_units) {
-            st4(packed + unit, word[i]);
+        const uint32_t off = t + i * kI4Threads;
+        if (off < rem) {
+            st4(packed0 + off, word[i]);
             if ((t & (LANES - 1)) == 0) {
-                scale_out[unit / LANES] = (uint16_t)sb[i];
-                zero_out[unit / LANES] = (uint8_t)z[i];
+                scale0[off / LANES] = (uint16_t)sb[i];
+                zero0[off / LANES] = (uint8_t)z[i];
             }
         }
     }
-    if (__builtin_amdgcn_ballot_w64(odd) == 0) return;
+    const int64_t base = first + t;
+    if (odd == 0) return;
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
         const int64_t unit = base + i * kI4Threads;

@@ -65,18 +65,24 @@ __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const Table tab)
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
     const int64_t total_units = job.units;
-    const int t = threadIdx.x;
+    const uint32_t t = threadIdx.x;
     const int64_t base = flat_block(tab) * (kM4Threads * kM4Unroll);
     if (base >= total_units) return;
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset
+    const int64_t left = total_units - base;
+    const uint32_t rem = left < kM4Threads * kM4Unroll ? (uint32_t)left : (uint32_t)(kM4Threads * kM4Unroll);
+    const uint16_t* __restrict__ w0 = w + base * 8;
+    uint32_t* __restrict__ packed0 = packed + base;
+    uint8_t* __restrict__ scale0 = scale + base / 4;        // `base` is a multiple of the four lanes of a group
     u32x4 v[kM4Unroll];
 #pragma unroll
     for (int i = 0; i < kM4Unroll; i++) {
-        const int64_t unit = base + i * kM4Threads + t;
-        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        const uint32_t off = t + i * kM4Threads;
+        v[i] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int i = 0; i < kM4Unroll; i++) {
-        const int64_t unit = base + i * kM4Threads + t;
+        const uint32_t off = t + i * kM4Threads;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max4(hmax_u16(m2));
         const uint32_t byte = mxfp4_scale_byte_bf16(mb);
@@ -96,9 +102,9 @@ __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const Table tab)
 #pragma unroll
             for (int j = 0; j < 8; j++) word |= mxfp4_code(f[j], mult) << (4 * j);
         }
-        if (unit < total_units) {
-            st4(packed + unit, word);
-            if ((t & 3) == 0) scale[unit >> 2] = (uint8_t)byte;
+        if (off < rem) {
+            st4(packed0 + off, word);
+            if ((t & 3) == 0) scale0[off >> 2] = (uint8_t)byte;
         }
     }
 }

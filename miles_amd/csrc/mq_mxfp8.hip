@@ -40,18 +40,24 @@ __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab)
     uint8_t* __restrict__ q = (uint8_t*)job.q;
     uint8_t* __restrict__ scale = (uint8_t*)job.s;
     const int64_t total_units = job.units;
-    const int t = threadIdx.x;
+    const uint32_t t = threadIdx.x;
     const int64_t base = flat_block(tab) * (kMxThreads * kMxUnroll);
     if (base >= total_units) return;
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset
+    const int64_t left = total_units - base;
+    const uint32_t rem = left < kMxThreads * kMxUnroll ? (uint32_t)left : (uint32_t)(kMxThreads * kMxUnroll);
+    const uint16_t* __restrict__ w0 = w + base * 8;
+    uint8_t* __restrict__ q0 = q + base * 8;
+    uint8_t* __restrict__ scale0 = scale + base / 4;        // `base` is a multiple of the four lanes of a group
     u32x4 v[kMxUnroll];
 #pragma unroll
     for (int i = 0; i < kMxUnroll; i++) {
-        const int64_t unit = base + i * kMxThreads + t;
-        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        const uint32_t off = t + i * kMxThreads;
+        v[i] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int i = 0; i < kMxUnroll; i++) {
-        const int64_t unit = base + i * kMxThreads + t;
+        const uint32_t off = t + i * kMxThreads;
         uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max4(hmax_u16(m2));   // bf16 pattern of the group amax, quad-uniform
         const float amax = u2f(mb << 16);
@@ -71,9 +77,9 @@ __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab)
             o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
             o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
         }
-        if (unit < total_units) {
-            st8(q + unit * 8, o);
-            if ((t & 3) == 0) scale[unit >> 2] = (uint8_t)e;
+        if (off < rem) {
+            st8(q0 + off * 8u, o);
+            if ((t & 3) == 0) scale0[off >> 2] = (uint8_t)e;
         }
     }
 }

@@ -266,11 +266,17 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
     const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
     const int64_t total_units = job.units;
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset
+    const int64_t left = total_units - base;
+    const uint32_t rem = left < kNvThreads * kNvUnroll ? (uint32_t)left : (uint32_t)(kNvThreads * kNvUnroll);
+    const uint16_t* __restrict__ w0 = w + base * 8;
+    uint32_t* __restrict__ q0 = q + base;
+    uint8_t* __restrict__ s80 = s8 + base / 2;        // `base` is a multiple of the two lanes of a block
     u32x4 v[kNvUnroll];
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
-        const int64_t unit = base + i * kNvThreads + t;
-        v[i] = unit < total_units ? ld16(w + unit * 8) : u32x4{0u, 0u, 0u, 0u};
+        const uint32_t off = (uint32_t)t + i * kNvThreads;
+        v[i] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
     }
     NvScales gs;
     gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
@@ -281,7 +287,7 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
     uint32_t seen = 0;
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
-        const int64_t unit = base + i * kNvThreads + t;
+        const uint32_t off = (uint32_t)t + i * kNvThreads;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max2(hmax_u16(m2));
         seen = umax(seen, mb);
@@ -312,9 +318,9 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
 #pragma unroll
             for (int j = 0; j < 8; j++) word |= sw_e2m1(f[j] * inv) << (4 * j);
         }
-        if (unit < total_units) {
-            st4(q + unit, word);
-            if ((t & 1) == 0) s8[unit >> 1] = (uint8_t)sc;
+        if (off < rem) {
+            st4(q0 + off, word);
+            if ((t & 1) == 0) s80[off >> 1] = (uint8_t)sc;
         }
     }
     return seen;
