@@ -305,7 +305,12 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
         } else if (mb < 0x7F80u && s_hp == s_hp) {
             sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
             const float s_f = hw_e4m3x2_decode<false>(sc).x;
-            const float inv = __builtin_fminf(1.0f / (s_f * gs.s_dec), kFltMax);
+            // 1 / (block scale x global decode scale): the refined hardware reciprocal where it equals the division (every
+            // divisor in 2^-91 .. 2^90, far below FLT_MAX), decided for the wavefront; an all-zero block has divisor 0
+            const float d = s_f * gs.s_dec;
+            float inv;
+            if (__builtin_amdgcn_ballot_w64(!shared_div_ok(d)) == 0) inv = recip_shared(d);
+            else inv = __builtin_fminf(1.0f / d, kFltMax);
             word = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
             word = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, word);
             word = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, word);
