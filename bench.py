@@ -169,7 +169,8 @@ def per_quantizer(gen):
         toggle[0] = 1.0 / toggle[0]
 
     run("C5a_nvfp4_every_amax_moved", "nvfp4", n, nvfp4_all,
-        "as C5a, worst case of the carried amax: every tensor's amax differs from the last sync's, so each is quantized twice",
+        "as C5a, worst case of the carried amax: every tensor's amax differs from the last sync's; the batch sees that "
+        "in the moved-record count of the syncs before and submits the plain two-pass form (the first-sync cost)",
         prepare=lambda b: b.carry_amax(), before_each=move_every_amax)
     os.environ["NVTE_NVFP4_4OVER6"] = "weights"        # Four Over Six: two candidates per block, e4m3 max 256
     try:

@@ -46,6 +46,7 @@ SIGNATURES = {
     "mq_run_jobs": [_vp, _i64, _vp],
     "mq_job_table_fill": [_vp, _i64, _vp],
     "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
+    "mq_run_jobs_feedback": [_vp, _i64, _vp, _vp, _vp],
     "mq_selftest_convert": [_vp, _vp],
     "mq_selftest_reciprocal": [_vp, _vp],
     "mq_copy_bytes": [_vp, _vp, _i64, _vp],

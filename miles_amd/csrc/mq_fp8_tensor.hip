@@ -21,7 +21,7 @@ constexpr int kFtUnroll = 2;
 
 // job.s = fp32 scale output, job.aux = amax record (section 0)
 template <int MODE, class Table>   // 1: fold and clear; 2: also compare with the amax the record held
-__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, float floor_v) {
+__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, float floor_v, uint32_t* moved_counter) {
     __shared__ uint32_t lds4[4];
     const FlatJob& job = tab.job[blockIdx.x];
     uint32_t* rec = (uint32_t*)job.aux;
@@ -38,9 +38,11 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, f
             const bool moved = rec[kRecAmax] != m;
             rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;
             rec[kRecVolatile] = moved ? 1u : 0u;
+            amax_feedback(moved_counter, moved);
         } else {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
+            amax_feedback(moved_counter, rec[kRecAmax] != m);
         }
         rec[kRecAmax] = m;
         float amax = u2f(m);
@@ -158,14 +160,14 @@ static int fp8_tensor_launch(const Table& tab, int n, float floor_v, bool carry,
     const dim3 folds((unsigned)n), blk(256), grid((unsigned)tab.max_blocks, (unsigned)n);
     if (carry) {
         if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<1, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
-        hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v);
+        hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
         if (tab.max_blocks > 0) {
             const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             hipLaunchKernelGGL((fp8_tensor_quant_kernel<2, Table>), dim3(redo, (unsigned)n), dim3(kFtThreads), 0, st, tab, floor_v);
         }
         return mq_check_launch("fp8 per-tensor quant (carried-over amax)");
     }
-    hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v);
+    hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
     if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<0, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
     return mq_check_launch("fp8 per-tensor quant");
 }

@@ -209,6 +209,11 @@ constexpr int kRecordSections = 4;      // MQ_NVFP4_SECTIONS
 constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (float bits)
 constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
 constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last run: the next carried run collects the amax first
+// A fold launched by the job driver also tells its caller how many records held another amax before (a counter in
+// device memory that only ever grows): a caller whose every amax keeps moving can then submit the plain two-pass form.
+__device__ __forceinline__ void amax_feedback(uint32_t* counter, bool moved) {
+    if (counter && moved) atomicAdd(counter, 1u);
+}
 
 struct CopyJob {      // rows of `bytes` bytes each (one row: a plain run), chunks_per_row chunks of the copy kernel per row
     const uint8_t* src;

@@ -124,7 +124,7 @@ constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 //   with the fresh amax -- the cost of the plain two-pass form, instead of two full quantizations.  The mark is dropped
 //   as soon as the amax has held still for one sync.
 template <int MODE, class Table>
-__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer) {
+__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer, uint32_t* moved_counter) {
     __shared__ uint32_t lds4[4];
     const int ji = blockIdx.x;
     const FlatJob& job = tab.job[ji];
@@ -146,9 +146,11 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float 
                                  rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
             rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;     // a volatile record has no codes yet
             rec[kRecVolatile] = moved ? 1u : 0u;
+            amax_feedback(moved_counter, moved);
         } else if (MODE == 1) {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
+            amax_feedback(moved_counter, rec[kRecAmax] != f2u(amax));
         }
         rec[kRecAmax] = f2u(amax);
         rec[kRecEncSixth] = f2u(gs.enc_sixth);
@@ -573,15 +575,15 @@ static int nvfp4_quant_launch(const Table& tab, int n, int e4m3_max, int flags, 
     const dim3 grid((unsigned)tab.max_blocks, (unsigned)n);
     if (mode == 2) {
         if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
-        hipLaunchKernelGGL((nvfp4_fold_kernel<2, Table>), folds, blk, 0, st, tab, numer);
+        hipLaunchKernelGGL((nvfp4_fold_kernel<2, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback());
         if (tab.max_blocks > 0) {
             const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)n), st);
         }
         return mq_check_launch("nvfp4 quant (carried-over amax)");
     }
-    if (mode == 1) hipLaunchKernelGGL((nvfp4_fold_kernel<1, Table>), folds, blk, 0, st, tab, numer);
-    else hipLaunchKernelGGL((nvfp4_fold_kernel<0, Table>), folds, blk, 0, st, tab, numer);
+    if (mode == 1) hipLaunchKernelGGL((nvfp4_fold_kernel<1, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback());
+    else hipLaunchKernelGGL((nvfp4_fold_kernel<0, Table>), folds, blk, 0, st, tab, numer, (uint32_t*)nullptr);
     if (tab.max_blocks > 0) launch_nvfp4_quant<0>(tab, flags, numer, grid, st);
     return mq_check_launch("nvfp4 quant");
 }
@@ -640,7 +642,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
     FlatTable fold{};
     fold.n = 1;
     fold.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), 0, global_scale, n_sections, 0};
-    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, st, fold, numer);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, st, fold, numer, (uint32_t*)nullptr);
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
@@ -655,7 +657,7 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
     FlatTable tab{};
     tab.n = 1;
     tab.job[0] = FlatJob{nullptr, nullptr, nullptr, record, 0, nullptr, n_sections, 0};
-    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f, (uint32_t*)nullptr);
     return mq_check_launch("nvfp4 fold");
 }
 

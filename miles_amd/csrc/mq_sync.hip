@@ -371,6 +371,15 @@ extern "C" int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table
 
 extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) { return mq_run_jobs_tabled(jobs, n, nullptr, stream); }
 
+extern "C" int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved,
+                                    void* stream) {
+    if ((uintptr_t)device_moved % 4 != 0) return mq_fail(MQ_ERR_ARG, "feedback counter must be 4-byte aligned");
+    mq_set_amax_feedback(device_moved);
+    const int rc = mq_run_jobs_tabled(jobs, n, device_table, stream);
+    mq_set_amax_feedback(nullptr);
+    return rc;
+}
+
 extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, void* stream) {
     if (n < 0 || (n > 0 && !jobs)) return mq_fail(MQ_ERR_ARG, "bad job list");
     if ((uintptr_t)device_table % 8 != 0) return mq_fail(MQ_ERR_ARG, "job table must be 8-byte aligned");

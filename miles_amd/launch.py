@@ -10,6 +10,7 @@ launch-bound without changing the per-tensor call signatures.
 
 from __future__ import annotations
 
+import collections
 import contextlib
 import ctypes
 import threading
@@ -21,6 +22,49 @@ from miles_amd import _lib
 _state = threading.local()
 
 
+class _AmaxFeedback:
+    """How many amax records moved in the syncs already finished, read without ever waiting for the GPU.
+
+    The folds of a `mq_run_jobs_feedback` call add to a device counter that only grows; after each whole submission the
+    counter is copied into one of a few pinned words and an event is recorded.  At the start of the next submission the
+    copies that have arrived are read: when more than half of the records moved per sync, the list is submitted in
+    the plain two-pass form (the carried-over amax would cost every such tensor a second pass), until they hold again.
+    A host that runs ahead of the GPU simply keeps its last decision."""
+
+    SLOTS = 8
+
+    def __init__(self, device, records: int) -> None:
+        self.counter = torch.zeros(1, dtype=torch.int32, device=device)
+        self.host = torch.zeros(self.SLOTS, dtype=torch.int32).pin_memory()
+        self.pending: collections.deque = collections.deque()     # (event, pinned slot, index of the sync it closes)
+        self.free = list(range(self.SLOTS))
+        self.records = records
+        self.syncs = 0
+        self.seen = (0, 0)          # (sync index, counter value) of the newest copy that was read
+        self.plain = False
+
+    def decide(self) -> bool:
+        while self.pending and self.pending[0][0].query():
+            _event, slot, index = self.pending.popleft()
+            total = int(self.host[slot]) & 0xFFFFFFFF
+            moved = (total - self.seen[1]) & 0xFFFFFFFF
+            syncs = index - self.seen[0]
+            self.seen = (index, total)
+            self.free.append(slot)
+            self.plain = moved * 2 > self.records * syncs
+        return self.plain
+
+    def submitted(self) -> None:
+        self.syncs += 1
+        if not self.free:
+            return                  # every pinned word still waits for its copy: this sync goes unreported
+        slot = self.free.pop()
+        self.host[slot:slot + 1].copy_(self.counter, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self.pending.append((event, slot, self.syncs))
+
+
 class JobBatch:
     """An ordered list of mq_job records plus the tensors they reference."""
 
@@ -28,6 +72,9 @@ class JobBatch:
         self._records: list[tuple] = []
         self._keep: list[torch.Tensor] = []
         self._array = None
+        self._array_plain = None   # the same list without MQ_NVFP4_CARRY_AMAX (see carry_amax)
+        self._feedback: _AmaxFeedback | None = None
+        self.last_form = None      # "carried" / "plain": the form of the newest submission of a list with carried amax
         self._table = None      # device copy of the launch descriptors (see freeze)
         self.device = None
         self.direct_calls = 0   # kernels launched inside the block without going through the job list
@@ -59,13 +106,14 @@ class JobBatch:
             self._keep = list(keep)
         self._array = None
 
-    def carry_amax(self) -> int:
+    def carry_amax(self, adaptive: bool = True) -> int:
         """After this list has run once: let later runs of the same list quantize NVFP4 and per-tensor FP8 tensors in
         one pass with the amax their record kept from the run before (MQ_NVFP4_CARRY_AMAX; the driver checks the amax on
         the way and quantizes a tensor again if it moved, so results do not change).  NVFP4 jobs are only flagged when
         every one of the list is one the packed kernels take (bf16, 16-byte aligned input, 4-byte aligned codes), so
         that every record goes through the same driver path on every run; per-tensor FP8 jobs always are.
-        Returns the number of jobs flagged."""
+        With `adaptive` the batch also watches how many records moved per sync (`_AmaxFeedback`) and submits the plain
+        two-pass form while most of them keep moving.  Returns the number of jobs flagged."""
         nv = [r for r in self._records if r[self.KIND] == _lib.JOB_NVFP4]
         nv_fit = bool(nv) and all(r[self.DTYPE] == _lib.DTYPE_CODE[torch.bfloat16] and (r[self.IN] or 0) % 16 == 0
                                   and (r[self.OUT] or 0) % 4 == 0 and r[self.COLS] % 16 == 0 for r in nv)
@@ -75,6 +123,10 @@ class JobBatch:
             self._records = [r[: self.P1] + (r[self.P1] | _lib.NVFP4_CARRY_AMAX,) + r[self.P1 + 1:]
                              if r[self.KIND] in kinds else r for r in self._records]
             self._array = None
+            self._array_plain = None
+            if adaptive and self.device is not None and self.device.type == "cuda":
+                records = len({r[self.AUX] for r in self._records if r[self.KIND] in kinds})
+                self._feedback = _AmaxFeedback(self.device, records)
         return flagged
 
     def amax_records(self) -> list[torch.Tensor]:
@@ -110,6 +162,7 @@ class JobBatch:
             for i, rec in enumerate(self._records):
                 arr[i] = _lib.Job(*rec)
             self._array = arr
+            self._array_plain = None
             self._table = None
             if self.device is not None and sum(r[self.KIND] in self._TABLE_KINDS for r in self._records) > _lib.MAX_GROUP:
                 host = torch.empty(len(self._records) * _lib.TABLE_ENTRY_BYTES, dtype=torch.uint8)
@@ -132,11 +185,33 @@ class JobBatch:
         if stop <= start:
             return
         arr = self.freeze()
+        current = _lib.stream_ptr(self.device)
         if stream is None:
-            stream = _lib.stream_ptr(self.device)
+            stream = current
+        # the feedback copy and its event go to torch's current stream: only a submission on that stream is watched
+        feedback = self._feedback if stream == current else None
+        if feedback is not None:
+            if start == 0:
+                self.last_form = "plain" if feedback.decide() else "carried"
+            if self.last_form == "plain":
+                arr = self._plain_array()
         ptr = ctypes.byref(arr, start * ctypes.sizeof(_lib.Job))
         table = None if self._table is None else self._table.data_ptr() + start * _lib.TABLE_ENTRY_BYTES
-        _lib.check(_lib.load().mq_run_jobs_tabled(ptr, stop - start, table, stream))
+        counter = None if feedback is None else feedback.counter.data_ptr()
+        _lib.check(_lib.load().mq_run_jobs_feedback(ptr, stop - start, table, counter, stream))
+        if feedback is not None and stop == len(self._records):
+            feedback.submitted()
+
+    def _plain_array(self):
+        """The job list without the carried-amax flag (same records, same device table)."""
+        if self._array_plain is None:
+            arr = (_lib.Job * len(self._records))()
+            for i, rec in enumerate(self._records):
+                if rec[self.KIND] in (_lib.JOB_NVFP4, _lib.JOB_FP8_TENSOR):
+                    rec = rec[: self.P1] + (rec[self.P1] & ~_lib.NVFP4_CARRY_AMAX,) + rec[self.P1 + 1:]
+                arr[i] = _lib.Job(*rec)
+            self._array_plain = arr
+        return self._array_plain
 
     def input_pointers(self) -> list[int]:
         return [rec[2] for rec in self._records]

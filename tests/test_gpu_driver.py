@@ -1266,3 +1266,23 @@ def test_amax_quantizers_over_a_device_table_first_run_carried_and_moved(oracle,
     check("settled")
     redo = torch.stack([r[_lib.RECORD_REDO_WORD] for r in batch.amax_records()]).cpu()
     assert int(redo.sum()) == 0
+    assert batch.last_form == "carried"
+    # Every amax moves on every sync: once the batch has seen that (the count of moved records comes back with the
+    # sync after), it submits the plain two-pass form, and returns to the carried one when the amaxes hold still.
+    factor = 2.0
+    forms = []
+    for step in range(4):
+        for w in dev:
+            w.mul_(factor)
+        for pair in pairs_dev if pair_outs else []:
+            pair[0].mul_(factor)
+        factor = 1.0 / factor
+        check(f"every amax moved, sync {step}")
+        forms.append(batch.last_form)
+    assert forms[0] == "carried" and forms[-1] == "plain" and "plain" in forms[1:3], forms
+    check("held still, reported by the plain form")
+    assert batch.last_form == "plain"
+    check("carried again")
+    assert batch.last_form == "carried"
+    check("and still")
+    assert batch.last_form == "carried"
