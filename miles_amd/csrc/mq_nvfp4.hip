@@ -181,7 +181,11 @@ __device__ __forceinline__ NvCandidate nv_candidate(const float f[8], float s_hp
     NvCandidate c;
     c.sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
     c.s_f = hw_e4m3x2_decode<false>(c.sc).x;
-    const float inv = __builtin_fminf(1.0f / (c.s_f * s_dec), kFltMax);
+    // the refined hardware reciprocal where it equals the division, decided for the wavefront (see nvfp4_quant_units)
+    const float d = c.s_f * s_dec;
+    float inv;
+    if (__builtin_amdgcn_ballot_w64(!shared_div_ok(d)) == 0) inv = recip_shared(d);
+    else inv = __builtin_fminf(1.0f / d, kFltMax);
     c.word = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
     c.word = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, c.word);
     c.word = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, c.word);
@@ -247,7 +251,10 @@ __device__ __forceinline__ float nv_pair_error(const float term[8], bool odd_lan
 template <int EM, bool FASTDIV>
 __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float bmax, float amax, const NvScales& gs,
                                                         float denom, bool odd_lane) {
-    const float s6_hp = (bmax / 6.0f) * gs.enc;
+    // bmax / 6: a bf16 numerator and a shared divisor, so the three-instruction sequence gives the IEEE quotient
+    // wherever its intermediates stay normal (decided for the wavefront; zero blocks and extreme maxima divide)
+    const bool plain_bmax = shared_div_ok(bmax);
+    const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate c4 = nv_candidate(f, s4_hp, gs.s_dec), c6 = nv_candidate(f, s6_hp, gs.s_dec);
     float t4[8], t6[8];
