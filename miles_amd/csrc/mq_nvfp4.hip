@@ -203,11 +203,14 @@ __device__ __forceinline__ void nv_decode8(uint32_t word, float q[8]) {
 // out as +0 whatever its sign: no error term can see that).  The numerators here are RN(RN(value * f32(scale)) * amax)
 // with value * f32(scale) either zero or in 2^-10 .. 2688, so one test of the tensor amax covers every element:
 // nv_fast_division(amax) allows the sequence for the whole tensor, otherwise every quotient is the IEEE division.
-__device__ __forceinline__ bool nv_fast_division(float amax) {
+// 0: IEEE divisions; 1: the sequence; 2: the sequence, and the amax has at most 12 significant bits (the amax of a bf16 or
+// fp16 tensor has), so that value x f32(scale) x amax -- 2, 4 and 12 bits -- is exact in whatever order it is taken
+__device__ __forceinline__ int nv_fast_division(float amax) {
     const uint32_t e = f2u(amax) & 0x7F800000u;
-    return e >= 0x17800000u /* 2^-80 */ && e <= 0x65800000u /* 2^76 */;
+    if (!(e >= 0x17800000u /* 2^-80 */ && e <= 0x65800000u /* 2^76 */)) return 0;
+    return (f2u(amax) & 0xFFFu) == 0 ? 2 : 1;
 }
-template <bool FASTDIV>
+template <int FASTDIV>
 __device__ __forceinline__ float div_by_numer(float x, float d, float y) {
     if (!FASTDIV) return x / d;
     const float q0 = x * y;
@@ -215,12 +218,14 @@ __device__ __forceinline__ float div_by_numer(float x, float d, float y) {
     return __builtin_fmaf(r, y, q0);
 }
 // error terms of this lane's eight elements; EM bit 0: squared error, bit 1: fp16 candidate error
-template <int EM, bool FASTDIV>
+template <int EM, int FASTDIV>
 __device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandidate& c, float amax, float enc, float denom,
                                                float term[8]) {
     float q[8];
     nv_decode8(c.word, q);
     const float denom_inv = 1.0f / denom;
+    // FASTDIV 2: every partial product of value x f32(scale) x amax is exact, one multiplication per element
+    const float scale_amax = c.s_f * amax;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         float diff;
@@ -230,7 +235,7 @@ __device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandida
             asm volatile("" : "+v"(hf));                          // keep the fp16 product a value of its own
             diff = hf - f[j] * enc;
         } else {
-            diff = div_by_numer<FASTDIV>((q[j] * c.s_f) * amax, denom, denom_inv) - f[j];
+            diff = div_by_numer<FASTDIV>(FASTDIV == 2 ? q[j] * scale_amax : (q[j] * c.s_f) * amax, denom, denom_inv) - f[j];
         }
         term[j] = (EM & 1) ? diff * diff : __builtin_fabsf(diff);
     }
@@ -248,7 +253,7 @@ __device__ __forceinline__ float nv_pair_error(const float term[8], bool odd_lan
     return odd_lane ? seeded : partner_total;
 }
 // the winning candidate for this lane's block; bmax is the block amax (pair-uniform)
-template <int EM, bool FASTDIV>
+template <int EM, int FASTDIV>
 __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float bmax, float amax, const NvScales& gs,
                                                         float denom, bool odd_lane) {
     // bmax / 6: a bf16 numerator and a shared divisor, so the three-instruction sequence gives the IEEE quotient
@@ -292,7 +297,7 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
     gs.s_dec = u2f(amax_bits[kRecSDec]);
     gs.enc = u2f(amax_bits[kRecEnc]);
     const float amax = u2f(amax_bits[kRecAmax]);
-    const bool fastdiv = nv_fast_division(amax);
+    const int fastdiv = nv_fast_division(amax);
     uint32_t seen = 0;
 #pragma unroll
     for (int i = 0; i < kNvUnroll; i++) {
@@ -307,8 +312,9 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
         uint32_t sc, word;
         if (FOS) {
             constexpr int EM = FOS > 0 ? FOS - 1 : 0;
-            const NvCandidate c = fastdiv ? nv_four_over_six<EM, true>(f, bmax, amax, gs, denom, (t & 1) != 0)
-                                          : nv_four_over_six<EM, false>(f, bmax, amax, gs, denom, (t & 1) != 0);
+            const NvCandidate c = fastdiv == 2   ? nv_four_over_six<EM, 2>(f, bmax, amax, gs, denom, (t & 1) != 0)
+                                  : fastdiv == 1 ? nv_four_over_six<EM, 1>(f, bmax, amax, gs, denom, (t & 1) != 0)
+                                                 : nv_four_over_six<EM, 0>(f, bmax, amax, gs, denom, (t & 1) != 0);
             sc = c.sc;
             word = c.word;
         } else if (mb < 0x7F80u && s_hp == s_hp) {
@@ -491,8 +497,10 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* _
     float s_f, q[8];
     if (FOS) {
         constexpr int EM = FOS > 0 ? FOS - 1 : 0;
-        const NvCandidate c = nv_fast_division(amax) ? nv_four_over_six<EM, true>(f, bmax, amax, gs, numer, (t & 1) != 0)
-                                                     : nv_four_over_six<EM, false>(f, bmax, amax, gs, numer, (t & 1) != 0);
+        const int fastdiv = nv_fast_division(amax);
+        const NvCandidate c = fastdiv == 2   ? nv_four_over_six<EM, 2>(f, bmax, amax, gs, numer, (t & 1) != 0)
+                              : fastdiv == 1 ? nv_four_over_six<EM, 1>(f, bmax, amax, gs, numer, (t & 1) != 0)
+                                             : nv_four_over_six<EM, 0>(f, bmax, amax, gs, numer, (t & 1) != 0);
         s_f = c.s_f;
         nv_decode8(c.word, q);
     } else if (m < 0x7F800000u && s_hp == s_hp) {

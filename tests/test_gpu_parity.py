@@ -979,6 +979,12 @@ def test_nvfp4_four_over_six_qdq_and_other_dtypes(oracle, monkeypatch, dtype, e4
     assert cfg.use_4over6 and cfg.e4m3_max == e4m3_max and cfg.error_use_fast_math == fp16 and cfg.error_mode.name == mode
     got = m.fused_nvfp4_qdq(x.to(DEV), m.compute_nvfp4_amax(x.to(DEV)), cfg)
     _assert_same(got, oracle.fused_nvfp4_qdq(x, e4m3_max=e4m3_max, flags=flags), "dequantized values")
+    # an amax handed in from elsewhere (a calibrated one, say) may use all 24 bits of its mantissa: value x scale x amax is
+    # then no longer exact in any order, and the kernel keeps the reference's order of the two multiplications
+    wide = torch.tensor(float(x.abs().max()) * 1.0001234, dtype=torch.float32)
+    assert int(wide.view(torch.int32)) & 0xFFF
+    got = m.fused_nvfp4_qdq(x.to(DEV), wide.to(DEV), cfg)
+    _assert_same(got, oracle.fused_nvfp4_qdq(x, amax=wide, e4m3_max=e4m3_max, flags=flags), "dequantized values (24-bit amax)")
     # fp16 / fp32 weights take the one-lane-per-block quantizer kernel
     xf = x.float() if dtype == torch.float16 else x.half()
     q, s, g = nvfp4_quantize_1d(xf.to(DEV))
