@@ -292,12 +292,15 @@ int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table);
 int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, void* stream);
 
-/* mq_run_jobs_tabled that also reports how many amax records moved (no counterpart in the reference).  Every fold of an
- * NVFP4 or per-tensor FP8 amax record made by the call adds 1 to *device_moved (a uint32 in device memory that the call
- * never clears) if the record held another amax before.  A caller that re-submits one job list reads the counter some
- * time later (an asynchronous copy; nothing waits for it) and, when most records keep moving from one submission to
- * the next -- where MQ_NVFP4_CARRY_AMAX costs a second pass over every tensor -- submits the list without the flag
- * until they hold still again; the records stay valid for either form.  device_table and device_moved may be NULL. */
+/* mq_run_jobs_tabled that also reports how many amax records moved (no counterpart in the reference).  device_moved
+ * points to four uint32 in device memory.  Words 0 and 1 are counters that the call never clears: every fold of NVFP4
+ * or per-tensor FP8 amax records made by the call adds the number of tensors it folded to word 1, and to word 0 the
+ * number of those whose record held another amax before.  Words 2 and 3 are the low and the high half of an address
+ * (0 = none) of two uint32 in host-visible memory (pinned, mapped) that every fold launch first refreshes with the
+ * counters as the launches before it left them, so that the host can read them at any time without a copy, an event or
+ * a wait.  When most tensors keep moving from one submission to the next -- where MQ_NVFP4_CARRY_AMAX costs a second
+ * pass over every such tensor -- the caller submits the list without the flag until they hold still again; the
+ * records stay valid for either form.  device_table and device_moved may be NULL. */
 int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved, void* stream);
 
 /* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the

@@ -25,6 +25,7 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, f
     __shared__ uint32_t lds4[4];
     const FlatJob& job = tab.job[blockIdx.x];
     uint32_t* rec = (uint32_t*)job.aux;
+    amax_feedback_folded(moved_counter, gridDim.x);
     uint32_t m = rec[threadIdx.x];
     rec[threadIdx.x] = 0;
     m = wave_max(m);
@@ -38,11 +39,11 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, f
             const bool moved = rec[kRecAmax] != m;
             rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;
             rec[kRecVolatile] = moved ? 1u : 0u;
-            amax_feedback(moved_counter, moved);
+            amax_feedback(moved_counter, moved, 1u);
         } else {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
-            amax_feedback(moved_counter, rec[kRecAmax] != m);
+            amax_feedback(moved_counter, rec[kRecAmax] != m, 1u);
         }
         rec[kRecAmax] = m;
         float amax = u2f(m);

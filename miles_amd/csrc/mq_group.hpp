@@ -209,10 +209,24 @@ constexpr int kRecordSections = 4;      // MQ_NVFP4_SECTIONS
 constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (float bits)
 constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
 constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last run: the next carried run collects the amax first
-// A fold launched by the job driver also tells its caller how many records held another amax before (a counter in
-// device memory that only ever grows): a caller whose every amax keeps moving can then submit the plain two-pass form.
-__device__ __forceinline__ void amax_feedback(uint32_t* counter, bool moved) {
-    if (counter && moved) atomicAdd(counter, 1u);
+// A fold launched by the job driver also tells its caller how many tensors' records held another amax before, and how
+// many tensors it folded (two counters in device memory that only ever grow: a copy taken at any time gives a
+// consistent rate): a caller whose every amax keeps moving can then submit the plain two-pass form.
+__device__ __forceinline__ void amax_feedback(uint32_t* counter, bool moved, uint32_t tensors) {
+    if (counter && moved) atomicAdd(counter, tensors);
+}
+// Once per fold launch: first the two counters as the launches before left them (a consistent pair) go to the caller's
+// host-visible mirror, if it named one in words 2 and 3, then this launch's tensors are added to the second counter.
+__device__ __forceinline__ void amax_feedback_folded(uint32_t* counter, uint32_t tensors) {
+    if (counter && blockIdx.x == 0 && threadIdx.x == 0) {
+        volatile uint32_t* mirror = (volatile uint32_t*)(((uint64_t)counter[3] << 32) | counter[2]);
+        if (mirror) {
+            const uint32_t moved = atomicAdd(counter, 0u), folded = atomicAdd(counter + 1, 0u);
+            mirror[0] = moved;
+            mirror[1] = folded;
+        }
+        atomicAdd(counter + 1, tensors);
+    }
 }
 
 struct CopyJob {      // rows of `bytes` bytes each (one row: a plain run), chunks_per_row chunks of the copy kernel per row

@@ -129,6 +129,7 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float 
     const int ji = blockIdx.x;
     const FlatJob& job = tab.job[ji];
     const int sections = MODE == 0 ? job.section : job.pad;
+    if (MODE != 0) amax_feedback_folded(moved_counter, gridDim.x);
     if (MODE != 0 && job.section != job.pad - 1) return;
     uint32_t* rec = (uint32_t*)job.aux;
     uint32_t m = 0;
@@ -146,11 +147,11 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float 
                                  rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
             rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;     // a volatile record has no codes yet
             rec[kRecVolatile] = moved ? 1u : 0u;
-            amax_feedback(moved_counter, moved);
+            amax_feedback(moved_counter, moved, (uint32_t)sections);
         } else if (MODE == 1) {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
-            amax_feedback(moved_counter, rec[kRecAmax] != f2u(amax));
+            amax_feedback(moved_counter, rec[kRecAmax] != f2u(amax), (uint32_t)sections);
         }
         rec[kRecAmax] = f2u(amax);
         rec[kRecEncSixth] = f2u(gs.enc_sixth);

@@ -373,7 +373,7 @@ extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) { return
 
 extern "C" int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved,
                                     void* stream) {
-    if ((uintptr_t)device_moved % 4 != 0) return mq_fail(MQ_ERR_ARG, "feedback counter must be 4-byte aligned");
+    if ((uintptr_t)device_moved % 4 != 0) return mq_fail(MQ_ERR_ARG, "feedback counters must be 4-byte aligned");
     mq_set_amax_feedback(device_moved);
     const int rc = mq_run_jobs_tabled(jobs, n, device_table, stream);
     mq_set_amax_feedback(nullptr);

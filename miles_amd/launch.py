@@ -10,7 +10,6 @@ launch-bound without changing the per-tensor call signatures.
 
 from __future__ import annotations
 
-import collections
 import contextlib
 import ctypes
 import threading
@@ -23,46 +22,31 @@ _state = threading.local()
 
 
 class _AmaxFeedback:
-    """How many amax records moved in the syncs already finished, read without ever waiting for the GPU.
+    """What share of the amax records moved in the syncs the GPU has finished, read without ever waiting for it.
 
-    The folds of a `mq_run_jobs_feedback` call add to a device counter that only grows; after each whole submission the
-    counter is copied into one of a few pinned words and an event is recorded.  At the start of the next submission the
-    copies that have arrived are read: when more than half of the records moved per sync, the list is submitted in
-    the plain two-pass form (the carried-over amax would cost every such tensor a second pass), until they hold again.
-    A host that runs ahead of the GPU simply keeps its last decision."""
+    The folds of a `mq_run_jobs_feedback` call add to two device counters that only grow -- tensors whose record held
+    another amax before, and tensors folded -- and every fold launch first mirrors the pair into two pinned words, so the
+    host reads them with no copy, no event and no wait.  At the start of a submission: when more than half of the tensors
+    folded since the last reading had moved, the list is submitted in the plain two-pass form (the carried-over amax
+    would cost every such tensor a second pass), until they hold again."""
 
-    SLOTS = 8
-
-    def __init__(self, device, records: int) -> None:
-        self.counter = torch.zeros(1, dtype=torch.int32, device=device)
-        self.host = torch.zeros(self.SLOTS, dtype=torch.int32).pin_memory()
-        self.pending: collections.deque = collections.deque()     # (event, pinned slot, index of the sync it closes)
-        self.free = list(range(self.SLOTS))
-        self.records = records
-        self.syncs = 0
-        self.seen = (0, 0)          # (sync index, counter value) of the newest copy that was read
+    def __init__(self, device) -> None:
+        self.mirror = torch.zeros(2, dtype=torch.int32).pin_memory()
+        self.mirror_words = self.mirror.numpy()       # the same pinned words, read without going through torch
+        address = self.mirror.data_ptr()
+        words = [0, 0, address & 0xFFFFFFFF, address >> 32]
+        self.counter = torch.tensor([w - (1 << 32) if w >= 1 << 31 else w for w in words], dtype=torch.int32).to(device)
+        self.seen = (0, 0)          # the counters as of the last reading that had new folds
         self.plain = False
 
     def decide(self) -> bool:
-        while self.pending and self.pending[0][0].query():
-            _event, slot, index = self.pending.popleft()
-            total = int(self.host[slot]) & 0xFFFFFFFF
-            moved = (total - self.seen[1]) & 0xFFFFFFFF
-            syncs = index - self.seen[0]
-            self.seen = (index, total)
-            self.free.append(slot)
-            self.plain = moved * 2 > self.records * syncs
+        moved_total, folded_total = (int(v) & 0xFFFFFFFF for v in self.mirror_words)
+        folded = (folded_total - self.seen[1]) & 0xFFFFFFFF
+        if folded:
+            moved = (moved_total - self.seen[0]) & 0xFFFFFFFF
+            self.seen = (moved_total, folded_total)
+            self.plain = moved * 2 > folded
         return self.plain
-
-    def submitted(self) -> None:
-        self.syncs += 1
-        if not self.free:
-            return                  # every pinned word still waits for its copy: this sync goes unreported
-        slot = self.free.pop()
-        self.host[slot:slot + 1].copy_(self.counter, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
-        self.pending.append((event, slot, self.syncs))
 
 
 class JobBatch:
@@ -125,8 +109,7 @@ class JobBatch:
             self._array = None
             self._array_plain = None
             if adaptive and self.device is not None and self.device.type == "cuda":
-                records = len({r[self.AUX] for r in self._records if r[self.KIND] in kinds})
-                self._feedback = _AmaxFeedback(self.device, records)
+                self._feedback = _AmaxFeedback(self.device)
         return flagged
 
     def amax_records(self) -> list[torch.Tensor]:
@@ -185,11 +168,9 @@ class JobBatch:
         if stop <= start:
             return
         arr = self.freeze()
-        current = _lib.stream_ptr(self.device)
         if stream is None:
-            stream = current
-        # the feedback copy and its event go to torch's current stream: only a submission on that stream is watched
-        feedback = self._feedback if stream == current else None
+            stream = _lib.stream_ptr(self.device)
+        feedback = self._feedback
         if feedback is not None:
             if start == 0:
                 self.last_form = "plain" if feedback.decide() else "carried"
@@ -199,8 +180,6 @@ class JobBatch:
         table = None if self._table is None else self._table.data_ptr() + start * _lib.TABLE_ENTRY_BYTES
         counter = None if feedback is None else feedback.counter.data_ptr()
         _lib.check(_lib.load().mq_run_jobs_feedback(ptr, stop - start, table, counter, stream))
-        if feedback is not None and stop == len(self._records):
-            feedback.submitted()
 
     def _plain_array(self):
         """The job list without the carried-amax flag (same records, same device table)."""
