@@ -1209,6 +1209,31 @@ def test_stream_probes_run_and_refuse_bad_arguments():
     assert lib.mq_stream_probe(0, None, dst.data_ptr(), nbytes, 2, stream) != 0
 
 
+def test_amax_feedback_counters_through_the_c_abi():
+    """mq_run_jobs_feedback with the caller's own counter words and no host mirror: tensors folded and tensors whose
+    record held another amax before, summed over the calls."""
+    from miles_amd import launch
+    from miles_amd.tools.convert_hf_to_fp8 import tensor_fp8
+
+    ws = [W.gaussian_outliers((64, 256), std=0.02, p_outlier=0.0, gain=1.0, seed=9700 + i).to(DEV) for i in range(5)]
+    with launch.recording() as batch:
+        outs = [tensor_fp8(w) for w in ws]
+    arr = batch.freeze()
+    lib = _lib.load()
+    words = torch.zeros(4, dtype=torch.int32, device=DEV)
+    stream = _lib.stream_ptr(torch.device(DEV))
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
+    ws[2].mul_(2.0)
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    moved, folded, lo, hi = words.cpu().tolist()
+    # the records start out uninitialised, so every first fold may or may not count as moved; afterwards only tensor 2
+    assert folded == 15 and 1 <= moved <= 6 and lo == 0 and hi == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr() + 2, stream) != 0      # misaligned words
+    assert outs[0][0].dtype == torch.float8_e4m3fn
+
+
 @pytest.mark.parametrize("fmt", ["nvfp4", "tensor_fp8"])
 def test_amax_quantizers_over_a_device_table_first_run_carried_and_moved(oracle, fmt):
     """NVFP4 (pairs sharing a record and single tensors) and per-tensor FP8 with more jobs than one launch's kernel
