@@ -30,8 +30,41 @@ class _AmaxFeedback:
     folded since the last reading had moved, the list is submitted in the plain two-pass form (the carried-over amax
     would cost every such tensor a second pass), until they hold again."""
 
-    def __init__(self, device) -> None:
-        self.mirror = torch.zeros(2, dtype=torch.int32).pin_memory()
+    # The GPU writes the mirror words whenever a fold runs, possibly after the batch that named them is gone: they come
+    # from one pinned block that lives as long as the process and is never handed back to torch's host allocator.  A
+    # slot re-used while an old sync still runs can at worst mislead one choice between two forms with equal results.
+    _POOL_SLOTS = 1024
+    _pool = None
+    _pool_free: list[int] = []
+    _pool_lock = threading.Lock()
+
+    @classmethod
+    def _take_slot(cls):
+        with cls._pool_lock:
+            if cls._pool is None:
+                cls._pool = torch.zeros(cls._POOL_SLOTS, 2, dtype=torch.int32).pin_memory()
+                cls._pool_free = list(range(cls._POOL_SLOTS - 1, -1, -1))
+            return cls._pool_free.pop() if cls._pool_free else None
+
+    @classmethod
+    def create(cls, device):
+        """A watcher, or None when every mirror slot is taken (the batch then simply keeps the carried form)."""
+        slot = cls._take_slot()
+        return None if slot is None else cls(device, slot)
+
+    def __del__(self):
+        slot = getattr(self, "_slot", None)
+        if slot is not None:
+            try:
+                with self._pool_lock:
+                    self._pool_free.append(slot)
+            except Exception:       # interpreter shutdown
+                pass
+
+    def __init__(self, device, slot: int) -> None:
+        self._slot = slot
+        self.mirror = self._pool[slot]
+        self.mirror.zero_()
         self.mirror_words = self.mirror.numpy()       # the same pinned words, read without going through torch
         address = self.mirror.data_ptr()
         words = [0, 0, address & 0xFFFFFFFF, address >> 32]
@@ -109,7 +142,7 @@ class JobBatch:
             self._array = None
             self._array_plain = None
             if adaptive and self.device is not None and self.device.type == "cuda":
-                self._feedback = _AmaxFeedback(self.device)
+                self._feedback = _AmaxFeedback.create(self.device)
         return flagged
 
     def amax_records(self) -> list[torch.Tensor]:
