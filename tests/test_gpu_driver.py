@@ -258,7 +258,7 @@ def test_moe_mxfp8_sync(oracle):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} round {round_}")
+            _same(g, w, f"{n} sync {sync_}")
         cpu = _moe_model(31)
         for k in dev:
             dev[k].copy_(cpu[k])
@@ -269,14 +269,14 @@ def test_moe_nvfp4_sync_pairs_share_amax(oracle):
     dev = {k: v.to(DEV) for k, v in cpu.items()}
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="deepseekv3",
                         quantization_config={"quant_method": "modelopt", "quant_algo": "NVFP4"}, send_bucket=None)
-    # round 0 records the plan (amax pass + quantize pass); later rounds replay it with the amax carried over: round 1 on
-    # new weights (every amax moved), round 2 on the same weights (none moved), round 3 with one expert's amax moved
+    # sync 0 records the plan (amax pass + quantize pass); later syncs replay it with the amax carried over: sync 1 on
+    # new weights (every amax moved), sync 2 on the same weights (none moved), sync 3 with one expert's amax moved
     changed = _moe_model(41)
     one_moved = {k: v.clone() for k, v in changed.items()}
     moved_name = next(k for k in one_moved if "linear_fc1" in k)
     one_moved[moved_name].mul_(2.0)
-    rounds = [cpu, changed, changed, one_moved]
-    for round_, cpu in enumerate(rounds):
+    syncs = [cpu, changed, changed, one_moved]
+    for sync_, cpu in enumerate(syncs):
         for k in dev:
             dev[k].copy_(cpu[k])
         flat = [nt for b in _run(upd) for nt in b]
@@ -295,7 +295,7 @@ def test_moe_nvfp4_sync_pairs_share_amax(oracle):
                 want += hf
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} round {round_}")
+            _same(g, w, f"{n} sync {sync_}")
     assert upd._plan.replayable
     assert any(r[upd._plan.batch.P1] & 8 for r in upd._plan.batch.records), "replays should carry the amax over"
 
@@ -347,7 +347,7 @@ def test_moe_int4_asymmetric_sync_is_planned_and_replayed(oracle, packed):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} round {round_}")
+            _same(g, w, f"{n} sync {sync_}")
         cpu = _moe_model(56 + round_)
         for k in dev:
             dev[k].copy_(cpu[k])
@@ -612,7 +612,7 @@ def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} round {round_}")
+            _same(g, w, f"{n} sync {sync_}")
         if round_ != 1:             # rounds 1 and 2 see the same weights: no amax moves between them
             cpu = _dense_model(63 + round_)
             for k in dev:
