@@ -258,7 +258,7 @@ def test_moe_mxfp8_sync(oracle):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} sync {sync_}")
+            _same(g, w, f"{n} sync {round_}")
         cpu = _moe_model(31)
         for k in dev:
             dev[k].copy_(cpu[k])
@@ -347,7 +347,7 @@ def test_moe_int4_asymmetric_sync_is_planned_and_replayed(oracle, packed):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} sync {sync_}")
+            _same(g, w, f"{n} sync {round_}")
         cpu = _moe_model(56 + round_)
         for k in dev:
             dev[k].copy_(cpu[k])
@@ -612,7 +612,7 @@ def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
                     want.append((hf, t))
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
-            _same(g, w, f"{n} sync {sync_}")
+            _same(g, w, f"{n} sync {round_}")
         if round_ != 1:             # rounds 1 and 2 see the same weights: no amax moves between them
             cpu = _dense_model(63 + round_)
             for k in dev:
