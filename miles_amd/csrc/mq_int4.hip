@@ -678,8 +678,16 @@ __global__ __launch_bounds__(256) void int4_unpack_kernel(const uint32_t* __rest
             f[2 * k] = ((float)((ev >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
             f[2 * k + 1] = ((float)((od >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
         }
-        if (i < words)
-            st16(y + i * 8, u32x4{hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])});
+        u32x4 o = {hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])};
+        // A NaN or infinite scale (decided for the wavefront): the products may be NaN -- the scale's own, or 0 x inf --
+        // and the reference's rounding to bf16 writes the one quiet NaN 0x7FC0 whatever the sign and the payload.
+        if (__builtin_amdgcn_ballot_w64((f2u(s[u]) & 0x7F800000u) == 0x7F800000u) != 0) {
+            uint32_t h[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) h[k] = f[k] != f[k] ? 0x7FC0u : hw_bf16x2(f[k], 0.0f) & 0xFFFFu;
+            o = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+        }
+        if (i < words) st16(y + i * 8, o);
     }
 }
 // any K (rows padded to whole words), any group size, any scale dtype: one lane per element

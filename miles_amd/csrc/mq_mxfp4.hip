@@ -268,6 +268,8 @@ __global__ __launch_bounds__(256) void mxfp4_to_fp8_kernel(const RecodeTable tab
             o[2 * j] = hw_e4m3x4(a.x * factor, a.y * factor, b.x * factor, b.y * factor);
             o[2 * j + 1] = hw_e4m3x4(cc.x * factor, cc.y * factor, d.x * factor, d.y * factor);
         }
+        // a NaN scale byte anywhere in the tile makes the tile scale, every offset and every product NaN: code 0x7F
+        if (smax == 255u) o[0] = o[1] = o[2] = o[3] = 0x7F7F7F7Fu;
         if (ok) st16(y + row * in_dim + pj * 256 + c * 16, u32x4{o[0], o[1], o[2], o[3]});
     }
 }
@@ -332,6 +334,8 @@ __global__ __launch_bounds__(256) void mxfp4_recode_flat_kernel(const RecodeTabl
         o[2 * j] = hw_e4m3x4(a.x * factor, a.y * factor, b.x * factor, b.y * factor);
         o[2 * j + 1] = hw_e4m3x4(cc.x * factor, cc.y * factor, d.x * factor, d.y * factor);
     }
+    // a NaN scale byte anywhere in the tile makes the tile scale, every offset and every product NaN: code 0x7F
+    if (smax == 255u) o[0] = o[1] = o[2] = o[3] = 0x7F7F7F7Fu;
     st16(job.y + (uint64_t)u * 16, u32x4{o[0], o[1], o[2], o[3]});
 }
 

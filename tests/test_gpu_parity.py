@@ -382,6 +382,12 @@ def test_int4_unpack_dequant(oracle, shape, G, sdt):
     m, k = shape
     packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
     scale = torch.exp(torch.randn((m, k // G), generator=g) * 3).to(sdt)
+    # non-finite scales: the reference's rounding to bf16 writes the one quiet NaN 0x7FC0 for any NaN (and for 0 x inf)
+    flat = scale.view(-1)
+    if flat.numel() >= 4:
+        flat[0], flat[1], flat[2] = float("nan"), float("inf"), float("-inf")
+        if sdt == torch.bfloat16:
+            flat.view(torch.int16)[3] = -42        # a NaN with a sign and a payload
     got = _dequantize_tensor(packed.to(DEV), scale.to(DEV), torch.tensor(shape, dtype=torch.int32), G)
     want = oracle.int4_unpack_dequant(packed, scale, shape, G)
     assert got.dtype == torch.bfloat16
@@ -542,7 +548,8 @@ def test_mxfp4_grouped_jobs(oracle):
 
 
 @pytest.mark.parametrize("shape,lo,hi", [((128, 128), 100, 140), ((256, 384), 120, 128), ((128, 256), 0, 30),
-                                         ((128, 128), 225, 255), ((2048, 7168), 110, 135)])
+                                         ((128, 128), 225, 255), ((2048, 7168), 110, 135),
+                                         ((256, 512), 250, 256), ((256, 256), 0, 256)])      # with the NaN byte 255
 def test_mxfp4_to_fp8_recode(oracle, shape, lo, hi):
     from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
 
