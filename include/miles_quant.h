@@ -231,6 +231,8 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
+ * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2) run their tuned 128x128 kernel on bf16 and on
+ * fp16 inputs; consecutive jobs share a launch when they also share the input dtype.
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
  * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list.
  * MQ_NVFP4_CARRY_AMAX in p1 of NVFP4 and FP8_TENSOR jobs (no counterpart in the reference): a caller that submits the
@@ -268,7 +270,8 @@ typedef struct mq_job {
     int32_t p0, p1;
     /* FP8 quantizers only: the input rows come in blocks of rows_per_block consecutive rows (stride ld) whose
      * first rows are block_stride elements apart -- e.g. the q / k / v rows of a fused per-group QKV weight,
-     * read in place.  0 / 0 = one block (plain matrix).  rows_per_block must be a multiple of the tile height. */
+     * read in place.  0 / 0 = one block (plain matrix).  rows_per_block must be a multiple of the tile height,
+     * the input bf16 or fp16. */
     int64_t rows_per_block, block_stride;
 } mq_job;
 /* Consecutive jobs of one kind (and, for the flat kernels, of similar size) are fused into launches of up to

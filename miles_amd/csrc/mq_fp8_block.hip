@@ -9,7 +9,7 @@
 //                                .../processors/quantizer_fp8.py:139-147); restated from its published source
 //   dequant y = bf16(float(q) * s[i/B][j/B])                            (reference: tools/fp8_cast_bf16.py:15-40)
 //
-// Fast path (bf16, 128x128 tiles, 16-byte aligned rows): one 512-lane workgroup (eight wavefronts) owns one tile.
+// Fast path (bf16 or fp16, 128x128 tiles, 16-byte aligned rows): one 512-lane workgroup (eight wavefronts) owns one tile.
 // Lane t loads four 16-byte row segments (rows t/16 + 32 i, columns 8 (t%16) ..+8) so that sixteen lanes read one
 // contiguous 256-byte tile row; the 32 values stay in registers, the tile amax is reduced with DPP inside each
 // wavefront and through eight LDS words across the wavefronts, and the tile is quantized from registers:
@@ -62,8 +62,22 @@ __device__ __forceinline__ TilePick pick_tile(const TileRef& tab) {
     const int32_t tiles = ((job.M + kTile - 1) / kTile) * ((job.K + kTile - 1) / kTile);
     return TilePick{(int32_t)blockIdx.y, xcd_contiguous_item(tiles)};
 }
-template <int MODE, class Table>
+// A 16-bit element of the input as a float: a bf16 is the upper half of the float, an fp16 goes through the converter
+// (exact, subnormals included).  The absolute bit patterns of both formats order like the values they stand for, so
+// the tile maximum is taken on the patterns and converted once.
+template <int F16>
+__device__ __forceinline__ float elem_lo(uint32_t w) {
+    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+    return bf16_lo(w);
+}
+template <int F16>
+__device__ __forceinline__ float elem_hi(uint32_t w) {
+    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    return bf16_hi(w);
+}
+template <int MODE, class Table, int F16>
 __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table tab) {
+    constexpr uint32_t kInfBits = F16 ? 0x7C00u : 0x7F80u;      // pattern of +inf; anything above is a NaN
     __shared__ uint32_t wave_amax[kTileWaves];
     const TilePick pick = pick_tile(tab);
     if (pick.tile < 0) return;
@@ -131,7 +145,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
     m = 0;
 #pragma unroll
     for (int k = 0; k < kTileWaves; k++) m = umax(m, wave_amax[k]);
-    if (MODE != 0 && m >= 0x7F80u) {
+    if (MODE != 0 && m >= kInfBits) {
         // An infinity or a NaN in the tile (rare, and uniform over the workgroup).  Mode 1: Triton's max, maximum and
         // clamp return the operand that is not NaN, so the tile maximum skips NaN and a NaN product clamps to -448.
         // Mode 2: torch's amax hands a NaN on, 2^ceil(log2(.)) of inf / NaN is inf / NaN, and nothing clamps.
@@ -144,7 +158,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     const uint32_t lo = u[k] & 0x7FFFu, hi = (u[k] >> 16) & 0x7FFFu;
-                    mf = umax(mf, umax(lo > 0x7F80u ? 0u : lo, hi > 0x7F80u ? 0u : hi));
+                    mf = umax(mf, umax(lo > kInfBits ? 0u : lo, hi > kInfBits ? 0u : hi));
                 }
             }
             mf = wave_max(mf);
@@ -154,17 +168,17 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
             mf = 0;
 #pragma unroll
             for (int k = 0; k < kTileWaves; k++) mf = umax(mf, wave_amax[k]);
-            const float finite_max = u2f(mf << 16);
+            const float finite_max = elem_lo<F16>(mf);
             sx = (finite_max > 1e-10f ? finite_max : 1e-10f) / kFp8Max;
         } else {
-            sx = u2f(m > 0x7F80u ? 0x7FC00000u : 0x7F800000u);
+            sx = u2f(m > kInfBits ? 0x7FC00000u : 0x7F800000u);
         }
         const float yx = 1.0f / sx;
         if (t == 0) tile_scales[tile] = sx;
 #pragma unroll 1
         for (int i = 0; i < kRowsPerThread; i++) {
-            const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                                bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+            const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                                elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
             uint32_t c[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
@@ -178,7 +192,7 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
         }
         return;
     }
-    const float amax = u2f(m << 16);
+    const float amax = elem_lo<F16>(m);
 
     float s;
     if (MODE == 0) s = amax / kFp8Max;
@@ -198,8 +212,8 @@ __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table 
 
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; i++) {
-        float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                      bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                      elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             // |w/s| <= 448 (1 + 2^-22): no clamp is needed, the convert rounds anything up to 464 to 448
@@ -536,7 +550,7 @@ using namespace mq;
 bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, const void* q, int64_t M, int64_t K,
                          int bm, int bk) {
     // rows and columns below 2^24: a lane addresses its tile with 32-bit byte offsets from the tile's base
-    return dtype == MQ_BF16 && bm == kTile && bk == kTile && sxn == 1 && (K % 8) == 0 && (sxm % 8) == 0 &&
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && bm == kTile && bk == kTile && sxn == 1 && (K % 8) == 0 && (sxm % 8) == 0 &&
            ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 && M <= 0x7FFFFFFF && K < (1 << 24) && sxm > 0 &&
            sxm < (1 << 24);
 }
@@ -551,21 +565,32 @@ int64_t mq_fp8_tile_job_finish(TileJob& j) {
     return (int64_t)((j.M + kTile - 1) / kTile) * tiles_k;
 }
 
-// n finished descriptors in device memory; max_tiles: the largest tensor's tile count
-int mq_fp8_tile_launch_table(int mode, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st) {
+template <class Table>
+static void tile_launch(int mode, bool f16, dim3 grid, hipStream_t st, const Table& tab) {
+    const dim3 blk(kTileThreads);
+    if (f16) {
+        if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, Table, 1>), grid, blk, 0, st, tab);
+        else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, Table, 1>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((fp8_block128_kernel<2, Table, 1>), grid, blk, 0, st, tab);
+    } else {
+        if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, Table, 0>), grid, blk, 0, st, tab);
+        else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, Table, 0>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((fp8_block128_kernel<2, Table, 0>), grid, blk, 0, st, tab);
+    }
+}
+
+// n finished descriptors in device memory, all of one 16-bit dtype; max_tiles: the largest tensor's tile count
+int mq_fp8_tile_launch_table(int mode, int dtype, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st) {
     if (n == 0 || max_tiles == 0) return MQ_OK;
     const int64_t gx = xcd_grid(max_tiles);
     if (gx >= 0x7FFFFFF0) return mq_fail(MQ_ERR_ARG, "too many tiles");
-    const TileRef ref{device_jobs};
-    const dim3 grid((unsigned)gx, (unsigned)n), blk(kTileThreads);
-    if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, TileRef>), grid, blk, 0, st, ref);
-    else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, TileRef>), grid, blk, 0, st, ref);
-    else hipLaunchKernelGGL((fp8_block128_kernel<2, TileRef>), grid, blk, 0, st, ref);
+    tile_launch(mode, dtype == MQ_F16, dim3((unsigned)gx, (unsigned)n), st, TileRef{device_jobs});
     return mq_check_launch("fp8 block quant");
 }
 
-// tab.job[i] filled by the caller (w, q, scale, ldw, M, K, row blocks); fills the division constants and `end`, launches
-int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
+// tab.job[i] filled by the caller (w, q, scale, ldw, M, K, row blocks), all of one 16-bit dtype; fills the division
+// constants and `end`, launches
+int mq_fp8_tile_launch_group(int mode, int dtype, TileTable& tab, hipStream_t st) {
     int64_t tiles = 0;
     for (int i = 0; i < tab.n; i++) {
         tiles += mq_fp8_tile_job_finish(tab.job[i]);
@@ -574,10 +599,7 @@ int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st) {
     }
     if (tiles == 0) return MQ_OK;
     seal_table(tab);
-    const int64_t grid = xcd_grid(tiles);
-    if (mode == 0) hipLaunchKernelGGL((fp8_block128_kernel<0, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
-    else if (mode == 1) hipLaunchKernelGGL((fp8_block128_kernel<1, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
-    else hipLaunchKernelGGL((fp8_block128_kernel<2, TileTable>), dim3((unsigned)grid), dim3(kTileThreads), 0, st, tab);
+    tile_launch(mode, dtype == MQ_F16, dim3((unsigned)xcd_grid(tiles)), st, tab);
     return mq_check_launch("fp8 block quant");
 }
 
@@ -591,7 +613,7 @@ static int fp8_block_launch(int mode, const void* w, int dtype, int64_t sxm, int
         TileTable tab{};
         tab.n = 1;
         tab.job[0] = TileJob{w, q, scale, (int32_t)sxm, (int32_t)M, (int32_t)K, 0, 0, 0, 0, 0};
-        return mq_fp8_tile_launch_group(mode, tab, stream);
+        return mq_fp8_tile_launch_group(mode, dtype, tab, stream);
     }
     const int64_t tiles_m = (M + bm - 1) / bm, tiles_k = (K + bk - 1) / bk;
     const int64_t tiles = tiles_m * tiles_k;

@@ -17,9 +17,9 @@ using namespace mq;
 // grouped launchers implemented next to their kernels
 bool mq_fp8_tile_fast_ok(const void* w, int dtype, int64_t sxm, int64_t sxn, const void* q, int64_t M, int64_t K,
                          int bm, int bk);
-int mq_fp8_tile_launch_group(int mode, TileTable& tab, hipStream_t st);
+int mq_fp8_tile_launch_group(int mode, int dtype, TileTable& tab, hipStream_t st);
 int64_t mq_fp8_tile_job_finish(TileJob& j);
-int mq_fp8_tile_launch_table(int mode, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st);
+int mq_fp8_tile_launch_table(int mode, int dtype, const TileJob* device_jobs, int n, int64_t max_tiles, hipStream_t st);
 bool mq_fp8_dequant_fast_ok(const void* x, const void* y, int64_t M, int64_t N, int block);
 int mq_fp8_dequant_launch_group(const MqDequantArgs* a, int n, hipStream_t st);
 bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q);
@@ -116,8 +116,9 @@ static int check_job(const mq_job& j) {
     }
     if (j.rows_per_block != 0) {
         const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST || j.kind == MQ_JOB_FP8_BLOCK_POW2;
-        if (!fp8q || j.rows_per_block < 0 || j.rows_per_block % 128 != 0 || j.p0 != 128 || j.p1 != 128 || j.dtype != MQ_BF16)
-            return mq_fail(MQ_ERR_ARG, "row-blocked input needs a bf16 FP8 128x128 job with rows_per_block % 128 == 0");
+        if (!fp8q || j.rows_per_block < 0 || j.rows_per_block % 128 != 0 || j.p0 != 128 || j.p1 != 128 ||
+            (j.dtype != MQ_BF16 && j.dtype != MQ_F16))
+            return mq_fail(MQ_ERR_ARG, "row-blocked input needs a bf16 or fp16 FP8 128x128 job with rows_per_block % 128 == 0");
     }
     return MQ_OK;
 }
@@ -187,7 +188,8 @@ static FlatJob flat_entry(const mq_job& jb) {
 }
 
 static bool same_group(const mq_job& a, const mq_job& b) {
-    return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1;
+    // the tile kernels are compiled per 16-bit input dtype; the other kinds' fast paths take one dtype, or any (copies)
+    return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1 && (!tile_kind(a.kind) || a.dtype == b.dtype);
 }
 
 // Copy jobs of one launch run in no particular order: a job that reads what an earlier job of the group writes (a
@@ -428,7 +430,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
             // (tensors of 256 tiles and more fill a searched launch of 64 well enough, and run 1-2 % faster in that form)
             if (j - i > kMaxGroup && mx < 256) {
                 const int mode = head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2;
-                int rc = mq_fp8_tile_launch_table(mode, (const TileJob*)table + i, (int)(j - i), mx, st);
+                int rc = mq_fp8_tile_launch_table(mode, head.dtype, (const TileJob*)table + i, (int)(j - i), mx, st);
                 if (rc) return rc;
                 i = j;
                 continue;
@@ -458,7 +460,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                     const mq_job& jb = jobs[i + t];
                     tab.job[t] = tile_entry(jb);
                 }
-                rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2, tab, st);
+                rc = mq_fp8_tile_launch_group(head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2, head.dtype, tab, st);
                 break;
             }
             case MQ_JOB_FP8_DEQUANT: {

@@ -35,7 +35,7 @@ def fp8_blockwise_cast(x: torch.Tensor, block_size=None) -> tuple[torch.Tensor, 
     if x.dim() == 3:
         B, R, N = x.shape
         if not (x.stride(2) == 1 and x.stride(1) == N and R % 128 == 0 and (bm, bn) == (128, 128)
-                and x.dtype == torch.bfloat16):
+                and x.dtype in (torch.bfloat16, torch.float16)):
             return fp8_blockwise_cast(x.reshape(B * R, N), block_size)
         M = B * R
         y = torch.empty(M, N, device=x.device, dtype=fp8_dtype)
@@ -70,7 +70,7 @@ def per_block_cast_to_fp8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     rpb, bstride = 0, 0
     if x.dim() == 3:
         B, R, N = x.shape
-        if x.stride(2) == 1 and x.stride(1) == N and R % 128 == 0 and x.dtype == torch.bfloat16:
+        if x.stride(2) == 1 and x.stride(1) == N and R % 128 == 0 and x.dtype in (torch.bfloat16, torch.float16):
             rpb, bstride, M, ld = R, x.stride(0), B * R, N
         else:
             x = x.reshape(B * R, N)

@@ -105,10 +105,10 @@ def _split_qkv_weight(args, layer: str, param: torch.Tensor):
     q, k, v = torch.split(grouped, [q_per_group, 1, 1], dim=1)
     # opt-in of the batched sync driver: hand q / k / v on as [groups, rows, hidden] VIEWS of the fused weight; the
     # FP8 kernel reads the row blocks in place and the regrouping copy disappears.  Only the tuned kernel reads such
-    # views, and it takes contiguous bf16 storage that starts on a 16-byte boundary: a parameter carved out of a flat
-    # buffer at an odd offset, or of another dtype, is regrouped with copy jobs like everywhere else.
-    in_place = (getattr(args, "qkv_row_block_views", False) and param.dtype == torch.bfloat16 and param.is_contiguous()
-                and param.data_ptr() % 16 == 0)
+    # views, and it takes contiguous bf16 or fp16 storage that starts on a 16-byte boundary: a parameter carved out of
+    # a flat buffer at an odd offset, or held in fp32, is regrouped with copy jobs like everywhere else.
+    in_place = (getattr(args, "qkv_row_block_views", False) and param.dtype in (torch.bfloat16, torch.float16)
+                and param.is_contiguous() and param.data_ptr() % 16 == 0)
     if in_place:
         return [(f"model.layers.{layer}.self_attn.{n}_proj.weight", t.flatten(1, 2))
                 for n, t in (("q", q), ("k", k), ("v", v))]

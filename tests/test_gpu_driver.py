@@ -1087,14 +1087,17 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     check("without the table")
 
 
-@pytest.mark.parametrize("odd", ["offset", "fp16"])
+@pytest.mark.parametrize("odd", ["offset", "fp32", "fp16"])
 def test_fused_qkv_that_the_tuned_kernel_cannot_read_in_place_is_regrouped(oracle, odd):
     """Row-blocked q / k / v views are switched on per model, by shape.  A fused qkv parameter that starts two bytes into
-    a flat buffer, or a model held in fp16, is outside what the tile kernel reads in place: the name map regroups it
-    with copy jobs instead, and the sync stays correct and replayable."""
+    a flat buffer, or a model held in fp32, is outside what the tile kernel reads in place: the name map regroups it
+    with copy jobs instead, and the sync stays correct and replayable.  A model held in fp16 is read in place like a
+    bf16 one (the tile kernel has an fp16 instance): no copy job reads its fused qkv weights."""
+    from miles_amd import _lib
+
     cpu = _dense_model(31)
-    if odd == "fp16":
-        cpu = {k: v.to(torch.float16) for k, v in cpu.items()}
+    if odd != "offset":
+        cpu = {k: v.to(torch.float16 if odd == "fp16" else torch.float32) for k, v in cpu.items()}
     dev = {}
     for k, v in cpu.items():
         if odd == "offset" and k.endswith("linear_qkv.weight"):
@@ -1116,6 +1119,10 @@ def test_fused_qkv_that_the_tuned_kernel_cannot_read_in_place_is_regrouped(oracl
         cpu = {k: (v.float() * 0.5).to(v.dtype) for k, v in cpu.items()}
         for k in dev:
             dev[k].copy_(cpu[k])
+    qkv = [(t.data_ptr(), t.data_ptr() + t.nbytes) for k, t in dev.items() if k.endswith("linear_qkv.weight")]
+    copies_of_qkv = [rec for rec in upd._plan.batch.records
+                     if rec[0] == _lib.JOB_COPY and any(lo <= rec[2] < hi for lo, hi in qkv)]
+    assert (len(copies_of_qkv) == 0) == (odd == "fp16")
 
 
 @pytest.mark.parametrize("rows,row_bytes,src_pitch,dst_pitch,offset", [

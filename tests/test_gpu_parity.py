@@ -124,6 +124,72 @@ def test_block_fp8_generic_blocks_and_dtypes(oracle, dtype, bs):
     assert block_fp8 is not None
 
 
+def _fp16_tile_case(shape, seed, *, specials):
+    g = torch.Generator().manual_seed(seed)
+    w = (0.05 * torch.randn(shape, generator=g)).to(torch.float16)
+    m, n = shape
+    if m >= 8 and n >= 64:
+        w[0, :32] = torch.arange(1, 33, dtype=torch.int16).view(torch.float16)               # subnormals
+        w[1, :32] = (torch.arange(0x3E0, 0x400, dtype=torch.int16) - 0x8000).to(torch.int16).view(torch.float16)
+        w[2, :4] = torch.tensor([-0.0, 0.0, 65504.0, -65504.0], dtype=torch.float16)
+        w[3, 8:16] = torch.tensor([6.1e-5, -6.1e-5, 6.0e-8, 1.2e-7, 448.0, 464.0, 0.0009765625, 3.0], dtype=torch.float16)
+    if m > 128 and n > 256:
+        w[128:256, 128:256] = 0                           # a tile of zeros
+        w[m - 1, 130] = -0.0
+        w[:128, 256:384] *= 1e-3                          # a tile whose values are mostly fp16 subnormals
+    if specials and m > 5 and n > 140:
+        w[5, 3] = float("inf")
+        w[4, 130] = float("nan")
+        w[m - 1, n - 1] = float("-inf")
+    return w
+
+
+@pytest.mark.parametrize("shape", [(384, 640), (130, 264), (127, 136), (1, 8), (8, 64), (1024, 2048)])
+def test_fp8_tile_kernels_read_fp16(oracle, shape):
+    """fp16 tensors take the same tuned 128x128 kernels as bf16 ones (their own instances): the three scale rules against
+    the oracle, with fp16 subnormals, the format's extremes, signed zeros, a zero tile and, where the rule defines it
+    (the two casts with reciprocal scales), infinities and NaNs; then bf16 and fp16 tensors alternating in one recorded
+    job list, which has to split its launches by dtype."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast, per_block_cast_to_fp8
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    w = _fp16_tile_case(shape, 31 + shape[1], specials=False)
+    q, s = block_fp8(w.to(DEV), [128, 128])
+    q_o, s_o = oracle.block_fp8(w, (128, 128))
+    _assert_same(s, s_o, "block_fp8 scale")
+    _assert_same(q, q_o, "block_fp8 codes")
+    for specials in (False, True):
+        x = _fp16_tile_case(shape, 77 + shape[0], specials=specials)
+        for name, fn, ref in (("fp8_blockwise_cast", fp8_blockwise_cast, oracle.fp8_blockwise_cast),
+                              ("per_block_cast_to_fp8", per_block_cast_to_fp8, oracle.per_block_cast_to_fp8)):
+            y, s = fn(x.to(DEV))
+            y_o, s_o = ref(x)
+            _assert_same(s, s_o, f"{name} scale (specials={specials})")
+            _assert_same(y, y_o, f"{name} codes (specials={specials})")
+    if shape[0] > 1000:
+        return
+    tensors = []
+    for i in range(10):
+        t = _fp16_tile_case(shape, 500 + i, specials=False)
+        tensors.append(t if i % 3 else t.float().to(torch.bfloat16))
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [fp8_blockwise_cast(t) for t in dev] + [block_fp8(t, [128, 128]) for t in dev]
+    for rep in range(2):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, t in enumerate(tensors):
+            for (got, want, what) in zip(outs[i] + outs[10 + i], oracle.fp8_blockwise_cast(t) + oracle.block_fp8(t, (128, 128)),
+                                         ("cast codes", "cast scale", "block codes", "block scale")):
+                _assert_same(got, want, f"tensor {i} ({t.dtype}) {what}, run {rep}")
+        for o in outs:
+            for t in o:
+                t.view(torch.uint8).fill_(0x5A)
+        if rep == 0:
+            batch.freeze()
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_tensor_and_channel_fp8(oracle, dtype):
     from miles_amd.tools.convert_hf_to_fp8 import quant_fp8
