@@ -30,6 +30,19 @@ __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uin
 // A 32-bit word holds two 16-bit elements, element 0 in the low half.
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xFFFF0000u); }
+// A 16-bit element of the input as a float: a bf16 is the upper half of the float, an fp16 goes through the converter
+// (exact, subnormals included).  The absolute bit patterns of both formats order like the values they stand for, so
+// kernels take maxima on the patterns and convert once.
+template <int F16>
+__device__ __forceinline__ float elem_lo(uint32_t w) {
+    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+    return bf16_lo(w);
+}
+template <int F16>
+__device__ __forceinline__ float elem_hi(uint32_t w) {
+    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+    return bf16_hi(w);
+}
 
 // |x| of both halves, compared as unsigned 16-bit integers: for bf16 (and fp16) the ordering of
 // non-negative finite values equals the ordering of their bit patterns, and a NaN pattern is

@@ -62,19 +62,6 @@ __device__ __forceinline__ TilePick pick_tile(const TileRef& tab) {
     const int32_t tiles = ((job.M + kTile - 1) / kTile) * ((job.K + kTile - 1) / kTile);
     return TilePick{(int32_t)blockIdx.y, xcd_contiguous_item(tiles)};
 }
-// A 16-bit element of the input as a float: a bf16 is the upper half of the float, an fp16 goes through the converter
-// (exact, subnormals included).  The absolute bit patterns of both formats order like the values they stand for, so
-// the tile maximum is taken on the patterns and converted once.
-template <int F16>
-__device__ __forceinline__ float elem_lo(uint32_t w) {
-    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)w);
-    return bf16_lo(w);
-}
-template <int F16>
-__device__ __forceinline__ float elem_hi(uint32_t w) {
-    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
-    return bf16_hi(w);
-}
 template <int MODE, class Table, int F16>
 __global__ __launch_bounds__(kTileThreads) void fp8_block128_kernel(const Table tab) {
     constexpr uint32_t kInfBits = F16 ? 0x7C00u : 0x7F80u;      // pattern of +inf; anything above is a NaN

@@ -32,8 +32,10 @@ __device__ __forceinline__ float e8m0_inverse(uint32_t e) {
     return u2f((254u - e) << 23);
 }
 
-template <class Table>
+// 16-bit inputs, bf16 or fp16 (F16): the two instances differ in the conversion to fp32 and in the infinity pattern
+template <class Table, int F16>
 __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab) {
+    constexpr uint32_t kInfBits = F16 ? 0x7C00u : 0x7F80u;
     const float inv448 = u2f(0x3B124925u);
     const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
@@ -59,14 +61,28 @@ __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab)
     for (int i = 0; i < kMxUnroll; i++) {
         const uint32_t off = t + i * kMxThreads;
         uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
-        const uint32_t mb = group_max4(hmax_u16(m2));   // bf16 pattern of the group amax, quad-uniform
-        const float amax = u2f(mb << 16);
+        uint32_t mb = group_max4(hmax_u16(m2));         // 16-bit pattern of the group amax, quad-uniform
+        const bool plain = mb < kInfBits;               // no infinity and no NaN in the group
+        if (mb > kInfBits) {
+            // a NaN in the group (rare; the four lanes of a group branch together): the published kernel takes the
+            // maximum with fmaxf, which skips a NaN, so the scale comes from the other elements and only the NaN
+            // elements themselves become the NaN code
+            const uint32_t u[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+            uint32_t mf = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t lo = u[k] & 0x7FFFu, hi = (u[k] >> 16) & 0x7FFFu;
+                mf = umax(mf, umax(lo > kInfBits ? 0u : lo, hi > kInfBits ? 0u : hi));
+            }
+            mb = group_max4(mf);
+        }
+        const float amax = elem_lo<F16>(mb);
         const uint32_t e = e8m0_ceil(amax * inv448);
         const float inv = e8m0_inverse(e);
-        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                            elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
         u32x2 o;
-        if (mb < 0x7F80u) {
+        if (plain) {
             // finite group: |x * inv| <= 448 by construction, no clamp needed
             o.x = hw_e4m3x4(f[0] * inv, f[1] * inv, f[2] * inv, f[3] * inv);
             o.y = hw_e4m3x4(f[4] * inv, f[5] * inv, f[6] * inv, f[7] * inv);
@@ -92,7 +108,10 @@ __global__ __launch_bounds__(256) void mxfp8_generic_kernel(const void* __restri
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < groups; g += stride) {
         uint32_t m = 0;
-        for (int j = 0; j < 32; j++) m = umax(m, f2u(load_f32(w, g * 32 + j, dtype)) & 0x7FFFFFFFu);
+        for (int j = 0; j < 32; j++) {
+            const uint32_t a = f2u(load_f32(w, g * 32 + j, dtype)) & 0x7FFFFFFFu;
+            m = umax(m, a > 0x7F800000u ? 0u : a);       // the published kernel's fmaxf skips a NaN
+        }
         const uint32_t e = e8m0_ceil(u2f(m) * inv448);
         const float inv = e8m0_inverse(e);
         scale[g] = (uint8_t)e;
@@ -105,23 +124,27 @@ __global__ __launch_bounds__(256) void mxfp8_generic_kernel(const void* __restri
 using namespace mq;
 
 bool mq_mxfp8_fast_ok(const void* w, int dtype, const void* q) {
-    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
 }
 
-// tab.job[i].units set by the caller; fills tab.end and launches
-int mq_mxfp8_launch_group(FlatTable& tab, hipStream_t st) {
+// tab.job[i].units set by the caller, every tensor of the one 16-bit dtype; fills tab.end and launches
+int mq_mxfp8_launch_group(int dtype, FlatTable& tab, hipStream_t st) {
     if (!flat_grid(tab, kMxThreads * kMxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp8_bf16_kernel<FlatTable>, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kMxThreads), 0, st, tab);
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kMxThreads);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((mxfp8_bf16_kernel<FlatTable, 1>), grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL((mxfp8_bf16_kernel<FlatTable, 0>), grid, blk, 0, st, tab);
     return mq_check_launch("mxfp8 quant");
 }
 
 // n descriptors in device memory; max_units: the largest tensor's 16-byte units
-int mq_mxfp8_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
+int mq_mxfp8_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kMxThreads * kMxUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (ref.max_blocks == 0 || n == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp8_bf16_kernel<FlatRef>, dim3((unsigned)ref.max_blocks, (unsigned)n), dim3(kMxThreads), 0, st, ref);
+    const dim3 grid((unsigned)ref.max_blocks, (unsigned)n), blk(kMxThreads);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((mxfp8_bf16_kernel<FlatRef, 1>), grid, blk, 0, st, ref);
+    else hipLaunchKernelGGL((mxfp8_bf16_kernel<FlatRef, 0>), grid, blk, 0, st, ref);
     return mq_check_launch("mxfp8 quant");
 }
 
@@ -137,7 +160,7 @@ extern "C" int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale,
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, q, scale, nullptr, groups * 4, nullptr, 0, 0};
-        return mq_mxfp8_launch_group(tab, st);
+        return mq_mxfp8_launch_group(dtype, tab, st);
     }
     int64_t blocks = (groups + 255) / 256;
     if (blocks > mq_grid_cap()) blocks = mq_grid_cap();

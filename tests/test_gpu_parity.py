@@ -343,6 +343,43 @@ def test_mxfp8_heavy_tails_3d_dtypes_and_errors(oracle):
         mxfp8_quantize(torch.zeros(4, 48, dtype=torch.bfloat16, device=DEV))
 
 
+@pytest.mark.parametrize("shape", [(384, 640), (8, 64), (5, 32), (1024, 2048)])
+def test_mxfp8_reads_fp16(oracle, shape):
+    """fp16 tensors take the tuned MXFP8 kernel's fp16 instance: subnormals, the format's extremes, signed zeros, groups
+    of zeros, infinities and NaNs against the oracle; then bf16 and fp16 tensors alternating in one recorded job list."""
+    from miles_amd import launch
+    from miles_amd.utils.mxfp8 import mxfp8_quantize
+
+    for specials in (False, True):
+        w = _fp16_tile_case(shape, 900 + shape[1], specials=specials)
+        if shape[0] > 4:
+            w[4, :32] = 0
+        q, s = mxfp8_quantize(w.to(DEV))
+        q_o, s_o = oracle.mxfp8_quantize(w)
+        _assert_same(s, s_o, f"scales (specials={specials})")
+        _assert_same(q, q_o, f"codes (specials={specials})")
+    if shape[0] > 1000:
+        return
+    tensors = []
+    for i in range(9):
+        t = _fp16_tile_case(shape, 950 + i, specials=False)
+        tensors.append(t if i % 3 else t.float().to(torch.bfloat16))
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [mxfp8_quantize(t) for t in dev]
+    for rep in range(2):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, t in enumerate(tensors):
+            for got, want, what in zip(outs[i], oracle.mxfp8_quantize(t), ("codes", "scales")):
+                _assert_same(got, want, f"tensor {i} ({t.dtype}) {what}, run {rep}")
+        for o in outs:
+            for t in o:
+                t.view(torch.uint8).fill_(0x5A)
+        if rep == 0:
+            batch.freeze()
+
+
 # ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((24, 7168), 128),
                                      ((16, 256), 32), ((5, 96), 32), ((9, 192), 64), ((3, 160), 160)])
