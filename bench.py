@@ -443,7 +443,7 @@ def roofline(plan, elems, steps, gpu_ms):
     avg_us = gpu_ms * 1e3 / (steps * launches)
     bytes_per_launch = elems * BYTES_PER_ELEM["fp8_block"] / launches
     achieved = bytes_per_launch / avg_us / 1e3
-    return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1, mq::TileTable>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+    return {"bound": "hbm", "kernel": "mq::fp8_block128_kernel<1, mq::TileTable, 0>", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM * elems / launches),
             "launches_per_sync": launches, "avg_launch_us": round(avg_us, 2),

@@ -39,8 +39,9 @@ __device__ __forceinline__ float ceil_pow2_scale(float v) {
     return u2f(((u >> 23) + ((u & 0x7FFFFFu) != 0)) << 23);
 }
 
-// The kernel is bound by vector-ALU issue as much as by memory (counters: ~85 % VALU busy at 6.3 TB/s), so everything
-// that is the same for the whole workgroup stays on the scalar unit: the job lookup, the tile's row and column (a
+// Everything that is the same for the whole workgroup stays on the scalar unit (with the job lookup and the tile
+// addressing in vector instructions the kernel issued 460 of them per wavefront; it issues about 200 now and the
+// vector unit is busy a third of the time, the memory system being what bounds it): the job lookup, the tile's row and column (a
 // multiply-high division with constants from the host), the 64-bit base addresses of the tile in the input and in the
 // output.  A lane adds 32-bit offsets to those bases.  Interior tiles take a path with no bounds tests at all; edge
 // tiles load from clamped (always valid) addresses and zero what lies outside, so that in both cases the four loads of
