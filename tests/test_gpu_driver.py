@@ -241,8 +241,9 @@ def _moe_model(seed, experts=4, ffn=128, hidden=256):
     return p
 
 
-def test_moe_mxfp8_sync(oracle):
-    cpu = _moe_model(30)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_moe_mxfp8_sync(oracle, dtype):
+    cpu = {k: v.to(dtype) for k, v in _moe_model(30).items()}
     dev = {k: v.to(DEV) for k, v in cpu.items()}
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3moe", quantization_config={"quant_method": "mxfp8"},
                         send_bucket=None)
@@ -259,7 +260,7 @@ def test_moe_mxfp8_sync(oracle):
         assert [n for n, _ in flat] == [n for n, _ in want]
         for (n, g), (_, w) in zip(flat, want):
             _same(g, w, f"{n} sync {round_}")
-        cpu = _moe_model(31)
+        cpu = {k: v.to(dtype) for k, v in _moe_model(31).items()}
         for k in dev:
             dev[k].copy_(cpu[k])
 
