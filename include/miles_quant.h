@@ -275,7 +275,8 @@ typedef struct mq_job {
     int64_t rows_per_block, block_stride;
 } mq_job;
 /* Consecutive jobs of one kind (and, for the flat kernels, of similar size) are fused into launches of up to
- * MQ_MAX_GROUP tensors, counted from the first job of the call. */
+ * MQ_MAX_GROUP tensors, counted from the first job of the call; a run of FP8 tile jobs of more than 36 864 tiles is
+ * cut into launches of equal size (the tile kernel streams faster in launches of moderate length). */
 #define MQ_MAX_GROUP 64
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 

@@ -178,6 +178,12 @@ static TileJob tile_entry(const mq_job& jb) {
     return TileJob{jb.in, jb.out, (float*)jb.scale, (int32_t)jb.ld, (int32_t)jb.rows, (int32_t)jb.cols,
                    (int32_t)jb.block_stride, (int32_t)(jb.rows_per_block / 128), 0, 0, 0};
 }
+// The tile kernel streams a few percent faster in launches of moderate length than in very long ones (measured on the
+// Qwen3-4B tensors: 0.770 of peak at 98 000 tiles per launch, 0.784 at 49 000, 0.790 at 31 000, 0.792 at 18 000; each
+// launch boundary costs about 4 us).  A run of tile jobs longer than this many tiles goes out as launches of equal size.
+#ifndef MQ_TILE_LAUNCH_TILES
+#define MQ_TILE_LAUNCH_TILES 36864
+#endif
 static int64_t tiles_of(const mq_job& jb) { return ((jb.rows + 127) / 128) * ((jb.cols + 127) / 128); }
 static FlatJob flat_entry(const mq_job& jb) {
     if (jb.kind == MQ_JOB_INT4_PACK_ASYM)       // zero points, packed zero points, groups per row
@@ -185,6 +191,16 @@ static FlatJob flat_entry(const mq_job& jb) {
     if (jb.kind == MQ_JOB_FP8_TENSOR)           // amax record, one section
         return FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, nullptr, 0, 1};
     return FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8, nullptr, 0, 0};
+}
+
+// jobs [i, j) hold `tiles` tiles: where the first of the equal launches they are cut into ends
+static int64_t tile_run_end(const mq_job* jobs, int64_t i, int64_t j, int64_t tiles) {
+    if (MQ_TILE_LAUNCH_TILES <= 0 || tiles <= MQ_TILE_LAUNCH_TILES) return j;
+    const int64_t launches = (tiles + MQ_TILE_LAUNCH_TILES - 1) / MQ_TILE_LAUNCH_TILES;
+    const int64_t target = (tiles + launches - 1) / launches;
+    int64_t acc = 0, t = i;
+    while (t < j && acc < target) acc += tiles_of(jobs[t++]);
+    return t;
 }
 
 static bool same_group(const mq_job& a, const mq_job& b) {
@@ -429,6 +445,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                 mx = nmx;
                 j++;
             }
+            j = tile_run_end(jobs, i, j, sum);
             // (tensors of 256 tiles and more fill a searched launch of 64 well enough, and run 1-2 % faster in that form)
             if (j - i > kMaxGroup && mx < 256) {
                 const int mode = head.kind == MQ_JOB_FP8_BLOCK ? 0 : head.kind == MQ_JOB_FP8_BLOCKWISE_CAST ? 1 : 2;
@@ -449,6 +466,11 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
             sum += e;
             mx = nmx;
             j++;
+        }
+        if (tile_kind(head.kind)) {
+            int64_t tiles = 0;
+            for (int64_t t = i; t < j; t++) tiles += tiles_of(jobs[t]);
+            j = tile_run_end(jobs, i, j, tiles);
         }
         const int cnt = (int)(j - i);
         int rc = MQ_OK;
