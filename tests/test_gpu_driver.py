@@ -1009,7 +1009,7 @@ def test_recording_a_sync_holds_no_more_than_a_few_buckets():
     assert outputs > 5 * plan.arena_bytes
 
 
-@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4", "int4_asym", "fp8", "block_fp8"])
+@pytest.mark.parametrize("fmt", ["mxfp8", "mxfp4", "int4", "int4_asym", "fp8", "block_fp8", "mxfp8_f16", "fp8_f16"])
 def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     """More than MQ_MAX_GROUP jobs of a table kind: the batch copies their descriptors to device memory and one launch
     covers the lot.  Shapes vary inside the 25 % band that keeps a group together, with a few far outside it (which
@@ -1021,6 +1021,9 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     from miles_amd.utils.mxfp4 import quantize_mxfp4
     from miles_amd.utils.mxfp8 import mxfp8_quantize
 
+    # (the two kernels with fp16 instances also run the list with every third tensor in fp16: launches split by dtype)
+    mixed_dtypes = fmt.endswith("_f16")
+    fmt = fmt.removesuffix("_f16")
     g = torch.Generator().manual_seed(77)
     shapes = [(int(torch.randint(52, 64, (1,), generator=g)), 256) for _ in range(150)]
     shapes[40], shapes[41], shapes[120] = (8, 128), (300, 256), (1, 128)
@@ -1030,6 +1033,8 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
         shapes = [(130 + (r * 7 + i) % 120, 264 + 8 * (i % 3)) for i, (r, k) in enumerate(shapes)]
         shapes[40], shapes[41], shapes[120], shapes[130] = (8, 128), (1300, 256), (1, 8), (256, 384)
     ws = [W.student_t_rows(s, std=0.02, seed=7700 + i) for i, s in enumerate(shapes)]
+    if mixed_dtypes:        # runs of fp16 tensors long enough for a table launch of their own, and single ones
+        ws = [w.to(torch.float16) if (i % 3 == 0 or 80 <= i < 150) else w for i, w in enumerate(ws)]
     dev = [w.to(DEV) for w in ws]
     tile_w = W.gaussian_outliers((256, 384), std=0.02, p_outlier=0.001, gain=20.0, seed=7)
 
