@@ -1093,6 +1093,42 @@ def test_launches_with_a_device_table_cover_hundreds_of_tensors(oracle, fmt):
     check("without the table")
 
 
+@pytest.mark.parametrize("form", ["searched", "table"])
+def test_long_runs_of_tile_jobs_are_cut_into_launches_of_equal_size(oracle, form):
+    """A run of FP8 tile jobs of more than 36 864 tiles goes out as several launches (the tile kernel streams faster in
+    launches of moderate length).  Both launch forms: 44 tensors of 896 tiles (descriptors in the kernel arguments,
+    cut in two) and 420 tensors of 96 tiles (device table, cut in two); every output against the oracle, also on the
+    replay and when the list is submitted in two ranges that start mid-run."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+
+    if form == "searched":
+        shapes, quantize, expected = [(2048, 7168)] * 44, lambda w: block_fp8(w, [128, 128]), lambda w: oracle.block_fp8(w, (128, 128))
+    else:
+        shapes = [(768, 2048) if i % 3 else (2048, 768) for i in range(420)]
+        quantize, expected = fp8_blockwise_cast, oracle.fp8_blockwise_cast
+    assert sum(-(-r // 128) * -(-c // 128) for r, c in shapes) > 36864
+    ws = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=9100 + i) for i, s in enumerate(shapes)]
+    dev = [w.to(DEV) for w in ws]
+    with launch.recording() as batch:
+        outs = [quantize(w) for w in dev]
+    batch.freeze()
+    assert (batch._table is not None) == (form == "table")
+    want = [expected(w) for w in ws]
+    half = len(batch) // 2 + 3
+    for what, run in (("one submission", batch.run), ("replay", batch.run),
+                      ("two ranges", lambda: (batch.run_range(0, half), batch.run_range(half, len(batch))))):
+        for out in outs:
+            for t in out:
+                t.view(torch.uint8).fill_(0x5A)
+        run()
+        torch.cuda.synchronize()
+        for i, (out, exp) in enumerate(zip(outs, want)):
+            for k, (got, w_) in enumerate(zip(out, exp)):
+                _same(got, w_, f"tensor {i} output {k} ({what})")
+
+
 @pytest.mark.parametrize("odd", ["offset", "fp32", "fp16"])
 def test_fused_qkv_that_the_tuned_kernel_cannot_read_in_place_is_regrouped(oracle, odd):
     """Row-blocked q / k / v views are switched on per model, by shape.  A fused qkv parameter that starts two bytes into
