@@ -231,8 +231,8 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
- * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2) run their tuned 128x128 kernel on bf16 and on
- * fp16 inputs; consecutive jobs share a launch when they also share the input dtype.
+ * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8 and INT4_PACK run their tuned kernels on
+ * bf16 and on fp16 inputs; consecutive jobs share a launch when they also share the input dtype.
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
  * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list.
  * MQ_NVFP4_CARRY_AMAX in p1 of NVFP4 and FP8_TENSOR jobs (no counterpart in the reference): a caller that submits the

@@ -49,11 +49,23 @@ __device__ __forceinline__ uint32_t code_bits(float q) { return f2u(q + 12582920
 // at that maximum 7 * scale_b overflows, and an infinity or a NaN breaks it too.  This function runs the chain as
 // written for one unit: NaN skipped by the group maximum as the reference's fmaxf reduction does, codes above 15
 // carrying into the next nibble as in its int32 sum.
-template <int LANES>
+// rounding of an fp32 value to the tensor's 16-bit dtype (as a float again, or as the stored pattern)
+template <int F16>
+__device__ __forceinline__ float round16(float x) {
+    if (F16) return (float)(_Float16)x;
+    return u2f(sw_bf16(x) << 16);
+}
+template <int F16>
+__device__ __forceinline__ uint16_t bits16(float x) {
+    if (F16) return __builtin_bit_cast(uint16_t, (_Float16)x);
+    return (uint16_t)sw_bf16(x);
+}
+template <int LANES, int F16>
 __device__ __forceinline__ void int4_pack_chain_unit(const u32x4 v, const int64_t unit, const bool live,
                                                                const int t, uint32_t* __restrict__ packed,
                                                                uint16_t* __restrict__ scale) {
-    const float f[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+    const float f[8] = {elem_lo<F16>(v.x), elem_hi<F16>(v.x), elem_lo<F16>(v.y), elem_hi<F16>(v.y),
+                        elem_lo<F16>(v.z), elem_hi<F16>(v.z), elem_lo<F16>(v.w), elem_hi<F16>(v.w)};
     uint32_t m = 0;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
@@ -61,25 +73,30 @@ __device__ __forceinline__ void int4_pack_chain_unit(const u32x4 v, const int64_
         m = umax(m, a > 0x7F800000u ? 0u : a);
     }
     const float s = __builtin_fmaxf(u2f(seg_max<LANES>(m)) * kSymCons, 1e-5f);
-    const float sb = u2f(sw_bf16(s) << 16);
+    const float sb = round16<F16>(s);
     uint32_t word = 0;
 #pragma unroll 1
     for (int j = 0; j < 8; j++) {
         const uint32_t pair = j < 2 ? v.x : j < 4 ? v.y : j < 6 ? v.z : v.w;
-        const float x = (j & 1) ? bf16_hi(pair) : bf16_lo(pair);
-        const float q0 = u2f(sw_bf16(__builtin_rintf(x / s)) << 16);
-        const float wv = u2f(sw_bf16(q0 * sb) << 16);
-        const float rv = clamp_keep_nan(u2f(sw_bf16(wv / sb) << 16), -128.0f, 127.0f);
+        const float x = (j & 1) ? elem_hi<F16>(pair) : elem_lo<F16>(pair);
+        const float q0 = round16<F16>(__builtin_rintf(x / s));
+        const float wv = round16<F16>(q0 * sb);
+        const float rv = clamp_keep_nan(round16<F16>(wv / sb), -128.0f, 127.0f);
         word += (uint32_t)(((int)__builtin_rintf(rv) + 8) & 0xFF) << (4 * j);
     }
     if (live) {
         st4(packed + unit, word);
-        if ((t & (LANES - 1)) == 0) scale[unit / LANES] = (uint16_t)sw_bf16(s);
+        if ((t & (LANES - 1)) == 0) scale[unit / LANES] = bits16<F16>(s);
     }
 }
 
-template <int LANES, class Table>
+// 16-bit inputs, bf16 or fp16 (F16).  The fused form rests on the reference's dequantize / requantize round trip in the
+// tensor's dtype being the identity on the codes: proved for bf16 scales, and checked over every fp16 scale from the
+// floor fp16(1e-5) up (all 31 576 patterns x the fifteen codes): it fails only where 7 x scale overflows, which needs a
+// group maximum of 65504, the largest fp16.
+template <int LANES, class Table, int F16>
 __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table tab) {
+    constexpr uint32_t kTopBits = F16 ? 0x7BFFu : 0x7F7Fu;      // the largest finite value; infinities and NaN lie above
     const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
@@ -107,15 +124,15 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = seg_max<LANES>(hmax_u16(m2));
         top = umax(top, mb);
-        const float amax = u2f(mb << 16);
+        const float amax = elem_lo<F16>(mb);
         const float s = __builtin_fmaxf(amax * kSymCons, 1e-5f);
         const float y = recip_shared(s);
-        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                            elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
         const bool fast = shared_div_ok(s);
         // |x / s| <= 7 (1 + 2^-23), so the pattern of q + (1.5 * 2^23 + 8) is 0x4B400000 + nibble: the eight patterns
         // are summed at their nibble's place (one shift-add each, modulo 2^32) and what the high bits added up to is
-        // taken off once.  (A wavefront that met an infinity, a NaN or the largest bf16 writes its words again below.)
+        // taken off once.  (A wavefront that met an infinity, a NaN or the largest finite value writes its words again below.)
         constexpr uint32_t kMagicSum = 0x4B400000u + (0x4B400000u << 4) + (0x4B400000u << 8);     // further shifts: 0
         uint32_t word = 0;
         if (__builtin_amdgcn_ballot_w64(!fast) == 0) {         // every scale of the wavefront in range: one straight run
@@ -132,17 +149,17 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_bf16_kernel(const Table 
         const uint32_t off = t + i * kI4Threads;
         if (off < rem) {
             st4(packed0 + off, word);
-            if ((t & (LANES - 1)) == 0) scale0[off / LANES] = (uint16_t)hw_bf16x2(s, 0.0f);
+            if ((t & (LANES - 1)) == 0) scale0[off / LANES] = F16 ? bits16<1>(s) : (uint16_t)hw_bf16x2(s, 0.0f);
         }
     }
-    // A group holding the largest finite bf16, an infinity or a NaN is outside the fused form: a wavefront that met one
+    // A group holding the largest finite value of the dtype, an infinity or a NaN is outside the fused form: a wavefront that met one
     // writes all of its groups again through the written-out chain (a scalar branch after the common path, which
     // therefore stays one straight instruction stream; the later store of a lane to the same address wins).
-    if (__builtin_amdgcn_ballot_w64(top >= 0x7F7Fu) == 0) return;
+    if (__builtin_amdgcn_ballot_w64(top >= kTopBits) == 0) return;
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
         const int64_t unit = base + i * kI4Threads + t;
-        int4_pack_chain_unit<LANES>(v[i], unit, unit < total_units, t, packed, scale);
+        int4_pack_chain_unit<LANES, F16>(v[i], unit, unit < total_units, t, packed, scale);
     }
 }
 
@@ -756,27 +773,36 @@ extern "C" int mq_int4_fake_quant(const void* x, int dtype, void* out, void* sca
 }
 
 bool mq_int4_pack_fast_ok(const void* w, int dtype, int group) {
-    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32);
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32);
 }
 
-int mq_int4_pack_launch_group(FlatTable& tab, int group, hipStream_t st) {
+template <class Table>
+static void int4_pack_launch(int dtype, int group, dim3 grid, hipStream_t st, const Table& tab) {
+    const dim3 blk(kI4Threads);
+    if (dtype == MQ_F16) {
+        if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, Table, 1>), grid, blk, 0, st, tab);
+        else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, Table, 1>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, Table, 1>), grid, blk, 0, st, tab);
+    } else {
+        if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, Table, 0>), grid, blk, 0, st, tab);
+        else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, Table, 0>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, Table, 0>), grid, blk, 0, st, tab);
+    }
+}
+
+// every tensor of a launch has the one 16-bit dtype
+int mq_int4_pack_launch_group(int dtype, FlatTable& tab, int group, hipStream_t st) {
     if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kI4Threads);
-    if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, FlatTable>), grid, blk, 0, st, tab);
-    else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, FlatTable>), grid, blk, 0, st, tab);
-    else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, FlatTable>), grid, blk, 0, st, tab);
+    int4_pack_launch(dtype, group, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), st, tab);
     return mq_check_launch("int4 pack");
 }
 
-int mq_int4_pack_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st) {
+int mq_int4_pack_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (ref.max_blocks == 0 || n == 0) return MQ_OK;
-    dim3 grid((unsigned)ref.max_blocks, (unsigned)n), blk(kI4Threads);
-    if (group == 128) hipLaunchKernelGGL((int4_pack_bf16_kernel<16, FlatRef>), grid, blk, 0, st, ref);
-    else if (group == 64) hipLaunchKernelGGL((int4_pack_bf16_kernel<8, FlatRef>), grid, blk, 0, st, ref);
-    else hipLaunchKernelGGL((int4_pack_bf16_kernel<4, FlatRef>), grid, blk, 0, st, ref);
+    int4_pack_launch(dtype, group, dim3((unsigned)ref.max_blocks, (unsigned)n), st, ref);
     return mq_check_launch("int4 pack");
 }
 
@@ -792,7 +818,7 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, packed, scale, nullptr, units, nullptr, 0, 0};
-        return mq_int4_pack_launch_group(tab, group, st);
+        return mq_int4_pack_launch_group(dtype, tab, group, st);
     }
     int64_t blocks = (units + 255) / 256;
     if (blocks > mq_grid_cap()) blocks = mq_grid_cap();

@@ -397,6 +397,55 @@ def test_int4_pack_layer(oracle, shape, G):
     _assert_same(packed, packed_o, "packed")
 
 
+@pytest.mark.parametrize("shape,G", [((4, 128), 128), ((16, 256), 128), ((64, 1024), 128), ((24, 7168), 128),
+                                     ((16, 256), 32), ((9, 192), 64), ((2048, 7168), 128)])
+def test_int4_pack_layer_fp16(oracle, shape, G):
+    """fp16 weights take the fused packer's fp16 instance (groups of 32 / 64 / 128): scales in fp16, the scale floor
+    (a subnormal fp16), subnormal inputs, ties, and groups whose maximum is 65504, where 7 x scale overflows in the
+    reference's fp16 round trip and the kernel has to follow the written-out chain; then bf16 and fp16 tensors
+    alternating in one recorded job list."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    def case(seed):
+        w = W.gaussian_outliers(shape, std=0.015, p_outlier=0.0005, gain=30.0, seed=seed, dtype=torch.float16)
+        w[0] = 0
+        w[1, :G] = 3e-6
+        w[2, :G] = torch.linspace(-1, 1, G).to(torch.float16)
+        w[3, :32] = torch.arange(1, 33, dtype=torch.int16).view(torch.float16)       # subnormals only: floor scale
+        if shape[0] > 8:
+            w[4, :G] = torch.linspace(-65504, 65504, G).to(torch.float16)
+            w[5, 7] = 65504.0
+            w[6, G - 1] = -65504.0
+            w[7, :G] = 65504.0
+            w[8, :G] = torch.linspace(-60000, 65472, G).to(torch.float16)              # just below the overflow
+        return w
+
+    w = case(4001)
+    packed, scale, zp = pack_layer(w.to(DEV), G)
+    packed_o, scale_o, _ = oracle.pack_layer(w, G)
+    assert zp is None and packed.dtype == torch.int32 and scale.dtype == torch.float16
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(packed, packed_o, "packed")
+    if shape[0] > 1000:
+        return
+    tensors = [case(4100 + i) if i % 3 else case(4100 + i).float().clamp(-3e4, 3e4).to(torch.bfloat16) for i in range(9)]
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [pack_layer(t, G)[:2] for t in dev]
+    for rep in range(2):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, t in enumerate(tensors):
+            for got, want, what in zip(outs[i], oracle.pack_layer(t, G)[:2], ("packed", "scales")):
+                _assert_same(got, want, f"tensor {i} ({t.dtype}) {what}, run {rep}")
+        for o in outs:
+            for t in o:
+                t.view(torch.uint8).fill_(0x5A)
+        if rep == 0:
+            batch.freeze()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_int4_pack_layer_other_dtypes(oracle, dtype):
     from miles_amd.kernels.quant.int4_fake import pack_layer
