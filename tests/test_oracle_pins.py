@@ -544,6 +544,26 @@ def test_int4_asym_round_trip_is_identity_for_unclamped_codes():
             assert torch.all(code == w1), (z, w1)
 
 
+def test_int4_sym_round_trip_in_fp16_is_identity_below_the_overflow():
+    # The fp16 instance of the symmetric packer emits rint(x/s) + 8 directly.  Exhaustive over every fp16 scale from the
+    # floor fp16(1e-5) (a subnormal) upwards and the fifteen codes: the reference's chain in fp16
+    # fp16(q * s) / s -> clamp -> round returns q unless 7 * s overflows, and the only group maximum whose scale
+    # fp16(max * f32(1/7)) reaches that is 65504, which the kernel sends through the written-out chain.
+    sb = torch.arange(1, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    sb = sb[sb >= torch.tensor(1e-5, dtype=torch.float16)]
+    assert sb.numel() == 31576 and sb[0].view(torch.int16).item() == 0xA8
+    safe = sb[sb.float() < 9360.0]
+    for q in range(-7, 8):
+        qt = torch.tensor(float(q), dtype=torch.float16)
+        r = (qt * safe) / safe
+        code = torch.round(torch.clamp(r, -128, 127)).to(torch.int8)
+        assert torch.all(code == q), q
+    amax = torch.arange(1, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16).float()
+    s = torch.maximum(amax * torch.tensor(1.0 / 7.0, dtype=torch.float32), torch.tensor(1e-5, dtype=torch.float32)).to(torch.float16)
+    overflowing = amax[(s.float() >= 9360.0)]
+    assert overflowing.tolist() == [65504.0]
+
+
 def test_int4_constant_rows_known_answer(oracle):
     for c in (0.5, 0.013, 3.0):
         w = torch.full((2, 128), c, dtype=torch.bfloat16)
