@@ -269,13 +269,114 @@ __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float 
     const float e4 = nv_pair_error(t4, odd_lane), e6 = nv_pair_error(t6, odd_lane);
     return e4 < e6 ? c4 : c6;
 }
+// ---- the same with one lane per block (the quantizer's form) ------------------------------------------------
+// With two lanes per block every block-level step (the two candidate scales, their reciprocals, the comparison) is
+// done twice, and the error sum, which has to run through the sixteen terms in element order, takes sixteen additions
+// in each lane of the pair.  The quantizer therefore regroups its data first: a lane ends up with the thirty-two
+// bytes of one whole block, and this kernel is bound by vector instructions, not by memory.
+struct NvCandidate16 {
+    uint32_t sc;        // e4m3 byte
+    uint32_t lo, hi;    // codes of elements 0..7 and 8..15
+    float s_f;          // f32(sc)
+};
+__device__ __forceinline__ NvCandidate16 nv_candidate16(const float f[16], float s_hp, float s_dec) {
+    NvCandidate16 c;
+    c.sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
+    c.s_f = hw_e4m3x2_decode<false>(c.sc).x;
+    const float d = c.s_f * s_dec;
+    float inv;
+    if (__builtin_amdgcn_ballot_w64(!shared_div_ok(d)) == 0) inv = recip_shared(d);
+    else inv = __builtin_fminf(1.0f / d, kFltMax);
+    c.lo = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
+    c.lo = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, c.lo);
+    c.lo = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, c.lo);
+    c.lo = hw_e2m1x2<3>(f[6] * inv, f[7] * inv, c.lo);
+    c.hi = hw_e2m1x2<0>(f[8] * inv, f[9] * inv, 0u);
+    c.hi = hw_e2m1x2<1>(f[10] * inv, f[11] * inv, c.hi);
+    c.hi = hw_e2m1x2<2>(f[12] * inv, f[13] * inv, c.hi);
+    c.hi = hw_e2m1x2<3>(f[14] * inv, f[15] * inv, c.hi);
+    return c;
+}
+template <int EM, int FASTDIV>
+__device__ __forceinline__ float nv_block_error(const float f[16], const NvCandidate16& c, float amax, float enc, float denom) {
+    float term[8], error = 0.0f;
+    NvCandidate half{c.sc, c.lo, c.s_f};
+    nv_error_terms<EM, FASTDIV>(f, half, amax, enc, denom, term);
+#pragma unroll
+    for (int j = 0; j < 8; j++) error = error + term[j];
+    half.word = c.hi;
+    nv_error_terms<EM, FASTDIV>(f + 8, half, amax, enc, denom, term);
+#pragma unroll
+    for (int j = 0; j < 8; j++) error = error + term[j];
+    return error;
+}
+template <int EM, int FASTDIV>
+__device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], float bmax, float amax, const NvScales& gs,
+                                                            float denom) {
+    const bool plain_bmax = shared_div_ok(bmax);
+    const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
+    const float s4_hp = s6_hp * 1.5f;
+    const NvCandidate16 c4 = nv_candidate16(f, s4_hp, gs.s_dec), c6 = nv_candidate16(f, s6_hp, gs.s_dec);
+    const float e4 = nv_block_error<EM, FASTDIV>(f, c4, amax, gs.enc, denom);
+    const float e6 = nv_block_error<EM, FASTDIV>(f, c6, amax, gs.enc, denom);
+    return e4 < e6 ? c4 : c6;
+}
 // error mode of a flags word, as the EM template argument
 static inline int nv_error_mode(int flags) { return ((flags & MQ_NVFP4_ERR_MSE) ? 1 : 0) | ((flags & MQ_NVFP4_ERR_FP16) ? 2 : 0); }
+
+// Four Over Six over kNvThreads * 2 units starting at `base`: loaded as the standard quantizer loads them (lane t takes
+// units t and kNvThreads + t, so a wavefront's loads are contiguous), then regrouped through LDS inside each wavefront so
+// that the even lane of a pair holds the block made of units 2p, 2p + 1 and the odd lane the block kNvThreads + 2p, + 1.
+// Returns the largest |element| of the lane's block (bf16 bits).
+template <int EM>
+__device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
+    static_assert(kNvUnroll == 2, "the regrouping pairs the two units of a lane");
+    __shared__ u32x4 stage[2 * kNvThreads];
+    const uint16_t* __restrict__ w = (const uint16_t*)job.w;
+    uint32_t* __restrict__ q = (uint32_t*)job.q;
+    uint8_t* __restrict__ s8 = (uint8_t*)job.s;
+    const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
+    const int64_t left = job.units - base;
+    const uint32_t rem = left < kNvThreads * 2 ? (uint32_t)left : (uint32_t)(kNvThreads * 2);
+    const uint16_t* __restrict__ w0 = w + base * 8;
+    uint32_t* __restrict__ q0 = q + base;
+    uint8_t* __restrict__ s80 = s8 + base / 2;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t off = (uint32_t)t + i * kNvThreads;
+        stage[off] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();        // (a wavefront reads back only what it wrote itself)
+    const uint32_t first = ((t & 1) ? (uint32_t)kNvThreads : 0u) + ((uint32_t)t & ~1u);      // the block's first unit
+    const u32x4 lo = stage[first], hi = stage[first + 1];
+    NvScales gs;
+    gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
+    gs.s_dec = u2f(amax_bits[kRecSDec]);
+    gs.enc = u2f(amax_bits[kRecEnc]);
+    const float amax = u2f(amax_bits[kRecAmax]);
+    const int fastdiv = nv_fast_division(amax);
+    const uint32_t m2 = max2_u16(max2_u16(max2_u16(abs2(lo.x), abs2(lo.y)), max2_u16(abs2(lo.z), abs2(lo.w))),
+                                 max2_u16(max2_u16(abs2(hi.x), abs2(hi.y)), max2_u16(abs2(hi.z), abs2(hi.w))));
+    const uint32_t mb = hmax_u16(m2);
+    const float bmax = u2f(mb << 16);
+    const float f[16] = {bf16_lo(lo.x), bf16_hi(lo.x), bf16_lo(lo.y), bf16_hi(lo.y), bf16_lo(lo.z), bf16_hi(lo.z), bf16_lo(lo.w), bf16_hi(lo.w),
+                         bf16_lo(hi.x), bf16_hi(hi.x), bf16_lo(hi.y), bf16_hi(hi.y), bf16_lo(hi.z), bf16_hi(hi.z), bf16_lo(hi.w), bf16_hi(hi.w)};
+    const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom)
+                            : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom)
+                                           : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom);
+    if (first < rem) {      // the tensor is whole blocks: both units of a block are inside or outside
+        st4(q0 + first, c.lo);
+        st4(q0 + first + 1, c.hi);
+        s80[first >> 1] = (uint8_t)c.sc;
+    }
+    return mb;
+}
 
 // kNvThreads * kNvUnroll units starting at `base` of one tensor; returns the largest |element| this lane saw (bf16 bits)
 // FOS = 0: standard quantizer; FOS = 1 + error mode: Four Over Six
 template <int FOS>
 __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
+    if (FOS) return nvfp4_fos_units<(FOS > 0 ? FOS - 1 : 0)>(job, base, t, denom);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
@@ -311,14 +412,7 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
         const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
                             bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
         uint32_t sc, word;
-        if (FOS) {
-            constexpr int EM = FOS > 0 ? FOS - 1 : 0;
-            const NvCandidate c = fastdiv == 2   ? nv_four_over_six<EM, 2>(f, bmax, amax, gs, denom, (t & 1) != 0)
-                                  : fastdiv == 1 ? nv_four_over_six<EM, 1>(f, bmax, amax, gs, denom, (t & 1) != 0)
-                                                 : nv_four_over_six<EM, 0>(f, bmax, amax, gs, denom, (t & 1) != 0);
-            sc = c.sc;
-            word = c.word;
-        } else if (mb < 0x7F80u && s_hp == s_hp) {
+        if (mb < 0x7F80u && s_hp == s_hp) {
             sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
             const float s_f = hw_e4m3x2_decode<false>(sc).x;
             // 1 / (block scale x global decode scale): the refined hardware reciprocal where it equals the division (every
