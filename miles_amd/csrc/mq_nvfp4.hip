@@ -220,11 +220,10 @@ __device__ __forceinline__ float div_by_numer(float x, float d, float y) {
 }
 // error terms of this lane's eight elements; EM bit 0: squared error, bit 1: fp16 candidate error
 template <int EM, int FASTDIV>
-__device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandidate& c, float amax, float enc, float denom,
+__device__ __forceinline__ void nv_error_terms(const float f[8], const NvCandidate& c, float amax, float enc, float denom, float denom_inv,
                                                float term[8]) {
     float q[8];
     nv_decode8(c.word, q);
-    const float denom_inv = 1.0f / denom;
     // FASTDIV 2: every partial product of value x f32(scale) x amax is exact, one multiplication per element
     const float scale_amax = c.s_f * amax;
 #pragma unroll
@@ -264,8 +263,9 @@ __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float 
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate c4 = nv_candidate(f, s4_hp, gs.s_dec), c6 = nv_candidate(f, s6_hp, gs.s_dec);
     float t4[8], t6[8];
-    nv_error_terms<EM, FASTDIV>(f, c4, amax, gs.enc, denom, t4);
-    nv_error_terms<EM, FASTDIV>(f, c6, amax, gs.enc, denom, t6);
+    const float denom_inv = 1.0f / denom;
+    nv_error_terms<EM, FASTDIV>(f, c4, amax, gs.enc, denom, denom_inv, t4);
+    nv_error_terms<EM, FASTDIV>(f, c6, amax, gs.enc, denom, denom_inv, t6);
     const float e4 = nv_pair_error(t4, odd_lane), e6 = nv_pair_error(t6, odd_lane);
     return e4 < e6 ? c4 : c6;
 }
@@ -298,27 +298,28 @@ __device__ __forceinline__ NvCandidate16 nv_candidate16(const float f[16], float
     return c;
 }
 template <int EM, int FASTDIV>
-__device__ __forceinline__ float nv_block_error(const float f[16], const NvCandidate16& c, float amax, float enc, float denom) {
+__device__ __forceinline__ float nv_block_error(const float f[16], const NvCandidate16& c, float amax, float enc, float denom,
+                                                float denom_inv) {
     float term[8], error = 0.0f;
     NvCandidate half{c.sc, c.lo, c.s_f};
-    nv_error_terms<EM, FASTDIV>(f, half, amax, enc, denom, term);
+    nv_error_terms<EM, FASTDIV>(f, half, amax, enc, denom, denom_inv, term);
 #pragma unroll
     for (int j = 0; j < 8; j++) error = error + term[j];
     half.word = c.hi;
-    nv_error_terms<EM, FASTDIV>(f + 8, half, amax, enc, denom, term);
+    nv_error_terms<EM, FASTDIV>(f + 8, half, amax, enc, denom, denom_inv, term);
 #pragma unroll
     for (int j = 0; j < 8; j++) error = error + term[j];
     return error;
 }
 template <int EM, int FASTDIV>
 __device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], float bmax, float amax, const NvScales& gs,
-                                                            float denom) {
+                                                            float denom, float denom_inv) {
     const bool plain_bmax = shared_div_ok(bmax);
     const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate16 c4 = nv_candidate16(f, s4_hp, gs.s_dec), c6 = nv_candidate16(f, s6_hp, gs.s_dec);
-    const float e4 = nv_block_error<EM, FASTDIV>(f, c4, amax, gs.enc, denom);
-    const float e6 = nv_block_error<EM, FASTDIV>(f, c6, amax, gs.enc, denom);
+    const float e4 = nv_block_error<EM, FASTDIV>(f, c4, amax, gs.enc, denom, denom_inv);
+    const float e6 = nv_block_error<EM, FASTDIV>(f, c6, amax, gs.enc, denom, denom_inv);
     return e4 < e6 ? c4 : c6;
 }
 // error mode of a flags word, as the EM template argument
@@ -361,9 +362,13 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
     const float bmax = u2f(mb << 16);
     const float f[16] = {bf16_lo(lo.x), bf16_hi(lo.x), bf16_lo(lo.y), bf16_hi(lo.y), bf16_lo(lo.z), bf16_hi(lo.z), bf16_lo(lo.w), bf16_hi(lo.w),
                          bf16_lo(hi.x), bf16_hi(hi.x), bf16_lo(hi.y), bf16_hi(hi.y), bf16_lo(hi.z), bf16_hi(hi.z), bf16_lo(hi.w), bf16_hi(hi.w)};
-    const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom)
-                            : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom)
-                                           : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom);
+    // the error's divisor 6 * e4m3_max is one of two constants and the same for the whole launch: its reciprocal is
+    // picked on the scalar unit
+    constexpr float kInv2688 = 1.0f / 2688.0f, kInv1536 = 1.0f / 1536.0f;
+    const float denom_inv = denom == 2688.0f ? kInv2688 : denom == 1536.0f ? kInv1536 : 1.0f / denom;
+    const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom, denom_inv)
+                            : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom, denom_inv)
+                                           : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom, denom_inv);
     if (first < rem) {      // the tensor is whole blocks: both units of a block are inside or outside
         st4(q0 + first, c.lo);
         st4(q0 + first + 1, c.hi);
