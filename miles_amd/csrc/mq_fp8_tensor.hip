@@ -147,8 +147,8 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Tabl
 
 using namespace mq;
 
-int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
-int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st);
+int mq_nvfp4_amax_launch_group(int dtype, FlatTable& tab, hipStream_t st);
+int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hipStream_t st);
 
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld) {
     return dtype == MQ_BF16 && cols % 8 == 0 && ld == cols && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 &&
@@ -181,7 +181,7 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
             amax.job[i].s = (void*)(uintptr_t)(tab.job[i].units * 8);      // element count, for the amax kernel's tail
             amax.job[i].section = 0;
         }
-        int rc = mq_nvfp4_amax_launch_group(amax, st);
+        int rc = mq_nvfp4_amax_launch_group(MQ_BF16, amax, st);
         if (rc) return rc;
     }
     if (!flat_grid(tab, kFtThreads * kFtUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
@@ -191,7 +191,7 @@ int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStr
 int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st) {
     if (n == 0) return MQ_OK;
     if (!carry) {
-        int rc = mq_nvfp4_amax_launch_table(device_jobs, n, st);
+        int rc = mq_nvfp4_amax_launch_table(MQ_BF16, device_jobs, n, st);
         if (rc) return rc;
     }
     FlatRef ref{device_jobs, 0, 0};

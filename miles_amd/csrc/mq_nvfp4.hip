@@ -41,7 +41,8 @@ constexpr int kAmaxUnroll = MQ_AMAX_UNROLL;             // 16-byte units per lan
 // the section.  job.units counts whole 16-byte units; job.s carries the element count for the sub-unit tail.
 // (descriptors of a device table are in the quantizer's form, whose tensors are whole units: no tail, and job.s is the
 // block-scale pointer there)
-template <class Table>
+// (16-bit inputs, bf16 or fp16: the maximum is taken on the absolute bit patterns and converted to the fp32 pattern once)
+template <class Table, int F16>
 __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const Table tab) {
     __shared__ uint32_t wave_amax[4];
     const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(256) void nvfp4_amax_bf16_kernel(const Table tab) {
     m = wave_max(m);
     if ((t & 63) == 0) wave_amax[t >> 6] = m;
     __syncthreads();
-    if (t == 0) section[blockIdx.x] = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3])) << 16;
+    if (t == 0) section[blockIdx.x] = f2u(elem_lo<F16>(umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]))));
 }
 
 __global__ __launch_bounds__(256) void nvfp4_amax_generic_kernel(const void* __restrict__ w, int dtype, int64_t numel,
@@ -329,7 +330,7 @@ static inline int nv_error_mode(int flags) { return ((flags & MQ_NVFP4_ERR_MSE) 
 // units t and kNvThreads + t, so a wavefront's loads are contiguous), then regrouped through LDS inside each wavefront so
 // that the even lane of a pair holds the block made of units 2p, 2p + 1 and the odd lane the block kNvThreads + 2p, + 1.
 // Returns the largest |element| of the lane's block (bf16 bits).
-template <int EM>
+template <int EM, int F16>
 __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
     static_assert(kNvUnroll == 2, "the regrouping pairs the two units of a lane");
     __shared__ u32x4 stage[2 * kNvThreads];
@@ -359,9 +360,11 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
     const uint32_t m2 = max2_u16(max2_u16(max2_u16(abs2(lo.x), abs2(lo.y)), max2_u16(abs2(lo.z), abs2(lo.w))),
                                  max2_u16(max2_u16(abs2(hi.x), abs2(hi.y)), max2_u16(abs2(hi.z), abs2(hi.w))));
     const uint32_t mb = hmax_u16(m2);
-    const float bmax = u2f(mb << 16);
-    const float f[16] = {bf16_lo(lo.x), bf16_hi(lo.x), bf16_lo(lo.y), bf16_hi(lo.y), bf16_lo(lo.z), bf16_hi(lo.z), bf16_lo(lo.w), bf16_hi(lo.w),
-                         bf16_lo(hi.x), bf16_hi(hi.x), bf16_lo(hi.y), bf16_hi(hi.y), bf16_lo(hi.z), bf16_hi(hi.z), bf16_lo(hi.w), bf16_hi(hi.w)};
+    const float bmax = elem_lo<F16>(mb);
+    const float f[16] = {elem_lo<F16>(lo.x), elem_hi<F16>(lo.x), elem_lo<F16>(lo.y), elem_hi<F16>(lo.y),
+                         elem_lo<F16>(lo.z), elem_hi<F16>(lo.z), elem_lo<F16>(lo.w), elem_hi<F16>(lo.w),
+                         elem_lo<F16>(hi.x), elem_hi<F16>(hi.x), elem_lo<F16>(hi.y), elem_hi<F16>(hi.y),
+                         elem_lo<F16>(hi.z), elem_hi<F16>(hi.z), elem_lo<F16>(hi.w), elem_hi<F16>(hi.w)};
     // the error's divisor 6 * e4m3_max is one of two constants and the same for the whole launch: its reciprocal is
     // picked on the scalar unit
     constexpr float kInv2688 = 1.0f / 2688.0f, kInv1536 = 1.0f / 1536.0f;
@@ -379,9 +382,10 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
 
 // kNvThreads * kNvUnroll units starting at `base` of one tensor; returns the largest |element| this lane saw (bf16 bits)
 // FOS = 0: standard quantizer; FOS = 1 + error mode: Four Over Six
-template <int FOS>
+template <int FOS, int F16>
 __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
-    if (FOS) return nvfp4_fos_units<(FOS > 0 ? FOS - 1 : 0)>(job, base, t, denom);
+    if (FOS) return nvfp4_fos_units<(FOS > 0 ? FOS - 1 : 0), F16>(job, base, t, denom);
+    constexpr uint32_t kInfBits = F16 ? 0x7C00u : 0x7F80u;
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
@@ -412,12 +416,12 @@ __device__ __forceinline__ uint32_t nvfp4_quant_units(const FlatJob& job, const 
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max2(hmax_u16(m2));
         seen = umax(seen, mb);
-        const float bmax = u2f(mb << 16);
+        const float bmax = elem_lo<F16>(mb);
         const float s_hp = bmax == 0.0f ? 0.0f : bmax * gs.enc_sixth;
-        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                            elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
         uint32_t sc, word;
-        if (mb < 0x7F80u && s_hp == s_hp) {
+        if (mb < kInfBits && s_hp == s_hp) {
             sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
             const float s_f = hw_e4m3x2_decode<false>(sc).x;
             // 1 / (block scale x global decode scale): the refined hardware reciprocal where it equals the division (every
@@ -466,7 +470,7 @@ __device__ __forceinline__ uint32_t nvfp4_amax_units(const FlatJob& job, const i
 // atomic max per workgroup into the tensor's section, cleared by the previous fold); the fold kernel then compares, and
 // PASS 2, a small grid striding over the blocks, quantizes again only the tensors whose amax did change.
 // PASS 0 is the second pass of the plain two-pass form (amax kernel, fold, quantize).
-template <int FOS, int PASS, class Table>
+template <int FOS, int PASS, class Table, int F16>
 __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Table tab, float denom) {
     const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const int t = threadIdx.x;
@@ -476,14 +480,14 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Tabl
         // an XCD takes a run of consecutive blocks in every trip of the grid, as the flat grids do (second pass 2 pct faster)
         const int64_t first = xcd_chunked_block(gridDim.x == kSectionWords ? kSectionWords / kXcds : tab.chunk);
         for (int64_t base = first * kPerBlock; base < job.units; base += (int64_t)gridDim.x * kPerBlock)
-            nvfp4_quant_units<FOS>(job, base, t, denom);
+            nvfp4_quant_units<FOS, F16>(job, base, t, denom);
         return;
     }
     const int64_t base = flat_block(tab) * kPerBlock;
     if (base >= job.units) return;
     uint32_t seen;
     if (PASS == 1 && ((const uint32_t*)job.aux)[kRecVolatile] != 0) seen = nvfp4_amax_units(job, base, t);
-    else seen = nvfp4_quant_units<FOS>(job, base, t, denom);
+    else seen = nvfp4_quant_units<FOS, F16>(job, base, t, denom);
     if (PASS == 1) {
         __shared__ uint32_t wave_seen[kNvThreads / 64];
         seen = wave_max(seen);
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Tabl
             uint32_t m = 0;
 #pragma unroll
             for (int k = 0; k < kNvThreads / 64; k++) m = umax(m, wave_seen[k]);
-            atomicMax((uint32_t*)job.aux + job.section * kSectionWords + (blockIdx.x & (kSectionWords - 1)), m << 16);
+            atomicMax((uint32_t*)job.aux + job.section * kSectionWords + (blockIdx.x & (kSectionWords - 1)), f2u(elem_lo<F16>(m)));
         }
     }
 }
@@ -648,38 +652,50 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_qdq_kernel(const uint16_t* _
 using namespace mq;
 
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q) {
-    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 4) == 0;
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 4) == 0;
 }
 
-// tab.job[i]: w, aux = amax record, section, units = numel / 8, s = (void*)numel
-int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st) {
-    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel<FlatTable>, dim3(kSectionWords, (unsigned)tab.n), dim3(256), 0, st, tab);
+// the 16-bit dtype of a launch's tensors rides in the flags word of the launch helpers below (not a public flag)
+constexpr int kNvFlagF16 = 1 << 30;
+
+// tab.job[i]: w, aux = amax record, section, units = numel / 8, s = (void*)numel; every tensor of the one 16-bit dtype
+int mq_nvfp4_amax_launch_group(int dtype, FlatTable& tab, hipStream_t st) {
+    const dim3 grid(kSectionWords, (unsigned)tab.n), blk(256);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((nvfp4_amax_bf16_kernel<FlatTable, 1>), grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL((nvfp4_amax_bf16_kernel<FlatTable, 0>), grid, blk, 0, st, tab);
     return mq_check_launch("nvfp4 amax");
 }
 // the same over n descriptors of a device table (the quantizer's form: whole units, section = place inside the record)
-int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st) {
+int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hipStream_t st) {
     if (n == 0) return MQ_OK;
     const FlatRef ref{device_jobs, 0, 0};
-    hipLaunchKernelGGL(nvfp4_amax_bf16_kernel<FlatRef>, dim3(kSectionWords, (unsigned)n), dim3(256), 0, st, ref);
+    const dim3 grid(kSectionWords, (unsigned)n), blk(256);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((nvfp4_amax_bf16_kernel<FlatRef, 1>), grid, blk, 0, st, ref);
+    else hipLaunchKernelGGL((nvfp4_amax_bf16_kernel<FlatRef, 0>), grid, blk, 0, st, ref);
     return mq_check_launch("nvfp4 amax");
 }
 
-template <int PASS, class Table>
-static void launch_nvfp4_quant(const Table& tab, int flags, float numer, dim3 grid, hipStream_t st) {
+template <int PASS, class Table, int F16>
+static void launch_nvfp4_quant_dtype(const Table& tab, int flags, float numer, dim3 grid, hipStream_t st) {
     const dim3 blk(kNvThreads);
     // Four Over Six keeps to launches of kernel-argument tables (its five error modes are not built in the other form)
     const int fos = (flags & MQ_NVFP4_4OVER6) ? 1 + nv_error_mode(flags) : 0;
     if constexpr (std::is_same<Table, FlatRef>::value) {
-        hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table>), grid, blk, 0, st, tab, numer);
+        hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table, F16>), grid, blk, 0, st, tab, numer);
     } else {
         switch (fos) {
-            case 0: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table>), grid, blk, 0, st, tab, numer); break;
-            case 1: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<1, PASS, Table>), grid, blk, 0, st, tab, numer); break;
-            case 2: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<2, PASS, Table>), grid, blk, 0, st, tab, numer); break;
-            case 3: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<3, PASS, Table>), grid, blk, 0, st, tab, numer); break;
-            default: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<4, PASS, Table>), grid, blk, 0, st, tab, numer); break;
+            case 0: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<0, PASS, Table, F16>), grid, blk, 0, st, tab, numer); break;
+            case 1: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<1, PASS, Table, F16>), grid, blk, 0, st, tab, numer); break;
+            case 2: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<2, PASS, Table, F16>), grid, blk, 0, st, tab, numer); break;
+            case 3: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<3, PASS, Table, F16>), grid, blk, 0, st, tab, numer); break;
+            default: hipLaunchKernelGGL((nvfp4_quant_bf16_kernel<4, PASS, Table, F16>), grid, blk, 0, st, tab, numer); break;
         }
     }
+}
+template <int PASS, class Table>
+static void launch_nvfp4_quant(const Table& tab, int flags, float numer, dim3 grid, hipStream_t st) {
+    if (flags & kNvFlagF16) launch_nvfp4_quant_dtype<PASS, Table, 1>(tab, flags, numer, grid, st);
+    else launch_nvfp4_quant_dtype<PASS, Table, 0>(tab, flags, numer, grid, st);
 }
 
 // fold + quantize (+ second pass) over a table whose grid is known: tab.chunk / tab.max_blocks are set
@@ -709,16 +725,17 @@ static int nvfp4_quant_launch(const Table& tab, int n, int e4m3_max, int flags, 
 //   record (adjacent entries); fold once per record, clear the sections, quantize.
 // mode 2 (job driver, carried-over amax; the sections were cleared by the previous sync's fold): quantize with the
 //   record's old scales while collecting the new partial maxima, fold and compare, quantize again where they differ.
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st) {
+int mq_nvfp4_quant_launch_group(int dtype, FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st) {
     if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    return nvfp4_quant_launch(tab, tab.n, e4m3_max, flags, mode, st);
+    return nvfp4_quant_launch(tab, tab.n, e4m3_max, flags | (dtype == MQ_F16 ? kNvFlagF16 : 0), mode, st);
 }
 // modes 1 and 2 over n descriptors of a device table (standard block scaling only); max_units: the largest tensor's units
-int mq_nvfp4_quant_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode, hipStream_t st) {
+int mq_nvfp4_quant_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode,
+                                hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (n == 0) return MQ_OK;
-    return nvfp4_quant_launch(ref, n, e4m3_max, 0, mode, st);
+    return nvfp4_quant_launch(ref, n, e4m3_max, dtype == MQ_F16 ? kNvFlagF16 : 0, mode, st);
 }
 
 extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* record, int section, void* stream) {
@@ -726,11 +743,11 @@ extern "C" int mq_nvfp4_amax(const void* w, int dtype, int64_t numel, void* reco
     if (dtype < MQ_BF16 || dtype > MQ_F32 || numel < 0) return mq_fail(MQ_ERR_ARG, "bad argument");
     if (section < 0 || section >= MQ_NVFP4_SECTIONS) return mq_fail(MQ_ERR_ARG, "bad amax record section");
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0) {
+    if ((dtype == MQ_BF16 || dtype == MQ_F16) && ((uintptr_t)w % 16) == 0) {
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, nullptr, (void*)(uintptr_t)numel, record, numel / 8, nullptr, section, 0};
-        return mq_nvfp4_amax_launch_group(tab, st);
+        return mq_nvfp4_amax_launch_group(dtype, tab, st);
     }
     hipLaunchKernelGGL(nvfp4_amax_generic_kernel, dim3(kSectionWords), dim3(256), 0, st, w, dtype, numel,
                        (uint32_t*)record + section * kSectionWords);
@@ -752,7 +769,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), blocks16 * 2, global_scale, n_sections, 0};
-        return mq_nvfp4_quant_launch_group(tab, e4m3_max, flags, 0, st);
+        return mq_nvfp4_quant_launch_group(blocks16 == 0 ? MQ_BF16 : dtype, tab, e4m3_max, flags, 0, st);
     }
     FlatTable fold{};
     fold.n = 1;

@@ -27,15 +27,16 @@ int mq_mxfp8_launch_group(int dtype, FlatTable& tab, hipStream_t st);
 bool mq_int4_pack_fast_ok(const void* w, int dtype, int group);
 int mq_int4_pack_launch_group(int dtype, FlatTable& tab, int group, hipStream_t st);
 bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
-int mq_nvfp4_amax_launch_group(FlatTable& tab, hipStream_t st);
-int mq_nvfp4_quant_launch_group(FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st);
+int mq_nvfp4_amax_launch_group(int dtype, FlatTable& tab, hipStream_t st);
+int mq_nvfp4_quant_launch_group(int dtype, FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
 int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
 int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st);
-int mq_nvfp4_amax_launch_table(const FlatJob* device_jobs, int n, hipStream_t st);
-int mq_nvfp4_quant_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode, hipStream_t st);
+int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hipStream_t st);
+int mq_nvfp4_quant_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode,
+                                hipStream_t st);
 int mq_mxfp8_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_int4_pack_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
@@ -284,7 +285,7 @@ static int run_nvfp4(const mq_job* jobs, int64_t n_all, int64_t i, int64_t j, co
                 }
                 const bool ragged = nmx * (r - i) * 4 > (bytes + b) * 5;
                 if (k > i && (r - i > cap || bytes + b > kNvfp4GroupBytes || jobs[k].p0 != jobs[i].p0 ||
-                              jobs[k].p1 != jobs[i].p1 || ragged))
+                              jobs[k].p1 != jobs[i].p1 || jobs[k].dtype != jobs[i].dtype || ragged))
                     break;
                 mx = nmx;
                 bytes += b;
@@ -293,8 +294,8 @@ static int run_nvfp4(const mq_job* jobs, int64_t n_all, int64_t i, int64_t j, co
             return k;
         };
         auto all_fast_in = [&](int64_t k) {
-            for (int64_t t = i; t < k; t++)
-                if (!job_fast(jobs[t])) return false;
+            for (int64_t t = i; t < k; t++)       // (the packed kernels are compiled per 16-bit dtype: one per launch)
+                if (!job_fast(jobs[t]) || jobs[t].dtype != jobs[i].dtype) return false;
             return true;
         };
         // a device table lifts the limit for standard block scaling when every job takes the packed kernels
@@ -325,9 +326,9 @@ static int run_nvfp4(const mq_job* jobs, int64_t n_all, int64_t i, int64_t j, co
                     const int64_t u = jobs[i + t].rows * jobs[i + t].cols / 8;
                     max_units = u > max_units ? u : max_units;
                 }
-                if (!carry) rc = mq_nvfp4_amax_launch_table(table + i, n, st);
+                if (!carry) rc = mq_nvfp4_amax_launch_table(jobs[i].dtype, table + i, n, st);
                 if (rc) return rc;
-                rc = mq_nvfp4_quant_launch_table(table + i, n, max_units, jobs[i].p0, carry ? 2 : 1, st);
+                rc = mq_nvfp4_quant_launch_table(jobs[i].dtype, table + i, n, max_units, jobs[i].p0, carry ? 2 : 1, st);
                 if (rc) return rc;
                 i = k;
                 continue;
@@ -340,14 +341,14 @@ static int run_nvfp4(const mq_job* jobs, int64_t n_all, int64_t i, int64_t j, co
                     const int64_t numel = jb.rows * jb.cols;
                     tab.job[t] = FlatJob{jb.in, nullptr, (void*)(uintptr_t)numel, jb.aux, numel / 8, nullptr, section[t], 0};
                 }
-                rc = mq_nvfp4_amax_launch_group(tab, st);
+                rc = mq_nvfp4_amax_launch_group(jobs[i].dtype, tab, st);
                 if (rc) return rc;
             }
             for (int t = 0; t < n; t++) {
                 const mq_job& jb = jobs[i + t];
                 tab.job[t] = FlatJob{jb.in, jb.out, jb.scale, jb.aux, jb.rows * jb.cols / 8, jb.aux2, section[t], sections[t]};
             }
-            rc = mq_nvfp4_quant_launch_group(tab, jobs[i].p0, jobs[i].p1 & ~MQ_NVFP4_CARRY_AMAX, carry ? 2 : 1, st);
+            rc = mq_nvfp4_quant_launch_group(jobs[i].dtype, tab, jobs[i].p0, jobs[i].p1 & ~MQ_NVFP4_CARRY_AMAX, carry ? 2 : 1, st);
             if (rc) return rc;
         } else {
             for (int t = 0; t < n; t++) {

@@ -127,13 +127,19 @@ class JobBatch:
         """After this list has run once: let later runs of the same list quantize NVFP4 and per-tensor FP8 tensors in
         one pass with the amax their record kept from the run before (MQ_NVFP4_CARRY_AMAX; the driver checks the amax on
         the way and quantizes a tensor again if it moved, so results do not change).  NVFP4 jobs are only flagged when
-        every one of the list is one the packed kernels take (bf16, 16-byte aligned input, 4-byte aligned codes), so
+        every one of the list is one the packed kernels take (bf16 or fp16, one dtype per record, 16-byte aligned input,
+        4-byte aligned codes), so
         that every record goes through the same driver path on every run; per-tensor FP8 jobs always are.
         With `adaptive` the batch also watches how many records moved per sync (`_AmaxFeedback`) and submits the plain
         two-pass form while most of them keep moving.  Returns the number of jobs flagged."""
         nv = [r for r in self._records if r[self.KIND] == _lib.JOB_NVFP4]
-        nv_fit = bool(nv) and all(r[self.DTYPE] == _lib.DTYPE_CODE[torch.bfloat16] and (r[self.IN] or 0) % 16 == 0
-                                  and (r[self.OUT] or 0) % 4 == 0 and r[self.COLS] % 16 == 0 for r in nv)
+        packed_dtypes = (_lib.DTYPE_CODE[torch.bfloat16], _lib.DTYPE_CODE[torch.float16])
+        record_dtypes: dict = {}
+        for r in nv:
+            record_dtypes.setdefault(r[self.AUX], set()).add(r[self.DTYPE])
+        nv_fit = (bool(nv) and all(len(d) == 1 for d in record_dtypes.values())
+                  and all(r[self.DTYPE] in packed_dtypes and (r[self.IN] or 0) % 16 == 0
+                          and (r[self.OUT] or 0) % 4 == 0 and r[self.COLS] % 16 == 0 for r in nv))
         kinds = {_lib.JOB_FP8_TENSOR} | ({_lib.JOB_NVFP4} if nv_fit else set())
         flagged = sum(r[self.KIND] in kinds for r in self._records)
         if flagged:

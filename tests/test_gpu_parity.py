@@ -1500,8 +1500,81 @@ def test_empty_tensors(oracle, shape):
 # ---------------------------------------------------------------------------------------------------
 # NVFP4 with the amax carried over from the previous run of the same job list: one pass when the amax did not move,
 # a second quantization of exactly the tensors whose amax did -- the results must never depend on which happened
+@pytest.mark.parametrize("fos", [None, (448, "MAE", False), (256, "MSE", False), (256, "MAE", True)],
+                         ids=["standard", "fos448", "fos256mse", "fos256f16err"])
+def test_nvfp4_reads_fp16(oracle, monkeypatch, fos):
+    """fp16 tensors take the packed NVFP4 kernels' fp16 instances (amax pass, quantizer, Four Over Six): blocks of
+    subnormals, of zeros, the format's extremes, every block its own magnitude; single calls, a gate / up pair, and a
+    recorded list of more than 64 jobs (device table where the mode has one) in which bf16 and fp16 tensors alternate,
+    run twice and then with the amax carried over."""
+    from miles_amd import launch
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
+
+    for name in ("NVTE_NVFP4_4OVER6", "NVTE_NVFP4_4OVER6_E4M3_USE_256", "NVTE_NVFP4_4OVER6_ERR_MODE",
+                 "NVTE_NVFP4_4OVER6_ERR_USE_FAST_MATH", "NVTE_USE_FAST_MATH"):
+        monkeypatch.delenv(name, raising=False)
+    kw = {}
+    if fos:
+        _fos_env(monkeypatch, *fos)
+        kw = {"e4m3_max": fos[0], "flags": oracle.NVFP4_4OVER6 | (oracle.NVFP4_ERR_MSE if fos[1] == "MSE" else 0)
+              | (oracle.NVFP4_ERR_FP16 if fos[2] else 0)}
+
+    def case(shape, seed, top):
+        g = torch.Generator().manual_seed(seed)
+        rows, cols = shape
+        ex = torch.randint(-14, 1, (rows, cols // 16, 1), generator=g).float()
+        w = (torch.randn(rows, cols // 16, 16, generator=g) * torch.exp2(ex)).reshape(rows, cols) * top
+        w = w.clamp(-65504, 65504).to(torch.float16)
+        w[0, :16] = 0
+        w[0, 16:32] = torch.arange(1, 17, dtype=torch.int16).view(torch.float16)      # a block of subnormals
+        if rows > 2:
+            w[2, 5] = 65504.0 if top > 100 else w[2, 5]
+            w[1] = 0
+        return w
+
+    for shape, top in (((1, 32), 1.0), ((64, 128), 1.0), ((200, 1024), 3000.0), ((37, 7168), 0.01)):
+        w = case(shape, 77 + shape[1], top)
+        got, want = nvfp4_quantize_1d(w.to(DEV)), oracle.nvfp4_quantize_1d(w, **kw)
+        for k, (a, b) in enumerate(zip(got, want)):
+            _assert_same(a, b, f"{shape} output {k}")
+    gate, up = case((96, 256), 5, 1.0), case((96, 256), 6, 40.0)
+    got, want = nvfp4_quantize_1d_pair(gate.to(DEV), up.to(DEV)), oracle.nvfp4_quantize_1d_pair(gate, up, **kw)
+    for half in range(2):
+        for k, (a, b) in enumerate(zip(got[half], want[half])):
+            _assert_same(a, b, f"pair half {half} output {k}")
+    tensors = []
+    for i in range(80):
+        t = case((24 + i % 5, 256), 300 + i, 1.0 + i % 7)
+        tensors.append(t if (i % 3 == 0 or i >= 50) else t.float().to(torch.bfloat16))
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [nvfp4_quantize_1d(t) for t in dev]
+    batch.device = torch.device(DEV)
+    batch.freeze()
+    want = [oracle.nvfp4_quantize_1d(t, **kw) for t in tensors]
+    for what in ("first run", "second run", "carried"):
+        if what == "carried":
+            assert batch.carry_amax() == len(tensors)
+        for o in outs:
+            for t in o[:2]:
+                t.view(torch.uint8).fill_(0x5A)
+        batch.run()
+        torch.cuda.synchronize()
+        for i, (o, wnt) in enumerate(zip(outs, want)):
+            for k, (a, b) in enumerate(zip(o, wnt)):
+                _assert_same(a, b, f"list tensor {i} ({tensors[i].dtype}) output {k}, {what}")
+    dev[3].mul_(2.0)            # an fp16 tensor's amax moves: quantized again with the new one
+    dev[60].mul_(0.5)
+    batch.run()
+    torch.cuda.synchronize()
+    for i in (3, 4, 60, 79):
+        for k, (a, b) in enumerate(zip(outs[i], oracle.nvfp4_quantize_1d(dev[i].cpu(), **kw))):
+            _assert_same(a, b, f"list tensor {i} output {k}, after its amax moved")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("four_over_six", [False, True])
-def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
+def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six, dtype):
     from miles_amd import launch
     from miles_amd.utils.nvfp4 import nvfp4_quantize_1d, nvfp4_quantize_1d_pair
 
@@ -1512,8 +1585,8 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six):
         monkeypatch.setenv("NVTE_NVFP4_4OVER6", "weights")
         kw = {"e4m3_max": 256, "flags": 1}
     shapes = [(256, 512), (384, 1024), (100, 256), (64, 2048), (512, 512), (128, 7168)]
-    cpu = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=1200 + i) for i, s in enumerate(shapes)]
-    pair_cpu = [W.gaussian_outliers((320, 768), std=0.02, p_outlier=0.001, gain=20.0, seed=1250 + i) for i in range(2)]
+    cpu = [W.gaussian_outliers(s, std=0.02, p_outlier=0.001, gain=20.0, seed=1200 + i, dtype=dtype) for i, s in enumerate(shapes)]
+    pair_cpu = [W.gaussian_outliers((320, 768), std=0.02, p_outlier=0.001, gain=20.0, seed=1250 + i, dtype=dtype) for i in range(2)]
     dev, pair_dev = [w.to(DEV) for w in cpu], [w.to(DEV) for w in pair_cpu]
     with launch.recording() as batch:
         outs = [nvfp4_quantize_1d(w) for w in dev[:3]]
