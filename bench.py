@@ -187,6 +187,16 @@ def per_quantizer(gen):
     run("C5b_fp8_dequant", "fp8_dequant", n, lambda: [weight_dequant(q, s) for q, s in quantized],
         "32 experts, FP8 block -> bf16")
     del quantized
+    # the same four quantizers on fp16 weights (a model trained in fp16): their kernels have fp16 instances
+    half = [(_synth((4096, 7168), gen, p=0).to(torch.float16), _synth((7168, 2048), gen, p=0).to(torch.float16)) for _ in range(32)]
+    parts = lambda: [t for fc1, fc2 in half for t in (*fc1.chunk(2, dim=0), fc2)]
+    note = "32 DeepSeek-V3-shaped experts held in fp16"
+    run("fp16_weights_fp8_blockwise_cast", "fp8_block", n, lambda: [fp8_blockwise_cast(t) for t in parts()], note)
+    run("fp16_weights_mxfp8", "mxfp8", n, lambda: [mxfp8_quantize(t) for t in parts()], note)
+    run("fp16_weights_int4_g128_pack", "int4_g128", n, lambda: [pack_layer(t, 128) for t in parts()], note)
+    run("fp16_weights_nvfp4", "nvfp4", n, lambda: [nvfp4_quantize_1d(t) for t in parts()], note + ", amax carried over",
+        prepare=lambda b: b.carry_amax())
+    del half
     res.update(adjacent_formats(gen))
     return res
 
