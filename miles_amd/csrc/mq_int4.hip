@@ -348,19 +348,27 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 __device__ __forceinline__ float order_unkey(uint32_t k) {
     return u2f(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
 }
-__device__ __forceinline__ void rd_bf16x2(float& a, float& b) {
-    const uint32_t p = hw_bf16x2(a, b);
-    a = bf16_lo(p);
-    b = bf16_hi(p);
+// two values rounded to the tensor's 16-bit dtype (bf16: the packed hardware conversion)
+template <int F16>
+__device__ __forceinline__ void rd16x2(float& a, float& b) {
+    if (F16) {
+        a = (float)(_Float16)a;
+        b = (float)(_Float16)b;
+    } else {
+        const uint32_t p = hw_bf16x2(a, b);
+        a = bf16_lo(p);
+        b = bf16_hi(p);
+    }
 }
 // One 16-byte unit of one lane, LANES neighbouring lanes hold the rest of the group: the chain as written, with IEEE
 // divisions.  The packed kernel sends here the wavefronts that met a group outside its fused form (minimum above zero
 // or far below it, huge scales, infinities, NaN).
-template <int LANES>
+template <int LANES, int F16>
 __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, const int64_t unit, const int t,
                                                uint32_t* __restrict__ packed, uint16_t* __restrict__ scale_out,
                                                uint8_t* __restrict__ zero_out) {
-    float f[8] = {bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y), bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+    float f[8] = {elem_lo<F16>(v.x), elem_hi<F16>(v.x), elem_lo<F16>(v.y), elem_hi<F16>(v.y),
+                  elem_lo<F16>(v.z), elem_hi<F16>(v.z), elem_lo<F16>(v.w), elem_hi<F16>(v.w)};
     float mx = f[0], mn = f[0];
 #pragma unroll
     for (int i = 1; i < 8; i++) { mx = __builtin_fmaxf(mx, f[i]); mn = __builtin_fminf(mn, f[i]); }
@@ -369,37 +377,37 @@ __device__ __forceinline__ void int4_asym_unit(const u32x4 v, const bool live, c
     mx = order_unkey(seg_max<LANES>(order_key(mx)));
     mn = order_unkey(~seg_max<LANES>(~order_key(mn)));
     const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
-    const float sb = u2f(sw_bf16(s) << 16);
+    const float sb = round16<F16>(s);
     const float z = __builtin_fminf(__builtin_fmaxf(-__builtin_rintf(mn / s), 0.0f), 15.0f) + 0.0f;
     uint32_t word = 0;
     float q[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = __builtin_rintf(f[i] / s) + z;
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i += 2) rd16x2<F16>(q[i], q[i + 1]);
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = q[i] - z;
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i += 2) rd16x2<F16>(q[i], q[i + 1]);
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = q[i] * sb;
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i += 2) rd16x2<F16>(q[i], q[i + 1]);
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = q[i] / sb;
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i += 2) rd16x2<F16>(q[i], q[i + 1]);
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = q[i] + z;
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) rd_bf16x2(q[i], q[i + 1]);
+    for (int i = 0; i < 8; i += 2) rd16x2<F16>(q[i], q[i + 1]);
 #pragma unroll
     for (int i = 0; i < 8; i++)
         word += (uint32_t)__builtin_rintf(clamp_keep_nan(q[i], 0.0f, 255.0f)) << (4 * i);
     if (live) {
         st4(packed + unit, word);
         if ((t & (LANES - 1)) == 0) {
-            scale_out[unit / LANES] = (uint16_t)sw_bf16(s);
+            scale_out[unit / LANES] = bits16<F16>(s);
             zero_out[unit / LANES] = (uint8_t)z;
         }
     }
@@ -445,7 +453,9 @@ __device__ __forceinline__ void seg_extrema(float& mx, float& mn) {
 // dequantize / requantize round trip in bf16 returns the code itself (checked exhaustively on the CPU: all scales x
 // all codes x all zero points).  A wavefront that met any other group (minimum above zero or far below it, huge or
 // non-finite values) writes its groups again through int4_asym_unit, the chain as written; the later store wins.
-template <int LANES, class Table>
+// (fp16 instance, F16: the same check over every fp16 scale from fp16(1e-5) upwards holds for all scales below 4096,
+// where 16 x scale stays finite; a group with a larger scale takes the chain.)
+template <int LANES, class Table, int F16>
 __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const Table tab) {
     const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
@@ -475,8 +485,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
     uint32_t word[kI4Unroll], sb[kI4Unroll], z[kI4Unroll];
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
-        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                            elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
         float mx = f[0], mn = f[0];
 #pragma unroll
         for (int j = 1; j < 8; j++) { mx = __builtin_fmaxf(mx, f[j]); mn = __builtin_fminf(mn, f[j]); }
@@ -487,7 +497,8 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
         seg_extrema<LANES>(mx, mn);
         const float s = __builtin_fmaxf((mx - mn) * kAsymCons, 1e-5f);
         const float ys = recip_shared(s);
-        sb[i] = hw_bf16x2(s, 0.0f);
+        sb[i] = F16 ? (uint32_t)bits16<1>(s) : hw_bf16x2(s, 0.0f);
+        if (F16) odd |= __builtin_amdgcn_ballot_w64(!(s < 4094.0f));        // fp16(s) below 4096: 16 x scale stays finite
         // The zero point unclamped: lo = rint(min / s) in [-15, 0].  Every quotient of the group then lies within +-16,
         // far from the range limits of the shared-divisor sequence, and bf16(s) <= 2^90 (1 + 2^-8) is far below 1e37.
         // One infinite extremum makes s infinite, which shared_div_ok refuses; a group of equal infinities has the
@@ -526,7 +537,7 @@ __global__ __launch_bounds__(kI4Threads) void int4_pack_asym_bf16_kernel(const T
 #pragma unroll
     for (int i = 0; i < kI4Unroll; i++) {
         const int64_t unit = base + i * kI4Threads;
-        int4_asym_unit<LANES>(v[i], unit < total_units, unit, t, packed, scale_out, zero_out);
+        int4_asym_unit<LANES, F16>(v[i], unit < total_units, unit, t, packed, scale_out, zero_out);
     }
 }
 
@@ -828,7 +839,7 @@ extern "C" int mq_int4_group_quant_pack(const void* w, int dtype, int32_t* packe
 }
 
 bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M) {
-    return dtype == MQ_BF16 && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32) && M % 8 == 0;
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && ((uintptr_t)w % 16) == 0 && (group == 128 || group == 64 || group == 32) && M % 8 == 0;
 }
 
 // tiles of the zero-point packer for a [rows, cols] tensor with groups of `group` elements
@@ -837,17 +848,23 @@ int64_t mq_int4_zero_tiles(int64_t rows, int64_t cols, int group) { return int4_
 // The two launches of an asymmetric pack for a group of tensors: codes + scales + zero points, then the zero points
 // packed eight rows to a word.  max_tiles: the most tiles the second launch has to cover in one tensor.
 template <class Table>
-static int int4_pack_asym_launch(const Table& tab, int n, int64_t max_tiles, int group, hipStream_t st) {
+static int int4_pack_asym_launch(int dtype, const Table& tab, int n, int64_t max_tiles, int group, hipStream_t st) {
     const dim3 grid((unsigned)tab.max_blocks, (unsigned)n), blk(kI4Threads);
-    if (group == 128) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<16, Table>), grid, blk, 0, st, tab);
-    else if (group == 64) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<8, Table>), grid, blk, 0, st, tab);
-    else hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<4, Table>), grid, blk, 0, st, tab);
+    if (dtype == MQ_F16) {
+        if (group == 128) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<16, Table, 1>), grid, blk, 0, st, tab);
+        else if (group == 64) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<8, Table, 1>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<4, Table, 1>), grid, blk, 0, st, tab);
+    } else {
+        if (group == 128) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<16, Table, 0>), grid, blk, 0, st, tab);
+        else if (group == 64) hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<8, Table, 0>), grid, blk, 0, st, tab);
+        else hipLaunchKernelGGL((int4_pack_asym_bf16_kernel<4, Table, 0>), grid, blk, 0, st, tab);
+    }
     int rc = mq_check_launch("int4 asymmetric pack");
     if (rc != MQ_OK) return rc;
     hipLaunchKernelGGL(int4_zero_pack_group_kernel<Table>, dim3((unsigned)max_tiles, (unsigned)n), dim3(256), 0, st, tab, group / 8);
     return mq_check_launch("int4 zero-point pack");
 }
-int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st) {
+int mq_int4_pack_asym_launch_group(int dtype, FlatTable& tab, int group, hipStream_t st) {
     if (!flat_grid(tab, kI4Threads * kI4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
     int64_t max_tiles = 1;
@@ -858,15 +875,15 @@ int mq_int4_pack_asym_launch_group(FlatTable& tab, int group, hipStream_t st) {
         max_tiles = tiles > max_tiles ? tiles : max_tiles;
     }
     if (max_tiles >= 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    return int4_pack_asym_launch(tab, tab.n, max_tiles, group, st);
+    return int4_pack_asym_launch(dtype, tab, tab.n, max_tiles, group, st);
 }
 // max_units: the largest tensor's 16-byte units; max_zero_tiles: the largest mq_int4_zero_tiles of the tensors
-int mq_int4_pack_asym_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, int64_t max_zero_tiles, int group,
-                                   hipStream_t st) {
+int mq_int4_pack_asym_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int64_t max_zero_tiles,
+                                   int group, hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kI4Threads * kI4Unroll) || max_zero_tiles >= 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (ref.max_blocks == 0 || n == 0) return MQ_OK;
-    return int4_pack_asym_launch(ref, n, max_zero_tiles < 1 ? 1 : max_zero_tiles, group, st);
+    return int4_pack_asym_launch(dtype, ref, n, max_zero_tiles < 1 ? 1 : max_zero_tiles, group, st);
 }
 
 extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* packed, void* scale, uint8_t* zero,
@@ -886,7 +903,7 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, packed, scale, zero, M * (K / 8), packed_zp, (int32_t)gpr, 0};
-        return mq_int4_pack_asym_launch_group(tab, group, st);
+        return mq_int4_pack_asym_launch_group(dtype, tab, group, st);
     } else if (dtype == MQ_BF16)
         hipLaunchKernelGGL(int4_pack_asym_kernel<MQ_BF16>, dim3((unsigned)blocks), dim3(256), 0, st, w, (uint32_t*)packed, scale, zero, groups, wpg, aligned);
     else if (dtype == MQ_F16)

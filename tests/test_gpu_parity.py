@@ -513,6 +513,61 @@ def test_int4_pack_layer_asymmetric_shifted_groups(oracle, G):
     _assert_same(packed, packed_o, "packed")
 
 
+@pytest.mark.parametrize("G", [32, 64, 128])
+def test_int4_pack_layer_asymmetric_fp16(oracle, G):
+    """The asymmetric packer's fp16 instance: zero points from clamped-at-15 to clamped-at-0 (the fused form ends exactly
+    at an unclamped zero point), scales around 4096 where 16 x scale leaves fp16 (those groups take the written-out
+    chain), the format's extremes, groups of subnormals, infinities and NaN next to ordinary groups; then bf16 and fp16
+    tensors alternating in one recorded job list."""
+    from miles_amd import launch
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+
+    rows, cols = 64, 2048
+    gen = torch.Generator().manual_seed(4301)
+    w = torch.randn(rows, cols, generator=gen) * 0.02
+    groups = w.view(rows, cols // G, G)
+    span = groups.amax(-1, keepdim=True) - groups.amin(-1, keepdim=True)
+    k = (torch.arange(rows * (cols // G), dtype=torch.float32).view(rows, cols // G, 1) % 97) * 0.25 - 4.0
+    groups += -groups.amin(-1, keepdim=True) - k / 15.0 * span
+    w = groups.reshape(rows, cols).to(torch.float16)
+    for i, top in enumerate((61000.0, 61400.0, 61440.0, 61500.0, 65504.0, 30000.0)):     # scales 4066 ... 4367 and 2000
+        w[16 + i, :G] = torch.linspace(0.0, top, G).to(torch.float16)
+        w[24 + i, G:2 * G] = torch.linspace(-top / 2, top / 2, G).to(torch.float16)
+    w[32, :G] = torch.linspace(-65504, 65504, G).to(torch.float16)
+    w[33, :32] = torch.arange(1, 33, dtype=torch.int16).view(torch.float16)              # subnormals: the scale floor
+    w[34, :G] = 65504.0
+    w[35, 3] = float("inf")
+    w[36, 5] = float("-inf")
+    w[37, 7] = float("nan")
+    w[38, :G] = float("inf")
+    w[39, :G] = float("nan")
+    packed, scale, zp = pack_layer(w.to(DEV), G, sym=False)
+    packed_o, scale_o, zp_o = oracle.pack_layer(w, G, sym=False)
+    assert scale.dtype == torch.float16
+    _assert_same(scale, scale_o, "scales")
+    _assert_same(zp, zp_o, "packed zero points")
+    _assert_same(packed, packed_o, "packed")
+    tensors = []
+    for i in range(9):
+        t = W.gaussian_outliers((32, 1024), std=0.015, p_outlier=0.0005, gain=30.0, seed=4400 + i, dtype=torch.float16)
+        t[1] = t[1].abs() + 0.25
+        t[2] = -t[2].abs() - 0.25
+        tensors.append(t if i % 3 else t.float().to(torch.bfloat16))
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [pack_layer(t, G, sym=False) for t in dev]
+    batch.freeze()
+    for rep in range(2):
+        for o in outs:
+            for t in o:
+                t.view(torch.uint8).fill_(0x5A)
+        batch.run()
+        torch.cuda.synchronize()
+        for i, t in enumerate(tensors):
+            for got, want, what in zip(outs[i], oracle.pack_layer(t, G, sym=False), ("packed", "scales", "zero points")):
+                _assert_same(got, want, f"tensor {i} ({t.dtype}) {what}, run {rep}")
+
+
 def test_int4_pack_layer_asymmetric_argument_checks():
     from miles_amd.kernels.quant.int4_fake import pack_layer
 

@@ -544,6 +544,23 @@ def test_int4_asym_round_trip_is_identity_for_unclamped_codes():
             assert torch.all(code == w1), (z, w1)
 
 
+def test_int4_asym_round_trip_in_fp16_is_identity_for_scales_below_4096():
+    # The fp16 instance of the asymmetric packer emits rint(x/s) + z directly when the zero point was not clamped (codes
+    # in [0, 16]) and the scale is below 4094 (so that fp16(s) < 4096).  Exhaustive over every fp16 scale from the floor,
+    # every code and zero point: the reference's chain in fp16 returns the code for every scale below 4096 and fails
+    # from 4096 on, where 16 x scale is no longer finite.
+    sb = torch.arange(1, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    sb = sb[sb >= torch.tensor(1e-5, dtype=torch.float16)]
+    bad = torch.zeros(sb.shape, dtype=torch.bool)
+    for z in range(16):
+        zt = torch.tensor(float(z), dtype=torch.float16)
+        for w1 in range(17):
+            w = torch.tensor(float(w1), dtype=torch.float16)
+            r = ((w - zt) * sb) / sb + zt
+            bad |= torch.round(torch.clamp(r, 0, 255)).to(torch.int16) != w1
+    assert bad.any() and sb[bad].min().item() == 4096.0 and not bad[sb.float() < 4096.0].any()
+
+
 def test_int4_sym_round_trip_in_fp16_is_identity_below_the_overflow():
     # The fp16 instance of the symmetric packer emits rint(x/s) + 8 directly.  Exhaustive over every fp16 scale from the
     # floor fp16(1e-5) (a subnormal) upwards and the fifteen codes: the reference's chain in fp16
