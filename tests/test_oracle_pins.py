@@ -462,6 +462,29 @@ def test_int4_asym_matches_torch_chain(oracle, shape, G, dtype):
     assert pzp.shape == (shape[1] // G, shape[0] // 8) and torch.equal(pzp, pzp_t)
 
 
+@pytest.mark.parametrize("G", [32, 128])
+def test_int4_fp16_overflow_corners_match_torch_chain(oracle, G):
+    # fp16 weights whose round trip in pack_layer leaves the finite range: a group maximum of 65504 (7 x scale rounds to
+    # infinity in the symmetric chain) and ranges whose scale reaches 4096 (16 x scale in the asymmetric chain).  The
+    # oracle against the torch op chains on exactly those groups, next to ordinary ones.
+    w = W.gaussian_outliers((16, 4 * G), std=0.015, p_outlier=0.0, gain=1.0, seed=4501, dtype=torch.float16)
+    w[1, :G] = torch.linspace(-65504, 65504, G).to(torch.float16)
+    w[2, 5] = 65504.0
+    w[3, :G] = 65504.0
+    for i, top in enumerate((61000.0, 61400.0, 61440.0, 61500.0, 65504.0)):
+        w[4 + i, :G] = torch.linspace(0.0, top, G).to(torch.float16)
+        w[9 + i, G:2 * G] = torch.linspace(-top / 2, top / 2, G).to(torch.float16)
+    out_t, scale_t = torch_fake_int4_sym(w, G)
+    packed, pscale, _ = oracle.pack_layer(w, G)
+    packed_t, pscale_t = torch_pack_layer_python_half(out_t, scale_t, G)
+    assert torch.equal(packed, packed_t) and torch.equal(pscale.view(torch.int16), pscale_t.view(torch.int16))
+    out_t, scale_t, zero_t = torch_fake_int4_asym(w, G)
+    packed, pscale, pzp = oracle.pack_layer(w, G, sym=False)
+    packed_t, pscale_t, pzp_t = torch_pack_layer_asym_python_half(out_t, scale_t, zero_t, G)
+    assert torch.equal(packed, packed_t) and torch.equal(pscale.view(torch.int16), pscale_t.view(torch.int16))
+    assert torch.equal(pzp, pzp_t)
+
+
 def test_int4_asym_known_answers(oracle):
     # a group spanning [0, 15] exactly: scale 1, zero 0, codes are the values themselves
     row = torch.arange(16, dtype=torch.float32).repeat(8)
