@@ -735,6 +735,35 @@ def test_int4_fake_quant_general_blocks_match_torch_chain(oracle, shape, block, 
         assert torch.equal(zero.view(bits), zero_t.view(bits))
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_fp16_inputs_match_the_torch_chains(oracle, seed):
+    # the oracle's reading of fp16 tensors (what the fp16 instances of the GPU kernels are compared with): every block its
+    # own magnitude, subnormals, the format's extremes and zero blocks, against the same torch op chains
+    g = torch.Generator().manual_seed(9000 + seed)
+    rows, cols = 130, 512
+    ex = torch.randint(-20, 12, (rows, cols // 16, 1), generator=g).float()
+    w = (torch.randn(rows, cols // 16, 16, generator=g) * torch.exp2(ex)).reshape(rows, cols).clamp(-65504, 65504).to(torch.float16)
+    w[0] = 0
+    w[1, :32] = torch.arange(1, 33, dtype=torch.int16).view(torch.float16)
+    w[2, :4] = torch.tensor([65504.0, -65504.0, 0.0, -0.0], dtype=torch.float16)
+    y, s = oracle.fp8_blockwise_cast(w)
+    y_t, s_t = torch_fp8_blockwise_cast(w)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(y, y_t)
+    y, s = oracle.per_block_cast_to_fp8(w)
+    y_t, s_t = torch_per_block_cast_to_fp8(w)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(y, y_t)
+    q, s = oracle.block_fp8(w, (128, 128))
+    q_t, s_t = torch_block_fp8(w, (128, 128))
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32)) and _same_fp8(q, q_t)
+    q, s = oracle.mxfp8_quantize(w)
+    q_t, s_t = torch_mxfp8(w)
+    assert torch.equal(s, s_t) and _same_fp8(q, q_t)
+    small = (w.float() * 2.0 ** -4).to(torch.float16)         # keeps 2688 / amax and the block scales in range
+    q, s, _ = oracle.nvfp4_quantize_1d(small)
+    q_t, s_t = torch_nvfp4(small)
+    assert _same_fp8(s, s_t) and torch.equal(q, q_t)
+
+
 @pytest.mark.parametrize("shape", W.SMALL_REFERENCE_SHAPES + [(130, 257), (256, 384)])
 @pytest.mark.parametrize("kind", W.PATTERNS)
 def test_fp8_power_of_two_scales_match_torch_chain(oracle, shape, kind):
