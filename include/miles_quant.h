@@ -231,7 +231,7 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
- * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, INT4_PACK, INT4_PACK_ASYM and NVFP4 run their tuned
+ * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, MXFP4, INT4_PACK, INT4_PACK_ASYM and NVFP4 run their tuned
  * kernels on bf16 and on fp16 inputs; consecutive jobs share a launch when they also share the input dtype (NVFP4 jobs
  * that share an amax record must have one dtype to take them).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that

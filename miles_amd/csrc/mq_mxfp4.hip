@@ -49,17 +49,25 @@ __device__ __forceinline__ uint32_t mxfp4_scale_byte_bf16(uint32_t amax_bits) {
     const int b = e - 2 + gt;
     return b < 0 ? 0u : (uint32_t)b;
 }
+// the same from the fp32 pattern of an amax that came from an fp16 tensor (its subnormals are normal fp32 values)
+__device__ __forceinline__ uint32_t mxfp4_scale_byte_f32(uint32_t amax_f32_bits) {
+    const int e = (int)(amax_f32_bits >> 23), gt = (amax_f32_bits & 0x7FFFFFu) > 0x400000u;
+    if (e == 255) return 254u;
+    const int b = e - 2 + gt;
+    return b < 0 ? 0u : (uint32_t)b;
+}
 // The reference's thresholds send a value that sits exactly on a bound to the smaller magnitude, the hardware
 // conversion rounds ties to even.  Stepping the magnitude down by one fp32 ulp first makes the two agree: a value
-// on a bound lands just below it, and a scaled bf16 value (8 significant bits) can never be the fp32 neighbour just
+// on a bound lands just below it, and a scaled bf16 or fp16 value (8 / 11 significant bits) can never be the fp32 neighbour just
 // above a bound, so nothing else moves across one.  Zero keeps its pattern (and its sign).
 __device__ __forceinline__ float step_toward_zero(float n) {
     const uint32_t u = f2u(n);
     return u2f(u - ((u & 0x7FFFFFFFu) != 0));
 }
 
-template <class Table>
+template <class Table, int F16>
 __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const Table tab) {
+    constexpr uint32_t kInfBits = F16 ? 0x7C00u : 0x7F80u;
     const FlatJob& job = flat_job(tab);
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ packed = (uint32_t*)job.q;
@@ -85,12 +93,12 @@ __global__ __launch_bounds__(kM4Threads) void mxfp4_bf16_kernel(const Table tab)
         const uint32_t off = t + i * kM4Threads;
         const uint32_t m2 = max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)));
         const uint32_t mb = group_max4(hmax_u16(m2));
-        const uint32_t byte = mxfp4_scale_byte_bf16(mb);
+        const uint32_t byte = F16 ? mxfp4_scale_byte_f32(f2u(elem_lo<1>(mb))) : mxfp4_scale_byte_bf16(mb);
         const float mult = mxfp4_normalizer(byte);
-        const float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                            bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        const float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                            elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
         uint32_t word = 0;
-        if (mb < 0x7F80u) {
+        if (mb < kInfBits) {
             float n[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) n[j] = step_toward_zero(f[j] * mult);
@@ -344,21 +352,25 @@ __global__ __launch_bounds__(256) void mxfp4_recode_flat_kernel(const RecodeTabl
 using namespace mq;
 
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group) {
-    return dtype == MQ_BF16 && group == 32 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)packed % 4) == 0;
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && group == 32 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)packed % 4) == 0;
 }
 
-int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st) {
+int mq_mxfp4_launch_group(int dtype, FlatTable& tab, hipStream_t st) {
     if (!flat_grid(tab, kM4Threads * kM4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (tab.max_blocks == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp4_bf16_kernel<FlatTable>, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(kM4Threads), 0, st, tab);
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(kM4Threads);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((mxfp4_bf16_kernel<FlatTable, 1>), grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL((mxfp4_bf16_kernel<FlatTable, 0>), grid, blk, 0, st, tab);
     return mq_check_launch("mxfp4 quant");
 }
 
-int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
+int mq_mxfp4_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st) {
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kM4Threads * kM4Unroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
     if (ref.max_blocks == 0 || n == 0) return MQ_OK;
-    hipLaunchKernelGGL(mxfp4_bf16_kernel<FlatRef>, dim3((unsigned)ref.max_blocks, (unsigned)n), dim3(kM4Threads), 0, st, ref);
+    const dim3 grid((unsigned)ref.max_blocks, (unsigned)n), blk(kM4Threads);
+    if (dtype == MQ_F16) hipLaunchKernelGGL((mxfp4_bf16_kernel<FlatRef, 1>), grid, blk, 0, st, ref);
+    else hipLaunchKernelGGL((mxfp4_bf16_kernel<FlatRef, 0>), grid, blk, 0, st, ref);
     return mq_check_launch("mxfp4 quant");
 }
 
@@ -373,7 +385,7 @@ extern "C" int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t
         FlatTable tab{};
         tab.n = 1;
         tab.job[0] = FlatJob{w, packed, scale, nullptr, numel / 8, nullptr, 0, 0};
-        return mq_mxfp4_launch_group(tab, st);
+        return mq_mxfp4_launch_group(dtype, tab, st);
     }
     const int64_t groups = numel / group, bytes = numel / 2;
     int64_t blocks = (groups + 255) / 256;

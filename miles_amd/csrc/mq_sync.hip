@@ -30,7 +30,7 @@ bool mq_nvfp4_fast_ok(const void* w, int dtype, const void* q);
 int mq_nvfp4_amax_launch_group(int dtype, FlatTable& tab, hipStream_t st);
 int mq_nvfp4_quant_launch_group(int dtype, FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st);
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
-int mq_mxfp4_launch_group(FlatTable& tab, hipStream_t st);
+int mq_mxfp4_launch_group(int dtype, FlatTable& tab, hipStream_t st);
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
 int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
 int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st);
@@ -38,7 +38,7 @@ int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hip
 int mq_nvfp4_quant_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode,
                                 hipStream_t st);
 int mq_mxfp8_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
-int mq_mxfp4_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
+int mq_mxfp4_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, hipStream_t st);
 int mq_int4_pack_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int group, hipStream_t st);
 bool mq_int4_pack_asym_fast_ok(const void* w, int dtype, int group, int64_t M);
 int mq_int4_pack_asym_launch_group(int dtype, FlatTable& tab, int group, hipStream_t st);
@@ -205,9 +205,10 @@ static int64_t tile_run_end(const mq_job* jobs, int64_t i, int64_t j, int64_t ti
 }
 
 static bool same_group(const mq_job& a, const mq_job& b) {
-    // the FP8 tile, MXFP8 and symmetric INT4 kernels are compiled per 16-bit input dtype; the other kinds' fast paths
-    // take one dtype, or any (copies)
-    const bool per_dtype = tile_kind(a.kind) || a.kind == MQ_JOB_MXFP8 || a.kind == MQ_JOB_INT4_PACK || a.kind == MQ_JOB_INT4_PACK_ASYM;
+    // the quantizer kernels are compiled per 16-bit input dtype; the other kinds' fast paths take one dtype, or any
+    // (copies)
+    const bool per_dtype = tile_kind(a.kind) || a.kind == MQ_JOB_MXFP8 || a.kind == MQ_JOB_MXFP4 || a.kind == MQ_JOB_INT4_PACK ||
+                           a.kind == MQ_JOB_INT4_PACK_ASYM;
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1 && (!per_dtype || a.dtype == b.dtype);
 }
 
@@ -509,7 +510,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                             zero_tiles = tiles > zero_tiles ? tiles : zero_tiles;
                         }
                     rc = head.kind == MQ_JOB_MXFP8       ? mq_mxfp8_launch_table(head.dtype, table + i, cnt, mx / 8, st)
-                         : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_table(table + i, cnt, mx / 8, st)
+                         : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_table(head.dtype, table + i, cnt, mx / 8, st)
                          : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_table(head.dtype, table + i, cnt, mx / 8, head.p0, st)
                                                          : mq_int4_pack_asym_launch_table(head.dtype, table + i, cnt, mx / 8, zero_tiles, head.p0, st);
                     break;
@@ -518,7 +519,7 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                 tab.n = cnt;
                 for (int t = 0; t < cnt; t++) tab.job[t] = flat_entry(jobs[i + t]);
                 rc = head.kind == MQ_JOB_MXFP8       ? mq_mxfp8_launch_group(head.dtype, tab, st)
-                     : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_group(tab, st)
+                     : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_group(head.dtype, tab, st)
                      : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_group(head.dtype, tab, head.p0, st)
                                                      : mq_int4_pack_asym_launch_group(head.dtype, tab, head.p0, st);
                 break;

@@ -741,6 +741,46 @@ def test_mxfp4_requantizing_a_checkpoint_is_the_identity():
         ("model.layers.0.experts.0.w1.weight_scale", torch.uint8, (64, 2))]
 
 
+def test_mxfp4_quantize_fp16(oracle):
+    """The MXFP4 quantizer's fp16 instance: every fp16 pattern as a group maximum (the scale byte is read off the fp32
+    pattern of the amax; subnormals, 65504, infinity and NaN included), ties at every bound in several binades, all
+    fp16 patterns as elements, and a recorded list mixing bf16 and fp16 tensors."""
+    from miles_amd import launch
+    from miles_amd.utils.mxfp4 import quantize_mxfp4
+
+    pats = torch.arange(0, 0x8000, dtype=torch.int32).to(torch.int16).view(torch.float16)          # 0 ... NaN patterns
+    amax_rows = torch.zeros(0x8000, 32, dtype=torch.float16)
+    amax_rows[:, 3] = pats                                      # one group per pattern: that value and small company
+    amax_rows[:, 7] = (pats.float() * -0.6).to(torch.float16)
+    amax_rows[:, 11] = (pats.float() * 0.31).to(torch.float16)
+    ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4, dtype=torch.float16)
+    tie_rows = torch.stack([ties, -ties, ties * 2 ** -10, ties * 2 ** 8, (ties.float() * 2 ** -14).to(torch.float16)])
+    everything = torch.arange(-0x8000, 0x8000, dtype=torch.int32).to(torch.int16).view(torch.float16).reshape(2048, 32)
+    for name, w in (("every amax", amax_rows), ("ties", tie_rows), ("every pattern", everything)):
+        packed, scale = quantize_mxfp4(w.to(DEV), 32)
+        packed_o, scale_o = oracle.quantize_mxfp4(w, 32)
+        bad = torch.isnan(w.float()).any(dim=1)                  # a NaN in the group: the reference's result is undefined
+        _assert_same(scale[~bad], scale_o[~bad], f"E8M0 scales ({name})")
+        _assert_same(packed[~bad], packed_o[~bad], f"packed codes ({name})")
+    tensors = []
+    for i in range(9):
+        t = W.student_t_rows((64 + 8 * i, 512), std=0.02, seed=6200 + i)
+        tensors.append(t.to(torch.float16) if i % 3 else t)
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [quantize_mxfp4(t, 32) for t in dev]
+    batch.freeze()
+    for rep in range(2):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, t in enumerate(tensors):
+            for got, want, what in zip(outs[i], oracle.quantize_mxfp4(t, 32), ("packed", "scales")):
+                _assert_same(got, want, f"tensor {i} ({t.dtype}) {what}, run {rep}")
+        for o in outs:
+            for t in o:
+                t.view(torch.uint8).fill_(0x5A)
+
+
 def test_mxfp4_grouped_jobs(oracle):
     from miles_amd import launch
     from miles_amd.utils.mxfp4 import quantize_mxfp4
