@@ -218,7 +218,7 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_FP8_BLOCK_POW2       w[rows,cols]  e4m3          fp32 tiles     -                           128, 128
  *   MQ_JOB_UE8M0_PACK           fp32 tiles    int32 words   -              -                           batch, tile_rows
  *   MQ_JOB_FP8_TENSOR           w[rows,cols]  e4m3          fp32 [1]       aux = amax record           floor bits, flags
- *     (tensor_fp8 / the per-tensor branch of the sync path, see mq_fp8_scaled_quant: bf16, contiguous, cols % 8 == 0,
+ *     (tensor_fp8 / the per-tensor branch of the sync path, see mq_fp8_scaled_quant: bf16 or fp16, contiguous, cols % 8 == 0,
  *      16-byte aligned input; p0 = bit pattern of 1e-12 rounded to the weight dtype; p1 = 0 or MQ_NVFP4_CARRY_AMAX)
  *   MQ_JOB_INT4_PACK_ASYM       w             int32 words   scales (dtype) aux = uint8 zero points,    group, -
  *                                                                          aux2 = int32 packed_zp
@@ -231,14 +231,14 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
- * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, MXFP4, INT4_PACK, INT4_PACK_ASYM and NVFP4 run their tuned
+ * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, MXFP4, INT4_PACK, INT4_PACK_ASYM, FP8_TENSOR and NVFP4 run their tuned
  * kernels on bf16 and on fp16 inputs; consecutive jobs share a launch when they also share the input dtype (NVFP4 jobs
  * that share an amax record must have one dtype to take them).
  * NVFP4: the driver reduces every job's tensor into a section of its record and then quantizes; jobs that
  * share one record (a gate/up pair; at most MQ_NVFP4_SECTIONS) must be adjacent in the list.
  * MQ_NVFP4_CARRY_AMAX in p1 of NVFP4 and FP8_TENSOR jobs (no counterpart in the reference): a caller that submits the
  * same job list again, amax records included and untouched in between, after at least one submission without the
- * flag, may set it on bf16 or fp16 jobs (per-tensor FP8: bf16).  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
+ * flag, may set it on bf16 or fp16 jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
  * submission, collects the new amax on the way, and quantizes a tensor a second time only if its amax changed
  * (results are identical either way; a weight tensor's amax rarely moves between two syncs).  A tensor whose amax did
  * change is marked volatile in its record: on the next submission the single pass only collects its amax and the

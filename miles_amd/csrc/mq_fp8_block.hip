@@ -319,7 +319,7 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restri
 //
 // per channel: a row lives in the registers of ROWLANES lanes (up to 8 sixteen-byte units each), so it is read once:
 // amax across the lanes, one scale, codes.  ROWLANES = 64: four rows per workgroup, no LDS; 256: one row.
-template <int ROWLANES>
+template <int ROWLANES, int F16>
 __global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* __restrict__ w, int64_t ldw, int64_t K,
                                                                int64_t M, float floor_v, uint8_t* __restrict__ q,
                                                                float* __restrict__ scale) {
@@ -344,22 +344,25 @@ __global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* _
         __syncthreads();
         m = umax(umax(wave_amax[0], wave_amax[1]), umax(wave_amax[2], wave_amax[3]));
     }
-    float amax = u2f(m << 16);
+    float amax = elem_lo<F16>(m);
     if (amax < floor_v) amax = floor_v;
     const float s = amax / kFp8Max, y = 1.0f / s;
     const bool fast_div = shared_div_ok(s);
+    // the hardware conversion takes finite quotients: an infinity or a NaN in the row, or a zero scale (fp16 has no
+    // 1e-12 floor, so a row of zeros divides 0 by 0), goes through the software conversion
+    const bool plain = m < (F16 ? 0x7C00u : 0x7F80u) && s > 0.0f;
     if (!row_ok) return;
     if (lane == 0) scale[row] = s;
 #pragma unroll
     for (int u = 0; u < kMaxUnits; u++) {
         const int64_t unit = lane + (int64_t)u * ROWLANES;
         if (unit >= units) continue;
-        float f[8] = {bf16_lo(v[u].x), bf16_hi(v[u].x), bf16_lo(v[u].y), bf16_hi(v[u].y),
-                      bf16_lo(v[u].z), bf16_hi(v[u].z), bf16_lo(v[u].w), bf16_hi(v[u].w)};
+        float f[8] = {elem_lo<F16>(v[u].x), elem_hi<F16>(v[u].x), elem_lo<F16>(v[u].y), elem_hi<F16>(v[u].y),
+                      elem_lo<F16>(v[u].z), elem_hi<F16>(v[u].z), elem_lo<F16>(v[u].w), elem_hi<F16>(v[u].w)};
 #pragma unroll
         for (int j = 0; j < 8; j++) f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
         u32x2 o;
-        if (m < 0x7F80u) {
+        if (plain) {
             o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
             o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
         } else {                                  // inf / NaN in the row: clamp and convert in software
@@ -643,15 +646,19 @@ static int fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, floa
     if (M == 0 || K == 0) return MQ_OK;
     if (M > 0x7FFFFFFF) return mq_fail(MQ_ERR_ARG, "too many rows");
     hipStream_t st = (hipStream_t)stream;
-    const bool aligned = dtype == MQ_BF16 && K % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0;
-    if (aligned && per_channel && K / 8 <= 2048) {
+    const bool aligned16 = (dtype == MQ_BF16 || dtype == MQ_F16) && K % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)w % 16) == 0 &&
+                           ((uintptr_t)q % 8) == 0;
+    const bool aligned = aligned16 && dtype == MQ_BF16;
+    if (aligned16 && per_channel && K / 8 <= 2048) {
         const uint16_t* wi = (const uint16_t*)w;
-        if (K / 8 <= 256)
-            hipLaunchKernelGGL(fp8_channel_bf16_kernel<64>, dim3((unsigned)((M + 3) / 4)), dim3(256), 0, st, wi, ldw, K, M,
-                               floor_in_dtype, (uint8_t*)q, scale);
-        else
-            hipLaunchKernelGGL(fp8_channel_bf16_kernel<256>, dim3((unsigned)M), dim3(256), 0, st, wi, ldw, K, M,
-                               floor_in_dtype, (uint8_t*)q, scale);
+        const dim3 narrow((unsigned)((M + 3) / 4)), wide((unsigned)M), blk(256);
+        if (dtype == MQ_F16) {
+            if (K / 8 <= 256) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 1>), narrow, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 1>), wide, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+        } else {
+            if (K / 8 <= 256) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 0>), narrow, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 0>), wide, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+        }
         return mq_check_launch("fp8 scaled quant");
     }
     if (aligned && !per_channel && ldw == K && M * (K / 8) < (1ll << 38)) {

@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, f
     }
 }
 
+template <int F16>
 __device__ __forceinline__ uint32_t fp8_tensor_quant_units(const FlatJob& job, const int64_t base, const int t, const float floor_v) {
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint8_t* __restrict__ q = (uint8_t*)job.q;
@@ -72,18 +73,23 @@ __device__ __forceinline__ uint32_t fp8_tensor_quant_units(const FlatJob& job, c
     for (int i = 0; i < kFtUnroll; i++) {
         const int64_t unit = base + i * kFtThreads + t;
         seen = umax(seen, hmax_u16(max2_u16(max2_u16(abs2(v[i].x), abs2(v[i].y)), max2_u16(abs2(v[i].z), abs2(v[i].w)))));
-        float f[8] = {bf16_lo(v[i].x), bf16_hi(v[i].x), bf16_lo(v[i].y), bf16_hi(v[i].y),
-                      bf16_lo(v[i].z), bf16_hi(v[i].z), bf16_lo(v[i].w), bf16_hi(v[i].w)};
+        float f[8] = {elem_lo<F16>(v[i].x), elem_hi<F16>(v[i].x), elem_lo<F16>(v[i].y), elem_hi<F16>(v[i].y),
+                      elem_lo<F16>(v[i].z), elem_hi<F16>(v[i].z), elem_lo<F16>(v[i].w), elem_hi<F16>(v[i].w)};
 #pragma unroll
         for (int j = 0; j < 8; j++) f[j] = fast_div ? div_by_shared(f[j], s, y) : f[j] / s;
 #pragma unroll
-        for (int j = 0; j < 8; j += 2) {           // the rounding to bf16
-            const uint32_t p = hw_bf16x2(f[j], f[j + 1]);
-            f[j] = bf16_lo(p);
-            f[j + 1] = bf16_hi(p);
+        for (int j = 0; j < 8; j += 2) {           // the rounding to the weight's dtype
+            if (F16) {
+                f[j] = (float)(_Float16)f[j];
+                f[j + 1] = (float)(_Float16)f[j + 1];
+            } else {
+                const uint32_t p = hw_bf16x2(f[j], f[j + 1]);
+                f[j] = bf16_lo(p);
+                f[j + 1] = bf16_hi(p);
+            }
         }
         u32x2 o;
-        if (abits < 0x7F800000u) {
+        if (abits < 0x7F800000u && s > 0.0f) {      // (a zero scale -- fp16 has no 1e-12 floor -- makes every quotient NaN)
             o.x = hw_e4m3x4(f[0], f[1], f[2], f[3]);
             o.y = hw_e4m3x4(f[4], f[5], f[6], f[7]);
         } else {                                   // inf / NaN amax: clamp and convert in software
@@ -100,7 +106,7 @@ __device__ __forceinline__ uint32_t fp8_tensor_quant_units(const FlatJob& job, c
 
 // PASS 0: second pass of the two-pass form; 1: single pass with the carried-over amax, new partial maxima collected;
 // 2: grid-stride second quantization of the tensors whose amax moved
-template <int PASS, class Table>
+template <int PASS, class Table, int F16>
 __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Table tab, float floor_v) {
     const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const int t = threadIdx.x;
@@ -110,7 +116,7 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Tabl
         // an XCD takes a run of consecutive blocks in every trip of the grid, as the flat grids do (second pass 2 pct faster)
         const int64_t first = xcd_chunked_block(gridDim.x == kSectionWords ? kSectionWords / kXcds : tab.chunk);
         for (int64_t base = first * kPerBlock; base < job.units; base += (int64_t)gridDim.x * kPerBlock)
-            fp8_tensor_quant_units(job, base, t, floor_v);
+            fp8_tensor_quant_units<F16>(job, base, t, floor_v);
         return;
     }
     const int64_t base = flat_block(tab) * kPerBlock;
@@ -127,7 +133,7 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Tabl
         }
         seen = hmax_u16(m2);
     } else {
-        seen = fp8_tensor_quant_units(job, base, t, floor_v);
+        seen = fp8_tensor_quant_units<F16>(job, base, t, floor_v);
     }
     if (PASS == 1) {
         __shared__ uint32_t wave_seen[kFtThreads / 64];
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(kFtThreads) void fp8_tensor_quant_kernel(const Tabl
             uint32_t m = 0;
 #pragma unroll
             for (int k = 0; k < kFtThreads / 64; k++) m = umax(m, wave_seen[k]);
-            atomicMax((uint32_t*)job.aux + (blockIdx.x & (kSectionWords - 1)), m << 16);
+            atomicMax((uint32_t*)job.aux + (blockIdx.x & (kSectionWords - 1)), f2u(elem_lo<F16>(m)));
         }
     }
 }
@@ -151,50 +157,56 @@ int mq_nvfp4_amax_launch_group(int dtype, FlatTable& tab, hipStream_t st);
 int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hipStream_t st);
 
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld) {
-    return dtype == MQ_BF16 && cols % 8 == 0 && ld == cols && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 &&
+    return (dtype == MQ_BF16 || dtype == MQ_F16) && cols % 8 == 0 && ld == cols && ((uintptr_t)w % 16) == 0 && ((uintptr_t)q % 8) == 0 &&
            rows * (cols / 8) < (1ll << 38);
 }
 
 // fold + quantize (+ second pass) over a table whose grid is known
-template <class Table>
-static int fp8_tensor_launch(const Table& tab, int n, float floor_v, bool carry, hipStream_t st) {
+template <class Table, int F16>
+static int fp8_tensor_launch_dtype(const Table& tab, int n, float floor_v, bool carry, hipStream_t st) {
     const dim3 folds((unsigned)n), blk(256), grid((unsigned)tab.max_blocks, (unsigned)n);
     if (carry) {
-        if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<1, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
+        if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<1, Table, F16>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
         hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
         if (tab.max_blocks > 0) {
             const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
-            hipLaunchKernelGGL((fp8_tensor_quant_kernel<2, Table>), dim3(redo, (unsigned)n), dim3(kFtThreads), 0, st, tab, floor_v);
+            hipLaunchKernelGGL((fp8_tensor_quant_kernel<2, Table, F16>), dim3(redo, (unsigned)n), dim3(kFtThreads), 0, st, tab, floor_v);
         }
         return mq_check_launch("fp8 per-tensor quant (carried-over amax)");
     }
     hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
-    if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<0, Table>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
+    if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<0, Table, F16>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
     return mq_check_launch("fp8 per-tensor quant");
+}
+template <class Table>
+static int fp8_tensor_launch(int dtype, const Table& tab, int n, float floor_v, bool carry, hipStream_t st) {
+    return dtype == MQ_F16 ? fp8_tensor_launch_dtype<Table, 1>(tab, n, floor_v, carry, st)
+                           : fp8_tensor_launch_dtype<Table, 0>(tab, n, floor_v, carry, st);
 }
 
 // tab.job[i]: w, q, s = fp32 scale out, aux = amax record, units = numel / 8.  carry: see the file header.
-int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st) {
+int mq_fp8_tensor_launch_group(int dtype, FlatTable& tab, float floor_v, bool carry, hipStream_t st) {
     if (!carry) {
         FlatTable amax = tab;
         for (int i = 0; i < tab.n; i++) {
             amax.job[i].s = (void*)(uintptr_t)(tab.job[i].units * 8);      // element count, for the amax kernel's tail
             amax.job[i].section = 0;
         }
-        int rc = mq_nvfp4_amax_launch_group(MQ_BF16, amax, st);
+        int rc = mq_nvfp4_amax_launch_group(dtype, amax, st);
         if (rc) return rc;
     }
     if (!flat_grid(tab, kFtThreads * kFtUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    return fp8_tensor_launch(tab, tab.n, floor_v, carry, st);
+    return fp8_tensor_launch(dtype, tab, tab.n, floor_v, carry, st);
 }
 // the same over n descriptors of a device table (section 0 in every entry); max_units: the largest tensor's units
-int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st) {
+int mq_fp8_tensor_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry,
+                               hipStream_t st) {
     if (n == 0) return MQ_OK;
     if (!carry) {
-        int rc = mq_nvfp4_amax_launch_table(MQ_BF16, device_jobs, n, st);
+        int rc = mq_nvfp4_amax_launch_table(dtype, device_jobs, n, st);
         if (rc) return rc;
     }
     FlatRef ref{device_jobs, 0, 0};
     if (!flat_grid(ref, max_units, kFtThreads * kFtUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
-    return fp8_tensor_launch(ref, n, floor_v, carry, st);
+    return fp8_tensor_launch(dtype, ref, n, floor_v, carry, st);
 }

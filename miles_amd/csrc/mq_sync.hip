@@ -32,8 +32,9 @@ int mq_nvfp4_quant_launch_group(int dtype, FlatTable& tab, int e4m3_max, int fla
 bool mq_mxfp4_fast_ok(const void* w, int dtype, const void* packed, int group);
 int mq_mxfp4_launch_group(int dtype, FlatTable& tab, hipStream_t st);
 bool mq_fp8_tensor_fast_ok(const void* w, int dtype, const void* q, int64_t rows, int64_t cols, int64_t ld);
-int mq_fp8_tensor_launch_group(FlatTable& tab, float floor_v, bool carry, hipStream_t st);
-int mq_fp8_tensor_launch_table(const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry, hipStream_t st);
+int mq_fp8_tensor_launch_group(int dtype, FlatTable& tab, float floor_v, bool carry, hipStream_t st);
+int mq_fp8_tensor_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, float floor_v, bool carry,
+                               hipStream_t st);
 int mq_nvfp4_amax_launch_table(int dtype, const FlatJob* device_jobs, int n, hipStream_t st);
 int mq_nvfp4_quant_launch_table(int dtype, const FlatJob* device_jobs, int n, int64_t max_units, int e4m3_max, int mode,
                                 hipStream_t st);
@@ -113,7 +114,7 @@ static int check_job(const mq_job& j) {
     if (j.kind == MQ_JOB_INT4_PACK_ASYM && !empty && (!j.aux || !j.aux2)) return mq_fail(MQ_ERR_ARG, "asymmetric INT4 job without zero-point outputs");
     if (j.kind == MQ_JOB_FP8_TENSOR) {
         if (!j.aux || !j.scale) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 job without an amax record or a scale pointer");
-        if (!empty && !job_fast(j)) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 jobs take contiguous bf16 tensors (cols % 8 == 0, 16-byte aligned)");
+        if (!empty && !job_fast(j)) return mq_fail(MQ_ERR_ARG, "per-tensor FP8 jobs take contiguous bf16 or fp16 tensors (cols % 8 == 0, 16-byte aligned)");
     }
     if (j.rows_per_block != 0) {
         const bool fp8q = j.kind == MQ_JOB_FP8_BLOCK || j.kind == MQ_JOB_FP8_BLOCKWISE_CAST || j.kind == MQ_JOB_FP8_BLOCK_POW2;
@@ -240,7 +241,7 @@ static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, const FlatJo
     const int64_t cap = table ? kTableGroup : kMaxGroup;
     while (i < j) {
         int64_t k = i, sum = 0, mx = 0;
-        while (k < j && k - i < cap && jobs[k].p0 == jobs[i].p0 && jobs[k].p1 == jobs[i].p1) {
+        while (k < j && k - i < cap && jobs[k].p0 == jobs[i].p0 && jobs[k].p1 == jobs[i].p1 && jobs[k].dtype == jobs[i].dtype) {
             const int64_t e = jobs[k].rows * jobs[k].cols;
             const int64_t nmx = e > mx ? e : mx;
             if (k > i && nmx * (k - i + 1) * 4 > (sum + e) * 5) break;       // padding of the 2-D grid under 25 %
@@ -254,12 +255,12 @@ static int run_fp8_tensor(const mq_job* jobs, int64_t i, int64_t j, const FlatJo
         const bool carry = (jobs[i].p1 & MQ_NVFP4_CARRY_AMAX) != 0;
         int rc;
         if (k - i > kMaxGroup) {
-            rc = mq_fp8_tensor_launch_table(table + i, (int)(k - i), mx / 8, floor_v, carry, (hipStream_t)stream);
+            rc = mq_fp8_tensor_launch_table(jobs[i].dtype, table + i, (int)(k - i), mx / 8, floor_v, carry, (hipStream_t)stream);
         } else {
             FlatTable tab{};
             tab.n = (int)(k - i);
             for (int64_t t = i; t < k; t++) tab.job[t - i] = flat_entry(jobs[t]);
-            rc = mq_fp8_tensor_launch_group(tab, floor_v, carry, (hipStream_t)stream);
+            rc = mq_fp8_tensor_launch_group(jobs[i].dtype, tab, floor_v, carry, (hipStream_t)stream);
         }
         if (rc) return rc;
         i = k;

@@ -60,7 +60,7 @@ def _scaled_fp8(weight: torch.Tensor, per_channel: bool):
     q = torch.empty((n, k), dtype=torch.float8_e4m3fn, device=w.device)
     scale = torch.empty((n, 1) if per_channel else (1,), dtype=torch.float32, device=w.device)
     floor = float(torch.tensor(1e-12, dtype=w.dtype).float())  # clamp(min=1e-12) acts in the weight dtype
-    if not per_channel and w.dtype == torch.bfloat16 and w.is_contiguous() and k % 8 == 0 and w.data_ptr() % 16 == 0:
+    if not per_channel and w.dtype in (torch.bfloat16, torch.float16) and w.is_contiguous() and k % 8 == 0 and w.data_ptr() % 16 == 0:
         # a job of the batched driver (grouped launches, replayable): amax record as for NVFP4
         record = torch.empty(_AMAX_RECORD_WORDS, dtype=torch.int32, device=w.device)
         floor_bits = int(torch.tensor(floor, dtype=torch.float32).view(torch.int32))

@@ -241,6 +241,70 @@ def test_tensor_and_channel_fp8_bf16_row_kernels(oracle, shape):
         _assert_same(q, q_o, f"{strategy} codes, strided rows")
 
 
+def _same_fp8_codes(got, want, what):
+    """Byte equality with the two e4m3 NaN codes 0x7F / 0xFF counted as one (the sign of a 0 / 0 is the host FPU's choice)."""
+    g, w = _u8(got).clone(), _u8(want).clone()
+    g[(g & 0x7F) == 0x7F] = 0x7F
+    w[(w & 0x7F) == 0x7F] = 0x7F
+    assert g.shape == w.shape and torch.equal(g, w), f"{what}: {(g != w).sum().item()} of {g.numel()} differ"
+
+
+@pytest.mark.parametrize("shape", [(64, 2048), (37, 7168), (5, 16384), (130, 264), (2048, 7168)])
+def test_tensor_and_channel_fp8_fp16(oracle, shape):
+    """fp16 weights on the per-channel row kernels and on the per-tensor job form: fp16 has no 1e-12 floor (it rounds to
+    zero), so a row / tensor of zeros divides 0 by 0 and every code is NaN; subnormals, the format's extremes, strided
+    rows; per tensor also as a recorded list that mixes bf16 and fp16 tensors and then carries the amax over."""
+    from miles_amd import launch
+    from miles_amd.tools.convert_hf_to_fp8 import quant_fp8
+
+    w = W.gaussian_outliers(shape, std=0.02, p_outlier=0.001, gain=25.0, seed=1400 + shape[1], dtype=torch.float16)
+    w[0] = 0
+    w[1, :64] = torch.tensor([-0.0, 0.0] * 32, dtype=torch.float16)
+    w[2] = 6e-8
+    w[2, 5] = -1.2e-7
+    w[3, :4] = torch.tensor([65504.0, -65504.0, 3.0, -1e-4], dtype=torch.float16)
+    for strategy, ref in (("tensor", oracle.tensor_fp8), ("channel", oracle.channel_fp8)):
+        q, s = quant_fp8(w.to(DEV), strategy)
+        q_o, s_o = ref(w)
+        _assert_same(s, s_o, f"{strategy} scale")
+        _same_fp8_codes(q, q_o, f"{strategy} codes")
+    z = torch.zeros(16, 256, dtype=torch.float16)
+    q, s = quant_fp8(z.to(DEV), "tensor")
+    q_o, s_o = oracle.tensor_fp8(z)
+    _assert_same(s, s_o, "zero tensor scale")
+    _same_fp8_codes(q, q_o, "zero tensor codes")
+    wide = W.gaussian_outliers((shape[0], shape[1] + 64), std=0.02, p_outlier=0.001, gain=25.0, seed=78, dtype=torch.float16)
+    q, s = quant_fp8(wide.to(DEV)[:, : shape[1]], "channel")
+    q_o, s_o = oracle.channel_fp8(wide[:, : shape[1]].contiguous())
+    _assert_same(s, s_o, "channel scale, strided rows")
+    _same_fp8_codes(q, q_o, "channel codes, strided rows")
+    if shape[0] > 1000:
+        return
+    tensors = [W.gaussian_outliers((24 + i, 512), std=0.02, p_outlier=0.001, gain=20.0, seed=1500 + i,
+                                   dtype=torch.float16 if i % 3 else torch.bfloat16) for i in range(9)]
+    dev = [t.to(DEV) for t in tensors]
+    with launch.recording() as batch:
+        outs = [quant_fp8(t, "tensor") for t in dev]
+    assert len(batch) == len(tensors) and batch.direct_calls == 0
+    batch.device = torch.device(DEV)
+
+    def check(what):
+        batch.run()
+        torch.cuda.synchronize()
+        for i, (t, (q, sc)) in enumerate(zip(dev, outs)):
+            q_o, s_o = oracle.tensor_fp8(t.cpu())
+            _assert_same(sc, s_o, f"{what}: tensor {i} ({t.dtype}) scale")
+            _same_fp8_codes(q, q_o, f"{what}: tensor {i} ({t.dtype}) codes")
+
+    check("first run")
+    assert batch.carry_amax() == len(tensors)
+    check("carried")
+    dev[1].mul_(2.0)
+    dev[5].mul_(0.25)
+    check("two fp16 amax moved")
+    check("settled")
+
+
 # ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape", FP8_SHAPES)
 @pytest.mark.parametrize("kind", W.PATTERNS)
