@@ -73,6 +73,21 @@ def _event_ms(fn, iters):
     return e0.elapsed_time(e1) / iters
 
 
+def _event_ms_each(fn, before_each, iters):
+    """As _event_ms, with `before_each()` run ahead of every repetition and kept out of the timed span (it stands for
+    what the trainer does between two syncs): one event pair per repetition."""
+    total = 0.0
+    for _ in range(iters):
+        before_each()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        total += e0.elapsed_time(e1)
+    return total / iters
+
+
 def _best_ms(fn):
     """Per-quantizer figure: the fastest of three timed runs of TIMED_ITERS repetitions (memory that the allocator mapped
     a moment ago streams slower on its first passes); a single run when counters are being collected."""
@@ -107,12 +122,10 @@ def per_quantizer(gen):
         batch, outs = _record(build)
         if prepare is not None:
             prepare(batch)
-        fn = batch.run
         if before_each is not None:
-            def fn():
-                before_each()
-                batch.run()
-        ms = _best_ms(fn)
+            ms = min(_event_ms_each(batch.run, before_each, TIMED_ITERS) for _ in range(1 if TIMED_ITERS == 1 else 3))
+        else:
+            ms = _best_ms(batch.run)
         gbps = elems * BYTES_PER_ELEM[key] / ms / 1e6
         res[name] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                      "elements": elems, "workload": note}
