@@ -599,6 +599,33 @@ def stream_ceilings():
         probe(f"tile128_2r_1w_K{k}", TILE_2_1, k, elems * 3)
         probe(f"tile128_read_only_K{k}", TILE_READ, k, elems * 2)
         probe(f"tile128_write_only_K{k}", TILE_WRITE, k, elems)
+    del x, y
+    res.update(tile_launch_lengths())
+    return res
+
+
+def tile_launch_lengths():
+    """The FP8 tile kernel on every 2-D weight of Qwen3-4B as one job list, with the driver's cut of long runs of tile
+    jobs set to different lengths (MQ_TILE_LAUNCH_TILES; 0: no cut, up to 64 tensors per launch)."""
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(1234)
+    _, weights, _ = qwen3_4b_megatron_weights(gen)
+    targets = [t for name, t in weights.items() if t.dim() == 2 and "embedding" not in name and "output_layer" not in name]
+    elems = sum(t.numel() for t in targets)
+    batch, outs = _record(lambda: [fp8_blockwise_cast(t) for t in targets])
+    res = {}
+    try:
+        for cap in (0, 98304, 49152, 36864, 24576, 16384, 8192, 4096):
+            os.environ["MQ_TILE_LAUNCH_TILES"] = str(cap)
+            for _ in range(3):
+                batch.run()
+            ms = _best_ms(batch.run)
+            res[f"qwen3_4b_fp8_cast_launches_of_{cap}_tiles"] = {"GBps": round(elems * BYTES_PER_ELEM["fp8_block"] / ms / 1e6, 1),
+                                                                 "ms": round(ms, 4)}
+    finally:
+        del os.environ["MQ_TILE_LAUNCH_TILES"]
     return res
 
 

@@ -6,6 +6,7 @@
 // list order.
 #include <vector>
 
+#include <stdlib.h>
 #include <string.h>
 
 #include "mq_api_internal.hpp"
@@ -197,8 +198,11 @@ static FlatJob flat_entry(const mq_job& jb) {
 
 // jobs [i, j) hold `tiles` tiles: where the first of the equal launches they are cut into ends
 static int64_t tile_run_end(const mq_job* jobs, int64_t i, int64_t j, int64_t tiles) {
-    if (MQ_TILE_LAUNCH_TILES <= 0 || tiles <= MQ_TILE_LAUNCH_TILES) return j;
-    const int64_t launches = (tiles + MQ_TILE_LAUNCH_TILES - 1) / MQ_TILE_LAUNCH_TILES;
+    // (the environment variable MQ_TILE_LAUNCH_TILES overrides the length, 0 switches the cutting off: for measurements)
+    int64_t cap = MQ_TILE_LAUNCH_TILES;
+    if (const char* env = getenv("MQ_TILE_LAUNCH_TILES")) cap = atoll(env);
+    if (cap <= 0 || tiles <= cap) return j;
+    const int64_t launches = (tiles + cap - 1) / cap;
     const int64_t target = (tiles + launches - 1) / launches;
     int64_t acc = 0, t = i;
     while (t < j && acc < target) acc += tiles_of(jobs[t++]);
