@@ -277,7 +277,8 @@ typedef struct mq_job {
 } mq_job;
 /* Consecutive jobs of one kind (and, for the flat kernels, of similar size) are fused into launches of up to
  * MQ_MAX_GROUP tensors, counted from the first job of the call; a run of FP8 tile jobs of more than 36 864 tiles is
- * cut into launches of equal size (the tile kernel streams faster in launches of moderate length). */
+ * cut into launches of equal size (the tile kernel streams faster in launches of moderate length; the environment
+ * variable MQ_TILE_LAUNCH_TILES overrides the length, 0 switches the cutting off). */
 #define MQ_MAX_GROUP 64
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
 
