@@ -37,7 +37,7 @@ BYTES_PER_ELEM = {"fp8_block": 2 + 1 + 4 / 16384, "fp8_dequant": 1 + 4 / 16384 +
                   # formats either side of the path: MXFP4 (group 32), INT4 unpack, asymmetric INT4 (one zero-point nibble per group)
                   "mxfp4": 2 + 0.5 + 1 / 32, "mxfp4_dequant": 0.5 + 1 / 32 + 2, "int4_unpack": 0.5 + 2 / 128 + 2,
                   "int4_g128_asym": 2 + 0.5 + 2 / 128 + 0.5 / 128, "fake_quant_bf16": 2 + 2, "act_quant": 2 + 1 + 4 / 128, "fake_int4_bf16": 2 + 2 + 2 / 128, "fp8_channel": 2 + 1,
-                  "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384}
+                  "mxfp4_to_fp8": 0.5 + 1 / 32 + 1 + 4 / 16384, "fp8_to_mxfp8": 1 + 4 / 16384 + 1 + 1 / 32}
 # HBM bytes per element of the FP8 tile kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
 # scaled by the same counter on a plain 1 GiB copy (read 2.0003 + write 1.0005 B per element)
 MEASURED_FP8_TRAFFIC_BYTES_PER_ELEM = 3.0008
@@ -370,6 +370,13 @@ def adjacent_formats(gen):
     run("next_mxfp4_to_fp8_recode", "mxfp4_to_fp8", batch.run,
         "MXFP4 -> e4m3 with 128x128 fp32 tile scales, one job list: tile scales, then a flat stream (single calls: 0.65 of peak at this size)")
     del batch, outs, m4
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.utils.mxfp8 import requantize_fp8_block_to_mxfp8
+    f8 = [block_fp8(w, [128, 128]) for w in ws]
+    batch, outs = _record(lambda: [requantize_fp8_block_to_mxfp8(q, s) for q, s in f8])
+    run("next_fp8_to_mxfp8", "fp8_to_mxfp8", batch.run,
+        "FP8 128x128 block-scaled codes (general fp32 scales) -> MXFP8 in one pass, as the MXFP8 converter submits a shard: one job list")
+    del batch, outs, f8
     i4 = [pack_layer(w, 128) for w in ws]
     run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")
     del i4

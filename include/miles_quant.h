@@ -97,6 +97,28 @@ int mq_fp8_block_quant_pow2(const void* w, int dtype, int64_t ldw, void* q, floa
  *   w [rows,K] contiguous, K % 32 == 0; q [rows,K] e4m3fn; scale [rows,K/32] E8M0 bytes */
 int mq_mxfp8_quant(const void* w, int dtype, void* q, uint8_t* scale, int64_t rows, int64_t K, void* stream);
 
+/* FP8 128x128 block-scaled source -> MXFP8           tools/convert_hf_to_mxfp8.py:56-102,180-195
+ * A source tensor is e4m3fn codes x [M,K] with one scale per 128x128 tile: a grid of at least ceil(M/128) rows and
+ * ceil(K/128) columns whose rows are lds elements apart (the reference crops a larger grid, :79,:91).
+ * mq_fp8_scales_pow2_flag: _load_source_scale_u8's test of an fp32 grid (:81-86): *flag (one uint32 on the device) <- 1
+ *   when every one of its rows x cols scales has a zero mantissa and a clear sign bit, else 0.  The caller reads the
+ *   flag and picks the branch, as the reference does with .item().
+ * mq_e8m0_expand_tile_scales: _source_fp8_to_mxfp8_scale_u8 (:98-102): out [M, groups] bytes (groups = K/32),
+ *   out[r,g] = exponent byte of tile (r/128, g/4); the grid holds the bytes themselves, or (scales_are_f32 != 0) fp32
+ *   powers of two whose byte is bits 23..30 (:85).  The codes of such a source are kept as they are.
+ * mq_fp8_block_to_mxfp8: every other source (:187-190): block_quant_dequant(x, s, [128,128], float32) -- SGLang's
+ *   function, third party: the scales repeated over their tiles and one fp32 multiply f32(code) * s -- followed by
+ *   mxfp8_quantize; q [M,K] e4m3fn, scale [M,K/32] E8M0 bytes; K % 32 == 0.  The fp32 tensor exists in registers only.
+ *   (A source tensor that stays unquantized becomes bf16 through mq_fp8_block_dequant, :203-215.)
+ * mq_e8m0_bytes_to_f32: the fp32 scales of a grid stored as exponent bytes (:93): out[i] = the float whose bits are
+ *   s[i] << 23, n contiguous values. */
+int mq_e8m0_bytes_to_f32(const uint8_t* s, float* out, int64_t n, void* stream);
+int mq_fp8_scales_pow2_flag(const float* s, int64_t rows, int64_t cols, int64_t lds, uint32_t* flag, void* stream);
+int mq_e8m0_expand_tile_scales(const void* s, int scales_are_f32, int64_t lds, uint8_t* out, int64_t M, int64_t groups,
+                               void* stream);
+int mq_fp8_block_to_mxfp8(const void* x, const float* s, int64_t lds, void* q, uint8_t* scale, int64_t M, int64_t K,
+                          void* stream);
+
 /* quantize_mxfp4(weight, group_size)                  miles/utils/mxfp4.py:11-31
  *   w: numel elements, contiguous, groups of `group` consecutive elements (numel % group == 0, numel % 2 == 0)
  *   packed [numel/2] bytes (element 2j in the low nibble: magnitude code | sign << 3); scale [numel/group] E8M0 */
@@ -229,6 +251,12 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_MXFP4_TO_FP8         e2m1 pairs    e4m3          fp32 tiles     aux = E8M0 bytes (in)       -
  *     (mq_mxfp4_to_fp8_block with out_dim = rows, in_dim = cols, both multiples of 128: the experts of a checkpoint
  *      shard re-coded in launches of up to MQ_MAX_GROUP tensors)
+ *   MQ_JOB_FP8_TO_MXFP8         e4m3          e4m3          E8M0 bytes     aux = fp32 tile scales (in) -
+ *     (mq_fp8_block_to_mxfp8 with M = rows, K = cols, lds = ld; 16-byte aligned tensors share launches of up to
+ *      MQ_MAX_GROUP)
+ *   MQ_JOB_E8M0_EXPAND          tile scales   E8M0 bytes    -              -                           -
+ *     (mq_e8m0_expand_tile_scales with M = rows, groups = cols, lds = ld; dtype MQ_F32: the grid holds fp32 powers of
+ *      two, any other dtype code: exponent bytes)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, MXFP4, INT4_PACK, INT4_PACK_ASYM, FP8_TENSOR and NVFP4 run their tuned
@@ -257,7 +285,9 @@ enum {
     MQ_JOB_UE8M0_PACK = 9,
     MQ_JOB_FP8_TENSOR = 10,
     MQ_JOB_INT4_PACK_ASYM = 11,
-    MQ_JOB_MXFP4_TO_FP8 = 12
+    MQ_JOB_MXFP4_TO_FP8 = 12,
+    MQ_JOB_FP8_TO_MXFP8 = 13,
+    MQ_JOB_E8M0_EXPAND = 14
 };
 typedef struct mq_job {
     int32_t kind;

@@ -29,6 +29,10 @@ SIGNATURES = {
     "mq_ue8m0_pack_scales": [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
     "mq_fp8_block_dequant": [_vp, _vp, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp8_quant": [_vp, _i32, _vp, _vp, _i64, _i64, _vp],
+    "mq_e8m0_bytes_to_f32": [_vp, _vp, _i64, _vp],
+    "mq_fp8_scales_pow2_flag": [_vp, _i64, _i64, _i64, _vp, _vp],
+    "mq_e8m0_expand_tile_scales": [_vp, _i32, _i64, _vp, _i64, _i64, _vp],
+    "mq_fp8_block_to_mxfp8": [_vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp],
     "mq_int4_fake_quant": [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp],
     "mq_int4_unpack_dequant": [_vp, _vp, _i32, _vp, _i64, _i64, _i32, _vp],
     "mq_mxfp4_to_fp8_block": [_vp, _vp, _vp, _vp, _i64, _i64, _vp],
@@ -61,7 +65,8 @@ NVFP4_CARRY_AMAX = 8                                      # MQ_NVFP4_CARRY_AMAX:
 RECORD_AMAX_WORD, RECORD_REDO_WORD, RECORD_VOLATILE_WORD = 1024, 1028, 1029
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
- JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM, JOB_MXFP4_TO_FP8) = range(13)
+ JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM, JOB_MXFP4_TO_FP8,
+ JOB_FP8_TO_MXFP8, JOB_E8M0_EXPAND) = range(15)
 
 
 class Job(_c.Structure):

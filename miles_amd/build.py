@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmiles_quant.so")
 
-SOURCES = ["mq_core.hip", "mq_fp8_block.hip", "mq_mxfp8.hip", "mq_mxfp4.hip", "mq_fake_quant.hip", "mq_int4.hip", "mq_nvfp4.hip", "mq_fp8_tensor.hip", "mq_selftest.hip", "mq_probe.hip",
+SOURCES = ["mq_core.hip", "mq_fp8_block.hip", "mq_mxfp8.hip", "mq_rescale.hip", "mq_mxfp4.hip", "mq_fake_quant.hip", "mq_int4.hip", "mq_nvfp4.hip", "mq_fp8_tensor.hip", "mq_selftest.hip", "mq_probe.hip",
            "mq_sync.hip"]
 
 FLAGS = [

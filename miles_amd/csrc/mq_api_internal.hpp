@@ -22,6 +22,14 @@ struct MqDequantArgs {
     int block;
 };
 
+struct MqRescaleArgs {
+    const void* x;
+    const float* s;
+    void* q;
+    uint8_t* scale;
+    int64_t M, K, lds;
+};
+
 namespace mq {
 __device__ __forceinline__ float load_f32(const void* p, int64_t i, int dtype) {
     if (dtype == MQ_BF16) return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)p)[i] << 16);

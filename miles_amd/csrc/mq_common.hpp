@@ -169,6 +169,23 @@ __device__ __forceinline__ float sw_e4m3fn_decode(uint32_t c) {
     return u2f(sign | ((e + 120u) << 23) | (m << 20));
 }
 
+// ---- E8M0 scales of the MX formats ---------------------------------------------------------------
+// exponent byte of the smallest power of two >= v, for v >= 0: saturating at 0xFE (inf included), 0 for v == 0 and for
+// subnormals up to 2^-127, 0xFF for a NaN
+__device__ __forceinline__ uint32_t e8m0_ceil(float v) {
+    const uint32_t u = f2u(v);
+    uint32_t e = u >> 23, m = u & 0x7FFFFFu;
+    if (u >= 0x7F800000u) return u == 0x7F800000u ? 0xFEu : 0xFFu;
+    if ((m > 0 && e != 0xFEu) && !(e == 0 && m <= 0x400000u)) e++;
+    return e;
+}
+// 2^(127 - e), exact (subnormal for the two largest bytes); 1 for byte 0
+__device__ __forceinline__ float e8m0_inverse(uint32_t e) {
+    if (e == 0) return 1.0f;
+    if (e >= 254) return u2f(e == 254 ? 0x00400000u : 0x00200000u);
+    return u2f((254u - e) << 23);
+}
+
 // ---- hardware conversions ---------------------------------------------------------------------
 // two floats -> two e4m3 bytes in the low (hi=false) or high (hi=true) half of `old`.
 // v_cvt_pk_fp8_f32 rounds to nearest even including into the subnormal range and rounds (448, 464]

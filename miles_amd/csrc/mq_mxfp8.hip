@@ -19,19 +19,6 @@ constexpr int kMxThreads = 256;
 #endif
 constexpr int kMxUnroll = MQ_MX_UNROLL;  // 16-byte units per lane (2 measured best on MI355X: 1 pays the prologue too often, 4 lowers occupancy)
 
-__device__ __forceinline__ uint32_t e8m0_ceil(float v) {
-    const uint32_t u = f2u(v);
-    uint32_t e = u >> 23, m = u & 0x7FFFFFu;
-    if (u >= 0x7F800000u) return u == 0x7F800000u ? 0xFEu : 0xFFu;
-    if ((m > 0 && e != 0xFEu) && !(e == 0 && m <= 0x400000u)) e++;
-    return e;
-}
-__device__ __forceinline__ float e8m0_inverse(uint32_t e) {
-    if (e == 0) return 1.0f;
-    if (e >= 254) return u2f(e == 254 ? 0x00400000u : 0x00200000u);
-    return u2f((254u - e) << 23);
-}
-
 // 16-bit inputs, bf16 or fp16 (F16): the two instances differ in the conversion to fp32 and in the infinity pattern
 template <class Table, int F16>
 __global__ __launch_bounds__(kMxThreads) void mxfp8_bf16_kernel(const Table tab) {

@@ -50,6 +50,8 @@ int64_t mq_int4_zero_tiles(int64_t rows, int64_t cols, int group);
 int mq_mxfp4_to_fp8_job(RecodeJob& job, const void* packed, const void* scale, void* y, void* tile_scale, int64_t out_dim,
                         int64_t in_dim);
 int mq_mxfp4_to_fp8_launch_group(const RecodeTable& tab, hipStream_t st);
+bool mq_fp8_to_mxfp8_fast_ok(const void* x, const void* q, int64_t M, int64_t K);
+int mq_fp8_to_mxfp8_launch_group(const MqRescaleArgs* a, int n, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -87,6 +89,8 @@ static bool job_fast(const mq_job& j) {
             return mq_fp8_tensor_fast_ok(j.in, j.dtype, j.out, j.rows, j.cols, j.ld);
         case MQ_JOB_MXFP4_TO_FP8:
             return true;               // check_job has refused what the kernel does not take
+        case MQ_JOB_FP8_TO_MXFP8:
+            return mq_fp8_to_mxfp8_fast_ok(j.in, j.out, j.rows, j.cols) && j.ld >= (j.cols + 127) / 128 && j.ld <= 0x7FFFFFFF;
         default:
             return false;
     }
@@ -94,7 +98,7 @@ static bool job_fast(const mq_job& j) {
 
 static int64_t copy_dst_pitch(const mq_job& j);
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_MXFP4_TO_FP8) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_E8M0_EXPAND) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
@@ -105,6 +109,10 @@ static int check_job(const mq_job& j) {
     }
     if (j.kind == MQ_JOB_UE8M0_PACK)
         return j.p0 >= 0 && j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-pack job");
+    if (j.kind == MQ_JOB_E8M0_EXPAND)
+        return j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-expansion job");
+    if (j.kind == MQ_JOB_FP8_TO_MXFP8 && !empty && (!j.aux || j.rows_per_block != 0))
+        return mq_fail(MQ_ERR_ARG, "FP8 to MXFP8 job without tile scales");
     if (j.kind == MQ_JOB_MXFP4_TO_FP8) {
         if (j.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "bad MXFP4 to FP8 job");
         RecodeJob probe;
@@ -149,6 +157,10 @@ static int run_single(const mq_job& j, void* stream) {
                                                  j.rows, j.cols, j.p0, stream);
         case MQ_JOB_UE8M0_PACK:
             return mq_ue8m0_pack_scales((const float*)j.in, (int32_t*)j.out, j.p0, j.rows, j.cols, j.p1, j.ld != 0, stream);
+        case MQ_JOB_FP8_TO_MXFP8:
+            return mq_fp8_block_to_mxfp8(j.in, (const float*)j.aux, j.ld, j.out, (uint8_t*)j.scale, j.rows, j.cols, stream);
+        case MQ_JOB_E8M0_EXPAND:
+            return mq_e8m0_expand_tile_scales(j.in, j.dtype == MQ_F32, j.ld, (uint8_t*)j.out, j.rows, j.cols, stream);
         case MQ_JOB_MXFP4_TO_FP8:
             return mq_mxfp4_to_fp8_block((const uint8_t*)j.in, (const uint8_t*)j.aux, j.out, (float*)j.scale, j.rows, j.cols, stream);
         default:
@@ -527,6 +539,15 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                      : head.kind == MQ_JOB_MXFP4     ? mq_mxfp4_launch_group(head.dtype, tab, st)
                      : head.kind == MQ_JOB_INT4_PACK ? mq_int4_pack_launch_group(head.dtype, tab, head.p0, st)
                                                      : mq_int4_pack_asym_launch_group(head.dtype, tab, head.p0, st);
+                break;
+            }
+            case MQ_JOB_FP8_TO_MXFP8: {
+                MqRescaleArgs a[kMaxGroup];
+                for (int t = 0; t < cnt; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    a[t] = MqRescaleArgs{jb.in, (const float*)jb.aux, jb.out, (uint8_t*)jb.scale, jb.rows, jb.cols, jb.ld};
+                }
+                rc = mq_fp8_to_mxfp8_launch_group(a, cnt, st);
                 break;
             }
             case MQ_JOB_MXFP4_TO_FP8: {

@@ -4,11 +4,12 @@
         [--num-layers-at-start-in-bf16 N] [--num-layers-at-end-in-bf16 N] [--extra-high-precision-layers-hf ...]
 
 Mirror of the reference's tools/convert_hf_to_mxfp8.py (`process_file` :123-228, `convert_mxfp8` :231-308).
-Sources: BF16/FP16/FP32 checkpoints, and block-scaled FP8 checkpoints whose [128,128] scales are powers of two
-(`scale_fmt: ue8m0`): those are re-labelled without touching the codes (`_source_fp8_to_mxfp8_scale_u8`,
-:98-102).  FP8 sources with general fp32 scales need SGLang's `block_quant_dequant` in the reference; here
-they are dequantized by the FP8 block dequant kernel's arithmetic in fp32 torch ops on the device and
-re-quantized.
+Sources: BF16/FP16/FP32 checkpoints, and block-scaled FP8 checkpoints (`scale_fmt: ue8m0`, [128,128] scales stored
+as exponent bytes or as fp32).  A tensor whose tile scales are powers of two keeps its codes and gets one exponent
+byte per 1x32 group (`_source_fp8_to_mxfp8_scale_u8`, :98-102: `mq_e8m0_expand_tile_scales`); a tensor with any other
+scale is dequantized to fp32 and quantized again in the reference (SGLang's `block_quant_dequant`, :187-190), which
+`mq_fp8_block_to_mxfp8` does in one pass over the codes; a tensor that stays in bf16 goes through the FP8 block
+dequantizer (:203-215).  The power-of-two test (:81-86) runs on the device, one flag per tensor, read once per shard.
 """
 
 from __future__ import annotations
@@ -21,9 +22,9 @@ import torch
 
 from miles_amd import launch
 from miles_amd.tools import _checkpoint as ckpt
-from miles_amd.tools.fp8_cast_bf16 import weight_dequant
 from miles_amd.utils.mxfp8 import (MXFP8_GROUP_SIZE, MXFP8_SKIP_WEIGHT_SUBSTRINGS, MXFP8_SOURCE_FP8_DTYPES,
-                                   should_use_mxfp8)
+                                   dequantize_fp8_source, expand_tile_scales_e8m0, exponent_bytes_to_fp32,
+                                   fp8_tile_scales_pow2, requantize_fp8_block_to_mxfp8, should_use_mxfp8)
 from miles_amd.utils.mxfp8 import mxfp8_quantize as quantize_mxfp8
 
 SOURCE_FP8_BLOCK_SIZE = [128, 128]
@@ -49,40 +50,14 @@ def _source_kind(cfg: dict) -> str:
                      "{quant_method=fp8, weight_block_size=[128, 128], scale_fmt=ue8m0} sources are supported.")
 
 
-def _tile_counts(weight: torch.Tensor) -> tuple[int, int]:
-    n, k = weight.shape[-2], weight.shape[-1]
-    return -(-n // SOURCE_FP8_BLOCK_SIZE[0]), -(-k // SOURCE_FP8_BLOCK_SIZE[1])
-
-
-def _load_source_scale_u8(weights, weight_key, weight, source_scale_index, input_path, device, current_filename):
-    """(fp32 scales, uint8 exponents or None, scale key) of a source FP8 weight."""
+def _source_scale(weights, weight_key, source_scale_index, input_path, device, current_filename):
+    """(tile-scale tensor as stored -- uint8 exponents or fp32 --, its key) of a source FP8 weight; the tensor may sit in
+    another shard (reference :65-72)."""
     scale_key = _strip_weight_suffix(weight_key) + SOURCE_FP8_SCALE_KEY_SUFFIX
     scale_file = source_scale_index[scale_key]
-    scale = weights[scale_key] if scale_file == current_filename and scale_key in weights else \
-        ckpt.load_tensor(input_path, scale_file, scale_key, device)
-    nt, kt = _tile_counts(weight)
-    if scale.dtype == torch.uint8:
-        u8 = scale[..., :nt, :kt].contiguous()
-        return (u8.to(torch.int32) << 23).view(torch.float32), u8, scale_key
-    assert scale.dtype == torch.float32
-    f32 = scale[..., :nt, :kt].contiguous()
-    bits = f32.view(torch.int32)
-    pow2 = not torch.any((bits & 0x007FFFFF) != 0).item() and not torch.any(bits < 0).item()
-    return f32, (((bits >> 23) & 0xFF).to(torch.uint8) if pow2 else None), scale_key
-
-
-def _source_fp8_to_mxfp8_scale_u8(weight: torch.Tensor, source_scale_u8: torch.Tensor) -> torch.Tensor:
-    """One exponent per 128x128 tile -> one per 1x32 group (repeat 128 down, 4 across), cropped."""
-    n, k = weight.shape[-2], weight.shape[-1]
-    wide = source_scale_u8.repeat_interleave(SOURCE_FP8_BLOCK_SIZE[0], dim=-2).repeat_interleave(
-        SOURCE_FP8_BLOCK_SIZE[1] // TARGET_MXFP8_BLOCK_SIZE[1], dim=-1)
-    return wide[..., :n, : k // TARGET_MXFP8_BLOCK_SIZE[1]].contiguous()
-
-
-def _dequant_fp32(weight: torch.Tensor, scale_fp32: torch.Tensor) -> torch.Tensor:
-    n, k = weight.shape
-    wide = scale_fp32.repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)[:, :k]
-    return (weight.float() * wide).contiguous()
+    if scale_file == current_filename and scale_key in weights:
+        return weights[scale_key], scale_key
+    return ckpt.load_tensor(input_path, scale_file, scale_key, device), scale_key
 
 
 def process_file(input_path, output_path, filename, result_collector, device, num_hidden_layers,
@@ -96,32 +71,48 @@ def process_file(input_path, output_path, filename, result_collector, device, nu
     skipped: list[str] = list(bf16_layers) if (num_layers_at_end_in_bf16 > 0 or num_layers_at_start_in_bf16 > 0) else []
     skip_substrings = (*MXFP8_SKIP_WEIGHT_SUBSTRINGS, *extra_high_precision_layers_hf, *bf16_layers)
 
-    def source_scale(key, tensor):
-        return _load_source_scale_u8(weights, key, tensor, source_scale_index, input_path, device, filename)
+    # what becomes of every .weight tensor: "quantize" (a high-precision source), "keep" (passed through), or, for the
+    # FP8 tensors of a block-scaled source, "relabel" (power-of-two tile scales: codes kept, one exponent per group),
+    # "requantize" (any other scales) and "dequantize" (a module that stays in bf16)
+    plan: dict[str, tuple] = {}
+    undecided = []            # FP8 tensors with fp32 scales: relabel or requantize, by the power-of-two test
+    for key, tensor in weights.items():
+        if not key.endswith(".weight"):
+            continue
+        fp8_source = source_is_block_fp8_ue8m0 and tensor.dtype in MXFP8_SOURCE_FP8_DTYPES
+        quantized = should_use_mxfp8(key, tuple(tensor.shape), tensor.dtype, skip_substrings=skip_substrings,
+                                     allow_source_fp8=source_is_block_fp8_ue8m0)
+        if not quantized and ".experts." not in key:
+            skipped.append(_strip_weight_suffix(key))
+        if not fp8_source:
+            plan[key] = ("quantize" if quantized else "keep", None, None)
+            continue
+        scale, scale_key = _source_scale(weights, key, source_scale_index, input_path, device, filename)
+        if not quantized:
+            plan[key] = ("dequantize", scale if scale.dtype == torch.float32 else exponent_bytes_to_fp32(scale), None)
+        elif scale.dtype == torch.uint8:
+            plan[key] = ("relabel", scale, scale_key)
+        else:
+            assert scale.dtype == torch.float32
+            plan[key] = ("requantize", scale, scale_key)
+            undecided.append(key)
+    for key, pow2 in zip(undecided, fp8_tile_scales_pow2((weights[k], plan[k][1]) for k in undecided)):
+        if pow2:
+            plan[key] = ("relabel", *plan[key][1:])
 
     with launch.deferred():
-        for key, tensor in weights.items():
-            if not key.endswith(".weight"):
-                continue
-            fp8_source = source_is_block_fp8_ue8m0 and tensor.dtype in MXFP8_SOURCE_FP8_DTYPES
-            if should_use_mxfp8(key, tuple(tensor.shape), tensor.dtype, skip_substrings=skip_substrings,
-                                allow_source_fp8=source_is_block_fp8_ue8m0):
-                if fp8_source:
-                    scale_f32, scale_u8, scale_key = source_scale(key, tensor)
-                    if scale_u8 is not None:
-                        out[key], out[scale_key] = tensor.contiguous(), _source_fp8_to_mxfp8_scale_u8(tensor, scale_u8)
-                    else:
-                        out[key], out[scale_key] = quantize_mxfp8(_dequant_fp32(tensor, scale_f32))
-                else:
-                    out[key], out[_strip_weight_suffix(key) + SOURCE_FP8_SCALE_KEY_SUFFIX] = quantize_mxfp8(tensor)
+        for key, (action, scale, scale_key) in plan.items():
+            tensor = weights[key]
+            if action == "quantize":
+                out[key], out[_strip_weight_suffix(key) + SOURCE_FP8_SCALE_KEY_SUFFIX] = quantize_mxfp8(tensor)
+            elif action == "relabel":
+                out[key], out[scale_key] = tensor.contiguous(), expand_tile_scales_e8m0(tensor, scale)
+            elif action == "requantize":
+                out[key], out[scale_key] = requantize_fp8_block_to_mxfp8(tensor, scale)
+            elif action == "dequantize":
+                out[key] = dequantize_fp8_source(tensor, scale)
             else:
-                if ".experts." not in key:
-                    skipped.append(_strip_weight_suffix(key))
-                if fp8_source:
-                    scale_f32, _, _ = source_scale(key, tensor)
-                    out[key] = weight_dequant(tensor.contiguous(), scale_f32)
-                else:
-                    out[key] = tensor
+                out[key] = tensor
     for key, tensor in weights.items():
         if key.endswith(".weight"):
             continue

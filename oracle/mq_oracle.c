@@ -409,6 +409,48 @@ void mqo_mxfp8(const void* w, int dtype, int64_t rows, int64_t K, uint8_t* q, ui
 }
 
 /* ------------------------------------------------------------------ */
+/* FP8 128x128 block-scaled source -> MXFP8                             */
+/* (tools/convert_hf_to_mxfp8.py:56-102,180-195)                        */
+/* ------------------------------------------------------------------ */
+/* The general-scale branch (:187-190):
+ *   w32 = block_quant_dequant(x, s, [128,128], torch.float32)   SGLang (third party, not in the tree): the tile scales
+ *         repeated 128 x 128, cropped, and ONE fp32 multiply  f32(e4m3(x)) * s[i/128, j/128]
+ *   q, scale = mxfp8_quantize(w32)                              mqo_mxfp8 on the fp32 tensor
+ * lds: row stride of the tile-scale grid in elements (the reference crops a larger grid, :79). */
+void mqo_fp8_block_to_mxfp8(const uint8_t* x, const float* s, int64_t lds, int64_t M, int64_t K,
+                            uint8_t* q, uint8_t* scale) {
+    float* w32 = (float*)malloc((size_t)(M * K > 0 ? M * K : 1) * sizeof(float));
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t c = 0; c < K; c++)
+            w32[r * K + c] = mqo_e4m3fn_to_f32(x[r * K + c]) * s[(r / 128) * lds + c / 128];
+    mqo_mxfp8(w32, MQ_F32, M, K, q, scale);
+    free(w32);
+}
+
+/* _load_source_scale_u8's test of an fp32 scale grid (:81-86): 1 when every mantissa is zero and no
+ * value has its sign bit set (the scales are then relabelled, not re-quantized), else 0. */
+int mqo_fp8_scales_pow2(const float* s, int64_t rows, int64_t cols, int64_t lds) {
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t c = 0; c < cols; c++) {
+            uint32_t u = f2u(s[r * lds + c]);
+            if ((u & 0x007FFFFFu) != 0 || (u >> 31) != 0) return 0;
+        }
+    return 1;
+}
+
+/* _source_fp8_to_mxfp8_scale_u8 (:98-102): one exponent byte per 128x128 tile -> one per 1x32 group
+ * (repeated 128 down and 4 across, cropped to [M, groups]).  is_f32: the grid holds fp32 powers of
+ * two and the byte is (bits >> 23) & 0xFF (:85); otherwise it holds the bytes themselves (:89-93). */
+void mqo_e8m0_expand_tile_scales(const void* s, int is_f32, int64_t lds, int64_t M, int64_t groups, uint8_t* out) {
+    for (int64_t r = 0; r < M; r++)
+        for (int64_t g = 0; g < groups; g++) {
+            int64_t i = (r / 128) * lds + g / 4;
+            out[r * groups + g] = is_f32 ? (uint8_t)((f2u(((const float*)s)[i]) >> 23) & 0xFFu) : ((const uint8_t*)s)[i];
+        }
+}
+
+/* ------------------------------------------------------------------ */
 /* MXFP4 (miles/utils/mxfp4.py:11-59): torch ops restated one by one    */
 /* ------------------------------------------------------------------ */
 /* quantize_mxfp4 (:11-31).  Groups of G consecutive elements of the flattened tensor.

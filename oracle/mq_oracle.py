@@ -67,6 +67,12 @@ def lib() -> ctypes.CDLL:
         L.mqo_fp8_block_dequant.argtypes = [vp, vp, i64, i64, i32, vp]
         L.mqo_mxfp8.restype = None
         L.mqo_mxfp8.argtypes = [vp, i32, i64, i64, vp, vp]
+        L.mqo_fp8_block_to_mxfp8.restype = None
+        L.mqo_fp8_block_to_mxfp8.argtypes = [vp, vp, i64, i64, i64, vp, vp]
+        L.mqo_fp8_scales_pow2.restype = i32
+        L.mqo_fp8_scales_pow2.argtypes = [vp, i64, i64, i64]
+        L.mqo_e8m0_expand_tile_scales.restype = None
+        L.mqo_e8m0_expand_tile_scales.argtypes = [vp, i32, i64, i64, i64, vp]
         L.mqo_int4_fake_quant.restype = None
         L.mqo_int4_fake_quant.argtypes = [vp, i32, i64, i64, i32, i32, vp, vp, vp]
         L.mqo_int4_fake_quant_block.restype = None
@@ -223,6 +229,48 @@ def mxfp8_quantize(weight: torch.Tensor):
     s = torch.empty((*weight.shape[:-1], k // 32), dtype=torch.uint8)
     lib().mqo_mxfp8(weight.data_ptr(), _DTYPE[weight.dtype], rows, k, q.data_ptr(), s.data_ptr())
     return q.view(torch.float8_e4m3fn), s
+
+
+def _tile_grid(weight: torch.Tensor, scale: torch.Tensor):
+    """The [ceil(M/128), ceil(K/128)] corner of a 2-D tile-scale grid and its row stride in elements."""
+    assert weight.dim() == 2 and scale.dim() == 2 and scale.stride(1) == 1
+    m, k = weight.shape
+    nt, kt = ceil_div(m, 128), ceil_div(k, 128)
+    assert scale.shape[0] >= nt and scale.shape[1] >= kt
+    return nt, kt, scale.stride(0)
+
+
+def fp8_block_to_mxfp8(weight: torch.Tensor, scale: torch.Tensor):
+    """tools/convert_hf_to_mxfp8.py:187-190: block_quant_dequant(w, s, [128,128], float32) -> mxfp8_quantize.
+    weight e4m3fn (or uint8 codes) [M,K], scale fp32 grid -> (e4m3fn [M,K], uint8 [M,K/32])."""
+    assert weight.device.type == "cpu" and weight.element_size() == 1 and scale.dtype == torch.float32
+    weight = weight.contiguous()
+    m, k = weight.shape
+    if k % 32 != 0:
+        raise ValueError(f"Last dim {k} must be divisible by 32 for MXFP8.")
+    _nt, _kt, lds = _tile_grid(weight, scale)
+    q = torch.empty((m, k), dtype=torch.uint8)
+    s = torch.empty((m, k // 32), dtype=torch.uint8)
+    lib().mqo_fp8_block_to_mxfp8(weight.data_ptr(), scale.data_ptr(), lds, m, k, q.data_ptr(), s.data_ptr())
+    return q.view(torch.float8_e4m3fn), s
+
+
+def fp8_scales_are_pow2(weight: torch.Tensor, scale: torch.Tensor) -> bool:
+    """tools/convert_hf_to_mxfp8.py:81-86 on the cropped grid of an fp32 scale tensor."""
+    assert scale.dtype == torch.float32
+    nt, kt, lds = _tile_grid(weight, scale)
+    return bool(lib().mqo_fp8_scales_pow2(scale.data_ptr(), nt, kt, lds))
+
+
+def expand_tile_scales_e8m0(weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """tools/convert_hf_to_mxfp8.py:85,98-102: exponent bytes of a tile-scale grid (uint8, or fp32 powers of two)
+    repeated to one byte per 1x32 group -> uint8 [M, K/32]."""
+    assert scale.dtype in (torch.uint8, torch.float32)
+    _nt, _kt, lds = _tile_grid(weight, scale)
+    m, k = weight.shape
+    out = torch.empty((m, k // 32), dtype=torch.uint8)
+    lib().mqo_e8m0_expand_tile_scales(scale.data_ptr(), int(scale.dtype == torch.float32), lds, m, k // 32, out.data_ptr())
+    return out
 
 
 # --------------------------------------------------------------------------

@@ -226,10 +226,68 @@ def fp8_act_quant() -> dict:
     return fam.save()
 
 
+def fp8_to_mxfp8() -> dict:
+    fam = Family("fp8_to_mxfp8", "torch_fp8_block_to_mxfp8 / torch_source_fp8_to_mxfp8_scale_u8 / torch_scales_pow2 = "
+                                 "tools/convert_hf_to_mxfp8.py:56-102,180-195 (block_quant_dequant is SGLang's: repeat, crop, "
+                                 "one fp32 multiply)",
+                 "torch CPU kernels running the reference's op chain; MXFP8 arithmetic as in the mxfp8 family (parity "
+                 "unpinned against Transformer Engine and SGLang)")
+    g = torch.Generator().manual_seed(31)
+    for shape in [(128, 256), (256, 384), (130, 288), (64, 96), (3, 2, 130, 160)]:
+        n, k = shape[-2:]
+        w = (torch.randn(shape, generator=g) * 0.02 * torch.exp(torch.randn(shape[:-1] + (1,), generator=g))).to(torch.bfloat16)
+        flat = w.reshape(-1, n, k)
+        pairs = [T.torch_block_fp8(m, (128, 128)) for m in flat]
+        codes = torch.stack([q for q, _ in pairs]).reshape(shape)
+        scale = torch.stack([s for _, s in pairs]).reshape(*shape[:-2], -(-n // 128), -(-k // 128))
+        q, s = T.torch_fp8_block_to_mxfp8(codes, scale)
+        name = "x".join(map(str, shape))
+        fam.add(f"requant_{name}_amax_scales", {"shape": list(shape), "scales": "amax / 448 of a bf16 tensor"},
+                codes=codes, tile_scale=scale, q=q, scale=s, pow2=np.asarray([int(T.torch_scales_pow2(scale))]))
+    # every code except the two NaN bytes, scales over forty binades (fp32-subnormal products included), a grid larger
+    # than the weight needs (the reference crops it)
+    codes = torch.arange(256, dtype=torch.uint8).repeat(260, 2)[:, :416].contiguous()
+    codes = torch.where((codes & 0x7F) == 0x7F, torch.zeros_like(codes), codes)
+    scale = torch.exp(torch.randn((4, 5), generator=g) * 9).float()
+    scale[0, 1], scale[1, 0], scale[2, 3] = 0.0, -scale[1, 0], 2.0 ** -140
+    q, s = T.torch_fp8_block_to_mxfp8(codes.view(T.F8), scale)
+    fam.add("requant_all_codes_260x416_wide_grid", {"shape": [260, 416], "scales": "lognormal, zero, negative, subnormal; grid 4x5"},
+            codes=codes, tile_scale=scale, q=q, scale=s, pow2=np.asarray([0]))
+    # power-of-two sources: the codes stay, the exponent bytes are repeated per 1x32 group
+    for shape in [(130, 288), (256, 512), (2, 140, 160)]:
+        n, k = shape[-2:]
+        grid = (*shape[:-2], -(-n // 128), -(-k // 128))
+        exps = torch.randint(100, 140, grid, generator=g)
+        f32 = torch.ldexp(torch.ones(grid), exps - 127).float()
+        u8 = exps.to(torch.uint8)
+        name = "x".join(map(str, shape))
+        fam.add(f"relabel_{name}", {"shape": list(shape)}, scale_f32=f32, scale_u8=u8,
+                expanded=T.torch_source_fp8_to_mxfp8_scale_u8(shape, u8),
+                bytes_from_f32=T.torch_source_scale_bytes(f32), pow2=np.asarray([int(T.torch_scales_pow2(f32))]))
+    for label, value in (("negative_pow2", -0.5), ("mantissa_bit", 1.0000001), ("zero", 0.0)):
+        f32 = torch.ldexp(torch.ones((2, 3)), torch.randint(-20, 5, (2, 3), generator=g)).float()
+        f32[1, 2] = value
+        fam.add(f"pow2_test_{label}", {"shape": [2, 3]}, scale_f32=f32, pow2=np.asarray([int(T.torch_scales_pow2(f32))]))
+    return fam.save()
+
+
+FAMILIES = (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4, fake_quant, fp8_act_quant, fp8_to_mxfp8)
+
+
 def main() -> None:
-    manifest = {"generator": "tests/golden/make_fixtures.py", "torch": torch.__version__,
-                "families": [f() for f in (fp8_block, fp8_blockwise, fp8_dequant, mxfp8, mxfp4, int4, nvfp4, fake_quant, fp8_act_quant)]}
-    with open(os.path.join(HERE, "manifest.json"), "w") as f:
+    """All families, or only those named on the command line (their entries replace the manifest's)."""
+    wanted = set(sys.argv[1:])
+    path = os.path.join(HERE, "manifest.json")
+    if wanted:
+        with open(path) as f:
+            manifest = json.load(f)
+        fresh = {fam["file"]: fam for fam in (f() for f in FAMILIES if f.__name__ in wanted)}
+        kept = [fresh.pop(fam["file"], fam) for fam in manifest["families"]]
+        manifest["families"] = kept + list(fresh.values())
+    else:
+        manifest = {"generator": "tests/golden/make_fixtures.py", "torch": torch.__version__,
+                    "families": [f() for f in FAMILIES]}
+    with open(path, "w") as f:
         json.dump(manifest, f, indent=1)
     total = sum(os.path.getsize(os.path.join(HERE, fam["file"])) for fam in manifest["families"])
     print(f"wrote {len(manifest['families'])} fixture files, {total / 1e6:.2f} MB, "

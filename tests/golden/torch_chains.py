@@ -60,6 +60,40 @@ def torch_mxfp8(w):
     return q.reshape(w.shape), e.to(torch.uint8).reshape(*w.shape[:-1], k // 32)
 
 
+def torch_block_quant_dequant_f32(codes, scale):
+    """SGLang's block_quant_dequant(x_q, x_s, [128, 128], torch.float32) as the reference calls it
+    (tools/convert_hf_to_mxfp8.py:187-189): the tile scales repeated over their tiles, cropped, one fp32 multiply."""
+    n, k = codes.shape[-2:]
+    wide = scale.repeat_interleave(128, dim=-2).repeat_interleave(128, dim=-1)[..., :n, :k]
+    return codes.to(torch.float32) * wide
+
+
+def torch_fp8_block_to_mxfp8(codes, scale):
+    """tools/convert_hf_to_mxfp8.py:187-190: dequantize to fp32, quantize again as MXFP8."""
+    nt, kt = -(-codes.shape[-2] // 128), -(-codes.shape[-1] // 128)
+    return torch_mxfp8(torch_block_quant_dequant_f32(codes, scale[..., :nt, :kt].contiguous()).contiguous())
+
+
+def torch_scales_pow2(scale_fp32):
+    """tools/convert_hf_to_mxfp8.py:81-84."""
+    bits = scale_fp32.contiguous().view(torch.int32)
+    return (not torch.any((bits & 0x007FFFFF) != 0).item()) and (not torch.any(bits < 0).item())
+
+
+def torch_source_scale_bytes(scale):
+    """tools/convert_hf_to_mxfp8.py:85 (fp32 powers of two) / :74-75 (stored bytes)."""
+    if scale.dtype == torch.uint8:
+        return scale
+    return ((scale.contiguous().view(torch.int32) >> 23) & 0xFF).to(torch.uint8)
+
+
+def torch_source_fp8_to_mxfp8_scale_u8(weight_shape, scale_u8):
+    """tools/convert_hf_to_mxfp8.py:98-102."""
+    n, k = weight_shape[-2:]
+    wide = scale_u8.repeat_interleave(128, dim=-2).repeat_interleave(4, dim=-1)
+    return wide[..., :n, : k // 32].contiguous()
+
+
 def torch_quantize_mxfp4(weight, group_size):
     """miles/utils/mxfp4.py:11-31."""
     blocks = weight.reshape(-1, group_size)

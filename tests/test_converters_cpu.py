@@ -109,23 +109,17 @@ def test_nvfp4_converter_uses_compact_bf16_moe_prefixes(tmp_path):
     assert index["metadata"]["total_size"] == sum(t.numel() * 2 for t in weights.values())   # bytes for this tool
 
 
-def test_mxfp8_source_detection_and_scale_relabelling():
+def test_mxfp8_source_detection_and_scale_lookup():
     assert MX._source_kind({}) == "bf16" and MX._source_kind({"quantization_config": {"quant_method": "bf16"}}) == "bf16"
     fp8 = {"quantization_config": {"quant_method": "fp8", "weight_block_size": [128, 128], "scale_fmt": "ue8m0"}}
     assert MX._source_kind(fp8) == "fp8_ue8m0"
     with pytest.raises(ValueError, match="Unsupported source quantization_config"):
         MX._source_kind({"quantization_config": {"quant_method": "fp8", "weight_block_size": [128, 128]}})
-    w = torch.zeros(200, 288, dtype=torch.uint8)
-    u8 = torch.tensor([[120, 121, 122], [130, 131, 132]], dtype=torch.uint8)
-    out = MX._source_fp8_to_mxfp8_scale_u8(w, u8)
-    assert out.shape == (200, 9)
-    assert out[0].tolist() == [120] * 4 + [121] * 4 + [122] and out[199].tolist() == [130] * 4 + [131] * 4 + [132]
-    # fp32 power-of-two scales are recognised and turned into exponents; others are not
-    weights = {"a.weight": w, "a.weight_scale_inv": torch.tensor([[0.5, 2.0, 1.0], [4.0, 0.25, 8.0]])}
-    f32, e, key = MX._load_source_scale_u8(weights, "a.weight", w, {"a.weight_scale_inv": "s"}, ".", "cpu", "s")
-    assert key == "a.weight_scale_inv" and e.tolist() == [[126, 128, 127], [129, 125, 130]]
-    weights["a.weight_scale_inv"] = torch.tensor([[0.5, 3.0, 1.0], [4.0, 0.25, 8.0]])
-    assert MX._load_source_scale_u8(weights, "a.weight", w, {"a.weight_scale_inv": "s"}, ".", "cpu", "s")[1] is None
+    # a weight's tile scales are looked up under `<name>.weight_scale_inv`, in this shard's tensors when they are there
+    scales = torch.tensor([[0.5, 2.0, 1.0], [4.0, 0.25, 8.0]])
+    weights = {"a.weight": torch.zeros(200, 288, dtype=torch.uint8), "a.weight_scale_inv": scales}
+    got, key = MX._source_scale(weights, "a.weight", {"a.weight_scale_inv": "s"}, ".", "cpu", "s")
+    assert key == "a.weight_scale_inv" and got is scales
     with pytest.raises(ValueError, match="Expected key ending"):
         MX._strip_weight_suffix("a.bias")
 

@@ -118,6 +118,25 @@ class _OracleImpl:
     def act_quant(self, x, block, fmt, inplace=False):
         return self.o.act_quant(x, block, fmt, inplace=inplace)
 
+    def _each(self, fn, weight, scale):
+        """The oracle takes one matrix at a time: apply to every matrix of a stacked tensor."""
+        n, k = weight.shape[-2:]
+        outs = [fn(w, s) for w, s in zip(weight.reshape(-1, n, k), scale.reshape(-1, *scale.shape[-2:]))]
+        return outs, weight.shape[:-2]
+
+    def fp8_block_to_mxfp8(self, codes, scale):
+        outs, lead = self._each(self.o.fp8_block_to_mxfp8, codes, scale)
+        return (torch.stack([q for q, _ in outs]).reshape(codes.shape),
+                torch.stack([s for _, s in outs]).reshape(*lead, codes.shape[-2], codes.shape[-1] // 32))
+
+    def expand_tile_scales(self, weight, scale):
+        outs, lead = self._each(self.o.expand_tile_scales_e8m0, weight, scale)
+        return torch.stack(outs).reshape(*lead, weight.shape[-2], weight.shape[-1] // 32)
+
+    def scales_pow2(self, weight, scale):
+        outs, _ = self._each(self.o.fp8_scales_are_pow2, weight, scale)
+        return all(outs)
+
 
 class _HipImpl:
     dev = DEV
@@ -170,6 +189,18 @@ class _HipImpl:
     def act_quant(self, x, block, fmt, inplace=False):
         from miles_amd.kernels.quant.fp8_act_quant import act_quant
         return act_quant(x.clone(), block, fmt, inplace=inplace)
+
+    def fp8_block_to_mxfp8(self, codes, scale):
+        from miles_amd.utils.mxfp8 import requantize_fp8_block_to_mxfp8
+        return requantize_fp8_block_to_mxfp8(codes, scale)
+
+    def expand_tile_scales(self, weight, scale):
+        from miles_amd.utils.mxfp8 import expand_tile_scales_e8m0
+        return expand_tile_scales_e8m0(weight, scale)
+
+    def scales_pow2(self, weight, scale):
+        from miles_amd.utils.mxfp8 import fp8_tile_scales_pow2
+        return fp8_tile_scales_pow2([(weight, scale)])[0]
 
 
 def _check_fp8_block(impl, case):
@@ -273,7 +304,31 @@ def _check_act_quant(impl, case):
     _same(impl.act_quant(x, info["block"], fmt, inplace=True), _t("fp8_act_quant", case, "qdq", dt), f"{case} quantize-dequantize")
 
 
-_CHECKS = [("fp8_block", _check_fp8_block), ("fp8_blockwise_cast", _check_fp8_blockwise), ("fp8_dequant", _check_fp8_dequant),
+def _check_fp8_to_mxfp8(impl, case):
+    fam = "fp8_to_mxfp8"
+    shape = _info(fam, case)["shape"]
+    want_pow2 = bool(_t(fam, case, "pow2").item())
+    if case.startswith("requant_"):
+        codes = _t(fam, case, "codes").view(torch.float8_e4m3fn).to(impl.dev)
+        tile_scale = _t(fam, case, "tile_scale").to(impl.dev)
+        assert impl.scales_pow2(codes, tile_scale) == want_pow2, f"{case} power-of-two test"
+        q, s = impl.fp8_block_to_mxfp8(codes, tile_scale)
+        _same(s, _t(fam, case, "scale"), f"{case} E8M0 scales")
+        _same(q, _t(fam, case, "q"), f"{case} codes")
+        return
+    f32 = _t(fam, case, "scale_f32").to(impl.dev)
+    weight = torch.empty(shape, dtype=torch.uint8, device=impl.dev).view(torch.float8_e4m3fn)
+    if case.startswith("pow2_test_"):
+        weight = torch.empty((f32.shape[0] * 128, f32.shape[1] * 128), dtype=torch.uint8, device=impl.dev)
+        assert impl.scales_pow2(weight, f32) == want_pow2, f"{case} power-of-two test"
+        return
+    assert impl.scales_pow2(weight, f32) == want_pow2, f"{case} power-of-two test"
+    want = _t(fam, case, "expanded")
+    _same(impl.expand_tile_scales(weight, f32), want, f"{case} group scales from fp32 powers of two")
+    _same(impl.expand_tile_scales(weight, _t(fam, case, "scale_u8").to(impl.dev)), want, f"{case} group scales from bytes")
+
+
+_CHECKS = [("fp8_to_mxfp8", _check_fp8_to_mxfp8), ("fp8_block", _check_fp8_block), ("fp8_blockwise_cast", _check_fp8_blockwise), ("fp8_dequant", _check_fp8_dequant),
            ("mxfp8", _check_mxfp8), ("mxfp4", _check_mxfp4), ("int4", _check_int4), ("nvfp4", _check_nvfp4), ("fake_quant", _check_fake_quant),
            ("fp8_act_quant", _check_act_quant)]
 _PARAMS = [pytest.param(fam, fn, case, id=f"{fam}-{case}") for fam, fn in _CHECKS for case in _cases(fam)]
