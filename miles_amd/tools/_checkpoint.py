@@ -37,9 +37,14 @@ def load_tensor(src: str, filename: str, key: str, device: str) -> torch.Tensor:
         return f.get_tensor(key)
 
 
-def save_shard(tensors: dict[str, torch.Tensor], dst: str, filename: str) -> None:
+_PT_FORMAT = {"format": "pt"}
+
+
+def save_shard(tensors: dict[str, torch.Tensor], dst: str, filename: str, metadata: dict | None = _PT_FORMAT) -> None:
+    """One safetensors file; the converters tag theirs `format: pt` as the reference's tools do, the snapshot export
+    writes none (`metadata=None`)."""
     safetensors.torch.save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(dst, filename),
-                                metadata={"format": "pt"})
+                                metadata=metadata)
 
 
 def read_config(src: str) -> dict | None:

@@ -3,8 +3,9 @@
 `HfWeightIteratorBase.iter_hf_weights` keeps the template of the reference's
 miles/backends/training_utils/weight_update/hf_weight_iterator/__init__.py:96-122
 (units -> atomic groups -> buckets).  `HfWeightIteratorDirect` is the single-GPU form of the reference's
-miles/backends/megatron_utils/update_weight/hf_weight_iterator_direct.py:77-146: parameters are taken in
-gather batches of at most `update_weight_buffer_size` bytes (`_pack_param_infos_by_size`, :246-259), each
+miles/backends/megatron_utils/update_weight/hf_weight_iterator_direct.py:77-146: parameters are taken in name
+order, the non-expert ones before the routed experts (:39-43, :85-108), in gather batches of at most
+`update_weight_buffer_size` bytes (`_pack_param_infos_by_size`, :246-259), each
 parameter goes through `convert_to_hf` (name map + quantizer), and -- unlike the reference, which launches a
 chain of kernels per tensor -- all quantizer calls of a batch are recorded and submitted as ONE
 `mq_run_jobs` call (grouped kernel launches).  The TP / EP / PP collectives of the reference are outside
@@ -14,6 +15,7 @@ this path: the iterator expects full (already gathered) parameters.
 from __future__ import annotations
 
 import dataclasses
+import re
 from abc import ABC, abstractmethod
 from argparse import Namespace
 from collections.abc import Iterator, Mapping, Sequence
@@ -73,6 +75,35 @@ def _pack_param_infos_by_size(args: Namespace, param_infos: Sequence[ParamInfo],
     return [b for b in batches if b]
 
 
+def is_routed_expert_param(name: str) -> bool:
+    """A parameter of the routed experts: under `.experts.`, but not an inner list of the shared experts
+    (reference: hf_weight_iterator_direct.py `is_routed_expert_param`)."""
+    return ".experts." in name and ".shared_experts." not in name
+
+
+def _split_param_infos(infos: Sequence[ParamInfo]) -> tuple[list[ParamInfo], list[ParamInfo]]:
+    """(non-expert infos, routed-expert infos), each sorted by parameter name: the order in which the reference
+    streams a model (`_get_megatron_local_param_infos`, hf_weight_iterator_direct.py:293-344 -- every non-expert
+    batch is sent before the first expert batch, :85-108)."""
+    ordered = sorted(infos, key=lambda info: info.name)
+    return ([i for i in ordered if not is_routed_expert_param(i.name)],
+            [i for i in ordered if is_routed_expert_param(i.name)])
+
+
+_GROUPED_EXPERT_WEIGHT = re.compile(r"\.weight(\d+)$")
+
+
+def _expert_share_of_this_rank(expert_infos: Sequence[ParamInfo]) -> list[ParamInfo]:
+    """The routed experts this rank converts.  The reference deals contiguous ranges of local experts to the expert
+    data-parallel replicas (`_partition_expert_infos`, :262-278) by the number at the end of a grouped weight's name;
+    one GPU is the only replica and takes them all, in name order, but a routed-expert parameter that does not name
+    its expert is refused as there."""
+    for info in expert_infos:
+        if _GROUPED_EXPERT_WEIGHT.search(info.name) is None:
+            raise ValueError(f"Cannot identify the routed expert in {info.name!r}")
+    return list(expert_infos)
+
+
 class HfWeightIteratorDirect(HfWeightIteratorBase):
     """Megatron-named full parameters -> quantized HF units, one batched kernel submission per gather batch."""
 
@@ -86,7 +117,13 @@ class HfWeightIteratorDirect(HfWeightIteratorBase):
 
     def _iter_hf_param_units(self, weights, *, materialize):
         infos = [ParamInfo(name, t.dtype, t.shape, t.numel() * t.element_size()) for name, t in weights.items()]
-        for batch in _pack_param_infos_by_size(self.args, infos):
+        non_expert_infos, expert_infos = _split_param_infos(infos)
+        # every non-expert batch first, then the expert batches, each in name order: what the reference hands its
+        # transfer protocol (the bucket composition of a mixture-of-experts sync follows from it)
+        batches = _pack_param_infos_by_size(self.args, non_expert_infos)
+        if expert_infos:
+            batches += _pack_param_infos_by_size(self.args, _expert_share_of_this_rank(expert_infos))
+        for batch in batches:
             if not materialize:
                 continue
             yield from self._convert_batch([(info.name, weights[info.name]) for info in batch])

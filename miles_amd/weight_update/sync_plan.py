@@ -31,6 +31,9 @@ from miles_amd.weight_update.hf_weight_iterator import HfWeightIteratorBase
 from miles_amd.weight_update.plan_memory import Placement
 
 
+_shape_of = operator.attrgetter("shape")
+
+
 def weights_signature(weights: Mapping[str, torch.Tensor]) -> tuple:
     """Identity of a parameter set: addresses, shapes and dtypes in order."""
     return tuple((name, t.data_ptr(), tuple(t.shape), t.dtype) for name, t in weights.items())
@@ -51,14 +54,15 @@ class SyncPlan:
         self._names: list[str] = []
         self._tensors: list[torch.Tensor] = []
         self._addresses: list[int] = []
-        self._numels: list[int] = []
+        self._shapes: list[torch.Size] = []
+        self.refusal: tuple[str, ...] = ()           # why the recording is not replayable (empty when it is)
 
     def remember(self, weights: Mapping[str, torch.Tensor]) -> None:
         """Keep the parameter objects themselves, for the quick form of `matches`."""
         self._names = list(weights)
         self._tensors = list(weights.values())
         self._addresses = [t.data_ptr() for t in self._tensors]
-        self._numels = [t.numel() for t in self._tensors]
+        self._shapes = [t.shape for t in self._tensors]
 
     @classmethod
     def record(cls, iterator: HfWeightIteratorBase, weights: Mapping[str, torch.Tensor], *,
@@ -82,27 +86,30 @@ class SyncPlan:
         # a replay reproduces the sync only if no kernel bypassed the job list, every job input is live parameter
         # storage, a declared constant or made by a job, and every handed-out tensor is one of those too (a tensor
         # that some torch op materialised would go stale)
-        replayable = (batch.direct_calls == 0 and placement.handed_out_ok and placement.packable
-                      and placement.inputs_alias)
-        plan = cls(batch, buckets, marks, weights_signature(weights), replayable, ring, arena_bytes)
+        refusal = tuple(reason for ok, reason in (
+            (batch.direct_calls == 0, f"{batch.direct_calls} kernel launches bypassed the job list"),
+            (placement.handed_out_ok, "a handed-out tensor is neither written by a job, nor parameter storage, nor a declared constant"),
+            (placement.packable, "a bucket cannot be laid out as one payload"),
+            (placement.inputs_alias, "a kernel input does not alias live parameter storage")) if not ok)
+        plan = cls(batch, buckets, marks, weights_signature(weights), not refusal, ring, arena_bytes)
+        plan.refusal = refusal
         plan.packable = placement.packable
         plan.remember(weights)
         return plan
 
     def matches(self, weights: Mapping[str, torch.Tensor]) -> bool:
         """True when `weights` is the parameter set the plan was recorded on.  Between RL steps the mapping holds
-        the very same tensor objects, so the usual answer costs one identity pass and one address per tensor (0.5 ms
-        for 12 288 expert tensors, against 5 ms for the full signature, which builds a shape tuple per tensor).
-        The quick form takes the shapes of unchanged objects at unchanged addresses with unchanged element counts as
-        unchanged: an in-place `set_` that keeps address and size but changes the shape would go unnoticed.  Anything else (other objects, other
-        names, another count) is decided by the full signature."""
+        the very same tensor objects, so the usual answer costs one identity pass, one address and one shape per tensor
+        (about 1 ms for 12 288 expert tensors, against 5 ms for the full signature, which also builds a tuple per
+        tensor); a tensor object keeps its dtype for life, so objects, addresses and shapes cover the signature.
+        Anything else (other objects, other names, another count) is decided by the full signature."""
         if not self.replayable:
             return False
         if len(weights) == len(self._tensors):
             tensors = list(weights.values())
             if all(map(operator.is_, tensors, self._tensors)) and list(weights) == self._names:
                 return (list(map(torch.Tensor.data_ptr, tensors)) == self._addresses
-                        and list(map(torch.Tensor.numel, tensors)) == self._numels)
+                        and list(map(_shape_of, tensors)) == self._shapes)
         return weights_signature(weights) == self.signature
 
     # a trailing launch smaller than this many elements is topped up with the next bucket's jobs

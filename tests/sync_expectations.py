@@ -23,11 +23,20 @@ def _bits(t: torch.Tensor) -> torch.Tensor:
     return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
 
 
+def reference_stream_order(names):
+    """Parameter names in the order the reference streams them (hf_weight_iterator_direct.py:39-43,85-108,339-341):
+    sorted by name, every parameter outside the routed experts before the first routed-expert parameter."""
+    routed = lambda n: ".experts." in n and ".shared_experts." not in n
+    ordered = sorted(names)
+    return [n for n in ordered if not routed(n)] + [n for n in ordered if routed(n)]
+
+
 def expected_dense_fp8(oracle, args, cpu_params, quantizer: str = "fp8_blockwise_cast"):
     """HF stream of a dense Qwen-style model synced to FP8 128x128: every *_proj.weight becomes codes + scales."""
     quantize = {"fp8_blockwise_cast": oracle.fp8_blockwise_cast, "block_fp8": lambda t: oracle.block_fp8(t, (128, 128))}[quantizer]
     out = []
-    for name, param in cpu_params.items():
+    for name in reference_stream_order(cpu_params):
+        param = cpu_params[name]
         if "word_embeddings" in name or "output_layer" in name:
             param = param[: args.vocab_size]
         for hf, t in name_maps.convert_qwen2_to_hf(args, name, param):
@@ -42,7 +51,8 @@ def expected_dense_fp8(oracle, args, cpu_params, quantizer: str = "fp8_blockwise
 def expected_moe(oracle, fmt: str, args, cpu_params, basenames=None):
     """HF stream of routed experts synced to `fmt` ("mxfp8", "int4_g128", "nvfp4")."""
     out = []
-    for name, param in cpu_params.items():
+    for name in reference_stream_order(cpu_params):
+        param = cpu_params[name]
         if fmt == "mxfp8":
             for hf, t in name_maps.convert_qwen3moe_to_hf(args, name, param):
                 q, s = oracle.mxfp8_quantize(t.contiguous())

@@ -11,6 +11,7 @@ from miles_amd import _lib
 from miles_amd import workloads as W
 from miles_amd.megatron_to_hf import name_maps
 from miles_amd.weight_update.updater import WeightUpdater
+from tests.sync_expectations import reference_stream_order
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -31,6 +32,11 @@ def _same(got, want, what):
     g, w = _bits(got), _bits(want)
     assert g.shape == w.shape, f"{what}: shape {tuple(g.shape)} vs {tuple(w.shape)}"
     assert torch.equal(g, w), f"{what}: {(g != w).sum().item()} of {g.numel()} differ"
+
+
+def _ordered(params):
+    """(name, parameter) pairs in the order the reference streams a model: by name, routed experts last."""
+    return [(n, params[n]) for n in reference_stream_order(params)]
 
 
 def _dense_model(seed):
@@ -61,7 +67,7 @@ def _dense_model(seed):
 def _expected_fp8(oracle, cpu_params):
     """(name, tensor) list the sync must produce: HF order of the name map, weights cast per tile."""
     out = []
-    for name, param in cpu_params.items():
+    for name, param in _ordered(cpu_params):
         if "word_embeddings" in name or "output_layer" in name:
             param = param[:1000]
         for hf, t in name_maps.convert_qwen2_to_hf(ARGS, name, param):
@@ -107,7 +113,14 @@ def test_dense_fp8_sync_matches_oracle_and_replays(oracle, use_plan):
     assert len(buckets) > 1
     for b in buckets[:-1]:      # a closed bucket stays under the limit unless it is a single oversized unit
         assert sum(t.nbytes for _, t in b) < ARGS.update_weight_buffer_size or len(b) <= 3
-    assert {"update_weights_implementation", "finalize_and_resume_engines"} <= set(upd.pop_metrics())
+    metrics = upd.pop_metrics()
+    assert set(metrics) == {"update_weights_implementation"} and upd.pop_metrics() == {}     # no finalize hook, no such span
+    finalized = []
+    upd.finalize = lambda version: (torch.cuda.synchronize(), finalized.append(version))
+    _run(upd)
+    metrics = upd.pop_metrics()
+    assert finalized == [upd.weight_version] and metrics["finalize_and_resume_engines"] > 0 and metrics["update_weights_implementation"] > 0
+    upd.finalize = None
     q_proj = dict(flat)["model.layers.0.self_attn.q_proj.weight"]
     assert q_proj.dtype == F8 and q_proj.shape == (512, 256)
     # the weights change in place (an optimizer step); the next sync must see the new values
@@ -160,7 +173,7 @@ def _family_expected(oracle, family, cpu):
         g = t.view(2, 4, 128, *t.shape[1:])
         return g[:, :2].reshape(512, *t.shape[1:]), g[:, 2].reshape(256, *t.shape[1:]), g[:, 3].reshape(256, *t.shape[1:])
 
-    for name, t in cpu.items():
+    for name, t in _ordered(cpu):
         if "decoder.layers." not in name:
             hf = {"embedding.word_embeddings.weight": "model.embed_tokens.weight", "output_layer.weight": "lm_head.weight",
                   "decoder.final_layernorm.weight": "model.norm.weight"}[name[len("module.module."):]]
@@ -250,7 +263,7 @@ def test_moe_mxfp8_sync(oracle, dtype):
     for round_ in range(2):
         flat = [nt for b in _run(upd) for nt in b]
         want = []
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             for hf, t in name_maps.convert_qwen3moe_to_hf(ARGS, name, param):
                 if "experts" in hf:
                     q, s = oracle.mxfp8_quantize(t.contiguous())
@@ -282,7 +295,7 @@ def test_moe_nvfp4_sync_pairs_share_amax(oracle):
             dev[k].copy_(cpu[k])
         flat = [nt for b in _run(upd) for nt in b]
         want = []
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             hf = name_maps.convert_deepseekv3_to_hf(ARGS, name, param)
             if "linear_fc1" in name:
                 (gn, g), (un, u) = hf
@@ -311,7 +324,7 @@ def test_moe_int4_compressed_tensors_sync(oracle):
                         packed_weight_basenames=basenames)
     flat = [nt for b in _run(upd) for nt in b]
     want = []
-    for name, param in cpu.items():
+    for name, param in _ordered(cpu):
         for hf, t in name_maps.convert_deepseekv3_to_hf(ARGS, name, param):
             if hf.removesuffix(".weight") in basenames:
                 packed, scale, _ = oracle.pack_layer(t.contiguous(), 128)
@@ -337,7 +350,7 @@ def test_moe_int4_asymmetric_sync_is_planned_and_replayed(oracle, packed):
     for round_ in range(3):
         flat = [nt for b in _run(upd) for nt in b]
         want = []
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             for hf, t in name_maps.convert_deepseekv3_to_hf(ARGS, name, param):
                 if hf.removesuffix(".weight") in basenames:
                     p_, s_, z_ = oracle.pack_layer(t.contiguous(), 128, sym=False)
@@ -557,7 +570,7 @@ def test_packed_buckets_int4_moe_two_syncs(oracle):
         upd.update_weights()
         torch.cuda.synchronize()
         want = []
-        for name, param in src.items():
+        for name, param in _ordered(src):
             for hf, t in name_maps.convert_deepseekv3_to_hf(ARGS, name, param):
                 if hf.removesuffix(".weight") in basenames:
                     p, s, _ = oracle.pack_layer(t.contiguous(), 128)
@@ -580,7 +593,7 @@ def test_dense_fp8_sync_with_power_of_two_scales(oracle, monkeypatch):
     upd = WeightUpdater(ARGS, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None)
     for _ in range(2):      # recorded plan, then its replay
         flat = dict(nt for b in _run(upd) for nt in b)
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             for hf, t in name_maps.convert_qwen2_to_hf(ARGS, name, param):
                 if hf.endswith("_proj.weight"):
                     q, s = oracle.per_block_cast_to_fp8(t.contiguous())
@@ -602,7 +615,7 @@ def test_dense_fp8_sync_with_one_scale_per_tensor(oracle, packed):
     for round_ in range(4):
         flat = [nt for b in _run(upd) for nt in b]
         want = []
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             if "word_embeddings" in name or "output_layer" in name:
                 param = param[:1000]
             for hf, t in name_maps.convert_qwen2_to_hf(ARGS, name, param):
@@ -640,7 +653,7 @@ def test_dense_fp8_sync_with_packed_ue8m0_scales(oracle, packed):
                         packed_buckets=packed)
     for _ in range(3):      # recorded plan, then two replays
         flat = dict(nt for b in _run(upd) for nt in b)
-        for name, param in cpu.items():
+        for name, param in _ordered(cpu):
             for hf, t in name_maps.convert_qwen2_to_hf(args, name, param):
                 if hf.endswith("_proj.weight"):
                     q, s = oracle.per_block_cast_to_fp8(t.contiguous())
@@ -701,7 +714,7 @@ def test_random_dense_models_sync_and_replay(oracle, seed, packed):
 
     def expected(params):
         out = []
-        for name, param in params.items():
+        for name, param in _ordered(params):
             for hf, t in name_maps.convert_qwen2_to_hf(args, name, param):
                 if hf.endswith("_proj.weight"):
                     q, s = oracle.fp8_blockwise_cast(t.contiguous())
@@ -757,7 +770,7 @@ def _random_moe_case(seed):
 
 def _moe_expected(oracle, fmt, args, params, basenames):
     want = []
-    for name, param in params.items():
+    for name, param in _ordered(params):
         if fmt == "mxfp8":
             for hf, t in name_maps.convert_qwen3moe_to_hf(args, name, param):
                 if "experts" in hf:
@@ -981,6 +994,47 @@ def test_plan_outputs_rotate_through_two_arenas(oracle):
     for (n, g), (_, w) in zip([nt for b in held for nt in b], _expected_fp8(oracle, cpu)):
         _same(g, w, f"{n} (an arena per bucket)")
     assert keep._plan.ring == len(held)
+
+
+@pytest.mark.parametrize("hand_back", ["host_wait", "stream_wait"])
+def test_a_consumer_on_another_stream_reads_the_right_bytes(oracle, hand_back):
+    """What a transfer protocol on its own stream (a broadcast, say) must do with a bucket of a two-arena plan: make its
+    stream wait for the launch stream before it reads, and before `send_bucket` returns either wait on the host for its
+    stream or make the launch stream wait for it -- bucket k + 2 is written into the memory of bucket k.  The consumer
+    here is slow on purpose (it sleeps on its stream before every copy), over six or more buckets and two syncs."""
+    cpu = _dense_model(70)
+    dev = {k: v.to(DEV) for k, v in cpu.items()}
+    args = Namespace(**{**vars(ARGS), "update_weight_buffer_size": 1 << 18})
+    upd = WeightUpdater(args, weights_getter=lambda: dev, model_name="qwen3", quantization_config=FP8_CFG, send_bucket=None)
+    side = torch.cuda.Stream(device=DEV)
+    copies = []
+
+    def consume(bucket):
+        launch_stream = torch.cuda.current_stream()
+        side.wait_stream(launch_stream)                  # the bucket's kernels are queued on the launch stream
+        with torch.cuda.stream(side):
+            torch.cuda._sleep(2_000_000)                 # about a millisecond: the reads run well after this call returns
+            copies.append([(n, t.clone()) for n, t in bucket])
+        if hand_back == "host_wait":
+            side.synchronize()
+        else:
+            launch_stream.wait_stream(side)              # nothing queued later on the launch stream overtakes the reads
+
+    for round_ in range(2):
+        copies.clear()
+        upd.send_bucket = consume
+        upd.update_weights()
+        torch.cuda.synchronize()
+        assert len(copies) >= 6
+        flat = [nt for b in copies for nt in b]
+        want = _expected_fp8(oracle, cpu)
+        assert [n for n, _ in flat] == [n for n, _ in want]
+        for (n, g), (_, w) in zip(flat, want):
+            _same(g, w, f"{n} (sync {round_}, {hand_back})")
+        cpu = _dense_model(71)
+        for k in dev:
+            dev[k].copy_(cpu[k])
+    assert upd._plan is not None and upd._plan.replayable and upd._plan.ring == 2
 
 
 def test_recording_a_sync_holds_no_more_than_a_few_buckets():

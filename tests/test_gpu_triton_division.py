@@ -1,0 +1,261 @@
+"""What Triton's fp32 `/` gives on this GPU for the two divisions of the sync path's FP8 quantizer.
+
+The reference's `_fp8_blockwise_cast_kernel` (miles/kernels/quant/fp8_blockwise.py:51-54) computes, per tile,
+`_absmax = maximum(max|x|, eps)`, `x_s = _absmax / fp8_max` and `s_inv = 1.0 / x_s` with Triton's `/` on fp32 scalars
+(`eps`, `fp8_max` are run-time arguments).  The oracle and the HIP kernel take both as IEEE divisions.  Triton does not
+promise a correctly rounded quotient, so this file measures it: a probe of its own (not the reference's kernel) runs the
+same three expressions on every tile maximum a bf16 or fp16 tensor can have and compares them with IEEE division.
+
+A second probe is a whole 128 x 128 tile quantizer written for this file from the same expressions (maximum floored at
+eps, the two divisions, clamp of the product, cast to e4m3): its bytes are compared with the HIP kernel's on finite data,
+on tiles holding infinities and NaN, and on one Qwen3-4B layer at full size.
+
+The counts are printed and written to gpurun_out/*.json when that folder exists.  Every test is skipped, with the reason,
+where Triton cannot compile for the GPU.
+"""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _tile_maxima():
+    """Every positive finite bf16 and fp16 value as fp32 (the tile maximum is exact in fp32), duplicates removed."""
+    bf = torch.arange(1, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    fp = torch.arange(1, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16).float()
+    return torch.unique(torch.cat([bf, fp])), bf.numel(), fp.numel()
+
+
+def _probe():
+    try:
+        import triton
+        import triton.language as tl
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton is not importable: {exc!r}")
+
+    @triton.jit
+    def elementwise(a_ptr, xs_ptr, sinv_ptr, n, eps, fp8_max, BLOCK: tl.constexpr):
+        offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+        mask = offs < n
+        a = tl.load(a_ptr + offs, mask=mask, other=1.0)
+        absmax = tl.maximum(a, eps)
+        x_s = absmax / fp8_max
+        s_inv = 1.0 / x_s
+        tl.store(xs_ptr + offs, x_s, mask=mask)
+        tl.store(sinv_ptr + offs, s_inv, mask=mask)
+
+    @triton.jit
+    def per_tile(a_ptr, xs_ptr, sinv_ptr, eps, fp8_max, BLOCK: tl.constexpr):
+        # the reference's shape of the computation: a reduction to a scalar, then scalar divisions
+        pid = tl.program_id(0)
+        x = tl.load(a_ptr + pid + tl.zeros([BLOCK], dtype=tl.int32))
+        absmax = tl.maximum(tl.max(tl.abs(x)), eps)
+        x_s = absmax / fp8_max
+        s_inv = 1.0 / x_s
+        tl.store(xs_ptr + pid, x_s)
+        tl.store(sinv_ptr + pid, s_inv)
+
+    return triton, elementwise, per_tile
+
+
+def _ulps(a, b):
+    return (a.view(torch.int32).to(torch.int64) - b.view(torch.int32).to(torch.int64)).abs()
+
+
+def test_triton_division_against_ieee(oracle):
+    triton, elementwise, per_tile = _probe()
+    amax, n_bf16, n_fp16 = _tile_maxima()
+    n = amax.numel()
+    eps, fp8_max = 1e-10, float(torch.finfo(torch.float8_e4m3fn).max)
+    a = amax.to(DEV)
+    results = {}
+    try:
+        xs, sinv = torch.empty_like(a), torch.empty_like(a)
+        elementwise[(triton.cdiv(n, 256),)](a, xs, sinv, n, eps, fp8_max, BLOCK=256)
+        torch.cuda.synchronize()
+        results["elementwise"] = (xs.cpu(), sinv.cpu())
+        xs2, sinv2 = torch.empty_like(a), torch.empty_like(a)
+        per_tile[(n,)](a, xs2, sinv2, eps, fp8_max, BLOCK=64)
+        torch.cuda.synchronize()
+        results["per_tile_scalar"] = (xs2.cpu(), sinv2.cpu())
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+
+    # IEEE: numpy's float32 division, and the oracle's own x_s for the same maxima (one 1 x 8 block per value)
+    floor = np.maximum(amax.numpy(), np.float32(eps))
+    want_xs = torch.from_numpy(floor / np.float32(fp8_max))
+    want_sinv = torch.from_numpy(np.float32(1.0) / want_xs.numpy())
+    sample = amax[:: max(n // 4096, 1)]
+    _y, oracle_xs = oracle.fp8_blockwise_cast(sample.reshape(-1, 1).repeat(1, 8).contiguous(), (1, 8))
+    sample_want = torch.from_numpy(np.maximum(sample.numpy(), np.float32(eps)) / np.float32(fp8_max))
+    assert torch.equal(oracle_xs.reshape(-1).view(torch.int32), sample_want.view(torch.int32)), "the oracle's x_s is not numpy's IEEE quotient"
+
+    report = {"tile_maxima": n, "bf16_patterns": n_bf16, "fp16_patterns": n_fp16, "triton": triton.__version__}
+    for form, (got_xs, got_sinv) in results.items():
+        d_xs, d_sinv = _ulps(got_xs, want_xs), _ulps(got_sinv, want_sinv)
+        # s_inv as Triton would have it from the IEEE x_s cannot be separated from its own x_s: also compare s_inv with
+        # the IEEE reciprocal of Triton's own x_s, which isolates the second division
+        own = torch.from_numpy(np.float32(1.0) / got_xs.numpy())
+        d_own = _ulps(got_sinv, own)
+        report[form] = {"x_s_differ": int((d_xs != 0).sum()), "x_s_max_ulp": int(d_xs.max()),
+                        "s_inv_differ": int((d_sinv != 0).sum()), "s_inv_max_ulp": int(d_sinv.max()),
+                        "s_inv_differ_from_ieee_reciprocal_of_own_x_s": int((d_own != 0).sum())}
+        # what a differing s_inv does to the codes: every bf16 x with |x| <= amax through clamp(x * s_inv) -> e4m3
+        bad = (d_sinv != 0).nonzero().reshape(-1)
+        changed = total = 0
+        for i in bad[:: max(bad.numel() // 64, 1)].tolist():
+            x = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+            x = x[x <= amax[i]]
+            ya = (x * got_sinv[i]).clamp(-fp8_max, fp8_max).to(torch.float8_e4m3fn).view(torch.uint8)
+            yb = (x * want_sinv[i]).clamp(-fp8_max, fp8_max).to(torch.float8_e4m3fn).view(torch.uint8)
+            changed += int((ya != yb).sum())
+            total += x.numel()
+        report[form]["codes_changed_of_sampled_inputs"] = [changed, total]
+    print("TRITON_DIVISION", json.dumps(report))
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "triton_division.json"), "w") as f:
+            json.dump(report, f, indent=1)
+    for form in results:
+        assert report[form]["x_s_max_ulp"] <= 1 and report[form]["s_inv_max_ulp"] <= 2, report
+
+
+def _tile_probe():
+    """A 128 x 128 tile quantizer written for this test from the reference's expressions (maximum of |x| floored at eps,
+    the two divisions, clamp of the product, cast to e4m3): what Triton makes of them on this GPU, end to end."""
+    try:
+        import triton
+        import triton.language as tl
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton is not importable: {exc!r}")
+
+    @triton.jit
+    def tile_quant(x_ptr, y_ptr, s_ptr, rows, cols, tiles_across, eps, lo, hi, B: tl.constexpr):
+        t = tl.program_id(0)
+        r = (t // tiles_across) * B + tl.arange(0, B)
+        c = (t % tiles_across) * B + tl.arange(0, B)
+        inside = (r < rows)[:, None] & (c < cols)[None, :]
+        at = r[:, None].to(tl.int64) * cols + c[None, :]
+        x = tl.load(x_ptr + at, mask=inside, other=0.0).to(tl.float32)
+        top = tl.maximum(tl.max(tl.abs(x)), eps)
+        scale = top / hi
+        inv = 1.0 / scale
+        y = tl.clamp(x * inv, lo, hi).to(y_ptr.dtype.element_ty)
+        tl.store(y_ptr + at, y, mask=inside)
+        tl.store(s_ptr + t, scale)
+
+    def run(x):
+        rows, cols = x.shape
+        tr, tc = -(-rows // 128), -(-cols // 128)
+        y = torch.empty((rows, cols), dtype=torch.float8_e4m3fn, device=x.device)
+        s = torch.empty((tr, tc), dtype=torch.float32, device=x.device)
+        hi = float(torch.finfo(torch.float8_e4m3fn).max)
+        tile_quant[(tr * tc,)](x, y, s, rows, cols, tc, 1e-10, -hi, hi, B=128, num_warps=8)
+        torch.cuda.synchronize()
+        return y, s
+
+    return run
+
+
+def _cases():
+    from miles_amd import workloads as W
+
+    gate = W.gaussian_outliers((384, 640), std=0.02, p_outlier=0.001, gain=20.0, seed=2001)
+    gate[128:256, 128:256] = 0                                   # an all-zero tile: the eps floor
+    yield "bf16 gaussian with outliers and a zero tile", gate
+    yield "bf16 ragged", W.gaussian_outliers((130, 264), std=0.02, p_outlier=0.001, gain=20.0, seed=5)
+    yield "fp16", W.gaussian_outliers((256, 384), std=0.02, p_outlier=0.001, gain=20.0, seed=6, dtype=torch.float16)
+    for kind in W.PATTERNS:
+        yield f"bf16 {kind}", W.reference_pattern(kind, (256, 128), spread=512.0, amplitude=16.0)
+    g = torch.Generator().manual_seed(7)
+    wide = (torch.randn((256, 256), generator=g) * torch.exp(torch.randn((256, 256), generator=g) * 8)).to(torch.bfloat16)
+    yield "bf16 sixty binades in one tile", wide
+    tiny = (torch.randn((128, 256), generator=g) * 1e-12).to(torch.bfloat16)
+    yield "bf16 below the eps floor", tiny
+
+
+def test_triton_tile_quantizer_gives_the_hip_kernels_bytes(oracle):
+    """The whole sync-path quantizer, as Triton compiles its expressions for this GPU, against the HIP kernel and the
+    oracle on finite inputs: scales and codes byte for byte."""
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    run = _tile_probe()
+    report = {}
+    for what, x in _cases():
+        try:
+            ty, ts = run(x.to(DEV))
+        except Exception as exc:          # pragma: no cover - depends on the image
+            pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+        hy, hs = fp8_blockwise_cast(x.to(DEV))
+        oy, os_ = oracle.fp8_blockwise_cast(x)
+        ty, ts = ty.cpu().view(torch.uint8), ts.cpu().view(torch.int32)
+        codes = int((ty != hy.cpu().view(torch.uint8)).sum())
+        scales = int((ts != hs.cpu().view(torch.int32)).sum())
+        report[what] = {"codes_differ": codes, "scales_differ": scales, "elements": x.numel()}
+        assert torch.equal(hy.cpu().view(torch.uint8), oy.view(torch.uint8)) and torch.equal(hs.cpu().view(torch.int32), os_.view(torch.int32)), what
+    print("TRITON_TILE_QUANTIZER", json.dumps(report))
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "triton_tile_quantizer.json"), "w") as f:
+            json.dump(report, f, indent=1)
+    assert all(v["codes_differ"] == 0 and v["scales_differ"] == 0 for v in report.values()), report
+
+
+def test_triton_tile_quantizer_on_non_finite_inputs():
+    """Where the HIP kernel's handling of infinities and NaN rests on a reading of Triton's max / maximum / clamp (the
+    operand that is not NaN is returned): the same probe on tiles that hold them.  The two e4m3 NaN codes count as one."""
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    run = _tile_probe()
+    g = torch.Generator().manual_seed(9)
+    base = (torch.randn((128, 384), generator=g) * 0.02).to(torch.bfloat16)
+    base[3, 5] = float("nan")                 # tile 0: a NaN among ordinary values
+    base[7, 128 + 9] = float("inf")           # tile 1: an infinity
+    base[9, 256 + 1], base[11, 256 + 2] = float("-inf"), float("nan")   # tile 2: both
+    try:
+        ty, ts = run(base.to(DEV))
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+    hy, hs = fp8_blockwise_cast(base.to(DEV))
+    ty, hy = ty.cpu().view(torch.uint8), hy.cpu().view(torch.uint8)
+    fold = lambda c: torch.where((c & 0x7F) == 0x7F, torch.full_like(c, 0x7F), c)
+    report = {}
+    for j, what in enumerate(("nan_in_tile", "inf_in_tile", "inf_and_nan_in_tile")):
+        cols = slice(128 * j, 128 * (j + 1))
+        report[what] = {"codes_differ": int((fold(ty[:, cols]) != fold(hy[:, cols])).sum()),
+                        "scale_triton": ts[0, j].item(), "scale_hip": hs[0, j].item()}
+    print("TRITON_TILE_NONFINITE", json.dumps(report))
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "triton_tile_nonfinite.json"), "w") as f:
+            json.dump(report, f, indent=1)
+    for what, r in report.items():
+        assert r["codes_differ"] == 0 and (r["scale_triton"] == r["scale_hip"]), (what, r)
+
+
+def test_triton_tile_quantizer_on_one_qwen3_4b_layer():
+    """The seven quantized tensors of one Qwen3-4B layer at full size (q, k, v, o, gate, up, down of the headline
+    workload's generator): Triton's bytes against the HIP kernel's."""
+    from miles_amd import workloads as W
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    run = _tile_probe()
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(2001)
+    shapes = [(4096, 2560), (1024, 2560), (1024, 2560), (2560, 4096), (9728, 2560), (9728, 2560), (2560, 9728)]
+    for shape in shapes:
+        x = W.device_gaussian_outliers(shape, gen, std=0.02, p_outlier=0.001, gain=20.0)
+        try:
+            ty, ts = run(x)
+        except Exception as exc:          # pragma: no cover - depends on the image
+            pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+        hy, hs = fp8_blockwise_cast(x)
+        assert torch.equal(ts.view(torch.int32), hs.view(torch.int32)), f"{shape}: scales"
+        assert torch.equal(ty.view(torch.uint8), hy.view(torch.uint8)), f"{shape}: codes"

@@ -98,6 +98,42 @@ class TestPacking:
         assert [[i.name for i in b] for b in _pack_param_infos_by_size(args, infos, size_multiplier=2)] == \
             [["layer.a"], ["layer.b"], ["layer.c"]]
 
+    def test_non_expert_parameters_stream_before_the_routed_experts_in_name_order(self):
+        """The reference sorts the parameter infos by name and sends every non-expert gather batch before the first
+        expert batch (hf_weight_iterator_direct.py:39-43, 85-108, 339-341); shared experts are not routed experts."""
+        from miles_amd.weight_update.hf_weight_iterator import (HfWeightIteratorDirect, _expert_share_of_this_rank,
+                                                                _split_param_infos, is_routed_expert_param)
+
+        L = "module.module.decoder.layers."
+        names = [L + "1.mlp.experts.linear_fc2.weight0", L + "0.mlp.experts.linear_fc1.weight10", L + "1.self_attention.linear_proj.weight",
+                 L + "0.mlp.experts.linear_fc1.weight2", L + "0.mlp.shared_experts.experts.0.linear_fc1.weight", L + "0.mlp.router.weight",
+                 "module.module.embedding.word_embeddings.weight", L + "10.mlp.router.weight", L + "2.mlp.router.weight"]
+        infos = [ParamInfo(n, torch.bfloat16, torch.Size([2]), 4) for n in names]
+        non_expert, expert = _split_param_infos(infos)
+        assert [i.name for i in non_expert] == [
+            L + "0.mlp.router.weight", L + "0.mlp.shared_experts.experts.0.linear_fc1.weight", L + "1.self_attention.linear_proj.weight",
+            L + "10.mlp.router.weight", L + "2.mlp.router.weight", "module.module.embedding.word_embeddings.weight"]
+        assert [i.name for i in expert] == [L + "0.mlp.experts.linear_fc1.weight10", L + "0.mlp.experts.linear_fc1.weight2",
+                                            L + "1.mlp.experts.linear_fc2.weight0"]
+        assert is_routed_expert_param(L + "3.mlp.experts.linear_fc1.weight7") and not is_routed_expert_param(names[4])
+        assert _expert_share_of_this_rank(expert) == expert
+        with pytest.raises(ValueError, match="Cannot identify the routed expert"):
+            _expert_share_of_this_rank([ParamInfo(L + "0.mlp.experts.linear_fc1.bias", torch.bfloat16, torch.Size([2]), 4)])
+
+        # the iterator walks them in that order whatever the order of the mapping, in batches of the buffer size
+        seen = []
+
+        class Spy(HfWeightIteratorDirect):
+            def _convert_batch(self, named_params):
+                seen.append([n for n, _ in named_params])
+                return []
+
+        it = Spy(Namespace(update_weight_buffer_size=8), model_name="qwen3moe", quantization_config=None)
+        assert list(it._iter_hf_param_units({n: torch.zeros(2, dtype=torch.bfloat16) for n in names}, materialize=True)) == []
+        want = [i.name for i in non_expert] + [i.name for i in expert]
+        assert [n for batch in seen for n in batch] == want
+        assert [len(b) for b in seen] == [2, 2, 2, 2, 1]        # six non-expert parameters, then three experts: no mixed batch
+
 
 # ---------------------------------------------------------------------------------------------------------
 QWEN_ARGS = Namespace(hidden_size=64, num_attention_heads=4, num_query_groups=2, kv_channels=16, vocab_size=100,
@@ -380,6 +416,11 @@ def test_sync_plan_matches_quick_and_full_forms():
     plan.remember(weights)
     assert plan.matches(weights)
     weights["p3"].resize_(2, 8)                                           # same object, same address, fewer elements
+    assert not plan.matches(weights)
+    plan.remember(weights)
+    plan.signature = weights_signature(weights)
+    assert plan.matches(weights)
+    weights["p4"].set_(weights["p4"].untyped_storage(), 0, (8, 4))        # same object, address and size, another shape
     assert not plan.matches(weights)
     plan.replayable = False
     plan.remember(weights)
