@@ -583,13 +583,13 @@ def stream_ceilings():
         res[name] = {"GBps": round(nbytes / ms / 1e6, 1), "ms": round(ms, 4)}
     del q
     # the library's probes: kernels that only move bytes, in the access shapes of the quantizers (2 GiB on the larger side)
-    from miles_amd import _lib
-    lib, stream, big = _lib.load(), _lib.stream_ptr(x.device), 1 << 31
-    FLAT_2_1, FLAT_1_2, LOOP_2_1, TILE_2_1, TILE_READ, TILE_WRITE = range(6)
+    from miles_amd import _lib, _probes
+    from miles_amd._probes import FLAT_1_2, FLAT_2_1, LOOP_2_1, TILE_2_1, TILE_READ, TILE_WRITE
+    lib, stream, big = _probes.load(), _lib.stream_ptr(x.device), 1 << 31
 
     def probe(name, shape, param, moved):
         def fn():
-            _lib.check(lib.mq_stream_probe(shape, x.data_ptr(), y.data_ptr(), big, param, stream))
+            _probes.check(lib.mqp_stream_probe(shape, x.data_ptr(), y.data_ptr(), big, param, stream))
         fn()
         torch.cuda.synchronize()
         ms = min(_event_ms(fn, 10) for _ in range(3))
@@ -613,7 +613,10 @@ def stream_ceilings():
 
 def tile_launch_lengths():
     """The FP8 tile kernel on every 2-D weight of Qwen3-4B as one job list, with the driver's cut of long runs of tile
-    jobs set to different lengths (MQ_TILE_LAUNCH_TILES; 0: no cut, up to 64 tensors per launch)."""
+    jobs set to different lengths (mq_tune_tile_launch_tiles; 0: no cut, up to 64 tensors per launch)."""
+    import ctypes
+
+    from miles_amd import _lib
     from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
 
     gen = torch.Generator(device=DEV)
@@ -623,16 +626,18 @@ def tile_launch_lengths():
     elems = sum(t.numel() for t in targets)
     batch, outs = _record(lambda: [fp8_blockwise_cast(t) for t in targets])
     res = {}
+    lib, compiled_in = _lib.load(), ctypes.c_int64(0)
+    _lib.check(lib.mq_tune_tile_launch_tiles(0, ctypes.byref(compiled_in)))
     try:
         for cap in (0, 98304, 49152, 36864, 24576, 16384, 8192, 4096):
-            os.environ["MQ_TILE_LAUNCH_TILES"] = str(cap)
+            _lib.check(lib.mq_tune_tile_launch_tiles(cap, None))
             for _ in range(3):
                 batch.run()
             ms = _best_ms(batch.run)
             res[f"qwen3_4b_fp8_cast_launches_of_{cap}_tiles"] = {"GBps": round(elems * BYTES_PER_ELEM["fp8_block"] / ms / 1e6, 1),
                                                                  "ms": round(ms, 4)}
     finally:
-        del os.environ["MQ_TILE_LAUNCH_TILES"]
+        _lib.check(lib.mq_tune_tile_launch_tiles(compiled_in.value, None))
     return res
 
 
@@ -658,7 +663,7 @@ def main():
         sys.exit("bench.py measures one GPU: this path has no cross-GPU part (run with --gpus 1)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs the MI355X: no GPU visible")
-    from miles_amd import _lib
+    from miles_amd import _lib, _probes
     from miles_amd.weight_update.updater import WeightUpdater
 
     _lib.load()   # fails loudly if the HIP library is not built
@@ -677,10 +682,10 @@ def main():
         src, dst = torch.empty(n, dtype=torch.uint8, device=DEV), torch.empty(n, dtype=torch.uint8, device=DEV)
         src.fill_(1)
         for _ in range(3):
-            _lib.check(_lib.load().mq_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
+            _probes.check(_probes.load().mqp_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
         del src, dst
         res = per_quantizer(gen)
-        print(json.dumps({"pmc_quantizers": "3 x mq_copy_bytes(1 GiB), then each workload twice",
+        print(json.dumps({"pmc_quantizers": "3 x mqp_copy_bytes(1 GiB), then each workload twice",
                           "elements": {k: v["elements"] for k, v in res.items()}}))
         return
     args, weights, elems = qwen3_4b_megatron_weights(gen)
@@ -703,11 +708,11 @@ def main():
         src, dst = torch.empty(n, dtype=torch.uint8, device=DEV), torch.empty(n, dtype=torch.uint8, device=DEV)
         src.fill_(1)
         for _ in range(3):
-            _lib.check(_lib.load().mq_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
+            _probes.check(_probes.load().mqp_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _lib.stream_ptr(torch.device(DEV))))
         for _ in range(2):
             updater.update_weights()
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_workload": "3 x mq_copy_bytes(1 GiB), 3 x Qwen3-4B FP8 sync", "quantized_elements": elems}))
+        print(json.dumps({"pmc_workload": "3 x mqp_copy_bytes(1 GiB), 3 x Qwen3-4B FP8 sync", "quantized_elements": elems}))
         return
     # bring the GPU out of its idle power state first: the first ~20 syncs after start-up run about 5 % slower than
     # the steady state however many warm-up steps are requested (untimed, like the warm-up steps that follow)

@@ -307,10 +307,14 @@ typedef struct mq_job {
 } mq_job;
 /* Consecutive jobs of one kind (and, for the flat kernels, of similar size) are fused into launches of up to
  * MQ_MAX_GROUP tensors, counted from the first job of the call; a run of FP8 tile jobs of more than 36 864 tiles is
- * cut into launches of equal size (the tile kernel streams faster in launches of moderate length; the environment
- * variable MQ_TILE_LAUNCH_TILES overrides the length, 0 switches the cutting off). */
+ * cut into launches of equal size (the tile kernel streams faster in launches of moderate length).
+ * mq_tune_tile_launch_tiles (no counterpart in the reference) sets that length for the process, 0 for no cutting, and
+ * stores the length it replaces in *previous (a host pointer, may be NULL); the environment variable
+ * MQ_TILE_LAUNCH_TILES, read once when the library first needs the length and ignored unless it holds a whole number,
+ * sets the starting value. */
 #define MQ_MAX_GROUP 64
 int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream);
+int mq_tune_tile_launch_tiles(int64_t tiles, int64_t* previous);
 
 /* mq_run_jobs with the per-tensor descriptors of its launches kept in device memory (no counterpart in the reference; for
  * callers that submit one job list again and again, as a replayed weight sync does).  The kernel arguments of a launch
@@ -338,37 +342,6 @@ int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, 
  * pass over every such tensor -- the caller submits the list without the flag until they hold still again; the
  * records stay valid for either form.  device_table and device_moved may be NULL. */
 int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved, void* stream);
-
-/* Conversion self-test: compares the gfx950 convert instructions used by the kernels with the
- * software round-to-nearest-even forms over every fp32 bit pattern.  counts: 8 uint64 on the device
- * (cleared by the call): [0] e4m3 mismatches for |x| <= 448, [1] NaN inputs whose e4m3 code is not
- * 0x7F/0xFF, [2] e2m1 mismatches over all non-NaN inputs, [3] bf16 mismatches over all non-NaN
- * inputs, [4] e4m3 decode mismatches (256 codes), [5] NaN inputs whose e2m1 code is not +-6,
- * [6] inputs in (448, 464] whose e4m3 code is not +-448, [7] 1 if the packed e2m1 convert does not put
- * its first operand in the low nibble.  The kernels rely on [0], [2], [3], [4], [7] being zero. */
-int mq_selftest_convert(uint64_t* counts, void* stream);
-
-/* Reciprocal self-test (no counterpart in the reference).  The INT4 packers divide a group's elements by its scale
- * through y = 1/scale, taken from the hardware reciprocal and one Newton step instead of an IEEE division; the codes are
- * only right if y is the correctly rounded reciprocal.  count: one uint64 on the device (cleared by the call) = divisors
- * of both signs in [2^-91, 2^90], the range in which the kernels use y, for which it differs from 1.0f / scale.
- * The kernels rely on it being zero. */
-int mq_selftest_reciprocal(uint64_t* count, void* stream);
-
-/* Plain 16-byte-per-lane copy used to calibrate achievable HBM bandwidth and rocprof counters. */
-int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream);
-
-/* Streaming probes (no counterpart in the reference; measurement only): kernels that only move bytes in the access
- * shapes of the quantizers, to calibrate what a shape reaches on a GPU.  nbytes counts the larger side; dst must hold
- * nbytes as well (the probes write at most that).
- *   MQ_PROBE_FLAT_2_1   16 bytes read, 8 written per unit, one-shot workgroups; param = units per lane (1, 2, 4, 8)
- *   MQ_PROBE_FLAT_1_2   8 bytes read, 16 written per unit; param = units per lane
- *   MQ_PROBE_LOOP_2_1   the 2:1 mix as a grid of param workgroups striding over the buffer (param % 512 == 0)
- *   MQ_PROBE_TILE_2_1 / _READ / _WRITE   128 x 128 tiles of a row-major matrix of 2-byte elements, param = its row
- *                       length K; both sides, the reads alone, the writes alone */
-enum { MQ_PROBE_FLAT_2_1 = 0, MQ_PROBE_FLAT_1_2 = 1, MQ_PROBE_LOOP_2_1 = 2, MQ_PROBE_TILE_2_1 = 3, MQ_PROBE_TILE_READ = 4,
-       MQ_PROBE_TILE_WRITE = 5 };
-int mq_stream_probe(int shape, const void* src, void* dst, int64_t nbytes, int64_t param, void* stream);
 
 #ifdef __cplusplus
 }

@@ -48,13 +48,10 @@ SIGNATURES = {
     "mq_nvfp4_fold": [_vp, _i32, _i32, _vp],
     "mq_nvfp4_qdq": [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _vp],
     "mq_run_jobs": [_vp, _i64, _vp],
+    "mq_tune_tile_launch_tiles": [_i64, _vp],
     "mq_job_table_fill": [_vp, _i64, _vp],
     "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
     "mq_run_jobs_feedback": [_vp, _i64, _vp, _vp, _vp],
-    "mq_selftest_convert": [_vp, _vp],
-    "mq_selftest_reciprocal": [_vp, _vp],
-    "mq_copy_bytes": [_vp, _vp, _i64, _vp],
-    "mq_stream_probe": [_i32, _vp, _vp, _i64, _i64, _vp],
 }
 
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs

@@ -1,4 +1,5 @@
-"""Builds libmiles_quant.so (the C-ABI HIP library) for gfx950 with hipcc, in-tree.
+"""Builds libmiles_quant.so (the C-ABI HIP library) and libmq_probes.so (self-tests and streaming probes that only
+the GPU tests and bench.py load; not part of the product) for gfx950 with hipcc, in-tree.
 
     python -m miles_amd.build
 
@@ -16,9 +17,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmiles_quant.so")
+PROBES_LIB_PATH = os.path.join(LIB_DIR, "libmq_probes.so")
 
-SOURCES = ["mq_core.hip", "mq_fp8_block.hip", "mq_mxfp8.hip", "mq_rescale.hip", "mq_mxfp4.hip", "mq_fake_quant.hip", "mq_int4.hip", "mq_nvfp4.hip", "mq_fp8_tensor.hip", "mq_selftest.hip", "mq_probe.hip",
-           "mq_sync.hip"]
+SOURCES = ["mq_core.hip", "mq_fp8_block.hip", "mq_mxfp8.hip", "mq_rescale.hip", "mq_mxfp4.hip", "mq_fake_quant.hip", "mq_int4.hip", "mq_nvfp4.hip", "mq_fp8_tensor.hip", "mq_sync.hip"]
+PROBE_SOURCES = ["mq_selftest.hip", "mq_probe.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",
@@ -34,10 +36,8 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = ["hipcc", *FLAGS, "-o", LIB_PATH, *srcs]
+def _link(target: str, sources: list[str], verbose: bool) -> None:
+    cmd = ["hipcc", *FLAGS, "-o", target, *(os.path.join(CSRC, s) for s in sources)]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -46,6 +46,13 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed:\n{out}")
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose: bool = False) -> str:
+    """Compiles both libraries; returns the path of the product library."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _link(LIB_PATH, SOURCES, verbose)
+    _link(PROBES_LIB_PATH, PROBE_SOURCES, verbose)
     return LIB_PATH
 
 

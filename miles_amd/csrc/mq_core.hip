@@ -111,10 +111,3 @@ extern "C" int mq_fill_u32(void* p, uint32_t value, int64_t n, void* stream) {
                        value, n);
     return mq_check_launch("fill");
 }
-
-extern "C" int mq_copy_bytes(const void* src, void* dst, int64_t nbytes, void* stream) {
-    if (!src || !dst || nbytes < 0 || (nbytes % 16) || ((uintptr_t)src % 16) || ((uintptr_t)dst % 16))
-        return mq_fail(MQ_ERR_ARG, "copy needs 16-byte aligned pointers and size");
-    if (nbytes == 0) return MQ_OK;
-    return mq_copy_launch_run(src, dst, nbytes, (hipStream_t)stream);
-}

@@ -1,7 +1,8 @@
 // Exhaustive agreement check between the gfx950 convert instructions the kernels use and the
-// software round-to-nearest-even forms in mq_common.hpp, over every fp32 bit pattern.
-#include "mq_api_internal.hpp"
+// software round-to-nearest-even forms in mq_common.hpp, over every fp32 bit pattern.  Built into libmq_probes.so
+// (loaded by the GPU tests), not into the product library.
 #include "mq_common.hpp"
+#include "mq_probes_internal.hpp"
 
 namespace mq {
 
@@ -66,22 +67,31 @@ __global__ __launch_bounds__(256) void selftest_reciprocal_kernel(uint64_t* coun
     }
 }
 
-}  // namespace mq
-
-extern "C" int mq_selftest_reciprocal(uint64_t* count, void* stream) {
-    if (!count) return mq_fail(MQ_ERR_ARG, "null pointer");
-    hipStream_t st = (hipStream_t)stream;
-    int rc = mq_fill_u32(count, 0u, 2, stream);
-    if (rc) return rc;
-    hipLaunchKernelGGL(mq::selftest_reciprocal_kernel, dim3(4096), dim3(256), 0, st, count);
-    return mq_check_launch("selftest reciprocal");
+__global__ void selftest_clear_kernel(uint32_t* p, int n) {
+    if ((int)threadIdx.x < n) p[threadIdx.x] = 0u;
 }
 
-extern "C" int mq_selftest_convert(uint64_t* counts, void* stream) {
-    if (!counts) return mq_fail(MQ_ERR_ARG, "null pointer");
+}  // namespace mq
+
+static int clear_words(void* p, int n, void* stream) {
+    hipLaunchKernelGGL(mq::selftest_clear_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (uint32_t*)p, n);
+    return mqp_check_launch("selftest clear");
+}
+
+extern "C" int mqp_selftest_reciprocal(uint64_t* count, void* stream) {
+    if (!count) return mqp_fail(MQP_ERR_ARG, "null pointer");
     hipStream_t st = (hipStream_t)stream;
-    int rc = mq_fill_u32(counts, 0u, 16, stream);
+    int rc = clear_words(count, 2, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(mq::selftest_reciprocal_kernel, dim3(4096), dim3(256), 0, st, count);
+    return mqp_check_launch("selftest reciprocal");
+}
+
+extern "C" int mqp_selftest_convert(uint64_t* counts, void* stream) {
+    if (!counts) return mqp_fail(MQP_ERR_ARG, "null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    int rc = clear_words(counts, 16, stream);
     if (rc) return rc;
     hipLaunchKernelGGL(mq::selftest_kernel, dim3(4096), dim3(256), 0, st, counts);
-    return mq_check_launch("selftest");
+    return mqp_check_launch("selftest");
 }

@@ -4,6 +4,7 @@
 // issues a few launches per layer instead of several per tensor.  Jobs that do not qualify for a grouped
 // fast path (other dtypes, block sizes, strides, alignment) run through the single-tensor entry points, in
 // list order.
+#include <atomic>
 #include <vector>
 
 #include <stdlib.h>
@@ -208,11 +209,31 @@ static FlatJob flat_entry(const mq_job& jb) {
     return FlatJob{jb.in, jb.out, jb.scale, nullptr, jb.rows * jb.cols / 8, nullptr, 0, 0};
 }
 
+// The cut length of this process: the compiled-in value, unless the environment variable MQ_TILE_LAUNCH_TILES held a
+// whole number when the library first needed it (anything else in the variable is ignored), or until
+// mq_tune_tile_launch_tiles sets another.  0 switches the cutting off.
+static std::atomic<int64_t>& tile_launch_cap() {
+    static std::atomic<int64_t> cap{[] {
+        int64_t v = MQ_TILE_LAUNCH_TILES;
+        if (const char* env = getenv("MQ_TILE_LAUNCH_TILES")) {
+            char* end = nullptr;
+            const long long parsed = strtoll(env, &end, 10);
+            if (end != env && *end == '\0' && parsed >= 0) v = parsed;
+        }
+        return v;
+    }()};
+    return cap;
+}
+extern "C" int mq_tune_tile_launch_tiles(int64_t tiles, int64_t* previous) {
+    if (tiles < 0) return mq_fail(MQ_ERR_ARG, "the launch length is a tile count, 0 for no cutting");
+    const int64_t old = tile_launch_cap().exchange(tiles);
+    if (previous) *previous = old;
+    return MQ_OK;
+}
+
 // jobs [i, j) hold `tiles` tiles: where the first of the equal launches they are cut into ends
 static int64_t tile_run_end(const mq_job* jobs, int64_t i, int64_t j, int64_t tiles) {
-    // (the environment variable MQ_TILE_LAUNCH_TILES overrides the length, 0 switches the cutting off: for measurements)
-    int64_t cap = MQ_TILE_LAUNCH_TILES;
-    if (const char* env = getenv("MQ_TILE_LAUNCH_TILES")) cap = atoll(env);
+    const int64_t cap = tile_launch_cap().load(std::memory_order_relaxed);
     if (cap <= 0 || tiles <= cap) return j;
     const int64_t launches = (tiles + cap - 1) / cap;
     const int64_t target = (tiles + launches - 1) / launches;

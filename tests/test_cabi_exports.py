@@ -1,4 +1,6 @@
-"""The C-ABI library loads and exports every symbol include/miles_quant.h declares (no GPU needed)."""
+"""The C-ABI libraries load and export every symbol their headers declare (no GPU needed): libmiles_quant.so for
+include/miles_quant.h, and libmq_probes.so -- self-tests and streaming probes, not part of the product -- for
+include/miles_quant_probes.h."""
 
 import ctypes
 import os
@@ -9,10 +11,10 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "miles_quant.h")).read()
+def _declared_symbols(header="miles_quant.h", prefix="mq_"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mq_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(" + prefix + r"[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_declares_the_expected_entry_points():
@@ -34,6 +36,22 @@ def test_library_exports_every_declared_symbol():
     # the ctypes signature table covers every declared compute entry point
     declared = set(_declared_symbols()) - {"mq_version", "mq_last_error"}
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+
+
+def test_probes_library_exports_its_header_and_the_product_library_holds_none_of_it():
+    from miles_amd import _lib, _probes
+
+    if not os.path.exists(_probes.lib_path()):
+        pytest.fail(f"{_probes.lib_path()} not built: run `python -m miles_amd.build`")
+    declared = _declared_symbols("miles_quant_probes.h", "mqp_")
+    lib = ctypes.CDLL(_probes.lib_path())
+    assert declared and not [s for s in declared if not hasattr(lib, s)]
+    assert set(declared) - {"mqp_last_error"} == set(_probes.SIGNATURES)
+    product = ctypes.CDLL(_lib.lib_path())
+    leaked = [s for s in declared + ["mq_selftest_convert", "mq_selftest_reciprocal", "mq_stream_probe", "mq_copy_bytes"]
+              if hasattr(product, s)]
+    assert not leaked, f"measurement scaffolding exported by the product library: {leaked}"
+    assert not [s for s in _declared_symbols() if s.startswith("mqp_")]
 
 
 def test_wrappers_refuse_cpu_tensors():

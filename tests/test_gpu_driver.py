@@ -1296,20 +1296,61 @@ def test_snapshot_publisher_writes_the_quantized_model(oracle, tmp_path):
 
 
 def test_stream_probes_run_and_refuse_bad_arguments():
-    """The measurement-only probes: every shape runs on a small buffer, stays inside it, and refuses what it cannot take."""
-    lib = _lib.load()
+    """The measurement-only probes of libmq_probes.so: every shape runs on a small buffer, stays inside it, and refuses
+    what it cannot take; the plain copy copies."""
+    from miles_amd import _probes
+
+    lib = _probes.load()
     nbytes = 3 * 128 * 1024 * 2 + 4096                   # a [384, 1024] matrix of 2-byte elements and a little more
     src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=DEV)
     guard = 4096
     dst = torch.full((nbytes + guard,), 0xA5, dtype=torch.uint8, device=DEV)
     stream = _lib.stream_ptr(src.device)
     for shape, param in ((0, 1), (0, 2), (0, 4), (0, 8), (1, 1), (1, 2), (2, 512), (3, 1024), (4, 1024), (5, 1024), (3, 128)):
-        assert lib.mq_stream_probe(shape, src.data_ptr(), dst.data_ptr(), nbytes, param, stream) == 0, (shape, param)
+        assert lib.mqp_stream_probe(shape, src.data_ptr(), dst.data_ptr(), nbytes, param, stream) == 0, (shape, param)
     torch.cuda.synchronize()
     assert bool((dst[nbytes:] == 0xA5).all())
     for shape, param, size in ((0, 3, nbytes), (2, 100, nbytes), (3, 100, nbytes), (9, 1, nbytes), (0, 2, nbytes + 8), (3, 1 << 30, nbytes)):
-        assert lib.mq_stream_probe(shape, src.data_ptr(), dst.data_ptr(), size, param, stream) != 0, (shape, param, size)
-    assert lib.mq_stream_probe(0, None, dst.data_ptr(), nbytes, 2, stream) != 0
+        assert lib.mqp_stream_probe(shape, src.data_ptr(), dst.data_ptr(), size, param, stream) != 0, (shape, param, size)
+    assert lib.mqp_stream_probe(0, None, dst.data_ptr(), nbytes, 2, stream) != 0
+    assert b"aligned" in lib.mqp_last_error()
+    dst.fill_(0xA5)
+    assert lib.mqp_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes - nbytes % 4096, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst[: nbytes - nbytes % 4096], src[: nbytes - nbytes % 4096]) and bool((dst[nbytes:] == 0xA5).all())
+    assert lib.mqp_copy_bytes(src.data_ptr(), dst.data_ptr(), 100, stream) != 0
+
+
+def test_the_launch_cut_can_be_tuned_and_results_do_not_depend_on_it(oracle):
+    """mq_tune_tile_launch_tiles sets the length at which runs of tile jobs are cut into launches and hands back the
+    one it replaces; the outputs are the same bytes whatever the length."""
+    import ctypes
+
+    from miles_amd import launch
+    from miles_amd.kernels.quant.fp8_blockwise import fp8_blockwise_cast
+
+    lib = _lib.load()
+    ws = [W.gaussian_outliers((512, 640), std=0.02, p_outlier=0.001, gain=20.0, seed=9300 + i) for i in range(12)]
+    dev = [w.to(DEV) for w in ws]
+    want = [oracle.fp8_blockwise_cast(w) for w in ws]
+    with launch.recording() as batch:
+        outs = [fp8_blockwise_cast(w) for w in dev]
+    batch.device = torch.device(DEV)
+    first, previous = ctypes.c_int64(-1), ctypes.c_int64(-1)
+    assert lib.mq_tune_tile_launch_tiles(50, ctypes.byref(first)) == 0 and first.value > 0       # 240 tiles in launches of 48
+    try:
+        for length in (50, 0, 7, 100000):
+            assert lib.mq_tune_tile_launch_tiles(length, ctypes.byref(previous)) == 0
+            for q, s in outs:
+                q.view(torch.uint8).fill_(0x5A), s.fill_(-1.0)
+            batch.run()
+            torch.cuda.synchronize()
+            for i, ((q, s), (wq, ws_)) in enumerate(zip(outs, want)):
+                _same(q, wq, f"tensor {i} codes (launches of {length})"), _same(s, ws_, f"tensor {i} scales (launches of {length})")
+        assert previous.value == 7
+        assert lib.mq_tune_tile_launch_tiles(-1, None) != 0
+    finally:
+        assert lib.mq_tune_tile_launch_tiles(first.value, None) == 0
 
 
 def test_amax_feedback_counters_through_the_c_abi():

@@ -39,9 +39,17 @@ def lib():
 
 
 # ---------------------------------------------------------------------------------------------------
-def test_hardware_converts_agree_with_software_rne(lib):
+@pytest.fixture(scope="module")
+def probes():
+    """libmq_probes.so: the device self-tests (not part of the product library)."""
+    from miles_amd import _probes
+
+    return _probes.load()
+
+
+def test_hardware_converts_agree_with_software_rne(probes):
     counts = torch.zeros(16, dtype=torch.int64, device=DEV)
-    assert lib.mq_selftest_convert(counts.data_ptr(), None) == 0
+    assert probes.mqp_selftest_convert(counts.data_ptr(), None) == 0
     torch.cuda.synchronize()
     c = counts.cpu().tolist()
     print("selftest counts", c[:8])
@@ -52,9 +60,9 @@ def test_hardware_converts_agree_with_software_rne(lib):
     assert c[7] == 0, "packed e2m1 convert nibble order"
 
 
-def test_refined_hardware_reciprocal_is_the_ieee_quotient(lib):
-    count = torch.ones(1, dtype=torch.int64, device=DEV)
-    assert lib.mq_selftest_reciprocal(count.data_ptr(), None) == 0
+def test_refined_hardware_reciprocal_is_the_ieee_quotient(probes):
+    count = torch.ones(2, dtype=torch.int64, device=DEV)[:1]
+    assert probes.mqp_selftest_reciprocal(count.data_ptr(), None) == 0
     torch.cuda.synchronize()
     assert count.item() == 0, "v_rcp_f32 + one Newton step differs from 1.0f / s inside the shared-divisor range"
 
