@@ -67,10 +67,13 @@ int mq_fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, float* s
  * hipMalloc).  The amax workspace is a static device array of MQ_FP8_STATIC_MAX_ROWS words (1 MiB, held by every
  * GPU the library runs on until the process ends); the call allocates nothing.  Results are those of
  * mq_fp8_scaled_quant.  per_channel != 0 with M > MQ_FP8_STATIC_MAX_ROWS is refused with MQ_ERR_ARG.
- * The device that is current at the call must be the one holding the tensors.  Every call on a GPU shares that
- * GPU's array: calls that overlap in time on one GPU (two streams, two host threads) race on it.  The first call
- * on a device looks the array's address up (hipGetSymbolAddress); make that call (M = 0 is enough) before
- * starting a graph capture. */
+ * The device that is current at the call must be the one holding the tensors.  Every call on a GPU takes its words
+ * from that GPU's one array, consecutive calls taking consecutive pieces of it (one 256-byte line for a per-tensor call,
+ * M words for a per-channel one) and starting over at its beginning when a piece no longer fits.  Calls that overlap in
+ * time on one GPU (two streams, two host threads) therefore race only when the pieces handed out while the earlier one
+ * is still running add up to more than the array: 4 096 per-tensor calls, or per-channel calls of 262 144 rows in all.
+ * A caller that keeps more than that in flight on one GPU must order its calls itself.  The first call on a device looks
+ * the array's address up (hipGetSymbolAddress); make that call (M = 0 is enough) before starting a graph capture. */
 #define MQ_FP8_STATIC_MAX_ROWS 262144
 int mq_fp8_scaled_quant_static(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M, int64_t K,
                                int per_channel, float floor_in_dtype, void* stream);
@@ -333,15 +336,17 @@ int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table);
 int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* device_table, void* stream);
 
 /* mq_run_jobs_tabled that also reports how many amax records moved (no counterpart in the reference).  device_moved
- * points to four uint32 in device memory.  Words 0 and 1 are counters that the call never clears: every fold of NVFP4
- * or per-tensor FP8 amax records made by the call adds the number of tensors it folded to word 1, and to word 0 the
- * number of those whose record held another amax before.  Words 2 and 3 are the low and the high half of an address
- * (0 = none) of two uint32 in host-visible memory (pinned, mapped) that every fold launch first refreshes with the
- * counters as the launches before it left them, so that the host can read them at any time without a copy, an event or
- * a wait.  When most tensors keep moving from one submission to the next -- where MQ_NVFP4_CARRY_AMAX costs a second
- * pass over every such tensor -- the caller submits the list without the flag until they hold still again; the
- * records stay valid for either form.  device_table and device_moved may be NULL. */
-int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved, void* stream);
+ * points to two uint32 in device memory, counters that the call never clears: every fold of NVFP4 or per-tensor FP8 amax
+ * records made by the call adds the number of tensors it folded to word 1, and to word 0 the number of those whose
+ * record held another amax before.  host_mirror (may be NULL) points to two uint32 of pinned host memory (hipHostMalloc;
+ * anything else is refused): every fold launch first refreshes them with the counters as the launches before it left
+ * them, so that the host can read them at any time without a copy, an event or a wait.  The mirror must stay allocated
+ * until every submitted call that named it has finished on the GPU: the kernels store through its address.
+ * When most tensors keep moving from one submission to the next -- where MQ_NVFP4_CARRY_AMAX costs a second pass over
+ * every such tensor -- the caller submits the list without the flag until they hold still again; the records stay valid
+ * for either form.  device_table and device_moved may be NULL (then host_mirror must be NULL too). */
+int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved,
+                         uint32_t* host_mirror, void* stream);
 
 #ifdef __cplusplus
 }

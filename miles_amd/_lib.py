@@ -51,7 +51,7 @@ SIGNATURES = {
     "mq_tune_tile_launch_tiles": [_i64, _vp],
     "mq_job_table_fill": [_vp, _i64, _vp],
     "mq_run_jobs_tabled": [_vp, _i64, _vp, _vp],
-    "mq_run_jobs_feedback": [_vp, _i64, _vp, _vp, _vp],
+    "mq_run_jobs_feedback": [_vp, _i64, _vp, _vp, _vp, _vp],
 }
 
 MAX_GROUP = 64                                            # MQ_MAX_GROUP: tensors per fused launch of mq_run_jobs

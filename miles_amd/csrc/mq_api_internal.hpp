@@ -7,10 +7,12 @@
 
 int mq_fail(int code, const char* msg);
 int mq_check_launch(const char* what);
-// Device counter that the amax fold kernels of the running mq_run_jobs_feedback call add to (null outside such a call):
-// set on entry, cleared on return, per host thread.
+// Device counters that the amax fold kernels of the running mq_run_jobs_feedback call add to, and the device-visible
+// address of the host mirror they refresh (both null outside such a call): set on entry, cleared on return, per host
+// thread.
 uint32_t* mq_amax_feedback();
-void mq_set_amax_feedback(uint32_t* device_counter);
+uint32_t* mq_amax_feedback_mirror();
+void mq_set_amax_feedback(uint32_t* device_counter, uint32_t* mirror);
 // upper bound on the grid of a grid-stride kernel: enough workgroups to fill 256 CUs several times over
 inline int64_t mq_grid_cap() { return 256 * 16; }
 

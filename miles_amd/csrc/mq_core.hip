@@ -8,8 +8,13 @@
 
 static thread_local char g_err[256] = "";
 static thread_local uint32_t* g_amax_feedback = nullptr;
+static thread_local uint32_t* g_amax_feedback_mirror = nullptr;
 uint32_t* mq_amax_feedback() { return g_amax_feedback; }
-void mq_set_amax_feedback(uint32_t* device_counter) { g_amax_feedback = device_counter; }
+uint32_t* mq_amax_feedback_mirror() { return g_amax_feedback_mirror; }
+void mq_set_amax_feedback(uint32_t* device_counter, uint32_t* mirror) {
+    g_amax_feedback = device_counter;
+    g_amax_feedback_mirror = mirror;
+}
 
 int mq_fail(int code, const char* msg) {
     snprintf(g_err, sizeof(g_err), "%s", msg);

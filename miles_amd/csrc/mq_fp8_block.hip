@@ -695,9 +695,13 @@ static __device__ __align__(256) uint32_t scratch[MQ_FP8_STATIC_MAX_ROWS];
 static constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_lock;
 static uint32_t* g_scratch_ptr[kMaxDevices];      // device address of `scratch` on each GPU, 0 until first use there
+static int64_t g_scratch_next[kMaxDevices];       // first word of the array that the next call on that GPU takes
 
-// address of `scratch` on the current device, or null with the error text set
-static uint32_t* scratch_on_current_device() {
+// `words` words of `scratch` on the current device for one call, or null with the error text set.  Calls take
+// consecutive pieces of the array (whole 256-byte lines), starting over at its beginning when a piece no longer fits:
+// two calls that are in flight together -- on two streams, from two host threads -- only share words when the pieces
+// handed out between them add up to more than the array.
+static uint32_t* scratch_on_current_device(int64_t words) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -714,7 +718,11 @@ static uint32_t* scratch_on_current_device() {
         }
         g_scratch_ptr[dev] = (uint32_t*)p;
     }
-    return g_scratch_ptr[dev];
+    const int64_t piece = (words + 63) / 64 * 64;
+    if (g_scratch_next[dev] + piece > MQ_FP8_STATIC_MAX_ROWS) g_scratch_next[dev] = 0;
+    uint32_t* at = g_scratch_ptr[dev] + g_scratch_next[dev];
+    g_scratch_next[dev] += piece;
+    return at;
 }
 
 extern "C" int mq_fp8_scaled_quant_static(const void* w, int dtype, int64_t ldw, void* q, float* scale, int64_t M,
@@ -722,7 +730,7 @@ extern "C" int mq_fp8_scaled_quant_static(const void* w, int dtype, int64_t ldw,
     if (per_channel && M > MQ_FP8_STATIC_MAX_ROWS)
         return mq_fail(MQ_ERR_ARG, "mq_fp8_scaled_quant_static: per-channel scales take at most MQ_FP8_STATIC_MAX_ROWS "
                                    "(262144) rows; use mq_fp8_scaled_quant with a workspace of its own");
-    uint32_t* ws = scratch_on_current_device();
+    uint32_t* ws = scratch_on_current_device(per_channel && M > 0 ? M : 1);
     if (!ws) return MQ_ERR_HIP;
     return fp8_scaled_quant(w, dtype, ldw, q, scale, ws, M, K, per_channel, floor_in_dtype, stream);
 }

@@ -21,11 +21,11 @@ constexpr int kFtUnroll = 2;
 
 // job.s = fp32 scale output, job.aux = amax record (section 0)
 template <int MODE, class Table>   // 1: fold and clear; 2: also compare with the amax the record held
-__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, float floor_v, uint32_t* moved_counter) {
+__global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, float floor_v, uint32_t* moved_counter, uint32_t* moved_mirror) {
     __shared__ uint32_t lds4[4];
     const FlatJob& job = tab.job[blockIdx.x];
     uint32_t* rec = (uint32_t*)job.aux;
-    amax_feedback_folded(moved_counter, gridDim.x);
+    amax_feedback_folded(moved_counter, moved_mirror, gridDim.x);
     uint32_t m = rec[threadIdx.x];
     rec[threadIdx.x] = 0;
     m = wave_max(m);
@@ -167,14 +167,14 @@ static int fp8_tensor_launch_dtype(const Table& tab, int n, float floor_v, bool 
     const dim3 folds((unsigned)n), blk(256), grid((unsigned)tab.max_blocks, (unsigned)n);
     if (carry) {
         if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<1, Table, F16>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
-        hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
+        hipLaunchKernelGGL((fp8_tensor_fold_kernel<2, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback(), mq_amax_feedback_mirror());
         if (tab.max_blocks > 0) {
             const unsigned redo = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             hipLaunchKernelGGL((fp8_tensor_quant_kernel<2, Table, F16>), dim3(redo, (unsigned)n), dim3(kFtThreads), 0, st, tab, floor_v);
         }
         return mq_check_launch("fp8 per-tensor quant (carried-over amax)");
     }
-    hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback());
+    hipLaunchKernelGGL((fp8_tensor_fold_kernel<1, Table>), folds, blk, 0, st, tab, floor_v, mq_amax_feedback(), mq_amax_feedback_mirror());
     if (tab.max_blocks > 0) hipLaunchKernelGGL((fp8_tensor_quant_kernel<0, Table, F16>), grid, dim3(kFtThreads), 0, st, tab, floor_v);
     return mq_check_launch("fp8 per-tensor quant");
 }

@@ -216,11 +216,12 @@ __device__ __forceinline__ void amax_feedback(uint32_t* counter, bool moved, uin
     if (counter && moved) atomicAdd(counter, tensors);
 }
 // Once per fold launch: first the two counters as the launches before left them (a consistent pair) go to the caller's
-// host-visible mirror, if it named one in words 2 and 3, then this launch's tensors are added to the second counter.
-__device__ __forceinline__ void amax_feedback_folded(uint32_t* counter, uint32_t tensors) {
+// host-visible mirror, if the call named one (a kernel argument: the host checked that it is pinned memory), then this
+// launch's tensors are added to the second counter.
+__device__ __forceinline__ void amax_feedback_folded(uint32_t* counter, uint32_t* mirror_words, uint32_t tensors) {
     if (counter && blockIdx.x == 0 && threadIdx.x == 0) {
-        volatile uint32_t* mirror = (volatile uint32_t*)(((uint64_t)counter[3] << 32) | counter[2]);
-        if (mirror) {
+        if (mirror_words) {
+            volatile uint32_t* mirror = mirror_words;
             const uint32_t moved = atomicAdd(counter, 0u), folded = atomicAdd(counter + 1, 0u);
             mirror[0] = moved;
             mirror[1] = folded;

@@ -125,12 +125,12 @@ constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 //   with the fresh amax -- the cost of the plain two-pass form, instead of two full quantizations.  The mark is dropped
 //   as soon as the amax has held still for one sync.
 template <int MODE, class Table>
-__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer, uint32_t* moved_counter) {
+__global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer, uint32_t* moved_counter, uint32_t* moved_mirror) {
     __shared__ uint32_t lds4[4];
     const int ji = blockIdx.x;
     const FlatJob& job = tab.job[ji];
     const int sections = MODE == 0 ? job.section : job.pad;
-    if (MODE != 0) amax_feedback_folded(moved_counter, gridDim.x);
+    if (MODE != 0) amax_feedback_folded(moved_counter, moved_mirror, gridDim.x);
     if (MODE != 0 && job.section != job.pad - 1) return;
     uint32_t* rec = (uint32_t*)job.aux;
     uint32_t m = 0;
@@ -706,15 +706,15 @@ static int nvfp4_quant_launch(const Table& tab, int n, int e4m3_max, int flags, 
     const dim3 grid((unsigned)tab.max_blocks, (unsigned)n);
     if (mode == 2) {
         if (tab.max_blocks > 0) launch_nvfp4_quant<1>(tab, flags, numer, grid, st);
-        hipLaunchKernelGGL((nvfp4_fold_kernel<2, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback());
+        hipLaunchKernelGGL((nvfp4_fold_kernel<2, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback(), mq_amax_feedback_mirror());
         if (tab.max_blocks > 0) {
             const unsigned redo_blocks = tab.max_blocks < kSectionWords ? (unsigned)tab.max_blocks : (unsigned)kSectionWords;
             launch_nvfp4_quant<2>(tab, flags, numer, dim3(redo_blocks, (unsigned)n), st);
         }
         return mq_check_launch("nvfp4 quant (carried-over amax)");
     }
-    if (mode == 1) hipLaunchKernelGGL((nvfp4_fold_kernel<1, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback());
-    else hipLaunchKernelGGL((nvfp4_fold_kernel<0, Table>), folds, blk, 0, st, tab, numer, (uint32_t*)nullptr);
+    if (mode == 1) hipLaunchKernelGGL((nvfp4_fold_kernel<1, Table>), folds, blk, 0, st, tab, numer, mq_amax_feedback(), mq_amax_feedback_mirror());
+    else hipLaunchKernelGGL((nvfp4_fold_kernel<0, Table>), folds, blk, 0, st, tab, numer, (uint32_t*)nullptr, (uint32_t*)nullptr);
     if (tab.max_blocks > 0) launch_nvfp4_quant<0>(tab, flags, numer, grid, st);
     return mq_check_launch("nvfp4 quant");
 }
@@ -774,7 +774,7 @@ extern "C" int mq_nvfp4_quant(const void* w, int dtype, const void* record, int 
     FlatTable fold{};
     fold.n = 1;
     fold.job[0] = FlatJob{w, q, block_scale, const_cast<void*>(record), 0, global_scale, n_sections, 0};
-    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, st, fold, numer, (uint32_t*)nullptr);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, st, fold, numer, (uint32_t*)nullptr, (uint32_t*)nullptr);
     int64_t nb = (blocks16 + 255) / 256;
     if (nb > mq_grid_cap()) nb = mq_grid_cap();
     hipLaunchKernelGGL(nvfp4_quant_generic_kernel, dim3((unsigned)nb), dim3(256), 0, st, w, dtype,
@@ -789,7 +789,7 @@ extern "C" int mq_nvfp4_fold(void* record, int n_sections, int e4m3_max, void* s
     FlatTable tab{};
     tab.n = 1;
     tab.job[0] = FlatJob{nullptr, nullptr, nullptr, record, 0, nullptr, n_sections, 0};
-    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f, (uint32_t*)nullptr);
+    hipLaunchKernelGGL((nvfp4_fold_kernel<0, FlatTable>), dim3(1), dim3(256), 0, (hipStream_t)stream, tab, (float)e4m3_max * 6.0f, (uint32_t*)nullptr, (uint32_t*)nullptr);
     return mq_check_launch("nvfp4 fold");
 }
 

@@ -432,11 +432,23 @@ extern "C" int mq_job_table_fill(const mq_job* jobs, int64_t n, void* host_table
 extern "C" int mq_run_jobs(const mq_job* jobs, int64_t n, void* stream) { return mq_run_jobs_tabled(jobs, n, nullptr, stream); }
 
 extern "C" int mq_run_jobs_feedback(const mq_job* jobs, int64_t n, const void* device_table, uint32_t* device_moved,
-                                    void* stream) {
-    if ((uintptr_t)device_moved % 4 != 0) return mq_fail(MQ_ERR_ARG, "feedback counters must be 4-byte aligned");
-    mq_set_amax_feedback(device_moved);
+                                    uint32_t* host_mirror, void* stream) {
+    if ((uintptr_t)device_moved % 4 != 0 || (uintptr_t)host_mirror % 4 != 0)
+        return mq_fail(MQ_ERR_ARG, "feedback counters and their mirror must be 4-byte aligned");
+    if (host_mirror && !device_moved) return mq_fail(MQ_ERR_ARG, "a feedback mirror needs the device counters it mirrors");
+    uint32_t* mirror = nullptr;
+    if (host_mirror) {
+        // the fold kernels store through this address: it has to be host memory the GPU can write (pinned, mapped)
+        hipPointerAttribute_t attr;
+        if (hipPointerGetAttributes(&attr, host_mirror) != hipSuccess || attr.type != hipMemoryTypeHost || !attr.devicePointer) {
+            (void)hipGetLastError();
+            return mq_fail(MQ_ERR_ARG, "the feedback mirror must be pinned host memory (hipHostMalloc)");
+        }
+        mirror = (uint32_t*)attr.devicePointer;
+    }
+    mq_set_amax_feedback(device_moved, mirror);
     const int rc = mq_run_jobs_tabled(jobs, n, device_table, stream);
-    mq_set_amax_feedback(nullptr);
+    mq_set_amax_feedback(nullptr, nullptr);
     return rc;
 }
 

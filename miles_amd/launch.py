@@ -25,8 +25,8 @@ class _AmaxFeedback:
     """What share of the amax records moved in the syncs the GPU has finished, read without ever waiting for it.
 
     The folds of a `mq_run_jobs_feedback` call add to two device counters that only grow -- tensors whose record held
-    another amax before, and tensors folded -- and every fold launch first mirrors the pair into two pinned words, so the
-    host reads them with no copy, no event and no wait.  At the start of a submission: when more than half of the tensors
+    another amax before, and tensors folded -- and every fold launch first mirrors the pair into two pinned words (their
+    address travels with every call, as a host argument), so the host reads them with no copy, no event and no wait.  At the start of a submission: when more than half of the tensors
     folded since the last reading had moved, the list is submitted in the plain two-pass form (the carried-over amax
     would cost every such tensor a second pass), until they hold again."""
 
@@ -66,9 +66,8 @@ class _AmaxFeedback:
         self.mirror = self._pool[slot]
         self.mirror.zero_()
         self.mirror_words = self.mirror.numpy()       # the same pinned words, read without going through torch
-        address = self.mirror.data_ptr()
-        words = [0, 0, address & 0xFFFFFFFF, address >> 32]
-        self.counter = torch.tensor([w - (1 << 32) if w >= 1 << 31 else w for w in words], dtype=torch.int32).to(device)
+        self.mirror_address = self.mirror.data_ptr()
+        self.counter = torch.zeros(2, dtype=torch.int32, device=device)
         self.seen = (0, 0)          # the counters as of the last reading that had new folds
         self.plain = False
 
@@ -217,8 +216,8 @@ class JobBatch:
                 arr = self._plain_array()
         ptr = ctypes.byref(arr, start * ctypes.sizeof(_lib.Job))
         table = None if self._table is None else self._table.data_ptr() + start * _lib.TABLE_ENTRY_BYTES
-        counter = None if feedback is None else feedback.counter.data_ptr()
-        _lib.check(_lib.load().mq_run_jobs_feedback(ptr, stop - start, table, counter, stream))
+        counter, mirror = (None, None) if feedback is None else (feedback.counter.data_ptr(), feedback.mirror_address)
+        _lib.check(_lib.load().mq_run_jobs_feedback(ptr, stop - start, table, counter, mirror, stream))
 
     def _plain_array(self):
         """The job list without the carried-amax flag (same records, same device table)."""

@@ -1364,17 +1364,31 @@ def test_amax_feedback_counters_through_the_c_abi():
         outs = [tensor_fp8(w) for w in ws]
     arr = batch.freeze()
     lib = _lib.load()
-    words = torch.zeros(4, dtype=torch.int32, device=DEV)
+    words = torch.zeros(2, dtype=torch.int32, device=DEV)
     stream = _lib.stream_ptr(torch.device(DEV))
-    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
-    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), None, stream) == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), None, stream) == 0
     ws[2].mul_(2.0)
-    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), stream) == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), None, stream) == 0
     torch.cuda.synchronize()
-    moved, folded, lo, hi = words.cpu().tolist()
+    moved, folded = words.cpu().tolist()
     # the records start out uninitialised, so every first fold may or may not count as moved; afterwards only tensor 2
-    assert folded == 15 and 1 <= moved <= 6 and lo == 0 and hi == 0
-    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr() + 2, stream) != 0      # misaligned words
+    assert folded == 15 and 1 <= moved <= 6
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr() + 2, None, stream) != 0      # misaligned words
+    # a host mirror: pinned memory is taken (every fold launch refreshes it with the counters the launches before left),
+    # anything else -- pageable host memory, device memory, a mirror without counters -- is refused before any launch
+    mirror = torch.zeros(2, dtype=torch.int32).pin_memory()
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), mirror.data_ptr(), stream) == 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), mirror.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert mirror.tolist() == [moved, 25] and words.cpu().tolist() == [moved, 30]      # nothing moved; the mirror lags one fold launch
+    pageable = torch.zeros(2, dtype=torch.int32)
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), pageable.data_ptr(), stream) != 0
+    assert b"pinned" in lib.mq_last_error()
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), words.data_ptr(), stream) != 0
+    assert lib.mq_run_jobs_feedback(arr, len(batch), None, None, mirror.data_ptr(), stream) != 0
+    torch.cuda.synchronize()
+    assert words.cpu().tolist() == [moved, 30]
     assert outs[0][0].dtype == torch.float8_e4m3fn
 
 

@@ -92,3 +92,35 @@ def test_static_entry_point_allocates_nothing_and_checks_its_limit():
     assert b"262144" in lib.mq_last_error()
     # an empty tensor is fine (and is the call to make before a graph capture)
     assert lib.mq_fp8_scaled_quant_static(None, 0, 0, None, None, 0, 0, 1, _floor(w.dtype), None) == 0
+
+
+def test_static_calls_in_flight_on_two_streams_take_different_words():
+    """Consecutive calls take consecutive pieces of the static array, so per-tensor calls queued on two streams at once
+    (every one of them used to clear, fill and read word 0) do not disturb each other's amax."""
+    from miles_amd import _lib
+
+    lib = _lib.load()
+    big = (W.gaussian_outliers((4096, 4096), std=3.0, p_outlier=0.01, gain=20.0, seed=21).float()).to(torch.bfloat16).to(DEV)
+    small = (W.gaussian_outliers((4096, 4096), std=0.01, p_outlier=0.0, gain=1.0, seed=22).float()).to(torch.bfloat16).to(DEV)
+    want = {}
+    for name, w in (("big", big), ("small", small)):
+        (q_ref, s_ref), _ = _both(lib, w, False)
+        want[name] = (q_ref.cpu(), s_ref.cpu())
+    streams = [torch.cuda.Stream(device=DEV), torch.cuda.Stream(device=DEV)]
+    outs = []
+    torch.cuda.synchronize()
+    for rep in range(8):                                   # sixteen calls queued without a wait in between
+        for (name, w), stream in zip((("big", big), ("small", small)), streams):
+            q = torch.full((4096, 4096), 0x55, dtype=torch.uint8, device=DEV)
+            s = torch.full((1,), -1.0, dtype=torch.float32, device=DEV)
+            outs.append((name, q, s))
+    torch.cuda.synchronize()
+    for i, (name, q, s) in enumerate(outs):
+        w = big if name == "big" else small
+        rc = lib.mq_fp8_scaled_quant_static(w.data_ptr(), 0, w.stride(0), q.data_ptr(), s.data_ptr(), 4096, 4096, 0,
+                                            _floor(w.dtype), streams[i % 2].cuda_stream)
+        assert rc == 0, lib.mq_last_error()
+    torch.cuda.synchronize()
+    for i, (name, q, s) in enumerate(outs):
+        assert torch.equal(s.cpu().view(torch.int32), want[name][1].view(torch.int32)), f"call {i} ({name}): scale differs"
+        assert torch.equal(q.cpu(), want[name][0]), f"call {i} ({name}): codes differ"
