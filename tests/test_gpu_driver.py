@@ -1381,14 +1381,14 @@ def test_amax_feedback_counters_through_the_c_abi():
     assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), mirror.data_ptr(), stream) == 0
     assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), mirror.data_ptr(), stream) == 0
     torch.cuda.synchronize()
-    assert mirror.tolist() == [moved, 25] and words.cpu().tolist() == [moved, 30]      # nothing moved; the mirror lags one fold launch
+    assert mirror.tolist() == [moved, 20] and words.cpu().tolist() == [moved, 25]      # nothing moved; the mirror lags one fold launch
     pageable = torch.zeros(2, dtype=torch.int32)
     assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), pageable.data_ptr(), stream) != 0
     assert b"pinned" in lib.mq_last_error()
     assert lib.mq_run_jobs_feedback(arr, len(batch), None, words.data_ptr(), words.data_ptr(), stream) != 0
     assert lib.mq_run_jobs_feedback(arr, len(batch), None, None, mirror.data_ptr(), stream) != 0
     torch.cuda.synchronize()
-    assert words.cpu().tolist() == [moved, 30]
+    assert words.cpu().tolist() == [moved, 25]
     assert outs[0][0].dtype == torch.float8_e4m3fn
 
 
