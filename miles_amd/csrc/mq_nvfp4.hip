@@ -312,6 +312,26 @@ __device__ __forceinline__ float nv_block_error(const float f[16], const NvCandi
     for (int j = 0; j < 8; j++) error = error + term[j];
     return error;
 }
+// A cheaper error sum that decides almost every block.  With a = RN(f32(scale) * amax / denom), the exact term's
+// dequantized value RN(q * f32(scale) * amax / denom) IS q * a for the codes that are powers of two (0.5, 1, 2, 4: scaling
+// by a power of two commutes with the rounding) and differs from q * a by at most 2^-23 of its size for 1.5, 3 and 6.
+// The estimate sums |q * a - x|, each term rounded once (an FMA), in element order.  Every step is within a few units in
+// the last place of the exact computation, so the estimated sum S' and the exact sum S of a candidate differ by at most
+//   2^-20 (31.4 a + 2 bmax) + 30.3 * 2^-24 S'
+// (per element: 2.01 * 2^-24 |deq| between the two dequantized values, 2^-24 (|deq| + |x|) for each of the two roundings
+// of the difference, |deq| <= 6 a (1 + 2^-22), |x| <= bmax; for the sums: recursive summation of sixteen non-negative
+// terms is within 15.1 * 2^-24 of their true sum, on both sides).  Whenever the two estimates are further apart than
+// the two bounds together, the exact sums compare the same way.
+__device__ __forceinline__ float nv_block_error_estimate(const float f[16], const NvCandidate16& c, float a) {
+    float q[8], sum = 0.0f;
+    nv_decode8(c.lo, q);
+#pragma unroll
+    for (int j = 0; j < 8; j++) sum = sum + __builtin_fabsf(__builtin_fmaf(q[j], a, -f[j]));
+    nv_decode8(c.hi, q);
+#pragma unroll
+    for (int j = 0; j < 8; j++) sum = sum + __builtin_fabsf(__builtin_fmaf(q[j], a, -f[8 + j]));
+    return sum;
+}
 template <int EM, int FASTDIV>
 __device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], float bmax, float amax, const NvScales& gs,
                                                             float denom, float denom_inv) {
@@ -319,6 +339,18 @@ __device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], f
     const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate16 c4 = nv_candidate16(f, s4_hp, gs.s_dec), c6 = nv_candidate16(f, s6_hp, gs.s_dec);
+    if (EM == 0 && FASTDIV == 2) {
+        // (FASTDIV 2: f32(scale) * amax is exact and its quotient by denom comes correctly rounded from the sequence)
+        const float a4 = div_by_numer<2>(c4.s_f * amax, denom, denom_inv), a6 = div_by_numer<2>(c6.s_f * amax, denom, denom_inv);
+        const float g4 = nv_block_error_estimate(f, c4, a4), g6 = nv_block_error_estimate(f, c6, a6);
+        // twice the bound's first part and four times its second: rounding in this line cannot bring it below the bound
+        const float guard = 0x1p-19f * (32.0f * (a4 + a6) + 4.0f * bmax + 4.0f * (g4 + g6));
+        // (an all-zero block, or two candidates with one scale byte -- the block that holds the tensor's maximum, whose
+        // scales both saturate: the candidates are the same, the tie goes to map-to-6, as g4 < g6 says; a NaN compares false)
+        const bool decided = __builtin_fabsf(g4 - g6) > guard || bmax == 0.0f || c4.sc == c6.sc;
+        if (__builtin_amdgcn_ballot_w64(!decided) == 0) return g4 < g6 ? c4 : c6;
+        // a wavefront with a block too close to call (a few blocks in 10 000, most of them exact ties) takes the exact sums below
+    }
     const float e4 = nv_block_error<EM, FASTDIV>(f, c4, amax, gs.enc, denom, denom_inv);
     const float e6 = nv_block_error<EM, FASTDIV>(f, c6, amax, gs.enc, denom, denom_inv);
     return e4 < e6 ? c4 : c6;
@@ -343,12 +375,24 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
     const uint16_t* __restrict__ w0 = w + base * 8;
     uint32_t* __restrict__ q0 = q + base;
     uint8_t* __restrict__ s80 = s8 + base / 2;
+    // both loads are issued before either is waited for: a lane past the end reads the workgroup's first unit again
+    // (always there) and drops it
+    u32x4 in[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const uint32_t off = (uint32_t)t + i * kNvThreads;
-        stage[off] = off < rem ? ld16(w0 + off * 8u) : u32x4{0u, 0u, 0u, 0u};
+        in[i] = ld16(w0 + (off < rem ? off : 0u) * 8u);
     }
-    __syncthreads();        // (a wavefront reads back only what it wrote itself)
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t off = (uint32_t)t + i * kNvThreads;
+        stage[off] = off < rem ? in[i] : u32x4{0u, 0u, 0u, 0u};
+    }
+    // A wavefront reads back only what its own lanes wrote, and the LDS serves one wavefront's accesses in the order
+    // it issued them: no workgroup barrier, only the compiler is told not to move the reads above the writes.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const uint32_t first = ((t & 1) ? (uint32_t)kNvThreads : 0u) + ((uint32_t)t & ~1u);      // the block's first unit
     const u32x4 lo = stage[first], hi = stage[first + 1];
     NvScales gs;
