@@ -1,4 +1,5 @@
-"""What Triton's fp32 `/` gives on this GPU for the two divisions of the sync path's FP8 quantizer.
+"""What Triton makes, on this GPU, of the expressions the reference's two Triton kernels on this path are written in:
+the sync path's FP8 quantizer (its two fp32 divisions first of all) and the FP8 block dequantizer.
 
 The reference's `_fp8_blockwise_cast_kernel` (miles/kernels/quant/fp8_blockwise.py:51-54) computes, per tile,
 `_absmax = maximum(max|x|, eps)`, `x_s = _absmax / fp8_max` and `s_inv = 1.0 / x_s` with Triton's `/` on fp32 scalars
@@ -259,3 +260,48 @@ def test_triton_tile_quantizer_on_one_qwen3_4b_layer():
         hy, hs = fp8_blockwise_cast(x)
         assert torch.equal(ts.view(torch.int32), hs.view(torch.int32)), f"{shape}: scales"
         assert torch.equal(ty.view(torch.uint8), hy.view(torch.uint8)), f"{shape}: codes"
+
+
+def test_triton_dequantizer_gives_the_hip_kernels_bytes(oracle):
+    """The FP8 block dequantizer of the reference is a Triton kernel too (tools/fp8_cast_bf16.py:15-27): decode the code
+    to fp32, one multiplication by the tile's scale, a store that rounds to bf16.  A probe written for this test from
+    those expressions (flat over the elements, the scale found per element) against the HIP kernel: every code byte
+    times scales over eighty binades, subnormal products and NaN codes included (any bf16 NaN counts as NaN)."""
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+
+    try:
+        import triton
+        import triton.language as tl
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton is not importable: {exc!r}")
+
+    @triton.jit
+    def decode_scale_store(code_ptr, scale_ptr, out_ptr, count, cols, tiles_across, BLOCK: tl.constexpr, TILE: tl.constexpr):
+        at = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+        live = at < count
+        value = tl.load(code_ptr + at, mask=live).to(tl.float32)
+        scale = tl.load(scale_ptr + (at // cols) // TILE * tiles_across + (at % cols) // TILE, mask=live)
+        tl.store(out_ptr + at, value * scale, mask=live)
+
+    g = torch.Generator().manual_seed(17)
+    rows, cols = 384, 640
+    codes = torch.arange(256, dtype=torch.uint8).repeat(rows, 3)[:, :cols].contiguous()
+    codes[200:] = torch.randint(0, 256, (rows - 200, cols), generator=g, dtype=torch.int32).to(torch.uint8)
+    scale = torch.exp(torch.randn((3, 5), generator=g) * 12).float()
+    scale[0, 0], scale[1, 1], scale[2, 2], scale[0, 4] = 0.0, -2.5, 2.0 ** -130, 2.0 ** 100
+    x, s = codes.view(torch.float8_e4m3fn).to(DEV), scale.to(DEV)
+    out = torch.empty((rows, cols), dtype=torch.bfloat16, device=DEV)
+    try:
+        decode_scale_store[(triton.cdiv(rows * cols, 1024),)](x, s, out, rows * cols, cols, 5, BLOCK=1024, TILE=128)
+        torch.cuda.synchronize()
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+    hip = weight_dequant(x, s)
+    want = oracle.weight_dequant(codes.view(torch.float8_e4m3fn), scale)
+    assert torch.equal(hip.cpu().view(torch.int16), want.view(torch.int16)), "the HIP dequantizer differs from the oracle"
+    t, h = out.cpu(), hip.cpu()
+    nan = torch.isnan(h)
+    assert torch.equal(torch.isnan(t), nan), "NaN in different places"
+    differ = int((t.view(torch.int16)[~nan] != h.view(torch.int16)[~nan]).sum())
+    print("TRITON_DEQUANTIZER", json.dumps({"elements": rows * cols, "nan_elements": int(nan.sum()), "values_differ": differ}))
+    assert differ == 0
