@@ -2,6 +2,7 @@
 
     python -m miles_amd.tools.convert_hf_to_mxfp8 --model-dir SRC --save-dir DST [--device cuda]
         [--num-layers-at-start-in-bf16 N] [--num-layers-at-end-in-bf16 N] [--extra-high-precision-layers-hf ...]
+        [--metadata-only]
 
 Mirror of the reference's tools/convert_hf_to_mxfp8.py (`process_file` :123-228, `convert_mxfp8` :231-308).
 Sources: BF16/FP16/FP32 checkpoints, and block-scaled FP8 checkpoints (`scale_fmt: ue8m0`, [128,128] scales stored
@@ -22,6 +23,7 @@ import torch
 
 from miles_amd import launch
 from miles_amd.tools import _checkpoint as ckpt
+from miles_amd.utils.hf_rollout_schema import create_mxfp8_rollout_schema
 from miles_amd.utils.mxfp8 import (MXFP8_GROUP_SIZE, MXFP8_SKIP_WEIGHT_SUBSTRINGS, MXFP8_SOURCE_FP8_DTYPES,
                                    dequantize_fp8_source, expand_tile_scales_e8m0, exponent_bytes_to_fp32,
                                    fp8_tile_scales_pow2, requantize_fp8_block_to_mxfp8, should_use_mxfp8)
@@ -164,7 +166,13 @@ def main(argv=None) -> None:
     ap.add_argument("--num-layers-at-start-in-bf16", type=int, default=0)
     ap.add_argument("--num-layers-at-end-in-bf16", type=int, default=0)
     ap.add_argument("--extra-high-precision-layers-hf", type=str, nargs="*", default=())
+    ap.add_argument("--metadata-only", action="store_true",
+                    help="Write a weightless MXFP8 rollout schema (config + tokenizer) instead of converting weights.")
     args, _ = ap.parse_known_args(argv)
+    if args.metadata_only:      # host work only: no device, no kernel (reference :359-362)
+        schema = create_mxfp8_rollout_schema(args.model_dir, args.save_dir)
+        print(f"Created metadata-only MXFP8 rollout schema at {schema}")
+        return
     if not torch.cuda.is_available():
         raise RuntimeError("CUDA is not available, cannot run MXFP8 quantization.")
     device = torch.device(f"cuda:{args.device}" if args.device.isdigit() else args.device)
