@@ -318,33 +318,51 @@ __global__ __launch_bounds__(256) void mxfp4_tile_smax_kernel(const RecodeTable 
         __syncthreads();
     }
 }
+#ifndef MQ_RECODE_UNROLL
+#define MQ_RECODE_UNROLL 2
+#endif
+// 16-element units per lane, 256 lanes apart, every load issued before the first conversion.  Measured on
+// 8 x [16384, 7168] as one job list: 5.79 / 6.20 / 6.11 TB/s with one / two / four units.
+constexpr int kRecodeUnroll = MQ_RECODE_UNROLL;
 __global__ __launch_bounds__(256) void mxfp4_recode_flat_kernel(const RecodeTable tab) {
     const RecodeJob& job = tab.job[blockIdx.y];
-    const int64_t u64 = xcd_chunked_block(job.flat_chunk) * 256 + threadIdx.x;
-    if (u64 >= job.units) return;
-    const uint32_t u = (uint32_t)u64;
+    const int64_t base64 = xcd_chunked_block(job.flat_chunk) * (256 * kRecodeUnroll) + threadIdx.x;
+    if (base64 >= job.units) return;
+    const uint32_t base = (uint32_t)base64;
     const uint32_t upr = (uint32_t)(job.in_dim / 16);
-    const uint32_t row = tile_div(u, job.magic_upr, job.shift_upr), cu = u - row * upr;
-    const u32x2 v = __builtin_nontemporal_load((const u32x2*)job.packed + u);
-    const uint32_t s = job.scale[u >> 1];
-    const uint32_t bits = f2u(job.tile_scale[(uint64_t)(row >> 7) * job.tiles_in + (cu >> 3)]);
-    const uint32_t e = bits >> 23;
-    const uint32_t smax = bits == 0x7FC00000u ? 255u : e != 0u ? e + 6u : (uint32_t)(31 - __builtin_clz(bits | 1u)) - 16u;
-    // offset = 2^(s - smax + 6) in (0, 64]; far below the e4m3 range every product rounds to (signed) zero anyway
-    const int k = (int)s - (int)smax + 6;
-    const float factor = u2f((uint32_t)((k < -60 ? -60 : k) + 127) << 23);
-    const uint32_t w[2] = {v.x, v.y};
-    uint32_t o[4];
+    u32x2 v[kRecodeUnroll];
+    uint32_t s[kRecodeUnroll], bits[kRecodeUnroll];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 1);
-        const f32x2 cc = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 3);
-        o[2 * j] = hw_e4m3x4(a.x * factor, a.y * factor, b.x * factor, b.y * factor);
-        o[2 * j + 1] = hw_e4m3x4(cc.x * factor, cc.y * factor, d.x * factor, d.y * factor);
+    for (int i = 0; i < kRecodeUnroll; i++) {
+        const uint32_t u = base + i * 256;
+        const uint32_t uc = u < job.units ? u : base;          // a dead unit repeats the lane's first one and stores nothing
+        const uint32_t row = tile_div(uc, job.magic_upr, job.shift_upr), cu = uc - row * upr;
+        v[i] = ((const u32x2*)job.packed)[uc];      // an ordinary load: 8-byte loads measured 0.5 % faster without the non-temporal hint
+        s[i] = job.scale[uc >> 1];
+        bits[i] = f2u(job.tile_scale[(uint64_t)(row >> 7) * job.tiles_in + (cu >> 3)]);
     }
-    // a NaN scale byte anywhere in the tile makes the tile scale, every offset and every product NaN: code 0x7F
-    if (smax == 255u) o[0] = o[1] = o[2] = o[3] = 0x7F7F7F7Fu;
-    st16(job.y + (uint64_t)u * 16, u32x4{o[0], o[1], o[2], o[3]});
+#pragma unroll
+    for (int i = 0; i < kRecodeUnroll; i++) {
+        const uint32_t u = base + i * 256;
+        if (u >= job.units) break;
+        const uint32_t e = bits[i] >> 23;
+        const uint32_t smax = bits[i] == 0x7FC00000u ? 255u : e != 0u ? e + 6u : (uint32_t)(31 - __builtin_clz(bits[i] | 1u)) - 16u;
+        // offset = 2^(s - smax + 6) in (0, 64]; far below the e4m3 range every product rounds to (signed) zero anyway
+        const int k = (int)s[i] - (int)smax + 6;
+        const float factor = u2f((uint32_t)((k < -60 ? -60 : k) + 127) << 23);
+        const uint32_t w[2] = {v[i].x, v[i].y};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 1);
+            const f32x2 cc = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 3);
+            o[2 * j] = hw_e4m3x4(a.x * factor, a.y * factor, b.x * factor, b.y * factor);
+            o[2 * j + 1] = hw_e4m3x4(cc.x * factor, cc.y * factor, d.x * factor, d.y * factor);
+        }
+        // a NaN scale byte anywhere in the tile makes the tile scale, every offset and every product NaN: code 0x7F
+        if (smax == 255u) o[0] = o[1] = o[2] = o[3] = 0x7F7F7F7Fu;
+        st16(job.y + (uint64_t)u * 16, u32x4{o[0], o[1], o[2], o[3]});
+    }
 }
 
 }  // namespace mq
@@ -446,7 +464,7 @@ int mq_mxfp4_to_fp8_job(RecodeJob& job, const void* packed, const void* scale, v
     if (units > 0 && units < 0x7FFFFFFFll && ((uintptr_t)scale & 3) == 0) {
         job.units = (uint32_t)units;
         tile_div_magic((uint32_t)(in_dim / 16), job.magic_upr, job.shift_upr);
-        job.flat_chunk = (int32_t)flat_chunk((units + 255) / 256);
+        job.flat_chunk = (int32_t)flat_chunk((units + 256 * kRecodeUnroll - 1) / (256 * kRecodeUnroll));
     }
     return MQ_OK;
 }
@@ -460,7 +478,7 @@ int mq_mxfp4_to_fp8_launch_group(const RecodeTable& tab, hipStream_t st) {
         flat = flat && (j.units != 0 || j.total_pairs == 0);
         const int64_t b = j.pairs_in ? j.total_pairs / j.pairs_in : 0;
         bands = b > bands ? b : bands;
-        const int64_t g = j.units ? flat_padded(((int64_t)j.units + 255) / 256, j.flat_chunk) : 0;
+        const int64_t g = j.units ? flat_padded(((int64_t)j.units + 256 * kRecodeUnroll - 1) / (256 * kRecodeUnroll), j.flat_chunk) : 0;
         blocks = g > blocks ? g : blocks;
     }
     if (flat) {
