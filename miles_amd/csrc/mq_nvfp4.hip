@@ -322,14 +322,27 @@ __device__ __forceinline__ float nv_block_error(const float f[16], const NvCandi
 // of the difference, |deq| <= 6 a (1 + 2^-22), |x| <= bmax; for the sums: recursive summation of sixteen non-negative
 // terms is within 15.1 * 2^-24 of their true sum, on both sides).  Whenever the two estimates are further apart than
 // the two bounds together, the exact sums compare the same way.
+//
+// The squared error (SQUARED) has the same estimate with each difference d' = RN(q * a - x) squared.  Per element the
+// exact difference d and d' are within E = 2^-24 (24.1 a + 2 bmax) of each other (the three contributions above), so
+// the squares differ by at most E (2 |d'| + E) and, rounded, by 2^-23 d'^2 more; over the block, with
+// sum |d'| <= 4 sqrt(sum d'^2), the estimated and the exact sum of a candidate differ by at most
+//   8.1 E sqrt(S') + 16.1 E^2 + 32.5 * 2^-24 S'.
+template <bool SQUARED>
 __device__ __forceinline__ float nv_block_error_estimate(const float f[16], const NvCandidate16& c, float a) {
     float q[8], sum = 0.0f;
     nv_decode8(c.lo, q);
 #pragma unroll
-    for (int j = 0; j < 8; j++) sum = sum + __builtin_fabsf(__builtin_fmaf(q[j], a, -f[j]));
+    for (int j = 0; j < 8; j++) {
+        const float d = __builtin_fmaf(q[j], a, -f[j]);
+        sum = sum + (SQUARED ? d * d : __builtin_fabsf(d));
+    }
     nv_decode8(c.hi, q);
 #pragma unroll
-    for (int j = 0; j < 8; j++) sum = sum + __builtin_fabsf(__builtin_fmaf(q[j], a, -f[8 + j]));
+    for (int j = 0; j < 8; j++) {
+        const float d = __builtin_fmaf(q[j], a, -f[8 + j]);
+        sum = sum + (SQUARED ? d * d : __builtin_fabsf(d));
+    }
     return sum;
 }
 template <int EM, int FASTDIV>
@@ -339,12 +352,22 @@ __device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], f
     const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
     const NvCandidate16 c4 = nv_candidate16(f, s4_hp, gs.s_dec), c6 = nv_candidate16(f, s6_hp, gs.s_dec);
-    if (EM == 0 && FASTDIV == 2) {
+    if ((EM == 0 || EM == 1) && FASTDIV == 2) {
         // (FASTDIV 2: f32(scale) * amax is exact and its quotient by denom comes correctly rounded from the sequence)
         const float a4 = div_by_numer<2>(c4.s_f * amax, denom, denom_inv), a6 = div_by_numer<2>(c6.s_f * amax, denom, denom_inv);
-        const float g4 = nv_block_error_estimate(f, c4, a4), g6 = nv_block_error_estimate(f, c6, a6);
-        // twice the bound's first part and four times its second: rounding in this line cannot bring it below the bound
-        const float guard = 0x1p-19f * (32.0f * (a4 + a6) + 4.0f * bmax + 4.0f * (g4 + g6));
+        const float g4 = nv_block_error_estimate<EM == 1>(f, c4, a4), g6 = nv_block_error_estimate<EM == 1>(f, c6, a6);
+        float guard;
+        if (EM == 0) {
+            // twice the bound's first part and four times its second: rounding in this line cannot bring it below the bound
+            guard = 0x1p-19f * (32.0f * (a4 + a6) + 4.0f * bmax + 4.0f * (g4 + g6));
+        } else {
+            // twice the squared error's bound for both candidates, and more (the hardware square root is within one unit
+            // in the last place; the small constant keeps a denormal sum from dropping out of it and is the floor below
+            // which two sums are too small to call)
+            const float e4 = 0x1p-24f * (25.0f * a4 + 2.0f * bmax), e6 = 0x1p-24f * (25.0f * a6 + 2.0f * bmax);
+            guard = 17.0f * (e4 * __builtin_amdgcn_sqrtf(g4 + 0x1p-100f) + e6 * __builtin_amdgcn_sqrtf(g6 + 0x1p-100f)) +
+                    33.0f * (e4 * e4 + e6 * e6) + 0x1p-17f * (g4 + g6) + 0x1p-100f;
+        }
         // (an all-zero block, or two candidates with one scale byte -- the block that holds the tensor's maximum, whose
         // scales both saturate: the candidates are the same, the tie goes to map-to-6, as g4 < g6 says; a NaN compares false)
         const bool decided = __builtin_fabsf(g4 - g6) > guard || bmax == 0.0f || c4.sc == c6.sc;
@@ -362,66 +385,89 @@ static inline int nv_error_mode(int flags) { return ((flags & MQ_NVFP4_ERR_MSE) 
 // units t and kNvThreads + t, so a wavefront's loads are contiguous), then regrouped through LDS inside each wavefront so
 // that the even lane of a pair holds the block made of units 2p, 2p + 1 and the odd lane the block kNvThreads + 2p, + 1.
 // Returns the largest |element| of the lane's block (bf16 bits).
+#ifndef MQ_NV_FOS_ROUNDS
+#define MQ_NV_FOS_ROUNDS 2
+#endif
+// consecutive pieces of kNvThreads * 2 units one Four Over Six workgroup takes.  Measured on 96 DeepSeek-V3 expert
+// matrices, steady state: 4.74 / 4.95 / 4.83 TB/s with one / two / three pieces (78 and 86 registers with two and three:
+// six and five wavefronts per SIMD instead of seven).
+constexpr int kFosRounds = MQ_NV_FOS_ROUNDS;
+// units a workgroup of the quantizer covers (FOS as in nvfp4_quant_units)
+constexpr int64_t nv_units_per_block(int fos) { return (int64_t)kNvThreads * kNvUnroll * (fos ? kFosRounds : 1); }
 template <int EM, int F16>
 __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const int64_t base, const int t, const float denom) {
     static_assert(kNvUnroll == 2, "the regrouping pairs the two units of a lane");
-    __shared__ u32x4 stage[2 * kNvThreads];
+    constexpr uint32_t kPiece = kNvThreads * 2;
+    __shared__ u32x4 stage[kPiece];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
     const uint32_t* __restrict__ amax_bits = (const uint32_t*)job.aux;
     const int64_t left = job.units - base;
-    const uint32_t rem = left < kNvThreads * 2 ? (uint32_t)left : (uint32_t)(kNvThreads * 2);
+    const uint32_t rem_all = left < kPiece * kFosRounds ? (uint32_t)left : kPiece * kFosRounds;
     const uint16_t* __restrict__ w0 = w + base * 8;
     uint32_t* __restrict__ q0 = q + base;
     uint8_t* __restrict__ s80 = s8 + base / 2;
-    // both loads are issued before either is waited for: a lane past the end reads the workgroup's first unit again
-    // (always there) and drops it
-    u32x4 in[2];
+    // every load of every piece is issued before the first is waited for: this kernel is bound by its arithmetic, some
+    // two hundred vector instructions per block, and a wavefront that computes on one piece while nothing of its own is
+    // in flight leaves the memory system idle.  A lane past the end reads the workgroup's first unit again (always
+    // there) and drops it.
+    u32x4 in[kFosRounds][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t off = (uint32_t)t + i * kNvThreads;
-        in[i] = ld16(w0 + (off < rem ? off : 0u) * 8u);
-    }
+    for (int r = 0; r < kFosRounds; r++)
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const uint32_t off = (uint32_t)t + i * kNvThreads;
-        stage[off] = off < rem ? in[i] : u32x4{0u, 0u, 0u, 0u};
-    }
-    // A wavefront reads back only what its own lanes wrote, and the LDS serves one wavefront's accesses in the order
-    // it issued them: no workgroup barrier, only the compiler is told not to move the reads above the writes.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const uint32_t first = ((t & 1) ? (uint32_t)kNvThreads : 0u) + ((uint32_t)t & ~1u);      // the block's first unit
-    const u32x4 lo = stage[first], hi = stage[first + 1];
+        for (int i = 0; i < 2; i++) {
+            const uint32_t off = r * kPiece + (uint32_t)t + i * kNvThreads;
+            in[r][i] = ld16(w0 + (off < rem_all ? off : 0u) * 8u);
+        }
     NvScales gs;
     gs.enc_sixth = u2f(amax_bits[kRecEncSixth]);
     gs.s_dec = u2f(amax_bits[kRecSDec]);
     gs.enc = u2f(amax_bits[kRecEnc]);
     const float amax = u2f(amax_bits[kRecAmax]);
     const int fastdiv = nv_fast_division(amax);
-    const uint32_t m2 = max2_u16(max2_u16(max2_u16(abs2(lo.x), abs2(lo.y)), max2_u16(abs2(lo.z), abs2(lo.w))),
-                                 max2_u16(max2_u16(abs2(hi.x), abs2(hi.y)), max2_u16(abs2(hi.z), abs2(hi.w))));
-    const uint32_t mb = hmax_u16(m2);
-    const float bmax = elem_lo<F16>(mb);
-    const float f[16] = {elem_lo<F16>(lo.x), elem_hi<F16>(lo.x), elem_lo<F16>(lo.y), elem_hi<F16>(lo.y),
-                         elem_lo<F16>(lo.z), elem_hi<F16>(lo.z), elem_lo<F16>(lo.w), elem_hi<F16>(lo.w),
-                         elem_lo<F16>(hi.x), elem_hi<F16>(hi.x), elem_lo<F16>(hi.y), elem_hi<F16>(hi.y),
-                         elem_lo<F16>(hi.z), elem_hi<F16>(hi.z), elem_lo<F16>(hi.w), elem_hi<F16>(hi.w)};
     // the error's divisor 6 * e4m3_max is one of two constants and the same for the whole launch: its reciprocal is
     // picked on the scalar unit
     constexpr float kInv2688 = 1.0f / 2688.0f, kInv1536 = 1.0f / 1536.0f;
     const float denom_inv = denom == 2688.0f ? kInv2688 : denom == 1536.0f ? kInv1536 : 1.0f / denom;
-    const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom, denom_inv)
-                            : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom, denom_inv)
-                                           : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom, denom_inv);
-    if (first < rem) {      // the tensor is whole blocks: both units of a block are inside or outside
-        st4(q0 + first, c.lo);
-        st4(q0 + first + 1, c.hi);
-        s80[first >> 1] = (uint8_t)c.sc;
+    uint32_t seen = 0;
+#pragma unroll
+    for (int r = 0; r < kFosRounds; r++) {
+        if (r * kPiece >= rem_all) break;      // the same for the whole workgroup
+        const uint32_t rem = rem_all - r * kPiece;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t off = (uint32_t)t + i * kNvThreads;
+            stage[off] = off < rem ? in[r][i] : u32x4{0u, 0u, 0u, 0u};
+        }
+        // A wavefront reads back only what its own lanes wrote, and the LDS serves one wavefront's accesses in the order
+        // it issued them: no workgroup barrier, only the compiler is told not to move the reads above the writes.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t first = ((t & 1) ? (uint32_t)kNvThreads : 0u) + ((uint32_t)t & ~1u);      // the block's first unit
+        const u32x4 lo = stage[first], hi = stage[first + 1];
+        // (and the next piece's writes stay below these reads)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t m2 = max2_u16(max2_u16(max2_u16(abs2(lo.x), abs2(lo.y)), max2_u16(abs2(lo.z), abs2(lo.w))),
+                                     max2_u16(max2_u16(abs2(hi.x), abs2(hi.y)), max2_u16(abs2(hi.z), abs2(hi.w))));
+        const uint32_t mb = hmax_u16(m2);
+        seen = umax(seen, mb);
+        const float bmax = elem_lo<F16>(mb);
+        const float f[16] = {elem_lo<F16>(lo.x), elem_hi<F16>(lo.x), elem_lo<F16>(lo.y), elem_hi<F16>(lo.y),
+                             elem_lo<F16>(lo.z), elem_hi<F16>(lo.z), elem_lo<F16>(lo.w), elem_hi<F16>(lo.w),
+                             elem_lo<F16>(hi.x), elem_hi<F16>(hi.x), elem_lo<F16>(hi.y), elem_hi<F16>(hi.y),
+                             elem_lo<F16>(hi.z), elem_hi<F16>(hi.z), elem_lo<F16>(hi.w), elem_hi<F16>(hi.w)};
+        const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom, denom_inv)
+                                : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom, denom_inv)
+                                               : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom, denom_inv);
+        if (first < rem) {      // the tensor is whole blocks: both units of a block are inside or outside
+            st8(q0 + r * kPiece + first, u32x2{c.lo, c.hi});      // `first` is even and `base` a multiple of the piece
+            s80[(r * kPiece + first) >> 1] = (uint8_t)c.sc;
+        }
     }
-    return mb;
+    return seen;
 }
 
 // kNvThreads * kNvUnroll units starting at `base` of one tensor; returns the largest |element| this lane saw (bf16 bits)
@@ -518,7 +564,7 @@ template <int FOS, int PASS, class Table, int F16>
 __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Table tab, float denom) {
     const FlatJob job = flat_job(tab);       // a copy in registers: a descriptor in device memory must not be re-read after the stores
     const int t = threadIdx.x;
-    constexpr int64_t kPerBlock = kNvThreads * kNvUnroll;
+    constexpr int64_t kPerBlock = nv_units_per_block(FOS);
     if (PASS == 2) {
         if (((const uint32_t*)job.aux)[kRecRedo] == 0) return;
         // an XCD takes a run of consecutive blocks in every trip of the grid, as the flat grids do (second pass 2 pct faster)
@@ -530,8 +576,11 @@ __global__ __launch_bounds__(kNvThreads) void nvfp4_quant_bf16_kernel(const Tabl
     const int64_t base = flat_block(tab) * kPerBlock;
     if (base >= job.units) return;
     uint32_t seen;
-    if (PASS == 1 && ((const uint32_t*)job.aux)[kRecVolatile] != 0) seen = nvfp4_amax_units(job, base, t);
-    else seen = nvfp4_quant_units<FOS, F16>(job, base, t, denom);
+    if (PASS == 1 && ((const uint32_t*)job.aux)[kRecVolatile] != 0) {
+        seen = 0;
+        for (int64_t piece = base; piece < base + kPerBlock && piece < job.units; piece += kNvThreads * kNvUnroll)
+            seen = umax(seen, nvfp4_amax_units(job, piece, t));
+    } else seen = nvfp4_quant_units<FOS, F16>(job, base, t, denom);
     if (PASS == 1) {
         __shared__ uint32_t wave_seen[kNvThreads / 64];
         seen = wave_max(seen);
@@ -770,7 +819,7 @@ static int nvfp4_quant_launch(const Table& tab, int n, int e4m3_max, int flags, 
 // mode 2 (job driver, carried-over amax; the sections were cleared by the previous sync's fold): quantize with the
 //   record's old scales while collecting the new partial maxima, fold and compare, quantize again where they differ.
 int mq_nvfp4_quant_launch_group(int dtype, FlatTable& tab, int e4m3_max, int flags, int mode, hipStream_t st) {
-    if (!flat_grid(tab, kNvThreads * kNvUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (!flat_grid(tab, nv_units_per_block(flags & MQ_NVFP4_4OVER6))) return mq_fail(MQ_ERR_ARG, "tensor too large");
     return nvfp4_quant_launch(tab, tab.n, e4m3_max, flags | (dtype == MQ_F16 ? kNvFlagF16 : 0), mode, st);
 }
 // modes 1 and 2 over n descriptors of a device table (standard block scaling only); max_units: the largest tensor's units

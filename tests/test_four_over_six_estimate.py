@@ -3,6 +3,7 @@ miles_amd/csrc/mq_nvfp4.hip) and computes the reference's exact error sums only 
 close to call.  This file checks the claim behind that on the CPU, in numpy's fp32 arithmetic, over millions of random
 blocks: whenever the two estimates differ by more than the kernel's guard, the exact sums -- the reference's
 `nvfp4_qdq.py:893-953` terms, restated as the oracle states them -- compare the same way; and the guard is rarely needed.
+Both error measures the estimate serves are covered: the sum of absolute differences (default) and of squares (MSE).
 """
 
 import numpy as np
@@ -44,6 +45,11 @@ def _seq_sum(terms):
     return total
 
 
+def _term(diff, squared):
+    with np.errstate(over="ignore", under="ignore"):
+        return (diff * diff).astype(F32) if squared else np.abs(diff)
+
+
 def _candidate(oracle, x, s_hp, s_dec):
     sc = oracle.f32_to_e4m3fn(torch.from_numpy(np.minimum(s_hp, F32(448.0))), sat=True)
     s_f = sc.view(torch.float8_e4m3fn).float().numpy()
@@ -54,10 +60,11 @@ def _candidate(oracle, x, s_hp, s_dec):
     return s_f, q.astype(F32)
 
 
+@pytest.mark.parametrize("squared", [False, True], ids=["mae", "mse"])
 @pytest.mark.parametrize("e4m3_max", [448, 256])
 @pytest.mark.parametrize("dtype_bits", [8, 16])       # bf16 (8 significant bits) and fp16 (11) values
-def test_the_estimate_decides_as_the_exact_error_sums_do(oracle, e4m3_max, dtype_bits):
-    x, bmax, amax = _blocks(1_500_000, seed=e4m3_max + dtype_bits, dtype_bits=dtype_bits)
+def test_the_estimate_decides_as_the_exact_error_sums_do(oracle, e4m3_max, dtype_bits, squared):
+    x, bmax, amax = _blocks(1_500_000, seed=e4m3_max + dtype_bits + 1000 * squared, dtype_bits=dtype_bits)
     denom = F32(6 * e4m3_max)
     with np.errstate(over="ignore"):
         enc = np.minimum(denom / amax, FLT_MAX).astype(F32)
@@ -69,16 +76,25 @@ def test_the_estimate_decides_as_the_exact_error_sums_do(oracle, e4m3_max, dtype
         s_f, q = _candidate(oracle, x, s_hp, s_dec)
         # the reference's terms: RN(RN(RN(q * s) * amax) / denom) - x, summed in element order in fp32
         dq = (((q * s_f[:, None]).astype(F32) * amax[:, None]).astype(F32) / denom).astype(F32)
-        exact[name] = _seq_sum(np.abs((dq - x).astype(F32)))
+        exact[name] = _seq_sum(_term((dq - x).astype(F32), squared))
         # the kernel's estimate: a = RN(s * amax / denom), terms |fma(q, a, -x)| (one rounding: taken through float64,
         # where q * a - x is exact)
         a = ((s_f * amax).astype(F32) / denom).astype(F32)
         fma = (q.astype(np.float64) * a[:, None].astype(np.float64) - x.astype(np.float64)).astype(F32)
-        estimate[name] = _seq_sum(np.abs(fma))
+        estimate[name] = _seq_sum(_term(fma, squared))
         slope[name] = a
         scale[name] = s_f
-    guard = (F32(2.0 ** -19) * (F32(32.0) * (slope["4"] + slope["6"]) + F32(4.0) * bmax
-                                + F32(4.0) * (estimate["4"] + estimate["6"]))).astype(F32)
+    if squared:
+        # the hardware square root may come out one unit in the last place low: taken two low here
+        with np.errstate(over="ignore", invalid="ignore"):
+            root = {k: (np.sqrt((estimate[k] + F32(2.0 ** -100)).astype(F32)) * F32(1 - 2.0 ** -22)).astype(F32)
+                    for k in "46"}
+            e = {k: (F32(2.0 ** -24) * (F32(25.0) * slope[k] + F32(2.0) * bmax)).astype(F32) for k in "46"}
+            guard = (F32(17.0) * (e["4"] * root["4"] + e["6"] * root["6"]) + F32(33.0) * (e["4"] * e["4"] + e["6"] * e["6"])
+                     + F32(2.0 ** -17) * (estimate["4"] + estimate["6"]) + F32(2.0 ** -100)).astype(F32)
+    else:
+        guard = (F32(2.0 ** -19) * (F32(32.0) * (slope["4"] + slope["6"]) + F32(4.0) * bmax
+                                    + F32(4.0) * (estimate["4"] + estimate["6"]))).astype(F32)
     # (two candidates with one scale byte are the same candidate: the block that holds the tensor's maximum)
     decided = (np.abs((estimate["4"] - estimate["6"]).astype(F32)) > guard) | (scale["4"] == scale["6"])
     pick4_exact = exact["4"] < exact["6"]
