@@ -363,7 +363,10 @@ def adjacent_formats(gen):
     res["next_mxfp4_quant"] = {"GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "ms": round(ms, 4),
                                "elements": elems, "workload": "8 x [16384,7168] bf16, group 32, one grouped launch"}
     del batch
-    run("next_mxfp4_dequant", "mxfp4_dequant", lambda: [dequantize_mxfp4(p, s, 32) for p, s in m4], "MXFP4 -> bf16")
+    # (the converters unpack a shard's tensors together, launch.deferred: the lines are job lists)
+    batch, outs = _record(lambda: [dequantize_mxfp4(p, s, 32) for p, s in m4])
+    run("next_mxfp4_dequant", "mxfp4_dequant", batch.run, "MXFP4 -> bf16, one job list (single calls: 0.80 of peak at this size)")
+    del batch, outs
     from miles_amd.tools.convert_mxfp4_to_fp8 import cast_e2m1fn_to_e4m3fn
     # the converter submits a shard's casts together (launch.deferred), so the line is a job list too
     batch, outs = _record(lambda: [cast_e2m1fn_to_e4m3fn(p.view(torch.int8), s) for p, s in m4])
@@ -378,7 +381,9 @@ def adjacent_formats(gen):
         "FP8 128x128 block-scaled codes (general fp32 scales) -> MXFP8 in one pass, as the MXFP8 converter submits a shard: one job list")
     del batch, outs, f8
     i4 = [pack_layer(w, 128) for w in ws]
-    run("next_int4_unpack", "int4_unpack", lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4], "INT4 g128 -> bf16")
+    batch, outs = _record(lambda: [_dequantize_tensor(p, s, shape, 128) for p, s, _ in i4])
+    run("next_int4_unpack", "int4_unpack", batch.run, "INT4 g128 -> bf16, one job list (single calls: 0.78 of peak at this size)")
+    del batch, outs
     del i4
     batch, outs = _record(lambda: [pack_layer(w, 128, sym=False) for w in ws])
     run("next_int4_g128_asym_pack", "int4_g128_asym", batch.run,

@@ -260,6 +260,11 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  *   MQ_JOB_E8M0_EXPAND          tile scales   E8M0 bytes    -              -                           -
  *     (mq_e8m0_expand_tile_scales with M = rows, groups = cols, lds = ld; dtype MQ_F32: the grid holds fp32 powers of
  *      two, any other dtype code: exponent bytes)
+ *   MQ_JOB_INT4_UNPACK          int32 words   bf16          -              aux = scales (dtype, in)    group, -
+ *     (mq_int4_unpack_dequant with M = rows, K = cols; dtype is the scales' dtype.  Jobs with one group size and one
+ *      scale dtype share launches of up to MQ_MAX_GROUP tensors: a checkpoint shard's experts unpacked together)
+ *   MQ_JOB_MXFP4_DEQUANT        e2m1 pairs    bf16          -              aux = E8M0 bytes (in)       group, -
+ *     (mq_mxfp4_dequant with bytes = rows * cols / 2; jobs of one group size share launches the same way)
  * ld is the input row stride in elements for the two FP8 quantizers (column stride 1) and ignored elsewhere;
  * rows_per_block / block_stride describe a row-blocked input (see the struct).
  * The three FP8 tile kinds (FP8_BLOCK, FP8_BLOCKWISE_CAST, FP8_BLOCK_POW2), MXFP8, MXFP4, INT4_PACK, INT4_PACK_ASYM, FP8_TENSOR and NVFP4 run their tuned
@@ -290,7 +295,9 @@ enum {
     MQ_JOB_INT4_PACK_ASYM = 11,
     MQ_JOB_MXFP4_TO_FP8 = 12,
     MQ_JOB_FP8_TO_MXFP8 = 13,
-    MQ_JOB_E8M0_EXPAND = 14
+    MQ_JOB_E8M0_EXPAND = 14,
+    MQ_JOB_INT4_UNPACK = 15,
+    MQ_JOB_MXFP4_DEQUANT = 16
 };
 typedef struct mq_job {
     int32_t kind;

@@ -63,7 +63,7 @@ RECORD_AMAX_WORD, RECORD_REDO_WORD, RECORD_VOLATILE_WORD = 1024, 1028, 1029
 
 (JOB_FP8_BLOCK, JOB_FP8_BLOCKWISE_CAST, JOB_FP8_DEQUANT, JOB_MXFP8, JOB_INT4_PACK, JOB_NVFP4, JOB_MXFP4,
  JOB_COPY, JOB_FP8_BLOCK_POW2, JOB_UE8M0_PACK, JOB_FP8_TENSOR, JOB_INT4_PACK_ASYM, JOB_MXFP4_TO_FP8,
- JOB_FP8_TO_MXFP8, JOB_E8M0_EXPAND) = range(15)
+ JOB_FP8_TO_MXFP8, JOB_E8M0_EXPAND, JOB_INT4_UNPACK, JOB_MXFP4_DEQUANT) = range(17)
 
 
 class Job(_c.Structure):

@@ -480,22 +480,28 @@ __global__ __launch_bounds__(kDqThreads) void fp8_dequant_kernel(const DequantTa
     if (base64 >= job.units) return;
     const uint32_t base = (uint32_t)base64;
     u32x2 in[kDqUnroll];
+    float scale[kDqUnroll];
+    // every load is issued before the first use: a lane past the end reads the workgroup's first unit again (always
+    // there) and stores nothing
 #pragma unroll
     for (int i = 0; i < kDqUnroll; i++) {
         const uint32_t unit = base + i * kDqThreads + threadIdx.x;
+        const uint32_t uc = unit < job.units ? unit : base;
         // an ordinary (cached) load: with the non-temporal hint the 8-byte code loads of this kernel, which writes
         // twice what it reads, ran 2 % slower (6.36 against 6.50 TB/s on 36 tensors of [4096, 2560]); the 4- and
         // 16-byte code loads of the other unpacking kernels measured the other way round and keep the hint
-        in[i] = unit < job.units ? *reinterpret_cast<const u32x2*>(job.x + (int64_t)unit * 8) : u32x2{0u, 0u};
+        in[i] = *reinterpret_cast<const u32x2*>(job.x + (int64_t)uc * 8);
+        const uint32_t th = __umulhi(job.magic, uc);
+        const uint32_t r = (th + ((uc - th) >> 1)) >> job.shift;
+        const uint32_t c = (uc - r * job.units_per_row) * 8u;
+        scale[i] = job.s[(int64_t)(r >> job.block_shift) * job.tiles_n + (c >> job.block_shift)];
     }
+    __builtin_amdgcn_sched_barrier(0);      // (and the scheduler keeps the first unit's arithmetic below the last load)
 #pragma unroll
     for (int i = 0; i < kDqUnroll; i++) {
         const uint32_t unit = base + i * kDqThreads + threadIdx.x;
         if (unit >= job.units) continue;
-        const uint32_t th = __umulhi(job.magic, unit);
-        const uint32_t r = (th + ((unit - th) >> 1)) >> job.shift;
-        const uint32_t c = (unit - r * job.units_per_row) * 8u;
-        const float sc = job.s[(int64_t)(r >> job.block_shift) * job.tiles_n + (c >> job.block_shift)];
+        const float sc = scale[i];
         const uint32_t wd[2] = {in[i].x, in[i].y};
         uint32_t o[4];
         // a NaN code (0x7F / 0xFF) or a non-finite scale must give the canonical bf16 NaN 0x7FC0

@@ -678,44 +678,72 @@ __global__ __launch_bounds__(kI4Threads) void int4_fake_rows_kernel(const void* 
 #define MQ_I4_UNPACK_UNROLL 2
 #endif
 constexpr int kI4UnpackUnroll = MQ_I4_UNPACK_UNROLL;   // words per lane, 256 lanes apart so every load and store instruction stays contiguous
+// One tensor of a launch's table per blockIdx.y: w = packed words, q = bf16 output, s = scales, units = words,
+// section = log2(words per group).
 template <int SDT>
-__global__ __launch_bounds__(256) void int4_unpack_kernel(const uint32_t* __restrict__ packed,
-                                                          const void* __restrict__ scale, uint16_t* __restrict__ y,
-                                                          int64_t words, int group_shift, int chunk) {
-    const int64_t base = xcd_chunked_block(chunk) * (256 * kI4UnpackUnroll) + threadIdx.x;
+__global__ __launch_bounds__(256) void int4_unpack_kernel(const FlatTable tab) {
+    const FlatJob job = flat_job(tab);
+    const uint32_t* __restrict__ packed = (const uint32_t*)job.w;
+    const void* __restrict__ scale = job.s;
+    uint16_t* __restrict__ y = (uint16_t*)job.q;
+    const int64_t words = job.units;
+    const int group_shift = job.section;
+    const int64_t first = flat_block(tab) * (256 * kI4UnpackUnroll);
+    if (first >= words) return;          // a smaller tensor of the group
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset; `first` is a multiple of
+    // the words of a group (at most 256 per unit of a lane, see mq_int4_unpack_fast_ok)
+    const int64_t left = words - first;
+    const uint32_t rem = left < 256 * kI4UnpackUnroll ? (uint32_t)left : (uint32_t)(256 * kI4UnpackUnroll);
+    const uint32_t* __restrict__ packed0 = packed + first;
+    uint16_t* __restrict__ y0 = y + first * 8;
+    const int64_t group0 = first >> group_shift;
     uint32_t word[kI4UnpackUnroll], sraw[kI4UnpackUnroll];
-    // every load is issued before the first use: lanes past the end re-read the last word instead of branching
+    // every load is issued before the first use: lanes past the end re-read the workgroup's first word instead of branching
 #pragma unroll
     for (int u = 0; u < kI4UnpackUnroll; u++) {
-        const int64_t i = base + u * 256 < words ? base + u * 256 : words - 1;
-        word[u] = __builtin_nontemporal_load(packed + i);
-        if (SDT == MQ_F32) sraw[u] = ((const uint32_t*)scale)[i >> group_shift];
-        else sraw[u] = ((const uint16_t*)scale)[i >> group_shift];
+        const uint32_t off = threadIdx.x + u * 256u;
+        const uint32_t i = off < rem ? off : 0u;
+        word[u] = __builtin_nontemporal_load(packed0 + i);
+        if (SDT == MQ_F32) sraw[u] = ((const uint32_t*)scale + group0)[i >> group_shift];
+        else sraw[u] = ((const uint16_t*)scale + group0)[i >> group_shift];
     }
+    // (the scheduler otherwise moves the first word's unpacking, and with it the wait for that word, above the second
+    // word's loads)
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < kI4UnpackUnroll; u++) {
-        const int64_t i = base + u * 256;
-        float s[kI4UnpackUnroll];
-        s[u] = SDT == MQ_F32 ? u2f(sraw[u]) : SDT == MQ_BF16 ? u2f(sraw[u] << 16)
-                                                             : (float)__builtin_bit_cast(_Float16, (uint16_t)sraw[u]);
-        // even nibbles and odd nibbles as bytes: one byte-to-float conversion each
+        const uint32_t off = threadIdx.x + u * 256u;
+        const float sc = SDT == MQ_F32 ? u2f(sraw[u]) : SDT == MQ_BF16 ? u2f(sraw[u] << 16)
+                                                                       : (float)__builtin_bit_cast(_Float16, (uint16_t)sraw[u]);
+        // even nibbles and odd nibbles as bytes: one byte-to-float conversion each.  (n - 8) * scale as
+        // fma(n, scale, -8 * scale): 8 * scale is exact and the FMA rounds the exact n * scale - 8 * scale once, which
+        // is the rounding of the product (itself exact for a bf16 or fp16 scale).
         const uint32_t ev = word[u] & 0x0F0F0F0Fu, od = (word[u] >> 4) & 0x0F0F0F0Fu;
+        const float minus8 = -8.0f * sc;
         float f[8];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            f[2 * k] = ((float)((ev >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
-            f[2 * k + 1] = ((float)((od >> (8 * k)) & 0xFFu) - 8.0f) * s[u];
+            f[2 * k] = __builtin_fmaf((float)((ev >> (8 * k)) & 0xFFu), sc, minus8);
+            f[2 * k + 1] = __builtin_fmaf((float)((od >> (8 * k)) & 0xFFu), sc, minus8);
         }
         u32x4 o = {hw_bf16x2(f[0], f[1]), hw_bf16x2(f[2], f[3]), hw_bf16x2(f[4], f[5]), hw_bf16x2(f[6], f[7])};
         // A NaN or infinite scale (decided for the wavefront): the products may be NaN -- the scale's own, or 0 x inf --
-        // and the reference's rounding to bf16 writes the one quiet NaN 0x7FC0 whatever the sign and the payload.
-        if (__builtin_amdgcn_ballot_w64((f2u(s[u]) & 0x7F800000u) == 0x7F800000u) != 0) {
+        // and the reference's rounding to bf16 writes the one quiet NaN 0x7FC0 whatever the sign and the payload.  A
+        // scale of 2^124 and more, whose eightfold is no longer finite, takes the same path, with the product as written,
+        // and so does a zero or negative one (the FMA's zeros are all +0; the product's carry the sign of n - 8 and of
+        // the scale).  One unsigned comparison covers them all.
+        if (__builtin_amdgcn_ballot_w64(f2u(sc) - 1u >= 0x7D800000u - 1u) != 0) {
             uint32_t h[8];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                f[2 * k] = ((float)((ev >> (8 * k)) & 0xFFu) - 8.0f) * sc;
+                f[2 * k + 1] = ((float)((od >> (8 * k)) & 0xFFu) - 8.0f) * sc;
+            }
 #pragma unroll
             for (int k = 0; k < 8; k++) h[k] = f[k] != f[k] ? 0x7FC0u : hw_bf16x2(f[k], 0.0f) & 0xFFFFu;
             o = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
         }
-        if (i < words) st16(y + i * 8, o);
+        if (off < rem) st16(y0 + off * 8u, o);
     }
 }
 // any K (rows padded to whole words), any group size, any scale dtype: one lane per element
@@ -918,6 +946,28 @@ extern "C" int mq_int4_group_quant_pack_asym(const void* w, int dtype, int32_t* 
     return mq_check_launch("int4 zero-point pack");
 }
 
+// the flat kernel takes whole words and groups of a power-of-two number of words
+bool mq_int4_unpack_fast_ok(const void* packed, const void* y, int64_t K, int group) {
+    const int upg = group / 8;
+    return group > 0 && group <= 2048 * kI4UnpackUnroll && K % 8 == 0 && group % 8 == 0 && (upg & (upg - 1)) == 0 &&
+           ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0;
+}
+FlatJob mq_int4_unpack_entry(const void* packed, const void* scale, void* y, int64_t M, int64_t K, int group) {
+    int shift = 0;
+    while ((1 << shift) < group / 8) shift++;
+    return FlatJob{packed, y, (void*)scale, nullptr, M * (K / 8), nullptr, shift, 0};
+}
+// up to kMaxGroup tensors with scales of one dtype in one launch
+int mq_int4_unpack_launch_group(int scale_dtype, FlatTable& tab, hipStream_t st) {
+    if (!flat_grid(tab, 256 * kI4UnpackUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) return MQ_OK;
+    const dim3 grid((unsigned)tab.max_blocks, (unsigned)tab.n), blk(256);
+    if (scale_dtype == MQ_BF16) hipLaunchKernelGGL(int4_unpack_kernel<MQ_BF16>, grid, blk, 0, st, tab);
+    else if (scale_dtype == MQ_F16) hipLaunchKernelGGL(int4_unpack_kernel<MQ_F16>, grid, blk, 0, st, tab);
+    else hipLaunchKernelGGL(int4_unpack_kernel<MQ_F32>, grid, blk, 0, st, tab);
+    return mq_check_launch("int4 unpack");
+}
+
 extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, int scale_dtype, void* y, int64_t M,
                                       int64_t K, int group, void* stream) {
     if ((!packed || !scale || !y) && M != 0 && K != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -925,23 +975,11 @@ extern "C" int mq_int4_unpack_dequant(const int32_t* packed, const void* scale, 
     if (K % group != 0) return mq_fail(MQ_ERR_ARG, "K must be a multiple of the group size");
     if (M == 0 || K == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
-    const int upg = group / 8;
-    if (K % 8 == 0 && group % 8 == 0 && (upg & (upg - 1)) == 0 && ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0) {
-        int shift = 0;
-        while ((1 << shift) < upg) shift++;
-        const int64_t words = M * (K / 8);
-        int64_t blocks = (words + 256 * kI4UnpackUnroll - 1) / (256 * kI4UnpackUnroll);
-        const int chunk = (int)flat_chunk(blocks);
-        blocks = flat_padded(blocks, chunk);
-        if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
-        const dim3 grid((unsigned)blocks), blk(256);
-        if (scale_dtype == MQ_BF16)
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_BF16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
-        else if (scale_dtype == MQ_F16)
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F16>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
-        else
-            hipLaunchKernelGGL(int4_unpack_kernel<MQ_F32>, grid, blk, 0, st, (const uint32_t*)packed, scale, (uint16_t*)y, words, shift, chunk);
-        return mq_check_launch("int4 unpack");
+    if (mq_int4_unpack_fast_ok(packed, y, K, group)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = mq_int4_unpack_entry(packed, scale, y, M, K, group);
+        return mq_int4_unpack_launch_group(scale_dtype, tab, st);
     }
     int64_t blocks = (M * K + 255) / 256;
     if (blocks > mq_grid_cap()) blocks = mq_grid_cap();

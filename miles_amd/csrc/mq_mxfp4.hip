@@ -168,21 +168,36 @@ template <int BYTE>
 __device__ __forceinline__ uint32_t hw_e2m1x2_to_bf16x2(uint32_t word, float factor) {
     return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, factor, BYTE));
 }
-__global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint32_t* __restrict__ packed,
-                                                            const uint8_t* __restrict__ scale,
-                                                            uint16_t* __restrict__ y, int64_t units,
-                                                            int group_shift, int chunk) {
-    const int64_t base = xcd_chunked_block(chunk) * (256 * kM4DqUnroll) + threadIdx.x;
+// One tensor of a launch's table per blockIdx.y: w = packed words, q = bf16 output, s = E8M0 bytes, units = words,
+// section = log2(words per group).
+__global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const FlatTable tab) {
+    const FlatJob job = flat_job(tab);
+    const uint32_t* __restrict__ packed = (const uint32_t*)job.w;
+    const uint8_t* __restrict__ scale = (const uint8_t*)job.s;
+    uint16_t* __restrict__ y = (uint16_t*)job.q;
+    const int64_t units = job.units;
+    const int group_shift = job.section;
+    const int64_t first = flat_block(tab) * (256 * kM4DqUnroll);
+    if (first >= units) return;          // a smaller tensor of the group
+    // everything a lane adds to the workgroup's (uniform) base addresses is a 32-bit offset; `first` is a multiple of
+    // the words of a group (at most 256 per unit of a lane, see mq_mxfp4_dequant_fast_ok)
+    const int64_t left = units - first;
+    const uint32_t rem = left < 256 * kM4DqUnroll ? (uint32_t)left : (uint32_t)(256 * kM4DqUnroll);
+    const uint32_t* __restrict__ packed0 = packed + first;
+    const uint8_t* __restrict__ scale0 = scale + (first >> group_shift);
+    uint16_t* __restrict__ y0 = y + first * 8;
     uint32_t word[kM4DqUnroll], s[kM4DqUnroll];
 #pragma unroll
     for (int i = 0; i < kM4DqUnroll; i++) {
-        const int64_t unit = base + i * 256 < units ? base + i * 256 : units - 1;   // past the end: re-read the last unit
-        word[i] = __builtin_nontemporal_load(packed + unit);
-        s[i] = scale[unit >> group_shift];
+        const uint32_t off = threadIdx.x + i * 256u;
+        const uint32_t unit = off < rem ? off : 0u;       // past the end: re-read the workgroup's first unit
+        word[i] = __builtin_nontemporal_load(packed0 + unit);
+        s[i] = scale0[unit >> group_shift];
     }
+    __builtin_amdgcn_sched_barrier(0);      // (the scheduler keeps the first unit's conversions below the last load)
 #pragma unroll
     for (int i = 0; i < kM4DqUnroll; i++) {
-        const int64_t unit = base + i * 256;
+        const uint32_t off = threadIdx.x + i * 256u;
         u32x4 o;
         if (s[i] >= 2u && s[i] <= 252u) {
             const float factor = u2f(s[i] << 23);
@@ -194,7 +209,7 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint32_t* __re
             for (int j = 0; j < 8; j++) c[j] = mxfp4_decode((word[i] >> (4 * j)) & 0xFu, s[i]);
             o = u32x4{c[0] | (c[1] << 16), c[2] | (c[3] << 16), c[4] | (c[5] << 16), c[6] | (c[7] << 16)};
         }
-        if (unit < units) st16(y + unit * 8, o);
+        if (off < rem) st16(y0 + off * 8u, o);
     }
 }
 __global__ __launch_bounds__(256) void mxfp4_dequant_generic_kernel(const uint8_t* __restrict__ packed,
@@ -341,6 +356,7 @@ __global__ __launch_bounds__(256) void mxfp4_recode_flat_kernel(const RecodeTabl
         s[i] = job.scale[uc >> 1];
         bits[i] = f2u(job.tile_scale[(uint64_t)(row >> 7) * job.tiles_in + (cu >> 3)]);
     }
+    __builtin_amdgcn_sched_barrier(0);      // (the scheduler keeps the first unit's arithmetic below the last load)
 #pragma unroll
     for (int i = 0; i < kRecodeUnroll; i++) {
         const uint32_t u = base + i * 256;
@@ -417,6 +433,25 @@ extern "C" int mq_mxfp4_quant(const void* w, int dtype, uint8_t* packed, uint8_t
     return mq_check_launch("mxfp4 pack");
 }
 
+// the flat kernel takes whole words and groups of a power-of-two number of words
+bool mq_mxfp4_dequant_fast_ok(const void* packed, const void* y, int64_t bytes, int group) {
+    const int upg = group / 8;
+    return group > 0 && group <= 2048 * kM4DqUnroll && group % 8 == 0 && (upg & (upg - 1)) == 0 && bytes % 4 == 0 &&
+           ((uintptr_t)packed % 4) == 0 && ((uintptr_t)y % 16) == 0;
+}
+FlatJob mq_mxfp4_dequant_entry(const void* packed, const void* scale, void* y, int64_t bytes, int group) {
+    int shift = 0;
+    while ((1 << shift) < group / 8) shift++;
+    return FlatJob{packed, y, (void*)scale, nullptr, bytes / 4, nullptr, shift, 0};
+}
+// up to kMaxGroup tensors in one launch
+int mq_mxfp4_dequant_launch_group(FlatTable& tab, hipStream_t st) {
+    if (!flat_grid(tab, 256 * kM4DqUnroll)) return mq_fail(MQ_ERR_ARG, "tensor too large");
+    if (tab.max_blocks == 0) return MQ_OK;
+    hipLaunchKernelGGL(mxfp4_dequant_kernel, dim3((unsigned)tab.max_blocks, (unsigned)tab.n), dim3(256), 0, st, tab);
+    return mq_check_launch("mxfp4 dequant");
+}
+
 extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, void* y, int64_t bytes, int group,
                                 void* stream) {
     if ((!packed || !scale || !y) && bytes != 0) return mq_fail(MQ_ERR_ARG, "null pointer");
@@ -424,19 +459,11 @@ extern "C" int mq_mxfp4_dequant(const uint8_t* packed, const uint8_t* scale, voi
     if ((2 * bytes) % group != 0) return mq_fail(MQ_ERR_ARG, "element count must be a multiple of the group size");
     if (bytes == 0) return MQ_OK;
     hipStream_t st = (hipStream_t)stream;
-    const int upg = group / 8;
-    if (group % 8 == 0 && (upg & (upg - 1)) == 0 && bytes % 4 == 0 && ((uintptr_t)packed % 4) == 0 &&
-        ((uintptr_t)y % 16) == 0) {
-        int shift = 0;
-        while ((1 << shift) < upg) shift++;
-        const int64_t units = bytes / 4;
-        int64_t blocks = (units + 256 * kM4DqUnroll - 1) / (256 * kM4DqUnroll);
-        const int64_t chunk = flat_chunk(blocks);
-        blocks = flat_padded(blocks, chunk);
-        if (blocks > 0x7FFFFFFFll) return mq_fail(MQ_ERR_ARG, "tensor too large");
-        hipLaunchKernelGGL(mxfp4_dequant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)packed, scale,
-                           (uint16_t*)y, units, shift, (int)chunk);
-        return mq_check_launch("mxfp4 dequant");
+    if (mq_mxfp4_dequant_fast_ok(packed, y, bytes, group)) {
+        FlatTable tab{};
+        tab.n = 1;
+        tab.job[0] = mq_mxfp4_dequant_entry(packed, scale, y, bytes, group);
+        return mq_mxfp4_dequant_launch_group(tab, st);
     }
     int64_t blocks = (bytes + 255) / 256;
     if (blocks > mq_grid_cap()) blocks = mq_grid_cap();

@@ -53,6 +53,12 @@ int mq_mxfp4_to_fp8_job(RecodeJob& job, const void* packed, const void* scale, v
 int mq_mxfp4_to_fp8_launch_group(const RecodeTable& tab, hipStream_t st);
 bool mq_fp8_to_mxfp8_fast_ok(const void* x, const void* q, int64_t M, int64_t K);
 int mq_fp8_to_mxfp8_launch_group(const MqRescaleArgs* a, int n, hipStream_t st);
+bool mq_int4_unpack_fast_ok(const void* packed, const void* y, int64_t K, int group);
+FlatJob mq_int4_unpack_entry(const void* packed, const void* scale, void* y, int64_t M, int64_t K, int group);
+int mq_int4_unpack_launch_group(int scale_dtype, FlatTable& tab, hipStream_t st);
+bool mq_mxfp4_dequant_fast_ok(const void* packed, const void* y, int64_t bytes, int group);
+FlatJob mq_mxfp4_dequant_entry(const void* packed, const void* scale, void* y, int64_t bytes, int group);
+int mq_mxfp4_dequant_launch_group(FlatTable& tab, hipStream_t st);
 int mq_copy_launch_group(CopyTable& tab, hipStream_t st);
 int mq_copy_launch_run(const void* src, void* dst, int64_t bytes, hipStream_t st);
 
@@ -92,6 +98,10 @@ static bool job_fast(const mq_job& j) {
             return true;               // check_job has refused what the kernel does not take
         case MQ_JOB_FP8_TO_MXFP8:
             return mq_fp8_to_mxfp8_fast_ok(j.in, j.out, j.rows, j.cols) && j.ld >= (j.cols + 127) / 128 && j.ld <= 0x7FFFFFFF;
+        case MQ_JOB_INT4_UNPACK:
+            return mq_int4_unpack_fast_ok(j.in, j.out, j.cols, j.p0);
+        case MQ_JOB_MXFP4_DEQUANT:
+            return mq_mxfp4_dequant_fast_ok(j.in, j.out, j.rows * j.cols / 2, j.p0);
         default:
             return false;
     }
@@ -99,7 +109,7 @@ static bool job_fast(const mq_job& j) {
 
 static int64_t copy_dst_pitch(const mq_job& j);
 static int check_job(const mq_job& j) {
-    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_E8M0_EXPAND) return mq_fail(MQ_ERR_ARG, "unknown job kind");
+    if (j.kind < MQ_JOB_FP8_BLOCK || j.kind > MQ_JOB_MXFP4_DEQUANT) return mq_fail(MQ_ERR_ARG, "unknown job kind");
     if (j.rows < 0 || j.cols < 0) return mq_fail(MQ_ERR_ARG, "job with a negative shape");
     const bool empty = j.rows == 0 || j.cols == 0;       // an empty tensor has no address
     if ((!j.in || !j.out) && !empty) return mq_fail(MQ_ERR_ARG, "job with a null tensor pointer");
@@ -114,6 +124,14 @@ static int check_job(const mq_job& j) {
         return j.rows_per_block == 0 ? MQ_OK : mq_fail(MQ_ERR_ARG, "bad scale-expansion job");
     if (j.kind == MQ_JOB_FP8_TO_MXFP8 && !empty && (!j.aux || j.rows_per_block != 0))
         return mq_fail(MQ_ERR_ARG, "FP8 to MXFP8 job without tile scales");
+    if (j.kind == MQ_JOB_INT4_UNPACK || j.kind == MQ_JOB_MXFP4_DEQUANT) {
+        // the entry points' own checks, made before anything of the list runs
+        if (j.rows_per_block != 0 || j.p0 <= 0 || (!empty && !j.aux)) return mq_fail(MQ_ERR_ARG, "unpacking job without scales or a group size");
+        if (j.kind == MQ_JOB_INT4_UNPACK && (j.dtype < MQ_BF16 || j.dtype > MQ_F32)) return mq_fail(MQ_ERR_ARG, "bad scale dtype");
+        if (j.kind == MQ_JOB_INT4_UNPACK ? j.cols % j.p0 != 0 : (j.rows * j.cols) % j.p0 != 0 || (j.rows * j.cols) % 2 != 0)
+            return mq_fail(MQ_ERR_ARG, "the element count must be a multiple of the group size");
+        return MQ_OK;
+    }
     if (j.kind == MQ_JOB_MXFP4_TO_FP8) {
         if (j.rows_per_block != 0) return mq_fail(MQ_ERR_ARG, "bad MXFP4 to FP8 job");
         RecodeJob probe;
@@ -164,6 +182,10 @@ static int run_single(const mq_job& j, void* stream) {
             return mq_e8m0_expand_tile_scales(j.in, j.dtype == MQ_F32, j.ld, (uint8_t*)j.out, j.rows, j.cols, stream);
         case MQ_JOB_MXFP4_TO_FP8:
             return mq_mxfp4_to_fp8_block((const uint8_t*)j.in, (const uint8_t*)j.aux, j.out, (float*)j.scale, j.rows, j.cols, stream);
+        case MQ_JOB_INT4_UNPACK:
+            return mq_int4_unpack_dequant((const int32_t*)j.in, j.aux, j.dtype, j.out, j.rows, j.cols, j.p0, stream);
+        case MQ_JOB_MXFP4_DEQUANT:
+            return mq_mxfp4_dequant((const uint8_t*)j.in, (const uint8_t*)j.aux, j.out, j.rows * j.cols / 2, j.p0, stream);
         default:
             return mq_fail(MQ_ERR_ARG, "unknown job kind");
     }
@@ -246,7 +268,7 @@ static bool same_group(const mq_job& a, const mq_job& b) {
     // the quantizer kernels are compiled per 16-bit input dtype; the other kinds' fast paths take one dtype, or any
     // (copies)
     const bool per_dtype = tile_kind(a.kind) || a.kind == MQ_JOB_MXFP8 || a.kind == MQ_JOB_MXFP4 || a.kind == MQ_JOB_INT4_PACK ||
-                           a.kind == MQ_JOB_INT4_PACK_ASYM;
+                           a.kind == MQ_JOB_INT4_PACK_ASYM || a.kind == MQ_JOB_INT4_UNPACK;
     return a.kind == b.kind && a.p0 == b.p0 && a.p1 == b.p1 && (!per_dtype || a.dtype == b.dtype);
 }
 
@@ -581,6 +603,20 @@ extern "C" int mq_run_jobs_tabled(const mq_job* jobs, int64_t n, const void* dev
                     a[t] = MqRescaleArgs{jb.in, (const float*)jb.aux, jb.out, (uint8_t*)jb.scale, jb.rows, jb.cols, jb.ld};
                 }
                 rc = mq_fp8_to_mxfp8_launch_group(a, cnt, st);
+                break;
+            }
+            case MQ_JOB_INT4_UNPACK:
+            case MQ_JOB_MXFP4_DEQUANT: {
+                FlatTable tab{};
+                tab.n = cnt;
+                for (int t = 0; t < cnt; t++) {
+                    const mq_job& jb = jobs[i + t];
+                    tab.job[t] = head.kind == MQ_JOB_INT4_UNPACK
+                                     ? mq_int4_unpack_entry(jb.in, jb.aux, jb.out, jb.rows, jb.cols, jb.p0)
+                                     : mq_mxfp4_dequant_entry(jb.in, jb.aux, jb.out, jb.rows * jb.cols / 2, jb.p0);
+                }
+                rc = head.kind == MQ_JOB_INT4_UNPACK ? mq_int4_unpack_launch_group(head.dtype, tab, st)
+                                                     : mq_mxfp4_dequant_launch_group(tab, st);
                 break;
             }
             case MQ_JOB_MXFP4_TO_FP8: {

@@ -294,9 +294,10 @@ def note_constant(t: torch.Tensor) -> None:
 
 
 def submit(kind, inp: torch.Tensor, out: torch.Tensor, scale, aux, aux2, rows, cols, ld, p0=0, p1=0,
-           rows_per_block=0, block_stride=0) -> None:
-    """Run (or record) one job.  Tensor arguments may be None where the job kind has no such operand."""
-    rec = (kind, _lib.DTYPE_CODE.get(inp.dtype, 0), inp.data_ptr(), out.data_ptr(),
+           rows_per_block=0, block_stride=0, dtype=None) -> None:
+    """Run (or record) one job.  Tensor arguments may be None where the job kind has no such operand; `dtype` is the
+    job's dtype code where that is not the input tensor's (the scales' dtype of an INT4 unpacking job)."""
+    rec = (kind, _lib.DTYPE_CODE.get(inp.dtype, 0) if dtype is None else dtype, inp.data_ptr(), out.data_ptr(),
            scale.data_ptr() if scale is not None else None, aux.data_ptr() if aux is not None else None,
            aux2.data_ptr() if aux2 is not None else None, rows, cols, ld, p0, p1, rows_per_block, block_stride)
     keep = [t for t in (inp, out, scale, aux, aux2) if t is not None]

@@ -53,10 +53,9 @@ def _dequantize_tensor(weight_packed: torch.Tensor, weight_scale: torch.Tensor, 
     if K % group_size != 0 or scale.numel() != M * (K // group_size):
         raise ValueError(f"Scale shape {tuple(scale.shape)} incompatible with weight shape {shape}")
     out = torch.empty((M, K), dtype=torch.bfloat16, device=packed.device)
-    launch.note_direct_call()
-    rc = _lib.load().mq_int4_unpack_dequant(packed.data_ptr(), scale.data_ptr(), _lib.dtype_code(scale, "_dequantize_tensor"),
-                                            out.data_ptr(), M, K, int(group_size), _lib.stream_ptr(packed.device))
-    _lib.check(rc)
+    # a job of the batched driver: inside `launch.deferred()` the experts of a whole shard share grouped launches
+    launch.submit(_lib.JOB_INT4_UNPACK, packed, out, None, scale, None, M, K, K, int(group_size),
+                  dtype=_lib.dtype_code(scale, "_dequantize_tensor"))
     return out
 
 
@@ -87,13 +86,14 @@ def convert_file(input_path: str, output_path: str, group_size: int, skip_existi
             else:
                 module = (key[: member.start("proj") - 1], member["proj"])        # (expert prefix, projection)
                 fields_of.setdefault(module, {})[member["field"]] = shard.get_tensor(key)
-    for (expert, proj), fields in fields_of.items():
-        if len(fields) < len(_FIELDS):
-            carried.update({f"{expert}.{proj}.{field}": value for field, value in fields.items()})
-            continue
-        carried[f"{expert}.{proj}.weight"] = _dequantize_tensor(fields["weight_packed"].to(torch.int32),
-                                                                fields["weight_scale"].to(torch.float32),
-                                                                fields["weight_shape"], group_size)
+    with launch.deferred():         # the shard's projections are unpacked together when the block ends
+        for (expert, proj), fields in fields_of.items():
+            if len(fields) < len(_FIELDS):
+                carried.update({f"{expert}.{proj}.{field}": value for field, value in fields.items()})
+                continue
+            carried[f"{expert}.{proj}.weight"] = _dequantize_tensor(fields["weight_packed"].to(torch.int32),
+                                                                    fields["weight_scale"].to(torch.float32),
+                                                                    fields["weight_shape"], group_size)
     os.makedirs(os.path.dirname(output_path), exist_ok=True)
     save_file({name: t.cpu().contiguous() for name, t in carried.items()}, output_path)
 

@@ -21,6 +21,7 @@ from pathlib import Path
 
 from safetensors.torch import safe_open, save_file
 
+from miles_amd import launch
 from miles_amd.utils.mxfp4 import dequantize_mxfp4
 
 PACKED, SCALE = ".weight_packed", ".weight_scale"
@@ -65,11 +66,14 @@ class Mxfp4Checkpoint:
             names = set(shard.keys())
             stems = sorted(n[: -len(PACKED)] for n in names if n.endswith(PACKED))
             scales = {n for n in names if n.endswith(SCALE)}
+            with launch.deferred():         # the shard's tensors are unpacked together when the block ends
+                for stem in stems:
+                    assert stem + SCALE in scales, f"Missing scale for {stem + PACKED}"
+                    scales.discard(stem + SCALE)
+                    codes, exponents = shard.get_tensor(stem + PACKED), shard.get_tensor(stem + SCALE)
+                    out[stem + ".weight"] = dequantize_mxfp4(codes.to(self.device), exponents.to(self.device), self.group_size)
             for stem in stems:
-                assert stem + SCALE in scales, f"Missing scale for {stem + PACKED}"
-                scales.discard(stem + SCALE)
-                codes, exponents = shard.get_tensor(stem + PACKED), shard.get_tensor(stem + SCALE)
-                out[stem + ".weight"] = dequantize_mxfp4(codes.to(self.device), exponents.to(self.device), self.group_size).cpu()
+                out[stem + ".weight"] = out[stem + ".weight"].cpu()
             assert not scales, f"Orphan MXFP4 scales in {name}: {sorted(scales)}"
             consumed = {stem + suffix for stem in stems for suffix in (PACKED, SCALE)}
             for other in sorted(names - consumed):

@@ -43,8 +43,7 @@ def dequantize_mxfp4(weight_packed: torch.Tensor, weight_scale: torch.Tensor, gr
     assert numel % group_size == 0
     assert scale.numel() == numel // group_size
     out = torch.empty((*packed.shape[:-1], packed.shape[-1] * 2), dtype=torch.bfloat16, device=packed.device)
-    launch.note_direct_call()
-    rc = _lib.load().mq_mxfp4_dequant(packed.data_ptr(), scale.data_ptr(), out.data_ptr(), packed.numel(),
-                                      int(group_size), _lib.stream_ptr(packed.device))
-    _lib.check(rc)
+    # a job of the batched driver: inside `launch.deferred()` the tensors of a whole shard share grouped launches
+    if numel:
+        launch.submit(_lib.JOB_MXFP4_DEQUANT, packed, out, None, scale, None, 1, numel, numel, int(group_size))
     return out

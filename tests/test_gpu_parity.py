@@ -667,6 +667,12 @@ def test_int4_unpack_dequant(oracle, shape, G, sdt):
         flat[0], flat[1], flat[2] = float("nan"), float("inf"), float("-inf")
         if sdt == torch.bfloat16:
             flat.view(torch.int16)[3] = -42        # a NaN with a sign and a payload
+    if flat.numel() >= 16:
+        # zero, negative and tiny scales (the sign of a zero product is the product's), and the largest finite ones
+        big = {torch.bfloat16: 3.0e38, torch.float16: 65504.0, torch.float32: 3.0e38}[sdt]
+        tiny = {torch.bfloat16: 1e-40, torch.float16: 6e-8, torch.float32: 1e-44}[sdt]
+        for at, v in enumerate((0.0, -0.0, -1.5, tiny, -tiny, big, -big, big / 4, big / 16, big / 32), start=4):
+            flat[at] = v
     got = _dequantize_tensor(packed.to(DEV), scale.to(DEV), torch.tensor(shape, dtype=torch.int32), G)
     want = oracle.int4_unpack_dequant(packed, scale, shape, G)
     assert got.dtype == torch.bfloat16
@@ -918,6 +924,62 @@ def test_mxfp4_to_fp8_recode_grouped(oracle):
         y_o, ts_o = oracle.cast_e2m1fn_to_e4m3fn(p, s)
         _assert_same(ts, ts_o, "tile scales (grouped, unaligned scales)")
         _assert_same(y, y_o, "e4m3 codes (grouped, unaligned scales)")
+
+
+def test_unpacking_jobs_grouped(oracle):
+    """A shard's INT4 experts unpacked, and its MXFP4 tensors dequantized, inside `launch.deferred()`: tensors of
+    different sizes share grouped launches (the largest sets the grid, a one-row tensor rides along); a tensor the flat
+    kernel does not take (a group that is no power-of-two number of words, scales of another dtype) goes out on its
+    own; values as from single calls, which are checked against the oracle."""
+    from miles_amd import launch
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4
+
+    g = torch.Generator().manual_seed(47)
+    cases = [((256, 512), 128, torch.bfloat16), ((1, 128), 128, torch.bfloat16), ((2048, 7168), 128, torch.bfloat16),
+             ((7168, 2048), 128, torch.bfloat16), ((3, 100), 20, torch.bfloat16), ((64, 256), 128, torch.float32),
+             ((64, 256), 32, torch.bfloat16), ((512, 1024), 128, torch.bfloat16)]
+    ins = []
+    for (m, k), G, sdt in cases:
+        packed = torch.randint(-2**31, 2**31 - 1, (m, -(-k // 8)), dtype=torch.int64, generator=g).to(torch.int32)
+        ins.append((packed, torch.exp(torch.randn((m, k // G), generator=g) * 3).to(sdt), (m, k), G))
+    dev = [(p.to(DEV), s.to(DEV), shape, G) for p, s, shape, G in ins]
+    with launch.deferred() as batch:
+        outs = [_dequantize_tensor(*args) for args in dev]
+    assert len(batch) == len(cases) and batch.direct_calls == 0
+    for (p, s, shape, G), got in zip(ins, outs):
+        _assert_same(got, oracle.int4_unpack_dequant(p, s, shape, G), f"INT4 unpack (grouped) {shape} group {G}")
+
+    m4 = []
+    for shape, G in (((256, 512), 32), ((1, 32), 32), ((2048, 7168), 32), ((7168, 2048), 32), ((16, 48), 16),
+                     ((8, 64), 2), ((512, 1024), 32)):
+        packed = torch.randint(0, 256, (shape[0], shape[1] // 2), dtype=torch.uint8, generator=g)
+        scale = torch.randint(0, 256, (shape[0] * shape[1] // G,), dtype=torch.int32, generator=g).to(torch.uint8)
+        m4.append((packed, scale, G))
+    with launch.deferred() as batch:
+        outs = [dequantize_mxfp4(p.to(DEV), s.to(DEV), G) for p, s, G in m4]
+    assert len(batch) == len(m4) and batch.direct_calls == 0
+    for (p, s, G), got in zip(m4, outs):
+        _assert_same(got, oracle.dequantize_mxfp4(p, s, G), f"MXFP4 dequantize (grouped) {tuple(p.shape)} group {G}")
+
+
+def test_unpacking_job_argument_checks(lib):
+    from miles_amd import _lib
+
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
+    def job(kind, rows, cols, group, dtype=0, aux=True):
+        return (_lib.Job * 1)(_lib.Job(kind, dtype, buf.data_ptr(), buf.data_ptr() + 32768, None,
+                                       buf.data_ptr() + 16384 if aux else None, None, rows, cols, cols, group, 0, 0, 0))
+    for kind in (_lib.JOB_INT4_UNPACK, _lib.JOB_MXFP4_DEQUANT):
+        assert lib.mq_run_jobs(job(kind, 8, 128, 32), 1, None) == 0
+        assert lib.mq_run_jobs(job(kind, 0, 128, 32, aux=False), 1, None) == 0     # an empty tensor has no address
+        assert lib.mq_run_jobs(job(kind, 8, 128, 0), 1, None) != 0                 # no group size
+        assert lib.mq_run_jobs(job(kind, 8, 128, 32, aux=False), 1, None) != 0     # no scales
+        assert b"unpacking job" in lib.mq_last_error()
+    assert lib.mq_run_jobs(job(_lib.JOB_INT4_UNPACK, 8, 100, 32), 1, None) != 0    # K not a multiple of the group
+    assert lib.mq_run_jobs(job(_lib.JOB_INT4_UNPACK, 8, 128, 32, dtype=3), 1, None) != 0
+    assert lib.mq_run_jobs(job(_lib.JOB_MXFP4_DEQUANT, 3, 11, 32), 1, None) != 0   # 33 elements
+    torch.cuda.synchronize()
 
 
 def test_mxfp4_to_fp8_job_argument_checks(lib):
