@@ -452,8 +452,10 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 // 1 KiB of consecutive output per store instruction.  Row and column of a unit come from a multiply-high
 // division by the row length (exact for every 32-bit unit index), not from an integer divide.
 constexpr int kDqThreads = 256;
+// (units per lane, alternating runs, one / two / four: 6.53-6.57 / 6.47-6.50 / 6.23-6.27 TB/s on 96 DeepSeek-V3 expert
+// matrices, 6.21-6.23 / 6.17-6.22 / 6.11-6.14 on eight [16384, 7168] tensors)
 #ifndef MQ_DQ_UNROLL
-#define MQ_DQ_UNROLL 2
+#define MQ_DQ_UNROLL 1
 #endif
 constexpr int kDqUnroll = MQ_DQ_UNROLL;
 struct DequantJob {
