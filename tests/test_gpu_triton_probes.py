@@ -305,3 +305,91 @@ def test_triton_dequantizer_gives_the_hip_kernels_bytes(oracle):
     differ = int((t.view(torch.int16)[~nan] != h.view(torch.int16)[~nan]).sum())
     print("TRITON_DEQUANTIZER", json.dumps({"elements": rows * cols, "nan_elements": int(nan.sum()), "values_differ": differ}))
     assert differ == 0
+
+
+@pytest.mark.parametrize("kind", ["fp8", "fp4", "compressed_kv"])
+def test_triton_fake_quantizers_give_the_hip_kernels_values(oracle, kind):
+    """The training-forward fake quantizers of the reference are one Triton kernel (miles/kernels/quant/fake_quant.py:
+    24-61): per group of 32 (16 for the compressed-KV form) the largest magnitude, a scale -- a power of two from the
+    bits of `amax / fmax`, or an e4m3 value -- a division by it (`/`, or `div_rn`), a clamp, a rounding to the e4m3 or
+    e2m1 grid (a cast, or `rint` of magnitude over step) and the product with the scale, stored in the input's dtype.  A
+    probe written for this test from those expressions against the HIP kernel on bf16, fp16 and fp32 data over many
+    binades: what Triton makes of the casts, `div_rn`, the maxima and the rounding to an integer on this GPU.  Triton
+    3.6.0's ROCm `libdevice` has no `rint` (the reference's own kernel does not compile with it in the two e2m1 modes); the
+    probe then takes `nearbyint`, the same function of its argument (nearest integer, ties to even)."""
+    from miles_amd.kernels.quant import fake_quant as fq
+
+    try:
+        import triton
+        import triton.language as tl
+        from triton.language.extra import libdevice
+    except Exception as exc:              # pragma: no cover - depends on the image
+        pytest.skip(f"triton is not importable: {exc!r}")
+
+    import triton.language.extra.hip.libdevice as rocm_libdevice
+    to_integer = libdevice.rint if hasattr(rocm_libdevice, "rint") else libdevice.nearbyint
+
+    @triton.jit
+    def group_round_trip(src, dst, groups, TOP: tl.constexpr, FLOOR: tl.constexpr, GRID4: tl.constexpr,
+                         BYTE_SCALE: tl.constexpr, WIDTH: tl.constexpr, TALL: tl.constexpr):
+        g = tl.program_id(0) * TALL + tl.arange(0, TALL)
+        at = g[:, None] * WIDTH + tl.arange(0, WIDTH)[None, :]
+        live = (g < groups)[:, None]
+        v = tl.load(src + at, mask=live, other=0.0).to(tl.float32)
+        top = tl.max(tl.abs(v), axis=1)
+        if BYTE_SCALE:
+            s = tl.minimum(tl.maximum(top * (1.0 / TOP), FLOOR), 448.0).to(tl.float8e4nv).to(tl.float32)
+            w = tl.div_rn(v, s[:, None])
+        else:
+            bits = (tl.maximum(top, FLOOR) * (1.0 / TOP)).to(tl.int32, bitcast=True)
+            e = ((bits >> 23) & 0xFF) + ((bits & 0x7FFFFF) != 0).to(tl.int32)
+            s = (e << 23).to(tl.float32, bitcast=True)
+            w = v / s[:, None]
+        w = tl.minimum(tl.maximum(w, -TOP), TOP)
+        if GRID4:
+            m = tl.abs(w)
+            step = tl.where(m < 2.0, 0.5, tl.where(m < 4.0, 1.0, 2.0))
+            r = to_integer(m / step) * step * tl.where(w > 0, 1.0, tl.where(w < 0, -1.0, 0.0))
+        else:
+            r = w.to(tl.float8e4nv).to(tl.float32)
+        tl.store(dst + at, (r * s[:, None]).to(dst.dtype.element_ty), mask=live)
+
+    width = 16 if kind == "compressed_kv" else 32
+    top, floor = {"fp8": (448.0, 1e-4), "fp4": (6.0, 6 * 2.0 ** -126), "compressed_kv": (6.0, 2.0 ** -9)}[kind]
+    hip_fn = {"fp8": fq.fake_quant_fp8_forward, "fp4": fq.fake_quant_fp4_forward,
+              "compressed_kv": fq.fake_quant_compressed_kv_forward}[kind]
+    g = torch.Generator().manual_seed(23)
+    report = {}
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        groups = 40_000
+        x = torch.randn((groups, width), generator=g) * torch.exp(torch.randn((groups, 1), generator=g) * 6)
+        x[:64] = 0.0                                              # all-zero groups
+        x[64:128] *= 1e-30                                        # far below every floor
+        x[128:192, ::3] = 0.0
+        x[192:256] = torch.round(x[192:256] * 4) / 4              # ties of the e2m1 grid
+        if dtype == torch.float16:
+            x = x.clamp(-6e4, 6e4)
+        x = x.to(dtype)
+        xd = x.to(DEV)
+        out = torch.empty_like(xd)
+        try:
+            group_round_trip[(triton.cdiv(groups, 64),)](xd, out, groups, TOP=top, FLOOR=floor, GRID4=kind != "fp8",
+                                                         BYTE_SCALE=kind == "compressed_kv", WIDTH=width, TALL=64)
+            torch.cuda.synchronize()
+        except Exception as exc:              # pragma: no cover - depends on the image
+            pytest.skip(f"triton could not compile or launch on this GPU: {type(exc).__name__}: {str(exc)[:200]}")
+        hip = hip_fn(xd).cpu()
+        want = oracle.fake_quant(x, kind)
+        bits = {torch.bfloat16: torch.int16, torch.float16: torch.int16, torch.float32: torch.int32}[dtype]
+        assert torch.equal(hip.view(bits), want.view(bits)), f"{dtype}: the HIP kernel differs from the oracle"
+        t = out.cpu()
+        differ = t.view(bits) != hip.view(bits)
+        # (+0 and -0 count as one value: the reference multiplies by an explicit sign, the probe with it)
+        differ &= ~((t == 0) & (hip == 0))
+        report[str(dtype)] = {"elements": x.numel(), "values_differ": int(differ.sum())}
+    print("TRITON_FAKE_QUANT", kind, json.dumps(report))
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, f"triton_fake_quant_{kind}.json"), "w") as f:
+            json.dump(report, f)
+    assert all(v["values_differ"] == 0 for v in report.values()), report
