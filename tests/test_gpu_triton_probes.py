@@ -11,7 +11,7 @@ A second probe is a whole 128 x 128 tile quantizer written for this file from th
 eps, the two divisions, clamp of the product, cast to e4m3): its bytes are compared with the HIP kernel's on finite data,
 on tiles holding infinities and NaN, and on one Qwen3-4B layer at full size.
 
-The counts are printed and written to gpurun_out/*.json when that folder exists.  Every test is skipped, with the reason,
+The counts are printed (and written to the directory MQ_PROBE_REPORT_DIR names, if any).  Every test is skipped, with the reason,
 where Triton cannot compile for the GPU.
 """
 
@@ -24,7 +24,14 @@ import torch
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _keep_report(name, report):
+    """The counts also go to a file when MQ_PROBE_REPORT_DIR names a directory."""
+    out_dir = os.environ.get("MQ_PROBE_REPORT_DIR")
+    if out_dir and os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, name), "w") as f:
+            json.dump(report, f, indent=1)
 
 
 def _tile_maxima():
@@ -120,10 +127,7 @@ def test_triton_division_against_ieee(oracle):
             total += x.numel()
         report[form]["codes_changed_of_sampled_inputs"] = [changed, total]
     print("TRITON_DIVISION", json.dumps(report))
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "triton_division.json"), "w") as f:
-            json.dump(report, f, indent=1)
+    _keep_report("triton_division.json", report)
     for form in results:
         assert report[form]["x_s_max_ulp"] <= 1 and report[form]["s_inv_max_ulp"] <= 2, report
 
@@ -202,10 +206,7 @@ def test_triton_tile_quantizer_gives_the_hip_kernels_bytes(oracle):
         report[what] = {"codes_differ": codes, "scales_differ": scales, "elements": x.numel()}
         assert torch.equal(hy.cpu().view(torch.uint8), oy.view(torch.uint8)) and torch.equal(hs.cpu().view(torch.int32), os_.view(torch.int32)), what
     print("TRITON_TILE_QUANTIZER", json.dumps(report))
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "triton_tile_quantizer.json"), "w") as f:
-            json.dump(report, f, indent=1)
+    _keep_report("triton_tile_quantizer.json", report)
     assert all(v["codes_differ"] == 0 and v["scales_differ"] == 0 for v in report.values()), report
 
 
@@ -233,10 +234,7 @@ def test_triton_tile_quantizer_on_non_finite_inputs():
         report[what] = {"codes_differ": int((fold(ty[:, cols]) != fold(hy[:, cols])).sum()),
                         "scale_triton": ts[0, j].item(), "scale_hip": hs[0, j].item()}
     print("TRITON_TILE_NONFINITE", json.dumps(report))
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, "triton_tile_nonfinite.json"), "w") as f:
-            json.dump(report, f, indent=1)
+    _keep_report("triton_tile_nonfinite.json", report)
     for what, r in report.items():
         assert r["codes_differ"] == 0 and (r["scale_triton"] == r["scale_hip"]), (what, r)
 
@@ -388,8 +386,5 @@ def test_triton_fake_quantizers_give_the_hip_kernels_values(oracle, kind):
         differ &= ~((t == 0) & (hip == 0))
         report[str(dtype)] = {"elements": x.numel(), "values_differ": int(differ.sum())}
     print("TRITON_FAKE_QUANT", kind, json.dumps(report))
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
-        with open(os.path.join(out_dir, f"triton_fake_quant_{kind}.json"), "w") as f:
-            json.dump(report, f)
+    _keep_report(f"triton_fake_quant_{kind}.json", report)
     assert all(v["values_differ"] == 0 for v in report.values()), report
