@@ -287,11 +287,13 @@ def full_configs(gen):
         torch.cuda.synchronize()
         first_s = time.perf_counter() - t0
         assert upd._plan is not None and upd._plan.replayable, key
-        for _ in range(3):
+        # untimed syncs until the GPU is out of its idle clocks (the first sync after a pause runs 10 % longer)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.2:
             upd.update_weights()
-        torch.cuda.synchronize()
+            torch.cuda.synchronize()
         seen.update(buckets=0, tensors=0)
-        steps = 5
+        steps = 10
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
@@ -337,9 +339,8 @@ def full_model_block_fp8(weights, elems):
 
 
 def adjacent_formats(gen):
-    """GB/s of the kernels either side of the path (MXFP4 pack / unpack, INT4 unpack, asymmetric INT4 pack).
-    The unpackers are single-tensor entry points, so they are timed as direct calls on eight [16384, 7168] tensors:
-    long enough launches that the GPU, not the host, sets the pace; the packers and the re-coder are job lists."""
+    """GB/s of the kernels either side of the path (MXFP4 pack / unpack, INT4 unpack, asymmetric INT4 pack, the two
+    re-coders) on eight [16384, 7168] tensors, each as one job list: the way the converters submit a shard."""
     from miles_amd.kernels.quant.int4_fake import pack_layer
     from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
     from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4

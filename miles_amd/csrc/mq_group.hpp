@@ -112,18 +112,22 @@ struct FlatTable {
 // workgroup works on is remapped so that an XCD takes runs of `chunk` consecutive blocks (up to MQ_FLAT_CHUNK,
 // 512 KiB of bf16 input at two units per lane) instead of every eighth one.  Measured on MI355X with chunks of
 // up to 64: MXFP4 quantize 6.42 -> 6.75 TB/s, MXFP8 on [768,2048] experts 6.20 -> 6.35, INT4 pack 6.40 -> 6.48.
-// The grid is padded to a whole number of 8 * chunk workgroups (surplus ones exit); the chunk is the largest power
-// of two whose padding stays under 3 %.
+// The grid is padded to a whole number of 8 * chunk workgroups (surplus ones exit); the chunk is the largest of
+// 1, 2, 3, 4, 6, 8, ... 48, 64 whose padding stays under 3 %.
 #ifndef MQ_FLAT_CHUNK
 #define MQ_FLAT_CHUNK 64
 #endif
-// (`chunk` is a power of two everywhere -- flat_chunk only makes such -- so the division is a shift: a division by a
-// run-time value costs every wavefront some forty dependent scalar instructions before its first load; the shift
-// measured 0.5 to 3 % faster on every flat kernel)
+// `chunk` is a power of two or three times one (flat_chunk makes no other), so the division is a shift, or a shift and
+// the multiply-high division by three, which is exact for every 32-bit value: a division by a run-time value costs every
+// wavefront some forty dependent scalar instructions before its first load (the shift measured 0.5 to 3 % faster on every
+// flat kernel).  The threefold chunks matter for tensors such as the [768, 2048] experts of Qwen3-30B-A3B: 384
+// workgroups, which a power of two above 16 would pad by a third, split into runs of 48 exactly (MXFP8 6.49 -> 6.8 TB/s).
 __device__ __forceinline__ int64_t xcd_chunked_block(int32_t chunk) {
     const int32_t bid = blockIdx.x, x = bid % kXcds, k = bid / kXcds;
     const int32_t shift = __builtin_ctz((uint32_t)chunk);
-    return ((int64_t)((k >> shift) * kXcds + x) << shift) + (k & (chunk - 1));
+    const uint32_t shifted = (uint32_t)k >> shift;
+    const uint32_t run = (chunk >> shift) == 3 ? __umulhi(shifted, 0xAAAAAAABu) >> 1 : shifted;      // k / chunk
+    return (int64_t)(run * kXcds + x) * chunk + (k - (int32_t)run * chunk);
 }
 // The same descriptors kept in device memory by a caller that submits one job list again and again: a launch is then not
 // bound to the kMaxGroup tensors that fit the kernel arguments.  A model of thousands of small tensors (MoE experts of
@@ -153,10 +157,11 @@ __device__ __forceinline__ FlatJob flat_job(const Table& tab) {
 }
 template <class Table>
 __device__ __forceinline__ int64_t flat_block(const Table& tab) { return xcd_chunked_block(tab.chunk); }
-// largest power-of-two chunk (up to MQ_FLAT_CHUNK) whose grid padding stays under 3 % of `blocks` workgroups
+// largest chunk of the form 2^a or 3 * 2^a (up to MQ_FLAT_CHUNK) whose grid padding stays under 3 % of `blocks` workgroups
 inline int64_t flat_chunk(int64_t blocks) {
     int64_t chunk = 1;
-    for (int64_t c = 2; c <= MQ_FLAT_CHUNK; c *= 2) {
+    for (int64_t c : {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64}) {
+        if (c > MQ_FLAT_CHUNK) break;
         const int64_t padded = (blocks + c * kXcds - 1) / (c * kXcds) * (c * kXcds);
         if ((padded - blocks) * 32 <= blocks) chunk = c;
     }
