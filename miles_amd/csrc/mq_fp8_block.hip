@@ -448,8 +448,8 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 
 // ---- dequant ----------------------------------------------------------------------------------
 // Fast path: N % 8 == 0, block a power of two >= 8, aligned pointers.  The tensor is a flat run of 8-code
-// units; each lane turns kDqUnroll units (8-byte loads) into bf16 (16-byte stores), so a wavefront writes
-// 1 KiB of consecutive output per store instruction.  Row and column of a unit come from a multiply-high
+// units; each lane turns kDqUnroll units (8-byte loads, kDqThreads units apart) into bf16 (16-byte stores), so a
+// wavefront writes 1 KiB of consecutive output per store instruction.  Row and column of a unit come from a multiply-high
 // division by the row length (exact for every 32-bit unit index), not from an integer divide.
 constexpr int kDqThreads = 256;
 // (units per lane, alternating runs, one / two / four: 6.53-6.57 / 6.47-6.50 / 6.23-6.27 TB/s on 96 DeepSeek-V3 expert
