@@ -427,6 +427,28 @@ def test_sync_plan_matches_quick_and_full_forms():
     assert not plan.matches(weights)
 
 
+def test_sync_plan_identity_test_leaves_the_collector_alone():
+    """The quick form runs once per sync over every parameter.  It must not hold thousands of freshly made container
+    objects (one `torch.Size` per tensor) at a time: that many allocations between two collections make Python's
+    collector run, and its full collection over the objects of a large plan stalls the sync for tens of milliseconds."""
+    import gc
+
+    from miles_amd.weight_update.sync_plan import SyncPlan, weights_signature
+
+    weights = {f"p{i}": torch.zeros(2, 3) for i in range(6000)}
+    plan = SyncPlan(batch=None, buckets=[], jobs_done_at_bucket=[], signature=weights_signature(weights), replayable=True)
+    plan.remember(weights)
+    gc.collect()
+    gc.disable()
+    try:
+        before = gc.get_count()[0]
+        assert plan.matches(weights)
+        grown = gc.get_count()[0] - before
+    finally:
+        gc.enable()
+    assert grown < 100, f"{grown} container allocations outlived their use in one identity test"
+
+
 def test_sync_plan_tops_up_small_trailing_launches_only():
     from miles_amd import _lib, launch
     from miles_amd.weight_update.sync_plan import SyncPlan
