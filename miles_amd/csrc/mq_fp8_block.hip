@@ -322,11 +322,12 @@ __global__ __launch_bounds__(256) void fp8_row_quant_kernel(const void* __restri
 template <int ROWLANES, int F16>
 __global__ __launch_bounds__(256) void fp8_channel_bf16_kernel(const uint16_t* __restrict__ w, int64_t ldw, int64_t K,
                                                                int64_t M, float floor_v, uint8_t* __restrict__ q,
-                                                               float* __restrict__ scale) {
+                                                               float* __restrict__ scale, int chunk) {
     __shared__ uint32_t wave_amax[4];
     constexpr int kRows = 256 / ROWLANES, kMaxUnits = 8;
     const int t = threadIdx.x, lane = t % ROWLANES;
-    const int64_t row = (int64_t)blockIdx.x * kRows + t / ROWLANES;
+    // an XCD takes runs of consecutive rows, as the flat kernels take runs of consecutive blocks
+    const int64_t row = xcd_chunked_block(chunk) * kRows + t / ROWLANES;
     const int64_t units = K / 8;
     const bool row_ok = row < M;
     const uint16_t* __restrict__ src = w + (row_ok ? row : M - 1) * ldw;
@@ -661,13 +662,16 @@ static int fp8_scaled_quant(const void* w, int dtype, int64_t ldw, void* q, floa
     const bool aligned = aligned16 && dtype == MQ_BF16;
     if (aligned16 && per_channel && K / 8 <= 2048) {
         const uint16_t* wi = (const uint16_t*)w;
-        const dim3 narrow((unsigned)((M + 3) / 4)), wide((unsigned)M), blk(256);
+        const bool four_rows = K / 8 <= 256;
+        const int64_t blocks = four_rows ? (M + 3) / 4 : M;
+        const int chunk = (int)flat_chunk(blocks);
+        const dim3 grid((unsigned)flat_padded(blocks, chunk)), blk(256);
         if (dtype == MQ_F16) {
-            if (K / 8 <= 256) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 1>), narrow, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
-            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 1>), wide, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+            if (four_rows) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 1>), grid, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale, chunk);
+            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 1>), grid, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale, chunk);
         } else {
-            if (K / 8 <= 256) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 0>), narrow, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
-            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 0>), wide, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale);
+            if (four_rows) hipLaunchKernelGGL((fp8_channel_bf16_kernel<64, 0>), grid, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale, chunk);
+            else hipLaunchKernelGGL((fp8_channel_bf16_kernel<256, 0>), grid, blk, 0, st, wi, ldw, K, M, floor_in_dtype, (uint8_t*)q, scale, chunk);
         }
         return mq_check_launch("fp8 scaled quant");
     }
