@@ -438,7 +438,7 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             const uint32_t off = (uint32_t)t + i * kNvThreads;
-            stage[off] = off < rem ? in[r][i] : u32x4{0u, 0u, 0u, 0u};
+            stage[off] = in[r][i];      // (a unit past the end holds the workgroup's first unit: real data, nothing new to any maximum)
         }
         // A wavefront reads back only what its own lanes wrote, and the LDS serves one wavefront's accesses in the order
         // it issued them: no workgroup barrier, only the compiler is told not to move the reads above the writes.
