@@ -30,8 +30,9 @@ extern "C" {
 #define MQ_NVFP4_SECTIONS 4
 #define MQ_NVFP4_RECORD_WORDS (MQ_NVFP4_SECTION_WORDS * (MQ_NVFP4_SECTIONS + 1))
 /* words of an amax record behind its sections: the folded amax (float bits), three scale factors derived from it,
- * then two state words of the carried-over amax (see MQ_NVFP4_CARRY_AMAX): REDO is 1 when the last carried submission
- * quantized the tensor in its second pass, VOLATILE is 1 when the amax moved on the last carried submission */
+ * then the state words of the carried-over amax (see MQ_NVFP4_CARRY_AMAX): REDO is 1 when the last carried submission
+ * quantized the tensor in its second pass, VOLATILE is 1 when the amax moved on the last two carried submissions (the
+ * word behind it counts them) */
 #define MQ_NVFP4_RECORD_AMAX_WORD (MQ_NVFP4_SECTION_WORDS * MQ_NVFP4_SECTIONS)
 #define MQ_NVFP4_RECORD_REDO_WORD (MQ_NVFP4_RECORD_AMAX_WORD + 4)
 #define MQ_NVFP4_RECORD_VOLATILE_WORD (MQ_NVFP4_RECORD_AMAX_WORD + 5)
@@ -276,10 +277,10 @@ int mq_nvfp4_qdq(const void* x, int dtype, const float* amax, void* y, int64_t n
  * same job list again, amax records included and untouched in between, after at least one submission without the
  * flag, may set it on bf16 or fp16 jobs.  The driver then quantizes in ONE pass with the amax and scales the record still holds from the last
  * submission, collects the new amax on the way, and quantizes a tensor a second time only if its amax changed
- * (results are identical either way; a weight tensor's amax rarely moves between two syncs).  A tensor whose amax did
- * change is marked volatile in its record: on the next submission the single pass only collects its amax and the
- * second pass quantizes it (what the plain two-pass form costs), and it returns to the single pass once its amax
- * has stayed the same for one submission. */
+ * (results are identical either way; a weight tensor's amax rarely moves between two syncs).  A tensor whose amax
+ * changed on two submissions in a row is marked volatile in its record: on the next submission the single pass only
+ * collects its amax and the second pass quantizes it (what the plain two-pass form costs), and it returns to the
+ * single pass once its amax has stayed the same for one submission. */
 enum {
     MQ_JOB_FP8_BLOCK = 0,
     MQ_JOB_FP8_BLOCKWISE_CAST = 1,

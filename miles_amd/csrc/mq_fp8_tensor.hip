@@ -34,15 +34,15 @@ __global__ __launch_bounds__(256) void fp8_tensor_fold_kernel(const Table tab, f
     if (threadIdx.x == 0) {
         m = umax(umax(lds4[0], lds4[1]), umax(lds4[2], lds4[3]));
         if (MODE == 2) {
-            // a record whose amax moved is marked volatile: the next carried run only collects its amax in the single
-            // pass and quantizes in the second one (the two-pass cost instead of two quantizations), until it holds still
+            // a record whose amax moved twice in a row is marked volatile: the next carried run only collects its amax in the
+            // single pass and quantizes in the second one (the two-pass cost instead of two quantizations), until it holds still
             const bool moved = rec[kRecAmax] != m;
-            rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;
-            rec[kRecVolatile] = moved ? 1u : 0u;
+            amax_record_after_carried_run(rec, moved);
             amax_feedback(moved_counter, moved, 1u);
         } else {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
+            rec[kRecMovedRuns] = 0;
             amax_feedback(moved_counter, rec[kRecAmax] != m, 1u);
         }
         rec[kRecAmax] = m;

@@ -217,7 +217,21 @@ constexpr int kSectionWords = 256;      // MQ_NVFP4_SECTION_WORDS: workgroups of
 constexpr int kRecordSections = 4;      // MQ_NVFP4_SECTIONS
 constexpr int kRecAmax = kRecordSections * kSectionWords;      // folded amax (float bits)
 constexpr int kRecRedo = kRecAmax + 4;  // the amax carried over from the last run turned out stale: quantize again
-constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last run: the next carried run collects the amax first
+constexpr int kRecVolatile = kRecAmax + 5;  // the amax moved on the last two runs: the next carried run collects the amax first
+constexpr int kRecMovedRuns = kRecAmax + 6; // carried runs in a row on which the amax moved (counted up to two)
+// What a fold of a carried run does with a record once it knows whether the amax moved.  A record that moved is
+// quantized a second time on this run (its codes were written with the stale amax).  Only a record that moved on two
+// runs in a row is marked volatile: the next carried run then just collects its amax in the single pass and quantizes
+// in the second one -- the plain two-pass cost, 4.56 bytes per element where a wasted quantization costs 5.12 -- until
+// the amax has held still for one run.  One move alone does not mark it: with an optimizer step between the syncs a
+// tensor's amax moves on one sync in five or so, mostly not on the next one too, and a record marked after a single move
+// paid the two-pass cost for nothing on the sync after every move.
+__device__ __forceinline__ void amax_record_after_carried_run(uint32_t* rec, bool moved) {
+    rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;     // a volatile record has no codes yet
+    const uint32_t runs = moved ? (rec[kRecMovedRuns] >= 1u ? 2u : 1u) : 0u;
+    rec[kRecMovedRuns] = runs;
+    rec[kRecVolatile] = runs >= 2u ? 1u : 0u;
+}
 // A fold launched by the job driver also tells its caller how many tensors' records held another amax before, and how
 // many tensors it folded (two counters in device memory that only ever grow: a copy taken at any time gives a
 // consistent rate): a caller whose every amax keeps moving can then submit the plain two-pass form.

@@ -120,10 +120,10 @@ constexpr int kRecEnc = kRecAmax + 3;                          // S_enc
 //   partial maxima with atomic max (see the carried-over amax below).  MODE 2 additionally checks the amax and scales
 //   the record held before against the new ones: all four words equal means the codes just written with the old values
 //   are final (kRecRedo = 0); otherwise the new values are stored and kRecRedo = 1 asks for a second quantization.
-//   A record whose amax moved is marked volatile (kRecVolatile): on the next carried sync the single pass only collects
-//   its partial maxima (no codes are written with an amax that is likely stale again) and the second pass quantizes it
-//   with the fresh amax -- the cost of the plain two-pass form, instead of two full quantizations.  The mark is dropped
-//   as soon as the amax has held still for one sync.
+//   A record whose amax moved on two syncs in a row is marked volatile (kRecVolatile): on the next carried sync the
+//   single pass only collects its partial maxima (no codes are written with an amax that is likely stale again) and the
+//   second pass quantizes it with the fresh amax -- the cost of the plain two-pass form, instead of two full
+//   quantizations.  The mark is dropped as soon as the amax has held still for one sync (amax_record_after_carried_run).
 template <int MODE, class Table>
 __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float numer, uint32_t* moved_counter, uint32_t* moved_mirror) {
     __shared__ uint32_t lds4[4];
@@ -146,12 +146,12 @@ __global__ __launch_bounds__(256) void nvfp4_fold_kernel(const Table tab, float 
         if (MODE == 2) {
             const bool moved = !(rec[kRecAmax] == f2u(amax) && rec[kRecEncSixth] == f2u(gs.enc_sixth) &&
                                  rec[kRecSDec] == f2u(gs.s_dec) && rec[kRecEnc] == f2u(gs.enc));
-            rec[kRecRedo] = (moved || rec[kRecVolatile] != 0) ? 1u : 0u;     // a volatile record has no codes yet
-            rec[kRecVolatile] = moved ? 1u : 0u;
+            amax_record_after_carried_run(rec, moved);
             amax_feedback(moved_counter, moved, (uint32_t)sections);
         } else if (MODE == 1) {
             rec[kRecRedo] = 0;
             rec[kRecVolatile] = 0;
+            rec[kRecMovedRuns] = 0;
             amax_feedback(moved_counter, rec[kRecAmax] != f2u(amax), (uint32_t)sections);
         }
         rec[kRecAmax] = f2u(amax);

@@ -1859,17 +1859,23 @@ def test_nvfp4_carried_amax_hits_and_misses(oracle, monkeypatch, four_over_six, 
     pair_dev[1].mul_(5.0)
     check("three amax moved")
     moved = [0, 1, 0, 1, 0, 1, 0]                  # records: tensors 0, 1, 2, the pair, tensors 3, 4, 5
-    assert state() == (moved, moved)               # quantized twice, and marked: the next run collects their amax first
+    assert state() == (moved, [0] * 7)             # quantized twice; one move alone does not mark a record
     check("and stayed")
-    assert state() == (moved, [0] * 7)             # the marked ones took the two-pass form once more, then settled
-    check("settled")
-    assert state() == ([0] * 7, [0] * 7)
+    assert state() == ([0] * 7, [0] * 7)           # the single pass with the new amax held
     dev[1].mul_(0.5)
     check("tensor 1 moved")
+    assert state() == ([0, 1, 0, 0, 0, 0, 0], [0] * 7)
     dev[1].mul_(0.5)
     dev[3].mul_(2.0)
-    check("tensor 1 moved again while marked, tensor 3 for the first time")
-    assert state() == ([0, 1, 0, 0, 1, 0, 0], [0, 1, 0, 0, 1, 0, 0])
+    check("tensor 1 moved again, tensor 3 for the first time")
+    assert state() == ([0, 1, 0, 0, 1, 0, 0], [0, 1, 0, 0, 0, 0, 0])      # twice in a row: marked
+    dev[1].mul_(2.0)
+    check("tensor 1 moved while marked: the single pass only collected its amax, the second pass quantized it")
+    assert state() == ([0, 1, 0, 0, 0, 0, 0], [0, 1, 0, 0, 0, 0, 0])
+    check("tensor 1 stayed: the two-pass form once more, and the mark is gone")
+    assert state() == ([0, 1, 0, 0, 0, 0, 0], [0] * 7)
+    check("settled")
+    assert state() == ([0] * 7, [0] * 7)
     dev[2].zero_()                                 # amax 0
     dev[0].view(-1)[7] = float("inf")              # amax inf
     check("zero tensor and an infinity")
