@@ -451,3 +451,48 @@ def test_strided_and_nd_views(oracle, view):
     if xc.dim() == 3:
         want = tuple(torch.stack(f) for f in zip(*[oracle.nvfp4_quantize_1d(cc[i]) for i in range(cc.shape[0])]))
         check("quantize_nvfp4 on a stack", quantize_nvfp4(xd), want)
+
+
+# rows of 256 elements whose flat grids (2048, 4096 or 8192 elements per workgroup, by kernel) come to workgroup counts
+# that select every run length the flat kernels deal to the XCDs: 1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64
+_RUN_LENGTH_ROWS = [16, 128, 192, 376, 512, 568, 752, 1024, 1136, 1519, 1520, 2048, 3024, 3040, 4096, 5999, 6000, 7984, 12000]
+
+
+@pytest.mark.parametrize("rows", _RUN_LENGTH_ROWS)
+def test_flat_kernels_on_every_xcd_run_length(oracle, rows):
+    """A flat kernel remaps its workgroup ids so that an XCD takes runs of consecutive blocks; the run length is picked
+    from the workgroup count (a power of two or three times one).  A wrong remap skips or repeats blocks, so every
+    quantizer's bytes are compared with the oracle's on sizes that select every run length, ragged ends included."""
+    from miles_amd import workloads as W
+    from miles_amd.kernels.quant.int4_fake import pack_layer
+    from miles_amd.tools.convert_hf_to_fp8 import block_fp8
+    from miles_amd.tools.convert_kimi_int4_to_bf16 import _dequantize_tensor
+    from miles_amd.tools.fp8_cast_bf16 import weight_dequant
+    from miles_amd.utils.mxfp4 import dequantize_mxfp4, quantize_mxfp4
+    from miles_amd.utils.mxfp8 import mxfp8_quantize, requantize_fp8_block_to_mxfp8
+    from miles_amd.utils.nvfp4 import nvfp4_quantize_1d
+
+    w = W.gaussian_outliers((rows, 256), std=0.02, p_outlier=0.001, gain=20.0, seed=4000 + rows)
+    d = w.to(DEV)
+
+    def same(got, want, what):
+        for k, (g_, w_) in enumerate(zip(got, want)):
+            if g_ is not None and w_ is not None:
+                _same(g_, w_, f"{what}, output {k}, {rows} rows")
+
+    same(mxfp8_quantize(d), oracle.mxfp8_quantize(w), "MXFP8")
+    same(pack_layer(d, 128)[:2], oracle.pack_layer(w, 128)[:2], "INT4 g128")
+    if rows % 8 == 0:           # the packed zero points take eight rows per word
+        same(pack_layer(d, 32, sym=False), oracle.pack_layer(w, 32, sym=False), "INT4 g32 asymmetric")
+    same(quantize_mxfp4(d, 32), oracle.quantize_mxfp4(w, 32), "MXFP4")
+    same(nvfp4_quantize_1d(d), oracle.nvfp4_quantize_1d(w), "NVFP4")
+    q, s = block_fp8(d, [128, 128])
+    q_o, s_o = oracle.block_fp8(w, [128, 128])
+    same((q, s), (q_o, s_o), "FP8 128 x 128")
+    same((weight_dequant(q, s),), (oracle.weight_dequant(q_o, s_o),), "FP8 dequantize")
+    same(requantize_fp8_block_to_mxfp8(q, s), oracle.fp8_block_to_mxfp8(q_o, s_o), "FP8 -> MXFP8")
+    p4, s4 = oracle.quantize_mxfp4(w, 32)
+    same((dequantize_mxfp4(p4.to(DEV), s4.to(DEV), 32),), (oracle.dequantize_mxfp4(p4, s4, 32),), "MXFP4 dequantize")
+    pk, sc, _ = oracle.pack_layer(w, 128)
+    same((_dequantize_tensor(pk.to(DEV), sc.to(DEV), (rows, 256), 128),), (oracle.int4_unpack_dequant(pk, sc, (rows, 256), 128),),
+         "INT4 unpack")
