@@ -278,16 +278,33 @@ __device__ __forceinline__ NvCandidate nv_four_over_six(const float f[8], float 
 struct NvCandidate16 {
     uint32_t sc;        // e4m3 byte
     uint32_t lo, hi;    // codes of elements 0..7 and 8..15
-    float s_f;          // f32(sc)
+    float a;            // RN(f32(sc) * amax / denom): what one unit of the code grid is worth (tensors that take the estimate)
 };
-__device__ __forceinline__ NvCandidate16 nv_candidate16(const float f[16], float s_hp, float s_dec) {
+// A candidate's block scale is one of 128 bytes, and what the quantizer needs of it -- the reciprocal
+// min(1 / (f32(byte) * S_dec), FLT_MAX) and, for the error estimate, RN(f32(byte) * amax / denom) -- depends on the byte
+// and the tensor only.  A workgroup therefore computes both for every byte once (128 lanes, one IEEE division each,
+// while its loads are in flight) into LDS, and a candidate is one 8-byte LDS read instead of a decode, a multiplication,
+// a range test, a refined reciprocal and a three-instruction division per block and candidate.
+struct NvScaleEntry {
+    float inv, a;
+};
+__device__ __forceinline__ void nv_fill_scale_table(NvScaleEntry* table, int t, float amax, float s_dec, bool estimate,
+                                                    float denom, float denom_inv) {
+    if (t < 128) {
+        const float s_f = hw_e4m3x2_decode<false>((uint32_t)t).x;
+        NvScaleEntry e;
+        e.inv = __builtin_fminf(1.0f / (s_f * s_dec), kFltMax);
+        // (only read where f32(byte) * amax is exact and the sequence gives its correctly rounded quotient)
+        e.a = estimate ? div_by_numer<2>(s_f * amax, denom, denom_inv) : 0.0f;
+        table[t] = e;
+    }
+}
+__device__ __forceinline__ NvCandidate16 nv_candidate16(const float f[16], float s_hp, const NvScaleEntry* table) {
     NvCandidate16 c;
     c.sc = hw_e4m3x2<false>(__builtin_fminf(s_hp, kFp8Max), 0.0f, 0u) & 0xFFu;
-    c.s_f = hw_e4m3x2_decode<false>(c.sc).x;
-    const float d = c.s_f * s_dec;
-    float inv;
-    if (__builtin_amdgcn_ballot_w64(!shared_div_ok(d)) == 0) inv = recip_shared(d);
-    else inv = __builtin_fminf(1.0f / d, kFltMax);
+    const NvScaleEntry e = table[c.sc & 0x7Fu];      // s_hp is not negative: the byte has no sign bit
+    const float inv = e.inv;
+    c.a = e.a;
     c.lo = hw_e2m1x2<0>(f[0] * inv, f[1] * inv, 0u);
     c.lo = hw_e2m1x2<1>(f[2] * inv, f[3] * inv, c.lo);
     c.lo = hw_e2m1x2<2>(f[4] * inv, f[5] * inv, c.lo);
@@ -302,7 +319,7 @@ template <int EM, int FASTDIV>
 __device__ __forceinline__ float nv_block_error(const float f[16], const NvCandidate16& c, float amax, float enc, float denom,
                                                 float denom_inv) {
     float term[8], error = 0.0f;
-    NvCandidate half{c.sc, c.lo, c.s_f};
+    NvCandidate half{c.sc, c.lo, hw_e4m3x2_decode<false>(c.sc).x};
     nv_error_terms<EM, FASTDIV>(f, half, amax, enc, denom, denom_inv, term);
 #pragma unroll
     for (int j = 0; j < 8; j++) error = error + term[j];
@@ -347,14 +364,14 @@ __device__ __forceinline__ float nv_block_error_estimate(const float f[16], cons
 }
 template <int EM, int FASTDIV>
 __device__ __forceinline__ NvCandidate16 nv_four_over_six16(const float f[16], float bmax, float amax, const NvScales& gs,
-                                                            float denom, float denom_inv) {
+                                                            float denom, float denom_inv, const NvScaleEntry* table) {
     const bool plain_bmax = shared_div_ok(bmax);
     const float s6_hp = (__builtin_amdgcn_ballot_w64(!plain_bmax) == 0 ? div_by_shared(bmax, 6.0f, 0x1.555556p-3f) : bmax / 6.0f) * gs.enc;
     const float s4_hp = s6_hp * 1.5f;
-    const NvCandidate16 c4 = nv_candidate16(f, s4_hp, gs.s_dec), c6 = nv_candidate16(f, s6_hp, gs.s_dec);
+    const NvCandidate16 c4 = nv_candidate16(f, s4_hp, table), c6 = nv_candidate16(f, s6_hp, table);
     if ((EM == 0 || EM == 1) && FASTDIV == 2) {
         // (FASTDIV 2: f32(scale) * amax is exact and its quotient by denom comes correctly rounded from the sequence)
-        const float a4 = div_by_numer<2>(c4.s_f * amax, denom, denom_inv), a6 = div_by_numer<2>(c6.s_f * amax, denom, denom_inv);
+        const float a4 = c4.a, a6 = c6.a;
         const float g4 = nv_block_error_estimate<EM == 1>(f, c4, a4), g6 = nv_block_error_estimate<EM == 1>(f, c6, a6);
         float guard;
         if (EM == 0) {
@@ -399,6 +416,7 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
     static_assert(kNvUnroll == 2, "the regrouping pairs the two units of a lane");
     constexpr uint32_t kPiece = kNvThreads * 2;
     __shared__ u32x4 stage[kPiece];
+    __shared__ NvScaleEntry scale_table[128];
     const uint16_t* __restrict__ w = (const uint16_t*)job.w;
     uint32_t* __restrict__ q = (uint32_t*)job.q;
     uint8_t* __restrict__ s8 = (uint8_t*)job.s;
@@ -430,6 +448,9 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
     // picked on the scalar unit
     constexpr float kInv2688 = 1.0f / 2688.0f, kInv1536 = 1.0f / 1536.0f;
     const float denom_inv = denom == 2688.0f ? kInv2688 : denom == 1536.0f ? kInv1536 : 1.0f / denom;
+    // (a workgroup that comes here again, in the striding second pass, writes the same values over the table: one tensor)
+    nv_fill_scale_table(scale_table, t, amax, gs.s_dec, fastdiv == 2 && EM < 2, denom, denom_inv);
+    __syncthreads();
     uint32_t seen = 0;
 #pragma unroll
     for (int r = 0; r < kFosRounds; r++) {
@@ -459,9 +480,9 @@ __device__ __forceinline__ uint32_t nvfp4_fos_units(const FlatJob& job, const in
                              elem_lo<F16>(lo.z), elem_hi<F16>(lo.z), elem_lo<F16>(lo.w), elem_hi<F16>(lo.w),
                              elem_lo<F16>(hi.x), elem_hi<F16>(hi.x), elem_lo<F16>(hi.y), elem_hi<F16>(hi.y),
                              elem_lo<F16>(hi.z), elem_hi<F16>(hi.z), elem_lo<F16>(hi.w), elem_hi<F16>(hi.w)};
-        const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom, denom_inv)
-                                : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom, denom_inv)
-                                               : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom, denom_inv);
+        const NvCandidate16 c = fastdiv == 2   ? nv_four_over_six16<EM, 2>(f, bmax, amax, gs, denom, denom_inv, scale_table)
+                                : fastdiv == 1 ? nv_four_over_six16<EM, 1>(f, bmax, amax, gs, denom, denom_inv, scale_table)
+                                               : nv_four_over_six16<EM, 0>(f, bmax, amax, gs, denom, denom_inv, scale_table);
         if (first < rem) {      // the tensor is whole blocks: both units of a block are inside or outside
             st8(q0 + r * kPiece + first, u32x2{c.lo, c.hi});      // `first` is even and `base` a multiple of the piece
             s80[(r * kPiece + first) >> 1] = (uint8_t)c.sc;
