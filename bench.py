@@ -24,7 +24,6 @@ import json
 import os
 import sys
 import time
-from argparse import Namespace
 
 import torch
 
